@@ -1,0 +1,259 @@
+// Shape-bucket dispatcher: the MI355X counterpart of the call_table / index_table that DTAS
+// splices into its generated host code (python/dtas/engine/tuner.py:156-299 builds the tables,
+// python/dtas/codegen/code_gen.py:242-405 emits them; emitted form
+// experiment/dtas_tuned/elementwise/add/float16/top1_256/host.cc:105-125).
+//
+// The dynamic extent n is cut into buckets [1, div], [div+1, 2*div], ... up to kUpperBound
+// (python/dtas/common/config.py:64-78); a call picks
+//     index = min((n - 1) / kRangeDiv, last)
+// and uses the config of that bucket.  (The reference's emitted statement is n / div, which
+// sends n = k*div to the bucket above the one whose label contains it; that is harmless there
+// because every bucket kernel is predicated on n, but here a bucket's config is sized for its
+// upper end, so the built-in tables use the labelled ranges exactly.  Tables produced by the
+// Python Engine keep the reference's statement.)  The reference fills each bucket by timing top-k
+// candidates on the GPU and keeps one kernel per merged bucket range; here each bucket's
+// config is a closed-form function of the bucket's upper end and the static extents, written
+// for gfx950 (256 CUs, wave64, 160 KiB LDS), evaluated at call time.  dtas_select_bucket
+// reports the merged range [lo, hi] of equal configs around n, named as the reference names
+// bucket kernels.
+#include "dtas_host.h"
+
+namespace dtas {
+
+namespace {
+thread_local char g_error[512] = {0};
+
+constexpr int64_t kRangeDiv = 16;      // bucket width of the built-in tables
+constexpr int64_t kUpperBound = 8192;  // dynamic extents above it share the last bucket
+constexpr int64_t kLastIndex = (kUpperBound + kRangeDiv - 1) / kRangeDiv - 1;
+
+dtas_config make(int variant, int block, int vec, int unroll, int t0 = 0, int t1 = 0, int t2 = 0, int split_k = 1,
+                 int64_t cap = 0) {
+  dtas_config c;
+  c.variant = variant;
+  c.block = block;
+  c.vec = vec;
+  c.unroll = unroll;
+  c.tile[0] = t0;
+  c.tile[1] = t1;
+  c.tile[2] = t2;
+  c.split_k = split_k;
+  c.grid_cap = cap;
+  return c;
+}
+
+bool same(const dtas_config& a, const dtas_config& b) {
+  return a.variant == b.variant && a.block == b.block && a.vec == b.vec && a.unroll == b.unroll &&
+         a.tile[0] == b.tile[0] && a.tile[1] == b.tile[1] && a.tile[2] == b.tile[2] && a.split_k == b.split_k &&
+         a.grid_cap == b.grid_cap;
+}
+
+int narrow_bytes(int op) {
+  switch (op) {
+    case DTAS_OP_ADD_F32: case DTAS_OP_COPY_F32: return 4;
+    case DTAS_OP_ADD_I8: case DTAS_OP_COPY_I8: return 1;
+    default: return 2;
+  }
+}
+
+// ---- per-family policies: config for a bucket whose upper end is n_hi -----------------
+
+// Elementwise: 128-bit accesses; few elements -> one access per thread so the work spreads
+// over more CUs, many elements -> 4 accesses in flight per thread.
+dtas_config elementwise_policy(int op, int64_t n_hi, int64_t H) {
+  const int vec = 16 / narrow_bytes(op);
+  const int64_t nvec = n_hi * (H > 0 ? H : 1) / vec;
+  const int unroll = nvec <= 256 * kNumCU * 2 ? 1 : nvec <= 256 * kNumCU * 8 ? 2 : 4;
+  return make(DTAS_ELT_VECTOR, 256, vec, unroll);
+}
+
+// Norms: n rows of static length H.  Up to a few rows per CU a whole workgroup per row hides
+// latency best; beyond that one wavefront per row keeps every reduction on the DPP path.
+dtas_config norm_policy(int op, int64_t n_hi, int64_t H) {
+  const int vec = op == DTAS_OP_RMS_NORM_F16 ? 8 : 4;
+  const int64_t nvec = (H + vec - 1) / vec;
+  const bool wave_fits = nvec <= 64 * 16;
+  if (wave_fits && n_hi > 2 * kNumCU) return make(DTAS_RED_WAVE_ROW, 256, vec, 1);
+  int block = 64;
+  while (block < 1024 && (nvec > block * 2)) block *= 2;  // aim for <= 2 vectors per lane
+  if (nvec > static_cast<int64_t>(block) * 16) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
+  return make(DTAS_RED_BLOCK_ROW, block, vec, 1);
+}
+
+// Softmax: 32*n rows of dynamic length n (the reduction axis is the dynamic one).
+dtas_config softmax_policy(int op, int64_t cols_hi, int64_t rows) {
+  const int vec = op == DTAS_OP_SOFTMAX_F16 ? 8 : 4;
+  const int64_t nvec = (cols_hi + vec - 1) / vec;
+  if (nvec <= 64 * 16 && (rows <= 0 || rows > 2 * kNumCU)) return make(DTAS_RED_WAVE_ROW, 256, vec, 1);
+  int block = 64;
+  while (block < 1024 && (nvec > block * 2)) block *= 2;
+  if (nvec > static_cast<int64_t>(block) * 16) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
+  return make(DTAS_RED_BLOCK_ROW, block, vec, 1);
+}
+
+// GEMV: rows per workgroup so that there are at least ~4 workgroups per CU.
+dtas_config gemv_policy(int64_t N, int64_t K) {
+  (void)K;
+  const int rows = N >= 8 * 4 * kNumCU ? 8 : N >= 4 * 4 * kNumCU ? 4 : N >= 2 * 4 * kNumCU ? 2 : 1;
+  return make(DTAS_GEMV_SPLITK, 256, 8, 2, rows);
+}
+
+// GEMM: M <= 64 streams W once (SKINNY).  Above that, the MFMA tile minimising
+// rounds(tiles / CUs) * tile_area / efficiency(tile): bigger tiles reuse LDS data better,
+// smaller ones fill the 256 CUs at small M (the reference scores tiles the same way,
+// python/dtas/policy/wmma_config_emiter.py:148-262).
+dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
+  (void)K;
+  if (M_hi <= 64) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
+  static const struct { int bm, bn; double eff; } kTiles[] = {
+      {256, 256, 1.00}, {256, 128, 0.85}, {128, 256, 0.85}, {128, 128, 0.70},
+      {64, 128, 0.50},  {128, 64, 0.50},  {64, 64, 0.35}};
+  double best = 0;
+  int pick = -1;
+  for (int i = 0; i < 7; ++i) {
+    const int64_t tiles = ceil_div(M_hi, kTiles[i].bm) * ceil_div(N > 0 ? N : 1, kTiles[i].bn);
+    const double cost = static_cast<double>(ceil_div(tiles, kNumCU)) * kTiles[i].bm * kTiles[i].bn / kTiles[i].eff;
+    if (pick < 0 || cost < best) {
+      best = cost;
+      pick = i;
+    }
+  }
+  return make(DTAS_GEMM_MFMA, 256, 8, 1, kTiles[pick].bm, kTiles[pick].bn, 64);
+}
+
+dtas_config policy(int op, int64_t n_hi, int64_t d0, int64_t d1) {
+  switch (op) {
+    case DTAS_OP_LAYER_NORM_F32_F16:
+    case DTAS_OP_RMS_NORM_F16: return norm_policy(op, n_hi, d0);
+    case DTAS_OP_SOFTMAX_F32_F16:
+    case DTAS_OP_SOFTMAX_F16: return softmax_policy(op, n_hi, d0);
+    case DTAS_OP_GEMV_F16: return gemv_policy(d0, d1);
+    case DTAS_OP_GEMM_F16: return gemm_policy(n_hi, d0, d1);
+    default: return elementwise_policy(op, n_hi, d0);
+  }
+}
+
+int64_t bucket_index(int64_t n) {
+  const int64_t i = n <= 0 ? 0 : (n - 1) / kRangeDiv;
+  return i > kLastIndex ? kLastIndex : i;
+}
+// upper end of the reference-style range [index*div + 1, (index + 1)*div]
+int64_t bucket_hi(int64_t index) { return (index + 1) * kRangeDiv; }
+
+const char* op_func_name(int op) {
+  switch (op) {
+    case DTAS_OP_ADD_F16: case DTAS_OP_ADD_F32: case DTAS_OP_ADD_I8: return "add";
+    case DTAS_OP_COPY_F16: case DTAS_OP_COPY_F32: case DTAS_OP_COPY_I8: return "copy";
+    case DTAS_OP_CAST_F16_F32: case DTAS_OP_CAST_F32_F16: return "cast";
+    case DTAS_OP_LAYER_NORM_F32_F16: return "fused_layer_norm_cast1";
+    case DTAS_OP_RMS_NORM_F16: return "rms_norm";
+    case DTAS_OP_SOFTMAX_F32_F16: case DTAS_OP_SOFTMAX_F16: return "fused_softmax_cast";
+    case DTAS_OP_GEMV_F16: return "fused_NT_matmul10_add5";
+    case DTAS_OP_GEMM_F16: return "fused_NT_matmul4_add1";
+  }
+  return "unknown";
+}
+
+int describe(int op, int64_t n, int64_t d0, int64_t d1, const dtas_config& cfg, int64_t la[7]) {
+  switch (op) {
+    case DTAS_OP_LAYER_NORM_F32_F16:
+    case DTAS_OP_RMS_NORM_F16: return describe_reduction(op, n, d0, cfg, la);
+    case DTAS_OP_SOFTMAX_F32_F16:
+    case DTAS_OP_SOFTMAX_F16: return describe_reduction(op, d0, d1, cfg, la);
+    case DTAS_OP_GEMV_F16: return describe_gemv(d0, d1, cfg, la);
+    case DTAS_OP_GEMM_F16: return describe_gemm(n, d0, d1, cfg, la);
+    default: return describe_eltwise(op, n * d0, cfg, la);
+  }
+}
+}  // namespace
+
+char* error_buffer() { return g_error; }
+void clear_error() { g_error[0] = 0; }
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return -1;
+}
+
+void bucket_kernel_name(char* dst, size_t cap, const char* func, const char* var, int64_t lo, int64_t hi) {
+  snprintf(dst, cap, "%s_%s_%lld_to_%lld__kernel", func, var, (long long)lo, (long long)hi);
+}
+
+Bucketed builtin_config(int op, int64_t n, int64_t d0, int64_t d1) {
+  Bucketed b;
+  b.index = static_cast<int32_t>(bucket_index(n < 0 ? 0 : n));
+  b.row = b.index;
+  b.lo = b.index * kRangeDiv + 1;
+  b.hi = bucket_hi(b.index);
+  // the last bucket also takes every n above the upper bound: size it for the n at hand
+  const int64_t n_hi = (b.index == kLastIndex && n > b.hi) ? n : b.hi;
+  b.cfg = policy(op, n_hi, d0, d1);
+  return b;
+}
+
+}  // namespace dtas
+
+extern "C" {
+
+int dtas_abi_version(void) { return DTAS_ABI_VERSION; }
+
+const char* dtas_last_error(void) { return dtas::error_buffer(); }
+
+int dtas_init(void) {
+  using namespace dtas;
+  clear_error();
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail("dtas_init: no HIP device: %s", hipGetErrorString(e));
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return fail("dtas_init: hipGetDeviceProperties: %s", hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail("dtas_init: device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+  return 0;
+}
+
+int dtas_select_bucket(int op, int64_t n, int64_t d0, int64_t d1, dtas_launch_info* out) {
+  using namespace dtas;
+  clear_error();
+  if (!out) return fail("dtas_select_bucket: out is NULL");
+  if (op < 0 || op >= DTAS_OP_COUNT) return fail("dtas_select_bucket: unknown op %d", op);
+  if (n < 0) return fail("dtas_select_bucket: negative dynamic extent %lld", (long long)n);
+  memset(out, 0, sizeof(*out));
+  const bool softmax = op == DTAS_OP_SOFTMAX_F16 || op == DTAS_OP_SOFTMAX_F32_F16;
+  // softmax: the dynamic extent is the row length; callers pass (n, rows, cols)
+  const Bucketed b = builtin_config(op, n, d0, d1);
+  // merge neighbouring buckets that resolve to the same config (tuner.py:211-299)
+  int64_t lo_idx = b.index, hi_idx = b.index;
+  while (lo_idx > 0 && same(policy(op, bucket_hi(lo_idx - 1), d0, d1), b.cfg)) --lo_idx;
+  while (hi_idx < kLastIndex && same(policy(op, bucket_hi(hi_idx + 1), d0, d1), b.cfg)) ++hi_idx;
+  // table_row = number of config changes below this bucket = row of the merged call table
+  int32_t row = 0;
+  for (int64_t i = 1; i <= lo_idx; ++i)
+    if (!same(policy(op, bucket_hi(i), d0, d1), policy(op, bucket_hi(i - 1), d0, d1))) ++row;
+  out->index = b.index;
+  out->table_row = row;
+  out->bucket_lo = lo_idx * kRangeDiv + 1;
+  out->bucket_hi = bucket_hi(hi_idx);
+  out->config = b.cfg;
+  const char* var = (op == DTAS_OP_GEMM_F16) ? "n" : (softmax ? "m" : "n");
+  bucket_kernel_name(out->name, sizeof(out->name), op_func_name(op), var, out->bucket_lo, out->bucket_hi);
+  const int64_t nn = n > 0 ? n : 1;
+  return describe(op, nn, d0, softmax ? nn : d1, b.cfg, out->launch_args);
+}
+
+int dtas_describe_launch(int op, int64_t n, int64_t d0, int64_t d1, const dtas_config* cfg, dtas_launch_info* out) {
+  using namespace dtas;
+  clear_error();
+  if (!out || !cfg) return fail("dtas_describe_launch: NULL argument");
+  if (op < 0 || op >= DTAS_OP_COUNT) return fail("dtas_describe_launch: unknown op %d", op);
+  memset(out, 0, sizeof(*out));
+  out->config = *cfg;
+  out->index = -1;
+  out->table_row = -1;
+  snprintf(out->name, sizeof(out->name), "%s_kernel", op_func_name(op));
+  return describe(op, n, d0, d1, *cfg, out->launch_args);
+}
+}

@@ -1,0 +1,79 @@
+// Device-side helpers for gfx950: 128-bit vector types, wave64 DPP reductions,
+// workgroup reductions through LDS.  Internal to libdtas_gfx950.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace dtas {
+
+typedef _Float16 half_t;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// ---- wave64 cross-lane reduction on the DPP datapath -------------------------------
+// quad_perm xor-1, quad_perm xor-2, row_half_mirror, row_mirror leave every lane of a
+// 16-lane row holding the row's result; row_bcast:15 / row_bcast:31 fold the four rows
+// into lane 63, which v_readlane broadcasts as a scalar.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_mov(float old, float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
+                                                                __builtin_bit_cast(int, v), CTRL,
+                                                                ROW_MASK, 0xf, false));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_mov<0xB1, 0xf>(0.f, v);
+  v += dpp_mov<0x4E, 0xf>(0.f, v);
+  v += dpp_mov<0x141, 0xf>(0.f, v);
+  v += dpp_mov<0x140, 0xf>(0.f, v);
+  v += dpp_mov<0x142, 0xa>(0.f, v);
+  v += dpp_mov<0x143, 0xc>(0.f, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_mov<0xB1, 0xf>(v, v));
+  v = fmaxf(v, dpp_mov<0x4E, 0xf>(v, v));
+  v = fmaxf(v, dpp_mov<0x141, 0xf>(v, v));
+  v = fmaxf(v, dpp_mov<0x140, 0xf>(v, v));
+  v = fmaxf(v, dpp_mov<0x142, 0xa>(v, v));
+  v = fmaxf(v, dpp_mov<0x143, 0xc>(v, v));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// ---- workgroup reduction: DPP inside each wavefront, one LDS slot per wavefront ------
+// `slots` needs blockDim.x / 64 floats; every thread of the workgroup must call.
+struct SumOp {
+  static __device__ __forceinline__ float wave(float v) { return wave_sum(v); }
+  static __device__ __forceinline__ float join(float a, float b) { return a + b; }
+};
+struct MaxOp {
+  static __device__ __forceinline__ float wave(float v) { return wave_max(v); }
+  static __device__ __forceinline__ float join(float a, float b) { return fmaxf(a, b); }
+};
+
+template <typename Op>
+__device__ __forceinline__ float block_reduce(float v, float* slots) {
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const float w = Op::wave(v);
+  if (nwaves == 1) return w;
+  __syncthreads();  // slots may still be read by the previous reduction
+  if ((threadIdx.x & 63) == 0) slots[wave] = w;
+  __syncthreads();
+  float r = slots[0];
+  for (int i = 1; i < nwaves; ++i) r = Op::join(r, slots[i]);
+  return r;
+}
+
+// ---- streaming (touch-once) global accesses ---------------------------------------
+template <typename V>
+__device__ __forceinline__ V load_stream(const V* p) { return __builtin_nontemporal_load(p); }
+template <typename V>
+__device__ __forceinline__ void store_stream(V v, V* p) { __builtin_nontemporal_store(v, p); }
+
+}  // namespace dtas

@@ -1,0 +1,313 @@
+// Elementwise add / copy / cast for gfx950.
+//
+// Replaces the kernels that DTAS's elementwise rule generates
+// (python/dtas/schedule/tir_elementwise.py:23-47: fuse all loops, split into
+// [grid, loop, 256 threads, vector], bind, vectorize; generated form
+// experiment/dtas_tuned/elementwise/add/float16/top1_256/tvm_device_kernels.cu:90-107).
+//
+// MI355X shape of the same idea: the fused (1, n, H) space is one flat array; a thread
+// moves `vec` contiguous elements per access (up to 128 bit on the narrower side), a
+// wavefront's 64 accesses are one contiguous span, each thread keeps `unroll` accesses in
+// flight, a workgroup is 256 threads (4 wavefronts) and walks tiles of 256*unroll vectors
+// grid-stride.  Accesses are marked non-temporal: every byte is touched once.
+#include "dtas_device.h"
+#include "dtas_host.h"
+
+namespace dtas {
+namespace {
+
+constexpr int kBlock = 256;
+
+// ---- raw fixed-size accesses ------------------------------------------------------
+template <int BYTES>
+struct Raw;
+template <>
+struct Raw<1> {
+  uint8_t d;
+  static __device__ __forceinline__ Raw load(const void* p, int64_t i) { return {load_stream(static_cast<const uint8_t*>(p) + i)}; }
+  __device__ __forceinline__ void store(void* p, int64_t i) const { store_stream(d, static_cast<uint8_t*>(p) + i); }
+};
+template <>
+struct Raw<2> {
+  uint16_t d;
+  static __device__ __forceinline__ Raw load(const void* p, int64_t i) { return {load_stream(static_cast<const uint16_t*>(p) + i)}; }
+  __device__ __forceinline__ void store(void* p, int64_t i) const { store_stream(d, static_cast<uint16_t*>(p) + i); }
+};
+template <>
+struct Raw<4> {
+  uint32_t d;
+  static __device__ __forceinline__ Raw load(const void* p, int64_t i) { return {load_stream(static_cast<const uint32_t*>(p) + i)}; }
+  __device__ __forceinline__ void store(void* p, int64_t i) const { store_stream(d, static_cast<uint32_t*>(p) + i); }
+};
+template <>
+struct Raw<8> {
+  u32x2 d;
+  static __device__ __forceinline__ Raw load(const void* p, int64_t i) { return {load_stream(static_cast<const u32x2*>(p) + i)}; }
+  __device__ __forceinline__ void store(void* p, int64_t i) const { store_stream(d, static_cast<u32x2*>(p) + i); }
+};
+template <>
+struct Raw<16> {
+  u32x4 d;
+  static __device__ __forceinline__ Raw load(const void* p, int64_t i) { return {load_stream(static_cast<const u32x4*>(p) + i)}; }
+  __device__ __forceinline__ void store(void* p, int64_t i) const { store_stream(d, static_cast<u32x4*>(p) + i); }
+};
+template <>
+struct Raw<32> {
+  u32x4 d[2];
+  static __device__ __forceinline__ Raw load(const void* p, int64_t i) {
+    const u32x4* q = static_cast<const u32x4*>(p) + 2 * i;
+    return {{load_stream(q), load_stream(q + 1)}};
+  }
+  __device__ __forceinline__ void store(void* p, int64_t i) const {
+    u32x4* q = static_cast<u32x4*>(p) + 2 * i;
+    store_stream(d[0], q);
+    store_stream(d[1], q + 1);
+  }
+};
+
+template <typename T, int VEC>
+struct Elems {
+  T v[VEC];
+};
+
+// ---- the three element functions ----------------------------------------------------
+// fp16 add is one IEEE rounding per lane (v_add_f16 / v_pk_add_f16), as the generated CUDA
+// does with per-lane `half` adds; int8 wraps modulo 256.
+template <typename T>
+struct AddOp {
+  typedef T In;
+  typedef T Out;
+  static constexpr int kInputs = 2;
+  static __device__ __forceinline__ T apply(T a, T b) { return a + b; }
+};
+template <>
+struct AddOp<int8_t> {
+  typedef int8_t In;
+  typedef int8_t Out;
+  static constexpr int kInputs = 2;
+  static __device__ __forceinline__ int8_t apply(int8_t a, int8_t b) {
+    return static_cast<int8_t>(static_cast<uint8_t>(static_cast<uint8_t>(a) + static_cast<uint8_t>(b)));
+  }
+};
+// Copy moves bit patterns through integer registers, so NaN payloads survive.
+template <typename Bits>
+struct CopyOp {
+  typedef Bits In;
+  typedef Bits Out;
+  static constexpr int kInputs = 1;
+  static __device__ __forceinline__ Bits apply(Bits a, Bits) { return a; }
+};
+// Cast: fp16 -> fp32 is exact; fp32 -> fp16 rounds to nearest even and overflows to +-inf
+// (v_cvt_f16_f32), fp16 subnormal results are kept.
+template <typename TI, typename TO>
+struct CastOp {
+  typedef TI In;
+  typedef TO Out;
+  static constexpr int kInputs = 1;
+  static __device__ __forceinline__ TO apply(TI a, TI) { return static_cast<TO>(a); }
+};
+
+// ---- kernels ------------------------------------------------------------------------
+template <typename Op, int VEC, int U>
+__global__ void __launch_bounds__(kBlock) elt_vector_kernel(const void* __restrict__ a, const void* __restrict__ b,
+                                                            void* __restrict__ out, int64_t nvec, int64_t count) {
+  typedef typename Op::In TI;
+  typedef typename Op::Out TO;
+  typedef Raw<VEC * sizeof(TI)> RI;
+  typedef Raw<VEC * sizeof(TO)> RO;
+  constexpr int64_t kTile = static_cast<int64_t>(kBlock) * U;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * kTile;
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * kTile; base < nvec; base += step) {
+    RI ra[U], rb[U];
+    const int64_t first = base + threadIdx.x;
+    const bool full = base + kTile <= nvec;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = first + u * kBlock;
+      if (full || i < nvec) {
+        ra[u] = RI::load(a, i);
+        if (Op::kInputs == 2) rb[u] = RI::load(b, i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = first + u * kBlock;
+      if (full || i < nvec) {
+        Elems<TI, VEC> ea, eb;
+        Elems<TO, VEC> eo;
+        __builtin_memcpy(&ea, &ra[u], sizeof(ea));
+        if (Op::kInputs == 2) __builtin_memcpy(&eb, &rb[u], sizeof(eb)); else eb = ea;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) eo.v[e] = Op::apply(ea.v[e], eb.v[e]);
+        RO ro;
+        __builtin_memcpy(&ro, &eo, sizeof(ro));
+        ro.store(out, i);
+      }
+    }
+  }
+  // the last count % VEC elements, one per thread of workgroup 0
+  if (blockIdx.x == 0) {
+    const int64_t i = nvec * VEC + threadIdx.x;
+    if (i < count) {
+      const TI x = static_cast<const TI*>(a)[i];
+      const TI y = Op::kInputs == 2 ? static_cast<const TI*>(b)[i] : x;
+      static_cast<TO*>(out)[i] = Op::apply(x, y);
+    }
+  }
+}
+
+template <typename Op, int VEC, int U>
+int launch_vector(const void* a, const void* b, void* out, int64_t count, int64_t grid, hipStream_t s) {
+  const int64_t nvec = count / VEC;
+  hipLaunchKernelGGL((elt_vector_kernel<Op, VEC, U>), dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, s, a, b, out,
+                     nvec, count);
+  return check_launch("elementwise");
+}
+
+template <typename Op, int VEC>
+int launch_unroll(int unroll, const void* a, const void* b, void* out, int64_t count, int64_t grid, hipStream_t s) {
+  switch (unroll) {
+    case 1: return launch_vector<Op, VEC, 1>(a, b, out, count, grid, s);
+    case 2: return launch_vector<Op, VEC, 2>(a, b, out, count, grid, s);
+    case 4: return launch_vector<Op, VEC, 4>(a, b, out, count, grid, s);
+    case 8: return launch_vector<Op, VEC, 8>(a, b, out, count, grid, s);
+  }
+  return fail("elementwise: unroll %d is not one of 1, 2, 4, 8", unroll);
+}
+
+// Widest access is 16 bytes on the narrower of the two element types (and so at most 32 on
+// the wider one); the three widths are the reference's candidates 128 / 64 / 32 bit
+// (python/dtas/policy/elementwise_config_emiter.py:9-34).
+template <typename Op>
+int launch_op(const dtas_config& cfg, const void* a, const void* b, void* out, int64_t count, int64_t grid,
+              hipStream_t s) {
+  constexpr int kNarrow = sizeof(typename Op::In) < sizeof(typename Op::Out) ? sizeof(typename Op::In)
+                                                                             : sizeof(typename Op::Out);
+  constexpr int kMaxVec = 16 / kNarrow;
+  if (cfg.variant == DTAS_ELT_SCALAR) return launch_unroll<Op, 1>(cfg.unroll, a, b, out, count, grid, s);
+  if (cfg.vec == kMaxVec) return launch_unroll<Op, kMaxVec>(cfg.unroll, a, b, out, count, grid, s);
+  if (cfg.vec == kMaxVec / 2) return launch_unroll<Op, kMaxVec / 2>(cfg.unroll, a, b, out, count, grid, s);
+  if (cfg.vec == kMaxVec / 4) return launch_unroll<Op, kMaxVec / 4>(cfg.unroll, a, b, out, count, grid, s);
+  return fail("elementwise: vector width %d not in {%d, %d, %d}", cfg.vec, kMaxVec, kMaxVec / 2, kMaxVec / 4);
+}
+
+struct EltInfo {
+  int in_bytes, out_bytes, inputs;
+  const char* name;
+};
+
+bool elt_info(int op, EltInfo* e) {
+  switch (op) {
+    case DTAS_OP_ADD_F16: *e = {2, 2, 2, "add"}; return true;
+    case DTAS_OP_ADD_F32: *e = {4, 4, 2, "add"}; return true;
+    case DTAS_OP_ADD_I8: *e = {1, 1, 2, "add"}; return true;
+    case DTAS_OP_COPY_F16: *e = {2, 2, 1, "copy"}; return true;
+    case DTAS_OP_COPY_F32: *e = {4, 4, 1, "copy"}; return true;
+    case DTAS_OP_COPY_I8: *e = {1, 1, 1, "copy"}; return true;
+    case DTAS_OP_CAST_F16_F32: *e = {2, 4, 1, "cast"}; return true;
+    case DTAS_OP_CAST_F32_F16: *e = {4, 2, 1, "cast"}; return true;
+  }
+  return false;
+}
+
+int run_eltwise(int op, const void* a, const void* b, void* out, int64_t n, int64_t H, const dtas_config* user,
+                void* stream) {
+  clear_error();
+  EltInfo e;
+  if (!elt_info(op, &e)) return fail("elementwise: unknown op %d", op);
+  if (n < 0 || H < 0) return fail("%s: negative extent n=%lld H=%lld", e.name, (long long)n, (long long)H);
+  if (H != 0 && n > INT64_MAX / 8 / H) return fail("%s: n*H overflows", e.name);
+  const int64_t count = n * H;
+  if (count == 0) return 0;
+  if (!a || !out || (e.inputs == 2 && !b)) return fail("%s: NULL buffer with n=%lld", e.name, (long long)n);
+  if (overlaps(a, count * e.in_bytes, out, count * e.out_bytes) ||
+      (e.inputs == 2 && overlaps(b, count * e.in_bytes, out, count * e.out_bytes)))
+    return fail("%s: output overlaps an input (PrimFunc is tir.noalias)", e.name);
+
+  dtas_config cfg = user ? *user : builtin_config(op, n, H, 0).cfg;
+  // A vector access needs its natural alignment on every buffer; the built-in choice steps
+  // down to element accesses for odd pointers, an explicit config is taken at its word.
+  if (cfg.variant == DTAS_ELT_VECTOR) {
+    const size_t ia = static_cast<size_t>(cfg.vec) * e.in_bytes, oa = static_cast<size_t>(cfg.vec) * e.out_bytes;
+    const size_t ia16 = ia > 16 ? 16 : ia, oa16 = oa > 16 ? 16 : oa;
+    const bool ok = cfg.vec > 0 && (ia & (ia - 1)) == 0 && aligned(a, ia16) && aligned(out, oa16) &&
+                    (e.inputs == 1 || aligned(b, ia16));
+    if (!ok) {
+      if (user) return fail("%s: buffers are not aligned for %d-element accesses", e.name, cfg.vec);
+      cfg.variant = DTAS_ELT_SCALAR;
+      cfg.vec = 1;
+    }
+  }
+  int64_t la[7];
+  if (describe_eltwise(op, count, cfg, la) != 0) return -1;
+  const int64_t grid = la[0];
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (op) {
+    case DTAS_OP_ADD_F16: return launch_op<AddOp<half_t>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_ADD_F32: return launch_op<AddOp<float>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_ADD_I8: return launch_op<AddOp<int8_t>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_COPY_F16: return launch_op<CopyOp<uint16_t>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_COPY_F32: return launch_op<CopyOp<uint32_t>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_COPY_I8: return launch_op<CopyOp<uint8_t>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_CAST_F16_F32: return launch_op<CastOp<half_t, float>>(cfg, a, b, out, count, grid, s);
+    case DTAS_OP_CAST_F32_F16: return launch_op<CastOp<float, half_t>>(cfg, a, b, out, count, grid, s);
+  }
+  return fail("elementwise: unknown op %d", op);
+}
+
+}  // namespace
+
+// grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
+// ElementwiseConfigEmiter.get_num_blocks (python/dtas/policy/elementwise_config_emiter.py:35-54)
+// with the per-thread unroll folded into the tile.
+int describe_eltwise(int op, int64_t count, const dtas_config& cfg, int64_t la[7]) {
+  EltInfo e;
+  if (!elt_info(op, &e)) return fail("elementwise: unknown op %d", op);
+  if (cfg.block != kBlock) return fail("%s: block must be %d threads, got %d", e.name, kBlock, cfg.block);
+  if (cfg.variant != DTAS_ELT_VECTOR && cfg.variant != DTAS_ELT_SCALAR)
+    return fail("%s: unknown variant %d", e.name, cfg.variant);
+  if (cfg.unroll != 1 && cfg.unroll != 2 && cfg.unroll != 4 && cfg.unroll != 8)
+    return fail("%s: unroll %d is not one of 1, 2, 4, 8", e.name, cfg.unroll);
+  const int narrow = e.in_bytes < e.out_bytes ? e.in_bytes : e.out_bytes;
+  const int vec = cfg.variant == DTAS_ELT_SCALAR ? 1 : cfg.vec;
+  if (cfg.variant == DTAS_ELT_VECTOR && !(vec == 16 / narrow || vec == 8 / narrow || vec == 4 / narrow) )
+    return fail("%s: vector width %d not in {%d, %d, %d}", e.name, vec, 16 / narrow, 8 / narrow, 4 / narrow);
+  if (vec < 1) return fail("%s: vector width %d", e.name, vec);
+  const int64_t nvec = count / vec;
+  int64_t grid = ceil_div(nvec > 0 ? nvec : 1, static_cast<int64_t>(kBlock) * cfg.unroll);
+  if (cfg.grid_cap > 0 && grid > cfg.grid_cap) grid = cfg.grid_cap;
+  if (grid > 0x7fffffff) grid = 0x7fffffff;
+  if (grid < 1) grid = 1;
+  for (int i = 0; i < 7; ++i) la[i] = 0;
+  la[0] = grid; la[1] = 1; la[2] = 1; la[3] = kBlock;
+  return 0;
+}
+
+}  // namespace dtas
+
+extern "C" {
+int dtas_add_f16(const void* A, const void* B, void* T, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_ADD_F16, A, B, T, n, H, cfg, stream);
+}
+int dtas_add_f32(const void* A, const void* B, void* T, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_ADD_F32, A, B, T, n, H, cfg, stream);
+}
+int dtas_add_i8(const void* A, const void* B, void* T, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_ADD_I8, A, B, T, n, H, cfg, stream);
+}
+int dtas_copy_f16(const void* A, void* B, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_COPY_F16, A, nullptr, B, n, H, cfg, stream);
+}
+int dtas_copy_f32(const void* A, void* B, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_COPY_F32, A, nullptr, B, n, H, cfg, stream);
+}
+int dtas_copy_i8(const void* A, void* B, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_COPY_I8, A, nullptr, B, n, H, cfg, stream);
+}
+int dtas_cast_f16_f32(const void* A, void* C, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_CAST_F16_F32, A, nullptr, C, n, H, cfg, stream);
+}
+int dtas_cast_f32_f16(const void* A, void* C, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
+  return dtas::run_eltwise(DTAS_OP_CAST_F32_F16, A, nullptr, C, n, H, cfg, stream);
+}
+}

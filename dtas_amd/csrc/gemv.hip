@@ -1,0 +1,156 @@
+// Decode GEMV for gfx950: y[N] = W[N,K] . x[K] (+ bias[N]), fp16 in/out, fp32 accumulate.
+//
+// Replaces the kernel DTAS's GEMV rule generates (python/dtas/schedule/tir_gemv.py:33-249:
+// two-level rfactor split-K over TR lanes x VEC_C elements, weight to registers with vector
+// loads, x staged in shared memory; example output
+// experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:8-92, block 32x16, grid N/16).
+//
+// MI355X shape: a workgroup owns `rows` consecutive rows of W and splits K over all of its
+// lanes and wavefronts: lane t takes the 128-bit chunks t, t+block, ... of every row, so each
+// wavefront access is one contiguous 1 KiB span of a W row and W is streamed from HBM exactly
+// once, non-temporal.  The matching x chunk is loaded once per step and reused for all `rows`
+// rows (x is a few KiB and stays in L2/L1).  fp32 partial sums are folded with DPP inside a
+// wavefront and through one LDS slot per wavefront across them.
+#include "dtas_device.h"
+#include "dtas_host.h"
+
+namespace dtas {
+namespace {
+
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // copy the lanes out first: a bit_cast applied directly to a vector element reads element 0
+    const unsigned ai = a[i], bi = b[i];
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, ai), __builtin_bit_cast(f16x2, bi), acc, false);
+  }
+  return acc;
+}
+
+__device__ __forceinline__ half_t finish(float acc, const half_t* bias, int64_t j) {
+  // round the fp32 sum to fp16 first, then "+ bias" as the PrimFunc's separate fp16 T_add block
+  half_t r = static_cast<half_t>(acc);
+  if (bias) r = static_cast<half_t>(static_cast<float>(r) + static_cast<float>(bias[j]));
+  return r;
+}
+
+template <int R>
+__global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
+                                                          const half_t* __restrict__ bias, half_t* __restrict__ y,
+                                                          int64_t N, int64_t K) {
+  __shared__ float part[8][R];
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+  const int64_t nvec = K >> 3;
+  const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+  const u32x4* wv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    // rows past N re-read the last row; their sums are never stored
+    const int64_t row = row0 + r < N ? row0 + r : N - 1;
+    wv[r] = reinterpret_cast<const u32x4*>(W + row * K);
+  }
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+#pragma unroll 2
+  for (int64_t i = threadIdx.x; i < nvec; i += blockDim.x) {
+    const u32x4 xr = xv[i];
+    u32x4 wr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wr[r] = load_stream(wv[r] + i);
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = dot8(xr, wr[r], acc[r]);
+  }
+
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float s = wave_sum(acc[r]);
+    if ((threadIdx.x & 63) == 0) part[wave][r] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < R && row0 + threadIdx.x < N) {
+    float s = 0.f;
+    for (int w = 0; w < nwaves; ++w) s += part[w][threadIdx.x];
+    y[row0 + threadIdx.x] = finish(s, bias, row0 + threadIdx.x);
+  }
+}
+
+// Any K and any alignment: one wavefront per row, element accesses.
+__global__ void __launch_bounds__(256) gemv_scalar_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
+                                                          const half_t* __restrict__ bias, half_t* __restrict__ y,
+                                                          int64_t N, int64_t K) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= N) return;  // whole wavefronts leave together; no workgroup barrier below
+  const half_t* w = W + row * K;
+  float acc = 0.f;
+  for (int64_t k = threadIdx.x & 63; k < K; k += 64) acc += static_cast<float>(x[k]) * static_cast<float>(w[k]);
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) y[row] = finish(acc, bias, row);
+}
+
+}  // namespace
+
+// launch_args: {grid, 1, 1, block, static LDS bytes, rows per workgroup, 0}
+int describe_gemv(int64_t N, int64_t K, const dtas_config& cfg, int64_t la[7]) {
+  (void)K;
+  for (int i = 0; i < 7; ++i) la[i] = 0;
+  la[1] = la[2] = 1;
+  if (cfg.variant != DTAS_GEMV_SPLITK) return fail("gemv: unknown variant %d", cfg.variant);
+  if (cfg.block < 64 || cfg.block > 512 || cfg.block % 64 != 0)
+    return fail("gemv: block must be a multiple of 64 in [64, 512], got %d", cfg.block);
+  const int rows = cfg.tile[0];
+  if (cfg.vec == 1) {  // element-access fallback: one wavefront per row
+    la[0] = ceil_div(N, 4);
+    la[3] = 256;
+    la[5] = 4;
+    return 0;
+  }
+  if (cfg.vec != 8) return fail("gemv: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+  if (rows != 1 && rows != 2 && rows != 4 && rows != 8) return fail("gemv: rows per workgroup %d not in {1, 2, 4, 8}", rows);
+  la[0] = ceil_div(N, rows);
+  la[3] = cfg.block;
+  la[4] = 8 * rows * 4;
+  la[5] = rows;
+  if (la[0] > 0x7fffffff) return fail("gemv: N=%lld needs too many workgroups", (long long)N);
+  return 0;
+}
+
+}  // namespace dtas
+
+extern "C" int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,
+                             const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (N < 0 || K < 0) return fail("gemv: negative extent N=%lld K=%lld", (long long)N, (long long)K);
+  if (N == 0) return 0;
+  if (K != 0 && N > INT64_MAX / 4 / K) return fail("gemv: N*K overflows");
+  if (!y || (K > 0 && (!x || !W))) return fail("gemv: NULL buffer");
+  if (overlaps(y, N * 2, W, N * K * 2) || overlaps(y, N * 2, x, K * 2)) return fail("gemv: output overlaps an input");
+  dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMV_F16, 1, N, K).cfg;
+  const bool vec_ok = K % 8 == 0 && aligned(x, 16) && aligned(W, 16);
+  if (cfg.vec == 8 && !vec_ok) {
+    if (user) return fail("gemv: 128-bit accesses need K %% 8 == 0 and 16-byte aligned x, W");
+    cfg.vec = 1;
+  }
+  int64_t la[7];
+  if (describe_gemv(N, K, cfg, la) != 0) return -1;
+  const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const half_t* xp = static_cast<const half_t*>(x);
+  const half_t* wp = static_cast<const half_t*>(W);
+  const half_t* bp = static_cast<const half_t*>(bias);
+  half_t* yp = static_cast<half_t*>(y);
+  if (cfg.vec == 1) {
+    hipLaunchKernelGGL(gemv_scalar_kernel, grid, block, 0, s, xp, wp, bp, yp, N, K);
+    return check_launch("gemv");
+  }
+  switch (cfg.tile[0]) {
+    case 1: hipLaunchKernelGGL(gemv_splitk_kernel<1>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
+    case 2: hipLaunchKernelGGL(gemv_splitk_kernel<2>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
+    case 4: hipLaunchKernelGGL(gemv_splitk_kernel<4>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
+    case 8: hipLaunchKernelGGL(gemv_splitk_kernel<8>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
+  }
+  return check_launch("gemv");
+}

@@ -1,0 +1,158 @@
+"""Entry points on torch tensors: each function enqueues one kernel of libdtas_gfx950.so.
+
+Destination passing, as in the reference (``rt_mod["add"](x, y, out)``,
+experiment/dtas_tuned/elementwise/add/profile_add.py:26): the caller allocates every buffer, outputs
+included; nothing is allocated or synchronised here.  Tensors must be contiguous device tensors; the
+kernel goes on torch's current stream.  ``cfg`` (a ``_lib.DtasConfig``) overrides the built-in bucket
+table.  torch is used for device memory and streams only.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import DtasConfig, check, lib
+
+_ELT = {
+    ("add", torch.float16): ("dtas_add_f16", _lib.OP_ADD_F16),
+    ("add", torch.float32): ("dtas_add_f32", _lib.OP_ADD_F32),
+    ("add", torch.int8): ("dtas_add_i8", _lib.OP_ADD_I8),
+    ("copy", torch.float16): ("dtas_copy_f16", _lib.OP_COPY_F16),
+    ("copy", torch.float32): ("dtas_copy_f32", _lib.OP_COPY_F32),
+    ("copy", torch.int8): ("dtas_copy_i8", _lib.OP_COPY_I8),
+}
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("dtas_amd kernels take device tensors; got a CPU tensor (there is no CPU path)")
+        if not t.is_contiguous():
+            raise ValueError("dtas_amd kernels take compact row-major buffers (strides == NULL in the reference)")
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _cfg(cfg: Optional[DtasConfig]):
+    return ctypes.byref(cfg) if cfg is not None else None
+
+
+def _rows_cols(t: torch.Tensor):
+    cols = t.shape[-1] if t.dim() > 0 else 1
+    rows = t.numel() // cols if cols else 0
+    return rows, cols
+
+
+def add(A: torch.Tensor, B: torch.Tensor, T_add: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """T_add = A + B, elementwise, fp16 / fp32 / int8 (int8 wraps)."""
+    _dev(A, B, T_add)
+    if not (A.dtype == B.dtype == T_add.dtype) or not (A.shape == B.shape == T_add.shape):
+        raise ValueError("add: A, B, T_add must agree in dtype and shape")
+    name, _ = _ELT[("add", A.dtype)]
+    n, H = _rows_cols(A)
+    check(getattr(lib(), name)(_p(A), _p(B), _p(T_add), n, H, _cfg(cfg), _stream()), name)
+
+
+def copy(A: torch.Tensor, B: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """B = A, bit for bit."""
+    _dev(A, B)
+    if A.dtype != B.dtype or A.shape != B.shape:
+        raise ValueError("copy: A and B must agree in dtype and shape")
+    name, _ = _ELT[("copy", A.dtype)]
+    n, H = _rows_cols(A)
+    check(getattr(lib(), name)(_p(A), _p(B), n, H, _cfg(cfg), _stream()), name)
+
+
+def cast(A: torch.Tensor, compute: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """compute = Cast(A): fp16 -> fp32 (exact) or fp32 -> fp16 (round to nearest even, overflow to inf)."""
+    _dev(A, compute)
+    if A.shape != compute.shape:
+        raise ValueError("cast: shapes differ")
+    key = (A.dtype, compute.dtype)
+    if key == (torch.float16, torch.float32):
+        name = "dtas_cast_f16_f32"
+    elif key == (torch.float32, torch.float16):
+        name = "dtas_cast_f32_f16"
+    else:
+        raise ValueError(f"cast: no kernel for {A.dtype} -> {compute.dtype}")
+    n, H = _rows_cols(A)
+    check(getattr(lib(), name)(_p(A), _p(compute), n, H, _cfg(cfg), _stream()), name)
+
+
+def layer_norm(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, out: torch.Tensor, eps: float = 1e-5,
+               cfg: Optional[DtasConfig] = None) -> None:
+    """fused_layer_norm_cast1: fp32 x, gamma, beta -> fp16 out, over the last axis."""
+    _dev(x, gamma, beta, out)
+    n, H = _rows_cols(x)
+    if x.dtype != torch.float32 or gamma.dtype != torch.float32 or beta.dtype != torch.float32 or out.dtype != torch.float16:
+        raise ValueError("layer_norm: expects fp32 x/gamma/beta and fp16 out")
+    if out.shape != x.shape or gamma.numel() != H or beta.numel() != H:
+        raise ValueError("layer_norm: shape mismatch")
+    check(lib().dtas_layer_norm_f32_f16(_p(x), _p(gamma), _p(beta), _p(out), n, H, eps, _cfg(cfg), _stream()),
+          "dtas_layer_norm_f32_f16")
+
+
+def rms_norm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float = 1e-5,
+             cfg: Optional[DtasConfig] = None) -> None:
+    """out = x * rsqrt(mean(x^2) + eps) * w over the last axis; fp16 in/out, fp32 arithmetic."""
+    _dev(x, w, out)
+    n, H = _rows_cols(x)
+    if x.dtype != torch.float16 or w.dtype != torch.float16 or out.dtype != torch.float16:
+        raise ValueError("rms_norm: expects fp16 x, w, out")
+    if out.shape != x.shape or w.numel() != H:
+        raise ValueError("rms_norm: shape mismatch")
+    check(lib().dtas_rms_norm_f16(_p(x), _p(w), _p(out), n, H, eps, _cfg(cfg), _stream()), "dtas_rms_norm_f16")
+
+
+def softmax(A: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """fused_softmax_cast: softmax over the last axis, fp32 or fp16 in, fp16 out."""
+    _dev(A, out)
+    if out.dtype != torch.float16 or out.shape != A.shape:
+        raise ValueError("softmax: out must be fp16 with A's shape")
+    rows, cols = _rows_cols(A)
+    if A.dtype == torch.float32:
+        name = "dtas_softmax_f32_f16"
+    elif A.dtype == torch.float16:
+        name = "dtas_softmax_f16"
+    else:
+        raise ValueError(f"softmax: no kernel for {A.dtype}")
+    check(getattr(lib(), name)(_p(A), _p(out), rows, cols, _cfg(cfg), _stream()), name)
+
+
+def gemv(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], y: torch.Tensor,
+         cfg: Optional[DtasConfig] = None) -> None:
+    """y[N] = W[N,K] . x[K] (+ bias[N]); fp16, fp32 accumulate."""
+    _dev(x, W, bias, y)
+    N, K = W.shape
+    if x.numel() != K or y.numel() != N or (bias is not None and bias.numel() != N):
+        raise ValueError("gemv: shape mismatch")
+    if any(t.dtype != torch.float16 for t in (x, W, y)) or (bias is not None and bias.dtype != torch.float16):
+        raise ValueError("gemv: expects fp16 tensors")
+    check(lib().dtas_gemv_f16(_p(x), _p(W), _p(bias), _p(y), N, K, _cfg(cfg), _stream()), "dtas_gemv_f16")
+
+
+def gemm(A: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], C: torch.Tensor,
+         cfg: Optional[DtasConfig] = None) -> None:
+    """C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]); fp16, fp32 accumulate on MFMA.  M is every leading
+    extent of A flattened."""
+    _dev(A, W, bias, C)
+    N, K = W.shape
+    if A.shape[-1] != K or C.shape[-1] != N:
+        raise ValueError("gemm: inner extents differ")
+    M = A.numel() // K if K else C.numel() // max(N, 1)
+    if C.numel() != M * N or (bias is not None and bias.numel() != N):
+        raise ValueError("gemm: shape mismatch")
+    if any(t.dtype != torch.float16 for t in (A, W, C)) or (bias is not None and bias.dtype != torch.float16):
+        raise ValueError("gemm: expects fp16 tensors")
+    check(lib().dtas_gemm_f16(_p(A), _p(W), _p(bias), _p(C), M, N, K, _cfg(cfg), _stream()), "dtas_gemm_f16")

@@ -1,0 +1,31 @@
+"""Launch candidates for the decode GEMV.
+
+The reference's GEMVConfigEmiter.emit_config is an unfinished stub that returns no candidates
+(python/dtas/policy/gemv_config_emiter.py:26-30); its GEMV experiments used the GEMVConfig defaults
+(block 32x16, grid N/16, python/dtas/common/config.py:339-356).  Here the candidates are rows of W per
+workgroup x threads splitting K, ranked so that every CU holds at least ~4 workgroups.
+"""
+from typing import List, Tuple
+
+from ..common.config import GEMVConfig, Range
+from .base_config_emiter import BaseConfigEmiter
+
+
+class GEMVConfigEmiter(BaseConfigEmiter):
+    def emit_config(self, range_tuple: Tuple[Range, ...], topk: int = 20) -> List[GEMVConfig]:
+        N, K = self.func_info.func.params[1].shape
+        out = []
+        for rows in (1, 2, 4, 8):
+            for threads in (256, 128, 512):
+                if threads * 8 > max(K, 512):
+                    continue
+                c = GEMVConfig()
+                c.TILE_S, c.TR = rows, threads
+                out.append(c)
+        want = 4 * self.arch.num_sm
+
+        def score(c: GEMVConfig):
+            groups = -(-N // c.TILE_S)
+            return (groups < want, -c.TILE_S if groups >= want else c.TILE_S, c.TR != 256)
+
+        return sorted(out, key=score)[:topk]

@@ -1,0 +1,134 @@
+"""Launch candidates for row reductions (layer norm, RMS norm, softmax).
+
+The occupancy arithmetic is the reference's ReductionConfigEmiter (python/dtas/policy/
+reduction_config_emiter.py:39-158): workgroup sizes warp*partition, +warp, ... while <= 1024 and <=
+row length; ``max_active = min(tpm // tx, [smem_sm // smem_row,] max_blocks)``; rows map 1:1 to
+workgroups unless there are more rows than ``num_sm * max_active * 32``; candidates sorted by
+(max_active, tx, vec) descending.  For ROCm the candidate set is the three gfx950 kernels instead:
+"local" (one wavefront per row, row in registers), "shared.dyn" (one workgroup per row) and "cache"
+(row re-read per pass), each only where its register budget holds the row.
+"""
+from typing import List, Optional, Tuple
+
+from ..common.config import Range, ReductionConfig, Var
+from .base_config_emiter import BaseConfigEmiter, dtype_bits
+
+
+class ReductionConfigEmiter(BaseConfigEmiter):
+    # the reference hard-wires "cache" (:85); its layer-norm artefacts came from "shared.dyn"
+    cuda_temp_storage = "cache"
+    # bytes of shared memory one row needs in "shared.dyn" mode; None = (row + 2) * bytes (:79)
+    cuda_smem_usage: Optional[int] = None
+
+    def plan_vectorize(self, re_range: Range, in_bytes: int, is_dynamic_reduction: bool = False):
+        def allowed(vec: int) -> bool:
+            bits = in_bytes * 8 * vec
+            if in_bytes == 2:
+                return vec % 2 == 0 and 32 <= bits <= 128
+            return 32 <= bits <= 128
+
+        valid = [v for v in (16, 8, 4, 3, 2, 1) if allowed(v)]
+        if is_dynamic_reduction:
+            return valid[0]
+        for vec in valid:
+            if re_range.end % vec == 0:
+                return vec
+        return None
+
+    def get_unroll_depth(self):
+        return 256
+
+    def get_num_blocks(self, config: ReductionConfig, row_range: Range, max_smem_usage: int, use_shared: bool = True,
+                       waves: int = 32) -> None:
+        limits = [self.arch.max_resident_threads_per_sm // config.len_tx, self.arch.max_resident_blocks_per_sm]
+        if use_shared:
+            limits.append(self.arch.max_smem_per_sm // max_smem_usage)
+        config.max_active_blocks_per_sm = min(limits)
+        max_blocks = self.arch.num_sm * config.max_active_blocks_per_sm * waves
+        if max_blocks >= row_range.start:
+            config.bx_factor, config.bx = 1, None
+        else:
+            config.bx, config.bx_factor = max(1, max_blocks), None
+
+    def generate_config_candidates(self, re_range: Range, row_range: Range, in_bytes: int,
+                                   is_dynamic_reduction: bool = False, topk: int = 20) -> List[ReductionConfig]:
+        if self.arch.platform != "CUDA":
+            return self._gfx950_candidates(re_range, row_range, in_bytes, topk)
+        max_smem_usage = self.cuda_smem_usage or (re_range.end + 2) * in_bytes
+        temp_storage = self.cuda_temp_storage
+        vec = self.plan_vectorize(re_range, in_bytes) if temp_storage == "shared.dyn" else None
+        configs = []
+        block = self.arch.warp_size * self.arch.sm_partition
+        while block <= self.arch.max_threads_per_block and block <= re_range.end:
+            c = ReductionConfig()
+            c.unroll_depth = self.get_unroll_depth()
+            c.temp_storage = temp_storage
+            c.len_tx = block
+            self.get_num_blocks(c, row_range, max_smem_usage, temp_storage == "shared.dyn", 32)
+            if vec is not None:
+                c.vector_size = vec
+            configs.append(c)
+            block += self.arch.warp_size
+        if len(configs) >= topk:
+            return sorted(configs, key=lambda c: (c.max_active_blocks_per_sm, c.len_tx, c.vector_size), reverse=True)[:topk]
+        return configs
+
+    def _gfx950_candidates(self, re_range: Range, row_range: Range, in_bytes: int, topk: int) -> List[ReductionConfig]:
+        vec = 16 // in_bytes
+        nvec = -(-re_range.end // vec)
+        many_rows = row_range.start > 2 * self.arch.num_sm
+        out: List[ReductionConfig] = []
+
+        def cand(storage: str, tx: int) -> ReductionConfig:
+            c = ReductionConfig()
+            c.temp_storage, c.len_tx, c.vector_size, c.unroll_depth = storage, tx, vec, 1
+            self.get_num_blocks(c, row_range, 64, storage == "shared.dyn", 32)
+            c.bx = None  # rows map 1:1 to wavefronts / workgroups; the kernels stride if capped
+            return c
+
+        wave_rows = [cand("local", tx) for tx in (256, 128, 512, 64)] if nvec <= 64 * 16 else []
+        block_rows = []
+        for tx in (256, 512, 1024, 128):
+            if tx * 16 >= nvec and tx <= max(64, nvec):
+                block_rows.append(cand("shared.dyn", tx))
+        # few rows: a workgroup per row first; many rows: a wavefront per row first
+        out = (wave_rows + block_rows) if many_rows else (block_rows + wave_rows)
+        stream = cand("cache", 1024 if re_range.end >= 4096 else 256)
+        stream.vector_size = 1
+        out.append(stream)
+        return out[:topk]
+
+    def emit_config(self, range_tuple: Tuple[Range, ...], topk: int = 20) -> List[ReductionConfig]:
+        re_len = self.func_info.red_len
+        rows = self.func_info.rows
+        re_range = None
+        row_range = None
+        if self.func_info.dyn_red:
+            for r in range_tuple:
+                if re_range is None and r.var.name == re_len.name:
+                    re_range = r
+                    # an extent that is both a row factor and the row length ([heads*n, n])
+                    if self._also_row_factor(r):
+                        row_range = self._scale(row_range, r, rows)
+                else:
+                    row_range = self._scale(row_range, r, rows)
+            if re_range is None:
+                raise ValueError("reduction_len is dynamic, but can't find reduction range info in range_tuple")
+        else:
+            re_range = Range(Var("re_len"), re_len, re_len)
+            for r in range_tuple:
+                row_range = self._scale(row_range, r, rows)
+        if row_range is None:
+            row_range = Range("row_range", rows, rows)
+        in_bytes = (dtype_bits(self.func_info.in_dtype) + 7) // 8
+        return self.generate_config_candidates(re_range, row_range, in_bytes, self.func_info.dyn_red, topk)
+
+    def _also_row_factor(self, r: Range) -> bool:
+        shape = self.func_info.func.params[0].shape
+        return any(e == r.var.name for e in shape[:-1])
+
+    @staticmethod
+    def _scale(row_range: Optional[Range], r: Range, rows: int) -> Range:
+        if row_range is None:
+            return Range("row_range", r.start * rows, r.end * rows)
+        return Range("row_range", row_range.start * r.start, row_range.end * r.end)

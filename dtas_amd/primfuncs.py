@@ -1,0 +1,128 @@
+"""The PrimFunc signatures the kernels stand behind, as ``PrimFunc`` descriptors.
+
+Each constructor cites the TVMScript it restates (paths relative to the reference checkout).
+Parameter order and the destination-passing convention (output buffer last) are the reference's;
+the hidden size and the static matmul extents are arguments because the benchmark configs use
+4096-wide shapes where the reference's model uses 2560.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+from .common.analisys import Block, Buffer, IRModule, PrimFunc
+
+
+def add(dtype: str = "float16", hidden: int = 2560) -> PrimFunc:
+    """T_add = A + B over (1, n, hidden): tuning_test/tune_ele_add.py:10-22 (committed as int8;
+    fp16 / fp32 artefacts under experiment/dtas_tuned/elementwise/add/)."""
+    shape = (1, "n", hidden)
+    return PrimFunc("add", [Buffer("A", shape, dtype), Buffer("B", shape, dtype), Buffer("T_add", shape, dtype)],
+                    [Block("T_add", "SSS", ["A", "B"], ["T_add"])], op="add",
+                    attrs={"op_pattern": 0, "tir.noalias": True})
+
+
+def copy(dtype: str = "float32", hidden: int = 2560) -> PrimFunc:
+    """B = A over (1, n, hidden): tuning_test/tune_ele_copy.py:10-21."""
+    shape = (1, "n", hidden)
+    return PrimFunc("copy", [Buffer("A", shape, dtype), Buffer("B", shape, dtype)],
+                    [Block("B", "SSS", ["A"], ["B"])], op="copy", attrs={"tir.noalias": True})
+
+
+def cast(src: str = "float16", dst: str = "float32", hidden: int = 2560) -> PrimFunc:
+    """compute = Cast(dst, A) over (1, n, hidden): tuning_test/tune_cast.py:10-21 (fp16 -> fp32)."""
+    shape = (1, "n", hidden)
+    return PrimFunc("cast", [Buffer("A", shape, src), Buffer("compute", shape, dst)],
+                    [Block("compute", "SSS", ["A"], ["compute"])], op="cast", attrs={"tir.noalias": True})
+
+
+def fused_layer_norm_cast1(hidden: int = 2560) -> PrimFunc:
+    """LayerNorm fp32 -> fp16 with gamma/beta: experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:607-636."""
+    return PrimFunc(
+        "fused_layer_norm_cast1",
+        [Buffer("lv6", (1, "n", hidden), "float32"), Buffer("param_1", (hidden,), "float32"),
+         Buffer("param_2", (hidden,), "float32"), Buffer("compute_intermediate", (1, "n", hidden), "float16")],
+        [Block("A_red_temp", "SSR", ["lv6"], ["A_red_temp_v0", "A_red_temp_v1"]),
+         Block("T_layer_norm", "SSS", ["lv6", "A_red_temp_v0", "A_red_temp_v1", "param_1", "param_2"],
+               ["T_layer_norm_intermediate"]),
+         Block("compute", "SSS", ["T_layer_norm_intermediate"], ["compute_intermediate"])],
+        op="layer_norm", attrs={"tir.noalias": True, "eps": 1e-5})
+
+
+def rms_norm(hidden: int = 4096, eps: float = 1e-5) -> PrimFunc:
+    """RMSNorm fp16 with fp16 weight; no counterpart in the reference (the benchmark's norm)."""
+    return PrimFunc(
+        "rms_norm",
+        [Buffer("x", ("n", hidden), "float16"), Buffer("weight", (hidden,), "float16"),
+         Buffer("out", ("n", hidden), "float16")],
+        [Block("sum_sq", "SR", ["x"], ["sum_sq"]), Block("norm", "SS", ["x", "sum_sq", "weight"], ["out"])],
+        op="rms_norm", attrs={"tir.noalias": True, "eps": eps})
+
+
+def fused_softmax_cast(rows: int = 1000, dtype: str = "float32") -> PrimFunc:
+    """Softmax over the dynamic last axis of (1, rows, n), fp16 out:
+    experiment/dtas_tuned/general_reduction/softmax/profile_dlight.py:8-52."""
+    return PrimFunc(
+        "fused_softmax_cast",
+        [Buffer("A", (1, rows, "n"), dtype), Buffer("compute_intermediate", (1, rows, "n"), "float16")],
+        _softmax_blocks("A"), op="softmax", attrs={"tir.noalias": True})
+
+
+def fused_softmax_cast3(heads: int = 32, dtype: str = "float32") -> PrimFunc:
+    """Softmax over m of (1, heads, n, m), fp16 out: before_dl.py:756-800 (two dynamic extents)."""
+    return PrimFunc(
+        "fused_softmax_cast3",
+        [Buffer("lv38", (1, heads, "n", "m"), dtype), Buffer("compute_intermediate", (1, heads, "n", "m"), "float16")],
+        _softmax_blocks("lv38"), op="softmax", attrs={"tir.noalias": True})
+
+
+def softmax_scores(heads: int = 32) -> PrimFunc:
+    """The benchmark's attention-score softmax: fp16 [heads*n, n] -> fp16, one dynamic extent n
+    that is both the row count factor and the row length."""
+    return PrimFunc(
+        "softmax_scores",
+        [Buffer("scores", (heads, "n", "n"), "float16"), Buffer("out", (heads, "n", "n"), "float16")],
+        _softmax_blocks("scores"), op="softmax", attrs={"tir.noalias": True})
+
+
+def _softmax_blocks(src: str):
+    return [Block("T_softmax_maxelem", "SSR", [src], ["T_softmax_maxelem"]),
+            Block("T_softmax_exp", "SSS", [src, "T_softmax_maxelem"], ["T_softmax_exp"]),
+            Block("T_softmax_expsum", "SSR", ["T_softmax_exp"], ["T_softmax_expsum"]),
+            Block("T_softmax_norm", "SSS", ["T_softmax_exp", "T_softmax_expsum"], ["T_softmax_norm"]),
+            Block("compute", "SSS", ["T_softmax_norm"], ["compute_intermediate"])]
+
+
+def fused_NT_matmul_add_gemv(N: int = 2560, K: int = 10240, bias: bool = True,
+                             name: Optional[str] = None) -> PrimFunc:
+    """y(1,1,N) = x(1,1,K) . W(N,K)^T (+ bias): fused_NT_matmul10_add5, before_dl.py:96-113."""
+    params = [Buffer("lv1825", (1, 1, K), "float16"), Buffer("param_1110", (N, K), "float16")]
+    blocks = [Block("NT_matmul", "SSSR", ["lv1825", "param_1110"], ["NT_matmul_intermediate"])]
+    if bias:
+        params.append(Buffer("param_1210", (N,), "float16"))
+        blocks.append(Block("T_add", "SSS", ["NT_matmul_intermediate", "param_1210"], ["T_add_intermediate"]))
+    params.append(Buffer("T_add_intermediate", (1, 1, N), "float16"))
+    return PrimFunc(name or ("fused_NT_matmul10_add5" if bias else "NT_matmul10"), params, blocks, op="matmul",
+                    attrs={"tir.noalias": True})
+
+
+def fused_NT_matmul_add_gemm(N: int = 2560, K: int = 10240, bias: bool = True,
+                             name: Optional[str] = None) -> PrimFunc:
+    """C(1,n,N) = A(1,n,K) . W(N,K)^T (+ bias), n dynamic: fused_NT_matmul4_add1, before_dl.py:320-341."""
+    params = [Buffer("lv55", (1, "n", K), "float16"), Buffer("param_11", (N, K), "float16")]
+    blocks = [Block("NT_matmul", "SSSR", ["lv55", "param_11"], ["NT_matmul_intermediate"])]
+    if bias:
+        params.append(Buffer("param_12", (N,), "float16"))
+        blocks.append(Block("T_add", "SSS", ["NT_matmul_intermediate", "param_12"], ["T_add_intermediate"]))
+    params.append(Buffer("T_add_intermediate", (1, "n", N), "float16"))
+    return PrimFunc(name or ("fused_NT_matmul4_add1" if bias else "NT_matmul4"), params, blocks, op="matmul",
+                    attrs={"tir.noalias": True})
+
+
+def module(*funcs: PrimFunc, upper_bound: Optional[dict] = None) -> IRModule:
+    """An IRModule of the given PrimFuncs; ``upper_bound`` is the ``tir_var_upper_bound`` attribute
+    (tuning_test/tune_cast.py:26 uses {"m": 512, "n": 4096})."""
+    attrs = {"tir_var_upper_bound": dict(upper_bound)} if upper_bound else {}
+    for f in funcs:
+        if upper_bound:
+            f.attrs.setdefault("tir_var_upper_bound", dict(upper_bound))
+    return IRModule(list(funcs), attrs)

@@ -1,0 +1,177 @@
+/*
+ * dtas_abi.h -- C ABI of libdtas_gfx950.so: hand-written gfx950 (MI355X) kernels for
+ * the PrimFuncs that DTAS's schedule rules cover, behind one shape-bucket dispatcher.
+ *
+ * What this replaces in the reference (paths relative to the reference checkout):
+ * DTAS emits, per PrimFunc, one TVM PackedFunc host function
+ *     int32_t <func>(void* args, int32_t* arg_type_ids, int32_t num_args, ...)
+ * (experiment/dtas_tuned/elementwise/add/float16/top1_256/host.cc:38-145) that unpacks
+ * DLTensor handles, reads the dynamic extent n from shape[1], looks up
+ * call_table[index_table[min(n/div, last)]] and launches the bucket's kernel with
+ * launch_args = {grid, block[, dyn smem]} through TVM's CUDA module.  Each entry
+ * point below is that host function with the DLTensor unpacking already done: plain
+ * device pointers and extents in, 0 / -1 out.  The kernel behind it is the replacement
+ * for the bucket kernels *_n_<lo>_to_<hi>__kernel in tvm_device_kernels.cu.
+ *
+ * Conventions (all entry points):
+ *  - destination passing: the caller owns every buffer, outputs included
+ *    (experiment/dtas_tuned/elementwise/cast/profile_cast.py:15-18);
+ *  - buffers are compact row-major, as the reference requires (strides == NULL,
+ *    host.cc:64-69); the leading batch-1 dim of (1, n, H) is not passed;
+ *  - `stream` is a hipStream_t (NULL = the default stream); nothing is allocated, nothing
+ *    synchronises, the kernel is enqueued on `stream` on the current device;
+ *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
+ *    reference's call_table holds); NULL = use the library's built-in bucket table;
+ *  - returns 0 on success, -1 on error (the reference's host functions do the same,
+ *    host.cc:75-83,133-143); dtas_last_error() gives the thread-local message;
+ *  - n == 0 (an empty dynamic extent) is a no-op that returns 0; negative extents, NULL
+ *    buffers with n > 0 and overlapping in/out buffers ("tir.noalias") are errors.
+ */
+#ifndef DTAS_ABI_H_
+#define DTAS_ABI_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DTAS_ABI_VERSION 1
+
+/* ---- op families = the reference's FuncKind (python/dtas/common/analisys.py:49-55) */
+enum dtas_kind {
+  DTAS_KIND_ELEMENTWISE = 0,
+  DTAS_KIND_REDUCTION = 1,
+  DTAS_KIND_GEMV = 2,
+  DTAS_KIND_GEMM = 3
+};
+
+/* ---- ops (one per PrimFunc / dtype combination with its own kernel set) */
+enum dtas_op {
+  DTAS_OP_ADD_F16 = 0,
+  DTAS_OP_ADD_F32,
+  DTAS_OP_ADD_I8,
+  DTAS_OP_COPY_F16,
+  DTAS_OP_COPY_F32,
+  DTAS_OP_COPY_I8,
+  DTAS_OP_CAST_F16_F32,
+  DTAS_OP_CAST_F32_F16,
+  DTAS_OP_LAYER_NORM_F32_F16,
+  DTAS_OP_RMS_NORM_F16,
+  DTAS_OP_SOFTMAX_F32_F16,
+  DTAS_OP_SOFTMAX_F16,
+  DTAS_OP_GEMV_F16,
+  DTAS_OP_GEMM_F16,
+  DTAS_OP_COUNT
+};
+
+/* ---- kernel variants (the `variant` field of dtas_config) */
+enum dtas_variant {
+  /* elementwise (python/dtas/schedule/tir_elementwise.py:23-47) */
+  DTAS_ELT_VECTOR = 0,    /* `vec`-wide accesses, `unroll` in flight per thread, grid-stride */
+  DTAS_ELT_SCALAR = 1,    /* one element per access: any alignment */
+  /* row reductions (python/dtas/schedule/tir_reduction.py:36-105) */
+  DTAS_RED_WAVE_ROW = 0,  /* one wavefront per row, row held in registers, DPP reduction */
+  DTAS_RED_BLOCK_ROW = 1, /* one workgroup per row, row in registers, DPP + LDS staging */
+  DTAS_RED_STREAM_ROW = 2,/* one workgroup per row, row re-read per pass: any length / alignment */
+  /* GEMV (python/dtas/schedule/tir_gemv.py:33-249) */
+  DTAS_GEMV_SPLITK = 0,   /* K split over the lanes and wavefronts of a workgroup */
+  /* GEMM (python/dtas/schedule/tir_wmma.py:20-222) */
+  DTAS_GEMM_MFMA = 0,     /* LDS-tiled MFMA, tile = tile[0] x tile[1] x tile[2] */
+  DTAS_GEMM_SKINNY = 1    /* small M: weight-streaming MFMA 16x16x32, split over N and K */
+};
+
+/* One row of a call table: the launch-relevant part of the reference's *Config classes
+ * (python/dtas/common/config.py:193-429: ElementwiseConfig{len_tx, vector_size, grid_size},
+ * ReductionConfig{len_tx, vector_size, temp_storage}, GEMVConfig{TS, TR, TILE_R, VEC_C},
+ * WMMAConfig{i, j, micro_shape}). */
+typedef struct dtas_config {
+  int32_t variant;  /* enum dtas_variant of the op's family */
+  int32_t block;    /* threads per workgroup = launch_args[1] */
+  int32_t vec;      /* elements per vector access */
+  int32_t unroll;   /* independent vector accesses in flight per thread / rows per wavefront */
+  int32_t tile[3];  /* GEMM: workgroup tile M, N, K; GEMV: rows per workgroup, -, - */
+  int32_t split_k;  /* GEMV/GEMM: number of K partitions (1 = none) */
+  int64_t grid_cap; /* upper limit on workgroups (then the kernel loops); 0 = no limit */
+} dtas_config;
+
+/* What the dispatcher decided for one call: the analogue of
+ * `kernel_entry_info info = call_table[index_table[index]]` (host.cc:105-125,
+ * python/dtas/codegen/runtime_packer.py:32-40). */
+typedef struct dtas_launch_info {
+  int64_t launch_args[7]; /* grid.x, grid.y, grid.z, block.x, dynamic LDS bytes, 0, 0 */
+  int64_t bucket_lo;      /* the merged bucket [lo, hi] of the dynamic extent that n fell in */
+  int64_t bucket_hi;
+  int32_t index;          /* min((n - 1) / range_div, last): position in the index table */
+  int32_t table_row;      /* index_table[index] */
+  dtas_config config;
+  char name[96];          /* "<func>_<var>_<lo>_to_<hi>__kernel" (python/dtas/common/config.py:28-31) */
+} dtas_launch_info;
+
+/* ---- library ------------------------------------------------------------ */
+int dtas_abi_version(void);
+/* Thread-local text of the last error on this thread ("" if none). */
+const char* dtas_last_error(void);
+/* Checks that the current device is a gfx950 part and warms the kernel images. */
+int dtas_init(void);
+
+/* The built-in bucket table: which config a call with these extents uses.
+ * n = the dynamic extent (rows n; softmax: cols when dynamic; GEMM: M), d0/d1 = static extents
+ * (elementwise/norm: H, 0; softmax: rows, cols; GEMV: N, K; GEMM: N, K). */
+int dtas_select_bucket(int op, int64_t n, int64_t d0, int64_t d1, dtas_launch_info* out);
+/* Resolve launch_args for an explicit config (used by tuners to inspect candidates). */
+int dtas_describe_launch(int op, int64_t n, int64_t d0, int64_t d1, const dtas_config* cfg,
+                         dtas_launch_info* out);
+
+/* ---- elementwise: tuning_test/tune_ele_add.py:10-22, tune_ele_copy.py:10-21,
+ *      tune_cast.py:10-21; dtype variants under experiment/dtas_tuned/elementwise/ ------- */
+/* T_add[n,H] = A[n,H] + B[n,H] */
+int dtas_add_f16(const void* A, const void* B, void* T_add, int64_t n, int64_t H,
+                 const dtas_config* cfg, void* stream);
+int dtas_add_f32(const void* A, const void* B, void* T_add, int64_t n, int64_t H,
+                 const dtas_config* cfg, void* stream);
+int dtas_add_i8(const void* A, const void* B, void* T_add, int64_t n, int64_t H,
+                const dtas_config* cfg, void* stream);
+/* B[n,H] = A[n,H], bit for bit */
+int dtas_copy_f16(const void* A, void* B, int64_t n, int64_t H, const dtas_config* cfg, void* stream);
+int dtas_copy_f32(const void* A, void* B, int64_t n, int64_t H, const dtas_config* cfg, void* stream);
+int dtas_copy_i8(const void* A, void* B, int64_t n, int64_t H, const dtas_config* cfg, void* stream);
+/* compute[n,H] = Cast(A[n,H]): fp16 -> fp32 is the reference's direction, fp32 -> fp16 the
+ * narrowing one (round to nearest even, overflow to +-inf) */
+int dtas_cast_f16_f32(const void* A, void* compute, int64_t n, int64_t H, const dtas_config* cfg,
+                      void* stream);
+int dtas_cast_f32_f16(const void* A, void* compute, int64_t n, int64_t H, const dtas_config* cfg,
+                      void* stream);
+
+/* ---- row reductions ------------------------------------------------------ */
+/* fused_layer_norm_cast1 (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:607-636):
+ * x fp32 [n,H], gamma/beta fp32 [H] -> out fp16 [n,H]; eps is 1e-5 in the PrimFunc. */
+int dtas_layer_norm_f32_f16(const void* x, const void* gamma, const void* beta, void* out,
+                            int64_t n, int64_t H, float eps, const dtas_config* cfg, void* stream);
+/* RMSNorm (no PrimFunc in the reference; the benchmark's norm): x fp16 [n,H], w fp16 [H]
+ * -> out fp16 [n,H] = x * rsqrt(mean(x^2) + eps) * w, fp32 arithmetic. */
+int dtas_rms_norm_f16(const void* x, const void* w, void* out, int64_t n, int64_t H, float eps,
+                      const dtas_config* cfg, void* stream);
+/* fused_softmax_cast (experiment/dtas_tuned/general_reduction/softmax/profile_dlight.py:8-52,
+ * before_dl.py:756-800): softmax over the last axis of A[rows, cols], fp32 math, fp16 out.
+ * The (1,32,n,m) form is rows = 32*n, cols = m. */
+int dtas_softmax_f32_f16(const void* A, void* out, int64_t rows, int64_t cols,
+                         const dtas_config* cfg, void* stream);
+int dtas_softmax_f16(const void* A, void* out, int64_t rows, int64_t cols, const dtas_config* cfg,
+                     void* stream);
+
+/* ---- GEMV: fused_NT_matmul10_add5 (before_dl.py:96-113) ------------------
+ * y[N] = W[N,K] . x[K] (+ bias[N] when bias != NULL); fp16 in/out, fp32 accumulate. */
+int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,
+                  const dtas_config* cfg, void* stream);
+
+/* ---- GEMM: fused_NT_matmul4_add1 (before_dl.py:320-341) -------------------
+ * C[M,N] = A[M,K] . W[N,K]^T (+ bias[N] when bias != NULL); M is the dynamic extent;
+ * fp16 in/out, fp32 accumulate on MFMA. */
+int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N,
+                  int64_t K, const dtas_config* cfg, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DTAS_ABI_H_ */

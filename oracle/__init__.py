@@ -1,0 +1,191 @@
+"""CPU oracle for the DTAS hot path -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+Two independent restatements of the PrimFunc math:
+
+* ``oracle.c``   -- ctypes bindings of ``cpu_ref.c`` (literal loop nests, fp32 / fp16
+  arithmetic as the PrimFunc text states; also timed as the CPU baseline);
+* ``oracle.np64`` -- closed forms in numpy float64 (the tolerance anchor that pins
+  ``cpu_ref.c`` and the GPU kernels alike).
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py``
+import this package.  The product (``dtas_amd``) never does.
+
+The reference holds no numerical tests or golden vectors for this path, so each
+function is pinned by closed forms, library routines, exhaustive enumeration and
+invariants (``tests/test_oracle_*.py``).  ``rms_norm`` has no counterpart in the
+reference at all: parity unpinned by the reference, closed form only.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libdtas_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile cpu_ref.c into libdtas_oracle.so (gcc, a second or two)."""
+    src = os.path.join(_HERE, "cpu_ref.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-B", "-C", _HERE, "libdtas_oracle.so"])
+    return _SO
+
+
+def _ptr(a: np.ndarray):
+    assert a.flags["C_CONTIGUOUS"], "oracle takes C-contiguous arrays"
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+class _C:
+    """Lazy ctypes view of libdtas_oracle.so."""
+
+    _lib = None
+
+    @classmethod
+    def lib(cls):
+        if cls._lib is None:
+            if not os.path.exists(_SO):
+                build()
+            lib = ctypes.CDLL(_SO)
+            vp, i64, ci, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+            sig = {
+                "oracle_add_f16": [vp, vp, vp, i64, ci],
+                "oracle_add_f32": [vp, vp, vp, i64, ci],
+                "oracle_add_i8": [vp, vp, vp, i64, ci],
+                "oracle_copy_bytes": [vp, vp, i64, ci],
+                "oracle_cast_f16_f32": [vp, vp, i64, ci],
+                "oracle_cast_f32_f16": [vp, vp, i64, ci],
+                "oracle_layer_norm_f32_f16": [vp, vp, vp, vp, i64, i64, f32, ci],
+                "oracle_rms_norm_f16": [vp, vp, vp, i64, i64, f32, ci],
+                "oracle_softmax_f32_f16": [vp, vp, i64, i64, ci],
+                "oracle_softmax_f16_f16": [vp, vp, i64, i64, ci],
+                "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
+                "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
+            }
+            for name, argtypes in sig.items():
+                fn = getattr(lib, name)
+                fn.argtypes = argtypes
+                fn.restype = None
+            lib.oracle_soft_h2f.argtypes = [ctypes.c_uint16]
+            lib.oracle_soft_h2f.restype = ctypes.c_float
+            lib.oracle_soft_f2h.argtypes = [ctypes.c_float]
+            lib.oracle_soft_f2h.restype = ctypes.c_uint16
+            lib.oracle_max_threads.argtypes = []
+            lib.oracle_max_threads.restype = ctypes.c_int
+            cls._lib = lib
+        return cls._lib
+
+
+class c:  # noqa: N801  (namespace, mirrors the C file)
+    """cpu_ref.c through ctypes.  Arrays in, new array out; ``threads`` splits rows."""
+
+    @staticmethod
+    def max_threads() -> int:
+        return int(_C.lib().oracle_max_threads())
+
+    @staticmethod
+    def add(a: np.ndarray, b: np.ndarray, threads: int = 1) -> np.ndarray:
+        assert a.dtype == b.dtype and a.shape == b.shape
+        out = np.empty_like(a)
+        fn = {"float16": "oracle_add_f16", "float32": "oracle_add_f32", "int8": "oracle_add_i8"}[a.dtype.name]
+        getattr(_C.lib(), fn)(_ptr(a), _ptr(b), _ptr(out), a.size, threads)
+        return out
+
+    @staticmethod
+    def copy(a: np.ndarray, threads: int = 1) -> np.ndarray:
+        out = np.empty_like(a)
+        _C.lib().oracle_copy_bytes(_ptr(a), _ptr(out), a.nbytes, threads)
+        return out
+
+    @staticmethod
+    def cast(a: np.ndarray, dtype: str, threads: int = 1) -> np.ndarray:
+        out = np.empty(a.shape, dtype=dtype)
+        key = (a.dtype.name, np.dtype(dtype).name)
+        fn = {("float16", "float32"): "oracle_cast_f16_f32", ("float32", "float16"): "oracle_cast_f32_f16"}[key]
+        getattr(_C.lib(), fn)(_ptr(a), _ptr(out), a.size, threads)
+        return out
+
+    @staticmethod
+    def layer_norm(x, gamma, beta, eps: float = 1e-5, threads: int = 1) -> np.ndarray:
+        assert x.dtype == np.float32 and gamma.dtype == np.float32 and beta.dtype == np.float32
+        H = x.shape[-1]
+        out = np.empty(x.shape, dtype=np.float16)
+        _C.lib().oracle_layer_norm_f32_f16(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.size // H, H, eps, threads)
+        return out
+
+    @staticmethod
+    def rms_norm(x, w, eps: float = 1e-5, threads: int = 1) -> np.ndarray:
+        assert x.dtype == np.float16 and w.dtype == np.float16
+        H = x.shape[-1]
+        out = np.empty_like(x)
+        _C.lib().oracle_rms_norm_f16(_ptr(x), _ptr(w), _ptr(out), x.size // H, H, eps, threads)
+        return out
+
+    @staticmethod
+    def softmax(x, threads: int = 1) -> np.ndarray:
+        cols = x.shape[-1]
+        out = np.empty(x.shape, dtype=np.float16)
+        fn = {"float16": "oracle_softmax_f16_f16", "float32": "oracle_softmax_f32_f16"}[x.dtype.name]
+        getattr(_C.lib(), fn)(_ptr(x), _ptr(out), x.size // max(cols, 1), cols, threads)
+        return out
+
+    @staticmethod
+    def gemm(a, w, bias=None, acc_f16: bool = False, threads: int = 1) -> np.ndarray:
+        """C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]); GEMV is M == 1."""
+        assert a.dtype == np.float16 and w.dtype == np.float16
+        K = a.shape[-1]
+        M, N = a.size // K, w.shape[0]
+        assert w.shape == (N, K)
+        out = np.empty(a.shape[:-1] + (N,), dtype=np.float16)
+        bp = _ptr(bias) if bias is not None else None
+        _C.lib().oracle_gemm_f16(_ptr(a), _ptr(w), bp, _ptr(out), M, N, K, int(acc_f16), threads)
+        return out
+
+    @staticmethod
+    def gemm_f32out(a, w, threads: int = 1) -> np.ndarray:
+        K = a.shape[-1]
+        M, N = a.size // K, w.shape[0]
+        out = np.empty(a.shape[:-1] + (N,), dtype=np.float32)
+        _C.lib().oracle_gemm_f16_f32out(_ptr(a), _ptr(w), _ptr(out), M, N, K, threads)
+        return out
+
+    @staticmethod
+    def soft_h2f(bits: int) -> float:
+        return float(_C.lib().oracle_soft_h2f(bits))
+
+    @staticmethod
+    def soft_f2h(v: float) -> int:
+        return int(_C.lib().oracle_soft_f2h(ctypes.c_float(v)))
+
+
+class np64:  # noqa: N801
+    """Closed forms in float64 -- independent of cpu_ref.c; the tolerance anchor."""
+
+    @staticmethod
+    def layer_norm(x, gamma, beta, eps=1e-5):
+        x = x.astype(np.float64)
+        mean = x.mean(-1, keepdims=True)
+        var = (x * x).mean(-1, keepdims=True) - mean * mean
+        return (x - mean) / np.sqrt(var + eps) * gamma.astype(np.float64) + beta.astype(np.float64)
+
+    @staticmethod
+    def rms_norm(x, w, eps=1e-5):
+        x = x.astype(np.float64)
+        return x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * w.astype(np.float64)
+
+    @staticmethod
+    def softmax(x):
+        x = x.astype(np.float64)
+        e = np.exp(x - x.max(-1, keepdims=True))
+        return e / e.sum(-1, keepdims=True)
+
+    @staticmethod
+    def gemm(a, w, bias=None):
+        r = a.astype(np.float64) @ w.astype(np.float64).T
+        if bias is not None:
+            r = r + bias.astype(np.float64)
+        return r

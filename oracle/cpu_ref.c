@@ -1,0 +1,275 @@
+/*
+ * CPU oracle for the DTAS hot path -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C restatement of the loop nests of the TIR PrimFuncs whose scheduled
+ * GPU kernels the library replaces.  Only tests, the smoke check and the
+ * cpu_baseline leg of the benchmark may load this file's shared object; the
+ * product path never calls into it.
+ *
+ * Every function follows the PrimFunc text it cites (paths are relative to the
+ * reference checkout): same accumulation dtype, same operation order inside a
+ * row (sequential over the reduction axis, as an unscheduled PrimFunc built
+ * for an llvm CPU target executes).  Rows are independent, so the optional
+ * OpenMP split over rows (nthreads > 1) does not change any result bit.
+ *
+ * Parity status: the reference holds no numerical tests or golden vectors, so
+ * every function here is pinned by closed forms, library routines (numpy /
+ * torch CPU), exhaustive enumeration and invariants in tests/ -- see each
+ * function's comment.  rms_norm has no counterpart in the reference at all
+ * ("parity unpinned" by the reference; pinned by its closed form only).
+ *
+ * Build: gcc -O3 -march=x86-64-v3 -fopenmp -shared -fPIC (see oracle/Makefile).
+ */
+#include <immintrin.h>
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+/* every function below names its thread-count parameter nthreads */
+#define OMP_FOR(nt) _Pragma("omp parallel for schedule(static) num_threads(nthreads)")
+#else
+#define OMP_FOR(nt) (void)(nt);
+#endif
+
+typedef uint16_t f16; /* IEEE binary16 bit pattern */
+
+/* ---- fp16 <-> fp32: hardware F16C (IEEE RNE, subnormals kept) ------------- */
+static inline float h2f(f16 h) { return _cvtsh_ss(h); }
+static inline f16 f2h(float f) { return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC); }
+
+/* ---- fp16 <-> fp32 in integer arithmetic only: pins the F16C path in tests - */
+float oracle_soft_h2f(f16 h) {
+  uint32_t s = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1fu, m = h & 0x3ffu, u;
+  if (e == 0) {
+    if (m == 0) {
+      u = s;
+    } else { /* subnormal: normalise */
+      int sh = 0;
+      while (!(m & 0x400u)) { m <<= 1; ++sh; }
+      u = s | ((uint32_t)(127 - 15 - sh + 1) << 23) | ((m & 0x3ffu) << 13);
+    }
+  } else if (e == 31) {
+    u = s | 0x7f800000u | (m << 13);
+  } else {
+    u = s | ((e + 112u) << 23) | (m << 13);
+  }
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+f16 oracle_soft_f2h(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  uint32_t s = (u >> 16) & 0x8000u, a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (f16)(s | 0x7e00u | ((a >> 13) & 0x3ffu)); /* NaN, quieted */
+  if (a >= 0x477ff000u) return (f16)(s | 0x7c00u); /* |x| >= 65520 -> inf (also inf) */
+  if (a < 0x33000001u) return (f16)s;              /* |x| <= 2^-25 -> +-0 (tie to even) */
+  int32_t e = (int32_t)(a >> 23) - 127;
+  uint32_t m = (a & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+  int shift = (e < -14) ? (13 + (-14 - e)) : 13; /* bits dropped */
+  uint32_t keep = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (keep & 1u))) ++keep;
+  if (e < -14) return (f16)(s | keep); /* subnormal (carry into exponent is the right bits) */
+  /* keep has the hidden bit at position 10; a rounding carry bumps the exponent */
+  return (f16)(s | (((uint32_t)(e + 15) << 10) + (keep - 0x400u)));
+}
+
+/* ===========================================================================
+ * Elementwise: tuning_test/tune_ele_add.py:10-22 (add), tune_cast.py:10-21
+ * (cast fp16->fp32), tune_ele_copy.py:10-21 (copy); fp16/fp32/int8 variants as
+ * in experiment/dtas_tuned/elementwise/{add,copy}/{float16,float32,int8}/ .
+ * The fused (1, n, H) iteration space is one flat array of count elements.
+ * ======================================================================== */
+
+/* T_add = A + B in fp16: one IEEE rounding of the exact sum (the exact sum of
+ * two fp16 values fits fp32 exactly or rounds innocuously: 24 >= 2*11+2).
+ * Pinned by: numpy.float16 addition over seeded and special-value inputs. */
+void oracle_add_f16(const f16* A, const f16* B, f16* out, int64_t count, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < count; ++i) out[i] = f2h(h2f(A[i]) + h2f(B[i]));
+}
+
+void oracle_add_f32(const float* A, const float* B, float* out, int64_t count, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < count; ++i) out[i] = A[i] + B[i];
+}
+
+/* int8 add wraps modulo 256 (two's complement), as the generated kernel's
+ * per-byte add does.  Pinned by: exhaustive 256x256 table vs numpy int8. */
+void oracle_add_i8(const int8_t* A, const int8_t* B, int8_t* out, int64_t count, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < count; ++i) out[i] = (int8_t)(uint8_t)((uint8_t)A[i] + (uint8_t)B[i]);
+}
+
+/* B = A, bit for bit (NaN payloads included). */
+void oracle_copy_bytes(const void* A, void* B, int64_t nbytes, int nthreads) {
+  const int64_t chunk = 1 << 20;
+  const int64_t nchunks = (nbytes + chunk - 1) / chunk;
+  OMP_FOR(nthreads)
+  for (int64_t c = 0; c < nchunks; ++c) {
+    int64_t lo = c * chunk, len = nbytes - lo < chunk ? nbytes - lo : chunk;
+    memcpy((char*)B + lo, (const char*)A + lo, (size_t)len);
+  }
+}
+
+/* compute = Cast(float32, A): exact widening.  Pinned by: all 65536 patterns
+ * against numpy and against oracle_soft_h2f. */
+void oracle_cast_f16_f32(const f16* A, float* out, int64_t count, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < count; ++i) out[i] = h2f(A[i]);
+}
+
+/* Narrowing cast: round to nearest even, overflow to +-inf, subnormals kept,
+ * NaN stays NaN.  Pinned by: boundary table + 2^24 random patterns vs numpy
+ * and vs oracle_soft_f2h. */
+void oracle_cast_f32_f16(const float* A, f16* out, int64_t count, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < count; ++i) out[i] = f2h(A[i]);
+}
+
+/* ===========================================================================
+ * Row reductions.
+ * ======================================================================== */
+
+/* fused_layer_norm_cast1: experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:607-
+ * 636 and experiment/dtas_tuned/general_reduction/layernorm/profile_dlight.py:
+ * 7-40.  s0 = sum x, s1 = sum x*x (fp32, sequential); the PrimFunc multiplies
+ * by the fp32 literal 1/H (0.000390625 for H = 2560), it does not divide;
+ * out = f16((x - s0*inv)*rsqrt(s1*inv - (s0*inv)*(s0*inv) + eps)*gamma + beta).
+ * Pinned by: fp64 numpy layer norm (atol 1e-2), torch.layer_norm on CPU,
+ * affine invariance, gamma=1/beta=0 => row mean 0 / variance 1. */
+void oracle_layer_norm_f32_f16(const float* x, const float* gamma, const float* beta, f16* out,
+                               int64_t n, int64_t H, float eps, int nthreads) {
+  const float inv = (float)(1.0 / (double)H);
+  OMP_FOR(nthreads)
+  for (int64_t r = 0; r < n; ++r) {
+    const float* xr = x + r * H;
+    float s0 = 0.f, s1 = 0.f;
+    for (int64_t k = 0; k < H; ++k) {
+      s0 = s0 + xr[k];
+      s1 = s1 + xr[k] * xr[k];
+    }
+    const float mean = s0 * inv;
+    const float rstd = 1.0f / sqrtf(s1 * inv - mean * mean + eps);
+    for (int64_t k = 0; k < H; ++k) out[r * H + k] = f2h((xr[k] - mean) * rstd * gamma[k] + beta[k]);
+  }
+}
+
+/* rms_norm: no counterpart in the reference (PARITY UNPINNED by the
+ * reference).  Closed form: ss = sum f32(x)^2 in fp32;
+ * out = f16(f32(x) * rsqrt(ss/H + eps) * f32(w)), one final rounding.
+ * Pinned by: fp64 numpy closed form (atol 1e-2), torch.nn.functional.rms_norm
+ * on CPU, scale invariance, w = 1 => row rms 1. */
+void oracle_rms_norm_f16(const f16* x, const f16* w, f16* out, int64_t n, int64_t H, float eps,
+                         int nthreads) {
+  const float inv = (float)(1.0 / (double)H);
+  OMP_FOR(nthreads)
+  for (int64_t r = 0; r < n; ++r) {
+    const f16* xr = x + r * H;
+    float ss = 0.f;
+    for (int64_t k = 0; k < H; ++k) {
+      float v = h2f(xr[k]);
+      ss = ss + v * v;
+    }
+    const float rs = 1.0f / sqrtf(ss * inv + eps);
+    for (int64_t k = 0; k < H; ++k) out[r * H + k] = f2h(h2f(xr[k]) * rs * h2f(w[k]));
+  }
+}
+
+/* fused_softmax_cast: experiment/dtas_tuned/general_reduction/softmax/
+ * profile_dlight.py:8-52 (3-D form) and experiment/ModelIR/dolly-v2-3b-q0f16/
+ * before_dl.py:756-800 (fused_softmax_cast3, 4-D (1,32,n,m) form): per row
+ * mx = max(-FLT_MAX, x...) (the init is -3.4028234663852886e+38, not -inf),
+ * e = exp(x - mx) in fp32, s = sum e (sequential), out = f16(e / s).
+ * Pinned by: fp64 numpy / scipy.special.softmax (atol 1e-2), rows sum to 1,
+ * shift invariance, a single column gives exactly 1.0, a constant row 1/cols. */
+void oracle_softmax_f32_f16(const float* x, f16* out, int64_t rows, int64_t cols, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t r = 0; r < rows; ++r) {
+    const float* xr = x + r * cols;
+    float mx = -3.4028234663852886e+38f;
+    for (int64_t k = 0; k < cols; ++k) mx = xr[k] > mx ? xr[k] : mx;
+    float s = 0.f;
+    for (int64_t k = 0; k < cols; ++k) s = s + expf(xr[k] - mx);
+    for (int64_t k = 0; k < cols; ++k) out[r * cols + k] = f2h(expf(xr[k] - mx) / s);
+  }
+}
+
+/* Same PrimFunc with an fp16 input buffer (the [32n, n] attention-score form):
+ * the values are widened to fp32 first, then the identical fp32 pipeline. */
+void oracle_softmax_f16_f16(const f16* x, f16* out, int64_t rows, int64_t cols, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t r = 0; r < rows; ++r) {
+    const f16* xr = x + r * cols;
+    float mx = -3.4028234663852886e+38f;
+    for (int64_t k = 0; k < cols; ++k) {
+      float v = h2f(xr[k]);
+      mx = v > mx ? v : mx;
+    }
+    float s = 0.f;
+    for (int64_t k = 0; k < cols; ++k) s = s + expf(h2f(xr[k]) - mx);
+    for (int64_t k = 0; k < cols; ++k) out[r * cols + k] = f2h(expf(h2f(xr[k]) - mx) / s);
+  }
+}
+
+/* ===========================================================================
+ * GEMV / GEMM: C[i, j] = sum_k A[i, k] * W[j, k] (+ bias[j]).
+ * GEMV is fused_NT_matmul10_add5 (before_dl.py:96-113), GEMM is
+ * fused_NT_matmul4_add1 (before_dl.py:320-341); GEMV is the M = 1 case.
+ * acc_f16 = 0: products and the running sum in fp32, one rounding to fp16 at
+ *              the end (then "+ bias" in fp16 if bias is given) -- the
+ *              fp32-accumulate contract of the benchmark configs.
+ * acc_f16 = 1: the PrimFunc text literally: the running sum is an fp16 buffer,
+ *              acc = f16(acc + f16(a*w)) for k ascending.
+ * Pinned by: fp64 numpy A @ W.T (rtol 1e-2), exact cases (K = 1, identity /
+ * permutation W, one-hot rows), brute force on tiny ragged shapes,
+ * torch.matmul on CPU.
+ * ======================================================================== */
+void oracle_gemm_f16(const f16* A, const f16* W, const f16* bias, f16* C, int64_t M, int64_t N,
+                     int64_t K, int acc_f16, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t ij = 0; ij < M * N; ++ij) {
+    const int64_t i = ij / N, j = ij % N;
+    const f16* a = A + i * K;
+    const f16* w = W + j * K;
+    f16 r;
+    if (acc_f16) {
+      f16 acc = 0;
+      for (int64_t k = 0; k < K; ++k) acc = f2h(h2f(acc) + h2f(f2h(h2f(a[k]) * h2f(w[k]))));
+      r = acc;
+    } else {
+      float acc = 0.f;
+      for (int64_t k = 0; k < K; ++k) acc = acc + h2f(a[k]) * h2f(w[k]);
+      r = f2h(acc);
+    }
+    if (bias) r = f2h(h2f(r) + h2f(bias[j]));
+    C[ij] = r;
+  }
+}
+
+/* The same sum with the fp32 accumulator returned unrounded; the parity tests
+ * use it to bound the GPU's fp32 partial-sum reordering separately from the
+ * final fp16 rounding. */
+void oracle_gemm_f16_f32out(const f16* A, const f16* W, float* C, int64_t M, int64_t N, int64_t K,
+                            int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t ij = 0; ij < M * N; ++ij) {
+    const int64_t i = ij / N, j = ij % N;
+    const f16* a = A + i * K;
+    const f16* w = W + j * K;
+    float acc = 0.f;
+    for (int64_t k = 0; k < K; ++k) acc = acc + h2f(a[k]) * h2f(w[k]);
+    C[ij] = acc;
+  }
+}
+
+int oracle_max_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

@@ -1,0 +1,126 @@
+"""Host-side flow of the reference's entry points on CPU: Engine.tune_module -> runtime module ->
+load_module_from_file; bucket index statement; argument binding.  No kernel is launched."""
+import json
+import os
+
+import pytest
+import torch
+
+import dtas_amd
+from dtas_amd import _lib, primfuncs as pf
+from dtas_amd.arch import MI355X
+from dtas_amd.codegen.runtime_packer import bind_extents, extents_of, load_module_from_file, op_id_of
+from dtas_amd.common.analisys import FuncInfo, FuncKind
+from dtas_amd.common.config import Range
+from dtas_amd.engine.tuner import Engine
+
+
+def _module():
+    return pf.module(pf.add("float16", 4096), pf.cast("float32", "float16", 4096), pf.copy("float16", 4096),
+                     pf.rms_norm(4096), pf.fused_layer_norm_cast1(2560), pf.softmax_scores(32),
+                     pf.fused_softmax_cast3(32), pf.fused_NT_matmul_add_gemv(4096, 4096, bias=False),
+                     pf.fused_NT_matmul_add_gemm(11008, 4096, bias=True), upper_bound={"n": 4096, "m": 512})
+
+
+def test_rule_selection():
+    kinds = {name: FuncInfo(f).kind for name, f in _module().functions_items()}
+    assert kinds["add"] == kinds["cast"] == kinds["copy"] == FuncKind.kFunc_Elementwise
+    assert kinds["rms_norm"] == kinds["fused_layer_norm_cast1"] == kinds["softmax_scores"] == FuncKind.kFunc_Reduction
+    assert kinds["NT_matmul10"] == FuncKind.kFunc_GEMV and kinds["fused_NT_matmul4_add1"] == FuncKind.kFunc_GEMM
+    assert [v.name for v in pf.fused_softmax_cast3().dynamic_args] == ["n", "m"]
+    assert op_id_of(pf.cast("float32", "float16")) == _lib.OP_CAST_F32_F16
+    assert op_id_of(pf.add("int8")) == _lib.OP_ADD_I8
+
+
+def test_tune_module_writes_tables_and_reloads(tmp_path):
+    eng = Engine(topk=10, parallel_build=True, work_dir=str(tmp_path))
+    rt = eng.tune_module(_module(), arch=MI355X(), range_div_factor=256)
+    assert os.path.exists(tmp_path / "dispatch_table.json") and os.path.exists(tmp_path / "dispatch_tables.h")
+    assert os.path.exists(tmp_path / "data_base" / "best_record.json")
+    records = json.load(open(tmp_path / "data_base" / "best_record.json"))
+    assert any(k.startswith("add_<n: Range(1, 256)>") for rec in records for k in rec)
+    add = rt.tables["add"]
+    assert len(add.index_table) == 16 and add.index_stmt() == "  int64_t index = (n/256) > 15 ? 15 : n/256;\n"
+    # every call-table row is launchable according to the C library
+    for name, table in rt.tables.items():
+        for entry in table.call_table:
+            hi = {r.var.name: r.end for r in entry.ranges}
+            _lib.describe_launch(op_id_of(table.func), *extents_of(table.func, hi), entry.abi)
+    # GEMM picks the weight-streaming kernel only where M fits it, big tiles at big M
+    gemm = rt.tables["fused_NT_matmul4_add1"]
+    assert gemm.select({"n": 4096}).abi.variant == _lib.GEMM_MFMA
+    assert list(gemm.select({"n": 4000}).abi.tile)[:2] == [256, 256]
+    # a static function (GEMV) has one row and no index table
+    assert rt.tables["NT_matmul10"].index_table == [] and len(rt.tables["NT_matmul10"].call_table) == 1
+
+    again = load_module_from_file(str(tmp_path))
+    for name, table in rt.tables.items():
+        other = again.tables[name]
+        assert other.index_table == table.index_table
+        assert [e.abi.to_dict() for e in other.call_table] == [e.abi.to_dict() for e in table.call_table]
+        assert [e.name for e in other.call_table] == [e.name for e in table.call_table]
+    with pytest.raises(FileNotFoundError):
+        load_module_from_file(str(tmp_path / "nope"))
+
+
+def test_index_statement_semantics(tmp_path):
+    rt = Engine(1, work_dir=str(tmp_path)).tune_module(pf.module(pf.rms_norm(4096), pf.fused_softmax_cast3(),
+                                                                 upper_bound={"n": 4096, "m": 512}), MI355X(), 256)
+    t = rt.tables["rms_norm"]
+    # C integer division, clamped: n = 255 -> 0, n = 256 -> 1 (the reference's n / div), n >= 4096 -> 15
+    assert [t.index({"n": n}) for n in (1, 255, 256, 511, 512, 4095, 4096, 10 ** 6)] == [0, 0, 1, 1, 2, 15, 15, 15]
+    t2 = rt.tables["fused_softmax_cast3"]
+    assert len(t2.index_table) == 16 * 2
+    assert t2.index({"n": 300, "m": 100}) == 1 * 2 + 0 and t2.index({"n": 300, "m": 300}) == 1 * 2 + 1
+    assert t2.index({"n": 10 ** 6, "m": 10 ** 6}) == 31
+    # each cell of the 2-D table points at the merged entry whose rectangle contains it
+    for a in range(16):
+        for b in range(2):
+            entry = t2.call_table[t2.index_table[a * 2 + b]]
+            rn, rm = entry.ranges
+            assert rn.start <= a * 256 + 1 <= rn.end and rm.start <= b * 256 + 1 <= rm.end
+
+
+def test_merge_two_dynamic_extents(tmp_path):
+    from dtas_amd.codegen.compile_result import CompileResult
+    from dtas_amd.common.config import ReductionConfig
+
+    def cr(tx):
+        c = ReductionConfig()
+        c.len_tx = tx
+        return CompileResult(c, c.to_abi(), "f")
+
+    eng = Engine(1, work_dir=str(tmp_path))
+    eng.upper_bound.update({"n": 768, "m": 512})
+    best = {}
+    for i, n0 in enumerate((1, 257, 513)):
+        for j, m0 in enumerate((1, 257)):
+            tx = 128 if i == 0 and j == 0 else 256 if i == 0 else 512
+            best[(Range("n", n0, n0 + 255), Range("m", m0, m0 + 255))] = cr(tx)
+    merged = eng.merge_same_configs(best)
+    got = [(rt[0].start, rt[0].end, rt[1].start, rt[1].end, c.config.len_tx) for rt, c in merged.items()]
+    assert got == [(1, 256, 1, 256, 128), (1, 256, 257, 512, 256), (257, 768, 1, 512, 512)]
+    table, stmt = eng.get_index_table(merged, 256)
+    assert table == [0, 1, 2, 2, 2, 2]
+
+
+def test_bind_extents_checks_the_signature():
+    f = pf.add("float16", 64)
+    a = torch.zeros(1, 5, 64, dtype=torch.float16)
+    assert bind_extents(f, [a, a, a]) == {"n": 5}
+    with pytest.raises(TypeError, match="takes 3 buffers"):
+        bind_extents(f, [a, a])
+    with pytest.raises(TypeError, match="float16"):
+        bind_extents(f, [a, a.float(), a])
+    with pytest.raises(ValueError, match="expects shape"):
+        bind_extents(f, [a, a, torch.zeros(1, 5, 32, dtype=torch.float16)])
+    with pytest.raises(ValueError, match="extent n"):
+        bind_extents(f, [a, a, torch.zeros(1, 6, 64, dtype=torch.float16)])
+
+
+def test_cpu_tensors_are_refused_not_computed_elsewhere():
+    from dtas_amd import ops
+
+    a = torch.zeros(4, 64, dtype=torch.float16)
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.add(a, a, a.clone())

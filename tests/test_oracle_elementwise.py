@@ -1,0 +1,127 @@
+"""Pins the elementwise part of the CPU oracle (oracle/cpu_ref.c) without the reference:
+IEEE-754 closed forms, numpy as the library routine, exhaustive enumeration where feasible."""
+import numpy as np
+import pytest
+
+ALL_F16 = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+
+
+def test_widen_all_65536_patterns(oracle):
+    h = ALL_F16.view(np.float16)
+    got = oracle.c.cast(h, "float32")
+    want = h.astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    # NaNs stay NaNs with their payload; the conversion instruction sets the quiet bit of a
+    # signalling NaN (IEEE 754 conversion), numpy's software path does not
+    quiet = np.uint32(0x00400000)
+    assert np.array_equal(got.view(np.uint32)[nan], want.view(np.uint32)[nan] | quiet)
+
+
+def test_soft_widen_matches_hardware_path(oracle):
+    got = np.array([oracle.c.soft_h2f(int(b)) for b in ALL_F16[::7]], dtype=np.float32)
+    want = ALL_F16[::7].view(np.float16).astype(np.float32)
+    nan = np.isnan(want)  # (a NaN's quiet bit does not survive the float -> Python double return)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    assert np.isnan(got[nan]).all()
+
+
+NARROW_BOUNDARIES = [0.0, -0.0, 65504.0, 65519.99, 65520.0, 65536.0, -65520.0, 1e10, -1e10, np.inf, -np.inf,
+                     2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 2.0 ** -26, 2.0 ** -14, 2.0 ** -14 * (1 - 2 ** -11),
+                     1.0 + 2.0 ** -11, 1.0 + 2.0 ** -11 + 2.0 ** -20, 1.0 + 3 * 2.0 ** -11, 2047.5, 2048.5, 2049.5,
+                     6.1e-5, 5.96e-8, 2.98e-8, 2.99e-8]
+
+
+def test_narrow_boundaries(oracle):
+    x = np.array(NARROW_BOUNDARIES, dtype=np.float32)
+    got = oracle.c.cast(x, "float16")
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert np.isinf(got[2 + 2]) and got[2] == np.float16(65504) and got[3] == np.float16(65504)  # 65520 -> inf
+    soft = np.array([oracle.c.soft_f2h(float(v)) for v in x], dtype=np.uint16)
+    assert np.array_equal(soft, want.view(np.uint16))
+
+
+def test_narrow_random_bit_patterns(oracle):
+    rng = np.random.default_rng(11)
+    bits = rng.integers(0, 2 ** 32, size=1 << 22, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32)
+    got = oracle.c.cast(x, "float16")
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = x.astype(np.float16)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+    # the integer-only conversion agrees on a sample (python-call bound)
+    idx = rng.integers(0, x.size, size=4000)
+    soft = np.array([oracle.c.soft_f2h(float(x[i])) if not np.isnan(x[i]) else 0 for i in idx], dtype=np.uint16)
+    ok = ~np.isnan(x[idx])
+    assert np.array_equal(soft[ok], want.view(np.uint16)[idx][ok])
+
+
+def test_narrow_scaled_normal_overflows_to_inf(oracle):
+    # the benchmark's cast input: normal(0,1) * 100 never overflows, * 1e5 does
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal(1 << 16) * 1e5).astype(np.float32)
+    got = oracle.c.cast(x, "float16")
+    assert np.isinf(got[np.abs(x) >= 65520]).all() and np.isfinite(got[np.abs(x) < 65504]).all()
+
+
+def test_add_f16_is_one_rounding_of_the_exact_sum(oracle):
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-1, 1, 1 << 18).astype(np.float16)
+    b = rng.uniform(-1, 1, 1 << 18).astype(np.float16)
+    got = oracle.c.add(a, b)
+    assert np.array_equal(got.view(np.uint16), (a + b).view(np.uint16))
+    exact = (a.astype(np.float64) + b.astype(np.float64)).astype(np.float16)  # fp64 holds the sum exactly
+    assert np.array_equal(got.view(np.uint16), exact.view(np.uint16))
+
+
+def test_add_f16_special_values(oracle):
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 65504, -65504, 6e-8, -6e-8, 6.1e-5, 1, -1], dtype=np.float16)
+    a, b = np.meshgrid(sp, sp)
+    a, b = np.ascontiguousarray(a.ravel()), np.ascontiguousarray(b.ravel())
+    got = oracle.c.add(a, b)
+    with np.errstate(all="ignore"):
+        want = a + b
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+    assert np.isnan(oracle.c.add(np.array([np.inf], np.float16), np.array([-np.inf], np.float16))[0])
+
+
+def test_add_f16_all_patterns_against_one_operand(oracle):
+    a = ALL_F16.view(np.float16)
+    for other in (np.float16(1.0), np.float16(-3.140625), np.float16(6e-8), np.float16(60000)):
+        b = np.full_like(a, other)
+        got = oracle.c.add(a, b)
+        with np.errstate(all="ignore"):
+            want = a + b
+        nan = np.isnan(want)
+        assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+
+
+def test_add_i8_wraps_exhaustive(oracle):
+    a, b = np.meshgrid(np.arange(-128, 128, dtype=np.int8), np.arange(-128, 128, dtype=np.int8))
+    a, b = np.ascontiguousarray(a.ravel()), np.ascontiguousarray(b.ravel())
+    got = oracle.c.add(a, b)
+    want = ((a.astype(np.int32) + b.astype(np.int32) + 128) % 256 - 128).astype(np.int8)
+    assert np.array_equal(got, want)
+    assert oracle.c.add(np.array([127], np.int8), np.array([1], np.int8))[0] == -128
+
+
+def test_add_f32_and_copy(oracle):
+    rng = np.random.default_rng(5)
+    a, b = rng.standard_normal(10001).astype(np.float32), rng.standard_normal(10001).astype(np.float32)
+    assert np.array_equal(oracle.c.add(a, b), a + b)
+    h = ALL_F16.view(np.float16)
+    assert np.array_equal(oracle.c.copy(h).view(np.uint16), ALL_F16)  # identity on bits, NaNs too
+
+
+def test_threads_do_not_change_bits(oracle):
+    rng = np.random.default_rng(9)
+    a = rng.uniform(-1, 1, (37, 4096)).astype(np.float16)
+    b = rng.uniform(-1, 1, (37, 4096)).astype(np.float16)
+    assert np.array_equal(oracle.c.add(a, b, threads=1).view(np.uint16), oracle.c.add(a, b, threads=4).view(np.uint16))
+    assert oracle.c.add(a[:0], b[:0]).size == 0  # empty extent

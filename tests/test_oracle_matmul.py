@@ -1,0 +1,88 @@
+"""Pins the GEMV / GEMM part of the CPU oracle: float64 product, exact special cases,
+brute force on tiny ragged shapes, torch CPU matmul, and the literal fp16-accumulate order."""
+import numpy as np
+import pytest
+import torch
+
+RTOL = 1e-2
+
+
+def _close(got, want, rtol=RTOL, atol=2e-3):
+    got, want = got.astype(np.float64), np.asarray(want, np.float64)
+    return np.all(np.abs(got - want) <= atol + rtol * np.abs(want))
+
+
+def _inputs(M, N, K, seed=6):
+    rng = np.random.default_rng(seed)
+    return rng.standard_normal((M, K)).astype(np.float16), (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 4096), (1, 33, 1000), (5, 7, 3), (16, 48, 256), (3, 130, 520)])
+def test_gemm_against_float64_and_torch(oracle, M, N, K):
+    a, w = _inputs(M, N, K)
+    got = oracle.c.gemm(a, w)
+    assert _close(got, oracle.np64.gemm(a, w))
+    ref = (torch.from_numpy(a).float() @ torch.from_numpy(w).float().T).numpy()
+    assert _close(got, ref)
+    # W is [N, K] and is used transposed: a transposed-operand mistake fails on a ragged shape
+    assert got.shape == (M, N)
+
+
+def test_gemm_exact_cases(oracle):
+    rng = np.random.default_rng(1)
+    # K = 1: each output is one fp16 x fp16 product, exact in fp32, rounded once
+    a = rng.standard_normal((4, 1)).astype(np.float16)
+    w = rng.standard_normal((6, 1)).astype(np.float16)
+    want = (a.astype(np.float32) * w.astype(np.float32).T).astype(np.float16)
+    assert np.array_equal(oracle.c.gemm(a, w).view(np.uint16), want.view(np.uint16))
+    # identity W returns A bit for bit; a permutation of W's rows permutes C's columns
+    a = rng.standard_normal((5, 32)).astype(np.float16)
+    eye = np.eye(32, dtype=np.float16)
+    assert np.array_equal(oracle.c.gemm(a, eye).view(np.uint16), a.view(np.uint16))
+    perm = rng.permutation(32)
+    assert np.array_equal(oracle.c.gemm(a, eye[perm].copy()).view(np.uint16), a[:, perm].view(np.uint16))
+    # one-hot x selects a column of W^T exactly (GEMV)
+    w = (rng.standard_normal((9, 64)) * 0.02).astype(np.float16)
+    x = np.zeros((1, 64), np.float16)
+    x[0, 17] = 1
+    assert np.array_equal(oracle.c.gemm(x, w).view(np.uint16).ravel(), w[:, 17].view(np.uint16))
+
+
+def test_gemm_bias_is_added_after_rounding(oracle):
+    a, w = _inputs(3, 10, 64)
+    bias = np.linspace(-1, 1, 10).astype(np.float16)
+    base = oracle.c.gemm(a, w)
+    want = (base.astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(oracle.c.gemm(a, w, bias).view(np.uint16), want.view(np.uint16))
+
+
+def test_gemm_brute_force_python_loops(oracle):
+    a, w = _inputs(2, 3, 5, seed=8)
+    got32 = oracle.c.gemm_f32out(a, w)
+    for i in range(2):
+        for j in range(3):
+            acc = np.float32(0)
+            for k in range(5):
+                acc = np.float32(acc + np.float32(a[i, k]) * np.float32(w[j, k]))
+            assert got32[i, j] == acc
+            assert oracle.c.gemm(a, w)[i, j] == np.float16(acc)
+
+
+def test_fp16_accumulate_follows_the_primfunc_text(oracle):
+    # acc = f16(acc + f16(a*w)), k ascending (before_dl.py:96-113 keeps the sum in an fp16 buffer)
+    a, w = _inputs(2, 4, 40, seed=9)
+    got = oracle.c.gemm(a, w, acc_f16=True)
+    for i in range(2):
+        for j in range(4):
+            acc = np.float16(0)
+            for k in range(40):
+                acc = np.float16(acc + np.float16(a[i, k] * w[j, k]))
+            assert got[i, j] == acc
+    # and it differs from fp32 accumulation on long sums (so the two modes are really distinct)
+    a, w = _inputs(1, 64, 4096, seed=10)
+    assert not np.array_equal(oracle.c.gemm(a, w, acc_f16=True), oracle.c.gemm(a, w))
+
+
+def test_threads_do_not_change_bits(oracle):
+    a, w = _inputs(7, 33, 100)
+    assert np.array_equal(oracle.c.gemm(a, w, threads=1).view(np.uint16), oracle.c.gemm(a, w, threads=4).view(np.uint16))

@@ -1,0 +1,101 @@
+"""Pins the row-reduction part of the CPU oracle: closed forms in float64, torch / scipy CPU
+routines, and invariants chosen so that a dropped term, a wrong sign or a wrong axis fails."""
+import numpy as np
+import pytest
+import torch
+from scipy.special import softmax as scipy_softmax
+
+ATOL = 1e-2  # the stated tolerance for fp16 outputs of the reductions
+
+
+def _ln_inputs(n=9, H=2560, seed=3):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((n, H)) * 2 + 0.5).astype(np.float32)
+    return x, rng.uniform(0.5, 1.5, H).astype(np.float32), rng.uniform(-1, 1, H).astype(np.float32)
+
+
+def test_layer_norm_closed_form_and_torch(oracle):
+    x, g, b = _ln_inputs()
+    got = oracle.c.layer_norm(x, g, b).astype(np.float64)
+    assert np.abs(got - oracle.np64.layer_norm(x, g, b)).max() < ATOL
+    ref = torch.nn.functional.layer_norm(torch.from_numpy(x), (x.shape[-1],), torch.from_numpy(g), torch.from_numpy(b), 1e-5)
+    assert np.abs(got - ref.numpy()).max() < ATOL
+
+
+def test_layer_norm_invariants(oracle):
+    x, g, b = _ln_inputs(n=5)
+    one, zero = np.ones_like(g), np.zeros_like(b)
+    y = oracle.c.layer_norm(x, one, zero).astype(np.float64)
+    assert np.abs(y.mean(-1)).max() < 1e-3 and np.abs(y.var(-1) - 1).max() < 1e-2
+    # affine invariance in x: LN(a*x + c) == LN(x) for a > 0
+    y2 = oracle.c.layer_norm((3.0 * x + 7.0).astype(np.float32), one, zero).astype(np.float64)
+    assert np.abs(y - y2).max() < ATOL
+    # sign: negating x negates the normalised value (catches a dropped mean or |.|)
+    y3 = oracle.c.layer_norm(-x, one, zero).astype(np.float64)
+    assert np.abs(y + y3).max() < ATOL
+    # gamma scales, beta shifts
+    y4 = oracle.c.layer_norm(x, 2 * one, zero + 0.25).astype(np.float64)
+    assert np.abs(y4 - (2 * y + 0.25)).max() < ATOL
+    # a constant row has zero variance: output is beta exactly (eps keeps rsqrt finite)
+    c = np.full((1, 2560), 3.25, np.float32)
+    assert np.abs(oracle.c.layer_norm(c, one, b).astype(np.float32) - b.astype(np.float16).astype(np.float32)).max() < 2e-3
+
+
+def test_layer_norm_uses_the_row_length_not_2560(oracle):
+    x, g, b = _ln_inputs(n=3, H=4096)
+    assert np.abs(oracle.c.layer_norm(x, g, b).astype(np.float64) - oracle.np64.layer_norm(x, g, b)).max() < ATOL
+
+
+def _rms_inputs(n=7, H=4096, seed=3):
+    rng = np.random.default_rng(seed)
+    return rng.standard_normal((n, H)).astype(np.float16), rng.uniform(0.5, 1.5, H).astype(np.float16)
+
+
+def test_rms_norm_closed_form_and_torch(oracle):
+    x, w = _rms_inputs()
+    got = oracle.c.rms_norm(x, w).astype(np.float64)
+    assert np.abs(got - oracle.np64.rms_norm(x, w)).max() < ATOL
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x).float(), (x.shape[-1],), torch.from_numpy(w).float(), 1e-5)
+    assert np.abs(got - ref.numpy()).max() < ATOL
+
+
+def test_rms_norm_invariants(oracle):
+    x, w = _rms_inputs(n=4)
+    one = np.ones_like(w)
+    y = oracle.c.rms_norm(x, one).astype(np.float64)
+    assert np.abs(np.sqrt((y * y).mean(-1)) - 1).max() < 2e-3            # unit rms
+    y2 = oracle.c.rms_norm((x * np.float16(4)).astype(np.float16), one).astype(np.float64)
+    assert np.abs(y - y2).max() < ATOL                                   # scale invariance
+    assert np.abs(oracle.c.rms_norm(-x, one).astype(np.float64) + y).max() < 1e-6   # odd in x: no mean subtraction
+    # unlike layer norm, a constant row is NOT mapped to zero
+    c = np.full((1, 4096), 2.0, np.float16)
+    assert np.abs(oracle.c.rms_norm(c, one).astype(np.float64) - 1.0).max() < 1e-3
+    # eps matters for a zero row: output is exactly zero, not NaN
+    assert not np.isnan(oracle.c.rms_norm(np.zeros((1, 4096), np.float16), one)).any()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("cols", [1, 2, 3, 7, 8, 31, 257, 1024, 4096])
+def test_softmax_closed_form_and_scipy(oracle, dtype, cols):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((13, cols)) * 2).astype(dtype)
+    got = oracle.c.softmax(x).astype(np.float64)
+    assert np.abs(got - oracle.np64.softmax(x)).max() < ATOL
+    assert np.abs(got - scipy_softmax(x.astype(np.float64), axis=-1)).max() < ATOL
+    assert np.abs(got.sum(-1) - 1).max() < cols * 2.0 ** -11 + 1e-3
+
+
+def test_softmax_invariants(oracle):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((6, 300)) * 2).astype(np.float32)
+    y = oracle.c.softmax(x).astype(np.float64)
+    assert np.abs(oracle.c.softmax(x + np.float32(5)).astype(np.float64) - y).max() < 1e-3     # shift invariance
+    assert (oracle.c.softmax(np.array([[3.5]], np.float32)) == np.float16(1.0)).all()            # single column
+    assert np.abs(oracle.c.softmax(np.full((2, 8), -2.0, np.float32)).astype(np.float64) - 0.125).max() == 0
+    assert np.array_equal(np.argmax(y, -1), np.argmax(x, -1))                                    # monotone, right axis
+    # large magnitudes: the max subtraction keeps exp finite
+    big = np.array([[1e4, 1e4 - 1, -1e4]], np.float32)
+    out = oracle.c.softmax(big).astype(np.float64)
+    assert np.isfinite(out).all() and abs(out[0, 0] - 1 / (1 + np.exp(-1))) < 1e-3 and out[0, 2] == 0
+    # rows are independent: permuting rows permutes outputs
+    assert np.array_equal(oracle.c.softmax(x[::-1].copy()), oracle.c.softmax(x)[::-1])

@@ -1,0 +1,201 @@
+"""GPU parity, elementwise add / copy / cast through the C ABI: bit-exact against the CPU oracle
+on the same seeded inputs, every kernel variant, ragged sizes, odd alignment, guard bands."""
+import numpy as np
+import pytest
+import torch
+
+from dtas_amd import _lib, ops
+from gpu_util import Guarded, assert_bits_equal, cfg, dev
+
+pytestmark = pytest.mark.gpu
+
+N_SWEEP = [1, 16, 128, 1024, 4096]
+ALL_F16 = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16)
+
+
+@pytest.mark.parametrize("n", N_SWEEP)
+def test_add_f16_benchmark_config(oracle, n):
+    rng0, rng1 = np.random.default_rng(0), np.random.default_rng(1)
+    a = rng0.uniform(-1, 1, (n, 4096)).astype(np.float16)
+    b = rng1.uniform(-1, 1, (n, 4096)).astype(np.float16)
+    out = Guarded(a.shape, torch.float16)
+    ops.add(dev(a), dev(b), out.t)
+    assert_bits_equal(out.check(), oracle.c.add(a, b, threads=8))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.int8])
+@pytest.mark.parametrize("n,H", [(1, 2560), (3, 2560), (257, 2560), (5, 2561), (1, 7), (2, 1)])
+def test_add_reference_shapes_and_ragged(oracle, dtype, n, H):
+    rng = np.random.default_rng(n * 131 + H)
+    if dtype == np.int8:
+        a = rng.integers(-128, 128, (1, n, H)).astype(np.int8)
+        b = rng.integers(-128, 128, (1, n, H)).astype(np.int8)
+    else:
+        a = rng.uniform(-1, 1, (1, n, H)).astype(dtype)
+        b = rng.uniform(-1, 1, (1, n, H)).astype(dtype)
+    out = Guarded(a.shape, torch.from_numpy(a).dtype)
+    ops.add(dev(a), dev(b), out.t)
+    assert_bits_equal(out.check(), oracle.c.add(a, b))
+
+
+def test_add_f16_special_values(oracle):
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 65504, -65504, 6e-8, -6e-8, 6.1e-5, 1, -1, 3e-5], dtype=np.float16)
+    a, b = np.meshgrid(sp, sp)
+    a, b = np.ascontiguousarray(a.ravel()[None]), np.ascontiguousarray(b.ravel()[None])
+    out = Guarded(a.shape, torch.float16)
+    ops.add(dev(a), dev(b), out.t)
+    assert_bits_equal(out.check(), oracle.c.add(a, b), nan_ok=True)
+    # every fp16 pattern plus a subnormal / a large value: subnormal results are kept, overflow goes to inf
+    for other in (np.float16(6e-8), np.float16(60000), np.float16(-1.5)):
+        a = ALL_F16.reshape(16, 4096)
+        b = np.full_like(a, other)
+        out = Guarded(a.shape, torch.float16)
+        ops.add(dev(a), dev(b), out.t)
+        assert_bits_equal(out.check(), oracle.c.add(a, b), nan_ok=True)
+
+
+def test_add_i8_wraps_exhaustive(oracle):
+    a, b = np.meshgrid(np.arange(-128, 128, dtype=np.int8), np.arange(-128, 128, dtype=np.int8))
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    out = Guarded(a.shape, torch.int8)
+    ops.add(dev(a), dev(b), out.t)
+    assert_bits_equal(out.check(), oracle.c.add(a, b))
+
+
+@pytest.mark.parametrize("n", N_SWEEP)
+def test_cast_f32_to_f16_benchmark_config(oracle, n):
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((n, 4096)) * 100).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    ops.cast(dev(x), out.t)
+    assert_bits_equal(out.check(), oracle.c.cast(x, "float16", threads=8))
+
+
+def test_cast_f32_to_f16_rounding_overflow_subnormals(oracle):
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal((64, 4096)) * 1e5).astype(np.float32)          # overflow to +-inf
+    tiny = (rng.standard_normal((64, 4096)) * 1e-6).astype(np.float32)      # fp16 subnormal results
+    patterns = rng.integers(0, 2 ** 32, size=(64, 4096), dtype=np.uint64).astype(np.uint32).view(np.float32)
+    edge = np.array([65504.0, 65519.99, 65520.0, -65520.0, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 2.0 ** -26,
+                     1 + 2.0 ** -11, 1 + 3 * 2.0 ** -11, 2049.5, np.inf, -np.inf, np.nan, 0.0, -0.0], np.float32)[None]
+    for src in (x, tiny, patterns, edge):
+        out = Guarded(src.shape, torch.float16)
+        ops.cast(dev(src), out.t)
+        got = out.check()
+        assert_bits_equal(got, oracle.c.cast(src, "float16"), nan_ok=True)
+    assert np.isinf(oracle.c.cast(x, "float16")).any() and (oracle.c.cast(tiny, "float16") != 0).any()
+
+
+def test_cast_f16_to_f32_all_patterns(oracle):
+    h = ALL_F16.reshape(1, 16, 4096)
+    out = Guarded(h.shape, torch.float32)
+    ops.cast(dev(h), out.t)
+    got = out.check()
+    want = oracle.c.cast(h, "float32")
+    assert_bits_equal(got, want, nan_ok=True)
+    assert np.array_equal(got[~np.isnan(got)], h.astype(np.float32)[~np.isnan(got)])
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.int8])
+@pytest.mark.parametrize("n", [1, 16, 1024])
+def test_copy_is_identity_on_bits(oracle, dtype, n):
+    rng = np.random.default_rng(3)
+    raw = rng.integers(0, 256, size=n * 4096 * np.dtype(dtype).itemsize, dtype=np.uint8)
+    a = raw.view(dtype).reshape(n, 4096)  # arbitrary bit patterns: NaN payloads, subnormals
+    out = Guarded(a.shape, torch.from_numpy(a).dtype)
+    ops.copy(dev(a), out.t)
+    got = out.check()
+    assert np.array_equal(got.view(np.uint8), oracle.c.copy(a).view(np.uint8))
+
+
+VARIANTS = [(op, vec, unroll) for op, vecs in (("add16", (8, 4, 2)), ("add32", (4, 2, 1)), ("add8", (16, 8, 4)),
+                                               ("castdown", (8, 4, 2)), ("castup", (8, 4, 2)))
+            for vec in vecs for unroll in (1, 2, 4, 8)]
+
+
+@pytest.mark.parametrize("op,vec,unroll", VARIANTS)
+def test_every_vector_variant(oracle, op, vec, unroll):
+    rng = np.random.default_rng(vec * 10 + unroll)
+    shape = (37, 2568)  # not a multiple of the largest tiles; divisible by 8 so every width is aligned
+    c = cfg(variant=_lib.ELT_VECTOR, vec=vec, unroll=unroll)
+    if op == "add16":
+        a, b = rng.uniform(-1, 1, shape).astype(np.float16), rng.uniform(-1, 1, shape).astype(np.float16)
+        out = Guarded(shape, torch.float16)
+        ops.add(dev(a), dev(b), out.t, c)
+        want = oracle.c.add(a, b)
+    elif op == "add32":
+        a, b = rng.uniform(-1, 1, shape).astype(np.float32), rng.uniform(-1, 1, shape).astype(np.float32)
+        out = Guarded(shape, torch.float32)
+        ops.add(dev(a), dev(b), out.t, c)
+        want = oracle.c.add(a, b)
+    elif op == "add8":
+        a, b = rng.integers(-128, 128, shape).astype(np.int8), rng.integers(-128, 128, shape).astype(np.int8)
+        out = Guarded(shape, torch.int8)
+        ops.add(dev(a), dev(b), out.t, c)
+        want = oracle.c.add(a, b)
+    elif op == "castdown":
+        a = (rng.standard_normal(shape) * 100).astype(np.float32)
+        out = Guarded(shape, torch.float16)
+        ops.cast(dev(a), out.t, c)
+        want = oracle.c.cast(a, "float16")
+    else:
+        a = rng.standard_normal(shape).astype(np.float16)
+        out = Guarded(shape, torch.float32)
+        ops.cast(dev(a), out.t, c)
+        want = oracle.c.cast(a, "float32")
+    assert_bits_equal(out.check(), want)
+
+
+def test_grid_cap_makes_the_kernel_loop(oracle):
+    rng = np.random.default_rng(4)
+    a, b = rng.uniform(-1, 1, (300, 4096)).astype(np.float16), rng.uniform(-1, 1, (300, 4096)).astype(np.float16)
+    out = Guarded(a.shape, torch.float16)
+    ops.add(dev(a), dev(b), out.t, cfg(vec=8, unroll=2, grid_cap=7))
+    assert_bits_equal(out.check(), oracle.c.add(a, b))
+
+
+def test_odd_alignment_steps_down_to_element_accesses(oracle):
+    rng = np.random.default_rng(5)
+    base_a, base_b = rng.uniform(-1, 1, 5000).astype(np.float16), rng.uniform(-1, 1, 5000).astype(np.float16)
+    da, db = dev(base_a), dev(base_b)
+    raw = torch.full((5100,), 9.0, dtype=torch.float16, device="cuda")
+    ops.add(da[1:4998], db[1:4998], raw[3:5000])            # 2-byte aligned views
+    got = raw.cpu().numpy()
+    assert_bits_equal(got[3:5000], oracle.c.add(base_a[1:4998].copy(), base_b[1:4998].copy()))
+    assert (got[:3] == 9).all() and (got[5000:] == 9).all()
+    with pytest.raises(_lib.DtasError, match="not aligned"):  # an explicit vector config is taken at its word
+        ops.add(da[1:4998], db[1:4998], raw[3:5000], cfg(vec=8, unroll=1))
+
+
+def test_errors_on_the_gpu_path():
+    a = torch.zeros(4, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        ops.add(a, a, a)
+    with pytest.raises(ValueError):
+        ops.add(a, a, torch.zeros(4, 64, dtype=torch.float32, device="cuda"))
+    ops.add(a[:0], a[:0], torch.zeros(0, 64, dtype=torch.float16, device="cuda"))  # empty extent: no-op
+
+
+def test_full_size_properties():
+    # n = 8192 (the top of the dynamic range): add is commutative and copy(copy(x)) == x, bit for bit
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = (torch.rand(8192, 4096, device="cuda", generator=g) * 2 - 1).half()
+    b = (torch.rand(8192, 4096, device="cuda", generator=g) * 2 - 1).half()
+    ab, ba, c1, c2 = (torch.empty_like(a) for _ in range(4))
+    ops.add(a, b, ab)
+    ops.add(b, a, ba)
+    ops.copy(a, c1)
+    ops.copy(c1, c2)
+    torch.cuda.synchronize()
+    assert torch.equal(ab.view(torch.int16), ba.view(torch.int16))
+    assert torch.equal(c2.view(torch.int16), a.view(torch.int16))
+    # x + 0 == x and widening then narrowing is the identity on fp16
+    z, f32, back = torch.zeros_like(a), torch.empty(8192, 4096, device="cuda"), torch.empty_like(a)
+    ops.add(a, z, ab)
+    ops.cast(a, f32)
+    ops.cast(f32, back)
+    torch.cuda.synchronize()
+    assert torch.equal(ab.view(torch.int16), a.view(torch.int16))
+    assert torch.equal(back.view(torch.int16), a.view(torch.int16))
+    # checksum of the sum against an independent fp64 accumulation on the device
+    assert abs(ab.double().sum().item() - a.double().sum().item()) == 0

@@ -1,0 +1,153 @@
+"""GPU parity, decode GEMV and dynamic-M GEMM through the C ABI: against the fp32-accumulating CPU
+oracle and the float64 product (rtol 1e-2), exact special cases, every tile variant on ragged
+shapes.  At the large benchmark sizes the oracle is run on sampled rows of A (rows are independent)."""
+import numpy as np
+import pytest
+import torch
+
+from dtas_amd import _lib, ops
+from gpu_util import Guarded, assert_bits_equal, cfg, dev
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 2e-3
+
+
+def _check(got, oracle_out, f64):
+    got = got.astype(np.float64)
+    assert np.isfinite(got).all()
+    assert (np.abs(got - f64) <= ATOL + RTOL * np.abs(f64)).all()
+    # against the oracle (same fp32 arithmetic, another summation order): about one fp16 ulp
+    want = oracle_out.astype(np.float64)
+    assert (np.abs(got - want) <= 1e-3 + 2.0 ** -9 * np.abs(want)).all()
+
+
+def _inputs(M, N, K, seed):
+    rng = np.random.default_rng(seed)
+    return rng.standard_normal((M, K)).astype(np.float16), (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+
+
+GEMV_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
+
+
+@pytest.mark.parametrize("N,K", GEMV_SHAPES)
+def test_gemv_benchmark_config(oracle, N, K):
+    x, w = _inputs(1, N, K, 5)
+    out = Guarded((1, N), torch.float16)
+    ops.gemv(dev(x), dev(w), None, out.t)
+    _check(out.check(), oracle.c.gemm(x, w, threads=8), oracle.np64.gemm(x, w))
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 8])
+@pytest.mark.parametrize("block", [64, 256, 512])
+@pytest.mark.parametrize("N,K", [(2560, 10240), (1001, 2560), (7, 8), (130, 520)])
+def test_gemv_every_variant_and_bias(oracle, rows, block, N, K):
+    x, w = _inputs(1, N, K, N + K)
+    bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
+    out = Guarded((1, 1, N), torch.float16)
+    ops.gemv(dev(x), dev(w), dev(bias), out.t, cfg(variant=_lib.GEMV_SPLITK, block=block, vec=8, unroll=2, tile=[rows, 0, 0]))
+    _check(out.check().reshape(1, N), oracle.c.gemm(x, w, bias), oracle.np64.gemm(x, w, bias))
+
+
+def test_gemv_exact_and_ragged(oracle):
+    rng = np.random.default_rng(2)
+    w = (rng.standard_normal((96, 64)) * 0.02).astype(np.float16)
+    x = np.zeros((1, 64), np.float16)
+    x[0, 17] = 1
+    out = Guarded((1, 96), torch.float16)
+    ops.gemv(dev(x), dev(w), None, out.t)
+    assert_bits_equal(out.check().ravel(), w[:, 17].copy())       # one-hot x selects a column of W exactly
+    # K not a multiple of 8: element-access kernel
+    x, w = _inputs(1, 33, 1003, 3)
+    out = Guarded((1, 33), torch.float16)
+    ops.gemv(dev(x), dev(w), None, out.t)
+    _check(out.check(), oracle.c.gemm(x, w), oracle.np64.gemm(x, w))
+    with pytest.raises(_lib.DtasError, match="128-bit accesses"):
+        ops.gemv(dev(x), dev(w), None, out.t, cfg(variant=_lib.GEMV_SPLITK, block=256, vec=8, unroll=2, tile=[4, 0, 0]))
+
+
+NK = [(4096, 4096), (11008, 4096), (4096, 11008)]
+
+
+@pytest.mark.parametrize("N,K", NK)
+@pytest.mark.parametrize("M", [1, 16, 64, 256])
+def test_gemm_benchmark_config_small_m(oracle, M, N, K):
+    a, w = _inputs(M, N, K, 6)
+    out = Guarded((M, N), torch.float16)
+    ops.gemm(dev(a), dev(w), None, out.t)
+    _check(out.check(), oracle.c.gemm(a, w, threads=8), oracle.np64.gemm(a, w))
+
+
+@pytest.mark.parametrize("N,K", NK)
+@pytest.mark.parametrize("M", [1024, 2048, 4096, 8192])
+def test_gemm_benchmark_config_large_m_sampled_rows(oracle, M, N, K):
+    g = torch.Generator(device="cuda").manual_seed(6)
+    a = torch.randn(M, K, device="cuda", generator=g).half()
+    w = (torch.randn(N, K, device="cuda", generator=g) * 0.02).half()
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    ops.gemm(a, w, None, out)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())                           # every element was written
+    rows = np.unique(np.concatenate([[0, 1, 31, 32, 127, 128, 255, 256, M - 1], np.random.default_rng(M).integers(0, M, 7)]))
+    idx = torch.from_numpy(rows).cuda()
+    a_s, w_h = a[idx].cpu().numpy(), w.cpu().numpy()
+    _check(out[idx].cpu().numpy(), oracle.c.gemm(a_s, w_h, threads=8), oracle.np64.gemm(a_s, w_h))
+    # linearity over all rows: (sum_i C[i, :]) == (sum_i A[i, :]) . W^T, accumulated in fp64 on the device
+    lhs = out.double().sum(0)
+    rhs = a.double().sum(0) @ w.double().T
+    assert float((lhs - rhs).abs().max()) < 1e-3 * M ** 0.5 + 0.5     # fp16 rounding of M outputs per column
+
+
+TILES = [(256, 256), (256, 128), (128, 256), (128, 128), (64, 128), (128, 64), (64, 64)]
+
+
+@pytest.mark.parametrize("bm,bn", TILES)
+@pytest.mark.parametrize("M,N,K", [(5, 7, 8), (33, 65, 72), (300, 260, 200), (257, 513, 264), (512, 512, 64), (64, 64, 1024)])
+def test_gemm_every_mfma_tile_on_ragged_shapes(oracle, bm, bn, M, N, K):
+    a, w = _inputs(M, N, K, M + N + K)
+    bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
+    out = Guarded((1, M, N), torch.float16)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[bm, bn, 64]))
+    _check(out.check().reshape(M, N), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+
+
+@pytest.mark.parametrize("rows,block", [(16, 512), (16, 64), (32, 256), (48, 512), (64, 512), (80, 128)])
+@pytest.mark.parametrize("N,K", [(64, 64), (100, 520), (4096, 1000 * 8), (33, 40)])
+def test_gemm_every_skinny_tile(oracle, rows, block, N, K):
+    for M in (rows, rows - 3, 1):
+        a, w = _inputs(M, N, K, M + N + K)
+        out = Guarded((M, N), torch.float16)
+        ops.gemm(dev(a), dev(w), None, out.t, cfg(variant=_lib.GEMM_SKINNY, block=block, vec=8, unroll=4, tile=[rows, 16, 32]))
+        _check(out.check(), oracle.c.gemm(a, w, threads=8), oracle.np64.gemm(a, w))
+
+
+def test_gemm_exact_cases(oracle):
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal((300, 256)).astype(np.float16)
+    eye = np.eye(256, dtype=np.float16)
+    perm = rng.permutation(256)
+    for tile in ([256, 256, 64], [64, 64, 64], [128, 256, 64]):
+        out = Guarded(a.shape, torch.float16)
+        ops.gemm(dev(a), dev(eye[perm].copy()), None, out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=tile))
+        assert_bits_equal(out.check(), a[:, perm].copy())             # a permutation matrix permutes columns exactly
+    # an asymmetric case pins which operand is transposed and the accumulator layout
+    a = np.zeros((70, 64), np.float16)
+    w = np.zeros((90, 64), np.float16)
+    a[np.arange(70), np.arange(70) % 64] = np.arange(1, 71)
+    w[np.arange(90), (np.arange(90) * 7) % 64] = 1
+    out = Guarded((70, 90), torch.float16)
+    ops.gemm(dev(a), dev(w), None, out.t)
+    assert_bits_equal(out.check(), oracle.c.gemm(a, w))
+
+
+def test_gemm_k_not_multiple_of_8_and_errors(oracle):
+    a, w = _inputs(9, 20, 77, 9)
+    out = Guarded((9, 20), torch.float16)
+    ops.gemm(dev(a), dev(w), None, out.t)                            # element-access kernel
+    _check(out.check(), oracle.c.gemm(a, w), oracle.np64.gemm(a, w))
+    big, wb = _inputs(40, 20, 80, 9)
+    with pytest.raises(_lib.DtasError, match="cannot hold"):
+        ops.gemm(dev(big), dev(wb), None, torch.empty(40, 20, dtype=torch.float16, device="cuda"),
+                 cfg(variant=_lib.GEMM_SKINNY, block=512, vec=8, tile=[16, 16, 32]))
+    with pytest.raises(_lib.DtasError, match="128-bit accesses"):
+        ops.gemm(dev(a), dev(w), None, out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[64, 64, 64]))

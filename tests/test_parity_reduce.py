@@ -1,0 +1,177 @@
+"""GPU parity, RMSNorm / LayerNorm / softmax through the C ABI against the CPU oracle and the
+float64 closed forms; tolerance atol 1e-2 (fp16 outputs, fp32 accumulation in another order)."""
+import numpy as np
+import pytest
+import torch
+
+from dtas_amd import _lib, ops
+from gpu_util import Guarded, cfg, dev
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 1e-2          # the benchmark's stated tolerance
+ATOL_ORACLE = 1e-3   # against the fp32 oracle the only differences are summation order and exp /
+RTOL_ORACLE = 2.0 ** -10  # rsqrt ulps: at most one fp16 ulp of the result (plus a small absolute term)
+
+
+def _check(got, oracle_out, f64):
+    got = got.astype(np.float64)
+    assert np.isfinite(got).all()
+    assert np.abs(got - f64).max() < ATOL
+    want = oracle_out.astype(np.float64)
+    assert (np.abs(got - want) <= ATOL_ORACLE + RTOL_ORACLE * np.abs(want)).all()
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 7, 16, 128, 257, 513, 1024, 4096])
+def test_rms_norm_benchmark_config(oracle, n):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((n, 4096)).astype(np.float16)
+    w = rng.uniform(0.5, 1.5, 4096).astype(np.float16)
+    out = Guarded(x.shape, torch.float16)
+    ops.rms_norm(dev(x), dev(w), out.t)
+    _check(out.check(), oracle.c.rms_norm(x, w, threads=8), oracle.np64.rms_norm(x, w))
+
+
+@pytest.mark.parametrize("H", [8, 64, 2560, 8192, 16384, 100, 4100, 12001])
+def test_rms_norm_other_row_lengths(oracle, H):
+    rng = np.random.default_rng(H)
+    x = rng.standard_normal((5, H)).astype(np.float16)
+    w = rng.uniform(0.5, 1.5, H).astype(np.float16)
+    out = Guarded(x.shape, torch.float16)
+    ops.rms_norm(dev(x), dev(w), out.t)
+    _check(out.check(), oracle.c.rms_norm(x, w), oracle.np64.rms_norm(x, w))
+
+
+RED_VARIANTS = [(_lib.RED_WAVE_ROW, b) for b in (64, 128, 256, 512)] + \
+               [(_lib.RED_BLOCK_ROW, b) for b in (64, 256, 512, 1024)] + [(_lib.RED_STREAM_ROW, b) for b in (64, 256, 1024)]
+
+
+@pytest.mark.parametrize("variant,block", RED_VARIANTS)
+@pytest.mark.parametrize("n,H", [(1, 4096), (9, 4096), (130, 2560), (6, 8192)])
+def test_rms_norm_every_variant(oracle, variant, block, n, H):
+    rng = np.random.default_rng(n + H)
+    x = rng.standard_normal((n, H)).astype(np.float16)
+    w = rng.uniform(0.5, 1.5, H).astype(np.float16)
+    out = Guarded(x.shape, torch.float16)
+    vec = 1 if variant == _lib.RED_STREAM_ROW else 8
+    ops.rms_norm(dev(x), dev(w), out.t, cfg=cfg(variant=variant, block=block, vec=vec))
+    _check(out.check(), oracle.c.rms_norm(x, w), oracle.np64.rms_norm(x, w))
+
+
+def test_rms_norm_grid_cap_and_invariants(oracle):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((1000, 4096)).astype(np.float16)
+    w = np.ones(4096, np.float16)
+    for variant in (_lib.RED_WAVE_ROW, _lib.RED_BLOCK_ROW):
+        out = Guarded(x.shape, torch.float16)
+        ops.rms_norm(dev(x), dev(w), out.t, cfg=cfg(variant=variant, block=256, vec=8, grid_cap=13))
+        got = out.check()
+        _check(got, oracle.c.rms_norm(x, w, threads=8), oracle.np64.rms_norm(x, w))
+        assert np.abs(np.sqrt((got.astype(np.float64) ** 2).mean(-1)) - 1).max() < 2e-3   # unit rms with w = 1
+
+
+@pytest.mark.parametrize("n", [1, 3, 100, 257, 1024, 4096])
+def test_layer_norm_reference_signature(oracle, n):
+    rng = np.random.default_rng(13)
+    x = (rng.standard_normal((1, n, 2560)) * 2 + 0.5).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, 2560).astype(np.float32)
+    b = rng.uniform(-1, 1, 2560).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    ops.layer_norm(dev(x), dev(g), dev(b), out.t)
+    _check(out.check(), oracle.c.layer_norm(x, g, b, threads=8), oracle.np64.layer_norm(x, g, b))
+
+
+@pytest.mark.parametrize("variant,block", RED_VARIANTS)
+def test_layer_norm_every_variant(oracle, variant, block):
+    rng = np.random.default_rng(14)
+    x = (rng.standard_normal((11, 2560)) * 2 + 0.5).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, 2560).astype(np.float32)
+    b = rng.uniform(-1, 1, 2560).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    vec = 1 if variant == _lib.RED_STREAM_ROW else 4
+    ops.layer_norm(dev(x), dev(g), dev(b), out.t, cfg=cfg(variant=variant, block=block, vec=vec))
+    _check(out.check(), oracle.c.layer_norm(x, g, b), oracle.np64.layer_norm(x, g, b))
+
+
+def test_layer_norm_odd_row_length(oracle):
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal((4, 1001)).astype(np.float32)
+    g, b = rng.uniform(0.5, 1.5, 1001).astype(np.float32), rng.uniform(-1, 1, 1001).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    ops.layer_norm(dev(x), dev(g), dev(b), out.t)
+    _check(out.check(), oracle.c.layer_norm(x, g, b), oracle.np64.layer_norm(x, g, b))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 7, 8, 16, 31, 64, 128, 257, 512, 1024])
+def test_softmax_f16_benchmark_config(oracle, n):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((32 * n, n)) * 2).astype(np.float16)
+    out = Guarded(x.shape, torch.float16)
+    ops.softmax(dev(x), out.t)
+    got = out.check()
+    _check(got, oracle.c.softmax(x, threads=8), oracle.np64.softmax(x))
+    assert np.abs(got.astype(np.float64).sum(-1) - 1).max() < n * 2.0 ** -11 + 1e-3
+
+
+@pytest.mark.parametrize("n", [2048, 4096])
+def test_softmax_f16_large_rows_sampled(oracle, n):
+    # [32n, n] is up to 1 GiB: run all of it, compare sampled rows with the oracle, row sums for all
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x = (torch.randn(32 * n, n, device="cuda", generator=g) * 2).half()
+    out = torch.empty_like(x)
+    ops.softmax(x, out)
+    torch.cuda.synchronize()
+    rows = np.unique(np.concatenate([[0, 1, 32 * n - 1], np.random.default_rng(n).integers(0, 32 * n, 61)]))
+    xs = x[torch.from_numpy(rows).cuda()].cpu().numpy()
+    got = out[torch.from_numpy(rows).cuda()].cpu().numpy()
+    _check(got, oracle.c.softmax(xs), oracle.np64.softmax(xs))
+    sums = out.float().sum(-1)
+    assert float((sums - 1).abs().max()) < n * 2.0 ** -11 + 1e-3
+    assert bool((out.argmax(-1) == x.argmax(-1)).float().mean() > 0.999)  # ties in fp16 aside
+
+
+@pytest.mark.parametrize("rows,cols", [(12800, 400), (1000, 1000), (32 * 5, 4096), (7, 8192), (3, 3000), (5, 20000)])
+def test_softmax_f32_reference_signature(oracle, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((1, rows, cols)) * 2).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    ops.softmax(dev(x), out.t)
+    _check(out.check(), oracle.c.softmax(x, threads=8), oracle.np64.softmax(x))
+
+
+@pytest.mark.parametrize("variant,block", RED_VARIANTS)
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_softmax_every_variant(oracle, variant, block, dtype):
+    rng = np.random.default_rng(16)
+    x = (rng.standard_normal((19, 2048)) * 2).astype(dtype)
+    out = Guarded(x.shape, torch.float16)
+    vec = 1 if variant == _lib.RED_STREAM_ROW else (8 if dtype == np.float16 else 4)
+    ops.softmax(dev(x), out.t, cfg=cfg(variant=variant, block=block, vec=vec))
+    _check(out.check(), oracle.c.softmax(x), oracle.np64.softmax(x))
+
+
+def test_softmax_special_rows(oracle):
+    x = np.zeros((4, 64), np.float16)
+    x[0] = -3.0                      # constant row -> 1/64 exactly
+    x[1, 5] = 30000                  # one dominant entry
+    x[2] = np.linspace(-60000, 60000, 64).astype(np.float16)
+    x[3, :] = -np.inf
+    x[3, 7] = 0                      # -inf entries contribute exactly zero
+    out = Guarded(x.shape, torch.float16)
+    ops.softmax(dev(x), out.t)
+    got = out.check()
+    assert (got[0] == np.float16(1 / 64)).all()
+    assert got[1, 5] == 1 and got[1].sum() == 1
+    assert got[3, 7] == 1 and got[3].sum() == 1
+    assert np.abs(got.astype(np.float64) - oracle.c.softmax(x).astype(np.float64)).max() < 2e-3
+
+
+def test_reduction_errors():
+    x = torch.zeros(4, 100, dtype=torch.float16, device="cuda")
+    w = torch.ones(100, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="128-bit row accesses"):
+        ops.rms_norm(x, w, torch.empty_like(x), cfg=cfg(variant=_lib.RED_WAVE_ROW, block=256, vec=8))
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        ops.rms_norm(x, w, x)
+    with pytest.raises(_lib.DtasError, match="block must be"):
+        ops.rms_norm(x, w, torch.empty_like(x), cfg=cfg(variant=_lib.RED_STREAM_ROW, block=100, vec=1))
