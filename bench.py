@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the DTAS hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-sweep] [--no-cpu]
+
+A "step" is one call of the workload's kernel through the C ABI on synthetic, seeded inputs that are
+already resident in device memory.  The headline workload is the elementwise fp32 -> fp16 cast over
+[4096, 4096] (the largest n of the elementwise sweep); buffers rotate through a pool larger than the
+256 MiB Infinity Cache so that every step streams from HBM.  W warm-up steps, then exactly K timed
+steps between two device synchronisations; `value` = algorithmic bytes * K / that time.
+
+The same JSON line also carries
+  roofline     : the workload's kernel against MI355X's published peak (HBM 8 TB/s, or dense fp16
+                 MFMA 2.5 PFLOP/s for the GEMM workloads); `achieved` uses the average per-launch
+                 duration measured with HIP events on the launch stream inside the timed region;
+  cpu_baseline : the CPU oracle (a port of the PrimFunc loop nest, oracle/cpu_ref.c) on a bounded
+                 sample of the same workload, on this machine's host cores;
+  sweep        : every op family over the dynamic extent n (GB/s or TFLOP/s and roofline fraction),
+                 HBM-streaming (rotating buffers) unless marked cache-resident.
+One GPU only: `--gpus N` with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # dense fp16 -> fp32 MFMA
+INFINITY_CACHE_BYTES = 256 << 20
+METRIC = "achieved HBM GB/s (eltwise/reduce/GEMV) + GEMM TFLOP/s, swept over dynamic n"
+
+
+# ---------------------------------------------------------------------------------------------
+# workloads: name -> builder returning (make_buffers(seed) -> tuple, run(buffers), bytes, flops, kernel)
+# ---------------------------------------------------------------------------------------------
+def _workload(name: str, n: int, extra=None):
+    import torch
+
+    from dtas_amd import ops
+
+    H = 4096
+    g = torch.Generator(device="cuda")
+
+    def uniform(shape, seed, lo=-1.0, hi=1.0, dtype=torch.float16):
+        g.manual_seed(seed)
+        return (torch.rand(shape, device="cuda", generator=g) * (hi - lo) + lo).to(dtype)
+
+    def normal(shape, seed, std=1.0, dtype=torch.float16):
+        g.manual_seed(seed)
+        return (torch.randn(shape, device="cuda", generator=g) * std).to(dtype)
+
+    if name == "add_f16":
+        make = lambda s: (uniform((n, H), 2 * s), uniform((n, H), 2 * s + 1), torch.empty(n, H, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.add(b[0], b[1], b[2]), 3 * 2 * n * H, 0
+    if name == "copy_f16":
+        make = lambda s: (normal((n, H), s, 100.0), torch.empty(n, H, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.copy(b[0], b[1]), 2 * 2 * n * H, 0
+    if name == "cast_f32_f16":
+        make = lambda s: (normal((n, H), s, 100.0, torch.float32), torch.empty(n, H, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.cast(b[0], b[1]), (4 + 2) * n * H, 0
+    if name == "cast_f16_f32":
+        make = lambda s: (normal((n, H), s, 100.0), torch.empty(n, H, dtype=torch.float32, device="cuda"))
+        return make, lambda b: ops.cast(b[0], b[1]), (4 + 2) * n * H, 0
+    if name == "rms_norm_f16":
+        w = uniform((H,), 3, 0.5, 1.5)
+        make = lambda s: (normal((n, H), s), w, torch.empty(n, H, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.rms_norm(b[0], b[1], b[2]), 2 * 2 * n * H + 2 * H, 0
+    if name == "layer_norm_f32_f16":
+        Hr = 2560
+        gm, bt = uniform((Hr,), 3, 0.5, 1.5, torch.float32), uniform((Hr,), 4, -1, 1, torch.float32)
+        make = lambda s: (normal((n, Hr), s, 1.0, torch.float32), gm, bt, torch.empty(n, Hr, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.layer_norm(b[0], b[1], b[2], b[3]), (4 + 2) * n * Hr + 8 * Hr, 0
+    if name == "softmax_f16":
+        R = 32 * n
+        make = lambda s: (normal((R, n), s, 2.0), torch.empty(R, n, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.softmax(b[0], b[1]), 2 * 2 * R * n, 0
+    if name == "gemv_f16":
+        N, K = extra
+        make = lambda s: (normal((1, K), s), normal((N, K), s + 100, 0.02), torch.empty(1, N, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.gemv(b[0], b[1], None, b[2]), 2 * N * K + 2 * K + 2 * N, 2 * N * K
+    if name == "gemm_f16":
+        N, K = extra
+        wt = normal((N, K), 100, 0.02)
+        make = lambda s: (normal((n, K), s), wt, torch.empty(n, N, dtype=torch.float16, device="cuda"))
+        return make, lambda b: ops.gemm(b[0], b[1], None, b[2]), 2 * (n * K + N * K + n * N), 2 * n * N * K
+    raise ValueError(f"unknown workload {name}")
+
+
+def _pool_bytes(bufs) -> int:
+    seen, total = set(), 0
+    for t in bufs:
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    return total
+
+
+def make_pool(make, streaming: bool, max_bytes: int = 6 << 30):
+    """Buffer sets to rotate through: enough distinct sets that a set has left the Infinity Cache
+    before it is used again (>= 3x its capacity), one set when cache-resident timing is wanted."""
+    first = make(0)
+    if not streaming:
+        return [first]
+    per = max(1, _pool_bytes(first))
+    count = max(2, min(64, -(-3 * INFINITY_CACHE_BYTES // per)))
+    count = max(2, min(count, max_bytes // per))
+    return [first] + [make(i) for i in range(1, count)]
+
+
+def time_kernel(run, pool, steps: int, warmup: int):
+    """(wall seconds for `steps` calls between two synchronisations, device seconds for the same
+    region from a pair of HIP events recorded on the launch stream before the first and after the
+    last call).  Launches are issued back to back, so device seconds / steps is the average launch
+    duration (kernel time plus the inter-kernel gap, which is what a caller sees)."""
+    import torch
+
+    for i in range(warmup):
+        run(pool[i % len(pool)])
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        run(pool[(warmup + i) % len(pool)])
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, start.elapsed_time(stop) * 1e-3 / steps
+
+
+def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool = True) -> dict:
+    make, run, nbytes, flops = _workload(name, n, extra)
+    pool = make_pool(make, streaming)
+    wall, mean_launch = time_kernel(run, pool, steps, warmup)
+    median_launch = mean_launch
+    out = {"op": name, "n": n, "us": round(mean_launch * 1e6, 3), "us_mean": round(mean_launch * 1e6, 3),
+           "ms_per_step": wall * 1e3 / steps, "bytes": nbytes, "flops": flops, "pool": len(pool),
+           "gbs": nbytes / median_launch / 1e9}
+    if extra:
+        out["NK"] = list(extra)
+    if flops and name == "gemm_f16":
+        out["tflops"] = flops / median_launch / 1e12
+        hbm_bound_s = nbytes / (HBM_PEAK_GBS * 1e9)
+        mfma_bound_s = flops / (MFMA_FP16_PEAK_TFLOPS * 1e12)
+        out["bound"] = "mfma" if mfma_bound_s >= hbm_bound_s else "hbm"
+        out["frac"] = (out["tflops"] / MFMA_FP16_PEAK_TFLOPS) if out["bound"] == "mfma" else out["gbs"] / HBM_PEAK_GBS
+    else:
+        out["bound"] = "hbm"
+        out["frac"] = out["gbs"] / HBM_PEAK_GBS
+    del pool
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+def cpu_baseline(name: str, n: int, budget_s: float = 12.0) -> dict:
+    """The CPU oracle on a bounded sample of the headline workload (1 thread = what an unscheduled
+    PrimFunc built for an llvm CPU target executes; all host cores reported beside it)."""
+    import numpy as np
+
+    import oracle
+
+    oracle.build()
+    H = 4096
+    rng = np.random.default_rng(2)
+    if name == "cast_f32_f16":
+        x = (rng.standard_normal((n, H)) * 100).astype(np.float32)
+        fn = lambda th: oracle.c.cast(x, "float16", threads=th)
+        nbytes = 6 * n * H
+    elif name == "add_f16":
+        a = rng.uniform(-1, 1, (n, H)).astype(np.float16)
+        b = rng.uniform(-1, 1, (n, H)).astype(np.float16)
+        fn = lambda th: oracle.c.add(a, b, threads=th)
+        nbytes = 6 * n * H
+    elif name == "copy_f16":
+        a = rng.standard_normal((n, H)).astype(np.float16)
+        fn = lambda th: oracle.c.copy(a, threads=th)
+        nbytes = 4 * n * H
+    else:
+        x = rng.standard_normal((n, H)).astype(np.float16)
+        w = rng.uniform(0.5, 1.5, H).astype(np.float16)
+        fn = lambda th: oracle.c.rms_norm(x, w, threads=th)
+        nbytes = 4 * n * H + 2 * H
+
+    def run(threads: int, budget: float):
+        fn(threads)  # page in
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn(threads)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el > budget or reps >= 200:
+                return nbytes * reps / el / 1e9, reps
+
+    cores = min(oracle.c.max_threads(), len(os.sched_getaffinity(0)))
+    one, reps1 = run(1, budget_s * 0.6)
+    many, repsn = run(cores, budget_s * 0.4)
+    return {"value": round(one, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{name} n={n} H={H}, {reps1} full passes of the oracle (oracle/cpu_ref.c), 1 thread",
+            "all_cores": {"value": round(many, 3), "cores": cores, "passes": repsn}}
+
+
+# ---------------------------------------------------------------------------------------------
+SWEEP_N = [1, 16, 128, 1024, 4096]
+SWEEP_M = [1, 16, 64, 256, 1024, 2048, 4096, 8192]
+GEMV_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
+GEMM_NK = [(4096, 4096), (11008, 4096), (4096, 11008)]
+
+
+def sweep(steps: int, warmup: int) -> list:
+    rows = []
+    for op in ("add_f16", "copy_f16", "cast_f32_f16", "cast_f16_f32", "rms_norm_f16", "layer_norm_f32_f16", "softmax_f16"):
+        for n in SWEEP_N:
+            rows.append(measure(op, n, None, steps, warmup))
+    for nk in GEMV_SHAPES:
+        rows.append(measure("gemv_f16", 1, nk, steps, warmup))
+    for nk in GEMM_NK:
+        for m in SWEEP_M:
+            rows.append(measure("gemm_f16", m, nk, max(5, steps // 2), max(2, warmup // 2), streaming=m < 2048))
+    return rows
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cast_f32_f16",
+                    help="cast_f32_f16 | add_f16 | copy_f16 | rms_norm_f16 | softmax_f16 | gemv_f16 | gemm_f16")
+    ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
+    ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cache-resident", action="store_true", help="time on one buffer set (no rotation)")
+    ap.add_argument("--out", default=None, help="also write the sweep rows to this JSON file")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: every kernel here runs on a single device and no collective exists "
+              f"(--gpus {args.gpus} is not supported)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from dtas_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the kernels have no CPU path)", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    if _lib.lib().dtas_init() != 0:
+        print(_lib.last_error(), file=sys.stderr)
+        return 2
+
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemm_f16") else None
+    head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
+    is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
+    info = None
+    try:
+        op = {"cast_f32_f16": _lib.OP_CAST_F32_F16, "add_f16": _lib.OP_ADD_F16, "copy_f16": _lib.OP_COPY_F16,
+              "rms_norm_f16": _lib.OP_RMS_NORM_F16}.get(args.workload)
+        if op is not None:
+            info = _lib.select_bucket(op, args.n, 4096, 0)
+    except _lib.DtasError:
+        info = None
+
+    line = {
+        "metric": METRIC,
+        "value": round(head["flops"] * args.steps / (head["ms_per_step"] * 1e-3 * args.steps) / 1e12, 3) if is_gemm
+        else round(head["bytes"] / (head["ms_per_step"] * 1e-3) / 1e9, 3),
+        "unit": "TFLOP/s" if is_gemm else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{args.workload} [n={args.n}, 4096]" if extra is None else f"{args.workload} M={args.n} NxK={args.nk}",
+                   "buffers": "rotating pool > 3x Infinity Cache" if not args.cache_resident else "single set (cache-resident)",
+                   "pool_sets": head["pool"],
+                   "kernel": info.name.decode() if info is not None else args.workload,
+                   "launch": list(info.launch_args)[:5] if info is not None else None},
+        "roofline": {
+            "bound": "mfma" if is_gemm else "hbm",
+            "achieved": round(head["tflops"], 3) if is_gemm else round(head["bytes"] / (head["us_mean"] * 1e-6) / 1e9, 3),
+            "peak": MFMA_FP16_PEAK_TFLOPS if is_gemm else HBM_PEAK_GBS,
+            "unit": "TFLOP/s" if is_gemm else "GB/s",
+            "frac": round((head["tflops"] / MFMA_FP16_PEAK_TFLOPS) if is_gemm
+                          else head["bytes"] / (head["us_mean"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "launch_us_mean": head["us_mean"],
+            "algorithmic_bytes_per_launch": head["bytes"],
+        },
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args.workload if args.workload in ("cast_f32_f16", "add_f16", "copy_f16") else "rms_norm_f16",
+                                            min(args.n, 4096))
+    else:
+        line["cpu_baseline"] = None
+    if not args.no_sweep:
+        rows = sweep(max(10, args.steps // 2), max(3, args.warmup // 2))
+        line["sweep"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
+                          if k in ("op", "n", "NK", "us", "gbs", "tflops", "bound", "frac")} for r in rows]
+        if args.out:
+            with open(args.out, "w") as f:
+                json.dump(rows, f, indent=1)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -118,7 +118,8 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
       pick = i;
     }
   }
-  return make(DTAS_GEMM_MFMA, 256, 8, 1, kTiles[pick].bm, kTiles[pick].bn, 64);
+  const int threads = kTiles[pick].bm == 256 && kTiles[pick].bn == 256 ? 512 : 256;
+  return make(DTAS_GEMM_MFMA, threads, 8, 1, kTiles[pick].bm, kTiles[pick].bn, 64);
 }
 
 dtas_config policy(int op, int64_t n_hi, int64_t d0, int64_t d1) {

@@ -7,22 +7,30 @@
 // two-stage software pipeline, accumulators through shared memory to a guarded vector
 // store; example output experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py).
 //
-// MI355X shape
-//   MFMA   : 256 threads = 4 wavefronts in a 2x2 grid; a wavefront owns (BM/2)x(BN/2) of the
-//            BMxBN tile as 32x32 blocks of v_mfma_f32_32x32x16_f16, accumulators in registers
-//            (256 per lane for the 256x256 tile).  K advances 64 at a time; both operands are
-//            K-contiguous, so a tile row is one 128-byte line = 8 chunks of 16 bytes.
-//            Global -> registers with 128-bit buffer loads (rows past M / N read as zero by the
-//            buffer's range check), registers -> LDS, LDS -> MFMA operands with 128-bit reads.
-//            LDS is double buffered (2 x (BM+BN) x 128 B, 128 KiB of the 160 KiB for 256x256):
-//            the loads of tile k+1 are in flight while tile k is multiplied, one barrier per
-//            k tile.  The LDS placement of chunk c of row r is swizzled so that both the
-//            row-major writes and the column-of-rows MFMA reads spread over all banks.
-//            Workgroup ids are remapped so that each XCD (own L2) works on a compact patch of
-//            the tile grid.
-//   SKINNY : M <= 64 (kernels exist up to 80 rows).  The work is streaming W once; a workgroup owns 16 columns of C and all
-//            of M, its wavefronts split K, v_mfma_f32_16x16x32_f16 operands are loaded
-//            straight from global memory, partial tiles are folded through LDS.
+// MFMA kernel (M > 64)
+//   tile     : BM x BN x 64 per workgroup; WM x WN wavefronts (8 for 256x256, else 4), each owning
+//              (BM/WM) x (BN/WN) as 32x32 blocks of v_mfma_f32_32x32x16_f16, fp32 accumulators
+//              in registers.  Both operands are K-contiguous, so a tile row is one 128-byte
+//              line = 8 chunks of 16 bytes.
+//   global   : 128-bit buffer loads that write LDS directly (no register staging, no
+//              ds_write): one wavefront instruction fills one 1 KiB block = 8 tile rows; which
+//              (row, chunk) a lane fetches is the inverse of the LDS swizzle.  Rows past M / N
+//              and chunks past K fall outside the buffer's range and arrive as zeros.
+//   LDS      : two stages of (BM + BN) x 128 B.  Chunk c of row r sits at a swizzled slot so
+//              that the MFMA operand reads (a column of 32 rows per half-wavefront, 128 bit
+//              per lane) spread over all 64 banks.
+//   pipeline : fragments of step s+1 are read from LDS while the MFMAs of step s issue (two
+//              register sets); the tile barrier sits before the last step of a k tile, the
+//              loads of tile k+2 are issued right after it into the stage just vacated, and the
+//              first fragments of tile k+1 are read under the last MFMAs of tile k.  The
+//              interleaving is pinned with scheduling barriers.
+//   epilogue : accumulators -> fp16 -> wavefront-private LDS region (xor-swizzled 8-byte
+//              slots) -> 8-byte coalesced row stores with the bias added on the way out.
+//   launch   : workgroup ids are remapped so that each XCD (own L2) works on a compact patch of
+//              the tile grid.
+// SKINNY kernel (M <= 64): the work is streaming W once; a workgroup owns 16 columns of C and
+//              all of M, its wavefronts split K, v_mfma_f32_16x16x32_f16 operands are loaded
+//              straight from global memory, partial tiles are folded through LDS.
 #include "dtas_device.h"
 #include "dtas_host.h"
 
@@ -62,18 +70,27 @@ __device__ __forceinline__ unsigned xcd_contiguous_id(unsigned wg, unsigned tota
   return xcd * base + (xcd < rem ? xcd : rem) + local;
 }
 
-template <int BM, int BN>
-__global__ void __launch_bounds__(256) gemm_mfma_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
-                                                        const half_t* __restrict__ bias, half_t* __restrict__ C,
-                                                        int64_t M, int64_t N, int64_t K, unsigned tiles_m,
-                                                        unsigned tiles_n) {
-  constexpr int WTM = BM / 2, WTN = BN / 2;  // wavefront tile
-  constexpr int MT = WTM / 32, NT = WTN / 32;
-  constexpr int LA = BM / 32, LB = BN / 32;  // 128-bit loads per thread per k tile
+#define DTAS_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <int BM, int BN, int WM, int WN>
+__global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
+                                                                 const half_t* __restrict__ W,
+                                                                 const half_t* __restrict__ bias,
+                                                                 half_t* __restrict__ C, int64_t M, int64_t N,
+                                                                 int64_t K, unsigned tiles_m, unsigned tiles_n) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;  // wavefront tile
+  constexpr int MT = WTM / 32, NT = WTN / 32;  // 32x32 blocks per wavefront
+  constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;  // 1 KiB block loads per wavefront per k tile
   constexpr int kABytes = BM * kRowBytes, kStage = (BM + BN) * kRowBytes;
+  static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
+  static_assert(BM * BN * 2 <= 2 * kStage, "epilogue staging must fit the operand stages");
   __shared__ __attribute__((aligned(1024))) char lds[2 * kStage];
 
-  const unsigned t = threadIdx.x, l = t & 63u, wv = t >> 6, wm = wv >> 1, wn = wv & 1u;
+  const unsigned t = threadIdx.x, l = t & 63u;
+  const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
 
   // ---- which tile: XCD-contiguous order, then groups of 8 tile rows walked column-wise
   const unsigned total = tiles_m * tiles_n;
@@ -85,22 +102,23 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const half_t* __restrict
   const unsigned tm = first_m + (pid % width) % gsize, tn = (pid % width) / gsize;
   const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
 
-  // ---- global side: chunk ld_c of rows ld_r + 32*i; rows past the operand's end are out of
-  // the buffer's range and read as zero
+  // ---- global side.  Lane p of a block load fills 16-byte slot p of the block, so it fetches
+  // the (row, chunk) that lds_chunk_offset places there; the block index of wavefront w's i-th
+  // load is i*NW + w, whose parity is w's (NW is even).
   const int64_t rows_a = M - m0 < BM ? M - m0 : BM, rows_w = N - n0 < BN ? N - n0 : BN;
   const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(A + m0 * K, static_cast<unsigned>(rows_a) * row_bytes);
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
-  const unsigned ld_r = t >> 3, ld_c = t & 7u;
-  const unsigned g_off = ld_r * row_bytes + ld_c * 16u;
-  const unsigned g_step = 32u * row_bytes;
-  const unsigned lds_wr = lds_chunk_offset(ld_r, ld_c);  // + i * 4096 for row ld_r + 32*i
+  const unsigned r_in = 2u * (l >> 4) + (((l >> 3) & 1u) ^ (wv & 1u));  // row inside the 8-row block
+  const unsigned c_in = (l & 7u) ^ r_in;                                // chunk of that row
+  const unsigned g_off = (8u * wv + r_in) * row_bytes + c_in * 16u;
+  const unsigned g_step = 8u * NW * row_bytes;
 
   // ---- LDS -> MFMA operands: lane l supplies row (l & 31), chunk 2*ks + (l >> 5)
   unsigned lds_rd[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) lds_rd[ks] = lds_chunk_offset(l & 31u, 2u * ks + (l >> 5));
-  const unsigned a_base = wm * (WTM / 2) * 256u, b_base = kABytes + wn * (WTN / 2) * 256u;
+  const unsigned a_base = wm * WTM * 128u, b_base = kABytes + wn * WTN * 128u;
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -111,66 +129,127 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(const half_t* __restrict
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int ktiles = static_cast<int>((K + kBK - 1) / kBK);
-  u32x4 sa[LA], sb[LB];
 
+  // tile kt -> LDS stage kt & 1, asynchronously (completion is counted by vmcnt)
   auto fetch = [&](int kt) {
-    const unsigned kb = static_cast<unsigned>(kt) * kRowBytes;
     // a chunk past K is pointed out of range; K % 8 == 0, so chunks are all-in or all-out
-    const unsigned off = (static_cast<int64_t>(kt) * kBK + ld_c * 8 < K) ? g_off + kb : kOob;
+    const unsigned off = (static_cast<int64_t>(kt) * kBK + c_in * 8 < K)
+                             ? g_off + static_cast<unsigned>(kt) * kRowBytes : kOob;
+    char* base = lds + (kt & 1) * kStage + wv * 1024;
 #pragma unroll
-    for (int i = 0; i < LA; ++i) sa[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, off + i * g_step, 0, 0);
+    for (int i = 0; i < LA; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < LB; ++i) sb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, off + i * g_step, 0, 0);
-  };
-  auto stash = [&](int buf) {
-    char* base = lds + buf * kStage + lds_wr;
-#pragma unroll
-    for (int i = 0; i < LA; ++i) *reinterpret_cast<u32x4*>(base + i * 4096) = sa[i];
-#pragma unroll
-    for (int i = 0; i < LB; ++i) *reinterpret_cast<u32x4*>(base + kABytes + i * 4096) = sb[i];
+    for (int i = 0; i < LB; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16,
+                                               off + i * g_step, 0, 0, 0);
   };
 
-  if (ktiles > 0) {
-    fetch(0);
-    stash(0);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const bool more = kt + 1 < ktiles;
-    if (more) fetch(kt + 1);
-    const char* buf = lds + (kt & 1) * kStage;
+  f16x8 fa[2][MT], fb[2][NT];
+  auto read_a = [&](int set, int i, const char* stage, int ks) {
+    fa[set][i] = *reinterpret_cast<const f16x8*>(stage + a_base + i * 4096 + lds_rd[ks]);
+  };
+  auto read_b = [&](int set, int j, const char* stage, int ks) {
+    fb[set][j] = *reinterpret_cast<const f16x8*>(stage + b_base + j * 4096 + lds_rd[ks]);
+  };
+  // The MT*NT MFMAs of register set `set`, with the MT+NT fragment reads of the next step (from
+  // `stage`, step `ks`, into the other set) spread evenly between them.  W rows are the first MFMA
+  // operand, so a lane ends up with 4 consecutive columns of one C row per accumulator quad.
+  auto step = [&](int set, const char* stage, int ks, bool reads) {
+    constexpr int kReads = MT + NT, kMfma = MT * NT;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      f16x8 fa[MT], fb[NT];
+    for (int q = 0; q < kMfma; ++q) {
+      if (reads) {
 #pragma unroll
-      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const f16x8*>(buf + a_base + i * 4096 + lds_rd[ks]);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const f16x8*>(buf + b_base + j * 4096 + lds_rd[ks]);
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) stash((kt + 1) & 1);
-    __syncthreads();
-  }
-
-  // ---- accumulators -> C: register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
-  // of its 32x32 block
-  const int64_t col_l = l & 31u, row_l = 4 * (l >> 5);
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const int64_t col = n0 + wn * WTN + j * 32 + col_l;
-      if (col < N) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int64_t row = m0 + wm * WTM + i * 32 + 8 * (v / 4) + row_l + (v % 4);
-          if (row < M) C[row * N + col] = finish(acc[i][j][v], bias, col);
+        for (int r = 0; r < kReads; ++r) {
+          if (r * kMfma / kReads == q) {
+            if (r < MT) read_a(set ^ 1, r, stage, ks); else read_b(set ^ 1, r - MT, stage, ks);
+          }
         }
       }
+      const int i = q / NT, j = q % NT;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+      DTAS_SCHED_FENCE();
+    }
+  };
+
+  // prologue: tile 0 resident, tile 1 in flight, fragments of (tile 0, step 0) in registers
+  if (ktiles > 0) fetch(0);
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  DTAS_SCHED_FENCE();
+  if (ktiles > 1) fetch(1);
+  if (ktiles > 0) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) read_b(0, j, lds, 0);
+  }
+  DTAS_SCHED_FENCE();
+
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const char* cur = lds + (kt & 1) * kStage;
+    const char* nxt = lds + ((kt + 1) & 1) * kStage;
+    step(0, cur, 1, true);
+    step(1, cur, 2, true);
+    step(0, cur, 3, true);
+    // tile kt+1 has landed and every wavefront has finished reading tile kt
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    if (kt + 2 < ktiles) fetch(kt + 2);  // into the stage tile kt occupied
+    DTAS_SCHED_FENCE();
+    step(1, nxt, 0, kt + 1 < ktiles);
+  }
+
+  // ---- epilogue.  acc[i][j][v] of lane l is C row i*32 + (l & 31), column
+  // j*32 + 8*(v/4) + 4*(l >> 5) + v%4 of the wavefront tile.  Each wavefront stages its tile in a
+  // private LDS region of WTM rows x WTN fp16 (8-byte slots, xor-swizzled by the row) and writes
+  // it out as 8-byte accesses that are contiguous along the row.
+  constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots;
+  char* region = lds + wv * (WTM * kRowB);
+  __syncthreads();  // every wavefront is done with the operand stages
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const unsigned m = i * 32 + (l & 31u);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f16x4 hv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(acc[i][j][g * 4 + e]);
+        const unsigned slot = j * 8 + g * 2 + (l >> 5);
+        *reinterpret_cast<f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8)) = hv;
+      }
+  }
+  // no barrier: a wavefront reads back only what it wrote itself
+  const unsigned slot = l % kSlots, rsub = l / kSlots;
+  const int64_t col = n0 + wn * WTN + slot * 4;
+  const bool vec_store = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(C) & 7u) == 0 && col + 3 < N;
+  float bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (col + e < N) bv[e] = static_cast<float>(bias[col + e]);
+  }
+#pragma unroll
+  for (int p = 0; p < WTM / kRowsPerPass; ++p) {
+    const unsigned m = p * kRowsPerPass + rsub;
+    f16x4 hv = *reinterpret_cast<const f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8));
+    const int64_t row = m0 + wm * WTM + m;
+    if (row >= M) continue;
+    if (bias) {  // "+ bias" is the PrimFunc's separate fp16 add: the sum was already rounded to fp16
+#pragma unroll
+      for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(static_cast<float>(hv[e]) + bv[e]);
+    }
+    half_t* dst = C + row * N + col;
+    if (vec_store) {
+      *reinterpret_cast<f16x4*>(dst) = hv;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (col + e < N) dst[e] = hv[e];
     }
   }
 }
@@ -256,14 +335,17 @@ __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restri
   }
 }
 
-template <int BM, int BN>
-int launch_mfma(const int64_t la[7], hipStream_t s, const half_t* A, const half_t* W, const half_t* bias, half_t* C,
-                int64_t M, int64_t N, int64_t K) {
+template <int BM, int BN, int WM, int WN>
+int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const half_t* bias, half_t* C, int64_t M, int64_t N,
+                int64_t K) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN>), dim3(static_cast<unsigned>(la[0])), dim3(256), 0, s, A, W, bias, C, M, N,
-                     K, tiles_m, tiles_n);
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN>), dim3(tiles_m * tiles_n), dim3(64 * WM * WN), 0, s, A, W, bias,
+                     C, M, N, K, tiles_m, tiles_n);
   return check_launch("gemm");
 }
+
+// threads per workgroup of the MFMA kernel for a tile: 8 wavefronts for 256x256, else 4
+inline int mfma_threads(int bm, int bn) { return bm == 256 && bn == 256 ? 512 : 256; }
 
 }  // namespace
 
@@ -284,12 +366,13 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
                        (bm == 128 && bn == 128) || (bm == 64 && bn == 128) || (bm == 128 && bn == 64) ||
                        (bm == 64 && bn == 64);
     if (!known || cfg.tile[2] != kBK) return fail("gemm: no MFMA kernel for tile %dx%dx%d", bm, bn, cfg.tile[2]);
-    if (cfg.block != 256) return fail("gemm: MFMA kernels use 256 threads, got %d", cfg.block);
+    if (cfg.block != mfma_threads(bm, bn))
+      return fail("gemm: the %dx%d MFMA kernel uses %d threads, got %d", bm, bn, mfma_threads(bm, bn), cfg.block);
     if (K * 2 * (bm > bn ? bm : bn) >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
     const int64_t tm = ceil_div(M, bm), tn = ceil_div(N, bn);
     if (tm * tn > 0x7fffffff) return fail("gemm: too many tiles");
     la[0] = tm * tn;
-    la[3] = 256;
+    la[3] = mfma_threads(bm, bn);
     la[4] = 2 * (bm + bn) * kRowBytes;
     la[5] = tm;
     la[6] = tn;
@@ -354,12 +437,12 @@ extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, voi
     return check_launch("gemm");
   }
   const int bm = cfg.tile[0], bn = cfg.tile[1];
-  if (bm == 256 && bn == 256) return launch_mfma<256, 256>(la, s, a, w, b, c, M, N, K);
-  if (bm == 256 && bn == 128) return launch_mfma<256, 128>(la, s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 256) return launch_mfma<128, 256>(la, s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 128) return launch_mfma<128, 128>(la, s, a, w, b, c, M, N, K);
-  if (bm == 64 && bn == 128) return launch_mfma<64, 128>(la, s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 64) return launch_mfma<128, 64>(la, s, a, w, b, c, M, N, K);
-  if (bm == 64 && bn == 64) return launch_mfma<64, 64>(la, s, a, w, b, c, M, N, K);
+  if (bm == 256 && bn == 256) return launch_mfma<256, 256, 2, 4>(s, a, w, b, c, M, N, K);
+  if (bm == 256 && bn == 128) return launch_mfma<256, 128, 2, 2>(s, a, w, b, c, M, N, K);
+  if (bm == 128 && bn == 256) return launch_mfma<128, 256, 2, 2>(s, a, w, b, c, M, N, K);
+  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2>(s, a, w, b, c, M, N, K);
+  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2>(s, a, w, b, c, M, N, K);
+  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2>(s, a, w, b, c, M, N, K);
+  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2>(s, a, w, b, c, M, N, K);
   return fail("gemm: no MFMA kernel for tile %dx%d", bm, bn);
 }

@@ -26,8 +26,14 @@ _ELT = {
 }
 
 
-def _stream() -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream():
+    """torch's current stream on the current device as a raw hipStream_t (0 = the default stream)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device()) or None
+    return torch.cuda.current_stream().cuda_stream or None
 
 
 def _dev(*tensors: torch.Tensor) -> None:
@@ -41,7 +47,8 @@ def _dev(*tensors: torch.Tensor) -> None:
 
 
 def _p(t: Optional[torch.Tensor]):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    # ints convert to void* through the argtypes; 0 (an empty tensor) becomes NULL
+    return None if t is None else (t.data_ptr() or None)
 
 
 def _cfg(cfg: Optional[DtasConfig]):

@@ -47,6 +47,9 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         for (mx, my), eff in _TILES:
             c = MFMAConfig()
             c.micro_shape_x, c.micro_shape_y = mx, my
+            if (mx, my) == (4, 4):
+                # the 256x256 kernel runs 2x4 wavefronts of 128x64 (two per SIMD)
+                c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 2, 4, 4, 2, 512
             if not self.check_valid(c):
                 continue
             tiles = -(-m_hi // c.tile_size_m) * -(-N // c.tile_size_n)

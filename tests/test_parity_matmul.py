@@ -98,6 +98,10 @@ def test_gemm_benchmark_config_large_m_sampled_rows(oracle, M, N, K):
     assert float((lhs - rhs).abs().max()) < 1e-3 * M ** 0.5 + 0.5     # fp16 rounding of M outputs per column
 
 
+def _threads(bm, bn):
+    return 512 if (bm, bn) == (256, 256) else 256
+
+
 TILES = [(256, 256), (256, 128), (128, 256), (128, 128), (64, 128), (128, 64), (64, 64)]
 
 
@@ -107,7 +111,7 @@ def test_gemm_every_mfma_tile_on_ragged_shapes(oracle, bm, bn, M, N, K):
     a, w = _inputs(M, N, K, M + N + K)
     bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
     out = Guarded((1, M, N), torch.float16)
-    ops.gemm(dev(a), dev(w), dev(bias), out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[bm, bn, 64]))
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, cfg(variant=_lib.GEMM_MFMA, block=_threads(bm, bn), vec=8, tile=[bm, bn, 64]))
     _check(out.check().reshape(M, N), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
 
 
@@ -128,7 +132,7 @@ def test_gemm_exact_cases(oracle):
     perm = rng.permutation(256)
     for tile in ([256, 256, 64], [64, 64, 64], [128, 256, 64]):
         out = Guarded(a.shape, torch.float16)
-        ops.gemm(dev(a), dev(eye[perm].copy()), None, out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=tile))
+        ops.gemm(dev(a), dev(eye[perm].copy()), None, out.t, cfg(variant=_lib.GEMM_MFMA, block=_threads(*tile[:2]), vec=8, tile=tile))
         assert_bits_equal(out.check(), a[:, perm].copy())             # a permutation matrix permutes columns exactly
     # an asymmetric case pins which operand is transposed and the accumulator layout
     a = np.zeros((70, 64), np.float16)
