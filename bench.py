@@ -38,15 +38,18 @@ METRIC = "achieved HBM GB/s (eltwise/reduce/GEMV) + GEMM TFLOP/s, swept over dyn
 
 
 # ---------------------------------------------------------------------------------------------
-# workloads: name -> builder returning (make_buffers(seed) -> tuple, run(buffers), bytes, flops, kernel)
+# workloads: name -> (make_buffers(seed) -> tuple of tensors, bind(buffers) -> zero-argument call of
+# the C-ABI entry point with the arguments already marshalled, algorithmic bytes, flops)
 # ---------------------------------------------------------------------------------------------
 def _workload(name: str, n: int, extra=None):
     import torch
 
-    from dtas_amd import ops
+    from dtas_amd import _lib
 
+    L = _lib.lib()
     H = 4096
     g = torch.Generator(device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream or None
 
     def uniform(shape, seed, lo=-1.0, hi=1.0, dtype=torch.float16):
         g.manual_seed(seed)
@@ -56,40 +59,54 @@ def _workload(name: str, n: int, extra=None):
         g.manual_seed(seed)
         return (torch.randn(shape, device="cuda", generator=g) * std).to(dtype)
 
+    def empty(shape, dtype=torch.float16):
+        return torch.empty(shape, dtype=dtype, device="cuda")
+
+    def call(fn, *args):
+        def run():
+            if fn(*args) != 0:
+                raise RuntimeError(_lib.last_error())
+        return run
+
+    P = lambda t: t.data_ptr()
     if name == "add_f16":
-        make = lambda s: (uniform((n, H), 2 * s), uniform((n, H), 2 * s + 1), torch.empty(n, H, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.add(b[0], b[1], b[2]), 3 * 2 * n * H, 0
+        make = lambda s: (uniform((n, H), 2 * s), uniform((n, H), 2 * s + 1), empty((n, H)))
+        return make, lambda b: call(L.dtas_add_f16, P(b[0]), P(b[1]), P(b[2]), n, H, None, stream), 3 * 2 * n * H, 0
     if name == "copy_f16":
-        make = lambda s: (normal((n, H), s, 100.0), torch.empty(n, H, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.copy(b[0], b[1]), 2 * 2 * n * H, 0
+        make = lambda s: (normal((n, H), s, 100.0), empty((n, H)))
+        return make, lambda b: call(L.dtas_copy_f16, P(b[0]), P(b[1]), n, H, None, stream), 2 * 2 * n * H, 0
     if name == "cast_f32_f16":
-        make = lambda s: (normal((n, H), s, 100.0, torch.float32), torch.empty(n, H, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.cast(b[0], b[1]), (4 + 2) * n * H, 0
+        make = lambda s: (normal((n, H), s, 100.0, torch.float32), empty((n, H)))
+        return make, lambda b: call(L.dtas_cast_f32_f16, P(b[0]), P(b[1]), n, H, None, stream), (4 + 2) * n * H, 0
     if name == "cast_f16_f32":
-        make = lambda s: (normal((n, H), s, 100.0), torch.empty(n, H, dtype=torch.float32, device="cuda"))
-        return make, lambda b: ops.cast(b[0], b[1]), (4 + 2) * n * H, 0
+        make = lambda s: (normal((n, H), s, 100.0), empty((n, H), torch.float32))
+        return make, lambda b: call(L.dtas_cast_f16_f32, P(b[0]), P(b[1]), n, H, None, stream), (4 + 2) * n * H, 0
     if name == "rms_norm_f16":
         w = uniform((H,), 3, 0.5, 1.5)
-        make = lambda s: (normal((n, H), s), w, torch.empty(n, H, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.rms_norm(b[0], b[1], b[2]), 2 * 2 * n * H + 2 * H, 0
+        make = lambda s: (normal((n, H), s), w, empty((n, H)))
+        return (make, lambda b: call(L.dtas_rms_norm_f16, P(b[0]), P(b[1]), P(b[2]), n, H, 1e-5, None, stream),
+                2 * 2 * n * H + 2 * H, 0)
     if name == "layer_norm_f32_f16":
         Hr = 2560
         gm, bt = uniform((Hr,), 3, 0.5, 1.5, torch.float32), uniform((Hr,), 4, -1, 1, torch.float32)
-        make = lambda s: (normal((n, Hr), s, 1.0, torch.float32), gm, bt, torch.empty(n, Hr, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.layer_norm(b[0], b[1], b[2], b[3]), (4 + 2) * n * Hr + 8 * Hr, 0
+        make = lambda s: (normal((n, Hr), s, 1.0, torch.float32), gm, bt, empty((n, Hr)))
+        return (make, lambda b: call(L.dtas_layer_norm_f32_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, Hr, 1e-5, None, stream),
+                (4 + 2) * n * Hr + 8 * Hr, 0)
     if name == "softmax_f16":
         R = 32 * n
-        make = lambda s: (normal((R, n), s, 2.0), torch.empty(R, n, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.softmax(b[0], b[1]), 2 * 2 * R * n, 0
+        make = lambda s: (normal((R, n), s, 2.0), empty((R, n)))
+        return make, lambda b: call(L.dtas_softmax_f16, P(b[0]), P(b[1]), R, n, None, stream), 2 * 2 * R * n, 0
     if name == "gemv_f16":
         N, K = extra
-        make = lambda s: (normal((1, K), s), normal((N, K), s + 100, 0.02), torch.empty(1, N, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.gemv(b[0], b[1], None, b[2]), 2 * N * K + 2 * K + 2 * N, 2 * N * K
+        make = lambda s: (normal((1, K), s), normal((N, K), s + 100, 0.02), empty((1, N)))
+        return (make, lambda b: call(L.dtas_gemv_f16, P(b[0]), P(b[1]), None, P(b[2]), N, K, None, stream),
+                2 * N * K + 2 * K + 2 * N, 2 * N * K)
     if name == "gemm_f16":
         N, K = extra
         wt = normal((N, K), 100, 0.02)
-        make = lambda s: (normal((n, K), s), wt, torch.empty(n, N, dtype=torch.float16, device="cuda"))
-        return make, lambda b: ops.gemm(b[0], b[1], None, b[2]), 2 * (n * K + N * K + n * N), 2 * n * N * K
+        make = lambda s: (normal((n, K), s), wt, empty((n, N)))
+        return (make, lambda b: call(L.dtas_gemm_f16, P(b[0]), P(b[1]), None, P(b[2]), n, N, K, None, stream),
+                2 * (n * K + N * K + n * N), 2 * n * N * K)
     raise ValueError(f"unknown workload {name}")
 
 
@@ -114,39 +131,47 @@ def make_pool(make, streaming: bool, max_bytes: int = 6 << 30):
     return [first] + [make(i) for i in range(1, count)]
 
 
-def time_kernel(run, pool, steps: int, warmup: int):
-    """(wall seconds for `steps` calls between two synchronisations, device seconds for the same
-    region from a pair of HIP events recorded on the launch stream before the first and after the
-    last call).  Launches are issued back to back, so device seconds / steps is the average launch
-    duration (kernel time plus the inter-kernel gap, which is what a caller sees)."""
+def time_kernel(calls, steps: int, warmup: int, min_warm_s: float = 0.2):
+    """(wall seconds for `steps` calls between two synchronisations, device seconds per call from a
+    pair of HIP events recorded on the launch stream before the first and after the last call).
+    Launches are issued back to back, so device seconds / steps is the average launch duration
+    (kernel time plus the inter-kernel gap, which is what a caller sees).  Warm-up runs at least
+    `warmup` calls and at least `min_warm_s` of them: clocks take a moment to settle."""
     import torch
 
-    for i in range(warmup):
-        run(pool[i % len(pool)])
+    t0, i = time.perf_counter(), 0
+    while i < warmup or time.perf_counter() - t0 < min_warm_s:
+        calls[i % len(calls)]()
+        i += 1
+        if i % 64 == 0:
+            torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     start.record()
-    for i in range(steps):
-        run(pool[(warmup + i) % len(pool)])
+    for k in range(steps):
+        calls[(i + k) % len(calls)]()
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return wall, start.elapsed_time(stop) * 1e-3 / steps
 
 
-def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool = True) -> dict:
-    make, run, nbytes, flops = _workload(name, n, extra)
+def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool = True, min_region_s: float = 2e-3) -> dict:
+    make, bind, nbytes, flops = _workload(name, n, extra)
     pool = make_pool(make, streaming)
-    wall, mean_launch = time_kernel(run, pool, steps, warmup)
-    median_launch = mean_launch
-    out = {"op": name, "n": n, "us": round(mean_launch * 1e6, 3), "us_mean": round(mean_launch * 1e6, 3),
-           "ms_per_step": wall * 1e3 / steps, "bytes": nbytes, "flops": flops, "pool": len(pool),
-           "gbs": nbytes / median_launch / 1e9}
+    calls = [bind(b) for b in pool]
+    wall, per_launch = time_kernel(calls, steps, warmup)
+    # short kernels: lengthen the timed region so that event and synchronisation costs vanish
+    if per_launch * steps < min_region_s:
+        steps2 = min(20000, int(min_region_s / max(per_launch, 1e-7)) + 1)
+        wall2, per_launch = time_kernel(calls, steps2, 0, 0.0)
+    out = {"op": name, "n": n, "us": round(per_launch * 1e6, 3), "ms_per_step": wall * 1e3 / steps,
+           "bytes": nbytes, "flops": flops, "pool": len(pool), "gbs": nbytes / per_launch / 1e9}
     if extra:
         out["NK"] = list(extra)
     if flops and name == "gemm_f16":
-        out["tflops"] = flops / median_launch / 1e12
+        out["tflops"] = flops / per_launch / 1e12
         hbm_bound_s = nbytes / (HBM_PEAK_GBS * 1e9)
         mfma_bound_s = flops / (MFMA_FP16_PEAK_TFLOPS * 1e12)
         out["bound"] = "mfma" if mfma_bound_s >= hbm_bound_s else "hbm"
@@ -154,7 +179,7 @@ def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool =
     else:
         out["bound"] = "hbm"
         out["frac"] = out["gbs"] / HBM_PEAK_GBS
-    del pool
+    del pool, calls
     return out
 
 
@@ -222,15 +247,15 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("gemv_f16", 1, nk, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
-            rows.append(measure("gemm_f16", m, nk, max(5, steps // 2), max(2, warmup // 2), streaming=m < 2048))
+            rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
     return rows
 
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | add_f16 | copy_f16 | rms_norm_f16 | softmax_f16 | gemv_f16 | gemm_f16")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
@@ -285,13 +310,12 @@ def main() -> int:
                    "launch": list(info.launch_args)[:5] if info is not None else None},
         "roofline": {
             "bound": "mfma" if is_gemm else "hbm",
-            "achieved": round(head["tflops"], 3) if is_gemm else round(head["bytes"] / (head["us_mean"] * 1e-6) / 1e9, 3),
+            "achieved": round(head["tflops"], 3) if is_gemm else round(head["gbs"], 3),
             "peak": MFMA_FP16_PEAK_TFLOPS if is_gemm else HBM_PEAK_GBS,
             "unit": "TFLOP/s" if is_gemm else "GB/s",
-            "frac": round((head["tflops"] / MFMA_FP16_PEAK_TFLOPS) if is_gemm
-                          else head["bytes"] / (head["us_mean"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "frac": round((head["tflops"] / MFMA_FP16_PEAK_TFLOPS) if is_gemm else head["gbs"] / HBM_PEAK_GBS, 4),
             "traffic": None,
-            "launch_us_mean": head["us_mean"],
+            "launch_us_mean": head["us"],
             "algorithmic_bytes_per_launch": head["bytes"],
         },
     }
@@ -301,7 +325,7 @@ def main() -> int:
     else:
         line["cpu_baseline"] = None
     if not args.no_sweep:
-        rows = sweep(max(10, args.steps // 2), max(3, args.warmup // 2))
+        rows = sweep(max(20, args.steps // 4), max(3, args.warmup // 4))
         line["sweep"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
                           if k in ("op", "n", "NK", "us", "gbs", "tflops", "bound", "frac")} for r in rows]
         if args.out:

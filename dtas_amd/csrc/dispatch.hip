@@ -48,54 +48,71 @@ bool same(const dtas_config& a, const dtas_config& b) {
          a.grid_cap == b.grid_cap;
 }
 
-int narrow_bytes(int op) {
+// bytes per element of the wider of an op's input / output types
+int wide_bytes(int op) {
   switch (op) {
-    case DTAS_OP_ADD_F32: case DTAS_OP_COPY_F32: return 4;
+    case DTAS_OP_ADD_F16: case DTAS_OP_COPY_F16: return 2;
     case DTAS_OP_ADD_I8: case DTAS_OP_COPY_I8: return 1;
-    default: return 2;
+    default: return 4;  // fp32 add / copy and both casts
   }
 }
 
 // ---- per-family policies: config for a bucket whose upper end is n_hi -----------------
+// The constants below were read off sweeps of every variant on an MI355X (GB/s per launch,
+// buffers rotating through more than the Infinity Cache).
 
-// Elementwise: 128-bit accesses; few elements -> one access per thread so the work spreads
-// over more CUs, many elements -> 4 accesses in flight per thread.
+// Elementwise: accesses of 128 bit on the wider side (a cast then moves 64 bit on the narrow
+// side: 128-bit narrow accesses would make the wide ones 256 bit per lane, which measured ~40 %
+// slower).  As many accesses in flight per thread (up to 8) as still leaves >= 4 workgroups per CU.
 dtas_config elementwise_policy(int op, int64_t n_hi, int64_t H) {
-  const int vec = 16 / narrow_bytes(op);
+  const int vec = 16 / wide_bytes(op);
   const int64_t nvec = n_hi * (H > 0 ? H : 1) / vec;
-  const int unroll = nvec <= 256 * kNumCU * 2 ? 1 : nvec <= 256 * kNumCU * 8 ? 2 : 4;
+  int unroll = 8;
+  while (unroll > 1 && nvec / (256 * unroll) < 4 * kNumCU) unroll /= 2;
   return make(DTAS_ELT_VECTOR, 256, vec, unroll);
 }
 
-// Norms: n rows of static length H.  Up to a few rows per CU a whole workgroup per row hides
-// latency best; beyond that one wavefront per row keeps every reduction on the DPP path.
+int pow2_at_most(int64_t v) {
+  int p = 1;
+  while (2 * p <= v) p *= 2;
+  return p;
+}
+
+// One workgroup per row, sized for about two 128-bit vectors per thread.
+dtas_config block_row(int vec, int64_t nvec) {
+  int block = pow2_at_most(nvec / 2 > 64 ? nvec / 2 : 64);
+  if (block > 1024) block = 1024;
+  if (nvec > static_cast<int64_t>(block) * 16) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
+  return make(DTAS_RED_BLOCK_ROW, block, vec, 1);
+}
+
+// Norms: n rows of static length H.  From ~8 rows per CU on, one wavefront per row (all
+// reductions on the DPP path, no barrier) wins, provided a lane holds at most 8 vectors; below
+// that, and for longer rows (fp32 rows of 2560 need 10), a workgroup per row hides latency better.
 dtas_config norm_policy(int op, int64_t n_hi, int64_t H) {
   const int vec = op == DTAS_OP_RMS_NORM_F16 ? 8 : 4;
   const int64_t nvec = (H + vec - 1) / vec;
-  const bool wave_fits = nvec <= 64 * 16;
-  if (wave_fits && n_hi > 2 * kNumCU) return make(DTAS_RED_WAVE_ROW, 256, vec, 1);
-  int block = 64;
-  while (block < 1024 && (nvec > block * 2)) block *= 2;  // aim for <= 2 vectors per lane
-  if (nvec > static_cast<int64_t>(block) * 16) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
-  return make(DTAS_RED_BLOCK_ROW, block, vec, 1);
+  if (n_hi >= 8 * kNumCU && nvec <= 64 * 8) return make(DTAS_RED_WAVE_ROW, 256, vec, 1);
+  return block_row(vec, nvec);
 }
 
-// Softmax: 32*n rows of dynamic length n (the reduction axis is the dynamic one).
+// Softmax: 32*n rows of dynamic length n (the reduction axis is the dynamic one).  One wavefront
+// per row up to 16 vectors per lane; short rows launch one row per workgroup so that the many
+// small workgroups spread evenly.
 dtas_config softmax_policy(int op, int64_t cols_hi, int64_t rows) {
   const int vec = op == DTAS_OP_SOFTMAX_F16 ? 8 : 4;
   const int64_t nvec = (cols_hi + vec - 1) / vec;
-  if (nvec <= 64 * 16 && (rows <= 0 || rows > 2 * kNumCU)) return make(DTAS_RED_WAVE_ROW, 256, vec, 1);
-  int block = 64;
-  while (block < 1024 && (nvec > block * 2)) block *= 2;
-  if (nvec > static_cast<int64_t>(block) * 16) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
-  return make(DTAS_RED_BLOCK_ROW, block, vec, 1);
+  if (nvec <= 64 * 16 && (rows <= 0 || rows > 2 * kNumCU))
+    return make(DTAS_RED_WAVE_ROW, nvec <= 64 ? 64 : 256, vec, 1);
+  return block_row(vec, nvec);
 }
 
-// GEMV: rows per workgroup so that there are at least ~4 workgroups per CU.
+// GEMV: one row of W per workgroup of 4 wavefronts keeps the most independent streams in
+// flight; long rows (K >= 8192) do better with 8 wavefronts on two rows.
 dtas_config gemv_policy(int64_t N, int64_t K) {
-  (void)K;
-  const int rows = N >= 8 * 4 * kNumCU ? 8 : N >= 4 * 4 * kNumCU ? 4 : N >= 2 * 4 * kNumCU ? 2 : 1;
-  return make(DTAS_GEMV_SPLITK, 256, 8, 2, rows);
+  (void)N;
+  if (K >= 8192) return make(DTAS_GEMV_SPLITK, 512, 8, 2, 2);
+  return make(DTAS_GEMV_SPLITK, 256, 8, 2, 1);
 }
 
 // GEMM: M <= 64 streams W once (SKINNY).  Above that, the MFMA tile minimising

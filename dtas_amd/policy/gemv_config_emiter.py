@@ -3,7 +3,7 @@
 The reference's GEMVConfigEmiter.emit_config is an unfinished stub that returns no candidates
 (python/dtas/policy/gemv_config_emiter.py:26-30); its GEMV experiments used the GEMVConfig defaults
 (block 32x16, grid N/16, python/dtas/common/config.py:339-356).  Here the candidates are rows of W per
-workgroup x threads splitting K, ranked so that every CU holds at least ~4 workgroups.
+workgroup x threads splitting K, ranked by what sweeps on an MI355X favoured.
 """
 from typing import List, Tuple
 
@@ -22,10 +22,11 @@ class GEMVConfigEmiter(BaseConfigEmiter):
                 c = GEMVConfig()
                 c.TILE_S, c.TR = rows, threads
                 out.append(c)
-        want = 4 * self.arch.num_sm
+        # measured on MI355X: one row per 4-wavefront workgroup is best or within noise for K = 4096;
+        # rows of K >= 8192 do better with 8 wavefronts on two rows
+        best = (2, 512) if K >= 8192 else (1, 256)
 
         def score(c: GEMVConfig):
-            groups = -(-N // c.TILE_S)
-            return (groups < want, -c.TILE_S if groups >= want else c.TILE_S, c.TR != 256)
+            return ((c.TILE_S, c.TR) != best, c.TILE_S, c.TR != 256)
 
         return sorted(out, key=score)[:topk]

@@ -76,7 +76,11 @@ class ReductionConfigEmiter(BaseConfigEmiter):
     def _gfx950_candidates(self, re_range: Range, row_range: Range, in_bytes: int, topk: int) -> List[ReductionConfig]:
         vec = 16 // in_bytes
         nvec = -(-re_range.end // vec)
-        many_rows = row_range.start > 2 * self.arch.num_sm
+        # a wavefront per row pays off from ~8 rows per CU and up to 8 vectors per lane (static rows);
+        # dynamic rows (softmax) have 32 rows per unit of row length, so many rows as soon as n > 16
+        many_rows = row_range.start >= 8 * self.arch.num_sm and (nvec <= 64 * 8 or self.func_info.dyn_red)
+        if self.func_info.dyn_red:
+            many_rows = row_range.end > 2 * self.arch.num_sm
         out: List[ReductionConfig] = []
 
         def cand(storage: str, tx: int) -> ReductionConfig:
@@ -86,9 +90,13 @@ class ReductionConfigEmiter(BaseConfigEmiter):
             c.bx = None  # rows map 1:1 to wavefronts / workgroups; the kernels stride if capped
             return c
 
-        wave_rows = [cand("local", tx) for tx in (256, 128, 512, 64)] if nvec <= 64 * 16 else []
+        wave_order = (64, 128, 256, 512) if nvec <= 64 else (256, 128, 512, 64)
+        wave_rows = [cand("local", tx) for tx in wave_order] if nvec <= 64 * 16 else []
+        pref = 64
+        while pref * 2 <= max(64, nvec // 2) and pref < 1024:
+            pref *= 2
         block_rows = []
-        for tx in (256, 512, 1024, 128):
+        for tx in sorted((64, 128, 256, 512, 1024), key=lambda t: (t != pref, abs(t - pref))):
             if tx * 16 >= nvec and tx <= max(64, nvec):
                 block_rows.append(cand("shared.dyn", tx))
         # few rows: a workgroup per row first; many rows: a wavefront per row first

@@ -67,7 +67,11 @@ def test_elementwise_launch_shape():
     assert info.launch_args[0] == -(-(4096 * 4096 // 8) // (256 * c.unroll)) and info.launch_args[3] == 256
     assert _lib.select_bucket(_lib.OP_ADD_I8, 1, 2560, 0).config.vec == 16
     assert _lib.select_bucket(_lib.OP_ADD_F32, 1, 2560, 0).config.vec == 4
-    assert _lib.select_bucket(_lib.OP_CAST_F32_F16, 1, 4096, 0).config.vec == 8
+    # a cast moves 128 bit on the wider side: 4 elements per access in either direction
+    assert _lib.select_bucket(_lib.OP_CAST_F32_F16, 1, 4096, 0).config.vec == 4
+    assert _lib.select_bucket(_lib.OP_CAST_F16_F32, 1, 4096, 0).config.vec == 4
+    # accesses in flight per thread shrink with the extent so that the grid still fills the CUs
+    assert [_lib.select_bucket(_lib.OP_ADD_F16, n, 4096, 0).config.unroll for n in (1, 128, 1024, 4096)] == [1, 1, 2, 8]
 
 
 def test_describe_launch_rejects_bad_configs():
