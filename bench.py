@@ -251,6 +251,17 @@ def sweep(steps: int, warmup: int) -> list:
     return rows
 
 
+def recorded_traffic(workload_key: str):
+    """HBM bytes per launch of this workload's kernel as measured with rocprofv3 --pmc (FETCH_SIZE and
+    WRITE_SIZE runs, calibrated on the copy kernel) and committed under profiles/; None when no
+    counter run was recorded for it.  Counters cannot be read from inside this process."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(workload_key, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        return None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -314,7 +325,7 @@ def main() -> int:
             "peak": MFMA_FP16_PEAK_TFLOPS if is_gemm else HBM_PEAK_GBS,
             "unit": "TFLOP/s" if is_gemm else "GB/s",
             "frac": round((head["tflops"] / MFMA_FP16_PEAK_TFLOPS) if is_gemm else head["gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": recorded_traffic(f"{args.workload} [n={args.n}, 4096]") if extra is None else None,
             "launch_us_mean": head["us"],
             "algorithmic_bytes_per_launch": head["bytes"],
         },

@@ -1,0 +1,93 @@
+"""End-to-end on the GPU through the reference's Python entry points: Engine.tune_module with
+on-device timing of the candidates, the runtime module's dispatch, load_module_from_file."""
+import numpy as np
+import pytest
+import torch
+
+from dtas_amd import _lib, primfuncs as pf
+from dtas_amd.arch import MI355X
+from dtas_amd.codegen.runtime_packer import load_module_from_file
+from dtas_amd.engine.tuner import Engine
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tuned(tmp_path_factory):
+    work_dir = str(tmp_path_factory.mktemp("tuned"))
+    mod = pf.module(pf.add("float16", 4096), pf.cast("float32", "float16", 4096), pf.rms_norm(4096),
+                    pf.softmax_scores(32), pf.fused_layer_norm_cast1(2560),
+                    pf.fused_NT_matmul_add_gemv(4096, 4096, bias=True), pf.fused_NT_matmul_add_gemm(4096, 4096, bias=True),
+                    upper_bound={"n": 1024})
+    eng = Engine(topk=4, parallel_build=True, work_dir=work_dir)
+    rt = eng.tune_module(mod, arch=MI355X(0, require_device=True), range_div_factor=256)
+    return rt, work_dir
+
+
+def test_candidates_were_timed_on_the_device(tuned):
+    import json, os
+
+    _, work_dir = tuned
+    records = json.load(open(os.path.join(work_dir, "data_base", "best_record.json")))
+    timed = [v["latency(ms)"] for rec in records for v in rec.values() if v["latency(ms)"] is not None]
+    assert timed and all(0 < t < 1000 for t in timed)
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 300, 1024, 2000])
+def test_module_functions_match_the_oracle(tuned, oracle, n):
+    rt, work_dir = tuned
+    again = load_module_from_file(work_dir)
+    rng = np.random.default_rng(n)
+    for mod in (rt, again):
+        a = rng.uniform(-1, 1, (1, n, 4096)).astype(np.float16)
+        b = rng.uniform(-1, 1, (1, n, 4096)).astype(np.float16)
+        out = torch.empty(1, n, 4096, dtype=torch.float16, device="cuda")
+        mod["add"](torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda(), out)
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), oracle.c.add(a, b).view(np.uint16))
+
+        x32 = (rng.standard_normal((1, n, 4096)) * 100).astype(np.float32)
+        mod["cast"](torch.from_numpy(x32).cuda(), out)
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), oracle.c.cast(x32, "float16").view(np.uint16))
+
+        x = rng.standard_normal((n, 4096)).astype(np.float16)
+        w = rng.uniform(0.5, 1.5, 4096).astype(np.float16)
+        o2 = torch.empty(n, 4096, dtype=torch.float16, device="cuda")
+        mod["rms_norm"](torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), o2)
+        assert np.abs(o2.cpu().numpy().astype(np.float64) - oracle.np64.rms_norm(x, w)).max() < 1e-2
+
+
+def test_gemm_gemv_and_softmax_through_the_module(tuned, oracle):
+    rt, _ = tuned
+    rng = np.random.default_rng(0)
+    W = (rng.standard_normal((4096, 4096)) * 0.02).astype(np.float16)
+    bias = rng.uniform(-1, 1, 4096).astype(np.float16)
+    for n in (3, 130, 700):
+        A = rng.standard_normal((1, n, 4096)).astype(np.float16)
+        C = torch.empty(1, n, 4096, dtype=torch.float16, device="cuda")
+        rt["fused_NT_matmul4_add1"](torch.from_numpy(A).cuda(), torch.from_numpy(W).cuda(), torch.from_numpy(bias).cuda(), C)
+        want = oracle.np64.gemm(A[0], W, bias)
+        assert (np.abs(C.cpu().numpy()[0].astype(np.float64) - want) <= 2e-3 + 1e-2 * np.abs(want)).all()
+    x = rng.standard_normal((1, 1, 4096)).astype(np.float16)
+    y = torch.empty(1, 1, 4096, dtype=torch.float16, device="cuda")
+    rt["fused_NT_matmul10_add5"](torch.from_numpy(x).cuda(), torch.from_numpy(W).cuda(), torch.from_numpy(bias).cuda(), y)
+    want = oracle.np64.gemm(x[0], W, bias)
+    assert (np.abs(y.cpu().numpy()[0].astype(np.float64) - want) <= 2e-3 + 1e-2 * np.abs(want)).all()
+    for n in (5, 64, 257):
+        s = (rng.standard_normal((32, n, n)) * 2).astype(np.float16)
+        so = torch.empty(32, n, n, dtype=torch.float16, device="cuda")
+        rt["softmax_scores"](torch.from_numpy(s).cuda(), so)
+        assert np.abs(so.cpu().numpy().astype(np.float64) - oracle.np64.softmax(s)).max() < 1e-2
+
+
+def test_time_evaluator_and_signature_errors(tuned):
+    rt, _ = tuned
+    a = torch.zeros(1, 64, 4096, dtype=torch.float16, device="cuda")
+    out = torch.empty_like(a)
+    res = rt.time_evaluator("add", number=5, min_repeat_ms=5)(a, a.clone(), out)
+    assert 0 < res.mean < 1e-2
+    with pytest.raises(TypeError):
+        rt["add"](a, a)
+    with pytest.raises(ValueError):
+        rt["add"](a, a.clone(), torch.empty(1, 64, 2560, dtype=torch.float16, device="cuda"))
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        rt["add"](a, a, a)
