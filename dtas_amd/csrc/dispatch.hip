@@ -115,28 +115,38 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
   return make(DTAS_GEMV_SPLITK, 256, 8, 2, 1);
 }
 
-// GEMM: M <= 64 streams W once (SKINNY).  Above that, the MFMA tile minimising
-// rounds(tiles / CUs) * tile_area / efficiency(tile): bigger tiles reuse LDS data better,
-// smaller ones fill the 256 CUs at small M (the reference scores tiles the same way,
-// python/dtas/policy/wmma_config_emiter.py:148-262).
+// GEMM, from sweeps of every tile x stage count over M on an MI355X:
+//  * M <= 32 and N <= 6144: the W-streaming SKINNY kernel (its time grows with N*K, the 64x64
+//    MFMA loop's with K only);
+//  * 256x256 (8 wavefronts, ping-pong) once it yields >= 150 workgroups;
+//  * else 128x128 once that yields >= 256 workgroups;
+//  * else 64x64: few workgroups, each latency bound, so as many LDS stages as possible.
+// LDS stages (depth of the load pipeline): more stages hide more latency but fewer workgroups
+// fit a CU; take the deepest pipeline with which all tiles are still co-resident (with a
+// margin when several workgroups share a CU), else 2.
 dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   (void)K;
-  if (M_hi <= 64) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
-  static const struct { int bm, bn; double eff; } kTiles[] = {
-      {256, 256, 1.00}, {256, 128, 0.85}, {128, 256, 0.85}, {128, 128, 0.70},
-      {64, 128, 0.50},  {128, 64, 0.50},  {64, 64, 0.35}};
-  double best = 0;
-  int pick = -1;
-  for (int i = 0; i < 7; ++i) {
-    const int64_t tiles = ceil_div(M_hi, kTiles[i].bm) * ceil_div(N > 0 ? N : 1, kTiles[i].bn);
-    const double cost = static_cast<double>(ceil_div(tiles, kNumCU)) * kTiles[i].bm * kTiles[i].bn / kTiles[i].eff;
-    if (pick < 0 || cost < best) {
-      best = cost;
-      pick = i;
+  if (M_hi <= 32 && N <= 6144) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
+  const int64_t n = N > 0 ? N : 1;
+  int bm, bn;
+  if (ceil_div(M_hi, 256) * ceil_div(n, 256) >= 150) {
+    return make(DTAS_GEMM_MFMA, 512, 8, 2, 256, 256, 64);
+  } else if (ceil_div(M_hi, 128) * ceil_div(n, 128) >= 256) {
+    bm = bn = 128;
+  } else {
+    bm = bn = 64;
+  }
+  const int64_t tiles = ceil_div(M_hi, bm) * ceil_div(n, bn);
+  const int64_t stage_bytes = static_cast<int64_t>(bm + bn) * 128;
+  int stages = 2;
+  for (int ns = 4; ns > 2; --ns) {
+    const int64_t per_cu = kLdsBytes / (ns * stage_bytes);
+    if (per_cu >= 1 && (per_cu == 1 ? tiles <= kNumCU : tiles * 4 <= kNumCU * per_cu * 3)) {
+      stages = ns;
+      break;
     }
   }
-  const int threads = kTiles[pick].bm == 256 && kTiles[pick].bn == 256 ? 512 : 256;
-  return make(DTAS_GEMM_MFMA, threads, 8, 1, kTiles[pick].bm, kTiles[pick].bn, 64);
+  return make(DTAS_GEMM_MFMA, 256, 8, stages, bm, bn, 64);
 }
 
 dtas_config policy(int op, int64_t n_hi, int64_t d0, int64_t d1) {

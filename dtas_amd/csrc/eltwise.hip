@@ -225,15 +225,14 @@ int run_eltwise(int op, const void* a, const void* b, void* out, int64_t n, int6
     return fail("%s: output overlaps an input (PrimFunc is tir.noalias)", e.name);
 
   dtas_config cfg = user ? *user : builtin_config(op, n, H, 0).cfg;
-  // A vector access needs its natural alignment on every buffer; the built-in choice steps
-  // down to element accesses for odd pointers, an explicit config is taken at its word.
+  // A vector access needs its natural alignment on every buffer; for odd pointers the call
+  // steps down to element accesses (a bucket's config must serve every n and buffer in it).
   if (cfg.variant == DTAS_ELT_VECTOR) {
     const size_t ia = static_cast<size_t>(cfg.vec) * e.in_bytes, oa = static_cast<size_t>(cfg.vec) * e.out_bytes;
     const size_t ia16 = ia > 16 ? 16 : ia, oa16 = oa > 16 ? 16 : oa;
     const bool ok = cfg.vec > 0 && (ia & (ia - 1)) == 0 && aligned(a, ia16) && aligned(out, oa16) &&
                     (e.inputs == 1 || aligned(b, ia16));
     if (!ok) {
-      if (user) return fail("%s: buffers are not aligned for %d-element accesses", e.name, cfg.vec);
       cfg.variant = DTAS_ELT_SCALAR;
       cfg.vec = 1;
     }

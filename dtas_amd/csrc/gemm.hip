@@ -19,11 +19,16 @@
 //   LDS      : two stages of (BM + BN) x 128 B.  Chunk c of row r sits at a swizzled slot so
 //              that the MFMA operand reads (a column of 32 rows per half-wavefront, 128 bit
 //              per lane) spread over all 64 banks.
-//   pipeline : fragments of step s+1 are read from LDS while the MFMAs of step s issue (two
-//              register sets); the tile barrier sits before the last step of a k tile, the
-//              loads of tile k+2 are issued right after it into the stage just vacated, and the
-//              first fragments of tile k+1 are read under the last MFMAs of tile k.  The
-//              interleaving is pinned with scheduling barriers.
+//   pipeline : 4-wavefront tiles: fragments of step s+1 are read from LDS while the MFMAs of step
+//              s issue (two register sets); the tile barrier sits before the last step of a k
+//              tile, the loads of tile k+2 are issued right after it into the stage just
+//              vacated, and the first fragments of tile k+1 are read under the last MFMAs of
+//              tile k.  The interleaving is pinned with scheduling barriers.
+//              8-wavefront tile (256x256): wavefronts w and w+4 share a SIMD and alternate
+//              roles ("ping-pong"): while one issues the 8 MFMAs of a step, the other reads its
+//              next fragments and issues its share of the next tile's loads; a workgroup
+//              barrier separates the phases, group 1 runs one phase behind group 0, so the MFMA
+//              pipe of every SIMD always has exactly one wavefront feeding it.
 //   epilogue : accumulators -> fp16 -> wavefront-private LDS region (xor-swizzled 8-byte
 //              slots) -> 8-byte coalesced row stores with the bias added on the way out.
 //   launch   : workgroup ids are remapped so that each XCD (own L2) works on a compact patch of
@@ -74,7 +79,7 @@ __device__ __forceinline__ unsigned xcd_contiguous_id(unsigned wg, unsigned tota
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ W,
                                                                  const half_t* __restrict__ bias,
@@ -86,8 +91,11 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;  // 1 KiB block loads per wavefront per k tile
   constexpr int kABytes = BM * kRowBytes, kStage = (BM + BN) * kRowBytes;
   static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
-  static_assert(BM * BN * 2 <= 2 * kStage, "epilogue staging must fit the operand stages");
-  __shared__ __attribute__((aligned(1024))) char lds[2 * kStage];
+  static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
+  static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
+  static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
+  static_assert(NS * kStage <= kLdsBytes, "stages exceed the LDS");
+  __shared__ __attribute__((aligned(1024))) char lds[NS * kStage];
 
   const unsigned t = threadIdx.x, l = t & 63u;
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
@@ -130,12 +138,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 
   const int ktiles = static_cast<int>((K + kBK - 1) / kBK);
 
-  // tile kt -> LDS stage kt & 1, asynchronously (completion is counted by vmcnt)
+  // tile kt -> LDS stage kt % NS, asynchronously (completion is counted by vmcnt)
   auto fetch = [&](int kt) {
     // a chunk past K is pointed out of range; K % 8 == 0, so chunks are all-in or all-out
     const unsigned off = (static_cast<int64_t>(kt) * kBK + c_in * 8 < K)
                              ? g_off + static_cast<unsigned>(kt) * kRowBytes : kOob;
-    char* base = lds + (kt & 1) * kStage + wv * 1024;
+    char* base = lds + (kt % NS) * kStage + wv * 1024;
 #pragma unroll
     for (int i = 0; i < LA; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
@@ -173,12 +181,74 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     }
   };
 
-  // prologue: tile 0 resident, tile 1 in flight, fragments of (tile 0, step 0) in registers
+  if constexpr (NW == 8) {
+    // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD)
+    // half of tile kt's block loads (every second one)
+    auto fetch_half = [&](int kt, int part) {
+      const unsigned off = (static_cast<int64_t>(kt) * kBK + c_in * 8 < K)
+                               ? g_off + static_cast<unsigned>(kt) * kRowBytes : kOob;
+      char* base = lds + (kt & 1) * kStage + wv * 1024;
+#pragma unroll
+      for (int i = 0; i < LA + LB; ++i) {
+        if (i % 2 != part) continue;
+        if (i < LA)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
+        else
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + (i - LA) * NW * 1024), 16,
+                                                   off + (i - LA) * g_step, 0, 0, 0);
+      }
+    };
+    const unsigned group = wv >> 2;
+    if (ktiles > 0) fetch(0);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    if (group == 1) {  // one phase behind group 0; group 0 makes up the barrier after the loop
+      __builtin_amdgcn_s_barrier();
+      DTAS_SCHED_FENCE();
+    }
+    for (int kt = 0; kt < ktiles; ++kt) {
+      const char* cur = lds + (kt & 1) * kStage;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int set = ks & 1;
+        // memory phase: this step's fragments; in steps 0 and 1 half of tile kt+1's loads each (its
+        // stage held tile kt-1, which every wavefront finished reading two phases ago at the latest)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) read_a(set, i, cur, ks);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) read_b(set, j, cur, ks);
+        if (ks < 2 && kt + 1 < ktiles) fetch_half(kt + 1, ks);
+        // fragments in registers before the barrier (after a tile's last step the other group may
+        // overwrite the stage); at the last step also this wavefront's loads of tile kt+1
+        if (ks == 3) __builtin_amdgcn_s_waitcnt(0x0070); else __builtin_amdgcn_s_waitcnt(0xC07F);
+        DTAS_SCHED_FENCE();
+        __builtin_amdgcn_s_barrier();
+        DTAS_SCHED_FENCE();
+        // MFMA phase
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+        DTAS_SCHED_FENCE();
+        __builtin_amdgcn_s_barrier();
+        DTAS_SCHED_FENCE();
+      }
+    }
+    if (group == 0) {
+      __builtin_amdgcn_s_barrier();
+      DTAS_SCHED_FENCE();
+    }
+  } else {
+  // NS stages: tile 0 resident, tiles 1 .. NS-1 in flight, fragments of (tile 0, step 0) in registers
   if (ktiles > 0) fetch(0);
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
   DTAS_SCHED_FENCE();
-  if (ktiles > 1) fetch(1);
+#pragma unroll
+  for (int p = 1; p < NS; ++p)
+    if (p < ktiles) fetch(p);
   if (ktiles > 0) {
 #pragma unroll
     for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
@@ -187,19 +257,26 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   }
   DTAS_SCHED_FENCE();
 
+  // vmcnt(n) with lgkmcnt(0): n is a compile-time field of the instruction
+  constexpr int kL = LA + LB;
   for (int kt = 0; kt < ktiles; ++kt) {
-    const char* cur = lds + (kt & 1) * kStage;
-    const char* nxt = lds + ((kt + 1) & 1) * kStage;
+    const char* cur = lds + (kt % NS) * kStage;
+    const char* nxt = lds + ((kt + 1) % NS) * kStage;
     step(0, cur, 1, true);
     step(1, cur, 2, true);
     step(0, cur, 3, true);
-    // tile kt+1 has landed and every wavefront has finished reading tile kt
-    __builtin_amdgcn_s_waitcnt(0x0070);
-    __builtin_amdgcn_s_barrier();
+    // tile kt+1 must have landed; tiles kt+2 .. (at most NS-2 of them) may stay in flight.  Loads
+    // complete in order, so it is enough to allow that many tiles' worth of loads outstanding.
+    const int ahead = ktiles - 2 - kt;  // tiles after kt+1 that have been requested, if < NS-2
+    if (NS >= 4 && ahead >= 2) __builtin_amdgcn_s_waitcnt(0x0070 | ((2 * kL) & 15) | (((2 * kL) >> 4) << 14));
+    else if (NS >= 3 && ahead >= 1) __builtin_amdgcn_s_waitcnt(0x0070 | (kL & 15) | ((kL >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();  // ... and every wavefront has finished reading tile kt
     DTAS_SCHED_FENCE();
-    if (kt + 2 < ktiles) fetch(kt + 2);  // into the stage tile kt occupied
+    if (kt + NS < ktiles) fetch(kt + NS);  // into the stage tile kt occupied
     DTAS_SCHED_FENCE();
     step(1, nxt, 0, kt + 1 < ktiles);
+  }
   }
 
   // ---- epilogue.  acc[i][j][v] of lane l is C row i*32 + (l & 31), column
@@ -278,14 +355,43 @@ __global__ void __launch_bounds__(512) gemm_skinny_kernel(const half_t* __restri
   for (int i = 0; i < MT; ++i) acc[i] = f32x4v{0.f, 0.f, 0.f, 0.f};
 
   const int64_t steps = K >> 5;  // whole 32-element steps; K % 32 is handled below
-#pragma unroll 4
-  for (int64_t s = wv; s < steps; s += nwaves) {
-    const f16x8 fw = __builtin_bit_cast(f16x8, load_stream(reinterpret_cast<const u32x4*>(wp + s * 32)));
-    f16x8 fa[MT];
+  // A wavefront takes pairs of consecutive steps (2p, 2p+1) for p = wv, wv + nwaves, ...: the two
+  // 64-byte pieces a lane row contributes per pair are the halves of one 128-byte line.  Two pairs
+  // at a time, so that 4 * (1 + MT) independent 1 KiB loads are in flight before the first MFMA.
+  const int64_t pairs = steps >> 1;
+  const int64_t mine = pairs > wv ? (pairs - wv + nwaves - 1) / nwaves : 0;
+  int64_t q = 0;
+  for (; q + 2 <= mine; q += 2) {
+    f16x8 fw[4], fa[4][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const f16x8*>(ap[i] + s * 32);
+    for (int u = 0; u < 4; ++u) {
+      const int64_t off = ((wv + (q + (u >> 1)) * nwaves) * 2 + (u & 1)) * 32;
+      fw[u] = __builtin_bit_cast(f16x8, load_stream(reinterpret_cast<const u32x4*>(wp + off)));
 #pragma unroll
-    for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[i], fw, acc[i], 0, 0, 0);
+      for (int i = 0; i < MT; ++i) fa[u][i] = *reinterpret_cast<const f16x8*>(ap[i] + off);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[u][i], fw[u], acc[i], 0, 0, 0);
+  }
+  for (; q < mine; ++q) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int64_t off = ((wv + q * nwaves) * 2 + u) * 32;
+      const f16x8 fw = __builtin_bit_cast(f16x8, load_stream(reinterpret_cast<const u32x4*>(wp + off)));
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const f16x8*>(ap[i] + off), fw, acc[i], 0, 0, 0);
+    }
+  }
+  // an odd number of whole steps: the last one goes to the wavefront after the last pair's
+  if ((steps & 1) && wv == pairs % nwaves) {
+    const int64_t off = (steps - 1) * 32;
+    const f16x8 fw = __builtin_bit_cast(f16x8, load_stream(reinterpret_cast<const u32x4*>(wp + off)));
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+      acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const f16x8*>(ap[i] + off), fw, acc[i], 0, 0, 0);
   }
   // K % 32 (a multiple of 8): the last partial step, chunks past K contribute zeros
   if ((K & 31) != 0 && wv == steps % nwaves) {
@@ -335,17 +441,19 @@ __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restri
   }
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const half_t* bias, half_t* C, int64_t M, int64_t N,
                 int64_t K) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN>), dim3(tiles_m * tiles_n), dim3(64 * WM * WN), 0, s, A, W, bias,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(tiles_m * tiles_n), dim3(64 * WM * WN), 0, s, A, W, bias,
                      C, M, N, K, tiles_m, tiles_n);
   return check_launch("gemm");
 }
 
 // threads per workgroup of the MFMA kernel for a tile: 8 wavefronts for 256x256, else 4
 inline int mfma_threads(int bm, int bn) { return bm == 256 && bn == 256 ? 512 : 256; }
+// LDS stages a tile can hold (160 KiB): 2 for 256x256, 3 for 256x128, 4 below that
+inline int mfma_max_stages(int bm, int bn) { return bm + bn >= 512 ? 2 : bm + bn >= 384 ? 3 : 4; }
 
 }  // namespace
 
@@ -371,9 +479,12 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     if (K * 2 * (bm > bn ? bm : bn) >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
     const int64_t tm = ceil_div(M, bm), tn = ceil_div(N, bn);
     if (tm * tn > 0x7fffffff) return fail("gemm: too many tiles");
+    // cfg.unroll = LDS stages (the depth of the load pipeline); 0 or 1 = as many as fit
+    if (cfg.unroll < 0 || cfg.unroll > mfma_max_stages(bm, bn))
+      return fail("gemm: the %dx%d tile holds at most %d LDS stages, got %d", bm, bn, mfma_max_stages(bm, bn), cfg.unroll);
     la[0] = tm * tn;
     la[3] = mfma_threads(bm, bn);
-    la[4] = 2 * (bm + bn) * kRowBytes;
+    la[4] = (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
     la[5] = tm;
     la[6] = tn;
     return 0;
@@ -410,10 +521,7 @@ extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, voi
   if (!user && M == 1) return dtas_gemv_f16(A, W, bias, C, N, K, nullptr, stream);
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMM_F16, M, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(A, 16) && aligned(W, 16);
-  if (cfg.vec == 8 && !vec_ok) {
-    if (user) return fail("gemm: 128-bit accesses need K %% 8 == 0 and 16-byte aligned A, W");
-    cfg.vec = 1;
-  }
+  if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
   int64_t la[7];
   if (describe_gemm(M, N, K, cfg, la) != 0) return -1;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -437,12 +545,23 @@ extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, voi
     return check_launch("gemm");
   }
   const int bm = cfg.tile[0], bn = cfg.tile[1];
-  if (bm == 256 && bn == 256) return launch_mfma<256, 256, 2, 4>(s, a, w, b, c, M, N, K);
-  if (bm == 256 && bn == 128) return launch_mfma<256, 128, 2, 2>(s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 256) return launch_mfma<128, 256, 2, 2>(s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2>(s, a, w, b, c, M, N, K);
-  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2>(s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2>(s, a, w, b, c, M, N, K);
-  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2>(s, a, w, b, c, M, N, K);
+  const int ns = cfg.unroll >= 2 ? cfg.unroll : 0;
+  if (bm == 256 && bn == 256) return launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K);
+  if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K)
+                                             : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K);
+  if (bm == 128 && bn == 256) return ns == 2 ? launch_mfma<128, 256, 2, 2, 2>(s, a, w, b, c, M, N, K)
+                                             : launch_mfma<128, 256, 2, 2, 3>(s, a, w, b, c, M, N, K);
+  if (bm == 128 && bn == 128) return ns == 2   ? launch_mfma<128, 128, 2, 2, 2>(s, a, w, b, c, M, N, K)
+                                     : ns == 3 ? launch_mfma<128, 128, 2, 2, 3>(s, a, w, b, c, M, N, K)
+                                               : launch_mfma<128, 128, 2, 2, 4>(s, a, w, b, c, M, N, K);
+  if (bm == 64 && bn == 128) return ns == 2   ? launch_mfma<64, 128, 2, 2, 2>(s, a, w, b, c, M, N, K)
+                                    : ns == 3 ? launch_mfma<64, 128, 2, 2, 3>(s, a, w, b, c, M, N, K)
+                                              : launch_mfma<64, 128, 2, 2, 4>(s, a, w, b, c, M, N, K);
+  if (bm == 128 && bn == 64) return ns == 2   ? launch_mfma<128, 64, 2, 2, 2>(s, a, w, b, c, M, N, K)
+                                    : ns == 3 ? launch_mfma<128, 64, 2, 2, 3>(s, a, w, b, c, M, N, K)
+                                              : launch_mfma<128, 64, 2, 2, 4>(s, a, w, b, c, M, N, K);
+  if (bm == 64 && bn == 64) return ns == 2   ? launch_mfma<64, 64, 2, 2, 2>(s, a, w, b, c, M, N, K)
+                                   : ns == 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, b, c, M, N, K)
+                                             : launch_mfma<64, 64, 2, 2, 4>(s, a, w, b, c, M, N, K);
   return fail("gemm: no MFMA kernel for tile %dx%d", bm, bn);
 }

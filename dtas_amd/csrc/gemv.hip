@@ -130,10 +130,7 @@ extern "C" int dtas_gemv_f16(const void* x, const void* W, const void* bias, voi
   if (overlaps(y, N * 2, W, N * K * 2) || overlaps(y, N * 2, x, K * 2)) return fail("gemv: output overlaps an input");
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMV_F16, 1, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(x, 16) && aligned(W, 16);
-  if (cfg.vec == 8 && !vec_ok) {
-    if (user) return fail("gemv: 128-bit accesses need K %% 8 == 0 and 16-byte aligned x, W");
-    cfg.vec = 1;
-  }
+  if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
   int64_t la[7];
   if (describe_gemv(N, K, cfg, la) != 0) return -1;
   const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));

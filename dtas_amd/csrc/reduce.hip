@@ -331,20 +331,15 @@ int run_reduction(int op, const void* x, const void* p1, const void* p2, void* o
 
   const bool vec_ok = cols % r.vec == 0 && aligned(x, 16) && aligned(out, r.vec * 2) &&
                       (!needs_p1 || aligned(p1, 16)) && (!needs_p2 || aligned(p2, 16));
-  dtas_config cfg;
-  if (user) {
-    cfg = *user;
-    if (cfg.variant != DTAS_RED_STREAM_ROW && !vec_ok)
-      return fail("%s: 128-bit row accesses need cols %% %d == 0 and 16-byte aligned buffers", r.name, r.vec);
-  } else {
-    // dynamic extent: the row count for the norms, the row length for softmax
-    const bool softmax = r.kind == kSoftmaxF32 || r.kind == kSoftmaxF16;
-    cfg = builtin_config(op, softmax ? cols : rows, softmax ? rows : cols, softmax ? cols : 0).cfg;
-    if (cfg.variant != DTAS_RED_STREAM_ROW && !vec_ok) {
-      cfg.variant = DTAS_RED_STREAM_ROW;
-      cfg.block = cols >= 4096 ? 1024 : cols >= 1024 ? 512 : 256;
-      cfg.vec = 1;
-    }
+  // dynamic extent: the row count for the norms, the row length for softmax
+  const bool softmax = r.kind == kSoftmaxF32 || r.kind == kSoftmaxF16;
+  dtas_config cfg = user ? *user : builtin_config(op, softmax ? cols : rows, softmax ? rows : cols, softmax ? cols : 0).cfg;
+  // 128-bit row accesses need cols % vec == 0 and 16-byte aligned buffers; other rows take the
+  // element-access kernel (a bucket's config must serve every n in the bucket)
+  if (cfg.variant != DTAS_RED_STREAM_ROW && !vec_ok) {
+    cfg.variant = DTAS_RED_STREAM_ROW;
+    if (!user) cfg.block = cols >= 4096 ? 1024 : cols >= 1024 ? 512 : 256;
+    cfg.vec = 1;
   }
   int64_t la[7];
   if (describe_reduction(op, rows, cols, cfg, la) != 0) return -1;

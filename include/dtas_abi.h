@@ -21,7 +21,9 @@
  *  - `stream` is a hipStream_t (NULL = the default stream); nothing is allocated, nothing
  *    synchronises, the kernel is enqueued on `stream` on the current device;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
- *    reference's call_table holds); NULL = use the library's built-in bucket table;
+ *    reference's call_table holds); NULL = use the library's built-in bucket table; either way a
+ *    128-bit variant steps down to its element-access kernel for extents or pointers that do not
+ *    allow 128-bit accesses (a bucket's row must serve every n and buffer that falls in it);
  *  - returns 0 on success, -1 on error (the reference's host functions do the same,
  *    host.cc:75-83,133-143); dtas_last_error() gives the thread-local message;
  *  - n == 0 (an empty dynamic extent) is a no-op that returns 0; negative extents, NULL
@@ -89,7 +91,7 @@ typedef struct dtas_config {
   int32_t variant;  /* enum dtas_variant of the op's family */
   int32_t block;    /* threads per workgroup = launch_args[1] */
   int32_t vec;      /* elements per vector access */
-  int32_t unroll;   /* independent vector accesses in flight per thread / rows per wavefront */
+  int32_t unroll;   /* independent vector accesses in flight per thread; GEMM: LDS stages (0 = max) */
   int32_t tile[3];  /* GEMM: workgroup tile M, N, K; GEMV: rows per workgroup, -, - */
   int32_t split_k;  /* GEMV/GEMM: number of K partitions (1 = none) */
   int64_t grid_cap; /* upper limit on workgroups (then the kernel loops); 0 = no limit */

@@ -163,8 +163,12 @@ def test_odd_alignment_steps_down_to_element_accesses(oracle):
     got = raw.cpu().numpy()
     assert_bits_equal(got[3:5000], oracle.c.add(base_a[1:4998].copy(), base_b[1:4998].copy()))
     assert (got[:3] == 9).all() and (got[5000:] == 9).all()
-    with pytest.raises(_lib.DtasError, match="not aligned"):  # an explicit vector config is taken at its word
-        ops.add(da[1:4998], db[1:4998], raw[3:5000], cfg(vec=8, unroll=1))
+    # an explicit vector config steps down the same way: a bucket's row must serve every buffer
+    raw.fill_(9.0)
+    ops.add(da[1:4998], db[1:4998], raw[3:5000], cfg(vec=8, unroll=4))
+    got = raw.cpu().numpy()
+    assert_bits_equal(got[3:5000], oracle.c.add(base_a[1:4998].copy(), base_b[1:4998].copy()))
+    assert (got[:3] == 9).all() and (got[5000:] == 9).all()
 
 
 def test_errors_on_the_gpu_path():
