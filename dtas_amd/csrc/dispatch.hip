@@ -72,39 +72,43 @@ dtas_config elementwise_policy(int op, int64_t n_hi, int64_t H) {
   return make(DTAS_ELT_VECTOR, 256, vec, unroll);
 }
 
-int pow2_at_most(int64_t v) {
-  int p = 1;
-  while (2 * p <= v) p *= 2;
-  return p;
-}
-
-// One workgroup per row, sized for about two 128-bit vectors per thread.
-dtas_config block_row(int vec, int64_t nvec) {
-  int block = pow2_at_most(nvec / 2 > 64 ? nvec / 2 : 64);
+// One workgroup per `rows_per_trip` rows, sized for about two 128-bit vectors per thread and row
+// (a multiple of 64 threads, so that 640 vectors take 320 threads x 2 and no lane idles).
+dtas_config block_row(int vec, int64_t nvec, int rows_per_trip) {
+  int64_t block = ((nvec + 1) / 2 + 63) / 64 * 64;
   if (block > 1024) block = 1024;
-  if (nvec > static_cast<int64_t>(block) * 16) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
-  return make(DTAS_RED_BLOCK_ROW, block, vec, 1);
+  const int64_t iters = (nvec + block - 1) / block;
+  if (iters > 8) return make(DTAS_RED_STREAM_ROW, 1024, 1, 1);
+  while (rows_per_trip > 1 && iters * rows_per_trip > 8) rows_per_trip /= 2;
+  return make(DTAS_RED_BLOCK_ROW, static_cast<int>(block), vec, rows_per_trip);
 }
 
-// Norms: n rows of static length H.  From ~8 rows per CU on, one wavefront per row (all
-// reductions on the DPP path, no barrier) wins, provided a lane holds at most 8 vectors; below
-// that, and for longer rows (fp32 rows of 2560 need 10), a workgroup per row hides latency better.
+// Norms: n rows of static length H, a workgroup per row.  From ~8 rows per CU on, a workgroup
+// takes several rows per trip: their loads are in flight together and the per-column parameters
+// are fetched once for all of them (4 rows for RMSNorm's one parameter vector, 2 for
+// LayerNorm's two fp32 ones, which cost registers).
 dtas_config norm_policy(int op, int64_t n_hi, int64_t H) {
   const int vec = op == DTAS_OP_RMS_NORM_F16 ? 8 : 4;
   const int64_t nvec = (H + vec - 1) / vec;
-  if (n_hi >= 8 * kNumCU && nvec <= 64 * 8) return make(DTAS_RED_WAVE_ROW, 256, vec, 1);
-  return block_row(vec, nvec);
+  if (op == DTAS_OP_RMS_NORM_F16) return block_row(vec, nvec, n_hi >= 8 * kNumCU ? 4 : 1);
+  // LayerNorm, 8 to 16 rows per CU: narrow workgroups (about five vectors per thread) are all
+  // co-resident and measured ~15 % faster than wide ones, which need a second, partial round.
+  const int64_t narrow = ((nvec + 4) / 5 + 63) / 64 * 64;
+  if (n_hi >= 8 * kNumCU && n_hi <= 16 * kNumCU && narrow <= 1024 && (nvec + narrow - 1) / narrow <= 5)
+    return make(DTAS_RED_BLOCK_ROW, static_cast<int>(narrow), vec, 2);
+  return block_row(vec, nvec, n_hi >= 8 * kNumCU ? 2 : 1);
 }
 
 // Softmax: 32*n rows of dynamic length n (the reduction axis is the dynamic one).  One wavefront
-// per row up to 16 vectors per lane; short rows launch one row per workgroup so that the many
-// small workgroups spread evenly.
+// per row (reductions on the DPP path only) up to 8 vectors per lane; short rows launch one
+// row per workgroup so that the many small workgroups spread evenly.  Longer rows, or few
+// rows, take a workgroup per row.
 dtas_config softmax_policy(int op, int64_t cols_hi, int64_t rows) {
   const int vec = op == DTAS_OP_SOFTMAX_F16 ? 8 : 4;
   const int64_t nvec = (cols_hi + vec - 1) / vec;
-  if (nvec <= 64 * 16 && (rows <= 0 || rows > 2 * kNumCU))
+  if (nvec < 64 * 8 && (rows <= 0 || rows > 2 * kNumCU))
     return make(DTAS_RED_WAVE_ROW, nvec <= 64 ? 64 : 256, vec, 1);
-  return block_row(vec, nvec);
+  return block_row(vec, nvec, 1);
 }
 
 // GEMV: one row of W per workgroup of 4 wavefronts keeps the most independent streams in

@@ -57,17 +57,45 @@ struct MaxOp {
   static __device__ __forceinline__ float join(float a, float b) { return fmaxf(a, b); }
 };
 
+// Workgroup reductions through 2 x 16 LDS slots.  Consecutive reductions alternate between the
+// two banks (`phase` counts them), so a bank is rewritten only after a barrier that every reader
+// of its previous contents has passed: one barrier per reduction.  The partial results are
+// joined in wavefront order by every thread, so all threads hold the same bits.
 template <typename Op>
-__device__ __forceinline__ float block_reduce(float v, float* slots) {
+__device__ __forceinline__ float block_reduce(float v, float* slots, int& phase) {
   const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const float w = Op::wave(v);
   if (nwaves == 1) return w;
-  __syncthreads();  // slots may still be read by the previous reduction
-  if ((threadIdx.x & 63) == 0) slots[wave] = w;
+  float* bank = slots + ((phase++ & 1) << 4);
+  if ((threadIdx.x & 63) == 0) bank[wave] = w;
   __syncthreads();
-  float r = slots[0];
-  for (int i = 1; i < nwaves; ++i) r = Op::join(r, slots[i]);
+  float r = bank[0];
+  for (int i = 1; i < nwaves; ++i) r = Op::join(r, bank[i]);
   return r;
+}
+
+// Two sums behind one barrier; `slots` holds 2 x 32 floats.
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* slots, int& phase) {
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const float wa = SumOp::wave(a), wb = SumOp::wave(b);
+  if (nwaves == 1) {
+    a = wa;
+    b = wb;
+    return;
+  }
+  float* bank = slots + ((phase++ & 1) << 5);
+  if ((threadIdx.x & 63) == 0) {
+    bank[wave] = wa;
+    bank[16 + wave] = wb;
+  }
+  __syncthreads();
+  float ra = bank[0], rb = bank[16];
+  for (int i = 1; i < nwaves; ++i) {
+    ra += bank[i];
+    rb += bank[16 + i];
+  }
+  a = ra;
+  b = rb;
 }
 
 // ---- streaming (touch-once) global accesses ---------------------------------------

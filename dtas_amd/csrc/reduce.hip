@@ -82,128 +82,206 @@ __device__ __forceinline__ void store_half_vec(half_t* dst, const float (&v)[VEC
   }
 }
 
-template <bool BLOCK, typename Op>
-__device__ __forceinline__ float group_reduce(float v, float* slots) {
-  return BLOCK ? block_reduce<Op>(v, slots) : Op::wave(v);
+// N independent reductions at once: DPP inside each wavefront, then (BLOCK) one LDS slot per
+// wavefront and value, joined in wavefront order by every thread.  Consecutive calls alternate
+// between two banks of N x 16 slots (`phase` counts them), so a bank is rewritten only after a
+// barrier that every reader of its previous contents has passed: one barrier per call.
+template <bool BLOCK, typename Op, int N>
+__device__ __forceinline__ void group_reduce(float (&a)[N], float* slots, int& phase) {
+#pragma unroll
+  for (int k = 0; k < N; ++k) a[k] = Op::wave(a[k]);
+  if (!BLOCK) return;
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  if (nwaves == 1) return;
+  float* bank = slots + (phase++ & 1) * (N * 16);
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) bank[k * 16 + wave] = a[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    float r = bank[k * 16];
+    for (int i = 1; i < nwaves; ++i) r = Op::join(r, bank[k * 16 + i]);
+    a[k] = r;
+  }
 }
 
-// ---- row held in registers ----------------------------------------------------------
+// ---- rows held in registers ---------------------------------------------------------
 // rows: number of rows; cols: row length, a multiple of kVec, every row 16-byte aligned.
-template <int OP, int ITERS, bool BLOCK>
-__global__ void __launch_bounds__(1024) row_reg_kernel(const void* __restrict__ xin, const void* __restrict__ p1,
-                                                       const void* __restrict__ p2, void* __restrict__ outp,
-                                                       int64_t rows, int64_t cols, float eps) {
+// A lane group (wavefront or workgroup) takes R consecutive rows per trip: all R x ITERS loads
+// are in flight together, the R rows share each barrier, and the per-column parameters
+// (w, or gamma and beta) are fetched once for the R rows.
+// More than 8 vectors per lane need more registers than a 1024-thread workgroup leaves each lane.
+template <int OP, int ITERS, bool BLOCK, int R>
+__global__ void __launch_bounds__(ITERS * R > 8 ? 512 : 1024) row_reg_kernel(
+    const void* __restrict__ xin, const void* __restrict__ p1, const void* __restrict__ p2, void* __restrict__ outp,
+    int64_t rows, int64_t cols, float eps) {
   typedef typename RowTraits<OP>::In In;
   constexpr int VEC = RowTraits<OP>::kVec;
   typedef RowVec<In, VEC> V;
-  __shared__ float slots[16];
+  __shared__ float slots[BLOCK ? 2 * 2 * R * 16 : 1];
+  int phase = 0;
 
   const int lane = BLOCK ? threadIdx.x : (threadIdx.x & 63);
   const int width = BLOCK ? blockDim.x : 64;
-  const int64_t rows_per_wg = BLOCK ? 1 : (blockDim.x >> 6);
+  const int64_t trip_rows = static_cast<int64_t>(R) * (BLOCK ? 1 : (blockDim.x >> 6));
   const int64_t nvec = cols / VEC;
   const float inv_cols = 1.0f / static_cast<float>(cols);
   half_t* out = static_cast<half_t*>(outp);
+  bool has[ITERS];  // which of this lane's vector slots lie inside the row
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) has[it] = lane + static_cast<int64_t>(it) * width < nvec;
 
-  // every thread of a workgroup runs the same number of trips (BLOCK: same row;
-  // WAVE: rows differ per wavefront but no workgroup barrier is used)
-  for (int64_t row = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (BLOCK ? 0 : (threadIdx.x >> 6)); row < rows;
-       row += static_cast<int64_t>(gridDim.x) * rows_per_wg) {
-    const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const In*>(xin) + row * cols);
-    V v[ITERS];
+  // A lane covers the same columns of every row, so its slices of the parameters are loaded
+  // once per kernel; very long rows re-read them from the cache per trip
+  // instead and keep the registers for the rows.
+  constexpr bool HOIST = (OP == kRms || OP == kLayerNorm) && ITERS * (R + (OP == kLayerNorm ? 2 : 1)) <= 16;
+  V pw[HOIST ? ITERS : 1], pb[HOIST ? ITERS : 1];
+  if (HOIST) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int64_t i = lane + static_cast<int64_t>(it) * width;
-      if (i < nvec) v[it].raw = load_stream(src + i);
+      if (has[it]) {
+        pw[it].raw = static_cast<const u32x4*>(p1)[lane + it * width];
+        if (OP == kLayerNorm) pb[it].raw = static_cast<const u32x4*>(p2)[lane + it * width];
+      }
     }
+  }
+  auto param = [&](const void* p, const V* held, int it) -> V {
+    if (HOIST) return held[it];
+    V r;
+    r.raw = static_cast<const u32x4*>(p)[lane + it * width];
+    return r;
+  };
 
-    if (OP == kRms) {
-      float ss = 0.f;
+  // every thread of a workgroup runs the same number of trips (BLOCK: same rows;
+  // WAVE: rows differ per wavefront but no workgroup barrier is used)
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * trip_rows + (BLOCK ? 0 : (threadIdx.x >> 6) * R); base < rows;
+       base += static_cast<int64_t>(gridDim.x) * trip_rows) {
+    V v[R][ITERS];
+    bool live[R];  // rows past the end take part in the barriers only
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      live[r] = base + r < rows;
+      const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const In*>(xin) + (base + r) * cols);
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
-        if (lane + static_cast<int64_t>(it) * width < nvec) {
+        v[r][it].raw = u32x4{0u, 0u, 0u, 0u};
+        if (live[r] && has[it]) v[r][it].raw = load_stream(src + lane + it * width);
+      }
+    }
+    auto store_row = [&](int r, int it, const float (&res)[VEC]) {
+      store_half_vec<VEC>(out + (base + r) * cols + (lane + static_cast<int64_t>(it) * width) * VEC, res);
+    };
+
+    if (OP == kRms) {
+      float ss[R];
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) {
-            const float f = v[it].get(e);
-            ss += f * f;
+      for (int r = 0; r < R; ++r) {
+        ss[r] = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          if (has[it]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const float f = v[r][it].get(e);
+              ss[r] += f * f;
+            }
           }
         }
       }
-      ss = group_reduce<BLOCK, SumOp>(ss, slots);
-      const float rs = __builtin_amdgcn_rsqf(ss * inv_cols + eps);
-      const u32x4* wv = static_cast<const u32x4*>(p1);
+      group_reduce<BLOCK, SumOp>(ss, slots, phase);
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
-        const int64_t i = lane + static_cast<int64_t>(it) * width;
-        if (i < nvec) {
-          V w;
-          w.raw = wv[i];
-          float r[VEC];
+        if (has[it]) {
+          const V w = param(p1, pw, it);
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) r[e] = v[it].get(e) * rs * w.get(e);
-          store_half_vec<VEC>(out + row * cols + i * VEC, r);
+          for (int r = 0; r < R; ++r) {
+            if (live[r]) {
+              const float rs = __builtin_amdgcn_rsqf(ss[r] * inv_cols + eps);
+              float res[VEC];
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) res[e] = v[r][it].get(e) * rs * w.get(e);
+              store_row(r, it, res);
+            }
+          }
         }
       }
     } else if (OP == kLayerNorm) {
-      float s0 = 0.f, s1 = 0.f;
+      float st[2 * R];  // sum and sum of squares per row
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          if (has[it]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const float f = v[r][it].get(e);
+              s0 += f;
+              s1 += f * f;
+            }
+          }
+        }
+        st[2 * r] = s0;
+        st[2 * r + 1] = s1;
+      }
+      group_reduce<BLOCK, SumOp>(st, slots, phase);
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
-        if (lane + static_cast<int64_t>(it) * width < nvec) {
+        if (has[it]) {
+          const V g = param(p1, pw, it), b = param(p2, pb, it);
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) {
-            const float f = v[it].get(e);
-            s0 += f;
-            s1 += f * f;
+          for (int r = 0; r < R; ++r) {
+            if (live[r]) {
+              const float mean = st[2 * r] * inv_cols;
+              const float rstd = __builtin_amdgcn_rsqf(st[2 * r + 1] * inv_cols - mean * mean + eps);
+              float res[VEC];
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) res[e] = (v[r][it].get(e) - mean) * rstd * g.get(e) + b.get(e);
+              store_row(r, it, res);
+            }
           }
         }
       }
-      s0 = group_reduce<BLOCK, SumOp>(s0, slots);
-      s1 = group_reduce<BLOCK, SumOp>(s1, slots);
-      const float mean = s0 * inv_cols;
-      const float rstd = __builtin_amdgcn_rsqf(s1 * inv_cols - mean * mean + eps);
-      const u32x4* gv = static_cast<const u32x4*>(p1);
-      const u32x4* bv = static_cast<const u32x4*>(p2);
-#pragma unroll
-      for (int it = 0; it < ITERS; ++it) {
-        const int64_t i = lane + static_cast<int64_t>(it) * width;
-        if (i < nvec) {
-          V g, b;
-          g.raw = gv[i];
-          b.raw = bv[i];
-          float r[VEC];
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) r[e] = (v[it].get(e) - mean) * rstd * g.get(e) + b.get(e);
-          store_half_vec<VEC>(out + row * cols + i * VEC, r);
-        }
-      }
     } else {  // softmax
-      float mx = kNegMax;
+      float mx[R], sm[R];
 #pragma unroll
-      for (int it = 0; it < ITERS; ++it) {
-        if (lane + static_cast<int64_t>(it) * width < nvec) {
+      for (int r = 0; r < R; ++r) {
+        mx[r] = kNegMax;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) mx = fmaxf(mx, v[it].get(e));
+        for (int it = 0; it < ITERS; ++it) {
+          if (has[it]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) mx[r] = fmaxf(mx[r], v[r][it].get(e));
+          }
         }
       }
-      mx = group_reduce<BLOCK, MaxOp>(mx, slots);
-      float s = 0.f;
+      group_reduce<BLOCK, MaxOp>(mx, slots, phase);
 #pragma unroll
-      for (int it = 0; it < ITERS; ++it) {
-        if (lane + static_cast<int64_t>(it) * width < nvec) {
+      for (int r = 0; r < R; ++r) {
+        sm[r] = 0.f;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) s += fast_exp(v[it].get(e) - mx);
+        for (int it = 0; it < ITERS; ++it) {
+          if (has[it]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) sm[r] += fast_exp(v[r][it].get(e) - mx[r]);
+          }
         }
       }
-      s = group_reduce<BLOCK, SumOp>(s, slots);
-      const float inv = 1.0f / s;
+      group_reduce<BLOCK, SumOp>(sm, slots, phase);
 #pragma unroll
-      for (int it = 0; it < ITERS; ++it) {
-        const int64_t i = lane + static_cast<int64_t>(it) * width;
-        if (i < nvec) {
-          float r[VEC];
+      for (int r = 0; r < R; ++r) {
+        if (!live[r]) continue;
+        const float inv = 1.0f / sm[r];
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) r[e] = fast_exp(v[it].get(e) - mx) * inv;
-          store_half_vec<VEC>(out + row * cols + i * VEC, r);
+        for (int it = 0; it < ITERS; ++it) {
+          if (has[it]) {
+            float res[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) res[e] = fast_exp(v[r][it].get(e) - mx[r]) * inv;
+            store_row(r, it, res);
+          }
         }
       }
     }
@@ -216,7 +294,8 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const void* __restrict
                                                           const void* __restrict__ p2, void* __restrict__ outp,
                                                           int64_t rows, int64_t cols, float eps) {
   typedef typename RowTraits<OP>::In In;
-  __shared__ float slots[16];
+  __shared__ float slots[64];
+  int phase = 0;
   const float inv_cols = 1.0f / static_cast<float>(cols);
   half_t* out = static_cast<half_t*>(outp);
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
@@ -228,7 +307,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const void* __restrict
         const float f = static_cast<float>(x[k]);
         ss += f * f;
       }
-      ss = block_reduce<SumOp>(ss, slots);
+      ss = block_reduce<SumOp>(ss, slots, phase);
       const float rs = __builtin_amdgcn_rsqf(ss * inv_cols + eps);
       const half_t* w = static_cast<const half_t*>(p1);
       for (int64_t k = threadIdx.x; k < cols; k += blockDim.x)
@@ -240,8 +319,7 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const void* __restrict
         s0 += f;
         s1 += f * f;
       }
-      s0 = block_reduce<SumOp>(s0, slots);
-      s1 = block_reduce<SumOp>(s1, slots);
+      block_sum2(s0, s1, slots, phase);
       const float mean = s0 * inv_cols;
       const float rstd = __builtin_amdgcn_rsqf(s1 * inv_cols - mean * mean + eps);
       const float* g = static_cast<const float*>(p1);
@@ -251,10 +329,10 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const void* __restrict
     } else {
       float mx = kNegMax;
       for (int64_t k = threadIdx.x; k < cols; k += blockDim.x) mx = fmaxf(mx, static_cast<float>(x[k]));
-      mx = block_reduce<MaxOp>(mx, slots);
+      mx = block_reduce<MaxOp>(mx, slots, phase);
       float s = 0.f;
       for (int64_t k = threadIdx.x; k < cols; k += blockDim.x) s += fast_exp(static_cast<float>(x[k]) - mx);
-      s = block_reduce<SumOp>(s, slots);
+      s = block_reduce<SumOp>(s, slots, phase);
       const float inv = 1.0f / s;
       for (int64_t k = threadIdx.x; k < cols; k += blockDim.x)
         o[k] = static_cast<half_t>(fast_exp(static_cast<float>(x[k]) - mx) * inv);
@@ -262,21 +340,27 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const void* __restrict
   }
 }
 
+// instantiated (vectors per lane, rows per trip) pairs: ITERS * R <= 16
 template <int OP, bool BLOCK>
-int launch_reg(int iters, dim3 grid, dim3 block, hipStream_t s, const void* x, const void* p1, const void* p2, void* out,
-               int64_t rows, int64_t cols, float eps) {
-#define DTAS_ROW_CASE(I)                                                                                         \
-  case I:                                                                                                        \
-    hipLaunchKernelGGL((row_reg_kernel<OP, I, BLOCK>), grid, block, 0, s, x, p1, p2, out, rows, cols, eps);      \
+int launch_reg(int iters, int rpt, dim3 grid, dim3 block, hipStream_t s, const void* x, const void* p1,
+               const void* p2, void* out, int64_t rows, int64_t cols, float eps) {
+#define DTAS_ROW_CASE(I, R)                                                                                      \
+  case I * 8 + R:                                                                                                \
+    hipLaunchKernelGGL((row_reg_kernel<OP, I, BLOCK, R>), grid, block, 0, s, x, p1, p2, out, rows, cols, eps);   \
     break;
-  switch (iters) {
-    DTAS_ROW_CASE(1)
-    DTAS_ROW_CASE(2)
-    DTAS_ROW_CASE(4)
-    DTAS_ROW_CASE(8)
-    DTAS_ROW_CASE(16)
+  switch (iters * 8 + rpt) {
+    DTAS_ROW_CASE(1, 1) DTAS_ROW_CASE(1, 2) DTAS_ROW_CASE(1, 4)
+    DTAS_ROW_CASE(2, 1) DTAS_ROW_CASE(2, 2) DTAS_ROW_CASE(2, 4)
+    DTAS_ROW_CASE(3, 1) DTAS_ROW_CASE(3, 2) DTAS_ROW_CASE(3, 4)
+    DTAS_ROW_CASE(4, 1) DTAS_ROW_CASE(4, 2) DTAS_ROW_CASE(4, 4)
+    DTAS_ROW_CASE(5, 1) DTAS_ROW_CASE(5, 2)
+    DTAS_ROW_CASE(6, 1) DTAS_ROW_CASE(6, 2)
+    DTAS_ROW_CASE(8, 1) DTAS_ROW_CASE(8, 2)
+    DTAS_ROW_CASE(10, 1)
+    DTAS_ROW_CASE(12, 1)
+    DTAS_ROW_CASE(16, 1)
     default:
-      return fail("reduction: %d vectors per lane is not one of 1, 2, 4, 8, 16", iters);
+      return fail("reduction: %d vectors per lane x %d rows per trip is not instantiated", iters, rpt);
   }
 #undef DTAS_ROW_CASE
   return check_launch("reduction");
@@ -297,11 +381,16 @@ bool red_info(int op, RedInfo* r) {
   return false;
 }
 
-int pow2_at_least(int64_t v) {
-  int p = 1;
-  while (p < v) p <<= 1;
-  return p;
+// the instantiated vectors-per-lane counts; 17 = too long
+int iters_at_least(int64_t v) {
+  static const int kIters[] = {1, 2, 3, 4, 5, 6, 8, 10, 12, 16};
+  for (int i : kIters)
+    if (i >= v) return i;
+  return 17;
 }
+
+// cfg.unroll of a register variant: rows a lane group takes per trip (0 and 1 both mean one)
+int rows_per_trip(const dtas_config& cfg) { return cfg.unroll <= 1 ? 1 : cfg.unroll; }
 
 template <int OP>
 int launch_rows(const dtas_config& cfg, const int64_t la[7], hipStream_t s, const void* x, const void* p1,
@@ -311,9 +400,9 @@ int launch_rows(const dtas_config& cfg, const int64_t la[7], hipStream_t s, cons
     hipLaunchKernelGGL((row_stream_kernel<OP>), grid, block, 0, s, x, p1, p2, out, rows, cols, eps);
     return check_launch("reduction");
   }
-  const int iters = static_cast<int>(la[5]);
-  if (cfg.variant == DTAS_RED_WAVE_ROW) return launch_reg<OP, false>(iters, grid, block, s, x, p1, p2, out, rows, cols, eps);
-  return launch_reg<OP, true>(iters, grid, block, s, x, p1, p2, out, rows, cols, eps);
+  const int iters = static_cast<int>(la[5]), rpt = rows_per_trip(cfg);
+  if (cfg.variant == DTAS_RED_WAVE_ROW) return launch_reg<OP, false>(iters, rpt, grid, block, s, x, p1, p2, out, rows, cols, eps);
+  return launch_reg<OP, true>(iters, rpt, grid, block, s, x, p1, p2, out, rows, cols, eps);
 }
 
 int run_reduction(int op, const void* x, const void* p1, const void* p2, void* out, int64_t rows, int64_t cols,
@@ -355,7 +444,20 @@ int run_reduction(int op, const void* x, const void* p1, const void* p2, void* o
 
 }  // namespace
 
-// launch_args: {grid, 1, 1, block, 0, vectors per lane (register variants), rows per workgroup}
+namespace {
+bool rows_per_trip_ok(const char* name, int iters, int rpt, int block) {
+  if (iters * rpt > 8 && block > 512) {
+    fail("%s: %d vectors per lane x %d rows per trip need a block of at most 512 threads, got %d", name, iters, rpt, block);
+    return false;
+  }
+  if (rpt == 1 || (rpt == 2 && iters <= 8) || (rpt == 4 && iters <= 4)) return true;
+  fail("%s: unroll (rows per trip) %d is not available with %d vectors per lane (1, 2 or 4; 2 up to 8 vectors, 4 up to 4)",
+       name, rpt, iters);
+  return false;
+}
+}  // namespace
+
+// launch_args: {grid, 1, 1, block, 0, vectors per lane (register variants), rows per workgroup and trip}
 int describe_reduction(int op, int64_t rows, int64_t cols, const dtas_config& cfg, int64_t la[7]) {
   RedInfo r;
   if (!red_info(op, &r)) return fail("reduction: unknown op %d", op);
@@ -365,20 +467,23 @@ int describe_reduction(int op, int64_t rows, int64_t cols, const dtas_config& cf
   la[1] = la[2] = 1;
   la[3] = cfg.block;
   int64_t grid;
+  const int rpt = rows_per_trip(cfg);
   if (cfg.variant == DTAS_RED_WAVE_ROW) {
     const int64_t nvec = ceil_div(cols, r.vec);
-    const int iters = pow2_at_least(ceil_div(nvec, 64));
+    const int iters = iters_at_least(ceil_div(nvec, 64));
     if (iters > 16) return fail("%s: a row of %lld elements does not fit one wavefront's registers", r.name, (long long)cols);
+    if (!rows_per_trip_ok(r.name, iters, rpt, cfg.block)) return -1;
     la[5] = iters;
-    la[6] = cfg.block / 64;
-    grid = ceil_div(rows, cfg.block / 64);
+    la[6] = cfg.block / 64 * rpt;
+    grid = ceil_div(rows, la[6]);
   } else if (cfg.variant == DTAS_RED_BLOCK_ROW) {
     const int64_t nvec = ceil_div(cols, r.vec);
-    const int iters = pow2_at_least(ceil_div(nvec, cfg.block));
+    const int iters = iters_at_least(ceil_div(nvec, cfg.block));
     if (iters > 16) return fail("%s: a row of %lld elements does not fit %d threads' registers", r.name, (long long)cols, cfg.block);
+    if (!rows_per_trip_ok(r.name, iters, rpt, cfg.block)) return -1;
     la[5] = iters;
-    la[6] = 1;
-    grid = rows;
+    la[6] = rpt;
+    grid = ceil_div(rows, rpt);
   } else if (cfg.variant == DTAS_RED_STREAM_ROW) {
     la[6] = 1;
     grid = rows;
