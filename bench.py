@@ -268,7 +268,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
-                    help="cast_f32_f16 | add_f16 | copy_f16 | rms_norm_f16 | softmax_f16 | gemv_f16 | gemm_f16")
+                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | "
+                         "gemv_f16 | gemm_f16")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -305,6 +306,16 @@ def main() -> int:
     except _lib.DtasError:
         info = None
 
+    if args.workload == "layer_norm_f32_f16":
+        workload_key = f"{args.workload} [n={args.n}, 2560]"
+    elif args.workload == "softmax_f16":
+        workload_key = f"{args.workload} [{32 * args.n}, n={args.n}]"
+    elif extra is None:
+        workload_key = f"{args.workload} [n={args.n}, 4096]"
+    elif args.workload == "gemv_f16":
+        workload_key = f"gemv_f16 M=1 NxK={args.nk}"
+    else:
+        workload_key = f"{args.workload} M={args.n} NxK={args.nk}"
     line = {
         "metric": METRIC,
         "value": round(head["flops"] * args.steps / (head["ms_per_step"] * 1e-3 * args.steps) / 1e12, 3) if is_gemm
@@ -314,7 +325,7 @@ def main() -> int:
         "ms_per_step": round(head["ms_per_step"], 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"{args.workload} [n={args.n}, 4096]" if extra is None else f"{args.workload} M={args.n} NxK={args.nk}",
+        "config": {"workload": workload_key,
                    "buffers": "rotating pool > 3x Infinity Cache" if not args.cache_resident else "single set (cache-resident)",
                    "pool_sets": head["pool"],
                    "kernel": info.name.decode() if info is not None else args.workload,
@@ -325,7 +336,7 @@ def main() -> int:
             "peak": MFMA_FP16_PEAK_TFLOPS if is_gemm else HBM_PEAK_GBS,
             "unit": "TFLOP/s" if is_gemm else "GB/s",
             "frac": round((head["tflops"] / MFMA_FP16_PEAK_TFLOPS) if is_gemm else head["gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": recorded_traffic(f"{args.workload} [n={args.n}, 4096]") if extra is None else None,
+            "traffic": recorded_traffic(workload_key),
             "launch_us_mean": head["us"],
             "algorithmic_bytes_per_launch": head["bytes"],
         },
