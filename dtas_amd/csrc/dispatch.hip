@@ -119,38 +119,53 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
   return make(DTAS_GEMV_SPLITK, 256, 8, 2, 1);
 }
 
-// GEMM, from sweeps of every tile x stage count over M on an MI355X:
-//  * M <= 32 and N <= 6144: the W-streaming SKINNY kernel (its time grows with N*K, the 64x64
-//    MFMA loop's with K only);
+// GEMM, from sweeps of every tile x stage count x K split over M on an MI355X:
 //  * 256x256 (8 wavefronts, ping-pong) once it yields >= 150 workgroups;
-//  * else 128x128 once that yields >= 256 workgroups;
-//  * else 64x64: few workgroups, each latency bound, so as many LDS stages as possible.
-// LDS stages (depth of the load pipeline): more stages hide more latency but fewer workgroups
-// fit a CU; take the deepest pipeline with which all tiles are still co-resident (with a
-// margin when several workgroups share a CU), else 2.
+//  * else 128x128 once that yields >= 256 workgroups, with the deepest LDS pipeline that keeps
+//    all tiles co-resident;
+//  * else few tiles: each workgroup's k loop is a chain of ~0.3 us (64x64) / ~0.6 us (128x128)
+//    steps however few CUs are busy, so K is split over up to 4 workgroups per tile (partials
+//    summed by the last one to arrive, ~1 us / ~4 us per partial).  The cheapest of the candidates
+//    under that model is taken; against it, for M <= 32, the W-streaming SKINNY kernel, whose
+//    time grows with N*K (about 3.5 TB/s of W) instead of with K.
+struct GemmChoice {
+  double us;
+  int tile, split;
+};
+
 dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
-  (void)K;
-  if (M_hi <= 32 && N <= 6144) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
-  const int64_t n = N > 0 ? N : 1;
-  int bm, bn;
-  if (ceil_div(M_hi, 256) * ceil_div(n, 256) >= 150) {
-    return make(DTAS_GEMM_MFMA, 512, 8, 2, 256, 256, 64);
-  } else if (ceil_div(M_hi, 128) * ceil_div(n, 128) >= 256) {
-    bm = bn = 128;
-  } else {
-    bm = bn = 64;
+  const int64_t n = N > 0 ? N : 1, k = K > 0 ? K : 1;
+  if (ceil_div(M_hi, 256) * ceil_div(n, 256) >= 150) return make(DTAS_GEMM_MFMA, 512, 8, 2, 256, 256, 64);
+  if (ceil_div(M_hi, 128) * ceil_div(n, 128) >= 256) {
+    const int64_t tiles = ceil_div(M_hi, 128) * ceil_div(n, 128);
+    int stages = 2;
+    for (int ns = 4; ns > 2; --ns) {
+      const int64_t per_cu = kLdsBytes / (ns * 256 * 128);
+      if (per_cu >= 1 && (per_cu == 1 ? tiles <= kNumCU : tiles * 4 <= kNumCU * per_cu * 3)) {
+        stages = ns;
+        break;
+      }
+    }
+    return make(DTAS_GEMM_MFMA, 256, 8, stages, 128, 128, 64);
   }
-  const int64_t tiles = ceil_div(M_hi, bm) * ceil_div(n, bn);
-  const int64_t stage_bytes = static_cast<int64_t>(bm + bn) * 128;
-  int stages = 2;
-  for (int ns = 4; ns > 2; --ns) {
-    const int64_t per_cu = kLdsBytes / (ns * stage_bytes);
-    if (per_cu >= 1 && (per_cu == 1 ? tiles <= kNumCU : tiles * 4 <= kNumCU * per_cu * 3)) {
-      stages = ns;
-      break;
+  const int64_t ktiles = ceil_div(k, 64);
+  GemmChoice best = {1e30, 64, 1};
+  for (int tile = 64; tile <= 128; tile *= 2) {
+    const double step_us = tile == 64 ? 0.33 : 0.62, partial_us = tile == 64 ? 1.0 : 4.0;
+    const int64_t tiles = ceil_div(M_hi, tile) * ceil_div(n, tile);
+    for (int split = 1; split <= 4; ++split) {
+      if (split > 1 && (ktiles / split < 8 || (tile == 128 && tiles * split > kNumCU))) continue;
+      const double wgs = static_cast<double>(tiles * split);
+      const double crowd = wgs <= kNumCU ? 1.0 : 0.82 * wgs / kNumCU;  // two per CU run at ~0.6 of the speed each
+      const double us = static_cast<double>(ceil_div(ktiles, split)) * step_us * crowd + (split > 1 ? partial_us * split : 0.0);
+      if (us < best.us) best = {us, tile, split};
     }
   }
-  return make(DTAS_GEMM_MFMA, 256, 8, stages, bm, bn, 64);
+  if (M_hi <= 32) {
+    const double skinny_us = static_cast<double>(n) * static_cast<double>(k) * 2.0 / 3.5e6 * (M_hi <= 8 ? 0.9 : M_hi <= 16 ? 0.95 : 1.35);
+    if (skinny_us <= best.us) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
+  }
+  return make(DTAS_GEMM_MFMA, 256, 8, 4, best.tile, best.tile, 64, best.split);
 }
 
 dtas_config policy(int op, int64_t n_hi, int64_t d0, int64_t d1) {

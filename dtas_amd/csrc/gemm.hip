@@ -39,10 +39,13 @@
 #include "dtas_device.h"
 #include "dtas_host.h"
 
+#include <mutex>
+
 namespace dtas {
 namespace {
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
+typedef float f32x2v __attribute__((ext_vector_type(2)));
 
 constexpr int kBK = 64;             // k extent of a tile: 128 bytes of fp16
 constexpr int kRowBytes = kBK * 2;  // one tile row in LDS
@@ -84,7 +87,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
                                                                  const half_t* __restrict__ W,
                                                                  const half_t* __restrict__ bias,
                                                                  half_t* __restrict__ C, int64_t M, int64_t N,
-                                                                 int64_t K, unsigned tiles_m, unsigned tiles_n) {
+                                                                 int64_t K, unsigned tiles_m, unsigned tiles_n,
+                                                                 unsigned nsplit, float* __restrict__ ws,
+                                                                 unsigned* __restrict__ arrivals) {
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wavefront tile
   constexpr int MT = WTM / 32, NT = WTN / 32;  // 32x32 blocks per wavefront
@@ -101,8 +106,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
 
   // ---- which tile: XCD-contiguous order, then groups of 8 tile rows walked column-wise
+  // nsplit > 1: nsplit consecutive workgroups (same XCD) share a tile and split its k tiles
   const unsigned total = tiles_m * tiles_n;
-  const unsigned pid = xcd_contiguous_id(blockIdx.x, total);
+  const unsigned wgid = xcd_contiguous_id(blockIdx.x, total * nsplit);
+  const unsigned pid = wgid / nsplit, z = wgid % nsplit;
   constexpr unsigned kGroup = 8;
   const unsigned width = kGroup * tiles_n;
   const unsigned first_m = (pid / width) * kGroup;
@@ -136,13 +143,17 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int ktiles = static_cast<int>((K + kBK - 1) / kBK);
+  // this workgroup's k tiles: kt0 .. kt0 + ktiles - 1 of the matrix (none, if the split runs out)
+  const int ktiles_all = static_cast<int>((K + kBK - 1) / kBK);
+  const int kt_per = (ktiles_all + static_cast<int>(nsplit) - 1) / static_cast<int>(nsplit);
+  const int kt0 = static_cast<int>(z) * kt_per;
+  const int ktiles = ktiles_all - kt0 < kt_per ? (ktiles_all - kt0 > 0 ? ktiles_all - kt0 : 0) : kt_per;
 
   // tile kt -> LDS stage kt % NS, asynchronously (completion is counted by vmcnt)
   auto fetch = [&](int kt) {
     // a chunk past K is pointed out of range; K % 8 == 0, so chunks are all-in or all-out
-    const unsigned off = (static_cast<int64_t>(kt) * kBK + c_in * 8 < K)
-                             ? g_off + static_cast<unsigned>(kt) * kRowBytes : kOob;
+    const unsigned off = (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K)
+                             ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
     char* base = lds + (kt % NS) * kStage + wv * 1024;
 #pragma unroll
     for (int i = 0; i < LA; ++i)
@@ -185,8 +196,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD)
     // half of tile kt's block loads (every second one)
     auto fetch_half = [&](int kt, int part) {
-      const unsigned off = (static_cast<int64_t>(kt) * kBK + c_in * 8 < K)
-                               ? g_off + static_cast<unsigned>(kt) * kRowBytes : kOob;
+      const unsigned off = (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K)
+                               ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
       char* base = lds + (kt & 1) * kStage + wv * 1024;
 #pragma unroll
       for (int i = 0; i < LA + LB; ++i) {
@@ -283,6 +294,64 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // j*32 + 8*(v/4) + 4*(l >> 5) + v%4 of the wavefront tile.  Each wavefront stages its tile in a
   // private LDS region of WTM rows x WTN fp16 (8-byte slots, xor-swizzled by the row) and writes
   // it out as 8-byte accesses that are contiguous along the row.
+  // ---- split K: every workgroup of a tile parks its fp32 partial tile in the workspace (in
+  // accumulator layout: 8 bytes per lane and register pair, lane-contiguous); the one that arrives
+  // last adds the nsplit partials in split order, so the sum does not depend on who was last, and
+  // goes on to the epilogue.  Nobody waits for anybody.
+  // The XCDs' L2 caches are not coherent with each other.  Partials and the arrival counter are
+  // therefore moved with device-scope accesses (they pass the L2), ordered by the barriers' waits,
+  // rather than with device-scope fences, which write back and invalidate a whole L2 on every use
+  // (measured: that made a two-way split slower than no split).
+  if (nsplit > 1) {
+    // (the flag lives in the operand stages, free by now: a second LDS object would make the
+    // compiler order every fragment read behind the outstanding direct-to-LDS loads)
+    volatile unsigned* is_last = reinterpret_cast<volatile unsigned*>(lds);
+    constexpr int kTilePairs = BM * BN / 2;  // 8-byte units per partial tile
+    unsigned long long* tile_ws = reinterpret_cast<unsigned long long*>(ws) + static_cast<size_t>(pid) * nsplit * kTilePairs;
+    unsigned long long* mine = tile_ws + static_cast<size_t>(z) * kTilePairs + wv * (MT * NT * 8 * 64);
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+          const f32x2v pr = {acc[i][j][2 * h], acc[i][j][2 * h + 1]};
+          __hip_atomic_store(mine + ((i * NT + j) * 8 + h) * 64 + l, __builtin_bit_cast(unsigned long long, pr),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    __syncthreads();  // every store of this workgroup has completed; nobody reads the stages any more
+    if (t == 0) {
+      const unsigned before = __hip_atomic_fetch_add(arrivals + pid, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *is_last = before == nsplit - 1 ? 1u : 0u;
+      if (before == nsplit - 1)  // re-armed for the next launch
+        __hip_atomic_store(arrivals + pid, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const bool last = *is_last != 0;
+    if (!last) return;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    for (unsigned k = 0; k < nsplit; ++k) {
+      const unsigned long long* part = tile_ws + static_cast<size_t>(k) * kTilePairs + wv * (MT * NT * 8 * 64);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int h = 0; h < 8; ++h) {
+            const unsigned long long raw =
+                __hip_atomic_load(part + ((i * NT + j) * 8 + h) * 64 + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const f32x2v pr = __builtin_bit_cast(f32x2v, raw);
+            acc[i][j][2 * h] += pr[0];
+            acc[i][j][2 * h + 1] += pr[1];
+          }
+    }
+  }
+
   constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots;
   char* region = lds + wv * (WTM * kRowB);
   __syncthreads();  // every wavefront is done with the operand stages
@@ -336,10 +405,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 // operands, loaded straight from global memory.  Result register v of lane l is row
 // 4*(l >> 4) + v, column l & 15 of the 16x16 block.
 template <int MT>
-__global__ void __launch_bounds__(512) gemm_skinny_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
+__global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
                                                           const half_t* __restrict__ bias, half_t* __restrict__ C,
                                                           int64_t M, int64_t N, int64_t K) {
-  __shared__ f32x4v part[8][MT][64];
+  __shared__ f32x4v part[16][MT][64];
   const unsigned t = threadIdx.x, l = t & 63u, wv = t >> 6, nwaves = blockDim.x >> 6;
   const int64_t n0 = static_cast<int64_t>(blockIdx.x) * 16;
   const int64_t wrow = n0 + (l & 15u) < N ? n0 + (l & 15u) : N - 1;  // clamped rows are never stored
@@ -356,22 +425,24 @@ __global__ void __launch_bounds__(512) gemm_skinny_kernel(const half_t* __restri
 
   const int64_t steps = K >> 5;  // whole 32-element steps; K % 32 is handled below
   // A wavefront takes pairs of consecutive steps (2p, 2p+1) for p = wv, wv + nwaves, ...: the two
-  // 64-byte pieces a lane row contributes per pair are the halves of one 128-byte line.  Two pairs
-  // at a time, so that 4 * (1 + MT) independent 1 KiB loads are in flight before the first MFMA.
+  // 64-byte pieces a lane row contributes per pair are the halves of one 128-byte line.  G pairs
+  // at a time, so that 2 * G * (1 + MT) independent 1 KiB loads are in flight before the first
+  // MFMA: the loop is a chain of memory round trips, and K = 4096 over 16 wavefronts is one of them.
+  constexpr int G = MT == 1 ? 4 : 2;
   const int64_t pairs = steps >> 1;
   const int64_t mine = pairs > wv ? (pairs - wv + nwaves - 1) / nwaves : 0;
   int64_t q = 0;
-  for (; q + 2 <= mine; q += 2) {
-    f16x8 fw[4], fa[4][MT];
+  for (; q + G <= mine; q += G) {
+    f16x8 fw[2 * G], fa[2 * G][MT];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 2 * G; ++u) {
       const int64_t off = ((wv + (q + (u >> 1)) * nwaves) * 2 + (u & 1)) * 32;
       fw[u] = __builtin_bit_cast(f16x8, load_stream(reinterpret_cast<const u32x4*>(wp + off)));
 #pragma unroll
       for (int i = 0; i < MT; ++i) fa[u][i] = *reinterpret_cast<const f16x8*>(ap[i] + off);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < 2 * G; ++u)
 #pragma unroll
       for (int i = 0; i < MT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[u][i], fw[u], acc[i], 0, 0, 0);
   }
@@ -441,12 +512,69 @@ __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restri
   }
 }
 
+// Split-K workspace of the current device: nsplit fp32 partial tiles per output tile and one
+// arrival counter per tile.  Allocated on first use and grown on demand (the only allocation in
+// the library); the counters are zero between launches (the last arriver of a tile re-arms it).
+// Launches that split K share it, so they must be ordered by one stream.
+constexpr size_t kMaxSplitWsBytes = size_t{1} << 30;
+constexpr int kMaxDevices = 64;
+struct SplitWorkspace {
+  float* partials = nullptr;
+  size_t partial_bytes = 0;
+  unsigned* arrivals = nullptr;
+  size_t tiles = 0;
+};
+SplitWorkspace g_split_ws[kMaxDevices];
+std::mutex g_split_ws_mutex;
+
+int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsigned** arrivals) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("gemm: cannot identify the current device");
+  std::lock_guard<std::mutex> lock(g_split_ws_mutex);
+  SplitWorkspace& w = g_split_ws[dev];
+  if (partial_bytes > w.partial_bytes) {
+    // kernels of earlier launches may still use the old buffer: hipFree waits for the device
+    if (w.partials && hipFree(w.partials) != hipSuccess) return fail("gemm: hipFree of the split-K workspace failed");
+    w.partials = nullptr;
+    w.partial_bytes = 0;
+    const size_t want = partial_bytes < (size_t{32} << 20) ? (size_t{32} << 20) : partial_bytes;
+    if (hipMalloc(reinterpret_cast<void**>(&w.partials), want) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail("gemm: cannot allocate %zu bytes of split-K workspace", want);
+    }
+    w.partial_bytes = want;
+  }
+  if (tiles > w.tiles) {
+    if (w.arrivals && hipFree(w.arrivals) != hipSuccess) return fail("gemm: hipFree of the split-K counters failed");
+    w.arrivals = nullptr;
+    w.tiles = 0;
+    const size_t want = tiles < 4096 ? 4096 : tiles;
+    if (hipMalloc(reinterpret_cast<void**>(&w.arrivals), want * sizeof(unsigned)) != hipSuccess ||
+        hipMemset(w.arrivals, 0, want * sizeof(unsigned)) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail("gemm: cannot allocate the split-K arrival counters");
+    }
+    w.tiles = want;
+  }
+  *partials = w.partials;
+  *arrivals = w.arrivals;
+  return 0;
+}
+
 template <int BM, int BN, int WM, int WN, int NS>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const half_t* bias, half_t* C, int64_t M, int64_t N,
-                int64_t K) {
+                int64_t K, int nsplit) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(tiles_m * tiles_n), dim3(64 * WM * WN), 0, s, A, W, bias,
-                     C, M, N, K, tiles_m, tiles_n);
+  const size_t tiles = static_cast<size_t>(tiles_m) * tiles_n;
+  float* partials = nullptr;
+  unsigned* arrivals = nullptr;
+  if (nsplit > 1) {
+    const size_t bytes = tiles * nsplit * BM * BN * sizeof(float);
+    if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
+    if (split_workspace(bytes, tiles, &partials, &arrivals) != 0) return -1;
+  }
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(static_cast<unsigned>(tiles * nsplit)), dim3(64 * WM * WN), 0,
+                     s, A, W, bias, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
 
@@ -482,7 +610,10 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     // cfg.unroll = LDS stages (the depth of the load pipeline); 0 or 1 = as many as fit
     if (cfg.unroll < 0 || cfg.unroll > mfma_max_stages(bm, bn))
       return fail("gemm: the %dx%d tile holds at most %d LDS stages, got %d", bm, bn, mfma_max_stages(bm, bn), cfg.unroll);
-    la[0] = tm * tn;
+    const int nsplit = cfg.split_k < 1 ? 1 : cfg.split_k;
+    if (nsplit > 16) return fail("gemm: split_k must be in [1, 16], got %d", cfg.split_k);
+    if (tm * tn * nsplit > 0x7fffffff) return fail("gemm: too many workgroups");
+    la[0] = tm * tn * nsplit;
     la[3] = mfma_threads(bm, bn);
     la[4] = (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
     la[5] = tm;
@@ -494,11 +625,11 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     if (cfg.tile[0] % 16 != 0 || mt < 1 || mt > 5 || cfg.tile[1] != 16)
       return fail("gemm: skinny tile must be {16,32,48,64,80}x16, got %dx%d", cfg.tile[0], cfg.tile[1]);
     if (M > cfg.tile[0]) return fail("gemm: skinny tile of %d rows cannot hold M=%lld", cfg.tile[0], (long long)M);
-    if (cfg.block < 64 || cfg.block > 512 || cfg.block % 64 != 0)
-      return fail("gemm: block must be a multiple of 64 in [64, 512], got %d", cfg.block);
+    if (cfg.block < 64 || cfg.block > 1024 || cfg.block % 64 != 0)
+      return fail("gemm: block must be a multiple of 64 in [64, 1024], got %d", cfg.block);
     la[0] = ceil_div(N, 16);
     la[3] = cfg.block;
-    la[4] = 8 * mt * 64 * 16;
+    la[4] = 16 * mt * 64 * 16;
     la[5] = 1;
     la[6] = la[0];
     return 0;
@@ -546,22 +677,23 @@ extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, voi
   }
   const int bm = cfg.tile[0], bn = cfg.tile[1];
   const int ns = cfg.unroll >= 2 ? cfg.unroll : 0;
-  if (bm == 256 && bn == 256) return launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K);
-  if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K)
-                                             : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 256) return ns == 2 ? launch_mfma<128, 256, 2, 2, 2>(s, a, w, b, c, M, N, K)
-                                             : launch_mfma<128, 256, 2, 2, 3>(s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 128) return ns == 2   ? launch_mfma<128, 128, 2, 2, 2>(s, a, w, b, c, M, N, K)
-                                     : ns == 3 ? launch_mfma<128, 128, 2, 2, 3>(s, a, w, b, c, M, N, K)
-                                               : launch_mfma<128, 128, 2, 2, 4>(s, a, w, b, c, M, N, K);
-  if (bm == 64 && bn == 128) return ns == 2   ? launch_mfma<64, 128, 2, 2, 2>(s, a, w, b, c, M, N, K)
-                                    : ns == 3 ? launch_mfma<64, 128, 2, 2, 3>(s, a, w, b, c, M, N, K)
-                                              : launch_mfma<64, 128, 2, 2, 4>(s, a, w, b, c, M, N, K);
-  if (bm == 128 && bn == 64) return ns == 2   ? launch_mfma<128, 64, 2, 2, 2>(s, a, w, b, c, M, N, K)
-                                    : ns == 3 ? launch_mfma<128, 64, 2, 2, 3>(s, a, w, b, c, M, N, K)
-                                              : launch_mfma<128, 64, 2, 2, 4>(s, a, w, b, c, M, N, K);
-  if (bm == 64 && bn == 64) return ns == 2   ? launch_mfma<64, 64, 2, 2, 2>(s, a, w, b, c, M, N, K)
-                                   : ns == 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, b, c, M, N, K)
-                                             : launch_mfma<64, 64, 2, 2, 4>(s, a, w, b, c, M, N, K);
+  const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
+  if (bm == 256 && bn == 256) return launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                             : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 128 && bn == 256) return ns == 2 ? launch_mfma<128, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                             : launch_mfma<128, 256, 2, 2, 3>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 128 && bn == 128) return ns == 2   ? launch_mfma<128, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                     : ns == 3 ? launch_mfma<128, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
+                                               : launch_mfma<128, 128, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 64 && bn == 128) return ns == 2   ? launch_mfma<64, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                    : ns == 3 ? launch_mfma<64, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
+                                              : launch_mfma<64, 128, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 128 && bn == 64) return ns == 2   ? launch_mfma<128, 64, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                    : ns == 3 ? launch_mfma<128, 64, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
+                                              : launch_mfma<128, 64, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 64 && bn == 64) return ns == 2   ? launch_mfma<64, 64, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                   : ns == 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
+                                             : launch_mfma<64, 64, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
   return fail("gemm: no MFMA kernel for tile %dx%d", bm, bn);
 }

@@ -157,3 +157,63 @@ def test_gemm_k_not_multiple_of_8_and_errors(oracle):
     out = Guarded((9, 20), torch.float16)   # an explicit MFMA config steps down to element accesses
     ops.gemm(dev(a), dev(w), None, out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[64, 64, 64]))
     _check(out.check(), oracle.c.gemm(a, w), oracle.np64.gemm(a, w))
+
+
+SPLIT_TILES = [(256, 256), (128, 128), (128, 64), (64, 64)]
+
+
+@pytest.mark.parametrize("bm,bn", SPLIT_TILES)
+@pytest.mark.parametrize("split", [2, 3, 4, 7])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 8), (70, 130, 136), (300, 260, 1096), (64, 512, 4096)])
+def test_gemm_split_k_on_ragged_shapes(oracle, bm, bn, split, M, N, K):
+    # K = 8 and 136 leave some of the K partitions without a single k tile; 1096 splits unevenly
+    a, w = _inputs(M, N, K, M + N + K + split)
+    bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
+    out = Guarded((M, N), torch.float16)
+    c = cfg(variant=_lib.GEMM_MFMA, block=_threads(bm, bn), vec=8, tile=[bm, bn, 64], split_k=split)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c)
+    _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+    info = _lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c)
+    assert info.launch_args[0] == -(-M // bm) * -(-N // bn) * split
+
+
+def test_gemm_split_k_is_reproducible_and_rearms_its_counters(oracle):
+    # the partial tiles are summed in partition order whichever workgroup arrives last, so repeated
+    # launches give identical bits; launches of other shapes in between share the same counters
+    shapes = [(64, 4096, 4096, 4, (64, 64)), (200, 1000, 2048, 3, (128, 128)), (512, 512, 8192, 2, (256, 256))]
+    first = {}
+    for rep in range(3):
+        for (M, N, K, split, (bm, bn)) in shapes:
+            a, w = _inputs(M, N, K, M + K)
+            out = Guarded((M, N), torch.float16)
+            ops.gemm(dev(a), dev(w), None, out.t, cfg(variant=_lib.GEMM_MFMA, block=_threads(bm, bn), vec=8, tile=[bm, bn, 64], split_k=split))
+            got = out.check()
+            if rep == 0:
+                first[(M, N, K)] = got
+                _check(got, oracle.c.gemm(a, w, threads=8), oracle.np64.gemm(a, w))
+            else:
+                assert_bits_equal(got, first[(M, N, K)])
+
+
+def test_gemm_split_k_many_launches_back_to_back():
+    # no synchronisation between launches: each reads the counters the previous one re-armed
+    M, N, K = 96, 2048, 4096
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.randn(M, K, device="cuda", generator=g).half()
+    w = (torch.randn(N, K, device="cuda", generator=g) * 0.02).half()
+    c = cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[64, 64, 64], split_k=4)
+    outs = [torch.empty(M, N, dtype=torch.float16, device="cuda") for _ in range(50)]
+    for o in outs:
+        ops.gemm(a, w, None, o, c)
+    torch.cuda.synchronize()
+    ref = a.float() @ w.float().T
+    for o in outs:
+        assert torch.equal(o, outs[0])
+    assert float((outs[0].float() - ref).abs().max()) < 2e-2
+
+
+def test_gemm_split_k_errors():
+    a, w = _inputs(64, 64, 64, 1)
+    with pytest.raises(_lib.DtasError, match="split_k"):
+        ops.gemm(dev(a), dev(w), None, torch.empty(64, 64, dtype=torch.float16, device="cuda"),
+                 cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[64, 64, 64], split_k=17))
