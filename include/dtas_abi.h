@@ -18,8 +18,13 @@
  *    (experiment/dtas_tuned/elementwise/cast/profile_cast.py:15-18);
  *  - buffers are compact row-major, as the reference requires (strides == NULL,
  *    host.cc:64-69); the leading batch-1 dim of (1, n, H) is not passed;
- *  - `stream` is a hipStream_t (NULL = the default stream); nothing is allocated, nothing
- *    synchronises, the kernel is enqueued on `stream` on the current device;
+ *  - `stream` is a hipStream_t (NULL = the default stream); nothing synchronises, the kernel is
+ *    enqueued on `stream` on the current device.  Nothing is allocated, with one exception:
+ *    dtas_gemm_f16 with K split over workgroups (split_k > 1, which the built-in table chooses
+ *    when M x N yields few tiles) keeps fp32 partial tiles in a per-device workspace that the
+ *    library allocates on first use and grows on demand (32 MiB at first, at most 1 GiB; growing
+ *    waits for the device).  Launches that use it share it: enqueue them on one stream, or pass
+ *    a cfg with split_k = 1 on the others;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
  *    reference's call_table holds); NULL = use the library's built-in bucket table; either way a
  *    128-bit variant steps down to its element-access kernel for extents or pointers that do not
@@ -91,9 +96,10 @@ typedef struct dtas_config {
   int32_t variant;  /* enum dtas_variant of the op's family */
   int32_t block;    /* threads per workgroup = launch_args[1] */
   int32_t vec;      /* elements per vector access */
-  int32_t unroll;   /* independent vector accesses in flight per thread; GEMM: LDS stages (0 = max) */
+  int32_t unroll;   /* elementwise/GEMV: independent vector accesses in flight per thread; row
+                       reductions: rows a lane group takes per trip (1, 2, 4); GEMM: LDS stages (0 = max) */
   int32_t tile[3];  /* GEMM: workgroup tile M, N, K; GEMV: rows per workgroup, -, - */
-  int32_t split_k;  /* GEMV/GEMM: number of K partitions (1 = none) */
+  int32_t split_k;  /* GEMM (MFMA): workgroups that share a tile and split its K extent, 1..16 (1 = none) */
   int64_t grid_cap; /* upper limit on workgroups (then the kernel loops); 0 = no limit */
 } dtas_config;
 
