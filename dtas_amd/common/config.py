@@ -154,11 +154,13 @@ class ReductionConfig(Config):
         # "cache" = re-read from L2 per pass (the reference's softmax artefacts)
         self.temp_storage = "shared.dyn"
         self.max_active_blocks_per_sm = 0
+        # rows a wavefront / workgroup takes per trip (1, 2, 4): they share barriers and parameter loads
+        self.rows_per_trip = 1
 
     def to_dict(self) -> Dict:
         return {"bx": self.bx, "len_tx": self.len_tx, "unroll_depth": self.unroll_depth,
                 "vector_size": self.vector_size, "temp_storage": self.temp_storage,
-                "max_active_blocks_per_sm": self.max_active_blocks_per_sm}
+                "max_active_blocks_per_sm": self.max_active_blocks_per_sm, "rows_per_trip": self.rows_per_trip}
 
     def from_dict(self, dic: Dict) -> "ReductionConfig":
         self.__init__()
@@ -168,6 +170,7 @@ class ReductionConfig(Config):
         self.temp_storage = dic["temp_storage"]
         self.bx = dic.get("bx")
         self.max_active_blocks_per_sm = dic.get("max_active_blocks_per_sm", 0)
+        self.rows_per_trip = dic.get("rows_per_trip", 1)
         return self
 
     def to_abi(self):
@@ -176,7 +179,7 @@ class ReductionConfig(Config):
                      "cache": _lib.RED_STREAM_ROW}[self.temp_storage]
         c.block = self.len_tx
         c.vec = 1 if self.temp_storage == "cache" else (self.vector_size or 1)
-        c.unroll, c.split_k = 1, 1
+        c.unroll, c.split_k = (1 if self.temp_storage == "cache" else self.rows_per_trip), 1
         c.grid_cap = self.bx or 0
         return c
 
@@ -231,6 +234,7 @@ class MFMAConfig(Config):
         self.skinny = False      # small M: weight-streaming 16x16x32 kernel, K split over wavefronts
         self.block_threads = 256
         self.stages = 0          # LDS stages of the load pipeline (0 = as many as the tile allows)
+        self.split_k = 1         # workgroups that share a tile and split its K extent
         self.in_vec_len_a = 8
         self.in_vec_len_b = 8
         self.swizzle = True
@@ -254,7 +258,7 @@ class MFMAConfig(Config):
                 "mfma_shape": (self.mfma_m, self.mfma_n, self.mfma_k), "i": self.i, "j": self.j,
                 "micro_shape": (self.micro_shape_x, self.micro_shape_y, self.micro_shape_k),
                 "skinny": self.skinny, "block_threads": self.block_threads, "stages": self.stages,
-                "in_vec_len_a": self.in_vec_len_a, "in_vec_len_b": self.in_vec_len_b}
+                "split_k": self.split_k, "in_vec_len_a": self.in_vec_len_a, "in_vec_len_b": self.in_vec_len_b}
 
     def from_dict(self, dic: Dict) -> "MFMAConfig":
         self.__init__()
@@ -264,6 +268,7 @@ class MFMAConfig(Config):
         self.skinny = dic.get("skinny", False)
         self.block_threads = dic.get("block_threads", 256)
         self.stages = dic.get("stages", 0)
+        self.split_k = dic.get("split_k", 1)
         return self
 
     def to_abi(self):
@@ -272,7 +277,7 @@ class MFMAConfig(Config):
         c.block, c.vec = self.block_threads, 8
         c.unroll = 4 if self.skinny else self.stages
         c.tile[0], c.tile[1], c.tile[2] = self.tile_size_m, self.tile_size_n, self.tile_size_k
-        c.split_k = 1
+        c.split_k = 1 if self.skinny else self.split_k
         return c
 
 

@@ -5,8 +5,9 @@ enumerate block tiles as i x j wavefronts of micro_x x micro_y matrix-core block
 those that do not fit shared memory / registers (:46-70) and rank by a roofline estimate in which a
 tile's throughput is min(matrix-core peak, bandwidth * flops-per-byte of the tile) and the job costs
 ceil(tiles / SMs) rounds (:148-262).  The candidate set is what libdtas_gfx950.so has kernels for:
-32x32x16 MFMA tiles from 64x64 to 256x256 with 2 to 4 LDS stages, plus, for M <= 64, the
-weight-streaming 16x16x32 kernel whose wavefronts split K.  The order is the one on-GPU sweeps favoured;
+32x32x16 MFMA tiles from 64x64 to 256x256 with 2 to 4 LDS stages, with K split over up to 4 workgroups
+per tile when M x N yields few tiles, plus, for M <= 64, the weight-streaming 16x16x32 kernel whose
+wavefronts split K.  The order is the one on-GPU sweeps favoured;
 with a GPU present the Engine times the top-k anyway.
 """
 from typing import List, Tuple
@@ -30,20 +31,45 @@ class MFMAConfigEmiter(BaseConfigEmiter):
     def max_stages(tile_m: int, tile_n: int) -> int:
         return 2 if tile_m + tile_n >= 512 else 3 if tile_m + tile_n >= 384 else 4
 
-    def preferred(self, m_hi: int, N: int):
-        """(tile_m, tile_n, stages) that sweeps on an MI355X favoured: 256x256 once it yields >= 150
-        workgroups, else 128x128 from 256 workgroups, else 64x64; the deepest load pipeline with which all
-        tiles stay co-resident (a margin when several workgroups share a CU), else 2 stages."""
+    def preferred(self, m_hi: int, N: int, K: int = 4096):
+        """(tile_m, tile_n, stages, split_k) that sweeps on an MI355X favoured: 256x256 once it yields
+        >= 150 workgroups, else 128x128 from 256 workgroups (the deepest load pipeline with which all tiles
+        stay co-resident).  With fewer tiles a workgroup's k loop is a serial chain of ~0.33 us (64x64) or
+        ~0.62 us (128x128) steps, so K is split over workgroups when the saved steps outweigh the ~1 us
+        (~4 us) each partial tile costs; more than one workgroup per CU run at ~0.6 of the speed each."""
         cdiv = lambda a, b: -(-a // b)
+        self._model_us = float("inf")
         if cdiv(m_hi, 256) * cdiv(N, 256) >= 150:
-            return 256, 256, 2
-        t = 128 if cdiv(m_hi, 128) * cdiv(N, 128) >= 256 else 64
-        tiles = cdiv(m_hi, t) * cdiv(N, t)
-        for ns in (4, 3):
-            per_cu = _LDS // (ns * 2 * t * 128)
-            if per_cu >= 1 and (tiles <= self.arch.num_sm if per_cu == 1 else tiles * 4 <= self.arch.num_sm * per_cu * 3):
-                return t, t, ns
-        return t, t, 2
+            return 256, 256, 2, 1
+        if cdiv(m_hi, 128) * cdiv(N, 128) >= 256:
+            tiles = cdiv(m_hi, 128) * cdiv(N, 128)
+            for ns in (4, 3):
+                per_cu = _LDS // (ns * 2 * 128 * 128)
+                if per_cu >= 1 and (tiles <= self.arch.num_sm if per_cu == 1 else tiles * 4 <= self.arch.num_sm * per_cu * 3):
+                    return 128, 128, ns, 1
+            return 128, 128, 2, 1
+        ktiles = cdiv(K, 64)
+        best = (float("inf"), 64, 1)
+        for t, step_us, partial_us in ((64, 0.33, 1.0), (128, 0.62, 4.0)):
+            tiles = cdiv(m_hi, t) * cdiv(N, t)
+            for split in (1, 2, 3, 4):
+                if split > 1 and (ktiles // split < 8 or (t == 128 and tiles * split > self.arch.num_sm)):
+                    continue
+                wgs = tiles * split
+                crowd = 1.0 if wgs <= self.arch.num_sm else 0.82 * wgs / self.arch.num_sm
+                us = cdiv(ktiles, split) * step_us * crowd + (partial_us * split if split > 1 else 0.0)
+                if us < best[0]:
+                    best = (us, t, split)
+        self._model_us = best[0]
+        return best[1], best[1], 4, best[2]
+
+    def prefers_skinny(self, m_hi: int, N: int, K: int) -> bool:
+        """M <= 32: the W-streaming kernel (about 3.5 TB/s of W, slower as M grows) against the model's
+        best MFMA candidate; call after preferred()."""
+        if m_hi > 32:
+            return False
+        us = N * K * 2.0 / 3.5e6 * (0.9 if m_hi <= 8 else 0.95 if m_hi <= 16 else 1.35)
+        return us <= self._model_us
 
     def emit_config(self, range_tuple: Tuple[Range, ...], topk: int = 20) -> List[MFMAConfig]:
         params = self.func_info.func.params
@@ -62,7 +88,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.micro_shape_k = 1, 1, -(-m_hi // 16), 1, 1
                 c.mfma_m, c.mfma_n, c.mfma_k = 16, 16, 32
                 out.append(c)
-        pref = self.preferred(m_hi, N)
+        pref = self.preferred(m_hi, N, K)
         scored = []
         for mx, my in _TILES:
             base = MFMAConfig()
@@ -78,10 +104,15 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                     continue
                 tiles = -(-m_hi // tm) * -(-N // tn)
                 c.num_wave = -(-tiles // self.arch.num_sm)
-                # rank: the measured preference first, then by distance in tile area and stage count
-                rank = (0 if (tm, tn, stages) == pref else 1, abs(tm * tn - pref[0] * pref[1]), abs(stages - pref[2]))
-                scored.append((rank, c))
+                splits = [1] + [sk for sk in (2, 3, 4) if tiles * sk <= 2 * self.arch.num_sm and -(-K // 64) // sk >= 8]
+                for sk in splits:
+                    cs = MFMAConfig().from_dict(c.to_dict())
+                    cs.split_k, cs.num_wave = sk, -(-tiles * sk // self.arch.num_sm)
+                    # rank: the measured preference first, then by distance in tile area, split and stage count
+                    rank = (0 if (tm, tn, stages, sk) == pref else 1, abs(tm * tn - pref[0] * pref[1]),
+                            abs(sk - pref[3]), abs(stages - pref[2]))
+                    scored.append((rank, cs))
         mfma = [c for _, c in sorted(scored, key=lambda t: t[0])]
-        # M <= 32 streams W (skinny first); above that the MFMA tiles lead
-        out = (out + mfma) if m_hi <= 32 else (mfma[:1] + out + mfma[1:])
+        # the W-streaming kernel leads only where it beats the best MFMA candidate under the model
+        out = (out + mfma) if self.prefers_skinny(m_hi, N, K) else (mfma[:1] + out + mfma[1:])
         return out[:topk]

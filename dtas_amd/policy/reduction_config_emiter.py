@@ -74,37 +74,51 @@ class ReductionConfigEmiter(BaseConfigEmiter):
         return configs
 
     def _gfx950_candidates(self, re_range: Range, row_range: Range, in_bytes: int, topk: int) -> List[ReductionConfig]:
+        """Candidates for libdtas_gfx950.so's row kernels, the library's own built-in choice first:
+        a workgroup per row with about two 128-bit vectors per thread (sized in multiples of 64 threads
+        so that no lane idles), several rows per trip once there are >= 8 rows per CU; for dynamic rows
+        (softmax: 32 rows per unit of row length) a wavefront per row below 512 vectors."""
         vec = 16 // in_bytes
         nvec = -(-re_range.end // vec)
-        # a wavefront per row pays off from ~8 rows per CU and up to 8 vectors per lane (static rows);
-        # dynamic rows (softmax) have 32 rows per unit of row length, so many rows as soon as n > 16
-        many_rows = row_range.start >= 8 * self.arch.num_sm and (nvec <= 64 * 8 or self.func_info.dyn_red)
-        if self.func_info.dyn_red:
-            many_rows = row_range.end > 2 * self.arch.num_sm
+        rows = row_range.end
+        many_rows = rows >= 8 * self.arch.num_sm
         out: List[ReductionConfig] = []
 
-        def cand(storage: str, tx: int) -> ReductionConfig:
+        def cand(storage: str, tx: int, rpt: int = 1) -> Optional[ReductionConfig]:
+            width = 64 if storage == "local" else tx
+            iters = -(-nvec // width)
+            if storage != "cache" and (iters > 16 or iters * rpt > 16 or (rpt == 2 and iters > 8) or (rpt == 4 and iters > 4)
+                                       or (iters * rpt > 8 and tx > 512)):
+                return None
             c = ReductionConfig()
-            c.temp_storage, c.len_tx, c.vector_size, c.unroll_depth = storage, tx, vec, 1
+            c.temp_storage, c.len_tx, c.vector_size, c.unroll_depth, c.rows_per_trip = storage, tx, vec, 1, rpt
             self.get_num_blocks(c, row_range, 64, storage == "shared.dyn", 32)
             c.bx = None  # rows map 1:1 to wavefronts / workgroups; the kernels stride if capped
             return c
 
-        wave_order = (64, 128, 256, 512) if nvec <= 64 else (256, 128, 512, 64)
-        wave_rows = [cand("local", tx) for tx in wave_order] if nvec <= 64 * 16 else []
-        pref = 64
-        while pref * 2 <= max(64, nvec // 2) and pref < 1024:
-            pref *= 2
+        def round64(v: int) -> int:
+            return min(1024, max(64, -(-v // 64) * 64))
+
+        pref = round64(-(-nvec // 2))                       # ~2 vectors per thread
+        narrow = round64(-(-nvec // 5))                     # ~5 vectors per thread
+        two_params = self.func_info.in_dtype == "float32" and not self.func_info.dyn_red   # layer norm: gamma and beta
+        multi = (2 if two_params else 4) if many_rows else 1
+        block_sizes = [pref, narrow] + [t for t in (64, 128, 256, 320, 512, 1024) if t not in (pref, narrow)]
+        if two_params and many_rows and rows <= 16 * self.arch.num_sm:
+            block_sizes = [narrow, pref] + block_sizes[2:]
         block_rows = []
-        for tx in sorted((64, 128, 256, 512, 1024), key=lambda t: (t != pref, abs(t - pref))):
-            if tx * 16 >= nvec and tx <= max(64, nvec):
-                block_rows.append(cand("shared.dyn", tx))
-        # few rows: a workgroup per row first; many rows: a wavefront per row first
-        out = (wave_rows + block_rows) if many_rows else (block_rows + wave_rows)
+        for tx in block_sizes:
+            for rpt in dict.fromkeys((multi, 1, 2, 4)):
+                if tx <= max(64, round64(nvec)):
+                    block_rows.append(cand("shared.dyn", tx, rpt))
+        wave_order = (64, 128, 256, 512) if nvec <= 64 else (256, 128, 512, 64)
+        wave_rows = [cand("local", tx, rpt) for rpt in (1, 2) for tx in wave_order]
+        wave_first = self.func_info.dyn_red and nvec < 64 * 8 and rows > 2 * self.arch.num_sm
+        ordered = (wave_rows + block_rows) if wave_first else (block_rows[:2] + wave_rows[:2] + block_rows[2:] + wave_rows[2:])
+        out = [c for c in ordered if c is not None]
         stream = cand("cache", 1024 if re_range.end >= 4096 else 256)
         stream.vector_size = 1
-        out.append(stream)
-        return out[:topk]
+        return out[:max(1, topk - 1)] + [stream]
 
     def emit_config(self, range_tuple: Tuple[Range, ...], topk: int = 20) -> List[ReductionConfig]:
         re_len = self.func_info.red_len

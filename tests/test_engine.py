@@ -124,3 +124,31 @@ def test_cpu_tensors_are_refused_not_computed_elsewhere():
     a = torch.zeros(4, 64, dtype=torch.float16)
     with pytest.raises(ValueError, match="no CPU path"):
         ops.add(a, a, a.clone())
+
+
+def _first_candidate(func, ranges):
+    from dtas_amd.schedule.schedule import get_config_emiter_template  # the rule -> emitter mapping the Engine uses
+    info = FuncInfo(func)
+    return get_config_emiter_template(info.kind)(info, MI355X()).emit_config(ranges, 20)[0].to_abi().to_dict()
+
+
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (2560, 10240)])
+def test_gemm_emitter_leads_with_the_librarys_builtin_choice(N, K):
+    # the closed-form policy exists twice (C tables for cfg == NULL, Python emitter for the tuner's
+    # first candidate): they must not drift apart
+    func = pf.fused_NT_matmul_add_gemm(N, K, bias=True)
+    for m_hi in (16, 32, 48, 64, 128, 256, 512, 1024, 2048, 4096, 8192):
+        want = _lib.select_bucket(_lib.OP_GEMM_F16, m_hi, N, K).config.to_dict()
+        got = _first_candidate(func, (Range("n", m_hi - 15, m_hi),))
+        keys = ("variant", "tile", "split_k") if want["variant"] == _lib.GEMM_SKINNY else ("variant", "block", "tile", "unroll", "split_k")
+        assert {k: got[k] for k in keys} == {k: want[k] for k in keys}, (m_hi, got, want)
+
+
+def test_reduction_emitters_lead_with_the_librarys_builtin_choice():
+    cases = [(pf.rms_norm(4096), _lib.OP_RMS_NORM_F16, 4096), (pf.fused_layer_norm_cast1(2560), _lib.OP_LAYER_NORM_F32_F16, 2560)]
+    for func, op, H in cases:
+        for n_hi in (16, 256, 1024, 2048, 4096, 8192):
+            want = _lib.select_bucket(op, n_hi, H, 0).config.to_dict()
+            got = _first_candidate(func, (Range("n", n_hi - 15, n_hi),))
+            for k in ("variant", "block", "vec", "unroll"):
+                assert got[k] == want[k], (func.name, n_hi, got, want)
