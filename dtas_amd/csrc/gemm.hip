@@ -80,6 +80,9 @@ __device__ __forceinline__ unsigned xcd_contiguous_id(unsigned wg, unsigned tota
 
 #define DTAS_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// s_waitcnt lgkmcnt(0) vmcnt(v): v is a field of the instruction (bits [3:0] and [15:14])
+constexpr int waitcnt_imm(int v) { return 0x0070 | (v & 15) | ((v >> 4) << 14); }
+
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 template <int BM, int BN, int WM, int WN, int NS>
@@ -99,8 +102,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
   static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
-  static_assert(NS * kStage <= kLdsBytes, "stages exceed the LDS");
-  __shared__ __attribute__((aligned(1024))) char lds[NS * kStage];
+  static_assert(NS * kStage <= kLdsBytes && (NW != 8 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
+  constexpr int kLdsAlloc = NW == 8 ? 5 * BM * kRowBytes : NS * kStage;  // 8 wavefronts: a ring of 5 operand units
+  __shared__ __attribute__((aligned(1024))) char lds[kLdsAlloc];
 
   const unsigned t = threadIdx.x, l = t & 63u;
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
@@ -193,46 +197,66 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   };
 
   if constexpr (NW == 8) {
-    // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD)
-    // half of tile kt's block loads (every second one)
-    auto fetch_half = [&](int kt, int part) {
+    // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD).
+    // The LDS is a ring of five 32 KiB units, filled in the order A(0) W(0) A(1) W(1) ...: unit u
+    // sits in slot u % 5.  While tile kt (two units) is multiplied, up to three more units are in
+    // flight or landed -- W(kt+1) and A(kt+2) are requested during tile kt, A(kt+1) was during tile
+    // kt-1 -- against one tile (two units) with two whole-tile stages: the global->LDS stream is
+    // what bounds this kernel, and it needs ~96 KiB per CU in flight to run at the L2's rate.
+    static_assert(BM == BN, "ring units are one operand's rows of a k tile");
+    constexpr int kUnit = BM * kRowBytes;
+    static_assert(5 * kUnit <= kLdsAlloc, "ring exceeds the LDS");
+    auto wrap5 = [](int v) { return v >= 5 ? v - 5 : v; };
+    auto fetch_unit = [&](const __amdgpu_buffer_rsrc_t& r, int kt, int slot) {
       const unsigned off = (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K)
                                ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
-      char* base = lds + (kt & 1) * kStage + wv * 1024;
+      char* base = lds + slot * kUnit + wv * 1024;
 #pragma unroll
-      for (int i = 0; i < LA + LB; ++i) {
-        if (i % 2 != part) continue;
-        if (i < LA)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
-        else
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + (i - LA) * NW * 1024), 16,
-                                                   off + (i - LA) * g_step, 0, 0, 0);
-      }
+      for (int i = 0; i < LA; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
     };
     const unsigned group = wv >> 2;
-    if (ktiles > 0) fetch(0);
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
+    if (ktiles > 0) {
+      fetch_unit(ra, 0, 0);
+      fetch_unit(rw, 0, 1);
+    }
+    if (ktiles > 1) {
+      fetch_unit(ra, 1, 2);
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA));  // tile 0 has landed, A(1) may be in flight
+    } else {
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+    }
     __builtin_amdgcn_s_barrier();
     DTAS_SCHED_FENCE();
     if (group == 1) {  // one phase behind group 0; group 0 makes up the barrier after the loop
       __builtin_amdgcn_s_barrier();
       DTAS_SCHED_FENCE();
     }
+    int slot_a = 0, slot_w = 1;  // slots of A(kt) and W(kt)
     for (int kt = 0; kt < ktiles; ++kt) {
-      const char* cur = lds + (kt & 1) * kStage;
+      const char* cur_a = lds + slot_a * kUnit + a_frag;
+      const char* cur_w = lds + slot_w * kUnit + b_frag;
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const int set = ks & 1;
-        // memory phase: this step's fragments; in steps 0 and 1 half of tile kt+1's loads each (its
-        // stage held tile kt-1, which every wavefront finished reading two phases ago at the latest)
+        // memory phase: this step's fragments; in step 0 the requests for W(kt+1), in step 1 those
+        // for A(kt+2), into the slots of A(kt-1) and W(kt-1), which every wavefront finished reading
+        // two phases ago at the latest
 #pragma unroll
-        for (int i = 0; i < MT; ++i) read_a(set, i, cur, ks);
+        for (int i = 0; i < MT; ++i) fa[set][i] = *reinterpret_cast<const f16x8*>(cur_a + i * 4096 + lds_rd[ks]);
 #pragma unroll
-        for (int j = 0; j < NT; ++j) read_b(set, j, cur, ks);
-        if (ks < 2 && kt + 1 < ktiles) fetch_half(kt + 1, ks);
+        for (int j = 0; j < NT; ++j) fb[set][j] = *reinterpret_cast<const f16x8*>(cur_w + j * 4096 + lds_rd[ks]);
+        if (ks == 0 && kt + 1 < ktiles) fetch_unit(rw, kt + 1, wrap5(slot_w + 2));
+        if (ks == 1 && kt + 2 < ktiles) fetch_unit(ra, kt + 2, wrap5(slot_a + 4));
         // fragments in registers before the barrier (after a tile's last step the other group may
-        // overwrite the stage); at the last step also this wavefront's loads of tile kt+1
-        if (ks == 3) __builtin_amdgcn_s_waitcnt(0x0070); else __builtin_amdgcn_s_waitcnt(0xC07F);
+        // overwrite the slots); at the last step also this wavefront's loads of tile kt+1: all
+        // but the newest unit's, A(kt+2), if that was requested
+        if (ks == 3) {
+          if (kt + 2 < ktiles) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0xC07F);
+        }
         DTAS_SCHED_FENCE();
         __builtin_amdgcn_s_barrier();
         DTAS_SCHED_FENCE();
@@ -246,6 +270,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         __builtin_amdgcn_s_barrier();
         DTAS_SCHED_FENCE();
       }
+      slot_a = wrap5(slot_a + 2);
+      slot_w = wrap5(slot_w + 2);
     }
     if (group == 0) {
       __builtin_amdgcn_s_barrier();
@@ -615,7 +641,9 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     if (tm * tn * nsplit > 0x7fffffff) return fail("gemm: too many workgroups");
     la[0] = tm * tn * nsplit;
     la[3] = mfma_threads(bm, bn);
-    la[4] = (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
+    // 256x256: a ring of five 32 KiB operand units; else whole-tile stages
+    la[4] = bm == 256 && bn == 256 ? 5 * 256 * kRowBytes
+                                   : (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
     la[5] = tm;
     la[6] = tn;
     return 0;

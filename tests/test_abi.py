@@ -42,7 +42,7 @@ def test_select_bucket_uses_labelled_ranges():
     assert a.config.variant == _lib.GEMM_SKINNY and list(a.config.tile) == [16, 16, 32]
     big = _lib.select_bucket(_lib.OP_GEMM_F16, 4096, 4096, 4096)
     assert big.config.variant == _lib.GEMM_MFMA and list(big.config.tile) == [256, 256, 64]
-    assert list(big.launch_args)[:4] == [256, 1, 1, 512] and big.launch_args[4] == 2 * 512 * 128  # two LDS stages
+    assert list(big.launch_args)[:4] == [256, 1, 1, 512] and big.launch_args[4] == 5 * 256 * 128  # a ring of five operand units
     assert big.bucket_lo <= 4096 <= big.bucket_hi
     # extents above the upper bound share the last bucket
     assert _lib.select_bucket(_lib.OP_GEMM_F16, 100000, 4096, 4096).index == 511
