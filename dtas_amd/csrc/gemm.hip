@@ -102,8 +102,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
   static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
-  static_assert(NS * kStage <= kLdsBytes && (NW != 8 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
-  constexpr int kLdsAlloc = NW == 8 ? 5 * BM * kRowBytes : NS * kStage;  // 8 wavefronts: a ring of 5 operand units
+  static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
+  constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
   __shared__ __attribute__((aligned(1024))) char lds[kLdsAlloc];
 
   const unsigned t = threadIdx.x, l = t & 63u;
@@ -113,12 +113,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // nsplit > 1: nsplit consecutive workgroups (same XCD) share a tile and split its k tiles
   const unsigned total = tiles_m * tiles_n;
   const unsigned wgid = xcd_contiguous_id(blockIdx.x, total * nsplit);
-  const unsigned pid = wgid / nsplit, z = wgid % nsplit;
+  // (divisions run on the vector ALU; pinning the results to scalar registers keeps every address
+  // and buffer descriptor derived from them scalar -- a descriptor left in vector registers turns
+  // each load into a loop over its distinct values)
+  const unsigned pid = __builtin_amdgcn_readfirstlane(wgid / nsplit), z = __builtin_amdgcn_readfirstlane(wgid % nsplit);
   constexpr unsigned kGroup = 8;
   const unsigned width = kGroup * tiles_n;
   const unsigned first_m = (pid / width) * kGroup;
   const unsigned gsize = tiles_m - first_m < kGroup ? tiles_m - first_m : kGroup;
-  const unsigned tm = first_m + (pid % width) % gsize, tn = (pid % width) / gsize;
+  const unsigned tm = __builtin_amdgcn_readfirstlane(first_m + (pid % width) % gsize);
+  const unsigned tn = __builtin_amdgcn_readfirstlane((pid % width) / gsize);
   const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
 
   // ---- global side.  Lane p of a block load fills 16-byte slot p of the block, so it fetches
@@ -277,6 +281,96 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       __builtin_amdgcn_s_barrier();
       DTAS_SCHED_FENCE();
     }
+  } else if constexpr (MT * NT == 16) {
+    // ---- four wavefronts with 128x128 tiles each (256 accumulator registers): every k step reads
+    // 8 KiB of fragments per wavefront for 16 MFMAs, two thirds of the LDS traffic per flop of the
+    // 8-wavefront split -- the LDS port (fragment reads plus the direct-to-LDS writes) is what the
+    // 8-wavefront kernel saturates.  One wavefront per SIMD has nobody to hide behind, so everything
+    // is interleaved with the MFMAs of the running step: the next step's 8 fragment reads before its
+    // first 8 MFMAs, 4 block loads between the last 8 (their per-lane offset is computed once per
+    // k tile, the block's offset rides in the scalar offset operand).  Same ring of five operand units.
+    static_assert(BM == BN && NW == 4, "ring units are one operand's rows of a k tile");
+    constexpr int kUnit = BM * kRowBytes;
+    static_assert(5 * kUnit <= kLdsAlloc && LA % 2 == 0 && 8 % (LA / 2) == 0, "ring exceeds the LDS");
+    constexpr int kHalf = LA / 2;  // block loads per wavefront and half unit
+    auto wrap5 = [](int v) { return v >= 5 ? v - 5 : v; };
+    const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
+    // per-lane byte offset of this lane's chunk in k tile kt of either operand (out of range past K)
+    auto lane_off = [&](int kt) -> unsigned {
+      return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+    };
+    // block load b of a unit (the descriptor is named here, not passed down through the lambdas)
+    auto fetch_one = [&](bool is_w, unsigned voff, int slot, int b) {
+      lds_ptr_t dst = (lds_ptr_t)(lds + slot * kUnit + wv * 1024 + b * NW * 1024);
+      if (is_w) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, dst, 16, voff, b * g_step, 0, 0);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff, b * g_step, 0, 0);
+    };
+    // MFMAs of register set `set`; reads of step `ks_next` of (pa, pw) into the other set; half `dpart`
+    // of a unit's loads.  DMA: 0 = none, 1 = always, 2 = if `cond`.
+    auto step4 = [&](int set, const char* pa, const char* pw, int ks_next, bool reads, int dma, bool cond, bool is_w,
+                     unsigned voff, int dslot, int dpart) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        if (reads && q < 8) {
+          if (q < 4) fa[set ^ 1][q] = *reinterpret_cast<const f16x8*>(pa + q * 4096 + lds_rd[ks_next]);
+          else fb[set ^ 1][q - 4] = *reinterpret_cast<const f16x8*>(pw + (q - 4) * 4096 + lds_rd[ks_next]);
+        }
+        const int i = q / 4, j = q % 4;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+        if (dma != 0 && q >= 8 && (q - 8) % (8 / kHalf) == 0) {
+          if (dma == 1 || cond) fetch_one(is_w, voff, dslot, dpart * kHalf + (q - 8) / (8 / kHalf));
+        }
+        DTAS_SCHED_FENCE();
+      }
+    };
+    if (ktiles > 0) {
+      const unsigned v0 = lane_off(0);
+#pragma unroll
+      for (int b = 0; b < LA; ++b) fetch_one(false, v0, 0, b);
+#pragma unroll
+      for (int b = 0; b < LA; ++b) fetch_one(true, v0, 1, b);
+    }
+    if (ktiles > 1) {
+      const unsigned v1 = lane_off(1);
+#pragma unroll
+      for (int b = 0; b < LA; ++b) fetch_one(false, v1, 2, b);
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA));
+    } else {
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+    }
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    if (ktiles > 0) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa[0][i] = *reinterpret_cast<const f16x8*>(lds + a_frag + i * 4096 + lds_rd[0]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb[0][j] = *reinterpret_cast<const f16x8*>(lds + kUnit + b_frag + j * 4096 + lds_rd[0]);
+    }
+    DTAS_SCHED_FENCE();
+    int slot_a = 0, slot_w = 1;  // slots of A(kt) and W(kt)
+    // one k tile; `steady`: tiles kt+1 and kt+2 exist (no conditions in the instruction stream)
+    auto k_tile = [&](int kt, bool steady) {
+      const char* pa = lds + slot_a * kUnit + a_frag;
+      const char* pw = lds + slot_w * kUnit + b_frag;
+      const int next_a = wrap5(slot_a + 2), next_w = wrap5(slot_w + 2), far_a = wrap5(slot_a + 4);
+      const bool w1 = kt + 1 < ktiles, a2 = kt + 2 < ktiles;
+      const int mode = steady ? 1 : 2;
+      const unsigned vw = lane_off(kt + 1), va = lane_off(kt + 2);
+      // W(kt+1) goes where A(kt-1) was, A(kt+2) where W(kt-1) was: free since the previous barrier
+      step4(0, pa, pw, 1, true, mode, w1, true, vw, next_w, 0);
+      step4(1, pa, pw, 2, true, mode, w1, true, vw, next_w, 1);
+      step4(0, pa, pw, 3, true, mode, a2, false, va, far_a, 0);
+      // tile kt+1 has landed: everything but the half unit of A(kt+2) just requested
+      if (steady || a2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(kHalf)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+      __builtin_amdgcn_s_barrier();  // ... for every wavefront, and all of them are done reading tile kt
+      DTAS_SCHED_FENCE();
+      step4(1, lds + next_a * kUnit + a_frag, lds + next_w * kUnit + b_frag, 0, steady || w1, mode, a2, false, va, far_a, 1);
+      slot_a = next_a;
+      slot_w = next_w;
+    };
+    int kt = 0;
+    for (; kt + 2 < ktiles; ++kt) k_tile(kt, true);
+    for (; kt < ktiles; ++kt) k_tile(kt, false);
   } else {
   // NS stages: tile 0 resident, tiles 1 .. NS-1 in flight, fragments of (tile 0, step 0) in registers
   if (ktiles > 0) fetch(0);
@@ -628,7 +722,9 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
                        (bm == 128 && bn == 128) || (bm == 64 && bn == 128) || (bm == 128 && bn == 64) ||
                        (bm == 64 && bn == 64);
     if (!known || cfg.tile[2] != kBK) return fail("gemm: no MFMA kernel for tile %dx%dx%d", bm, bn, cfg.tile[2]);
-    if (cfg.block != mfma_threads(bm, bn))
+    // 256x256 comes as 8 wavefronts (two per SIMD, alternating phases) or 4 (one per SIMD, 128x128 each)
+    const bool four_waves = bm == 256 && bn == 256 && cfg.block == 256;
+    if (cfg.block != mfma_threads(bm, bn) && !four_waves)
       return fail("gemm: the %dx%d MFMA kernel uses %d threads, got %d", bm, bn, mfma_threads(bm, bn), cfg.block);
     if (K * 2 * (bm > bn ? bm : bn) >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
     const int64_t tm = ceil_div(M, bm), tn = ceil_div(N, bn);
@@ -640,7 +736,7 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     if (nsplit > 16) return fail("gemm: split_k must be in [1, 16], got %d", cfg.split_k);
     if (tm * tn * nsplit > 0x7fffffff) return fail("gemm: too many workgroups");
     la[0] = tm * tn * nsplit;
-    la[3] = mfma_threads(bm, bn);
+    la[3] = four_waves ? 256 : mfma_threads(bm, bn);
     // 256x256: a ring of five 32 KiB operand units; else whole-tile stages
     la[4] = bm == 256 && bn == 256 ? 5 * 256 * kRowBytes
                                    : (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
@@ -706,7 +802,9 @@ extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, voi
   const int bm = cfg.tile[0], bn = cfg.tile[1];
   const int ns = cfg.unroll >= 2 ? cfg.unroll : 0;
   const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
-  if (bm == 256 && bn == 256) return launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 256 && bn == 256)
+    return cfg.block == 256 ? launch_mfma<256, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                            : launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K, sk);
   if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
                                              : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk);
   if (bm == 128 && bn == 256) return ns == 2 ? launch_mfma<128, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)

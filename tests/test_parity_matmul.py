@@ -103,6 +103,19 @@ def _threads(bm, bn):
     return 512 if (bm, bn) == (256, 256) else 256
 
 
+@pytest.mark.parametrize("M,N,K", [(5, 7, 8), (300, 260, 200), (257, 513, 264), (512, 512, 64), (256, 256, 1024), (700, 300, 4104)])
+@pytest.mark.parametrize("split", [1, 3])
+def test_gemm_256x256_with_four_wavefronts(oracle, M, N, K, split):
+    # block = 256 selects the variant with one wavefront per SIMD and 128x128 wavefront tiles
+    a, w = _inputs(M, N, K, M + N + K)
+    bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
+    out = Guarded((M, N), torch.float16)
+    c = cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[256, 256, 64], split_k=split)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c)
+    _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+    assert list(_lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c).launch_args)[3:5] == [256, 5 * 256 * 128]
+
+
 TILES = [(256, 256), (256, 128), (128, 256), (128, 128), (64, 128), (128, 64), (64, 64)]
 
 
