@@ -211,22 +211,28 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     constexpr int kUnit = BM * kRowBytes;
     static_assert(5 * kUnit <= kLdsAlloc, "ring exceeds the LDS");
     auto wrap5 = [](int v) { return v >= 5 ? v - 5 : v; };
-    auto fetch_unit = [&](const __amdgpu_buffer_rsrc_t& r, int kt, int slot) {
-      const unsigned off = (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K)
-                               ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+    // per-lane byte offset of this lane's chunk in k tile kt of either operand (out of range past K)
+    auto lane_off = [&](int kt) -> unsigned {
+      return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+    };
+    // this wavefront's LA block loads of one unit; the block's row offset rides in the scalar offset
+    auto fetch_unit = [&](bool is_w, unsigned voff, int slot) {
       char* base = lds + slot * kUnit + wv * 1024;
 #pragma unroll
-      for (int i = 0; i < LA; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
+      for (int i = 0; i < LA; ++i) {
+        if (is_w) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + i * NW * 1024), 16, voff, i * g_step, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, voff, i * g_step, 0, 0);
+      }
     };
     const unsigned group = wv >> 2;
     const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
     if (ktiles > 0) {
-      fetch_unit(ra, 0, 0);
-      fetch_unit(rw, 0, 1);
+      const unsigned v0 = lane_off(0);
+      fetch_unit(false, v0, 0);
+      fetch_unit(true, v0, 1);
     }
     if (ktiles > 1) {
-      fetch_unit(ra, 1, 2);
+      fetch_unit(false, lane_off(1), 2);
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA));  // tile 0 has landed, A(1) may be in flight
     } else {
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
@@ -238,9 +244,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       DTAS_SCHED_FENCE();
     }
     int slot_a = 0, slot_w = 1;  // slots of A(kt) and W(kt)
-    for (int kt = 0; kt < ktiles; ++kt) {
+    // one k tile; `steady`: tiles kt+1 and kt+2 exist (no conditions in the instruction stream)
+    auto pp_tile = [&](int kt, bool steady) {
       const char* cur_a = lds + slot_a * kUnit + a_frag;
       const char* cur_w = lds + slot_w * kUnit + b_frag;
+      const bool w1 = steady || kt + 1 < ktiles, a2 = steady || kt + 2 < ktiles;
+      const unsigned vw = lane_off(kt + 1), va = lane_off(kt + 2);
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const int set = ks & 1;
@@ -251,13 +260,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         for (int i = 0; i < MT; ++i) fa[set][i] = *reinterpret_cast<const f16x8*>(cur_a + i * 4096 + lds_rd[ks]);
 #pragma unroll
         for (int j = 0; j < NT; ++j) fb[set][j] = *reinterpret_cast<const f16x8*>(cur_w + j * 4096 + lds_rd[ks]);
-        if (ks == 0 && kt + 1 < ktiles) fetch_unit(rw, kt + 1, wrap5(slot_w + 2));
-        if (ks == 1 && kt + 2 < ktiles) fetch_unit(ra, kt + 2, wrap5(slot_a + 4));
+        if (ks == 0 && w1) fetch_unit(true, vw, wrap5(slot_w + 2));
+        if (ks == 1 && a2) fetch_unit(false, va, wrap5(slot_a + 4));
         // fragments in registers before the barrier (after a tile's last step the other group may
         // overwrite the slots); at the last step also this wavefront's loads of tile kt+1: all
         // but the newest unit's, A(kt+2), if that was requested
         if (ks == 3) {
-          if (kt + 2 < ktiles) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+          if (a2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
         } else {
           __builtin_amdgcn_s_waitcnt(0xC07F);
         }
@@ -276,7 +285,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       }
       slot_a = wrap5(slot_a + 2);
       slot_w = wrap5(slot_w + 2);
-    }
+    };
+    int kt = 0;
+    for (; kt + 2 < ktiles; ++kt) pp_tile(kt, true);
+    for (; kt < ktiles; ++kt) pp_tile(kt, false);
     if (group == 0) {
       __builtin_amdgcn_s_barrier();
       DTAS_SCHED_FENCE();
