@@ -163,13 +163,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     const unsigned off = (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K)
                              ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
     char* base = lds + (kt % NS) * kStage + wv * 1024;
+    // (the block's row offset rides in the scalar offset operand: no vector add per load)
 #pragma unroll
     for (int i = 0; i < LA; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off + i * g_step, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, 0);
 #pragma unroll
     for (int i = 0; i < LB; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16,
-                                               off + i * g_step, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
   };
 
   f16x8 fa[2][MT], fb[2][NT];
