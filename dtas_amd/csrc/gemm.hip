@@ -383,15 +383,110 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     int kt = 0;
     for (; kt + 2 < ktiles; ++kt) k_tile(kt, true);
     for (; kt < ktiles; ++kt) k_tile(kt, false);
+  } else if constexpr (NS >= 3) {
+    // ---- NS >= 3 whole-tile stages, for grids with about one workgroup (one wavefront per SIMD) per
+    // CU: nothing hides a burst of loads or a run of scalar bookkeeping, so the kL block loads of a
+    // tile are issued in four parts between the MFMAs of four consecutive steps (part 0 right after
+    // the barrier that frees the stage, parts 1-3 in the next tile's first three steps), with their
+    // per-lane offset computed once and the block offsets in the scalar operand; the steady-state
+    // loop carries no conditions.
+    constexpr int kL = LA + LB;
+    auto lane_off = [&](int kt) -> unsigned {
+      return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+    };
+    // block load l (0 .. kL-1: A blocks, then W blocks) of a tile into `stage`
+    auto fetch_one = [&](int l_, unsigned voff, char* stage) {
+      if (l_ < LA)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(stage + wv * 1024 + l_ * NW * 1024), 16, voff, l_ * g_step, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(stage + kABytes + wv * 1024 + (l_ - LA) * NW * 1024), 16, voff,
+                                                 (l_ - LA) * g_step, 0, 0);
+    };
+    // MFMAs of `set`, the next step's fragment reads, and part `part` of a tile's loads (if `dma`)
+    auto step_dma = [&](int set, const char* stage, int ks, bool reads, bool dma, int part, unsigned voff, char* dst) {
+      constexpr int kReads = MT + NT, kMfma = MT * NT;
+#pragma unroll
+      for (int q = 0; q < kMfma; ++q) {
+        if (reads) {
+#pragma unroll
+          for (int r = 0; r < kReads; ++r)
+            if (r * kMfma / kReads == q) {
+              if (r < MT) read_a(set ^ 1, r, stage, ks); else read_b(set ^ 1, r - MT, stage, ks);
+            }
+        }
+        const int i = q / NT, j = q % NT;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
+        if (dma) {
+          // loads part*kL/4 .. (part+1)*kL/4 - 1, spread over the step's MFMAs
+          const int lo = part * kL / 4, hi = (part + 1) * kL / 4;
+#pragma unroll
+          for (int l_ = 0; l_ < kL; ++l_)
+            if (l_ >= lo && l_ < hi && (l_ - lo) * kMfma / (hi - lo) == q) fetch_one(l_, voff, dst);
+        }
+        DTAS_SCHED_FENCE();
+      }
+    };
+    if (ktiles > 0) {
+      const unsigned v0 = lane_off(0);
+#pragma unroll
+      for (int l_ = 0; l_ < kL; ++l_) fetch_one(l_, v0, lds);
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    // tiles 1 .. NS-2 whole, part 0 of tile NS-1
+#pragma unroll
+    for (int p = 1; p < NS; ++p) {
+      if (p < ktiles) {
+        const unsigned vp = lane_off(p);
+#pragma unroll
+        for (int l_ = 0; l_ < (p < NS - 1 ? kL : kL / 4); ++l_) fetch_one(l_, vp, lds + p * kStage);
+      }
+    }
+    if (ktiles > 0) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) read_b(0, j, lds, 0);
+    }
+    DTAS_SCHED_FENCE();
+    int cur_s = 0;  // stage of tile kt
+    auto wrap = [](int v) { return v >= NS ? v - NS : v; };
+    auto k_tile = [&](int kt, bool steady) {
+      char* cur = lds + cur_s * kStage;
+      char* nxt = lds + wrap(cur_s + 1) * kStage;
+      char* late = lds + wrap(cur_s + NS - 1) * kStage;  // stage of tile kt-1 = of tile kt+NS-1
+      const bool have_late = steady || kt + NS - 1 < ktiles, have_new = steady || kt + NS < ktiles;
+      const unsigned v_late = lane_off(kt + NS - 1), v_new = lane_off(kt + NS);
+      step_dma(0, cur, 1, true, have_late, 1, v_late, late);
+      step_dma(1, cur, 2, true, have_late, 2, v_late, late);
+      step_dma(0, cur, 3, true, have_late, 3, v_late, late);
+      // tile kt+1 must have landed; later tiles (at most NS-2 of them) may stay in flight.  Loads
+      // complete in order, so it is enough to allow that many tiles' worth of loads outstanding.
+      if (steady) {
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * kL));
+      } else {
+        const int ahead = ktiles - 2 - kt;  // tiles after kt+1 that have been requested
+        if (NS >= 4 && ahead >= 2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * kL));
+        else if (ahead >= 1) __builtin_amdgcn_s_waitcnt(waitcnt_imm(kL));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+      }
+      __builtin_amdgcn_s_barrier();  // ... and every wavefront has finished reading tile kt
+      DTAS_SCHED_FENCE();
+      step_dma(1, nxt, 0, steady || kt + 1 < ktiles, have_new, 0, v_new, cur);
+      cur_s = wrap(cur_s + 1);
+    };
+    static_assert((NS - 2) * kL <= 63, "outstanding loads must fit the vmcnt field");
+    int kt = 0;
+    for (; kt + NS < ktiles; ++kt) k_tile(kt, true);
+    for (; kt < ktiles; ++kt) k_tile(kt, false);
   } else {
-  // NS stages: tile 0 resident, tiles 1 .. NS-1 in flight, fragments of (tile 0, step 0) in registers
+  // two stages: tile 0 resident, tile 1 in flight, fragments of (tile 0, step 0) in registers
   if (ktiles > 0) fetch(0);
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
   DTAS_SCHED_FENCE();
-#pragma unroll
-  for (int p = 1; p < NS; ++p)
-    if (p < ktiles) fetch(p);
+  if (1 < ktiles) fetch(1);
   if (ktiles > 0) {
 #pragma unroll
     for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
@@ -399,22 +494,14 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     for (int j = 0; j < NT; ++j) read_b(0, j, lds, 0);
   }
   DTAS_SCHED_FENCE();
-
-  // vmcnt(n) with lgkmcnt(0): n is a compile-time field of the instruction
-  constexpr int kL = LA + LB;
   for (int kt = 0; kt < ktiles; ++kt) {
     const char* cur = lds + (kt % NS) * kStage;
     const char* nxt = lds + ((kt + 1) % NS) * kStage;
     step(0, cur, 1, true);
     step(1, cur, 2, true);
     step(0, cur, 3, true);
-    // tile kt+1 must have landed; tiles kt+2 .. (at most NS-2 of them) may stay in flight.  Loads
-    // complete in order, so it is enough to allow that many tiles' worth of loads outstanding.
-    const int ahead = ktiles - 2 - kt;  // tiles after kt+1 that have been requested, if < NS-2
-    if (NS >= 4 && ahead >= 2) __builtin_amdgcn_s_waitcnt(0x0070 | ((2 * kL) & 15) | (((2 * kL) >> 4) << 14));
-    else if (NS >= 3 && ahead >= 1) __builtin_amdgcn_s_waitcnt(0x0070 | (kL & 15) | ((kL >> 4) << 14));
-    else __builtin_amdgcn_s_waitcnt(0x0070);
-    __builtin_amdgcn_s_barrier();  // ... and every wavefront has finished reading tile kt
+    __builtin_amdgcn_s_waitcnt(0x0070);  // tile kt+1 has landed
+    __builtin_amdgcn_s_barrier();        // ... and every wavefront has finished reading tile kt
     DTAS_SCHED_FENCE();
     if (kt + NS < ktiles) fetch(kt + NS);  // into the stage tile kt occupied
     DTAS_SCHED_FENCE();
