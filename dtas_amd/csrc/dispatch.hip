@@ -119,53 +119,51 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
   return make(DTAS_GEMV_SPLITK, 256, 8, 2, 1);
 }
 
-// GEMM, from sweeps of every tile x stage count x K split over M on an MI355X:
-//  * 256x256 (8 wavefronts, ping-pong) once it yields >= 150 workgroups;
-//  * else 128x128 once that yields >= 256 workgroups, with the deepest LDS pipeline that keeps
-//    all tiles co-resident;
-//  * else few tiles: each workgroup's k loop is a chain of ~0.3 us (64x64) / ~0.6 us (128x128)
-//    steps however few CUs are busy, so K is split over up to 4 workgroups per tile (partials
-//    summed by the last one to arrive, ~1 us / ~4 us per partial).  The cheapest of the candidates
-//    under that model is taken; against it, for M <= 32, the W-streaming SKINNY kernel, whose
-//    time grows with N*K (about 3.5 TB/s of W) instead of with K.
+// GEMM: a cost model fitted to sweeps of every tile x stage count x K split over M on an MI355X.
+// A candidate's time is (rounds of workgroups over the chip) x (time of one k tile) x (k tiles):
+//  * time of one k tile with every CU busy: 256x256 1.80 us, 256x128 (3 stages) 1.045 us, 128x128
+//    0.665 us with 4 stages (one workgroup per CU) or 1.14 us per round of two per CU with 2 stages;
+//  * a partly filled last round is faster than a full one: x (0.55 + 0.45 * fill);
+//  * 64x64 (two per CU): 0.33 us per k tile up to 256 workgroups, x 0.82 * workgroups / 256 beyond;
+//  * few tiles: K split over up to 4 workgroups per tile (128x128 and 64x64), each partial tile
+//    costing ~4 us / ~1 us for the last workgroup to add up;
+//  * M <= 32: the W-streaming SKINNY kernel, whose time grows with N*K (about 3.5 TB/s of W).
 struct GemmChoice {
   double us;
-  int tile, split;
+  int bm, bn, block, stages, split;
 };
+
+double gemm_rounds(double wgs, double slots) {
+  const double full = static_cast<double>(static_cast<int64_t>(wgs / slots));
+  const double rem = wgs - full * slots;
+  return full + (rem > 0 ? 0.55 + 0.45 * rem / slots : 0.0);
+}
 
 dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   const int64_t n = N > 0 ? N : 1, k = K > 0 ? K : 1;
-  if (ceil_div(M_hi, 256) * ceil_div(n, 256) >= 150) return make(DTAS_GEMM_MFMA, 512, 8, 2, 256, 256, 64);
-  if (ceil_div(M_hi, 128) * ceil_div(n, 128) >= 256) {
-    const int64_t tiles = ceil_div(M_hi, 128) * ceil_div(n, 128);
-    int stages = 2;
-    for (int ns = 4; ns > 2; --ns) {
-      const int64_t per_cu = kLdsBytes / (ns * 256 * 128);
-      if (per_cu >= 1 && (per_cu == 1 ? tiles <= kNumCU : tiles * 4 <= kNumCU * per_cu * 3)) {
-        stages = ns;
-        break;
-      }
-    }
-    return make(DTAS_GEMM_MFMA, 256, 8, stages, 128, 128, 64);
-  }
   const int64_t ktiles = ceil_div(k, 64);
-  GemmChoice best = {1e30, 64, 1};
-  for (int tile = 64; tile <= 128; tile *= 2) {
-    const double step_us = tile == 64 ? 0.33 : 0.62, partial_us = tile == 64 ? 1.0 : 4.0;
-    const int64_t tiles = ceil_div(M_hi, tile) * ceil_div(n, tile);
-    for (int split = 1; split <= 4; ++split) {
-      if (split > 1 && (ktiles / split < 8 || (tile == 128 && tiles * split > kNumCU))) continue;
-      const double wgs = static_cast<double>(tiles * split);
-      const double crowd = wgs <= kNumCU ? 1.0 : 0.82 * wgs / kNumCU;  // two per CU run at ~0.6 of the speed each
-      const double us = static_cast<double>(ceil_div(ktiles, split)) * step_us * crowd + (split > 1 ? partial_us * split : 0.0);
-      if (us < best.us) best = {us, tile, split};
-    }
+  GemmChoice best = {1e30, 64, 64, 256, 4, 1};
+  auto consider = [&](double us, int bm, int bn, int block, int stages, int split) {
+    if (us < best.us) best = {us, bm, bn, block, stages, split};
+  };
+  auto tiles_of = [&](int bm, int bn) { return static_cast<double>(ceil_div(M_hi, bm) * ceil_div(n, bn)); };
+  const double kt = static_cast<double>(ktiles);
+  consider(gemm_rounds(tiles_of(256, 256), kNumCU) * 1.80 * kt, 256, 256, 512, 2, 1);
+  consider(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.045 * kt, 256, 128, 256, 3, 1);
+  consider(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 128, 128, 256, 2, 1);
+  for (int split = 1; split <= 4; ++split) {
+    if (split > 1 && ktiles / split < 8) continue;
+    const double steps = static_cast<double>(ceil_div(ktiles, split));
+    const double t128 = tiles_of(128, 128) * split, t64 = tiles_of(64, 64) * split;
+    if (split == 1 || t128 <= kNumCU)
+      consider(gemm_rounds(t128, kNumCU) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 128, 128, 256, 4, split);
+    consider((t64 <= kNumCU ? 1.0 : 0.82 * t64 / kNumCU) * 0.33 * steps + (split > 1 ? 1.0 * split : 0.0), 64, 64, 256, 4, split);
   }
   if (M_hi <= 32) {
     const double skinny_us = static_cast<double>(n) * static_cast<double>(k) * 2.0 / 3.5e6 * (M_hi <= 8 ? 0.9 : M_hi <= 16 ? 0.95 : 1.35);
     if (skinny_us <= best.us) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
   }
-  return make(DTAS_GEMM_MFMA, 256, 8, 4, best.tile, best.tile, 64, best.split);
+  return make(DTAS_GEMM_MFMA, best.block, 8, best.stages, best.bm, best.bn, 64, best.split);
 }
 
 dtas_config policy(int op, int64_t n_hi, int64_t d0, int64_t d1) {

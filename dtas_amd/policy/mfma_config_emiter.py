@@ -32,36 +32,40 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         return 2 if tile_m + tile_n >= 512 else 3 if tile_m + tile_n >= 384 else 4
 
     def preferred(self, m_hi: int, N: int, K: int = 4096):
-        """(tile_m, tile_n, stages, split_k) that sweeps on an MI355X favoured: 256x256 once it yields
-        >= 150 workgroups, else 128x128 from 256 workgroups (the deepest load pipeline with which all tiles
-        stay co-resident).  With fewer tiles a workgroup's k loop is a serial chain of ~0.33 us (64x64) or
-        ~0.62 us (128x128) steps, so K is split over workgroups when the saved steps outweigh the ~1 us
-        (~4 us) each partial tile costs; more than one workgroup per CU run at ~0.6 of the speed each."""
+        """(tile_m, tile_n, stages, split_k) under the cost model fitted to sweeps on an MI355X (the same
+        one the library's built-in table uses): time = rounds of workgroups over the chip x time of one
+        k tile x k tiles.  One k tile with every CU busy: 256x256 1.80 us, 256x128 (3 stages) 1.045 us,
+        128x128 0.665 us (4 stages, one workgroup per CU) or 1.14 us per round of two per CU (2 stages);
+        a partly filled last round costs 0.55 + 0.45 * fill of a full one; 64x64 0.33 us per k tile up to
+        one workgroup per CU, x 0.82 * workgroups / CUs beyond; with few tiles K is split over up to 4
+        workgroups per tile at ~4 us (128x128) / ~1 us (64x64) per partial tile."""
         cdiv = lambda a, b: -(-a // b)
-        self._model_us = float("inf")
-        if cdiv(m_hi, 256) * cdiv(N, 256) >= 150:
-            return 256, 256, 2, 1
-        if cdiv(m_hi, 128) * cdiv(N, 128) >= 256:
-            tiles = cdiv(m_hi, 128) * cdiv(N, 128)
-            for ns in (4, 3):
-                per_cu = _LDS // (ns * 2 * 128 * 128)
-                if per_cu >= 1 and (tiles <= self.arch.num_sm if per_cu == 1 else tiles * 4 <= self.arch.num_sm * per_cu * 3):
-                    return 128, 128, ns, 1
-            return 128, 128, 2, 1
+        cus = self.arch.num_sm
         ktiles = cdiv(K, 64)
-        best = (float("inf"), 64, 1)
-        for t, step_us, partial_us in ((64, 0.33, 1.0), (128, 0.62, 4.0)):
-            tiles = cdiv(m_hi, t) * cdiv(N, t)
-            for split in (1, 2, 3, 4):
-                if split > 1 and (ktiles // split < 8 or (t == 128 and tiles * split > self.arch.num_sm)):
-                    continue
-                wgs = tiles * split
-                crowd = 1.0 if wgs <= self.arch.num_sm else 0.82 * wgs / self.arch.num_sm
-                us = cdiv(ktiles, split) * step_us * crowd + (partial_us * split if split > 1 else 0.0)
-                if us < best[0]:
-                    best = (us, t, split)
+
+        def rounds(wgs, slots):
+            full, rem = divmod(wgs, slots)
+            return full + ((0.55 + 0.45 * rem / slots) if rem else 0.0)
+
+        tiles = lambda bm, bn: cdiv(m_hi, bm) * cdiv(N, bn)
+        cands = [(rounds(tiles(256, 256), cus) * 1.80 * ktiles, (256, 256, 2, 1)),
+                 (rounds(tiles(256, 128), cus) * 1.045 * ktiles, (256, 128, 3, 1)),
+                 (rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, (128, 128, 2, 1))]
+        for split in (1, 2, 3, 4):
+            if split > 1 and ktiles // split < 8:
+                continue
+            steps = cdiv(ktiles, split)
+            t128, t64 = tiles(128, 128) * split, tiles(64, 64) * split
+            if split == 1 or t128 <= cus:
+                cands.append((rounds(t128, cus) * 0.665 * steps + (4.0 * split if split > 1 else 0.0), (128, 128, 4, split)))
+            cands.append(((1.0 if t64 <= cus else 0.82 * t64 / cus) * 0.33 * steps + (1.0 * split if split > 1 else 0.0),
+                          (64, 64, 4, split)))
+        best = cands[0]
+        for c in cands[1:]:          # first strict minimum, in the library's order of evaluation
+            if c[0] < best[0]:
+                best = c
         self._model_us = best[0]
-        return best[1], best[1], 4, best[2]
+        return best[1]
 
     def prefers_skinny(self, m_hi: int, N: int, K: int) -> bool:
         """M <= 32: the W-streaming kernel (about 3.5 TB/s of W, slower as M grows) against the model's
