@@ -23,6 +23,8 @@ ELT_VECTOR, ELT_SCALAR = 0, 1
 RED_WAVE_ROW, RED_BLOCK_ROW, RED_STREAM_ROW = 0, 1, 2
 GEMV_SPLITK = 0
 GEMM_MFMA, GEMM_SKINNY = 0, 1
+# enum dtas_epilogue
+EPI_BIAS, EPI_BIAS_ADD2, EPI_BIAS_ADD2_CAST_F32, EPI_BIAS_GELU = 0, 1, 2, 3
 
 
 class DtasConfig(ctypes.Structure):
@@ -90,6 +92,7 @@ SIGNATURES = {
     "dtas_softmax_f16": [_vp, _vp, _i64, _i64, _cfg, _vp],
     "dtas_gemv_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _cfg, _vp],
     "dtas_gemm_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],
+    "dtas_gemm_f16_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_int32, _cfg, _vp],
 }
 
 _lib = None

@@ -127,11 +127,17 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
     elif op == "softmax":
         ops.softmax(tensors[0], tensors[1], abi)
     elif op == "matmul":
-        bias = tensors[2] if len(tensors) == 4 else None
-        if FuncInfo(func).kind == FuncKind.kFunc_GEMV:
-            ops.gemv(tensors[0], tensors[1], bias, tensors[-1], abi)
+        epilogue = int(func.attrs.get("epilogue", 0))
+        if epilogue in (_lib.EPI_BIAS_ADD2, _lib.EPI_BIAS_ADD2_CAST_F32):   # A, W, bias, res1, res2, out
+            ops.gemm(tensors[0], tensors[1], tensors[2], tensors[5], abi, epilogue=epilogue, res1=tensors[3], res2=tensors[4])
+        elif epilogue == _lib.EPI_BIAS_GELU:                                  # A, W, bias, out
+            ops.gemm(tensors[0], tensors[1], tensors[2], tensors[3], abi, epilogue=epilogue)
         else:
-            ops.gemm(tensors[0], tensors[1], bias, tensors[-1], abi)
+            bias = tensors[2] if len(tensors) == 4 else None
+            if FuncInfo(func).kind == FuncKind.kFunc_GEMV:
+                ops.gemv(tensors[0], tensors[1], bias, tensors[-1], abi)
+            else:
+                ops.gemm(tensors[0], tensors[1], bias, tensors[-1], abi)
     else:
         raise ValueError(f"no kernel family for op {op!r}")
 

@@ -64,10 +64,45 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
 
-__device__ __forceinline__ half_t finish(float acc, const half_t* bias, int64_t j) {
-  half_t r = static_cast<half_t>(acc);
-  if (bias) r = static_cast<half_t>(static_cast<float>(r) + static_cast<float>(bias[j]));
-  return r;
+// What follows the product, as the fused PrimFuncs spell it: every intermediate is an fp16 tensor,
+// so every step below rounds to fp16 (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:163-200
+// fused_NT_matmul2_add1_add3_add3, :202-246 ..._cast, :248-318 fused_NT_matmul3_add2_gelu).
+struct GemmEpilogue {
+  const half_t* bias;  // [N] or NULL
+  const half_t* res1;  // [M, N]: ADD2 kinds
+  const half_t* res2;  // [M, N]: ADD2 kinds
+  int kind;            // enum dtas_epilogue
+  int out_f32;         // the output buffer holds fp32 (ADD2_CAST_F32)
+};
+
+__device__ __forceinline__ half_t round_h(float v) { return static_cast<half_t>(v); }
+
+// mm: the product already rounded to fp16.  Returns the fp16 result (the cast kind widens it).
+__device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& ep, float bias_j, float r1, float r2) {
+  half_t t = mm;
+  if (ep.bias) t = round_h(static_cast<float>(t) + bias_j);
+  if (ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32) {
+    t = round_h(r1 + static_cast<float>(t));   // T_add_1 = lv58 + T_add
+    t = round_h(static_cast<float>(t) + r2);   // T_add_2 = T_add_1 + lv2
+  } else if (ep.kind == DTAS_EPI_BIAS_GELU) {
+    const float x = static_cast<float>(t);
+    const half_t m = round_h(x * static_cast<float>(static_cast<half_t>(0.70710678118654757f)));
+    const half_t e = round_h(erff(static_cast<float>(m)));
+    const half_t h = round_h(static_cast<float>(e) * 0.5f);
+    const half_t a = round_h(0.5f + static_cast<float>(h));
+    t = round_h(x * static_cast<float>(a));
+  }
+  return t;
+}
+
+// one element, any alignment (skinny and element-access kernels)
+__device__ __forceinline__ void finish(float acc, const GemmEpilogue& ep, void* C, int64_t row, int64_t col, int64_t N) {
+  const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const half_t r = epilogue_value(round_h(acc), ep, ep.bias ? static_cast<float>(ep.bias[col]) : 0.f,
+                                  add2 ? static_cast<float>(ep.res1[row * N + col]) : 0.f,
+                                  add2 ? static_cast<float>(ep.res2[row * N + col]) : 0.f);
+  if (ep.out_f32) static_cast<float*>(C)[row * N + col] = static_cast<float>(r);
+  else static_cast<half_t*>(C)[row * N + col] = r;
 }
 
 // Position of workgroup `wg` in a tile order in which each XCD gets a contiguous span:
@@ -88,8 +123,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 template <int BM, int BN, int WM, int WN, int NS>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ W,
-                                                                 const half_t* __restrict__ bias,
-                                                                 half_t* __restrict__ C, int64_t M, int64_t N,
+                                                                 GemmEpilogue ep, void* __restrict__ C, int64_t M,
+                                                                 int64_t N,
                                                                  int64_t K, unsigned tiles_m, unsigned tiles_n,
                                                                  unsigned nsplit, float* __restrict__ ws,
                                                                  unsigned* __restrict__ arrivals) {
@@ -591,12 +626,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // no barrier: a wavefront reads back only what it wrote itself
   const unsigned slot = l % kSlots, rsub = l / kSlots;
   const int64_t col = n0 + wn * WTN + slot * 4;
-  const bool vec_store = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(C) & 7u) == 0 && col + 3 < N;
+  const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  // 8-byte accesses to C and the residuals (16-byte to an fp32 C) where extents and pointers allow
+  const bool vec_store = (N % 4 == 0) && col + 3 < N &&
+                         (reinterpret_cast<uintptr_t>(C) & (ep.out_f32 ? 15u : 7u)) == 0 &&
+                         (!add2 || ((reinterpret_cast<uintptr_t>(ep.res1) | reinterpret_cast<uintptr_t>(ep.res2)) & 7u) == 0);
   float bv[4] = {0.f, 0.f, 0.f, 0.f};
-  if (bias) {
+  if (ep.bias) {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      if (col + e < N) bv[e] = static_cast<float>(bias[col + e]);
+      if (col + e < N) bv[e] = static_cast<float>(ep.bias[col + e]);
   }
 #pragma unroll
   for (int p = 0; p < WTM / kRowsPerPass; ++p) {
@@ -604,17 +643,45 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     f16x4 hv = *reinterpret_cast<const f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8));
     const int64_t row = m0 + wm * WTM + m;
     if (row >= M) continue;
-    if (bias) {  // "+ bias" is the PrimFunc's separate fp16 add: the sum was already rounded to fp16
+    const int64_t at = row * N + col;
+    if (ep.kind != DTAS_EPI_BIAS || ep.bias) {  // "+ bias" etc. act on the sum already rounded to fp16
+      f16x4 r1v = {}, r2v = {};
+      if (add2) {
+        if (vec_store) {
+          r1v = *reinterpret_cast<const f16x4*>(ep.res1 + at);
+          r2v = *reinterpret_cast<const f16x4*>(ep.res2 + at);
+        } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(static_cast<float>(hv[e]) + bv[e]);
-    }
-    half_t* dst = C + row * N + col;
-    if (vec_store) {
-      *reinterpret_cast<f16x4*>(dst) = hv;
-    } else {
+          for (int e = 0; e < 4; ++e)
+            if (col + e < N) {
+              r1v[e] = ep.res1[at + e];
+              r2v[e] = ep.res2[at + e];
+            }
+        }
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (col + e < N) dst[e] = hv[e];
+        hv[e] = epilogue_value(hv[e], ep, bv[e], static_cast<float>(r1v[e]), static_cast<float>(r2v[e]));
+    }
+    if (ep.out_f32) {
+      float* dst = static_cast<float*>(C) + at;
+      if (vec_store) {
+        *reinterpret_cast<f32x4v*>(dst) = f32x4v{static_cast<float>(hv[0]), static_cast<float>(hv[1]),
+                                                 static_cast<float>(hv[2]), static_cast<float>(hv[3])};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < N) dst[e] = static_cast<float>(hv[e]);
+      }
+    } else {
+      half_t* dst = static_cast<half_t*>(C) + at;
+      if (vec_store) {
+        *reinterpret_cast<f16x4*>(dst) = hv;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < N) dst[e] = hv[e];
+      }
     }
   }
 }
@@ -625,8 +692,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 // 4*(l >> 4) + v, column l & 15 of the 16x16 block.
 template <int MT>
 __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
-                                                          const half_t* __restrict__ bias, half_t* __restrict__ C,
-                                                          int64_t M, int64_t N, int64_t K) {
+                                                          GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
+                                                          int64_t K) {
   __shared__ f32x4v part[16][MT][64];
   const unsigned t = threadIdx.x, l = t & 63u, wv = t >> 6, nwaves = blockDim.x >> 6;
   const int64_t n0 = static_cast<int64_t>(blockIdx.x) * 16;
@@ -710,7 +777,7 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int64_t row = i * 16 + 4 * (ll >> 4) + v;
-        if (row < M) C[row * N + col] = finish(s[v], bias, col);
+        if (row < M) finish(s[v], ep, C, row, col, N);
       }
     }
   }
@@ -718,8 +785,8 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
 
 // Any K and alignment: one thread per element of C.
 __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
-                                                          const half_t* __restrict__ bias, half_t* __restrict__ C,
-                                                          int64_t M, int64_t N, int64_t K) {
+                                                          GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
+                                                          int64_t K) {
   const int64_t total = M * N;
   for (int64_t ij = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; ij < total;
        ij += static_cast<int64_t>(gridDim.x) * blockDim.x) {
@@ -727,7 +794,7 @@ __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restri
     const half_t* w = W + (ij % N) * K;
     float acc = 0.f;
     for (int64_t k = 0; k < K; ++k) acc += static_cast<float>(a[k]) * static_cast<float>(w[k]);
-    C[ij] = finish(acc, bias, ij % N);
+    finish(acc, ep, C, ij / N, ij % N, N);
   }
 }
 
@@ -781,7 +848,7 @@ int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsign
 }
 
 template <int BM, int BN, int WM, int WN, int NS>
-int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const half_t* bias, half_t* C, int64_t M, int64_t N,
+int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
                 int64_t K, int nsplit) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
   const size_t tiles = static_cast<size_t>(tiles_m) * tiles_n;
@@ -793,7 +860,7 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const half_t* b
     if (split_workspace(bytes, tiles, &partials, &arrivals) != 0) return -1;
   }
   hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(static_cast<unsigned>(tiles * nsplit)), dim3(64 * WM * WN), 0,
-                     s, A, W, bias, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
+                     s, A, W, ep, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
 
@@ -864,15 +931,30 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
 
 extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
                              const dtas_config* user, void* stream) {
+  return dtas_gemm_f16_fused(A, W, bias, nullptr, nullptr, C, M, N, K, DTAS_EPI_BIAS, user, stream);
+}
+
+extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bias, const void* res1, const void* res2,
+                                   void* C, int64_t M, int64_t N, int64_t K, int32_t epilogue, const dtas_config* user,
+                                   void* stream) {
   using namespace dtas;
   clear_error();
+  if (epilogue < DTAS_EPI_BIAS || epilogue > DTAS_EPI_BIAS_GELU) return fail("gemm: unknown epilogue %d", epilogue);
+  const bool add2 = epilogue == DTAS_EPI_BIAS_ADD2 || epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const int out_bytes = epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32 ? 4 : 2;
   if (M < 0 || N < 0 || K < 0) return fail("gemm: negative extent M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
   if (M == 0 || N == 0) return 0;
   if ((K != 0 && (M > INT64_MAX / 4 / K || N > INT64_MAX / 4 / K)) || M > INT64_MAX / 4 / N) return fail("gemm: extents overflow");
   if (!C || (K > 0 && (!A || !W))) return fail("gemm: NULL buffer");
-  if (overlaps(C, M * N * 2, A, M * K * 2) || overlaps(C, M * N * 2, W, N * K * 2)) return fail("gemm: output overlaps an input");
-  // one row of A is the decode GEMV: same PrimFunc shape, dedicated kernel
-  if (!user && M == 1) return dtas_gemv_f16(A, W, bias, C, N, K, nullptr, stream);
+  if (add2 && (!res1 || !res2)) return fail("gemm: the add-add epilogue needs both residual buffers");
+  if (!add2 && (res1 || res2)) return fail("gemm: residual buffers given for an epilogue that takes none");
+  if (overlaps(C, M * N * out_bytes, A, M * K * 2) || overlaps(C, M * N * out_bytes, W, N * K * 2) ||
+      (add2 && (overlaps(C, M * N * out_bytes, res1, M * N * 2) || overlaps(C, M * N * out_bytes, res2, M * N * 2))))
+    return fail("gemm: output overlaps an input");
+  // one row of A with the plain epilogue is the decode GEMV: same PrimFunc shape, dedicated kernel
+  if (!user && M == 1 && epilogue == DTAS_EPI_BIAS) return dtas_gemv_f16(A, W, bias, C, N, K, nullptr, stream);
+  const GemmEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1),
+                           static_cast<const half_t*>(res2), epilogue, out_bytes == 4 ? 1 : 0};
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMM_F16, M, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(A, 16) && aligned(W, 16);
   if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
@@ -881,8 +963,8 @@ extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, voi
   hipStream_t s = static_cast<hipStream_t>(stream);
   const half_t* a = static_cast<const half_t*>(A);
   const half_t* w = static_cast<const half_t*>(W);
-  const half_t* b = static_cast<const half_t*>(bias);
-  half_t* c = static_cast<half_t*>(C);
+  const GemmEpilogue& b = ep;
+  void* c = C;
   if (cfg.vec == 1) {
     hipLaunchKernelGGL(gemm_scalar_kernel, dim3(static_cast<unsigned>(la[0])), dim3(256), 0, s, a, w, b, c, M, N, K);
     return check_launch("gemm");

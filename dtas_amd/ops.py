@@ -150,16 +150,27 @@ def gemv(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], y: torc
 
 
 def gemm(A: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], C: torch.Tensor,
-         cfg: Optional[DtasConfig] = None) -> None:
-    """C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]); fp16, fp32 accumulate on MFMA.  M is every leading
-    extent of A flattened."""
-    _dev(A, W, bias, C)
+         cfg: Optional[DtasConfig] = None, epilogue: int = 0, res1: Optional[torch.Tensor] = None,
+         res2: Optional[torch.Tensor] = None) -> None:
+    """C[M,N] = epilogue(A[M,K] . W[N,K]^T); fp16 operands, fp32 accumulate on MFMA.  M is every leading
+    extent of A flattened.  epilogue (``_lib.EPI_*``): 0 ``+ bias``; 1 ``(res1 + (mm + bias)) + res2``;
+    2 the same into an fp32 C; 3 ``gelu(mm + bias)`` -- each step rounded to fp16 as in the fused
+    PrimFuncs (before_dl.py:163-318)."""
+    _dev(A, W, bias, C, res1, res2)
     N, K = W.shape
     if A.shape[-1] != K or C.shape[-1] != N:
         raise ValueError("gemm: inner extents differ")
     M = A.numel() // K if K else C.numel() // max(N, 1)
     if C.numel() != M * N or (bias is not None and bias.numel() != N):
         raise ValueError("gemm: shape mismatch")
-    if any(t.dtype != torch.float16 for t in (A, W, C)) or (bias is not None and bias.dtype != torch.float16):
-        raise ValueError("gemm: expects fp16 tensors")
-    check(lib().dtas_gemm_f16(_p(A), _p(W), _p(bias), _p(C), M, N, K, _cfg(cfg), _stream()), "dtas_gemm_f16")
+    want_out = torch.float32 if epilogue == _lib.EPI_BIAS_ADD2_CAST_F32 else torch.float16
+    if any(t.dtype != torch.float16 for t in (A, W)) or C.dtype != want_out or \
+            any(t is not None and t.dtype != torch.float16 for t in (bias, res1, res2)):
+        raise ValueError("gemm: expects fp16 operands (and an fp32 C for the cast epilogue)")
+    if any(t is not None and t.numel() != M * N for t in (res1, res2)):
+        raise ValueError("gemm: residual shape mismatch")
+    if epilogue == _lib.EPI_BIAS and res1 is None and res2 is None:
+        check(lib().dtas_gemm_f16(_p(A), _p(W), _p(bias), _p(C), M, N, K, _cfg(cfg), _stream()), "dtas_gemm_f16")
+    else:
+        check(lib().dtas_gemm_f16_fused(_p(A), _p(W), _p(bias), _p(res1), _p(res2), _p(C), M, N, K, epilogue, _cfg(cfg),
+                                        _stream()), "dtas_gemm_f16_fused")

@@ -179,6 +179,25 @@ int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64
 int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N,
                   int64_t K, const dtas_config* cfg, void* stream);
 
+/* ---- GEMM with the model's fused epilogues ------------------------------------
+ * The PrimFuncs keep every intermediate as an fp16 tensor, so each step rounds to fp16:
+ *  DTAS_EPI_BIAS               C = mm (+ bias)                        fused_NT_matmul4_add1, before_dl.py:320-341
+ *  DTAS_EPI_BIAS_ADD2          C = (res1 + (mm + bias)) + res2        fused_NT_matmul2_add1_add3_add3, :163-200
+ *  DTAS_EPI_BIAS_ADD2_CAST_F32 the same, widened into an fp32 C       fused_NT_matmul2_add1_add3_add3_cast, :202-246
+ *  DTAS_EPI_BIAS_GELU          t = mm + bias; C = t * (0.5 + 0.5 * erf(t * fp16(0.7071...)))
+ *                                                                      fused_NT_matmul3_add2_gelu, :248-318
+ * mm = A[M,K] . W[N,K]^T accumulated in fp32 and rounded to fp16 once.  res1, res2: [M,N] fp16,
+ * required by the ADD2 kinds and NULL otherwise; bias may be NULL for any kind. */
+enum dtas_epilogue {
+  DTAS_EPI_BIAS = 0,
+  DTAS_EPI_BIAS_ADD2 = 1,
+  DTAS_EPI_BIAS_ADD2_CAST_F32 = 2,
+  DTAS_EPI_BIAS_GELU = 3
+};
+int dtas_gemm_f16_fused(const void* A, const void* W, const void* bias, const void* res1,
+                        const void* res2, void* C, int64_t M, int64_t N, int64_t K,
+                        int32_t epilogue, const dtas_config* cfg, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -65,6 +65,7 @@ class _C:
                 "oracle_softmax_f16_f16": [vp, vp, i64, i64, ci],
                 "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
+                "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
             }
             for name, argtypes in sig.items():
                 fn = getattr(lib, name)
@@ -146,6 +147,18 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         return out
 
     @staticmethod
+    def gemm_fused(a, w, bias, res1, res2, kind: int, acc_f16: bool = False, threads: int = 1) -> np.ndarray:
+        """GEMM + fused epilogue (0 bias, 1 bias+add+add, 2 the same widened to fp32, 3 bias+gelu)."""
+        assert a.dtype == np.float16 and w.dtype == np.float16
+        K = a.shape[-1]
+        M, N = a.size // K, w.shape[0]
+        out = np.empty(a.shape[:-1] + (N,), dtype=np.float32 if kind == 2 else np.float16)
+        opt = lambda t: _ptr(t) if t is not None else None
+        _C.lib().oracle_gemm_f16_fused(_ptr(a), _ptr(w), opt(bias), opt(res1), opt(res2), _ptr(out), M, N, K, kind,
+                                       int(acc_f16), threads)
+        return out
+
+    @staticmethod
     def gemm_f32out(a, w, threads: int = 1) -> np.ndarray:
         K = a.shape[-1]
         M, N = a.size // K, w.shape[0]
@@ -188,4 +201,15 @@ class np64:  # noqa: N801
         r = a.astype(np.float64) @ w.astype(np.float64).T
         if bias is not None:
             r = r + bias.astype(np.float64)
+        return r
+
+    @staticmethod
+    def gemm_fused(a, w, bias, res1, res2, kind):
+        """The fused epilogues in float64, no intermediate rounding (the tolerance anchor)."""
+        from scipy.special import erf
+        r = np64.gemm(a, w, bias)
+        if kind in (1, 2):
+            r = res1.astype(np.float64) + r + res2.astype(np.float64)
+        elif kind == 3:
+            r = r * (0.5 + 0.5 * erf(r * 0.70710678118654757))
         return r

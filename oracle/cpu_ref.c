@@ -266,6 +266,55 @@ void oracle_gemm_f16_f32out(const f16* A, const f16* W, float* C, int64_t M, int
   }
 }
 
+/* ==========================================================================
+ * GEMM with the model's fused epilogues: fused_NT_matmul2_add1_add3_add3
+ * (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:163-200), ..._add3_cast (:202-246) and
+ * fused_NT_matmul3_add2_gelu (:248-318).  Every intermediate of those PrimFuncs is an fp16
+ * buffer, so every line below rounds to fp16, in the PrimFunc's operand order.
+ *   kind 0: C = mm (+ bias)                              (same as oracle_gemm_f16)
+ *   kind 1: C = (res1 + (mm + bias)) + res2              fp16 out
+ *   kind 2: the same, T.Cast("float32")                  fp32 out
+ *   kind 3: t = mm + bias; C = t * (0.5 + f16(f16(erf(f32(f16(t * f16(0.70710678...))))) * 0.5))
+ * mm is the fp32-accumulated product rounded once (acc_f16 = 1: the literal fp16 running sum).
+ * erf is libm's erff; the device uses its own erff, both well inside the fp16 rounding that
+ * follows except at rounding boundaries, which the parity tests allow for (1 fp16 ulp).
+ * Pinned by: numpy float16 arithmetic step by step, scipy.special.erf in float64 (tolerance),
+ * kind 1 with zero residuals == kind 0, gelu(0) = 0, gelu(x) -> x / 0 for large |x|, kind 2 ==
+ * widened kind 1.
+ * ======================================================================== */
+void oracle_gemm_f16_fused(const f16* A, const f16* W, const f16* bias, const f16* res1, const f16* res2,
+                           void* C, int64_t M, int64_t N, int64_t K, int kind, int acc_f16, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t ij = 0; ij < M * N; ++ij) {
+    const int64_t i = ij / N, j = ij % N;
+    const f16* a = A + i * K;
+    const f16* w = W + j * K;
+    f16 t;
+    if (acc_f16) {
+      f16 acc = 0;
+      for (int64_t k = 0; k < K; ++k) acc = f2h(h2f(acc) + h2f(f2h(h2f(a[k]) * h2f(w[k]))));
+      t = acc;
+    } else {
+      float acc = 0.f;
+      for (int64_t k = 0; k < K; ++k) acc = acc + h2f(a[k]) * h2f(w[k]);
+      t = f2h(acc);
+    }
+    if (bias) t = f2h(h2f(t) + h2f(bias[j]));                    /* T_add */
+    if (kind == 1 || kind == 2) {
+      t = f2h(h2f(res1[ij]) + h2f(t));                           /* T_add_1 = lv58 + T_add */
+      t = f2h(h2f(t) + h2f(res2[ij]));                           /* T_add_2 = T_add_1 + lv2 */
+    } else if (kind == 3) {
+      const f16 m = f2h(h2f(t) * h2f(f2h(0.70710678118654757f))); /* T_multiply */
+      const f16 e = f2h(erff(h2f(m)));                            /* compute .. compute_2 */
+      const f16 h = f2h(h2f(e) * 0.5f);                           /* T_multiply_1 */
+      const f16 g = f2h(0.5f + h2f(h));                           /* T_add_1 */
+      t = f2h(h2f(t) * h2f(g));                                   /* T_multiply_2 */
+    }
+    if (kind == 2) ((float*)C)[ij] = h2f(t);
+    else ((f16*)C)[ij] = t;
+  }
+}
+
 int oracle_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

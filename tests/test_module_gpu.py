@@ -18,7 +18,8 @@ def tuned(tmp_path_factory):
     mod = pf.module(pf.add("float16", 4096), pf.cast("float32", "float16", 4096), pf.rms_norm(4096),
                     pf.softmax_scores(32), pf.fused_layer_norm_cast1(2560),
                     pf.fused_NT_matmul_add_gemv(4096, 4096, bias=True), pf.fused_NT_matmul_add_gemm(4096, 4096, bias=True),
-                    upper_bound={"n": 1024})
+                    pf.fused_NT_matmul_add_add_add(2560, 2560), pf.fused_NT_matmul_add_add_add(2560, 2560, cast=True),
+                    pf.fused_NT_matmul_add_gelu(2560, 2560), upper_bound={"n": 1024})
     eng = Engine(topk=4, parallel_build=True, work_dir=work_dir)
     rt = eng.tune_module(mod, arch=MI355X(0, require_device=True), range_div_factor=256)
     return rt, work_dir
@@ -91,3 +92,28 @@ def test_time_evaluator_and_signature_errors(tuned):
         rt["add"](a, a.clone(), torch.empty(1, 64, 2560, dtype=torch.float16, device="cuda"))
     with pytest.raises(_lib.DtasError, match="overlaps"):
         rt["add"](a, a, a)
+
+
+def test_fused_epilogues_through_the_module(tuned, oracle):
+    rt, work_dir = tuned
+    again = load_module_from_file(work_dir)
+    rng = np.random.default_rng(4)
+    W = (rng.standard_normal((2560, 2560)) * 0.02).astype(np.float16)
+    bias = rng.uniform(-1, 1, 2560).astype(np.float16)
+    t = lambda a: torch.from_numpy(a).cuda()
+    for mod in (rt, again):
+        for n in (2, 300):
+            A = rng.standard_normal((1, n, 2560)).astype(np.float16)
+            r1 = rng.standard_normal((1, n, 2560)).astype(np.float16)
+            r2 = rng.standard_normal((1, n, 2560)).astype(np.float16)
+            out = torch.empty(1, n, 2560, dtype=torch.float16, device="cuda")
+            mod["fused_NT_matmul2_add1_add3_add3"](t(A), t(W), t(bias), t(r1), t(r2), out)
+            want = oracle.np64.gemm_fused(A[0], W, bias, r1[0], r2[0], 1)
+            scale = np.maximum(np.abs(want), np.maximum(np.abs(r1[0]), np.abs(r2[0])).astype(np.float64))
+            assert (np.abs(out.cpu().numpy()[0].astype(np.float64) - want) <= 4e-3 + 1e-2 * scale).all()
+            out32 = torch.empty(1, n, 2560, dtype=torch.float32, device="cuda")
+            mod["fused_NT_matmul2_add1_add3_add3_cast"](t(A), t(W), t(bias), t(r1), t(r2), out32)
+            assert torch.equal(out32, out.float())
+            mod["fused_NT_matmul3_add2_gelu"](t(A), t(W), t(bias), out)
+            want = oracle.np64.gemm_fused(A[0], W, bias, None, None, 3)
+            assert (np.abs(out.cpu().numpy()[0].astype(np.float64) - want) <= 4e-3 + 1e-2 * np.abs(want)).all()

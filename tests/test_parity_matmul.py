@@ -230,3 +230,75 @@ def test_gemm_split_k_errors():
     with pytest.raises(_lib.DtasError, match="split_k"):
         ops.gemm(dev(a), dev(w), None, torch.empty(64, 64, dtype=torch.float16, device="cuda"),
                  cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[64, 64, 64], split_k=17))
+
+
+def _fused_inputs(M, N, K, seed):
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    w = (rng.standard_normal((N, K)) * 0.03).astype(np.float16)
+    bias = rng.uniform(-1, 1, N).astype(np.float16)
+    r1 = rng.standard_normal((M, N)).astype(np.float16)
+    r2 = rng.standard_normal((M, N)).astype(np.float16)
+    return a, w, bias, r1, r2
+
+
+def _check_fused(got, want_oracle, want_f64, kind, r1=None, r2=None):
+    got = got.astype(np.float64)
+    assert np.isfinite(got).all()
+    # the fp16 rounding after every step acts at the magnitude of the intermediates: where the residuals
+    # cancel, the result is small but carries their rounding
+    scale = np.abs(want_f64)
+    if kind in (1, 2):
+        scale = np.maximum(scale, np.maximum(np.abs(r1.astype(np.float64)), np.abs(r2.astype(np.float64))))
+    assert (np.abs(got - want_f64) <= 4e-3 + RTOL * scale).all()
+    # against the oracle: the product may differ by an fp16 ulp (fp32 summation order), and each later
+    # fp16 rounding step can carry that over; gelu also sits on another erf implementation
+    want = want_oracle.astype(np.float64)
+    assert (np.abs(got - want) <= 2e-3 + 2.0 ** -8 * scale).all()
+    assert (got == want).mean() > 0.9
+
+
+FUSED_CONFIGS = [None,
+                 dict(variant=0, block=512, vec=8, tile=[256, 256, 64]),
+                 dict(variant=0, block=256, vec=8, tile=[256, 256, 64]),
+                 dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64]),
+                 dict(variant=0, block=256, vec=8, unroll=4, tile=[64, 64, 64], split_k=3),
+                 dict(variant=1, block=512, vec=8, unroll=4, tile=[80, 16, 32])]
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3])
+@pytest.mark.parametrize("which", range(len(FUSED_CONFIGS)))
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 7, 8), (70, 130, 136), (77, 2560, 520)])
+def test_gemm_fused_epilogues(oracle, kind, which, M, N, K):
+    # fused_NT_matmul2_add1_add3_add3(_cast) and fused_NT_matmul3_add2_gelu through every kernel family
+    a, w, bias, r1, r2 = _fused_inputs(M, N, K, M + N + K + kind)
+    res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+    out = Guarded((M, N), torch.float32 if kind == 2 else torch.float16)
+    c = None if FUSED_CONFIGS[which] is None else cfg(**FUSED_CONFIGS[which])
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c, epilogue=kind, res1=res[0], res2=res[1])
+    want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+    _check_fused(out.check(), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+
+
+@pytest.mark.parametrize("kind,N,K", [(1, 2560, 2560), (2, 2560, 2560), (3, 10240, 2560)])
+def test_gemm_fused_at_the_models_shapes(oracle, kind, N, K):
+    M = 300
+    a, w, bias, r1, r2 = _fused_inputs(M, N, K, kind)
+    res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+    out = Guarded((1, M, N), torch.float32 if kind == 2 else torch.float16)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, None, epilogue=kind, res1=res[0], res2=res[1])
+    want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+    _check_fused(out.check().reshape(M, N), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+
+
+def test_gemm_fused_argument_errors():
+    a, w, bias, r1, r2 = _fused_inputs(8, 16, 16, 1)
+    out = torch.empty(8, 16, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="residual"):
+        _lib.check(_lib.lib().dtas_gemm_f16_fused(dev(a).data_ptr(), dev(w).data_ptr(), None, None, None, out.data_ptr(),
+                                                  8, 16, 16, _lib.EPI_BIAS_ADD2, None, None), "fused")
+    with pytest.raises(_lib.DtasError, match="epilogue"):
+        _lib.check(_lib.lib().dtas_gemm_f16_fused(dev(a).data_ptr(), dev(w).data_ptr(), None, None, None, out.data_ptr(),
+                                                  8, 16, 16, 9, None, None), "fused")
+    with pytest.raises(ValueError, match="fp32 C"):
+        ops.gemm(dev(a), dev(w), None, out, None, epilogue=_lib.EPI_BIAS_ADD2_CAST_F32, res1=dev(r1), res2=dev(r2))
