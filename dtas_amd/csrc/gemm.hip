@@ -71,9 +71,16 @@ struct GemmEpilogue {
   const half_t* bias;  // [N] or NULL
   const half_t* res1;  // [M, N]: ADD2 kinds
   const half_t* res2;  // [M, N]: ADD2 kinds
-  int kind;            // enum dtas_epilogue
-  int out_f32;         // the output buffer holds fp32 (ADD2_CAST_F32)
+  int kind;            // enum dtas_epilogue, or kEpiScores
+  int out_f32;         // the output buffer holds fp32 (ADD2_CAST_F32, scores)
+  float scale;         // scores: the fp16 constant the product is multiplied by
+  // batched launches (grid.y = batch): element strides between consecutive problems
+  int64_t stride_a, stride_w, stride_c, stride_res;
 };
+
+// Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):
+// fp32(min(max(fp16(mm * fp16(scale)), -65504), mask)), mask = res1 shared by all heads.
+constexpr int kEpiScores = 100;
 
 __device__ __forceinline__ half_t round_h(float v) { return static_cast<half_t>(v); }
 
@@ -84,6 +91,10 @@ __device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& 
   if (ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32) {
     t = round_h(r1 + static_cast<float>(t));   // T_add_1 = lv58 + T_add
     t = round_h(static_cast<float>(t) + r2);   // T_add_2 = T_add_1 + lv2
+  } else if (ep.kind == kEpiScores) {
+    t = round_h(static_cast<float>(t) * ep.scale);                       // T_divide (a multiply by fp16(1/sqrt(d)))
+    t = round_h(fmaxf(static_cast<float>(t), -65504.f));                 // T_maximum
+    t = round_h(fminf(static_cast<float>(t), r1));                       // T_minimum with the mask
   } else if (ep.kind == DTAS_EPI_BIAS_GELU) {
     const float x = static_cast<float>(t);
     const half_t m = round_h(x * static_cast<float>(static_cast<half_t>(0.70710678118654757f)));
@@ -99,7 +110,7 @@ __device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& 
 __device__ __forceinline__ void finish(float acc, const GemmEpilogue& ep, void* C, int64_t row, int64_t col, int64_t N) {
   const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
   const half_t r = epilogue_value(round_h(acc), ep, ep.bias ? static_cast<float>(ep.bias[col]) : 0.f,
-                                  add2 ? static_cast<float>(ep.res1[row * N + col]) : 0.f,
+                                  add2 || ep.kind == kEpiScores ? static_cast<float>(ep.res1[row * N + col]) : 0.f,
                                   add2 ? static_cast<float>(ep.res2[row * N + col]) : 0.f);
   if (ep.out_f32) static_cast<float*>(C)[row * N + col] = static_cast<float>(r);
   else static_cast<half_t*>(C)[row * N + col] = r;
@@ -143,6 +154,14 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 
   const unsigned t = threadIdx.x, l = t & 63u;
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
+
+  // ---- which problem of a batched launch
+  const int64_t batch = blockIdx.y;
+  A += batch * ep.stride_a;
+  W += batch * ep.stride_w;
+  C = static_cast<char*>(C) + batch * ep.stride_c * (ep.out_f32 ? 4 : 2);
+  if (ep.res1) ep.res1 += batch * ep.stride_res;
+  if (ep.res2) ep.res2 += batch * ep.stride_res;
 
   // ---- which tile: XCD-contiguous order, then groups of 8 tile rows walked column-wise
   // nsplit > 1: nsplit consecutive workgroups (same XCD) share a tile and split its k tiles
@@ -627,10 +646,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const unsigned slot = l % kSlots, rsub = l / kSlots;
   const int64_t col = n0 + wn * WTN + slot * 4;
   const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const bool use_r1 = add2 || ep.kind == kEpiScores;
   // 8-byte accesses to C and the residuals (16-byte to an fp32 C) where extents and pointers allow
   const bool vec_store = (N % 4 == 0) && col + 3 < N &&
                          (reinterpret_cast<uintptr_t>(C) & (ep.out_f32 ? 15u : 7u)) == 0 &&
-                         (!add2 || ((reinterpret_cast<uintptr_t>(ep.res1) | reinterpret_cast<uintptr_t>(ep.res2)) & 7u) == 0);
+                         (!use_r1 || (reinterpret_cast<uintptr_t>(ep.res1) & 7u) == 0) &&
+                         (!add2 || (reinterpret_cast<uintptr_t>(ep.res2) & 7u) == 0);
   float bv[4] = {0.f, 0.f, 0.f, 0.f};
   if (ep.bias) {
 #pragma unroll
@@ -646,16 +667,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     const int64_t at = row * N + col;
     if (ep.kind != DTAS_EPI_BIAS || ep.bias) {  // "+ bias" etc. act on the sum already rounded to fp16
       f16x4 r1v = {}, r2v = {};
-      if (add2) {
+      if (use_r1) {
         if (vec_store) {
           r1v = *reinterpret_cast<const f16x4*>(ep.res1 + at);
-          r2v = *reinterpret_cast<const f16x4*>(ep.res2 + at);
+          if (add2) r2v = *reinterpret_cast<const f16x4*>(ep.res2 + at);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
             if (col + e < N) {
               r1v[e] = ep.res1[at + e];
-              r2v[e] = ep.res2[at + e];
+              if (add2) r2v[e] = ep.res2[at + e];
             }
         }
       }
@@ -849,7 +870,7 @@ int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsign
 
 template <int BM, int BN, int WM, int WN, int NS>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
-                int64_t K, int nsplit) {
+                int64_t K, int nsplit, int batch = 1) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
   const size_t tiles = static_cast<size_t>(tiles_m) * tiles_n;
   float* partials = nullptr;
@@ -859,7 +880,9 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
     if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
     if (split_workspace(bytes, tiles, &partials, &arrivals) != 0) return -1;
   }
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(static_cast<unsigned>(tiles * nsplit)), dim3(64 * WM * WN), 0,
+  if (batch > 1 && nsplit > 1) return fail("gemm: a batched launch cannot split K");
+  if (batch < 1 || batch > 65535) return fail("gemm: batch must be in [1, 65535], got %d", batch);
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(static_cast<unsigned>(tiles * nsplit), batch), dim3(64 * WM * WN), 0,
                      s, A, W, ep, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
@@ -954,7 +977,7 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   // one row of A with the plain epilogue is the decode GEMV: same PrimFunc shape, dedicated kernel
   if (!user && M == 1 && epilogue == DTAS_EPI_BIAS) return dtas_gemv_f16(A, W, bias, C, N, K, nullptr, stream);
   const GemmEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1),
-                           static_cast<const half_t*>(res2), epilogue, out_bytes == 4 ? 1 : 0};
+                           static_cast<const half_t*>(res2), epilogue, out_bytes == 4 ? 1 : 0, 0.f, 0, 0, 0, 0};
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMM_F16, M, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(A, 16) && aligned(W, 16);
   if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
@@ -1003,4 +1026,55 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
                                    : ns == 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
                                              : launch_mfma<64, 64, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
   return fail("gemm: no MFMA kernel for tile %dx%d", bm, bn);
+}
+
+extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const void* mask, void* out, int64_t heads,
+                                        int64_t n, int64_t m, int64_t d, float scale, const dtas_config* user,
+                                        void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (heads < 0 || n < 0 || m < 0 || d < 0)
+    return fail("attn_scores: negative extent heads=%lld n=%lld m=%lld d=%lld", (long long)heads, (long long)n, (long long)m, (long long)d);
+  if (heads == 0 || n == 0 || m == 0) return 0;
+  if (heads > 65535) return fail("attn_scores: at most 65535 heads, got %lld", (long long)heads);
+  if (d > 0 && (n > INT64_MAX / 8 / d / heads || m > INT64_MAX / 8 / d / heads)) return fail("attn_scores: extents overflow");
+  if (n > INT64_MAX / 8 / m / heads) return fail("attn_scores: extents overflow");
+  if (!Q || !Kmat || !mask || !out) return fail("attn_scores: NULL buffer");
+  if (d % 8 != 0 || !aligned(Q, 16) || !aligned(Kmat, 16))
+    return fail("attn_scores: the head dimension must be a multiple of 8 and Q, K 16-byte aligned (d=%lld)", (long long)d);
+  if (overlaps(out, heads * n * m * 4, Q, heads * n * d * 2) || overlaps(out, heads * n * m * 4, Kmat, heads * m * d * 2) ||
+      overlaps(out, heads * n * m * 4, mask, n * m * 2))
+    return fail("attn_scores: output overlaps an input");
+  dtas_config cfg;
+  if (user) {
+    cfg = *user;
+  } else {
+    // the fp32 scores (4*n*m bytes per head) are what this op moves: any tile does, take the largest
+    // that still gives every CU a workgroup
+    const int64_t t128 = heads * ceil_div(n, 128) * ceil_div(m, 128);
+    const int tile = t128 >= kNumCU ? 128 : 64;
+    cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {tile, tile, kBK}, 1, 0};
+  }
+  if (cfg.variant != DTAS_GEMM_MFMA || cfg.vec != 8) return fail("attn_scores: only the MFMA kernels (vec 8) serve this op");
+  if (cfg.split_k > 1) return fail("attn_scores: K is the head dimension, it is not split");
+  int64_t la[7];
+  if (describe_gemm(n, m, d, cfg, la) != 0) return -1;
+  GemmEpilogue ep = {nullptr, static_cast<const half_t*>(mask), nullptr, kEpiScores, 1,
+                     static_cast<float>(static_cast<half_t>(scale)), n * d, m * d, n * m, 0};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const half_t* a = static_cast<const half_t*>(Q);
+  const half_t* w = static_cast<const half_t*>(Kmat);
+  const int bm = cfg.tile[0], bn = cfg.tile[1], ns = cfg.unroll >= 2 ? cfg.unroll : 2, b = static_cast<int>(heads);
+  if (bm == 256 && bn == 256)
+    return cfg.block == 256 ? launch_mfma<256, 256, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b)
+                            : launch_mfma<256, 256, 2, 4, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  if (bm == 256 && bn == 128) return launch_mfma<256, 128, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  if (bm == 128 && bn == 256) return launch_mfma<128, 256, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  if (bm == 128 && bn == 128)
+    return ns >= 3 ? launch_mfma<128, 128, 2, 2, 3>(s, a, w, ep, out, n, m, d, 1, b) : launch_mfma<128, 128, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  if (bm == 64 && bn == 64)
+    return ns >= 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, ep, out, n, m, d, 1, b) : launch_mfma<64, 64, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
+  return fail("attn_scores: no MFMA kernel for tile %dx%d", bm, bn);
 }

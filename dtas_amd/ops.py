@@ -174,3 +174,21 @@ def gemm(A: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], C: torc
     else:
         check(lib().dtas_gemm_f16_fused(_p(A), _p(W), _p(bias), _p(res1), _p(res2), _p(C), M, N, K, epilogue, _cfg(cfg),
                                         _stream()), "dtas_gemm_f16_fused")
+
+
+def attn_scores(Q: torch.Tensor, K: torch.Tensor, mask: torch.Tensor, out: torch.Tensor, scale: float = 0.11179039301310044,
+                cfg: Optional[DtasConfig] = None) -> None:
+    """out[h,n,m] (fp32) = min(max(fp16(Q[h,n,:] . K[h,m,:]) * fp16(scale), -65504), mask[n,m]), each step an fp16
+    value: fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160).  Q (..., heads, n, d),
+    K (..., heads, m, d), mask (..., n, m) with leading extents of 1."""
+    _dev(Q, K, mask, out)
+    heads, n, d = Q.shape[-3:]
+    m = K.shape[-2]
+    if K.shape[-3:] != (heads, m, d) or mask.shape[-2:] != (n, m) or out.shape[-3:] != (heads, n, m):
+        raise ValueError("attn_scores: shape mismatch")
+    if Q.numel() != heads * n * d or K.numel() != heads * m * d or mask.numel() != n * m or out.numel() != heads * n * m:
+        raise ValueError("attn_scores: leading extents must be 1")
+    if any(t.dtype != torch.float16 for t in (Q, K, mask)) or out.dtype != torch.float32:
+        raise ValueError("attn_scores: expects fp16 inputs and an fp32 output")
+    check(lib().dtas_attn_scores_f16_f32(_p(Q), _p(K), _p(mask), _p(out), heads, n, m, d, scale, _cfg(cfg), _stream()),
+          "dtas_attn_scores_f16_f32")

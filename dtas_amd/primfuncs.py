@@ -157,6 +157,21 @@ def fused_NT_matmul_add_gelu(N: int = 10240, K: int = 2560, name: Optional[str] 
                     attrs={"tir.noalias": True, "epilogue": 3})
 
 
+def fused_NT_matmul_divide_maximum_minimum_cast(heads: int = 32, head_dim: int = 80,
+                                                scale: float = 0.11179039301310044, name: Optional[str] = None) -> PrimFunc:
+    """scores(1,heads,n,m) fp32 = min(max(fp16(Q(1,heads,n,d) . K(1,heads,m,d)^T) * fp16(scale), -65504), mask(1,1,n,m)):
+    fused_NT_matmul1_divide_maximum_minimum_cast2, before_dl.py:116-160; n and m dynamic."""
+    params = [Buffer("lv30", (1, heads, "n", head_dim), "float16"), Buffer("lv31", (1, heads, "m", head_dim), "float16"),
+              Buffer("lv5", (1, 1, "n", "m"), "float16"), Buffer("compute_intermediate", (1, heads, "n", "m"), "float32")]
+    blocks = [Block("NT_matmul", "SSSSR", ["lv30", "lv31"], ["NT_matmul_intermediate"]),
+              Block("T_divide", "SSSS", ["NT_matmul_intermediate"], ["T_divide_intermediate"]),
+              Block("T_maximum", "SSSS", ["T_divide_intermediate"], ["T_maximum_intermediate"]),
+              Block("T_minimum", "SSSS", ["T_maximum_intermediate", "lv5"], ["T_minimum_intermediate"]),
+              Block("compute", "SSSS", ["T_minimum_intermediate"], ["compute_intermediate"])]
+    return PrimFunc(name or "fused_NT_matmul1_divide_maximum_minimum_cast2", params, blocks, op="attn_scores",
+                    attrs={"tir.noalias": True, "scale": scale})
+
+
 def module(*funcs: PrimFunc, upper_bound: Optional[dict] = None) -> IRModule:
     """An IRModule of the given PrimFuncs; ``upper_bound`` is the ``tir_var_upper_bound`` attribute
     (tuning_test/tune_cast.py:26 uses {"m": 512, "n": 4096})."""

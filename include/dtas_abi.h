@@ -198,6 +198,15 @@ int dtas_gemm_f16_fused(const void* A, const void* W, const void* bias, const vo
                         const void* res2, void* C, int64_t M, int64_t N, int64_t K,
                         int32_t epilogue, const dtas_config* cfg, void* stream);
 
+/* ---- attention scores: fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160) ----
+ * out[h,i,j] = fp32(min(max(fp16(fp16(Q[h,i,:] . K[h,j,:]) * fp16(scale)), -65504), mask[i,j]))
+ * Q[heads,n,d], K[heads,m,d], mask[n,m] fp16 (shared by the heads), out[heads,n,m] fp32; n and m are the
+ * dynamic extents, d (80 in the model) a multiple of 8.  One batched launch over the heads on the MFMA
+ * kernels; cfg, when given, is a DTAS_GEMM_MFMA row for the per-head (n, m, d) problem. */
+int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, void* out, int64_t heads,
+                             int64_t n, int64_t m, int64_t d, float scale, const dtas_config* cfg,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif

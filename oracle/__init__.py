@@ -66,6 +66,7 @@ class _C:
                 "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
+                "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
             }
             for name, argtypes in sig.items():
                 fn = getattr(lib, name)
@@ -159,6 +160,16 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         return out
 
     @staticmethod
+    def attn_scores(q, k, mask, scale: float, acc_f16: bool = False, threads: int = 1) -> np.ndarray:
+        """fp32 scores[h,n,m] of fp16 q[h,n,d], k[h,m,d], mask[n,m]: scale, clamp at -65504, min with the mask."""
+        heads, n, d = q.shape
+        m = k.shape[1]
+        assert k.shape == (heads, m, d) and mask.shape == (n, m)
+        out = np.empty((heads, n, m), dtype=np.float32)
+        _C.lib().oracle_attn_scores_f16_f32(_ptr(q), _ptr(k), _ptr(mask), _ptr(out), heads, n, m, d, scale, int(acc_f16), threads)
+        return out
+
+    @staticmethod
     def gemm_f32out(a, w, threads: int = 1) -> np.ndarray:
         K = a.shape[-1]
         M, N = a.size // K, w.shape[0]
@@ -202,6 +213,11 @@ class np64:  # noqa: N801
         if bias is not None:
             r = r + bias.astype(np.float64)
         return r
+
+    @staticmethod
+    def attn_scores(q, k, mask, scale):
+        s_ = np.einsum("hnd,hmd->hnm", q.astype(np.float64), k.astype(np.float64)) * float(np.float16(scale))
+        return np.minimum(np.maximum(s_, -65504.0), mask.astype(np.float64)[None])
 
     @staticmethod
     def gemm_fused(a, w, bias, res1, res2, kind):

@@ -315,6 +315,44 @@ void oracle_gemm_f16_fused(const f16* A, const f16* W, const f16* bias, const f1
   }
 }
 
+/* ==========================================================================
+ * Attention scores: fused_NT_matmul1_divide_maximum_minimum_cast2
+ * (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:116-160).
+ *   NT_matmul[h,i,j] = sum_k Q[h,i,k] * K[h,j,k]            (fp16 buffer)
+ *   T_divide  = NT_matmul * T.float16(0.11179...)            (a multiply by the fp16 constant)
+ *   T_maximum = max(T_divide, T.float16(-65504))
+ *   T_minimum = min(T_maximum, mask[0,0,i,j])
+ *   compute   = T.Cast("float32", T_minimum)
+ * The product is accumulated in fp32 and rounded once (acc_f16 = 1: the literal fp16 running sum).
+ * Pinned by: numpy float16 arithmetic step by step (bit-exact), the float64 closed form, a mask of
+ * +65504 (no effect) / -65504 (everything masked) / a causal triangle, heads independent, -inf
+ * products clamped to -65504.
+ * ======================================================================== */
+void oracle_attn_scores_f16_f32(const f16* Q, const f16* Kmat, const f16* mask, float* out, int64_t heads, int64_t n,
+                                int64_t m, int64_t d, float scale, int acc_f16, int nthreads) {
+  const f16 scale_h = f2h(scale);
+  OMP_FOR(nthreads)
+  for (int64_t idx = 0; idx < heads * n * m; ++idx) {
+    const int64_t h = idx / (n * m), i = (idx / m) % n, j = idx % m;
+    const f16* q = Q + (h * n + i) * d;
+    const f16* k = Kmat + (h * m + j) * d;
+    f16 t;
+    if (acc_f16) {
+      f16 acc = 0;
+      for (int64_t e = 0; e < d; ++e) acc = f2h(h2f(acc) + h2f(f2h(h2f(q[e]) * h2f(k[e]))));
+      t = acc;
+    } else {
+      float acc = 0.f;
+      for (int64_t e = 0; e < d; ++e) acc = acc + h2f(q[e]) * h2f(k[e]);
+      t = f2h(acc);
+    }
+    t = f2h(h2f(t) * h2f(scale_h));
+    t = f2h(fmaxf(h2f(t), -65504.f));
+    t = f2h(fminf(h2f(t), h2f(mask[i * m + j])));
+    out[idx] = h2f(t);
+  }
+}
+
 int oracle_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();
