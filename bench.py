@@ -107,6 +107,28 @@ def _workload(name: str, n: int, extra=None):
         make = lambda s: (normal((n, K), s), wt, empty((n, N)))
         return (make, lambda b: call(L.dtas_gemm_f16, P(b[0]), P(b[1]), None, P(b[2]), n, N, K, None, stream),
                 2 * (n * K + N * K + n * N), 2 * n * N * K)
+    if name == "attn_scores_f16_f32":
+        # fused_NT_matmul1_divide_maximum_minimum_cast2: 32 heads of 80, n = m; the fp32 scores dominate the bytes
+        heads, d = 32, 80
+        mask = torch.full((n, n), 65504.0, dtype=torch.float16, device="cuda").tril_().add_(
+            torch.full((n, n), -65504.0, dtype=torch.float16, device="cuda").triu_(1))
+        make = lambda s: (normal((heads, n, d), s), normal((heads, n, d), s + 50), mask, empty((heads, n, n), torch.float32))
+        return (make, lambda b: call(L.dtas_attn_scores_f16_f32, P(b[0]), P(b[1]), P(b[2]), P(b[3]), heads, n, n, d,
+                                     0.11179039301310044, None, stream),
+                2 * 2 * heads * n * d + 2 * n * n + 4 * heads * n * n, 2 * heads * n * n * d)
+    if name in ("gemm_add2_f16", "gemm_gelu_f16"):
+        # fused_NT_matmul2_add1_add3_add3 at (N, K) = (2560, 2560); fused_NT_matmul3_add2_gelu at (10240, 2560)
+        N, K = extra
+        wt, bias = normal((N, K), 100, 0.02), uniform((N,), 101)
+        if name == "gemm_add2_f16":
+            make = lambda s: (normal((n, K), s), wt, bias, normal((n, N), s + 1), normal((n, N), s + 2), empty((n, N)))
+            return (make, lambda b: call(L.dtas_gemm_f16_fused, P(b[0]), P(b[1]), P(b[2]), P(b[3]), P(b[4]), P(b[5]), n, N, K,
+                                         _lib.EPI_BIAS_ADD2, None, stream),
+                    2 * (n * K + N * K + 3 * n * N + N), 2 * n * N * K)
+        make = lambda s: (normal((n, K), s), wt, bias, empty((n, N)))
+        return (make, lambda b: call(L.dtas_gemm_f16_fused, P(b[0]), P(b[1]), P(b[2]), None, None, P(b[3]), n, N, K,
+                                     _lib.EPI_BIAS_GELU, None, stream),
+                2 * (n * K + N * K + n * N + N), 2 * n * N * K)
     raise ValueError(f"unknown workload {name}")
 
 
@@ -170,7 +192,7 @@ def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool =
            "bytes": nbytes, "flops": flops, "pool": len(pool), "gbs": nbytes / per_launch / 1e9}
     if extra:
         out["NK"] = list(extra)
-    if flops and name == "gemm_f16":
+    if flops and name in ("gemm_f16", "gemm_add2_f16", "gemm_gelu_f16", "attn_scores_f16_f32"):
         out["tflops"] = flops / per_launch / 1e12
         hbm_bound_s = nbytes / (HBM_PEAK_GBS * 1e9)
         mfma_bound_s = flops / (MFMA_FP16_PEAK_TFLOPS * 1e12)
@@ -248,6 +270,12 @@ def sweep(steps: int, warmup: int) -> list:
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
+    # the model's own fused shapes (dolly-v2-3b: hidden 2560, 32 heads of 80)
+    for m in (16, 256, 2048):
+        rows.append(measure("gemm_add2_f16", m, (2560, 2560), max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure("gemm_gelu_f16", m, (10240, 2560), max(10, steps // 2), max(2, warmup // 2)))
+    for n in (128, 1024, 2048):
+        rows.append(measure("attn_scores_f16_f32", n, None, max(10, steps // 2), max(2, warmup // 2)))
     return rows
 
 
@@ -268,8 +296,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
-                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | "
-                         "gemv_f16 | gemm_f16")
+                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | "
+                         "gemv_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last four take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -294,7 +322,7 @@ def main() -> int:
         print(_lib.last_error(), file=sys.stderr)
         return 2
 
-    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemm_f16") else None
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemm_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
     info = None

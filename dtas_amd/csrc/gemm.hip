@@ -40,6 +40,7 @@
 #include "dtas_host.h"
 
 #include <mutex>
+#include <type_traits>
 
 namespace dtas {
 namespace {
@@ -84,18 +85,21 @@ constexpr int kEpiScores = 100;
 
 __device__ __forceinline__ half_t round_h(float v) { return static_cast<half_t>(v); }
 
-// mm: the product already rounded to fp16.  Returns the fp16 result (the cast kind widens it).
-__device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& ep, float bias_j, float r1, float r2) {
+// mm: the product already rounded to fp16.  Returns the fp16 result (the cast kinds widen it).
+// KIND is a compile-time constant where the caller has dispatched on it (the tile epilogue: one
+// specialised store loop per kind keeps erf and the residual handling out of the plain path).
+template <int KIND>
+__device__ __forceinline__ half_t epilogue_value_k(half_t mm, bool has_bias, float scale, float bias_j, float r1, float r2) {
   half_t t = mm;
-  if (ep.bias) t = round_h(static_cast<float>(t) + bias_j);
-  if (ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32) {
+  if (has_bias) t = round_h(static_cast<float>(t) + bias_j);
+  if (KIND == DTAS_EPI_BIAS_ADD2 || KIND == DTAS_EPI_BIAS_ADD2_CAST_F32) {
     t = round_h(r1 + static_cast<float>(t));   // T_add_1 = lv58 + T_add
     t = round_h(static_cast<float>(t) + r2);   // T_add_2 = T_add_1 + lv2
-  } else if (ep.kind == kEpiScores) {
-    t = round_h(static_cast<float>(t) * ep.scale);                       // T_divide (a multiply by fp16(1/sqrt(d)))
+  } else if (KIND == kEpiScores) {
+    t = round_h(static_cast<float>(t) * scale);                          // T_divide (a multiply by fp16(1/sqrt(d)))
     t = round_h(fmaxf(static_cast<float>(t), -65504.f));                 // T_maximum
     t = round_h(fminf(static_cast<float>(t), r1));                       // T_minimum with the mask
-  } else if (ep.kind == DTAS_EPI_BIAS_GELU) {
+  } else if (KIND == DTAS_EPI_BIAS_GELU) {
     const float x = static_cast<float>(t);
     const half_t m = round_h(x * static_cast<float>(static_cast<half_t>(0.70710678118654757f)));
     const half_t e = round_h(erff(static_cast<float>(m)));
@@ -104,6 +108,17 @@ __device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& 
     t = round_h(x * static_cast<float>(a));
   }
   return t;
+}
+
+__device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& ep, float bias_j, float r1, float r2) {
+  const bool hb = ep.bias != nullptr;
+  switch (ep.kind) {
+    case DTAS_EPI_BIAS_ADD2:
+    case DTAS_EPI_BIAS_ADD2_CAST_F32: return epilogue_value_k<DTAS_EPI_BIAS_ADD2>(mm, hb, ep.scale, bias_j, r1, r2);
+    case DTAS_EPI_BIAS_GELU: return epilogue_value_k<DTAS_EPI_BIAS_GELU>(mm, hb, ep.scale, bias_j, r1, r2);
+    case kEpiScores: return epilogue_value_k<kEpiScores>(mm, hb, ep.scale, bias_j, r1, r2);
+    default: return epilogue_value_k<DTAS_EPI_BIAS>(mm, hb, ep.scale, bias_j, r1, r2);
+  }
 }
 
 // one element, any alignment (skinny and element-access kernels)
@@ -658,52 +673,86 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     for (int e = 0; e < 4; ++e)
       if (col + e < N) bv[e] = static_cast<float>(ep.bias[col + e]);
   }
+  // one store loop per epilogue kind, chosen once (kind is uniform)
+  auto store_tile = [&](auto kind_tag) {
+    constexpr int KIND = decltype(kind_tag)::value;
+    constexpr bool kAdd2 = KIND == DTAS_EPI_BIAS_ADD2 || KIND == DTAS_EPI_BIAS_ADD2_CAST_F32;
+    constexpr bool kUseR1 = kAdd2 || KIND == kEpiScores;
+    constexpr bool kOutF32 = KIND == DTAS_EPI_BIAS_ADD2_CAST_F32 || KIND == kEpiScores;
+    const bool has_bias = ep.bias != nullptr;
+    // passes in groups of G: the group's residual / mask vectors are requested together, before the
+    // first of them is needed (one at a time, every pass would wait out a memory round trip)
+    constexpr int kPasses = WTM / kRowsPerPass;
+    // as many as the registers hold (two per vector): all 32 for one operand, 16 for two; erf's code
+    // is long, so its loop body stays small
+    constexpr int kWant = KIND == DTAS_EPI_BIAS_GELU ? 2 : kAdd2 ? 16 : kUseR1 ? 32 : 4;
+    constexpr int G = kPasses % kWant == 0 ? kWant : (kPasses % 8 == 0 ? 8 : (kPasses % 4 == 0 ? 4 : 1));
+#pragma unroll 1
+    for (int p0 = 0; p0 < kPasses; p0 += G) {
+      f16x4 r1v[G] = {}, r2v[G] = {};
+      if (kUseR1) {
 #pragma unroll
-  for (int p = 0; p < WTM / kRowsPerPass; ++p) {
-    const unsigned m = p * kRowsPerPass + rsub;
-    f16x4 hv = *reinterpret_cast<const f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8));
-    const int64_t row = m0 + wm * WTM + m;
-    if (row >= M) continue;
-    const int64_t at = row * N + col;
-    if (ep.kind != DTAS_EPI_BIAS || ep.bias) {  // "+ bias" etc. act on the sum already rounded to fp16
-      f16x4 r1v = {}, r2v = {};
-      if (use_r1) {
-        if (vec_store) {
-          r1v = *reinterpret_cast<const f16x4*>(ep.res1 + at);
-          if (add2) r2v = *reinterpret_cast<const f16x4*>(ep.res2 + at);
-        } else {
+        for (int u = 0; u < G; ++u) {
+          const int64_t row = m0 + wm * WTM + (p0 + u) * kRowsPerPass + rsub;
+          if (row >= M) continue;
+          const int64_t at = row * N + col;
+          if (vec_store) {
+            r1v[u] = *reinterpret_cast<const f16x4*>(ep.res1 + at);
+            if (kAdd2) r2v[u] = *reinterpret_cast<const f16x4*>(ep.res2 + at);
+          } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (col + e < N) {
-              r1v[e] = ep.res1[at + e];
-              if (add2) r2v[e] = ep.res2[at + e];
-            }
+            for (int e = 0; e < 4; ++e)
+              if (col + e < N) {
+                r1v[u][e] = ep.res1[at + e];
+                if (kAdd2) r2v[u][e] = ep.res2[at + e];
+              }
+          }
         }
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        hv[e] = epilogue_value(hv[e], ep, bv[e], static_cast<float>(r1v[e]), static_cast<float>(r2v[e]));
-    }
-    if (ep.out_f32) {
-      float* dst = static_cast<float*>(C) + at;
-      if (vec_store) {
-        *reinterpret_cast<f32x4v*>(dst) = f32x4v{static_cast<float>(hv[0]), static_cast<float>(hv[1]),
-                                                 static_cast<float>(hv[2]), static_cast<float>(hv[3])};
-      } else {
+      for (int u = 0; u < G; ++u) {
+        const unsigned m = (p0 + u) * kRowsPerPass + rsub;
+        f16x4 hv = *reinterpret_cast<const f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8));
+        const int64_t row = m0 + wm * WTM + m;
+        if (row >= M) continue;
+        const int64_t at = row * N + col;
+        if (KIND != DTAS_EPI_BIAS || has_bias) {  // "+ bias" etc. act on the sum already rounded to fp16
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (col + e < N) dst[e] = static_cast<float>(hv[e]);
-      }
-    } else {
-      half_t* dst = static_cast<half_t*>(C) + at;
-      if (vec_store) {
-        *reinterpret_cast<f16x4*>(dst) = hv;
-      } else {
+          for (int e = 0; e < 4; ++e)
+            hv[e] = epilogue_value_k<KIND>(hv[e], has_bias, ep.scale, bv[e], static_cast<float>(r1v[u][e]),
+                                           static_cast<float>(r2v[u][e]));
+        }
+        if (kOutF32) {
+          float* dst = static_cast<float*>(C) + at;
+          if (vec_store) {
+            const f32x4v wide = {static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]),
+                                 static_cast<float>(hv[3])};
+            if (KIND == kEpiScores) __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));  // 4*heads*n*m bytes: streamed
+            else *reinterpret_cast<f32x4v*>(dst) = wide;
+          } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (col + e < N) dst[e] = hv[e];
+            for (int e = 0; e < 4; ++e)
+              if (col + e < N) dst[e] = static_cast<float>(hv[e]);
+          }
+        } else {
+          half_t* dst = static_cast<half_t*>(C) + at;
+          if (vec_store) {
+            *reinterpret_cast<f16x4*>(dst) = hv;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (col + e < N) dst[e] = hv[e];
+          }
+        }
       }
     }
+  };
+  switch (ep.kind) {
+    case DTAS_EPI_BIAS_ADD2: store_tile(std::integral_constant<int, DTAS_EPI_BIAS_ADD2>{}); break;
+    case DTAS_EPI_BIAS_ADD2_CAST_F32: store_tile(std::integral_constant<int, DTAS_EPI_BIAS_ADD2_CAST_F32>{}); break;
+    case DTAS_EPI_BIAS_GELU: store_tile(std::integral_constant<int, DTAS_EPI_BIAS_GELU>{}); break;
+    case kEpiScores: store_tile(std::integral_constant<int, kEpiScores>{}); break;
+    default: store_tile(std::integral_constant<int, DTAS_EPI_BIAS>{}); break;
   }
 }
 
@@ -1049,11 +1098,12 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   if (user) {
     cfg = *user;
   } else {
-    // the fp32 scores (4*n*m bytes per head) are what this op moves: any tile does, take the largest
-    // that still gives every CU a workgroup
+    // the fp32 scores (4*n*m bytes per head) are what this op moves, and with two k tiles a workgroup
+    // is mostly latency: measured best are 64x64 while 128x128 tiles do not give every CU a
+    // workgroup, 128x128 up to ~1M scores per head, 128x64 (three workgroups per CU) beyond
     const int64_t t128 = heads * ceil_div(n, 128) * ceil_div(m, 128);
-    const int tile = t128 >= kNumCU ? 128 : 64;
-    cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {tile, tile, kBK}, 1, 0};
+    const int bm = t128 >= kNumCU ? 128 : 64, bn = t128 < kNumCU ? 64 : (n * m >= (int64_t{1} << 20) ? 64 : 128);
+    cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {bm, bn, kBK}, 1, 0};
   }
   if (cfg.variant != DTAS_GEMM_MFMA || cfg.vec != 8) return fail("attn_scores: only the MFMA kernels (vec 8) serve this op");
   if (cfg.split_k > 1) return fail("attn_scores: K is the head dimension, it is not split");
