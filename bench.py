@@ -116,6 +116,13 @@ def _workload(name: str, n: int, extra=None):
         return (make, lambda b: call(L.dtas_attn_scores_f16_f32, P(b[0]), P(b[1]), P(b[2]), P(b[3]), heads, n, n, d,
                                      0.11179039301310044, None, stream),
                 2 * 2 * heads * n * d + 2 * n * n + 4 * heads * n * n, 2 * heads * n * n * d)
+    if name == "attn_pv_f16":
+        # matmul8 (n = m) / matmul10 (extra = (1, m): one query row): 32 heads of 80; the probabilities dominate the bytes
+        heads, d = 32, 80
+        rows, m = (extra if extra else (n, n))
+        make = lambda s: (uniform((heads, rows, m), s), normal((heads, m, d), s + 50), empty((heads, rows, d)))
+        return (make, lambda b: call(L.dtas_attn_pv_f16, P(b[0]), P(b[1]), P(b[2]), heads, rows, m, d, None, stream),
+                2 * heads * (rows * m + m * d + rows * d), 2 * heads * rows * m * d)
     if name in ("gemm_add2_f16", "gemm_gelu_f16"):
         # fused_NT_matmul2_add1_add3_add3 at (N, K) = (2560, 2560); fused_NT_matmul3_add2_gelu at (10240, 2560)
         N, K = extra
@@ -192,7 +199,7 @@ def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool =
            "bytes": nbytes, "flops": flops, "pool": len(pool), "gbs": nbytes / per_launch / 1e9}
     if extra:
         out["NK"] = list(extra)
-    if flops and name in ("gemm_f16", "gemm_add2_f16", "gemm_gelu_f16", "attn_scores_f16_f32"):
+    if flops and name in ("gemm_f16", "gemm_add2_f16", "gemm_gelu_f16", "attn_scores_f16_f32", "attn_pv_f16"):
         out["tflops"] = flops / per_launch / 1e12
         hbm_bound_s = nbytes / (HBM_PEAK_GBS * 1e9)
         mfma_bound_s = flops / (MFMA_FP16_PEAK_TFLOPS * 1e12)
@@ -276,6 +283,8 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("gemm_gelu_f16", m, (10240, 2560), max(10, steps // 2), max(2, warmup // 2)))
     for n in (128, 1024, 2048):
         rows.append(measure("attn_scores_f16_f32", n, None, max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure("attn_pv_f16", n, None, max(10, steps // 2), max(2, warmup // 2)))
+    rows.append(measure("attn_pv_f16", 1, (1, 2048), steps, warmup))      # matmul10: decoding against 2048 keys
     return rows
 
 
@@ -296,7 +305,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
-                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | "
+                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
                          "gemv_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last four take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")

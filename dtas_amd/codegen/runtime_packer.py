@@ -128,6 +128,8 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.softmax(tensors[0], tensors[1], abi)
     elif op == "attn_scores":                                                 # Q, K, mask, out
         ops.attn_scores(tensors[0], tensors[1], tensors[2], tensors[3], func.attrs.get("scale", 0.11179039301310044), abi)
+    elif op == "attn_pv":                                                     # P, V, out
+        ops.attn_pv(tensors[0], tensors[1], tensors[2], abi)
     elif op == "matmul":
         epilogue = int(func.attrs.get("epilogue", 0))
         if epilogue in (_lib.EPI_BIAS_ADD2, _lib.EPI_BIAS_ADD2_CAST_F32):   # A, W, bias, res1, res2, out

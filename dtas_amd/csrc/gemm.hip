@@ -146,7 +146,9 @@ constexpr int waitcnt_imm(int v) { return 0x0070 | (v & 15) | ((v >> 4) << 14); 
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-template <int BM, int BN, int WM, int WN, int NS>
+// WT: W is given k-major ([K][N], N contiguous -- the V operand of attention's P.V); its tiles are
+// then transposed on the way into the LDS (two stages, 4 wavefronts only).
+template <int BM, int BN, int WM, int WN, int NS, bool WT = false>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ W,
                                                                  GemmEpilogue ep, void* __restrict__ C, int64_t M,
@@ -162,6 +164,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
   static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
+  static_assert(!WT || (NS == 2 && NW == 4), "the transposing W path is written for two stages and 4 wavefronts");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
   static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
   constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
@@ -236,10 +239,60 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
     for (int i = 0; i < LA; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, 0);
+    if constexpr (!WT) {
 #pragma unroll
-    for (int i = 0; i < LB; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
+      for (int i = 0; i < LB; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
+    }
   };
+
+  // ---- k-major W.  A tile is 64 k x BN columns of W[K][N]; an item is 8 columns of two
+  // consecutive k rows: a lane loads the two 16-byte pieces into registers (wt_load, with tile
+  // kt's other loads) and later (wt_commit, once the stage is free) stores eight 4-byte words
+  // {W[k][c], W[k+1][c]} to where the row-major path would have put them.  Item -> lane is chosen
+  // so that a wavefront's 64 stores hit 64 distinct banks: 32 k pairs x 2 adjacent column chunks.
+  // Columns past N are never written: the W halves of both stages are zeroed once, up front.
+  constexpr int kWtItems = WT ? 4 * BN / (64 * NW) : 1;
+  u32x4 wt_reg[kWtItems][2];
+  auto wt_item = [&](int i, unsigned& cc, unsigned& kp) {
+    const unsigned item = t + i * 64 * NW;
+    cc = ((item >> 6) << 1) | (item & 1u);
+    kp = (item >> 1) & 31u;
+  };
+  auto wt_load = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < kWtItems; ++i) {
+      unsigned cc, kp;
+      wt_item(i, cc, kp);
+      const int64_t col = n0 + cc * 8, k = static_cast<int64_t>(kt0 + kt) * kBK + 2 * kp;
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      wt_reg[i][0] = (col < N && k < K) ? *reinterpret_cast<const u32x4*>(W + k * N + col) : zero;
+      wt_reg[i][1] = (col < N && k + 1 < K) ? *reinterpret_cast<const u32x4*>(W + (k + 1) * N + col) : zero;
+    }
+  };
+  auto wt_commit = [&](int kt) {
+    char* base = lds + (kt % NS) * kStage + kABytes;
+#pragma unroll
+    for (int i = 0; i < kWtItems; ++i) {
+      unsigned cc, kp;
+      wt_item(i, cc, kp);
+      if (n0 + cc * 8 >= N) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const unsigned a = wt_reg[i][0][j], b = wt_reg[i][1][j];
+        const unsigned r = cc * 8 + 2 * j;
+        *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r, kp >> 2) + (kp & 3u) * 4u) = (a & 0xffffu) | (b << 16);
+        *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r + 1, kp >> 2) + (kp & 3u) * 4u) = (a >> 16) | (b & 0xffff0000u);
+      }
+    }
+  };
+  if constexpr (WT) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int s = 0; s < NS; ++s)
+      for (unsigned at = t * 16u; at < static_cast<unsigned>(BN * kRowBytes); at += 64 * NW * 16)
+        *reinterpret_cast<u32x4*>(lds + s * kStage + kABytes + at) = zero;
+    __syncthreads();
+  }
 
   f16x8 fa[2][MT], fb[2][NT];
   auto read_a = [&](int set, int i, const char* stage, int ks) {
@@ -551,11 +604,17 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     for (; kt < ktiles; ++kt) k_tile(kt, false);
   } else {
   // two stages: tile 0 resident, tile 1 in flight, fragments of (tile 0, step 0) in registers
-  if (ktiles > 0) fetch(0);
+  if (ktiles > 0) {
+    fetch(0);
+    if constexpr (WT) { wt_load(0); wt_commit(0); }
+  }
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
   DTAS_SCHED_FENCE();
-  if (1 < ktiles) fetch(1);
+  if (1 < ktiles) {
+    fetch(1);
+    if constexpr (WT) wt_load(1);
+  }
   if (ktiles > 0) {
 #pragma unroll
     for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
@@ -569,10 +628,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     step(0, cur, 1, true);
     step(1, cur, 2, true);
     step(0, cur, 3, true);
+    if constexpr (WT) {
+      if (kt + 1 < ktiles) wt_commit(kt + 1);  // its stage was tile kt-1's: free since the last barrier
+    }
     __builtin_amdgcn_s_waitcnt(0x0070);  // tile kt+1 has landed
     __builtin_amdgcn_s_barrier();        // ... and every wavefront has finished reading tile kt
     DTAS_SCHED_FENCE();
-    if (kt + NS < ktiles) fetch(kt + NS);  // into the stage tile kt occupied
+    if (kt + NS < ktiles) {  // into the stage tile kt occupied
+      fetch(kt + NS);
+      if constexpr (WT) wt_load(kt + NS);
+    }
     DTAS_SCHED_FENCE();
     step(1, nxt, 0, kt + 1 < ktiles);
   }
@@ -853,18 +918,83 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
   }
 }
 
-// Any K and alignment: one thread per element of C.
+// Any K and alignment: one thread per element of C.  blockIdx.y = problem of a batched launch;
+// w_kmajor: W is [K][N] instead of [N][K].
 __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
                                                           GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
-                                                          int64_t K) {
+                                                          int64_t K, bool w_kmajor) {
+  const int64_t batch = blockIdx.y;
+  A += batch * ep.stride_a;
+  W += batch * ep.stride_w;
+  C = static_cast<char*>(C) + batch * ep.stride_c * (ep.out_f32 ? 4 : 2);
+  if (ep.res1) ep.res1 += batch * ep.stride_res;
+  if (ep.res2) ep.res2 += batch * ep.stride_res;
   const int64_t total = M * N;
   for (int64_t ij = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; ij < total;
        ij += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const half_t* a = A + (ij / N) * K;
-    const half_t* w = W + (ij % N) * K;
+    const half_t* w = w_kmajor ? W + ij % N : W + (ij % N) * K;
+    const int64_t wk = w_kmajor ? N : 1;
     float acc = 0.f;
-    for (int64_t k = 0; k < K; ++k) acc += static_cast<float>(a[k]) * static_cast<float>(w[k]);
+    for (int64_t k = 0; k < K; ++k) acc += static_cast<float>(a[k]) * static_cast<float>(w[k * wk]);
     finish(acc, ep, C, ij / N, ij % N, N);
+  }
+}
+
+// P.V for a handful of query rows (decoding): out[h, r, :] = sum_k P[h, r, k] * V[h, k, :].
+// Workgroup = (head, 8 columns of V, R rows of P); thread t takes k = t, t + 256, ...: a 16-byte piece
+// of V's row k and P[h, r, k] of each row, eight k at a time with every load requested before the
+// first is used -- with m <= 2048 that is the whole job in one memory round trip, and round trips
+// are what this op costs.  The pieces of one row of V are 16 bytes out of every 2*d, so the d/8
+// workgroups of a head are given consecutive ids on one XCD and share the lines in its L2.
+template <int R>
+__global__ void __launch_bounds__(256) attn_pv_rows_kernel(const half_t* __restrict__ P, const half_t* __restrict__ V,
+                                                           half_t* __restrict__ out, int64_t n, int64_t m, int64_t d) {
+  __shared__ float part[4][R][8];
+  const unsigned chunks = static_cast<unsigned>(d / 8);
+  const unsigned id = xcd_contiguous_id(blockIdx.x, gridDim.x);
+  const unsigned h = id / chunks, cc = id % chunks, t = threadIdx.x;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * R;
+  const int rows = n - r0 < R ? static_cast<int>(n - r0) : R;
+  const half_t* p = P + (static_cast<int64_t>(h) * n + r0) * m;
+  const half_t* v = V + static_cast<int64_t>(h) * m * d + cc * 8;
+  float acc[R][8];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+  for (int64_t kb = t; kb < m; kb += 8 * 256) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    u32x4 vraw[8];
+    half_t pk[8][R];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t k = kb + u * 256;
+      vraw[u] = k < m ? *reinterpret_cast<const u32x4*>(v + k * d) : zero;  // (cached: the head's other workgroups want the line too)
+#pragma unroll
+      for (int r = 0; r < R; ++r) pk[u][r] = (k < m && r < rows) ? p[r * m + k] : static_cast<half_t>(0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const f16x8 vv = __builtin_bit_cast(f16x8, vraw[u]);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[r][e] += static_cast<float>(pk[u][r]) * static_cast<float>(vv[e]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float sum = wave_sum(acc[r][e]);
+      if ((t & 63u) == 0) part[t >> 6][r][e] = sum;
+    }
+  __syncthreads();
+  if (t < static_cast<unsigned>(rows) * 8u) {
+    const unsigned r = t / 8, e = t % 8;
+    out[(static_cast<int64_t>(h) * n + r0 + r) * d + cc * 8 + e] =
+        static_cast<half_t>(part[0][r][e] + part[1][r][e] + part[2][r][e] + part[3][r][e]);
   }
 }
 
@@ -917,7 +1047,7 @@ int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsign
   return 0;
 }
 
-template <int BM, int BN, int WM, int WN, int NS>
+template <int BM, int BN, int WM, int WN, int NS, bool WT = false>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
                 int64_t K, int nsplit, int batch = 1) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
@@ -931,7 +1061,7 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   }
   if (batch > 1 && nsplit > 1) return fail("gemm: a batched launch cannot split K");
   if (batch < 1 || batch > 65535) return fail("gemm: batch must be in [1, 65535], got %d", batch);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS>), dim3(static_cast<unsigned>(tiles * nsplit), batch), dim3(64 * WM * WN), 0,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT>), dim3(static_cast<unsigned>(tiles * nsplit), batch), dim3(64 * WM * WN), 0,
                      s, A, W, ep, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
@@ -1038,7 +1168,7 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   const GemmEpilogue& b = ep;
   void* c = C;
   if (cfg.vec == 1) {
-    hipLaunchKernelGGL(gemm_scalar_kernel, dim3(static_cast<unsigned>(la[0])), dim3(256), 0, s, a, w, b, c, M, N, K);
+    hipLaunchKernelGGL(gemm_scalar_kernel, dim3(static_cast<unsigned>(la[0])), dim3(256), 0, s, a, w, b, c, M, N, K, false);
     return check_launch("gemm");
   }
   if (cfg.variant == DTAS_GEMM_SKINNY) {
@@ -1127,4 +1257,75 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   if (bm == 64 && bn == 64)
     return ns >= 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, ep, out, n, m, d, 1, b) : launch_mfma<64, 64, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
   return fail("attn_scores: no MFMA kernel for tile %dx%d", bm, bn);
+}
+
+extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int64_t n, int64_t m, int64_t d,
+                                const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (heads < 0 || n < 0 || m < 0 || d < 0)
+    return fail("attn_pv: negative extent heads=%lld n=%lld m=%lld d=%lld", (long long)heads, (long long)n, (long long)m, (long long)d);
+  if (heads == 0 || n == 0 || d == 0) return 0;
+  if (heads > 65535) return fail("attn_pv: at most 65535 heads, got %lld", (long long)heads);
+  if ((m > 0 && n > INT64_MAX / 8 / m / heads) || n > INT64_MAX / 8 / d / heads || (m > 0 && d > INT64_MAX / 8 / m / heads))
+    return fail("attn_pv: extents overflow");
+  if (!out || (m > 0 && (!P || !V))) return fail("attn_pv: NULL buffer");
+  if (overlaps(out, heads * n * d * 2, P, heads * n * m * 2) || overlaps(out, heads * n * d * 2, V, heads * m * d * 2))
+    return fail("attn_pv: output overlaps an input");
+  const bool v_vec = d % 8 == 0 && aligned(V, 16);                  // 16-byte pieces of V's rows
+  const bool p_vec = m % 8 == 0 && aligned(P, 16) && aligned(out, 8);  // 16-byte pieces of P's rows
+  dtas_config cfg;
+  if (user) {
+    cfg = *user;
+  } else if (n <= 12 && v_vec) {
+    // a handful of rows (decoding): the row kernel, two rows per workgroup (measured best for 2..8
+    // rows: more rows per workgroup mean fewer workgroups than the 256 CUs want)
+    cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : 2, 8, 0}, 1, 0};
+  } else {
+    // what this op moves is P (2*n*m bytes per head): 128-row tiles once they give every CU a workgroup
+    const int bm = heads * ceil_div(n, 128) >= kNumCU ? 128 : 64;
+    cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {bm, d <= 64 ? 64 : 128, kBK}, 1, 0};
+  }
+  if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_SKINNY && !v_vec) cfg.vec = 1;
+  if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && (!(v_vec && p_vec) || m == 0)) cfg.vec = 1;  // m == 0: zeros
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const half_t* a = static_cast<const half_t*>(P);
+  const half_t* w = static_cast<const half_t*>(V);
+  half_t* c = static_cast<half_t*>(out);
+  const int b = static_cast<int>(heads);
+  GemmEpilogue ep = {nullptr, nullptr, nullptr, DTAS_EPI_BIAS, 0, 1.f, n * m, m * d, n * d, 0};
+  if (cfg.vec == 1) {
+    int64_t grid = ceil_div(n * d, 256);
+    grid = grid > 4096 ? 4096 : grid;
+    hipLaunchKernelGGL(gemm_scalar_kernel, dim3(static_cast<unsigned>(grid), b), dim3(256), 0, s, a, w, ep, out, n, d, m, true);
+    return check_launch("attn_pv");
+  }
+  if (cfg.vec != 8) return fail("attn_pv: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+  if (cfg.variant == DTAS_GEMM_SKINNY) {
+    const int R = cfg.tile[0];
+    if (cfg.block != 256 || cfg.tile[1] != 8) return fail("attn_pv: the row kernel uses 256 threads and 8-column pieces");
+    if (R != 1 && R != 2 && R != 4 && R != 8) return fail("attn_pv: the row kernel takes 1, 2, 4 or 8 rows per workgroup, got %d", R);
+    if (cfg.split_k > 1) return fail("attn_pv: the row kernel does not split K");
+    const int64_t blocks = ceil_div(n, R);
+    if (heads * (d / 8) > 0x7fffffff || blocks > 65535) return fail("attn_pv: too many workgroups for the row kernel");
+    const dim3 grid(static_cast<unsigned>(heads * (d / 8)), static_cast<unsigned>(blocks));
+    switch (R) {
+      case 1: hipLaunchKernelGGL(attn_pv_rows_kernel<1>, grid, dim3(256), 0, s, a, w, c, n, m, d); break;
+      case 2: hipLaunchKernelGGL(attn_pv_rows_kernel<2>, grid, dim3(256), 0, s, a, w, c, n, m, d); break;
+      case 4: hipLaunchKernelGGL(attn_pv_rows_kernel<4>, grid, dim3(256), 0, s, a, w, c, n, m, d); break;
+      default: hipLaunchKernelGGL(attn_pv_rows_kernel<8>, grid, dim3(256), 0, s, a, w, c, n, m, d); break;
+    }
+    return check_launch("attn_pv");
+  }
+  if (cfg.variant != DTAS_GEMM_MFMA) return fail("attn_pv: unknown variant %d", cfg.variant);
+  if (cfg.split_k > 1) return fail("attn_pv: a batched launch cannot split K");
+  if (cfg.unroll > 2) return fail("attn_pv: the transposing kernels hold two LDS stages, got %d", cfg.unroll);
+  int64_t la[7];
+  if (describe_gemm(n, d, m, cfg, la) != 0) return -1;
+  const int bm = cfg.tile[0], bn = cfg.tile[1];
+  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
+  return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
 }

@@ -192,3 +192,19 @@ def attn_scores(Q: torch.Tensor, K: torch.Tensor, mask: torch.Tensor, out: torch
         raise ValueError("attn_scores: expects fp16 inputs and an fp32 output")
     check(lib().dtas_attn_scores_f16_f32(_p(Q), _p(K), _p(mask), _p(out), heads, n, m, d, scale, _cfg(cfg), _stream()),
           "dtas_attn_scores_f16_f32")
+
+
+def attn_pv(P: torch.Tensor, V: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """out[h,n,:] = sum_k P[h,n,k] * V[h,k,:], fp16 with fp32 accumulation: matmul8 (before_dl.py:915-929) and,
+    with n = 1, matmul10 (:899-912).  P (..., heads, n, m), V (..., heads, m, d), out (..., heads, n, d) with
+    leading extents of 1."""
+    _dev(P, V, out)
+    heads, n, m = P.shape[-3:]
+    d = V.shape[-1]
+    if V.shape[-3:] != (heads, m, d) or out.shape[-3:] != (heads, n, d):
+        raise ValueError("attn_pv: shape mismatch")
+    if P.numel() != heads * n * m or V.numel() != heads * m * d or out.numel() != heads * n * d:
+        raise ValueError("attn_pv: leading extents must be 1")
+    if any(t.dtype != torch.float16 for t in (P, V, out)):
+        raise ValueError("attn_pv: expects fp16 buffers")
+    check(lib().dtas_attn_pv_f16(_p(P), _p(V), _p(out), heads, n, m, d, _cfg(cfg), _stream()), "dtas_attn_pv_f16")

@@ -172,6 +172,16 @@ def fused_NT_matmul_divide_maximum_minimum_cast(heads: int = 32, head_dim: int =
                     attrs={"tir.noalias": True, "scale": scale})
 
 
+def matmul_pv(heads: int = 32, head_dim: int = 80, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """out(1,heads,n,d) = P(1,heads,n,m) . V(1,heads,m,d), the attention output: matmul8 (before_dl.py:915-929;
+    n and m dynamic) or, with ``decode``, matmul10 (:899-912; n = 1, m dynamic)."""
+    n = 1 if decode else "n"
+    params = [Buffer("A", (1, heads, n, "m"), "float16"), Buffer("B", (1, heads, "m", head_dim), "float16"),
+              Buffer("matmul", (1, heads, n, head_dim), "float16")]
+    blocks = [Block("matmul", "SSSSR", ["A", "B"], ["matmul"])]
+    return PrimFunc(name or ("matmul10" if decode else "matmul8"), params, blocks, op="attn_pv", attrs={"tir.noalias": True})
+
+
 def module(*funcs: PrimFunc, upper_bound: Optional[dict] = None) -> IRModule:
     """An IRModule of the given PrimFuncs; ``upper_bound`` is the ``tir_var_upper_bound`` attribute
     (tuning_test/tune_cast.py:26 uses {"m": 512, "n": 4096})."""

@@ -67,6 +67,7 @@ class _C:
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
                 "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
+                "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
             }
             for name, argtypes in sig.items():
                 fn = getattr(lib, name)
@@ -170,6 +171,16 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         return out
 
     @staticmethod
+    def attn_pv(p, v, acc_f16: bool = False, threads: int = 1) -> np.ndarray:
+        """fp16 out[h,n,d] = p[h,n,m] . v[h,m,d]."""
+        heads, n, m = p.shape
+        d = v.shape[2]
+        assert v.shape == (heads, m, d) and p.dtype == np.float16 and v.dtype == np.float16
+        out = np.empty((heads, n, d), dtype=np.float16)
+        _C.lib().oracle_attn_pv_f16(_ptr(p), _ptr(v), _ptr(out), heads, n, m, d, int(acc_f16), threads)
+        return out
+
+    @staticmethod
     def gemm_f32out(a, w, threads: int = 1) -> np.ndarray:
         K = a.shape[-1]
         M, N = a.size // K, w.shape[0]
@@ -218,6 +229,10 @@ class np64:  # noqa: N801
     def attn_scores(q, k, mask, scale):
         s_ = np.einsum("hnd,hmd->hnm", q.astype(np.float64), k.astype(np.float64)) * float(np.float16(scale))
         return np.minimum(np.maximum(s_, -65504.0), mask.astype(np.float64)[None])
+
+    @staticmethod
+    def attn_pv(p, v):
+        return np.einsum("hnm,hmd->hnd", p.astype(np.float64), v.astype(np.float64))
 
     @staticmethod
     def gemm_fused(a, w, bias, res1, res2, kind):

@@ -353,6 +353,34 @@ void oracle_attn_scores_f16_f32(const f16* Q, const f16* Kmat, const f16* mask, 
   }
 }
 
+/* ========================================================================
+ * attention output: matmul8 (before_dl.py:915-929) and, with n = 1, matmul10 (:899-912)
+ *   matmul[0, h, i, e] = sum_k A[0, h, i, k] * B[0, h, k, e]        (an fp16 buffer)
+ * P[heads, n, m], V[heads, m, d] (k-major: V's rows run along d), out[heads, n, d].  The product is
+ * accumulated in fp32 and rounded once (acc_f16 = 1: the literal fp16 running sum, k ascending).
+ * Pinned by: numpy's float64 matmul, P = identity / a one-hot row selector (out = rows of V, bit
+ * exact), a constant row 1/m of P (column means of V), linearity in P for exactly representable
+ * data, heads independent, m = 0 (zeros), n = 1 equal to a row of the n > 1 case.
+ * ======================================================================== */
+void oracle_attn_pv_f16(const f16* P, const f16* V, f16* out, int64_t heads, int64_t n, int64_t m, int64_t d,
+                        int acc_f16, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t idx = 0; idx < heads * n * d; ++idx) {
+    const int64_t h = idx / (n * d), i = (idx / d) % n, e = idx % d;
+    const f16* p = P + (h * n + i) * m;
+    const f16* v = V + h * m * d + e;
+    if (acc_f16) {
+      f16 acc = 0;
+      for (int64_t k = 0; k < m; ++k) acc = f2h(h2f(acc) + h2f(f2h(h2f(p[k]) * h2f(v[k * d]))));
+      out[idx] = acc;
+    } else {
+      float acc = 0.f;
+      for (int64_t k = 0; k < m; ++k) acc = acc + h2f(p[k]) * h2f(v[k * d]);
+      out[idx] = f2h(acc);
+    }
+  }
+}
+
 int oracle_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

@@ -72,3 +72,112 @@ def test_scores_through_the_primfunc_descriptor(oracle):
     call_primfunc(func, tensors)
     torch.cuda.synchronize()
     _check(out.cpu().numpy().reshape(32, 40, 56), q, k, mask, oracle)
+
+
+# ---- P.V: matmul8 / matmul10 (before_dl.py:915-929, :899-912) --------------------------------------------
+
+def _pv_inputs(heads, n, m, d, seed):
+    rng = np.random.default_rng(seed)
+    p = rng.random((heads, n, m)).astype(np.float32)
+    p = (p / np.maximum(p.sum(-1, keepdims=True), 1e-6)).astype(np.float16)       # rows like a softmax's
+    v = rng.standard_normal((heads, m, d)).astype(np.float16)
+    return p, v
+
+
+def _check_pv(got, p, v, oracle):
+    want = oracle.c.attn_pv(p, v, threads=8)
+    f64 = oracle.np64.attn_pv(p, v)
+    assert np.isfinite(got).all()
+    assert (np.abs(got.astype(np.float64) - f64) <= 1e-3 + 1e-2 * np.abs(f64)).all()     # rtol 1e-2 against float64
+    assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 1e-4 + 2.0 ** -9 * np.abs(want)).all()
+    if got.size:
+        assert (got == want).mean() > 0.97      # the rest: one fp16 ulp from the fp32 summation order
+
+
+@pytest.mark.parametrize("n,m", [(1, 1), (1, 77), (1, 2048), (3, 300), (8, 129), (9, 64), (9, 77), (64, 64), (130, 200),
+                                 (257, 520), (1024, 1024)])
+def test_pv_builtin_config(oracle, n, m):
+    p, v = _pv_inputs(32, n, m, 80, 3 * n + m)
+    out = Guarded((1, 32, n, 80), torch.float16)
+    ops.attn_pv(dev(p).view(1, 32, n, m), dev(v).view(1, 32, m, 80), out.t)
+    _check_pv(out.check().reshape(32, n, 80), p, v, oracle)
+
+
+@pytest.mark.parametrize("tile", [(64, 64), (64, 128), (128, 64), (128, 128)])
+@pytest.mark.parametrize("heads,n,m,d", [(3, 70, 136, 80), (2, 300, 264, 64), (1, 33, 8, 8), (2, 50, 72, 136), (1, 129, 1032, 128)])
+def test_pv_every_tile(oracle, tile, heads, n, m, d):
+    p, v = _pv_inputs(heads, n, m, d, n + m + d)
+    out = Guarded((heads, n, d), torch.float16)
+    ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[tile[0], tile[1], 64]))
+    _check_pv(out.check(), p, v, oracle)
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 8])
+@pytest.mark.parametrize("heads,n,m,d", [(32, 1, 515, 80), (32, 1, 4096, 80), (3, 3, 64, 8), (2, 11, 1000, 128), (1, 8, 1, 16),
+                                         (2, 5, 300, 264)])
+def test_pv_row_kernel(oracle, rows, heads, n, m, d):
+    p, v = _pv_inputs(heads, n, m, d, n + m + d + rows)
+    out = Guarded((heads, n, d), torch.float16)
+    ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, block=256, vec=8, unroll=1, tile=[rows, 8, 0]))
+    _check_pv(out.check(), p, v, oracle)
+
+
+def test_pv_selector_rows_are_exact_and_edge_cases(oracle):
+    # P = identity picks the rows of V: any operand mix-up (a transposed V, a shifted k) shows as wrong bits
+    rng = np.random.default_rng(5)
+    v = rng.standard_normal((4, 200, 80)).astype(np.float16)
+    eye = np.ascontiguousarray(np.broadcast_to(np.eye(200, dtype=np.float16), (4, 200, 200)))
+    out = Guarded((4, 200, 80), torch.float16)
+    ops.attn_pv(dev(eye), dev(v), out.t)
+    assert np.array_equal(out.check().view(np.uint16), v.view(np.uint16))
+    # element-access fallback: m % 8 != 0, d % 8 != 0, an odd V pointer
+    for (n, m, d) in [(40, 77, 80), (12, 16, 12)]:
+        p, v = _pv_inputs(2, n, m, d, n + m)
+        out = Guarded((2, n, d), torch.float16)
+        ops.attn_pv(dev(p), dev(v), out.t)
+        _check_pv(out.check(), p, v, oracle)
+    p, v = _pv_inputs(2, 40, 80, 80, 6)
+    vbuf = torch.empty(2 * 80 * 80 + 1, dtype=torch.float16, device="cuda")
+    vbuf[1:].copy_(dev(v).flatten())
+    out = Guarded((2, 40, 80), torch.float16)
+    ops.attn_pv(dev(p), vbuf[1:].view(2, 80, 80), out.t)
+    _check_pv(out.check(), p, v, oracle)
+    # m == 0: an empty sum is zeros; n == 0: a no-op
+    out = Guarded((2, 5, 80), torch.float16)
+    ops.attn_pv(torch.empty(2, 5, 0, dtype=torch.float16, device="cuda"), torch.empty(2, 0, 80, dtype=torch.float16, device="cuda"), out.t)
+    assert (out.check() == 0).all()
+    assert _lib.lib().dtas_attn_pv_f16(None, None, None, 32, 0, 16, 80, None, None) == 0
+
+
+def test_pv_errors():
+    p, v = _pv_inputs(2, 16, 16, 80, 1)
+    out = torch.empty(2, 16, 80, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="split"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=2))
+    with pytest.raises(_lib.DtasError, match="two LDS stages"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=3, tile=[64, 64, 64]))
+    with pytest.raises(_lib.DtasError, match="no transposing"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[256, 128, 64]))
+    with pytest.raises(_lib.DtasError, match="1, 2, 4 or 8"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_SKINNY, block=256, vec=8, unroll=1, tile=[3, 8, 0]))
+    with pytest.raises(_lib.DtasError, match="does not split"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_SKINNY, block=256, vec=8, unroll=1, tile=[1, 8, 0], split_k=2))
+    pd = dev(p)
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        check_rc = _lib.lib().dtas_attn_pv_f16(pd.data_ptr(), dev(v).data_ptr(), pd.data_ptr(), 2, 16, 16, 80, None, None)
+        _lib.check(check_rc, "dtas_attn_pv_f16")
+
+
+def test_pv_through_the_primfunc_descriptors(oracle):
+    from dtas_amd import primfuncs as pf
+    from dtas_amd.codegen.runtime_packer import bind_extents, call_primfunc
+
+    for decode, n in ((False, 40), (True, 1)):
+        func = pf.matmul_pv(32, 80, decode=decode)
+        p, v = _pv_inputs(32, n, 56, 80, 9 + n)
+        out = torch.empty(1, 32, n, 80, dtype=torch.float16, device="cuda")
+        tensors = (dev(p).view(1, 32, n, 56), dev(v).view(1, 32, 56, 80), out)
+        assert bind_extents(func, tensors) == ({"m": 56} if decode else {"n": 40, "m": 56})
+        call_primfunc(func, tensors)
+        torch.cuda.synchronize()
+        _check_pv(out.cpu().numpy().reshape(32, n, 80), p, v, oracle)
