@@ -101,6 +101,15 @@ def _workload(name: str, n: int, extra=None):
         make = lambda s: (normal((1, K), s), normal((N, K), s + 100, 0.02), empty((1, N)))
         return (make, lambda b: call(L.dtas_gemv_f16, P(b[0]), P(b[1]), None, P(b[2]), N, K, None, stream),
                 2 * N * K + 2 * K + 2 * N, 2 * N * K)
+    if name == "gemv_q8_f16":
+        # fused_fused_decode2_fused_NT_matmul_add: 8-bit weights (4 to a word) with an fp16 scale per 32, dequantised in registers
+        N, K = extra
+        def make(s):
+            g = torch.Generator(device="cuda").manual_seed(s + 200)
+            wq = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device="cuda", generator=g)
+            return normal((1, K), s), wq, uniform((N, K // 32), s + 100, 0.001, 0.02), empty((1, N))
+        return (make, lambda b: call(L.dtas_gemv_q8_f16, P(b[0]), P(b[1]), P(b[2]), None, P(b[3]), N, K, 0, None, stream),
+                N * K + 2 * N * (K // 32) + 2 * K + 2 * N, 2 * N * K)
     if name == "gemm_f16":
         N, K = extra
         wt = normal((N, K), 100, 0.02)
@@ -274,6 +283,8 @@ def sweep(steps: int, warmup: int) -> list:
             rows.append(measure(op, n, None, steps, warmup))
     for nk in GEMV_SHAPES:
         rows.append(measure("gemv_f16", 1, nk, steps, warmup))
+    for nk in GEMV_SHAPES:
+        rows.append(measure("gemv_q8_f16", 1, nk, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
@@ -306,7 +317,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
-                         "gemv_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last four take --nk; attn_scores n = m)")
+                         "gemv_f16 | gemv_q8_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -331,7 +342,7 @@ def main() -> int:
         print(_lib.last_error(), file=sys.stderr)
         return 2
 
-    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemm_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_q8_f16", "gemm_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
     info = None
@@ -347,10 +358,12 @@ def main() -> int:
         workload_key = f"{args.workload} [n={args.n}, 2560]"
     elif args.workload == "softmax_f16":
         workload_key = f"{args.workload} [{32 * args.n}, n={args.n}]"
+    elif args.workload in ("attn_scores_f16_f32", "attn_pv_f16"):
+        workload_key = f"{args.workload} [32 heads of 80, n=m={args.n}]"
     elif extra is None:
         workload_key = f"{args.workload} [n={args.n}, 4096]"
-    elif args.workload == "gemv_f16":
-        workload_key = f"gemv_f16 M=1 NxK={args.nk}"
+    elif args.workload in ("gemv_f16", "gemv_q8_f16"):
+        workload_key = f"{args.workload} M=1 NxK={args.nk}"
     else:
         workload_key = f"{args.workload} M={args.n} NxK={args.nk}"
     line = {

@@ -32,7 +32,7 @@ def _torch_dtype(name: str):
     if _TORCH_DTYPES is None:
         import torch
 
-        _TORCH_DTYPES = {"float16": torch.float16, "float32": torch.float32, "int8": torch.int8}
+        _TORCH_DTYPES = {"float16": torch.float16, "float32": torch.float32, "int8": torch.int8, "uint32": torch.uint32}
     return _TORCH_DTYPES[name]
 
 
@@ -53,6 +53,10 @@ def op_id_of(func: PrimFunc) -> int:
     if func.op == "matmul":
         return _lib.OP_GEMV_F16 if FuncInfo(func).kind == FuncKind.kFunc_GEMV else _lib.OP_GEMM_F16
     raise ValueError(f"no kernel family for op {func.op!r}")
+
+
+# PrimFuncs the tuner does not search: the library picks their kernel and launch shape per call
+LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "gemv_q8")
 
 
 def _concrete(shape, values: Dict[str, int]) -> Tuple[int, ...]:
@@ -97,7 +101,8 @@ def bind_extents(func: PrimFunc, tensors: Sequence) -> Dict[str, int]:
                         f"got {len(tensors)}")
     values: Dict[str, int] = {}
     for buf, t in zip(func.params, tensors):
-        if t.dtype != _torch_dtype(buf.dtype):
+        # (a uint32 buffer is also accepted as int32: the same words, and the dtype torch is fluent in)
+        if t.dtype != _torch_dtype(buf.dtype) and not (buf.dtype == "uint32" and str(t.dtype) == "torch.int32"):
             raise TypeError(f"{func.name}: buffer {buf.name} is {buf.dtype}, got {t.dtype}")
         if t.dim() != len(buf.shape):
             raise ValueError(f"{func.name}: buffer {buf.name} has {len(buf.shape)} dims, got shape {tuple(t.shape)}")
@@ -130,6 +135,10 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.attn_scores(tensors[0], tensors[1], tensors[2], tensors[3], func.attrs.get("scale", 0.11179039301310044), abi)
     elif op == "attn_pv":                                                     # P, V, out
         ops.attn_pv(tensors[0], tensors[1], tensors[2], abi)
+    elif op == "decode_q8":                                                   # Wq, scale, W
+        ops.decode_q8(tensors[0], tensors[1], tensors[2], abi)
+    elif op == "gemv_q8":                                                     # Wq, scale, x, bias, y
+        ops.gemv_q8(tensors[2], tensors[0], tensors[1], tensors[3], tensors[4], abi, int(func.attrs.get("epilogue", 0)))
     elif op == "matmul":
         epilogue = int(func.attrs.get("epilogue", 0))
         if epilogue in (_lib.EPI_BIAS_ADD2, _lib.EPI_BIAS_ADD2_CAST_F32):   # A, W, bias, res1, res2, out
@@ -224,7 +233,9 @@ class FunctionTable:
         expr = f"({a}/{div} * {s1} + {b}/{div})"
         return f"  int64_t index = {expr} > {last} ? {last} : {expr};\n"
 
-    def select(self, values: Dict[str, int]) -> KernelEntryInfo:
+    def select(self, values: Dict[str, int]) -> Optional[KernelEntryInfo]:
+        if not self.call_table:      # a function whose launch shape the library chooses itself
+            return None
         if not self.index_table:
             return self.call_table[0]
         return self.call_table[self.index_table[self.index(values)]]
@@ -268,7 +279,8 @@ class RuntimeModule:
 
         def packed_func(*tensors):
             values = bind_extents(table.func, tensors)
-            call_primfunc(table.func, tensors, table.select(values).abi)
+            entry = table.select(values)
+            call_primfunc(table.func, tensors, entry.abi if entry is not None else None)
 
         packed_func.__name__ = name
         return packed_func
@@ -276,8 +288,8 @@ class RuntimeModule:
     def get_function(self, name: str):
         return self[name]
 
-    def entry_for(self, name: str, **values: int) -> KernelEntryInfo:
-        """Which call-table row a call with these dynamic extents uses."""
+    def entry_for(self, name: str, **values: int) -> Optional[KernelEntryInfo]:
+        """Which call-table row a call with these dynamic extents uses (None: the library's own choice)."""
         return self.tables[name].select(values)
 
     def time_evaluator(self, func_name: str, dev=None, number: int = 10, repeat: int = 1, min_repeat_ms: float = 0):

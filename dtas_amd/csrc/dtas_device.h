@@ -98,6 +98,17 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* slots, int
   b = rb;
 }
 
+// ---- erf-GELU on an fp16 value, every step an fp16 tensor as the fused PrimFuncs spell it
+// (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:248-318): t * (0.5 + 0.5 * erf(t * fp16(0.7071...)))
+__device__ __forceinline__ half_t gelu_erf_f16_steps(half_t t) {
+  const float x = static_cast<float>(t);
+  const half_t m = static_cast<half_t>(x * static_cast<float>(static_cast<half_t>(0.70710678118654757f)));
+  const half_t e = static_cast<half_t>(erff(static_cast<float>(m)));
+  const half_t h = static_cast<half_t>(static_cast<float>(e) * 0.5f);
+  const half_t a = static_cast<half_t>(0.5f + static_cast<float>(h));
+  return static_cast<half_t>(x * static_cast<float>(a));
+}
+
 // ---- streaming (touch-once) global accesses ---------------------------------------
 template <typename V>
 __device__ __forceinline__ V load_stream(const V* p) { return __builtin_nontemporal_load(p); }

@@ -100,12 +100,7 @@ __device__ __forceinline__ half_t epilogue_value_k(half_t mm, bool has_bias, flo
     t = round_h(fmaxf(static_cast<float>(t), -65504.f));                 // T_maximum
     t = round_h(fminf(static_cast<float>(t), r1));                       // T_minimum with the mask
   } else if (KIND == DTAS_EPI_BIAS_GELU) {
-    const float x = static_cast<float>(t);
-    const half_t m = round_h(x * static_cast<float>(static_cast<half_t>(0.70710678118654757f)));
-    const half_t e = round_h(erff(static_cast<float>(m)));
-    const half_t h = round_h(static_cast<float>(e) * 0.5f);
-    const half_t a = round_h(0.5f + static_cast<float>(h));
-    t = round_h(x * static_cast<float>(a));
+    t = gelu_erf_f16_steps(t);
   }
   return t;
 }

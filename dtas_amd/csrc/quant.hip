@@ -1,0 +1,221 @@
+// 8-bit weights with fp16 group scales (the q8f16_1 layout) for gfx950: the standalone dequantiser
+// and the decode GEMV that dequantises in registers.
+//
+// Layout and arithmetic, as the PrimFuncs spell them
+// (experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py:335-343 fused_decode3, :401-426
+// fused_fused_decode2_fused_NT_matmul_add, :428-502 fused_fused_decode4_fused_NT_matmul3_add2_gelu):
+//   Wq[N, K/4] uint32: element j of a row is byte j % 4 of word j / 4;  S[N, K/32] fp16: one scale per 32
+//   W[i, j] = (fp16(byte) - fp16(127)) * S[i, j / 32]           -- fp16 arithmetic, one rounding (the product)
+//   y[i]    = sum_k x[k] * W[i, k]  (+ bias[i], then GELU)      -- fp32 accumulation here, fp16 after
+//
+// byte -> fp16 without a conversion: 0x6400 is 1024.0 and fp16 counts in ones from 1024 to 2047, so
+// 0x6400 | byte is 1024 + byte exactly; one byte permute builds two such halves from a weight word,
+// one packed subtract of 1151 leaves byte - 127 (exact), one packed multiply by the scale rounds as
+// the PrimFunc's fp16 product does, one dot2 accumulates against x in fp32: 4 VALU instructions per
+// two weights, so the kernel stays bound by the weight stream (one byte per weight).
+#include "dtas_device.h"
+#include "dtas_host.h"
+
+namespace dtas {
+namespace {
+
+// the four weights of a word as two packed fp16 pairs: {W[4w], W[4w+1]}, {W[4w+2], W[4w+3]}
+__device__ __forceinline__ void dequant_word(unsigned word, f16x2 scale2, f16x2& lo, f16x2& hi) {
+  const f16x2 bias2 = {static_cast<half_t>(1151.f), static_cast<half_t>(1151.f)};
+  const unsigned plo = __builtin_amdgcn_perm(0x64646464u, word, 0x04010400u);  // bytes: b0, 0x64, b1, 0x64
+  const unsigned phi = __builtin_amdgcn_perm(0x64646464u, word, 0x04030402u);  // bytes: b2, 0x64, b3, 0x64
+  lo = (__builtin_bit_cast(f16x2, plo) - bias2) * scale2;
+  hi = (__builtin_bit_cast(f16x2, phi) - bias2) * scale2;
+}
+
+// One thread = 16 weights (16 bytes in, 32 bytes out).  K % 32 == 0, so a thread's 16 weights share a
+// scale and the flat scale index is (16 i) / 32.
+__global__ void __launch_bounds__(256) decode_q8_kernel(const u32x4* __restrict__ Wq, const half_t* __restrict__ S,
+                                                        u32x4* __restrict__ W, int64_t chunks) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < chunks;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const u32x4 q = load_stream(Wq + i);
+    const half_t s = S[i >> 1];
+    const f16x2 s2 = {s, s};
+    u32x4 out[2];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      f16x2 lo, hi;
+      const unsigned word = q[w];
+      dequant_word(word, s2, lo, hi);
+      out[w >> 1][(w & 1) * 2] = __builtin_bit_cast(unsigned, lo);
+      out[w >> 1][(w & 1) * 2 + 1] = __builtin_bit_cast(unsigned, hi);
+    }
+    store_stream(out[0], W + 2 * i);
+    store_stream(out[1], W + 2 * i + 1);
+  }
+}
+
+// any alignment: one thread per weight
+__global__ void __launch_bounds__(256) decode_q8_scalar_kernel(const unsigned char* __restrict__ Wq,
+                                                               const half_t* __restrict__ S, half_t* __restrict__ W,
+                                                               int64_t total) {
+  for (int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; j < total;
+       j += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const half_t q = static_cast<half_t>(static_cast<float>(Wq[j])) - static_cast<half_t>(127.f);  // little endian: byte j
+    W[j] = q * S[j >> 5];
+  }
+}
+
+__device__ __forceinline__ half_t finish_q8(float acc, const half_t* bias, int64_t j, int kind) {
+  half_t t = static_cast<half_t>(acc);
+  if (bias) t = static_cast<half_t>(static_cast<float>(t) + static_cast<float>(bias[j]));
+  if (kind == DTAS_EPI_BIAS_GELU) t = gelu_erf_f16_steps(t);
+  return t;
+}
+
+// Workgroup = R rows of Wq; lane t takes the 16-byte chunks t, t + block, ... (16 weights, 32 bytes
+// of x) of every row, so a wavefront reads 1 KiB of a row at a time, non-temporal.
+template <int R>
+__global__ void __launch_bounds__(512) gemv_q8_kernel(const half_t* __restrict__ x, const unsigned* __restrict__ Wq,
+                                                      const half_t* __restrict__ S, const half_t* __restrict__ bias,
+                                                      half_t* __restrict__ y, int64_t N, int64_t K, int kind) {
+  __shared__ float part[8][R];
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+  const int64_t nchunk = K >> 4, ngroup = K >> 5;
+  const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+  const u32x4* wv[R];
+  const half_t* sv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r < N ? row0 + r : N - 1;  // rows past N re-read the last row; never stored
+    wv[r] = reinterpret_cast<const u32x4*>(Wq + row * (K >> 2));
+    sv[r] = S + row * ngroup;
+  }
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+#pragma unroll 2
+  for (int64_t i = threadIdx.x; i < nchunk; i += blockDim.x) {
+    const u32x4 x0 = xv[2 * i], x1 = xv[2 * i + 1];
+    u32x4 q[R];
+    half_t s[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      q[r] = load_stream(wv[r] + i);
+      s[r] = sv[r][i >> 1];
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const f16x2 s2 = {s[r], s[r]};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        f16x2 lo, hi;
+        const unsigned word = q[r][w];
+        dequant_word(word, s2, lo, hi);
+        const unsigned xa = w < 2 ? x0[2 * w] : x1[2 * w - 4], xb = w < 2 ? x0[2 * w + 1] : x1[2 * w - 3];
+        acc[r] = __builtin_amdgcn_fdot2(lo, __builtin_bit_cast(f16x2, xa), acc[r], false);
+        acc[r] = __builtin_amdgcn_fdot2(hi, __builtin_bit_cast(f16x2, xb), acc[r], false);
+      }
+    }
+  }
+
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float sum = wave_sum(acc[r]);
+    if ((threadIdx.x & 63) == 0) part[wave][r] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x < R && row0 + threadIdx.x < N) {
+    float sum = 0.f;
+    for (int w = 0; w < nwaves; ++w) sum += part[w][threadIdx.x];
+    y[row0 + threadIdx.x] = finish_q8(sum, bias, row0 + threadIdx.x, kind);
+  }
+}
+
+// any alignment: one wavefront per row, byte accesses
+__global__ void __launch_bounds__(256) gemv_q8_scalar_kernel(const half_t* __restrict__ x, const unsigned char* __restrict__ Wq,
+                                                             const half_t* __restrict__ S, const half_t* __restrict__ bias,
+                                                             half_t* __restrict__ y, int64_t N, int64_t K, int kind) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= N) return;  // whole wavefronts leave together; no workgroup barrier below
+  float acc = 0.f;
+  for (int64_t k = threadIdx.x & 63; k < K; k += 64) {
+    const half_t q = static_cast<half_t>(static_cast<float>(Wq[row * K + k])) - static_cast<half_t>(127.f);
+    const half_t w = q * S[row * (K >> 5) + (k >> 5)];
+    acc += static_cast<float>(x[k]) * static_cast<float>(w);
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) y[row] = finish_q8(acc, bias, row, kind);
+}
+
+int check_q8_shape(const char* what, int64_t N, int64_t K) {
+  if (N < 0 || K < 0) return fail("%s: negative extent N=%lld K=%lld", what, (long long)N, (long long)K);
+  if (K % 32 != 0) return fail("%s: K must be a multiple of the scale group, 32 (K=%lld)", what, (long long)K);
+  if (K != 0 && N > INT64_MAX / 4 / K) return fail("%s: N*K overflows", what);
+  return 0;
+}
+
+}  // namespace
+}  // namespace dtas
+
+extern "C" int dtas_decode_q8_f16(const void* Wq, const void* scale, void* W, int64_t N, int64_t K, const dtas_config* user,
+                                  void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (check_q8_shape("decode_q8", N, K) != 0) return -1;
+  if (N == 0 || K == 0) return 0;
+  if (!Wq || !scale || !W) return fail("decode_q8: NULL buffer");
+  if (overlaps(W, N * K * 2, Wq, N * K) || overlaps(W, N * K * 2, scale, N * (K / 32) * 2))
+    return fail("decode_q8: output overlaps an input");
+  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, 256, 16, 1, {0, 0, 0}, 1, 0};
+  if (cfg.block != 256) return fail("decode_q8: the kernels use 256 threads, got %d", cfg.block);
+  if (cfg.vec != 16 && cfg.vec != 1) return fail("decode_q8: vector width must be 16 (128 bits of weights) or 1, got %d", cfg.vec);
+  if (cfg.vec == 16 && !(aligned(Wq, 16) && aligned(W, 16))) cfg.vec = 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t items = cfg.vec == 16 ? N * K / 16 : N * K;
+  int64_t grid = ceil_div(items, 256);
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  grid = grid > cap ? cap : grid;
+  if (cfg.vec == 16)
+    hipLaunchKernelGGL(decode_q8_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x4*>(Wq),
+                       static_cast<const half_t*>(scale), static_cast<u32x4*>(W), items);
+  else
+    hipLaunchKernelGGL(decode_q8_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s,
+                       static_cast<const unsigned char*>(Wq), static_cast<const half_t*>(scale), static_cast<half_t*>(W), items);
+  return check_launch("decode_q8");
+}
+
+extern "C" int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale, const void* bias, void* y, int64_t N,
+                                int64_t K, int32_t epilogue, const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (check_q8_shape("gemv_q8", N, K) != 0) return -1;
+  if (epilogue != DTAS_EPI_BIAS && epilogue != DTAS_EPI_BIAS_GELU)
+    return fail("gemv_q8: epilogue must be DTAS_EPI_BIAS or DTAS_EPI_BIAS_GELU, got %d", epilogue);
+  if (N == 0) return 0;
+  if (!y || (K > 0 && (!x || !Wq || !scale))) return fail("gemv_q8: NULL buffer");
+  if (overlaps(y, N * 2, Wq, N * K) || overlaps(y, N * 2, x, K * 2) || overlaps(y, N * 2, scale, N * (K / 32) * 2))
+    return fail("gemv_q8: output overlaps an input");
+  // measured over the model's and the benchmark's shapes: 256 threads; 2 rows per workgroup, 4 once that
+  // still leaves every CU a dozen workgroups
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 4 : 2, 0, 0}, 1, 0};
+  if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
+  int64_t la[7];
+  if (describe_gemv(N, K, cfg, la) != 0) return -1;
+  const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const half_t* xp = static_cast<const half_t*>(x);
+  const half_t* sp = static_cast<const half_t*>(scale);
+  const half_t* bp = static_cast<const half_t*>(bias);
+  half_t* yp = static_cast<half_t*>(y);
+  if (cfg.vec == 1) {
+    hipLaunchKernelGGL(gemv_q8_scalar_kernel, grid, block, 0, s, xp, static_cast<const unsigned char*>(Wq), sp, bp, yp, N, K, epilogue);
+    return check_launch("gemv_q8");
+  }
+  const unsigned* wp = static_cast<const unsigned*>(Wq);
+  switch (cfg.tile[0]) {
+    case 1: hipLaunchKernelGGL(gemv_q8_kernel<1>, grid, block, 0, s, xp, wp, sp, bp, yp, N, K, epilogue); break;
+    case 2: hipLaunchKernelGGL(gemv_q8_kernel<2>, grid, block, 0, s, xp, wp, sp, bp, yp, N, K, epilogue); break;
+    case 4: hipLaunchKernelGGL(gemv_q8_kernel<4>, grid, block, 0, s, xp, wp, sp, bp, yp, N, K, epilogue); break;
+    case 8: hipLaunchKernelGGL(gemv_q8_kernel<8>, grid, block, 0, s, xp, wp, sp, bp, yp, N, K, epilogue); break;
+  }
+  return check_launch("gemv_q8");
+}

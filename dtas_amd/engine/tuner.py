@@ -15,7 +15,7 @@ from typing import Dict, List, Tuple
 from ..arch import Arch
 from ..codegen.code_gen import CodeGenerator
 from ..codegen.compile_result import CompileResult
-from ..codegen.runtime_packer import RuntimeModule, RuntimePacker
+from ..codegen.runtime_packer import LIBRARY_CHOSEN_OPS, RuntimeModule, RuntimePacker
 from ..common.analisys import FuncInfo, IRModule, PrimFunc
 from ..common.config import Range, generate_range_list
 from ..logging import debug_info, get_log_level
@@ -51,6 +51,10 @@ class Engine:
         cg = CodeGenerator(getattr(arch, "target", "gfx950"))
         for name, func in mod.functions_items():
             if not isinstance(func, PrimFunc):
+                continue
+            if func.op in LIBRARY_CHOSEN_OPS:   # served with the library's built-in choice: an empty call table
+                cg.gen_code_for_func(func, {}, [], range_div_factor,
+                                     {v.name: self.upper_bound.setdefault(v.name, DEFAULT_UPPER_BOUND) for v in func.dynamic_args})
                 continue
             ranges_best_result, _, _ = self.tune_func(func, name, arch, True, range_div_factor)
             index_table, index_stmt = self.get_index_table(ranges_best_result, range_div_factor)

@@ -208,3 +208,37 @@ def attn_pv(P: torch.Tensor, V: torch.Tensor, out: torch.Tensor, cfg: Optional[D
     if any(t.dtype != torch.float16 for t in (P, V, out)):
         raise ValueError("attn_pv: expects fp16 buffers")
     check(lib().dtas_attn_pv_f16(_p(P), _p(V), _p(out), heads, n, m, d, _cfg(cfg), _stream()), "dtas_attn_pv_f16")
+
+
+def _q8_shapes(what: str, Wq: torch.Tensor, scale: torch.Tensor):
+    if Wq.dim() != 2 or Wq.dtype not in (torch.int32, torch.uint32) or scale.dtype != torch.float16:
+        raise ValueError(f"{what}: expects 32-bit words [N, K/4] and fp16 scales [N, K/32]")
+    N, K = Wq.shape[0], Wq.shape[1] * 4
+    if K % 32 != 0 or tuple(scale.shape) != (N, K // 32):
+        raise ValueError(f"{what}: K = {K} and scales {tuple(scale.shape)} do not form groups of 32")
+    return N, K
+
+
+def decode_q8(Wq: torch.Tensor, scale: torch.Tensor, W: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """W[N,K] (fp16) = (fp16(byte) - 127) * scale[N, K/32]; element j of a row is byte j % 4 of word j / 4 of
+    Wq[N, K/4]: fused_decode3 (dolly-v2-3b-q8f16_1/before_dl.py:335-343)."""
+    _dev(Wq, scale, W)
+    N, K = _q8_shapes("decode_q8", Wq, scale)
+    if W.dtype != torch.float16 or W.numel() != N * K:
+        raise ValueError("decode_q8: expects an fp16 output of N * K elements")
+    check(lib().dtas_decode_q8_f16(_p(Wq), _p(scale), _p(W), N, K, _cfg(cfg), _stream()), "dtas_decode_q8_f16")
+
+
+def gemv_q8(x: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor], y: torch.Tensor,
+            cfg: Optional[DtasConfig] = None, epilogue: int = 0) -> None:
+    """y[N] = x[K] . decode_q8(Wq, scale)^T (+ bias[N]; ``_lib.EPI_BIAS_GELU``: then GELU), the weights dequantised
+    in registers: fused_fused_decode2_fused_NT_matmul_add / fused_fused_decode4_fused_NT_matmul3_add2_gelu
+    (dolly-v2-3b-q8f16_1/before_dl.py:401-426, :428-502)."""
+    _dev(x, Wq, scale, bias, y)
+    N, K = _q8_shapes("gemv_q8", Wq, scale)
+    if x.numel() != K or y.numel() != N or (bias is not None and bias.numel() != N):
+        raise ValueError("gemv_q8: shape mismatch")
+    if any(t.dtype != torch.float16 for t in (x, y)) or (bias is not None and bias.dtype != torch.float16):
+        raise ValueError("gemv_q8: expects fp16 x, bias and y")
+    check(lib().dtas_gemv_q8_f16(_p(x), _p(Wq), _p(scale), _p(bias), _p(y), N, K, epilogue, _cfg(cfg), _stream()),
+          "dtas_gemv_q8_f16")

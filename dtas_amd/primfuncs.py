@@ -182,6 +182,31 @@ def matmul_pv(heads: int = 32, head_dim: int = 80, decode: bool = False, name: O
     return PrimFunc(name or ("matmul10" if decode else "matmul8"), params, blocks, op="attn_pv", attrs={"tir.noalias": True})
 
 
+def fused_decode(N: int = 2560, K: int = 2560, name: Optional[str] = None) -> PrimFunc:
+    """W(N,K) fp16 = (fp16(byte) - 127) * scale(N, K/32) of 8-bit weights packed four to a uint32 word:
+    fused_decode3, dolly-v2-3b-q8f16_1/before_dl.py:335-343."""
+    params = [Buffer("model_params_9", (N, K // 4), "uint32"), Buffer("model_params_10", (N, K // 32), "float16"),
+              Buffer("decode_intermediate", (N, K), "float16")]
+    blocks = [Block("decode", "SS", ["model_params_9", "model_params_10"], ["decode_intermediate"])]
+    return PrimFunc(name or "fused_decode3", params, blocks, op="decode_q8", attrs={"tir.noalias": True})
+
+
+def fused_decode_NT_matmul_add(N: int = 7680, K: int = 2560, gelu: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """y(1,1,N) = x(1,1,K) . decode(Wq, scale)^T + bias (then GELU): fused_fused_decode2_fused_NT_matmul_add
+    (dolly-v2-3b-q8f16_1/before_dl.py:401-426) or, with ``gelu``, fused_fused_decode4_fused_NT_matmul3_add2_gelu
+    (:428-502; N = 10240).  Parameters: Wq, scale, x, bias, out."""
+    out = "T_multiply_intermediate_intermediate" if gelu else "T_add_intermediate_intermediate"
+    params = [Buffer("lv4", (N, K // 4), "uint32"), Buffer("lv5", (N, K // 32), "float16"), Buffer("lv3", (1, 1, K), "float16"),
+              Buffer("param_8", (N,), "float16"), Buffer(out, (1, 1, N), "float16")]
+    blocks = [Block("decode", "SS", ["lv4", "lv5"], ["decode_intermediate_intermediate"]),
+              Block("NT_matmul", "SSSR", ["lv3", "decode_intermediate_intermediate"], ["NT_matmul_intermediate"]),
+              Block("T_add", "SSS", ["NT_matmul_intermediate", "param_8"], [out if not gelu else "T_add_intermediate"])]
+    if gelu:
+        blocks.append(Block("T_multiply_2", "SSS", ["T_add_intermediate"], [out]))
+    return PrimFunc(name or ("fused_fused_decode4_fused_NT_matmul3_add2_gelu" if gelu else "fused_fused_decode2_fused_NT_matmul_add"),
+                    params, blocks, op="gemv_q8", attrs={"tir.noalias": True, "epilogue": 3 if gelu else 0})
+
+
 def module(*funcs: PrimFunc, upper_bound: Optional[dict] = None) -> IRModule:
     """An IRModule of the given PrimFuncs; ``upper_bound`` is the ``tir_var_upper_bound`` attribute
     (tuning_test/tune_cast.py:26 uses {"m": 512, "n": 4096})."""

@@ -218,6 +218,25 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
 int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int64_t n, int64_t m,
                      int64_t d, const dtas_config* cfg, void* stream);
 
+/* ---- 8-bit weights with fp16 group scales (the q8f16_1 layout of
+ * experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py) ----
+ * Wq[N, K/4] uint32: element j of a row is byte j % 4 of word j / 4; scale[N, K/32] fp16; K % 32 == 0.
+ *   W[i,j] = (fp16(byte) - fp16(127)) * scale[i, j/32]       (fp16 arithmetic: the product is rounded once)
+ *
+ * dtas_decode_q8_f16: fused_decode3 (:335-343), the dequantiser on its own: W[N,K] fp16 out.  cfg, when given:
+ *   {DTAS_ELT_VECTOR, block 256, vec 16 (one 128-bit access of weights) or 1}.
+ * dtas_gemv_q8_f16: y[N] = x[K] . W^T (+ bias[N]) with W dequantised in registers, never written:
+ *   fused_fused_decode2_fused_NT_matmul_add (:401-426; epilogue DTAS_EPI_BIAS) and
+ *   fused_fused_decode4_fused_NT_matmul3_add2_gelu (:428-502; DTAS_EPI_BIAS_GELU); fp32 accumulation, then
+ *   the fp16 steps of dtas_gemm_f16_fused.  cfg, when given, is a DTAS_GEMV_SPLITK row as for dtas_gemv_f16
+ *   (vec 8 = 128-bit accesses); NULL = 256 threads and 2 (N >= 16384: 4) rows per workgroup.
+ * The dynamic-n forms of these PrimFuncs (decode + GEMM, :371-399, :504-581) are served as the model's own
+ * graph serves fused_decode3: dtas_decode_q8_f16 into a caller-owned fp16 W, then dtas_gemm_f16_fused. */
+int dtas_decode_q8_f16(const void* Wq, const void* scale, void* W, int64_t N, int64_t K,
+                       const dtas_config* cfg, void* stream);
+int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale, const void* bias, void* y,
+                     int64_t N, int64_t K, int32_t epilogue, const dtas_config* cfg, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

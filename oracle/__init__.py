@@ -68,6 +68,8 @@ class _C:
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
                 "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
                 "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
+                "oracle_decode_q8_f16": [vp, vp, vp, i64, i64, ci],
+                "oracle_gemv_q8_f16": [vp, vp, vp, vp, vp, i64, i64, ci, ci, ci],
             }
             for name, argtypes in sig.items():
                 fn = getattr(lib, name)
@@ -181,6 +183,25 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         return out
 
     @staticmethod
+    def decode_q8(wq, scale, threads: int = 1) -> np.ndarray:
+        """fp16 W[N,K] of uint32 wq[N,K/4] (byte j % 4 of word j / 4) and fp16 scale[N,K/32]."""
+        N, K = wq.shape[0], wq.shape[1] * 4
+        assert wq.dtype == np.uint32 and scale.dtype == np.float16 and scale.shape == (N, K // 32)
+        out = np.empty((N, K), dtype=np.float16)
+        _C.lib().oracle_decode_q8_f16(_ptr(wq), _ptr(scale), _ptr(out), N, K, threads)
+        return out
+
+    @staticmethod
+    def gemv_q8(x, wq, scale, bias=None, kind: int = 0, acc_f16: bool = False, threads: int = 1) -> np.ndarray:
+        """fp16 y[N] = x[K] . decode_q8(wq, scale)^T (+ bias; kind 3: GELU)."""
+        N, K = wq.shape[0], wq.shape[1] * 4
+        assert x.dtype == np.float16 and x.size == K and scale.shape == (N, K // 32)
+        out = np.empty(x.shape[:-1] + (N,), dtype=np.float16)
+        bp = _ptr(bias) if bias is not None else None
+        _C.lib().oracle_gemv_q8_f16(_ptr(x), _ptr(wq), _ptr(scale), bp, _ptr(out), N, K, kind, int(acc_f16), threads)
+        return out
+
+    @staticmethod
     def gemm_f32out(a, w, threads: int = 1) -> np.ndarray:
         K = a.shape[-1]
         M, N = a.size // K, w.shape[0]
@@ -229,6 +250,11 @@ class np64:  # noqa: N801
     def attn_scores(q, k, mask, scale):
         s_ = np.einsum("hnd,hmd->hnm", q.astype(np.float64), k.astype(np.float64)) * float(np.float16(scale))
         return np.minimum(np.maximum(s_, -65504.0), mask.astype(np.float64)[None])
+
+    @staticmethod
+    def decode_q8(wq, scale):
+        q = wq.view(np.uint8).reshape(wq.shape[0], -1).astype(np.float64) - 127.0      # little endian: byte j of the row
+        return q * np.repeat(scale.astype(np.float64), 32, axis=1)
 
     @staticmethod
     def attn_pv(p, v):

@@ -381,6 +381,54 @@ void oracle_attn_pv_f16(const f16* P, const f16* V, f16* out, int64_t heads, int
   }
 }
 
+/* ========================================================================
+ * 8-bit weights with fp16 group scales (experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py)
+ *   decode[i, j] = (Cast("float16", (Wq[i, j/4] >> (8 * (j % 4))) & 255) - float16(127)) * S[i, j/32]
+ * fused_decode3 (:335-343) stores it; fused_fused_decode2_fused_NT_matmul_add (:401-426) and
+ * fused_fused_decode4_fused_NT_matmul3_add2_gelu (:428-502) multiply x by it (fp32 accumulation here,
+ * acc_f16 = 1 the literal fp16 running sum), then + bias (and GELU) in fp16 steps as in
+ * oracle_gemm_f16_fused.
+ * Pinned by: numpy float16 arithmetic on the bytes of the little-endian words (bit-exact), bytes
+ * 127 / 0 / 255 (0, -127 s, 128 s), the byte order inside a word, the scale group boundary at 32,
+ * float64 closed form; the GEMV equals the pinned GEMM oracle on the decoded matrix bit for bit.
+ * ======================================================================== */
+static f16 decode_q8(const uint32_t* Wq, const f16* S, int64_t K, int64_t i, int64_t j) {
+  const uint32_t byte = (Wq[i * (K / 4) + j / 4] >> (8 * (j % 4))) & 255u;
+  const f16 q = f2h(h2f(f2h((float)byte)) - 127.f);
+  return f2h(h2f(q) * h2f(S[i * (K / 32) + j / 32]));
+}
+
+void oracle_decode_q8_f16(const uint32_t* Wq, const f16* S, f16* W, int64_t N, int64_t K, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t ij = 0; ij < N * K; ++ij) W[ij] = decode_q8(Wq, S, K, ij / K, ij % K);
+}
+
+void oracle_gemv_q8_f16(const f16* x, const uint32_t* Wq, const f16* S, const f16* bias, f16* y, int64_t N, int64_t K,
+                        int kind, int acc_f16, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < N; ++i) {
+    f16 t;
+    if (acc_f16) {
+      f16 acc = 0;
+      for (int64_t k = 0; k < K; ++k) acc = f2h(h2f(acc) + h2f(f2h(h2f(x[k]) * h2f(decode_q8(Wq, S, K, i, k)))));
+      t = acc;
+    } else {
+      float acc = 0.f;
+      for (int64_t k = 0; k < K; ++k) acc = acc + h2f(x[k]) * h2f(decode_q8(Wq, S, K, i, k));
+      t = f2h(acc);
+    }
+    if (bias) t = f2h(h2f(t) + h2f(bias[i]));
+    if (kind == 3) {
+      const f16 m = f2h(h2f(t) * h2f(f2h(0.70710678118654757f)));
+      const f16 e = f2h(erff(h2f(m)));
+      const f16 h = f2h(h2f(e) * 0.5f);
+      const f16 g = f2h(0.5f + h2f(h));
+      t = f2h(h2f(t) * h2f(g));
+    }
+    y[i] = t;
+  }
+}
+
 int oracle_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

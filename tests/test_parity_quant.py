@@ -1,0 +1,139 @@
+"""GPU parity of the q8f16_1 kernels (dequantiser and dequantising GEMV,
+experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py:335-343, :401-426, :428-502) through the C ABI against the
+CPU oracle: the dequantised weights are bit-exact (integer bytes, one fp16 product); the GEMV is held to rtol 1e-2
+against float64 and to an fp16 ulp or two of the oracle (fp32 summation order)."""
+import numpy as np
+import pytest
+import torch
+
+from dtas_amd import _lib, ops
+from gpu_util import Guarded, cfg, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _weights(N, K, seed):
+    rng = np.random.default_rng(seed)
+    wq = rng.integers(0, 2 ** 32, (N, K // 4), dtype=np.uint32)
+    scale = (rng.random((N, K // 32)) * 0.02 + 0.001).astype(np.float16)
+    return wq, scale
+
+
+def _words(wq):
+    return torch.from_numpy(wq.view(np.int32)).cuda()
+
+
+@pytest.mark.parametrize("N,K", [(1, 32), (3, 96), (2560, 2560), (7680, 2560), (50, 10240)])
+def test_decode_is_bit_exact(oracle, N, K):
+    wq, scale = _weights(N, K, N + K)
+    out = Guarded((N, K), torch.float16)
+    ops.decode_q8(_words(wq), dev(scale), out.t)
+    assert np.array_equal(out.check().view(np.uint16), oracle.c.decode_q8(wq, scale, threads=8).view(np.uint16))
+
+
+def test_decode_every_byte_value_scalar_path_and_errors(oracle):
+    # all 256 byte values against scales that make the fp16 product round, overflow and go subnormal
+    wq = np.tile(np.arange(256, dtype=np.uint8), 4).reshape(4, 256).view(np.uint32)
+    scale = np.array([[1 / 3, 0.1, 7.0, 1e-3, 1.0, 6e-8, 0.5, 600.0]] * 4, np.float16)   # 600 * (255 - 127) overflows
+    want = oracle.c.decode_q8(np.ascontiguousarray(wq), scale)
+    for vec in (16, 1):
+        out = Guarded((4, 256), torch.float16)
+        ops.decode_q8(_words(np.ascontiguousarray(wq)), dev(scale), out.t, cfg(variant=_lib.ELT_VECTOR, block=256, vec=vec))
+        got = out.check()
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert np.isinf(want).any() and (want == 0).any()
+    # an output that is only 2-byte aligned takes the element path
+    buf = torch.empty(4 * 256 + 1, dtype=torch.float16, device="cuda")
+    ops.decode_q8(_words(np.ascontiguousarray(wq)), dev(scale), buf[1:].view(4, 256))
+    torch.cuda.synchronize()
+    assert np.array_equal(buf[1:].cpu().numpy().reshape(4, 256).view(np.uint16), want.view(np.uint16))
+    with pytest.raises(ValueError, match="groups of 32"):
+        ops.decode_q8(torch.zeros(2, 4, dtype=torch.int32, device="cuda"), torch.zeros(2, 1, dtype=torch.float16, device="cuda"),
+                      torch.zeros(2, 16, dtype=torch.float16, device="cuda"))
+    L = _lib.lib()
+    assert L.dtas_decode_q8_f16(None, None, None, 4, 48, None, None) == -1 and b"multiple of the scale group" in L.dtas_last_error()
+    assert L.dtas_decode_q8_f16(None, None, None, 0, 64, None, None) == 0
+
+
+def _check_gemv(got, x, wq, scale, bias, kind, oracle):
+    want = oracle.c.gemv_q8(x, wq, scale, bias, kind=kind, threads=8)
+    w64 = oracle.c.decode_q8(wq, scale, threads=8).astype(np.float64)
+    f64 = w64 @ x.astype(np.float64) + (bias.astype(np.float64) if bias is not None else 0.0)
+    if kind == _lib.EPI_BIAS_GELU:
+        from scipy.special import erf
+        f64 = f64 * (0.5 + 0.5 * erf(f64 * 0.70710678118654757))
+    mag = np.abs(w64) @ np.abs(x.astype(np.float64)) * 2.0 ** -11 + 2e-3       # what rounding the sum to fp16 can move
+    assert np.isfinite(got).all()
+    assert (np.abs(got.astype(np.float64) - f64) <= 1e-2 * np.abs(f64) + mag).all()
+    assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 2.0 ** -9 * np.abs(want) + 2e-3).all()
+    assert (got == want).mean() > 0.9
+
+
+@pytest.mark.parametrize("N,K", [(7680, 2560), (2560, 10240), (10240, 2560), (50280, 2560), (33, 64), (5, 32)])
+@pytest.mark.parametrize("kind", [_lib.EPI_BIAS, _lib.EPI_BIAS_GELU])
+def test_gemv_builtin_config(oracle, N, K, kind):
+    rng = np.random.default_rng(N + K + kind)
+    wq, scale = _weights(N, K, N * 3 + K)
+    x = rng.standard_normal(K).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    out = Guarded((1, 1, N), torch.float16)
+    ops.gemv_q8(dev(x).view(1, 1, K), _words(wq), dev(scale), dev(bias), out.t, None, kind)
+    _check_gemv(out.check().reshape(N), x, wq, scale, bias, kind, oracle)
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 8])
+@pytest.mark.parametrize("block", [64, 256, 512])
+def test_gemv_every_row_count_and_block(oracle, rows, block):
+    rng = np.random.default_rng(rows + block)
+    N, K = 101, 1056                       # N not a multiple of the rows per workgroup; K/16 = 66 chunks over up to 512 lanes
+    wq, scale = _weights(N, K, rows * 7 + block)
+    x = rng.standard_normal(K).astype(np.float16)
+    out = Guarded((N,), torch.float16)
+    ops.gemv_q8(dev(x), _words(wq), dev(scale), None, out.t, cfg(variant=_lib.GEMV_SPLITK, block=block, vec=8, unroll=2, tile=[rows, 0, 0]))
+    _check_gemv(out.check(), x, wq, scale, None, _lib.EPI_BIAS, oracle)
+
+
+def test_gemv_exact_cases_scalar_path_and_errors(oracle):
+    # a one-hot x picks a column of the dequantised matrix, bit for bit
+    wq, scale = _weights(64, 128, 5)
+    w = oracle.c.decode_q8(wq, scale)
+    for k in (0, 3, 31, 32, 127):
+        x = np.zeros(128, np.float16)
+        x[k] = 1
+        out = Guarded((64,), torch.float16)
+        ops.gemv_q8(dev(x), _words(wq), dev(scale), None, out.t)
+        assert np.array_equal(out.check().view(np.uint16), w[:, k].view(np.uint16))
+    # odd x pointer -> element path
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal(128).astype(np.float16)
+    xbuf = torch.empty(129, dtype=torch.float16, device="cuda")
+    xbuf[1:].copy_(dev(x))
+    out = Guarded((64,), torch.float16)
+    ops.gemv_q8(xbuf[1:], _words(wq), dev(scale), None, out.t)
+    _check_gemv(out.check(), x, wq, scale, None, _lib.EPI_BIAS, oracle)
+    y = torch.empty(64, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="epilogue must be"):
+        ops.gemv_q8(dev(x), _words(wq), dev(scale), None, y, None, _lib.EPI_BIAS_ADD2)
+    assert _lib.lib().dtas_gemv_q8_f16(None, None, None, None, None, 0, 64, 0, None, None) == 0
+
+
+def test_q8_through_the_primfunc_descriptors_and_engine(oracle):
+    from dtas_amd import primfuncs as pf
+    from dtas_amd.arch import MI355X
+    from dtas_amd.engine.tuner import Engine
+
+    rng = np.random.default_rng(8)
+    N, K = 7680, 2560
+    wq, scale = _weights(N, K, 9)
+    x = rng.standard_normal(K).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    mod = pf.module(pf.fused_decode_NT_matmul_add(N, K), pf.fused_decode(N, K), pf.matmul_pv(32, 80, decode=True))
+    rt = Engine(topk=2, parallel_build=False).tune_module(mod, MI355X())
+    assert rt.entry_for("fused_fused_decode2_fused_NT_matmul_add") is None      # the library's own choice
+    y = torch.empty(1, 1, N, dtype=torch.float16, device="cuda")
+    rt["fused_fused_decode2_fused_NT_matmul_add"](_words(wq), dev(scale), dev(x).view(1, 1, K), dev(bias), y)
+    W = torch.empty(N, K, dtype=torch.float16, device="cuda")
+    rt["fused_decode3"](_words(wq), dev(scale), W)
+    torch.cuda.synchronize()
+    _check_gemv(y.cpu().numpy().reshape(N), x, wq, scale, bias, _lib.EPI_BIAS, oracle)
+    assert np.array_equal(W.cpu().numpy().view(np.uint16), oracle.c.decode_q8(wq, scale, threads=8).view(np.uint16))
