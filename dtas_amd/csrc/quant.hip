@@ -28,26 +28,36 @@ __device__ __forceinline__ void dequant_word(unsigned word, f16x2 scale2, f16x2&
   hi = (__builtin_bit_cast(f16x2, phi) - bias2) * scale2;
 }
 
-// One thread = 16 weights (16 bytes in, 32 bytes out).  K % 32 == 0, so a thread's 16 weights share a
-// scale and the flat scale index is (16 i) / 32.
-__global__ void __launch_bounds__(256) decode_q8_kernel(const u32x4* __restrict__ Wq, const half_t* __restrict__ S,
-                                                        u32x4* __restrict__ W, int64_t chunks) {
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < chunks;
-       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const u32x4 q = load_stream(Wq + i);
-    const half_t s = S[i >> 1];
-    const f16x2 s2 = {s, s};
-    u32x4 out[2];
+// One item = 8 weights: 8 bytes in, 16 bytes out, so that a wavefront's loads and stores are each one
+// contiguous span (512 bytes in, 1 KiB out).  A thread requests four items, a grid stride apart, before
+// it uses the first.  K % 32 == 0, so an item's weights share a scale and the flat scale index is (8 i) / 32.
+__global__ void __launch_bounds__(256) decode_q8_kernel(const u32x2* __restrict__ Wq, const half_t* __restrict__ S,
+                                                        u32x4* __restrict__ W, int64_t items) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i0 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i0 < items; i0 += 4 * stride) {
+    u32x2 q[4];
+    half_t s[4];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      f16x2 lo, hi;
-      const unsigned word = q[w];
-      dequant_word(word, s2, lo, hi);
-      out[w >> 1][(w & 1) * 2] = __builtin_bit_cast(unsigned, lo);
-      out[w >> 1][(w & 1) * 2 + 1] = __builtin_bit_cast(unsigned, hi);
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i < items) {
+        q[u] = load_stream(Wq + i);
+        s[u] = S[i >> 2];
+      }
     }
-    store_stream(out[0], W + 2 * i);
-    store_stream(out[1], W + 2 * i + 1);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i >= items) break;
+      const f16x2 s2 = {s[u], s[u]};
+      f16x2 a, b, c, d;
+      const unsigned w0 = q[u][0], w1 = q[u][1];
+      dequant_word(w0, s2, a, b);
+      dequant_word(w1, s2, c, d);
+      const u32x4 out = {__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, c),
+                         __builtin_bit_cast(unsigned, d)};
+      store_stream(out, W + i);
+    }
   }
 }
 
@@ -165,17 +175,17 @@ extern "C" int dtas_decode_q8_f16(const void* Wq, const void* scale, void* W, in
   if (!Wq || !scale || !W) return fail("decode_q8: NULL buffer");
   if (overlaps(W, N * K * 2, Wq, N * K) || overlaps(W, N * K * 2, scale, N * (K / 32) * 2))
     return fail("decode_q8: output overlaps an input");
-  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, 256, 16, 1, {0, 0, 0}, 1, 0};
+  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, 256, 8, 1, {0, 0, 0}, 1, 0};
   if (cfg.block != 256) return fail("decode_q8: the kernels use 256 threads, got %d", cfg.block);
-  if (cfg.vec != 16 && cfg.vec != 1) return fail("decode_q8: vector width must be 16 (128 bits of weights) or 1, got %d", cfg.vec);
-  if (cfg.vec == 16 && !(aligned(Wq, 16) && aligned(W, 16))) cfg.vec = 1;
+  if (cfg.vec != 8 && cfg.vec != 1) return fail("decode_q8: vector width must be 8 (128-bit stores) or 1, got %d", cfg.vec);
+  if (cfg.vec == 8 && !(aligned(Wq, 8) && aligned(W, 16))) cfg.vec = 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t items = cfg.vec == 16 ? N * K / 16 : N * K;
-  int64_t grid = ceil_div(items, 256);
+  const int64_t items = cfg.vec == 8 ? N * K / 8 : N * K;
+  int64_t grid = ceil_div(items, cfg.vec == 8 ? 4 * 256 : 256);
   const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
   grid = grid > cap ? cap : grid;
-  if (cfg.vec == 16)
-    hipLaunchKernelGGL(decode_q8_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x4*>(Wq),
+  if (cfg.vec == 8)
+    hipLaunchKernelGGL(decode_q8_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x2*>(Wq),
                        static_cast<const half_t*>(scale), static_cast<u32x4*>(W), items);
   else
     hipLaunchKernelGGL(decode_q8_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s,

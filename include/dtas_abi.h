@@ -224,7 +224,7 @@ int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int
  *   W[i,j] = (fp16(byte) - fp16(127)) * scale[i, j/32]       (fp16 arithmetic: the product is rounded once)
  *
  * dtas_decode_q8_f16: fused_decode3 (:335-343), the dequantiser on its own: W[N,K] fp16 out.  cfg, when given:
- *   {DTAS_ELT_VECTOR, block 256, vec 16 (one 128-bit access of weights) or 1}.
+ *   {DTAS_ELT_VECTOR, block 256, vec 8 (8 weights per access: 128-bit stores) or 1}.
  * dtas_gemv_q8_f16: y[N] = x[K] . W^T (+ bias[N]) with W dequantised in registers, never written:
  *   fused_fused_decode2_fused_NT_matmul_add (:401-426; epilogue DTAS_EPI_BIAS) and
  *   fused_fused_decode4_fused_NT_matmul3_add2_gelu (:428-502; DTAS_EPI_BIAS_GELU); fp32 accumulation, then

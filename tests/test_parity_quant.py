@@ -36,7 +36,7 @@ def test_decode_every_byte_value_scalar_path_and_errors(oracle):
     wq = np.tile(np.arange(256, dtype=np.uint8), 4).reshape(4, 256).view(np.uint32)
     scale = np.array([[1 / 3, 0.1, 7.0, 1e-3, 1.0, 6e-8, 0.5, 600.0]] * 4, np.float16)   # 600 * (255 - 127) overflows
     want = oracle.c.decode_q8(np.ascontiguousarray(wq), scale)
-    for vec in (16, 1):
+    for vec in (8, 1):
         out = Guarded((4, 256), torch.float16)
         ops.decode_q8(_words(np.ascontiguousarray(wq)), dev(scale), out.t, cfg(variant=_lib.ELT_VECTOR, block=256, vec=vec))
         got = out.check()
