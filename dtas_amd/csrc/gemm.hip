@@ -75,8 +75,11 @@ struct GemmEpilogue {
   int kind;            // enum dtas_epilogue, or kEpiScores
   int out_f32;         // the output buffer holds fp32 (ADD2_CAST_F32, scores)
   float scale;         // scores: the fp16 constant the product is multiplied by
-  // batched launches (grid.y = batch): element strides between consecutive problems
+  // batched launches: element strides between consecutive problems, and how many there are (the MFMA
+  // launcher fills `batches`; the element-access kernel takes the problem from blockIdx.y)
   int64_t stride_a, stride_w, stride_c, stride_res;
+  unsigned batches;
+  unsigned tiles_pinned;  // batched launches: an XCD keeps its tiles and walks the problems (see the kernel)
 };
 
 // Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):
@@ -168,21 +171,34 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const unsigned t = threadIdx.x, l = t & 63u;
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
 
-  // ---- which problem of a batched launch
-  const int64_t batch = blockIdx.y;
+  // ---- which problem of a batched launch, which tile.  Workgroup ids are dealt round-robin over the
+  // XCDs; xcd_contiguous_id gives each XCD a contiguous span of (problem, tile) instead, so the tiles of
+  // one problem (which share its W -- the keys or values of an attention head) meet in one L2.
+  // With ep.tiles_pinned (the scores: every problem reads the same mask) an XCD instead keeps one
+  // span of tiles and walks the problems, so its part of the shared operand stays in its L2.
+  const unsigned total = tiles_m * tiles_n, per_batch = total * nsplit;
+  // (divisions run on the vector ALU; pinning the results to scalar registers keeps every address
+  // and buffer descriptor derived from them scalar -- a descriptor left in vector registers turns
+  // each load into a loop over its distinct values)
+  unsigned batch_u, wgid;
+  if (ep.tiles_pinned && per_batch % kNumXCD == 0) {
+    const unsigned span = per_batch / kNumXCD, xcd = blockIdx.x % kNumXCD, local = blockIdx.x / kNumXCD;
+    batch_u = __builtin_amdgcn_readfirstlane(local / span);
+    wgid = xcd * span + local % span;
+  } else {
+    const unsigned gid = xcd_contiguous_id(blockIdx.x, per_batch * ep.batches);
+    batch_u = __builtin_amdgcn_readfirstlane(gid / per_batch);
+    wgid = gid - batch_u * per_batch;
+  }
+  const int64_t batch = batch_u;
   A += batch * ep.stride_a;
   W += batch * ep.stride_w;
   C = static_cast<char*>(C) + batch * ep.stride_c * (ep.out_f32 ? 4 : 2);
   if (ep.res1) ep.res1 += batch * ep.stride_res;
   if (ep.res2) ep.res2 += batch * ep.stride_res;
 
-  // ---- which tile: XCD-contiguous order, then groups of 8 tile rows walked column-wise
+  // ---- tiles in groups of 8 tile rows walked column-wise
   // nsplit > 1: nsplit consecutive workgroups (same XCD) share a tile and split its k tiles
-  const unsigned total = tiles_m * tiles_n;
-  const unsigned wgid = xcd_contiguous_id(blockIdx.x, total * nsplit);
-  // (divisions run on the vector ALU; pinning the results to scalar registers keeps every address
-  // and buffer descriptor derived from them scalar -- a descriptor left in vector registers turns
-  // each load into a loop over its distinct values)
   const unsigned pid = __builtin_amdgcn_readfirstlane(wgid / nsplit), z = __builtin_amdgcn_readfirstlane(wgid % nsplit);
   constexpr unsigned kGroup = 8;
   const unsigned width = kGroup * tiles_n;
@@ -1056,8 +1072,11 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   }
   if (batch > 1 && nsplit > 1) return fail("gemm: a batched launch cannot split K");
   if (batch < 1 || batch > 65535) return fail("gemm: batch must be in [1, 65535], got %d", batch);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT>), dim3(static_cast<unsigned>(tiles * nsplit), batch), dim3(64 * WM * WN), 0,
-                     s, A, W, ep, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
+  if (tiles * nsplit * batch > 0x7fffffffu) return fail("gemm: too many workgroups");
+  GemmEpilogue batched = ep;
+  batched.batches = static_cast<unsigned>(batch);
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT>), dim3(static_cast<unsigned>(tiles * nsplit * batch)), dim3(64 * WM * WN), 0,
+                     s, A, W, batched, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
 
@@ -1235,7 +1254,10 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   int64_t la[7];
   if (describe_gemm(n, m, d, cfg, la) != 0) return -1;
   GemmEpilogue ep = {nullptr, static_cast<const half_t*>(mask), nullptr, kEpiScores, 1,
-                     static_cast<float>(static_cast<half_t>(scale)), n * d, m * d, n * m, 0};
+                     static_cast<float>(static_cast<half_t>(scale)), n * d, m * d, n * m, 0, 1,
+                     // a mask beyond an L2's reach (4 MiB) is kept in place, one part per XCD; below that
+                     // the heads' keys gain more from contiguous spans (measured at n = m = 512 .. 2048)
+                     n * m >= (int64_t{1} << 21) ? 1u : 0u};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const half_t* a = static_cast<const half_t*>(Q);
   const half_t* w = static_cast<const half_t*>(Kmat);
