@@ -615,16 +615,29 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     for (; kt < ktiles; ++kt) k_tile(kt, false);
   } else {
   // two stages: tile 0 resident, tile 1 in flight, fragments of (tile 0, step 0) in registers
+  // (row-major W: tile 1 is requested together with tile 0 -- both stages are free -- and only tile 0
+  // is waited for; with two k tiles in all, as in the attention scores, that is one round trip less)
   if (ktiles > 0) {
     fetch(0);
     if constexpr (WT) { wt_load(0); wt_commit(0); }
   }
-  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  if constexpr (!WT) {
+    if (1 < ktiles) {
+      fetch(1);
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA + LB));  // tile 1's loads may stay outstanding
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0070);
+    }
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  }
   __builtin_amdgcn_s_barrier();
   DTAS_SCHED_FENCE();
-  if (1 < ktiles) {
-    fetch(1);
-    if constexpr (WT) wt_load(1);
+  if constexpr (WT) {
+    if (1 < ktiles) {
+      fetch(1);
+      wt_load(1);
+    }
   }
   if (ktiles > 0) {
 #pragma unroll
@@ -762,7 +775,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // as many as the registers hold (two per vector): all 32 for one operand, 16 for two; erf's code
     // is long, so its loop body stays small
     constexpr int kWant = KIND == DTAS_EPI_BIAS_GELU ? 2 : kAdd2 ? 16 : kUseR1 ? 32 : 4;
-    constexpr int G = kPasses % kWant == 0 ? kWant : (kPasses % 8 == 0 ? 8 : (kPasses % 4 == 0 ? 4 : 1));
+    constexpr int G = kPasses <= kWant ? kPasses : kPasses % kWant == 0 ? kWant : (kPasses % 8 == 0 ? 8 : (kPasses % 4 == 0 ? 4 : 1));
 #pragma unroll 1
     for (int p0 = 0; p0 < kPasses; p0 += G) {
       f16x4 r1v[G] = {}, r2v[G] = {};
@@ -829,6 +842,156 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     case DTAS_EPI_BIAS_GELU: store_tile(std::integral_constant<int, DTAS_EPI_BIAS_GELU>{}); break;
     case kEpiScores: store_tile(std::integral_constant<int, kEpiScores>{}); break;
     default: store_tile(std::integral_constant<int, DTAS_EPI_BIAS>{}); break;
+  }
+}
+
+// Attention scores for head dimensions up to 128 (two k tiles): out[h] = epilogue(Q[h] . K[h]^T).
+// What the op moves is its fp32 output, and a workgroup of the general kernel lives mostly in two
+// waits -- for its operands, then for its stores to drain -- while its LDS keeps further workgroups
+// off the CU.  Here a workgroup walks tiles (stride = grid): it requests the whole Q and K tiles and
+// its part of the mask at once, multiplies, stages the result through the LDS and issues the stores;
+// the next tile's loads are then in flight together with those stores.  Tiles are numbered as the
+// batched launches of gemm_mfma_kernel number their workgroups (an XCD keeps one span of tiles when
+// `pinned`, so its part of the mask stays in its L2); operand layout in the LDS as there.
+template <int BM, int BN>
+__global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kmat,
+                                                          const half_t* __restrict__ mask, float* __restrict__ out,
+                                                          int64_t n, int64_t m, int64_t d, float scale, unsigned tiles_m,
+                                                          unsigned tiles_n, unsigned heads, unsigned pinned) {
+  constexpr int NW = 4, WN = 2, WTM = BM / 2, WTN = BN / 2, MT = WTM / 32, NT = WTN / 32;
+  constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
+  constexpr int kABytes = BM * kRowBytes, kStage = (BM + BN) * kRowBytes;
+  static_assert(BM * BN * 2 <= 2 * kStage, "epilogue staging must fit the operand tiles");
+  __shared__ __attribute__((aligned(1024))) char lds[2 * kStage];
+
+  const unsigned t = threadIdx.x, l = t & 63u;
+  const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
+  const int ktiles = static_cast<int>((d + kBK - 1) / kBK);  // 1 or 2
+  const unsigned row_bytes = static_cast<unsigned>(d) * 2u;
+  const unsigned r_in = 2u * (l >> 4) + (((l >> 3) & 1u) ^ (wv & 1u));
+  const unsigned c_in = (l & 7u) ^ r_in;
+  const unsigned g_off = (8u * wv + r_in) * row_bytes + c_in * 16u;
+  const unsigned g_step = 8u * NW * row_bytes;
+  unsigned lds_rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) lds_rd[ks] = lds_chunk_offset(l & 31u, 2u * ks + (l >> 5));
+  const unsigned a_base = wm * WTM * 128u, b_base = kABytes + wn * WTN * 128u;
+
+  constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots, kPasses = WTM / kRowsPerPass;
+  const unsigned slot = l % kSlots, rsub = l / kSlots;
+  char* region = lds + wv * (WTM * kRowB);
+  const bool ptr_ok = (m % 4 == 0) && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
+
+  const unsigned per_batch = tiles_m * tiles_n, total = per_batch * heads;
+  for (unsigned tix = blockIdx.x; tix < total; tix += gridDim.x) {
+    unsigned batch, pid;
+    if (pinned && per_batch % kNumXCD == 0) {
+      const unsigned span = per_batch / kNumXCD, xcd = tix % kNumXCD, local = tix / kNumXCD;
+      batch = __builtin_amdgcn_readfirstlane(local / span);
+      pid = __builtin_amdgcn_readfirstlane(xcd * span + local % span);
+    } else {
+      const unsigned gid = xcd_contiguous_id(tix, total);
+      batch = __builtin_amdgcn_readfirstlane(gid / per_batch);
+      pid = __builtin_amdgcn_readfirstlane(gid % per_batch);
+    }
+    const unsigned tm = __builtin_amdgcn_readfirstlane(pid / tiles_n), tn = __builtin_amdgcn_readfirstlane(pid % tiles_n);
+    const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
+    const int64_t rows_a = n - m0 < BM ? n - m0 : BM, rows_w = m - n0 < BN ? m - n0 : BN;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Q + (static_cast<int64_t>(batch) * n + m0) * d, static_cast<unsigned>(rows_a) * row_bytes);
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(Kmat + (static_cast<int64_t>(batch) * m + n0) * d, static_cast<unsigned>(rows_w) * row_bytes);
+    // ---- every k tile of both operands, asynchronously (rows past the extents and the K tail read as zeros)
+    for (int kt = 0; kt < ktiles; ++kt) {
+      const unsigned off = (static_cast<int64_t>(kt) * kBK + c_in * 8 < d) ? g_off + static_cast<unsigned>(kt) * kRowBytes : kOob;
+      char* base = lds + kt * kStage + wv * 1024;
+#pragma unroll
+      for (int i = 0; i < LA; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, 0);
+#pragma unroll
+      for (int i = 0; i < LB; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
+    }
+    // ---- this lane's part of the mask tile
+    const int64_t col = n0 + wn * WTN + slot * 4;
+    const bool vec_ok = ptr_ok && col + 3 < m;
+    f16x4 mk[kPasses];
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int64_t row = m0 + wm * WTM + p * kRowsPerPass + rsub;
+      const f16x4 zero = {};
+      mk[p] = zero;
+      if (row >= n) continue;
+      if (vec_ok) {
+        mk[p] = *reinterpret_cast<const f16x4*>(mask + row * m + col);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < m) mk[p][e] = mask[row * m + col + e];
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // the operands have landed (and the previous tile's stores have left)
+    __builtin_amdgcn_s_barrier();
+
+    f32x16 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    for (int kt = 0; kt < ktiles; ++kt) {
+      const char* stage = lds + kt * kStage;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        f16x8 fa[MT], fb[NT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const f16x8*>(stage + a_base + i * 4096 + lds_rd[ks]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const f16x8*>(stage + b_base + j * 4096 + lds_rd[ks]);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+      }
+    }
+    __syncthreads();  // every wavefront is done with the operand tiles
+
+    // ---- epilogue: acc[i][j][v] of lane l is row i*32 + (l & 31), column j*32 + 8*(v/4) + 4*(l >> 5) + v%4 of
+    // the wavefront tile; staged in a wavefront-private LDS region (8-byte slots, xor-swizzled by the row)
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const unsigned mr = i * 32 + (l & 31u);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f16x4 hv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(acc[i][j][g * 4 + e]);
+          const unsigned sl = j * 8 + g * 2 + (l >> 5);
+          *reinterpret_cast<f16x4*>(region + mr * kRowB + ((sl ^ (mr & (kSlots - 1))) * 8)) = hv;
+        }
+    }
+    // no barrier: a wavefront reads back only what it wrote itself
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const unsigned mr = p * kRowsPerPass + rsub;
+      f16x4 hv = *reinterpret_cast<const f16x4*>(region + mr * kRowB + ((slot ^ (mr & (kSlots - 1))) * 8));
+      const int64_t row = m0 + wm * WTM + mr;
+      if (row >= n) continue;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        hv[e] = epilogue_value_k<kEpiScores>(hv[e], false, scale, 0.f, static_cast<float>(mk[p][e]), 0.f);
+      float* dst = out + (static_cast<int64_t>(batch) * n + row) * m + col;
+      if (vec_ok) {
+        const f32x4v wide = {static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]), static_cast<float>(hv[3])};
+        __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));  // 4*heads*n*m bytes: streamed
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (col + e < m) dst[e] = static_cast<float>(hv[e]);
+      }
+    }
+    __syncthreads();  // the staging regions are free: the next tile's operands may land
   }
 }
 
@@ -1238,6 +1401,18 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   if (overlaps(out, heads * n * m * 4, Q, heads * n * d * 2) || overlaps(out, heads * n * m * 4, Kmat, heads * m * d * 2) ||
       overlaps(out, heads * n * m * 4, mask, n * m * 2))
     return fail("attn_scores: output overlaps an input");
+  if (!user && d <= 2 * kBK) {
+    // the walking kernel: 128x64 tiles, at most three workgroups per CU (their LDS allows no more)
+    const unsigned tm = static_cast<unsigned>(ceil_div(n, 128)), tn = static_cast<unsigned>(ceil_div(m, 64));
+    const int64_t total = static_cast<int64_t>(tm) * tn * heads;
+    if (total > 0x7fffffff) return fail("attn_scores: too many tiles");
+    const int64_t grid = total < 3 * kNumCU ? total : 3 * kNumCU;
+    hipLaunchKernelGGL((attn_scores_kernel<128, 64>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const half_t*>(Q), static_cast<const half_t*>(Kmat), static_cast<const half_t*>(mask),
+                       static_cast<float*>(out), n, m, d, static_cast<float>(static_cast<half_t>(scale)), tm, tn,
+                       static_cast<unsigned>(heads), n * m >= (int64_t{1} << 21) ? 1u : 0u);
+    return check_launch("attn_scores");
+  }
   dtas_config cfg;
   if (user) {
     cfg = *user;

@@ -38,6 +38,17 @@ def test_scores_builtin_config(oracle, n, m):
     _check(out.check().reshape(32, n, m), q, k, mask, oracle)
 
 
+@pytest.mark.parametrize("heads,n,m,d", [(3, 70, 131, 8), (2, 129, 65, 64), (5, 300, 260, 128), (2, 100, 90, 136), (1, 1, 3, 72),
+                                         (40, 520, 512, 80)])
+def test_scores_builtin_other_head_dims(oracle, heads, n, m, d):
+    # d <= 128 is served by the kernel that walks tiles (one or two k tiles), beyond that by the general one;
+    # 40 heads x 5 x 8 tiles = 1600 tiles: more than one tile per workgroup
+    q, k, mask = _inputs(heads, n, m, d, n + m + d)
+    out = Guarded((heads, n, m), torch.float32)
+    ops.attn_scores(dev(q), dev(k), dev(mask), out.t, SCALE)
+    _check(out.check(), q, k, mask, oracle)
+
+
 @pytest.mark.parametrize("tile,block,stages", [((64, 64), 256, 2), ((64, 64), 256, 3), ((128, 128), 256, 2), ((128, 64), 256, 2),
                                                ((64, 128), 256, 2), ((256, 128), 256, 2), ((256, 256), 512, 2), ((256, 256), 256, 2)])
 @pytest.mark.parametrize("heads,n,m,d", [(3, 70, 131, 80), (2, 300, 260, 64), (1, 33, 7, 8)])
