@@ -100,10 +100,31 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* slots, int
 
 // ---- erf-GELU on an fp16 value, every step an fp16 tensor as the fused PrimFuncs spell it
 // (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:248-318): t * (0.5 + 0.5 * erf(t * fp16(0.7071...)))
+// erf of a value that is an fp16 number, for a result that is rounded to fp16: x * P(x^2) with P a
+// degree-10 polynomial fitted for relative error on [0, 2.75], +-1 beyond (erf rounds to 1.0 in fp16 from
+// 2.596 on).  Over all 63 488 finite fp16 inputs the rounded result differs from libm's erff rounded in
+// 6 (by one fp16 ulp); it costs 15 instructions where erff costs ~35, which the GELU epilogue of a GEMM
+// pays per output element.
+__device__ __forceinline__ float erf_of_f16(float x) {
+  const float t = fmaf(x * x, 0.2644628f, -1.f);
+  float p = 3.507727815e-04f;
+  p = fmaf(p, t, -1.175096375e-03f);
+  p = fmaf(p, t, 2.496362897e-03f);
+  p = fmaf(p, t, -6.172187161e-03f);
+  p = fmaf(p, t, 1.496723015e-02f);
+  p = fmaf(p, t, -3.152125701e-02f);
+  p = fmaf(p, t, 5.924283713e-02f);
+  p = fmaf(p, t, -1.007829085e-01f);
+  p = fmaf(p, t, 1.577374041e-01f);
+  p = fmaf(p, t, -2.427380979e-01f);
+  p = fmaf(p, t, 5.111947656e-01f);
+  return fabsf(x) >= 2.75f ? copysignf(1.f, x) : x * p;
+}
+
 __device__ __forceinline__ half_t gelu_erf_f16_steps(half_t t) {
   const float x = static_cast<float>(t);
   const half_t m = static_cast<half_t>(x * static_cast<float>(static_cast<half_t>(0.70710678118654757f)));
-  const half_t e = static_cast<half_t>(erff(static_cast<float>(m)));
+  const half_t e = static_cast<half_t>(erf_of_f16(static_cast<float>(m)));
   const half_t h = static_cast<half_t>(static_cast<float>(e) * 0.5f);
   const half_t a = static_cast<half_t>(0.5f + static_cast<float>(h));
   return static_cast<half_t>(x * static_cast<float>(a));

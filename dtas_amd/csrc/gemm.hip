@@ -772,9 +772,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // passes in groups of G: the group's residual / mask vectors are requested together, before the
     // first of them is needed (one at a time, every pass would wait out a memory round trip)
     constexpr int kPasses = WTM / kRowsPerPass;
-    // as many as the registers hold (two per vector): all 32 for one operand, 16 for two; erf's code
-    // is long, so its loop body stays small
-    constexpr int kWant = KIND == DTAS_EPI_BIAS_GELU ? 2 : kAdd2 ? 16 : kUseR1 ? 32 : 4;
+    // as many as the registers hold (two per vector): all 32 for one operand, 16 for two
+    constexpr int kWant = KIND == DTAS_EPI_BIAS_GELU ? 4 : kAdd2 ? 16 : kUseR1 ? 32 : 4;
     constexpr int G = kPasses <= kWant ? kPasses : kPasses % kWant == 0 ? kWant : (kPasses % 8 == 0 ? 8 : (kPasses % 4 == 0 ? 4 : 1));
 #pragma unroll 1
     for (int p0 = 0; p0 < kPasses; p0 += G) {

@@ -302,3 +302,24 @@ def test_gemm_fused_argument_errors():
                                                   8, 16, 16, 9, None, None), "fused")
     with pytest.raises(ValueError, match="fp32 C"):
         ops.gemm(dev(a), dev(w), None, out, None, epilogue=_lib.EPI_BIAS_ADD2_CAST_F32, res1=dev(r1), res2=dev(r2))
+
+
+def test_gelu_over_every_fp16_preactivation(oracle):
+    """A product that is exactly x (one 1 in W) for every finite fp16 x: the epilogue's erf is a polynomial
+    fitted for fp16 inputs and outputs, the oracle's is libm's; the rounded results may differ in a handful
+    of the 63 488 values, by one fp16 ulp."""
+    bits = np.concatenate([np.arange(0, 0x7c00, dtype=np.uint16), np.arange(0x8000, 0xfc00, dtype=np.uint16)])
+    a = np.zeros((bits.size, 8), np.float16)
+    a[:, 0] = bits.view(np.float16)
+    w = np.zeros((8, 8), np.float16)
+    w[:, 0] = 1                                                       # every column of C repeats x
+    want = oracle.c.gemm_fused(a, w, None, None, None, 3, threads=8)
+    for conf in (None, dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64])):
+        out = Guarded((bits.size, 8), torch.float16)
+        ops.gemm(dev(a), dev(w), None, out.t, cfg(**conf) if conf else None, epilogue=_lib.EPI_BIAS_GELU)
+        got = out.check()
+        assert np.isfinite(got).all()
+        diff = got.view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32)
+        assert np.abs(diff).max() <= 1
+        assert (diff[:, 0] != 0).sum() <= 16, (diff[:, 0] != 0).sum()
+    # the decode path (q8 GEMV) and the skinny kernel share the same steps
