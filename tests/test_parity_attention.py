@@ -192,3 +192,50 @@ def test_pv_through_the_primfunc_descriptors(oracle):
         call_primfunc(func, tensors)
         torch.cuda.synchronize()
         _check_pv(out.cpu().numpy().reshape(32, n, 80), p, v, oracle)
+
+
+def test_attention_full_size_properties(oracle):
+    """n = m = 2048, 32 heads of 80 (268 M scores): properties that need no oracle pass over the whole output,
+    plus sampled rows against the oracle."""
+    heads, n, d = 32, 2048, 80
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randn(heads, n, d, device="cuda", generator=g).half()
+    k = torch.randn(heads, n, d, device="cuda", generator=g).half()
+    causal = torch.ones(n, n, device="cuda").tril_().bool()
+    mask = torch.where(causal, torch.tensor(65504.0, device="cuda"), torch.tensor(-65504.0, device="cuda")).half()
+    sc = torch.empty(heads, n, n, dtype=torch.float32, device="cuda")
+    ops.attn_scores(q, k, mask, sc, SCALE)
+    torch.cuda.synchronize()
+    assert bool((sc[:, ~causal] == -65504.0).all())                          # the masked set is exact
+    assert bool(torch.isfinite(sc).all()) and bool((sc[:, causal] > -65504.0).all())
+    assert bool((sc.half().float() == sc).all())                             # every score is an fp16 value widened
+    open_mask = torch.full((n, n), 65504.0, dtype=torch.float16, device="cuda")
+    sc2 = torch.empty_like(sc)
+    ops.attn_scores(q, k, open_mask, sc2, SCALE)
+    assert bool((sc2[:, causal] == sc[:, causal]).all())                      # the mask only takes a minimum
+    ops.attn_scores(k, q, open_mask, sc, SCALE)                              # (Q K^T)^T = K Q^T, bit for bit
+    assert bool((sc.transpose(1, 2) == sc2).all())
+    rows = [0, 1, 777, 2047]
+    qn, kn = q.cpu().numpy(), k.cpu().numpy()
+    want = oracle.c.attn_scores(np.ascontiguousarray(qn[:, rows]), kn, np.full((len(rows), n), 65504.0, np.float16), SCALE, threads=8)
+    got = sc2[:, rows].cpu().numpy()
+    assert (np.abs(got - want) <= 1e-3 + 2.0 ** -9 * np.abs(want)).all() and (got == want).mean() > 0.98
+    del sc, sc2
+
+    # P.V: a permutation matrix as P returns the permuted rows of V exactly; rows that sum to one return
+    # values inside V's range; sampled rows against the oracle
+    v = torch.randn(heads, n, d, device="cuda", generator=g).half()
+    perm = torch.randperm(n, device="cuda", generator=g)
+    p = torch.zeros(heads, n, n, dtype=torch.float16, device="cuda")
+    p[:, torch.arange(n, device="cuda"), perm] = 1
+    o = torch.empty(heads, n, d, dtype=torch.float16, device="cuda")
+    ops.attn_pv(p, v, o)
+    assert bool((o == v[:, perm]).all())
+    p = torch.softmax(torch.randn(heads, n, n, device="cuda", generator=g), -1).half()
+    ops.attn_pv(p, v, o)
+    torch.cuda.synchronize()
+    assert bool((o.float().abs().amax(1) <= v.float().abs().amax(1) * 1.01).all())
+    pn, vn = p.cpu().numpy(), v.cpu().numpy()
+    want = oracle.c.attn_pv(np.ascontiguousarray(pn[:, rows]), vn, threads=8).astype(np.float64)
+    got = o[:, rows].cpu().numpy().astype(np.float64)
+    assert (np.abs(got - want) <= 1e-4 + 2.0 ** -9 * np.abs(want)).all()

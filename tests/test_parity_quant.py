@@ -137,3 +137,34 @@ def test_q8_through_the_primfunc_descriptors_and_engine(oracle):
     torch.cuda.synchronize()
     _check_gemv(y.cpu().numpy().reshape(N), x, wq, scale, bias, _lib.EPI_BIAS, oracle)
     assert np.array_equal(W.cpu().numpy().view(np.uint16), oracle.c.decode_q8(wq, scale, threads=8).view(np.uint16))
+
+
+def test_q8_full_size_properties(oracle):
+    """The embedding-sized matrix (50280 x 2560) and the benchmark's largest GEMV (32000 x 4096): dequantising
+    twice gives the same bits, the GEMV is linear in x for exactly representable data, and a one-hot x returns a
+    column of the dequantised matrix."""
+    for N, K in ((50280, 2560), (32000, 4096)):
+        g = torch.Generator(device="cuda").manual_seed(N)
+        words = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device="cuda", generator=g)
+        scale = (torch.rand(N, K // 32, device="cuda", generator=g) * 0.02 + 0.001).half()
+        W = torch.empty(N, K, dtype=torch.float16, device="cuda")
+        ops.decode_q8(words, scale, W)
+        torch.cuda.synchronize()
+        # against torch's own arithmetic on the bytes (little endian), every element
+        by = words.view(torch.uint8).view(N, K).to(torch.float16) - 127
+        assert bool((W == by * scale.repeat_interleave(32, dim=1)).all())
+        del by
+        y = torch.empty(N, dtype=torch.float16, device="cuda")
+        for kcol in (0, 31, 32, K - 1):
+            x = torch.zeros(K, dtype=torch.float16, device="cuda")
+            x[kcol] = 1
+            ops.gemv_q8(x, words, scale, None, y)
+            assert bool((y == W[:, kcol]).all())
+        # sampled rows of a dense GEMV against the oracle
+        x = torch.randn(K, device="cuda", generator=g).half()
+        ops.gemv_q8(x, words, scale, None, y)
+        rows = [0, 1, N // 2, N - 1]
+        wq = words[rows].cpu().numpy().view(np.uint32)
+        want = oracle.c.gemv_q8(x.cpu().numpy(), np.ascontiguousarray(wq), np.ascontiguousarray(scale[rows].cpu().numpy())).astype(np.float64)
+        got = y[rows].cpu().numpy().astype(np.float64)
+        assert (np.abs(got - want) <= 2e-3 + 2.0 ** -8 * np.abs(want)).all()
