@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
   static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
-  static_assert(!WT || (NS == 2 && NW == 4), "the transposing W path is written for two stages and 4 wavefronts");
+  static_assert(!WT || (NS <= 3 && NW == 4), "the transposing W path is written for two or three stages and 4 wavefronts");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
   static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
   constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
@@ -258,30 +258,36 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   };
 
   // ---- k-major W.  A tile is 64 k x BN columns of W[K][N]; an item is 8 columns of two
-  // consecutive k rows: a lane loads the two 16-byte pieces into registers (wt_load, with tile
-  // kt's other loads) and later (wt_commit, once the stage is free) stores eight 4-byte words
-  // {W[k][c], W[k+1][c]} to where the row-major path would have put them.  Item -> lane is chosen
-  // so that a wavefront's 64 stores hit 64 distinct banks: 32 k pairs x 2 adjacent column chunks.
-  // Columns past N are never written: the W halves of both stages are zeroed once, up front.
+  // consecutive k rows: a lane loads the two 16-byte pieces into registers (wt_load, issued just
+  // before the tile's A blocks) and later (wt_commit, once the tile is next in line) stores eight
+  // 4-byte words {W[k][c], W[k+1][c]} to where the row-major path would have put them.  Item -> lane
+  // is chosen so that a wavefront's 64 stores hit 64 distinct banks: 32 k pairs x 2 adjacent column
+  // chunks.  The pieces come through buffer loads (out of range -> zeros), so every lane issues the
+  // same number of loads per tile whatever its columns: the waits below count them.  Columns past N
+  // are never written: the W parts of all stages are zeroed once, up front.
   constexpr int kWtItems = WT ? 4 * BN / (64 * NW) : 1;
-  u32x4 wt_reg[kWtItems][2];
+  constexpr int kWtSlots = WT ? NS - 1 : 1;  // register sets: one per tile in flight
+  u32x4 wt_reg[kWtSlots][kWtItems][2];
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(W, WT ? static_cast<unsigned>(K * N * 2) : 0u);
   auto wt_item = [&](int i, unsigned& cc, unsigned& kp) {
     const unsigned item = t + i * 64 * NW;
     cc = ((item >> 6) << 1) | (item & 1u);
     kp = (item >> 1) & 31u;
   };
-  auto wt_load = [&](int kt) {
+  auto wt_load = [&](int kt, auto slot_tag) {
+    constexpr int SLOT = decltype(slot_tag)::value;
 #pragma unroll
     for (int i = 0; i < kWtItems; ++i) {
       unsigned cc, kp;
       wt_item(i, cc, kp);
       const int64_t col = n0 + cc * 8, k = static_cast<int64_t>(kt0 + kt) * kBK + 2 * kp;
-      const u32x4 zero = {0u, 0u, 0u, 0u};
-      wt_reg[i][0] = (col < N && k < K) ? *reinterpret_cast<const u32x4*>(W + k * N + col) : zero;
-      wt_reg[i][1] = (col < N && k + 1 < K) ? *reinterpret_cast<const u32x4*>(W + (k + 1) * N + col) : zero;
+      const unsigned at = static_cast<unsigned>((k * N + col) * 2), row = static_cast<unsigned>(N) * 2u;
+      wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k < K) ? at : kOob, 0, 0);
+      wt_reg[SLOT][i][1] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k + 1 < K) ? at + row : kOob, 0, 0);
     }
   };
-  auto wt_commit = [&](int kt) {
+  auto wt_commit = [&](int kt, auto slot_tag) {
+    constexpr int SLOT = decltype(slot_tag)::value;
     char* base = lds + (kt % NS) * kStage + kABytes;
 #pragma unroll
     for (int i = 0; i < kWtItems; ++i) {
@@ -290,7 +296,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       if (n0 + cc * 8 >= N) continue;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const unsigned a = wt_reg[i][0][j], b = wt_reg[i][1][j];
+        const unsigned a = wt_reg[SLOT][i][0][j], b = wt_reg[SLOT][i][1][j];
         const unsigned r = cc * 8 + 2 * j;
         *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r, kp >> 2) + (kp & 3u) * 4u) = (a & 0xffffu) | (b << 16);
         *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r + 1, kp >> 2) + (kp & 3u) * 4u) = (a >> 16) | (b & 0xffff0000u);
@@ -333,7 +339,66 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     }
   };
 
-  if constexpr (NW == 8) {
+  if constexpr (WT) {
+    // ---- k-major W: NS stages, NS-1 tiles requested ahead (W pieces to registers, then the A blocks
+    // to the LDS, so the loads of a tile are contiguous in the order they complete in).  This path
+    // is bound by the bytes of A in flight, not by MFMA issue: loads go out in one burst per tile.
+    constexpr int AH = NS - 1;
+    constexpr int kTileLoads = LA + 2 * kWtItems;  // per lane and tile
+    static_assert((AH - 1) * kTileLoads <= 63, "outstanding loads must fit the vmcnt field");
+    using Slot0 = std::integral_constant<int, 0>;
+    using Slot1 = std::integral_constant<int, (AH > 1 ? 1 : 0)>;
+    if (0 < ktiles) { wt_load(0, Slot0{}); fetch(0); }
+    if (AH > 1 && 1 < ktiles) { wt_load(1, Slot1{}); fetch(1); }
+    if (AH > 1 && 1 < ktiles) __builtin_amdgcn_s_waitcnt(waitcnt_imm(kTileLoads));
+    else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+    if (0 < ktiles) wt_commit(0, Slot0{});
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the transposed words are in the LDS
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    if (ktiles > 0) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) read_b(0, j, lds, 0);
+    }
+    DTAS_SCHED_FENCE();
+    // tile kt: its W sits in register slot kt % AH until committed, which frees the slot for tile kt + AH.
+    // `steady`: tiles kt+1 .. kt+AH all exist -- no conditions in the body (a conditional load leaves the
+    // compiler merging old and new register values, which it resolves with copies that wait for the loads)
+    auto k_tile = [&](int kt, auto slot_tag, auto next_slot_tag, auto steady_tag) {
+      constexpr bool kSteady = decltype(steady_tag)::value;
+      const char* cur = lds + (kt % NS) * kStage;
+      const char* nxt = lds + ((kt + 1) % NS) * kStage;
+      if (kSteady || kt + AH < ktiles) {  // into the stage tile kt-1 occupied: free since the last barrier
+        wt_load(kt + AH, slot_tag);
+        fetch(kt + AH);
+      }
+      DTAS_SCHED_FENCE();
+      step(0, cur, 1, true);
+      step(1, cur, 2, true);
+      step(0, cur, 3, true);
+      if (kSteady || kt + 1 < ktiles) {
+        // tile kt+1 must be complete; a tile requested after it may stay in flight
+        if (AH > 1 && (kSteady || kt + 2 < ktiles)) __builtin_amdgcn_s_waitcnt(waitcnt_imm(kTileLoads));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+        wt_commit(kt + 1, next_slot_tag);
+      }
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();        // tile kt+1 is whole, and every wavefront has finished reading tile kt
+      DTAS_SCHED_FENCE();
+      step(1, nxt, 0, kSteady || kt + 1 < ktiles);
+    };
+    int kt = 0;
+    for (; kt + 2 * AH - 1 < ktiles; kt += AH) {  // the AH tiles of a round and the AH after them exist
+      k_tile(kt, Slot0{}, Slot1{}, std::true_type{});
+      if constexpr (AH > 1) k_tile(kt + 1, Slot1{}, Slot0{}, std::true_type{});
+    }
+    for (; kt < ktiles; kt += AH) {
+      k_tile(kt, Slot0{}, Slot1{}, std::false_type{});
+      if (AH > 1 && kt + 1 < ktiles) k_tile(kt + 1, Slot1{}, Slot0{}, std::false_type{});
+    }
+  } else if constexpr (NW == 8) {
     // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD).
     // The LDS is a ring of five 32 KiB units, filled in the order A(0) W(0) A(1) W(1) ...: unit u
     // sits in slot u % 5.  While tile kt (two units) is multiplied, up to three more units are in
@@ -617,28 +682,15 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // two stages: tile 0 resident, tile 1 in flight, fragments of (tile 0, step 0) in registers
   // (row-major W: tile 1 is requested together with tile 0 -- both stages are free -- and only tile 0
   // is waited for; with two k tiles in all, as in the attention scores, that is one round trip less)
-  if (ktiles > 0) {
-    fetch(0);
-    if constexpr (WT) { wt_load(0); wt_commit(0); }
-  }
-  if constexpr (!WT) {
-    if (1 < ktiles) {
-      fetch(1);
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA + LB));  // tile 1's loads may stay outstanding
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0070);
-    }
+  if (ktiles > 0) fetch(0);
+  if (1 < ktiles) {
+    fetch(1);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA + LB));  // tile 1's loads may stay outstanding
   } else {
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   }
   __builtin_amdgcn_s_barrier();
   DTAS_SCHED_FENCE();
-  if constexpr (WT) {
-    if (1 < ktiles) {
-      fetch(1);
-      wt_load(1);
-    }
-  }
   if (ktiles > 0) {
 #pragma unroll
     for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
@@ -652,16 +704,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     step(0, cur, 1, true);
     step(1, cur, 2, true);
     step(0, cur, 3, true);
-    if constexpr (WT) {
-      if (kt + 1 < ktiles) wt_commit(kt + 1);  // its stage was tile kt-1's: free since the last barrier
-    }
     __builtin_amdgcn_s_waitcnt(0x0070);  // tile kt+1 has landed
     __builtin_amdgcn_s_barrier();        // ... and every wavefront has finished reading tile kt
     DTAS_SCHED_FENCE();
-    if (kt + NS < ktiles) {  // into the stage tile kt occupied
-      fetch(kt + NS);
-      if constexpr (WT) wt_load(kt + NS);
-    }
+    if (kt + NS < ktiles) fetch(kt + NS);  // into the stage tile kt occupied
     DTAS_SCHED_FENCE();
     step(1, nxt, 0, kt + 1 < ktiles);
   }
@@ -1473,9 +1519,16 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     // rows: more rows per workgroup mean fewer workgroups than the 256 CUs want)
     cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : 2, 8, 0}, 1, 0};
   } else {
-    // what this op moves is P (2*n*m bytes per head): 128-row tiles once they give every CU a workgroup
-    const int bm = heads * ceil_div(n, 128) >= kNumCU ? 128 : 64;
-    cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {bm, d <= 64 ? 64 : 128, kBK}, 1, 0};
+    // what this op moves is P (2*n*m bytes per head).  Measured over n = m = 128 .. 4096 with 32 heads of 80:
+    // 64-row tiles while 128-row tiles would leave most CUs idle; three stages when a CU holds one
+    // workgroup anyway (up to one 128-row tile per CU, or 256-row tiles once there are two rounds of
+    // them); in between, two workgroups of two stages per CU
+    const int64_t t128 = heads * ceil_div(n, 128);
+    const int bn = d <= 64 ? 64 : 128;
+    if (t128 <= kNumCU / 4) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, bn, kBK}, 1, 0};
+    else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
+    else if (t128 > 2 * kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
+    else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
   }
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_SKINNY && !v_vec) cfg.vec = 1;
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && (!(v_vec && p_vec) || m == 0)) cfg.vec = 1;  // m == 0: zeros
@@ -1510,10 +1563,15 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   }
   if (cfg.variant != DTAS_GEMM_MFMA) return fail("attn_pv: unknown variant %d", cfg.variant);
   if (cfg.split_k > 1) return fail("attn_pv: a batched launch cannot split K");
-  if (cfg.unroll > 2) return fail("attn_pv: the transposing kernels hold two LDS stages, got %d", cfg.unroll);
+  if (cfg.unroll > 3) return fail("attn_pv: the transposing kernels hold two or three LDS stages, got %d", cfg.unroll);
+  if (m * d >= (int64_t{1} << 31)) return fail("attn_pv: a head's V exceeds the 4 GiB a buffer descriptor spans");
   int64_t la[7];
   if (describe_gemm(n, d, m, cfg, la) != 0) return -1;
   const int bm = cfg.tile[0], bn = cfg.tile[1];
+  const bool three = cfg.unroll == 3;
+  if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
   if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
   if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
   if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);

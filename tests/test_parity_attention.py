@@ -114,12 +114,14 @@ def test_pv_builtin_config(oracle, n, m):
     _check_pv(out.check().reshape(32, n, 80), p, v, oracle)
 
 
-@pytest.mark.parametrize("tile", [(64, 64), (64, 128), (128, 64), (128, 128)])
-@pytest.mark.parametrize("heads,n,m,d", [(3, 70, 136, 80), (2, 300, 264, 64), (1, 33, 8, 8), (2, 50, 72, 136), (1, 129, 1032, 128)])
-def test_pv_every_tile(oracle, tile, heads, n, m, d):
+@pytest.mark.parametrize("tile,stages", [((64, 64), 2), ((64, 128), 2), ((128, 64), 2), ((128, 128), 2), ((128, 128), 3), ((256, 128), 3)])
+@pytest.mark.parametrize("heads,n,m,d", [(3, 70, 136, 80), (2, 300, 264, 64), (1, 33, 8, 8), (2, 50, 72, 136), (1, 129, 1032, 128),
+                                         (2, 260, 64, 80), (2, 20, 128, 80), (1, 515, 192, 80)])
+def test_pv_every_tile(oracle, tile, stages, heads, n, m, d):
+    # m = 8 .. 1032: one k tile, two, three (every prologue / drain case of the two- and three-stage pipelines), many
     p, v = _pv_inputs(heads, n, m, d, n + m + d)
     out = Guarded((heads, n, d), torch.float16)
-    ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[tile[0], tile[1], 64]))
+    ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=stages, tile=[tile[0], tile[1], 64]))
     _check_pv(out.check(), p, v, oracle)
 
 
@@ -165,7 +167,9 @@ def test_pv_errors():
     out = torch.empty(2, 16, 80, dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.DtasError, match="split"):
         ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=2))
-    with pytest.raises(_lib.DtasError, match="two LDS stages"):
+    with pytest.raises(_lib.DtasError, match="two or three LDS stages"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=4, tile=[64, 64, 64]))
+    with pytest.raises(_lib.DtasError, match="three stages come with"):
         ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=3, tile=[64, 64, 64]))
     with pytest.raises(_lib.DtasError, match="no transposing"):
         ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[256, 128, 64]))
