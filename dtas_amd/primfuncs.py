@@ -207,6 +207,23 @@ def fused_decode_NT_matmul_add(N: int = 7680, K: int = 2560, gelu: bool = False,
                     params, blocks, op="gemv_q8", attrs={"tir.noalias": True, "epilogue": 3 if gelu else 0})
 
 
+def fused_decode_NT_matmul_add_dyn(N: int = 7680, K: int = 2560, gelu: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """out(1,n,N) = A(1,n,K) . decode(Wq, scale)^T + bias (then GELU), n dynamic: fused_fused_decode2_fused_NT_matmul6_add4
+    (dolly-v2-3b-q8f16_1/before_dl.py:371-399) or, with ``gelu``, fused_fused_decode4_fused_NT_matmul9_add6_gelu1
+    (:504-581).  Parameters: Wq, scale, A, bias, out.  Served as the model's own graph serves fused_decode3: the
+    weights are dequantised into an fp16 matrix (held by the runtime module), then multiplied by the fp16 GEMM."""
+    out = "T_multiply_intermediate_intermediate" if gelu else "T_add_intermediate_intermediate"
+    params = [Buffer("lv780", (N, K // 4), "uint32"), Buffer("lv781", (N, K // 32), "float16"), Buffer("lv779", (1, "n", K), "float16"),
+              Buffer("param_810", (N,), "float16"), Buffer(out, (1, "n", N), "float16")]
+    blocks = [Block("decode", "SS", ["lv780", "lv781"], ["decode_intermediate_intermediate"]),
+              Block("NT_matmul", "SSSR", ["lv779", "decode_intermediate_intermediate"], ["NT_matmul_intermediate"]),
+              Block("T_add", "SSS", ["NT_matmul_intermediate", "param_810"], [out if not gelu else "T_add_intermediate"])]
+    if gelu:
+        blocks.append(Block("T_multiply_2", "SSS", ["T_add_intermediate"], [out]))
+    return PrimFunc(name or ("fused_fused_decode4_fused_NT_matmul9_add6_gelu1" if gelu else "fused_fused_decode2_fused_NT_matmul6_add4"),
+                    params, blocks, op="gemm_q8", attrs={"tir.noalias": True, "epilogue": 3 if gelu else 0})
+
+
 def module(*funcs: PrimFunc, upper_bound: Optional[dict] = None) -> IRModule:
     """An IRModule of the given PrimFuncs; ``upper_bound`` is the ``tir_var_upper_bound`` attribute
     (tuning_test/tune_cast.py:26 uses {"m": 512, "n": 4096})."""

@@ -168,3 +168,28 @@ def test_q8_full_size_properties(oracle):
         want = oracle.c.gemv_q8(x.cpu().numpy(), np.ascontiguousarray(wq), np.ascontiguousarray(scale[rows].cpu().numpy())).astype(np.float64)
         got = y[rows].cpu().numpy().astype(np.float64)
         assert (np.abs(got - want) <= 2e-3 + 2.0 ** -8 * np.abs(want)).all()
+
+
+def test_q8_dynamic_n_primfuncs_through_the_module(oracle):
+    """fused_fused_decode2_fused_NT_matmul6_add4 / ..decode4.._gelu1 (n dynamic): dequantise, then the fp16 GEMM;
+    n = 1 goes to the dequantising GEMV.  Against the oracle's GEMM on the oracle's dequantised matrix."""
+    from dtas_amd import primfuncs as pf
+    from dtas_amd.arch import MI355X
+    from dtas_amd.engine.tuner import Engine
+
+    rng = np.random.default_rng(21)
+    N, K = 640, 512
+    wq, scale = _weights(N, K, 22)
+    bias = rng.standard_normal(N).astype(np.float16)
+    w = oracle.c.decode_q8(wq, scale)
+    mod = pf.module(pf.fused_decode_NT_matmul_add_dyn(N, K), pf.fused_decode_NT_matmul_add_dyn(N, K, gelu=True))
+    rt = Engine(topk=2, parallel_build=False).tune_module(mod, MI355X())
+    for name, kind in (("fused_fused_decode2_fused_NT_matmul6_add4", 0), ("fused_fused_decode4_fused_NT_matmul9_add6_gelu1", 3)):
+        for n in (1, 7, 200):
+            a = rng.standard_normal((1, n, K)).astype(np.float16)
+            out = torch.empty(1, n, N, dtype=torch.float16, device="cuda")
+            rt[name](_words(wq), dev(scale), dev(a), dev(bias), out)
+            torch.cuda.synchronize()
+            want = oracle.c.gemm_fused(a[0], w, bias, None, None, kind, threads=8).astype(np.float64)
+            got = out.cpu().numpy()[0].astype(np.float64)
+            assert (np.abs(got - want) <= 4e-3 + 2.0 ** -8 * np.abs(want)).all(), (name, n)
