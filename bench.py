@@ -101,6 +101,12 @@ def _workload(name: str, n: int, extra=None):
         make = lambda s: (normal((1, K), s), normal((N, K), s + 100, 0.02), empty((1, N)))
         return (make, lambda b: call(L.dtas_gemv_f16, P(b[0]), P(b[1]), None, P(b[2]), N, K, None, stream),
                 2 * N * K + 2 * K + 2 * N, 2 * N * K)
+    if name == "gemv_f32":
+        # NT_matmul5: the fp32 vocabulary projection of the decode graph (50280 x 2560)
+        N, K = extra
+        make = lambda s: (normal((1, K), s, 1.0, torch.float32), normal((N, K), s + 100, 0.02, torch.float32), empty((1, N), torch.float32))
+        return (make, lambda b: call(L.dtas_gemv_f32, P(b[0]), P(b[1]), P(b[2]), N, K, None, stream),
+                4 * N * K + 4 * K + 4 * N, 2 * N * K)
     if name == "gemv_q8_f16":
         # fused_fused_decode2_fused_NT_matmul_add: 8-bit weights (4 to a word) with an fp16 scale per 32, dequantised in registers
         N, K = extra
@@ -285,6 +291,7 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("gemv_f16", 1, nk, steps, warmup))
     for nk in GEMV_SHAPES:
         rows.append(measure("gemv_q8_f16", 1, nk, steps, warmup))
+    rows.append(measure("gemv_f32", 1, (50280, 2560), steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
@@ -317,7 +324,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
-                         "gemv_f16 | gemv_q8_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
+                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -342,7 +349,7 @@ def main() -> int:
         print(_lib.last_error(), file=sys.stderr)
         return 2
 
-    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_q8_f16", "gemm_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemm_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
     info = None
@@ -362,7 +369,7 @@ def main() -> int:
         workload_key = f"{args.workload} [32 heads of 80, n=m={args.n}]"
     elif extra is None:
         workload_key = f"{args.workload} [n={args.n}, 4096]"
-    elif args.workload in ("gemv_f16", "gemv_q8_f16"):
+    elif args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16"):
         workload_key = f"{args.workload} M=1 NxK={args.nk}"
     else:
         workload_key = f"{args.workload} M={args.n} NxK={args.nk}"

@@ -56,7 +56,7 @@ def op_id_of(func: PrimFunc) -> int:
 
 
 # PrimFuncs the tuner does not search: the library picks their kernel and launch shape per call
-LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "gemv_q8", "gemm_q8")
+LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "gemv_q8", "gemm_q8", "gemv_f32")
 
 # fp16 copies of 8-bit weight matrices for the dynamic-n q8 PrimFuncs: one buffer per (device, N, K), reused by
 # every call (the C library itself allocates nothing; the PrimFunc has no parameter for the intermediate)
@@ -149,6 +149,8 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.attn_scores(tensors[0], tensors[1], tensors[2], tensors[3], func.attrs.get("scale", 0.11179039301310044), abi)
     elif op == "attn_pv":                                                     # P, V, out
         ops.attn_pv(tensors[0], tensors[1], tensors[2], abi)
+    elif op == "gemv_f32":                                                    # x, W, y
+        ops.gemv_f32(tensors[0], tensors[1], tensors[2], abi)
     elif op == "decode_q8":                                                   # Wq, scale, W
         ops.decode_q8(tensors[0], tensors[1], tensors[2], abi)
     elif op == "gemm_q8":                                                     # Wq, scale, A, bias, out; n dynamic

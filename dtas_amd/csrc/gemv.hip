@@ -77,6 +77,61 @@ __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restri
   }
 }
 
+// fp32 operands and result (NT_matmul5, experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:8-19: the
+// 50280 x 2560 vocabulary projection of the decode graph): the same workgroup shape, 4 elements per
+// 128-bit access, fused multiply-adds in fp32.
+template <int R>
+__global__ void __launch_bounds__(512) gemv_f32_kernel(const float* __restrict__ x, const float* __restrict__ W,
+                                                       float* __restrict__ y, int64_t N, int64_t K) {
+  __shared__ float part[8][R];
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+  const int64_t nvec = K >> 2;
+  const f32x4* xv = reinterpret_cast<const f32x4*>(x);
+  const f32x4* wv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r < N ? row0 + r : N - 1;  // rows past N re-read the last row; never stored
+    wv[r] = reinterpret_cast<const f32x4*>(W + row * K);
+  }
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+#pragma unroll 2
+  for (int64_t i = threadIdx.x; i < nvec; i += blockDim.x) {
+    const f32x4 xr = xv[i];
+    f32x4 wr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wr[r] = load_stream(wv[r] + i);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[r] = fmaf(xr[e], wr[r][e], acc[r]);
+  }
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float s = wave_sum(acc[r]);
+    if ((threadIdx.x & 63) == 0) part[wave][r] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x < R && row0 + threadIdx.x < N) {
+    float s = 0.f;
+    for (int w = 0; w < nwaves; ++w) s += part[w][threadIdx.x];
+    y[row0 + threadIdx.x] = s;
+  }
+}
+
+__global__ void __launch_bounds__(256) gemv_f32_scalar_kernel(const float* __restrict__ x, const float* __restrict__ W,
+                                                              float* __restrict__ y, int64_t N, int64_t K) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= N) return;  // whole wavefronts leave together; no workgroup barrier below
+  const float* w = W + row * K;
+  float acc = 0.f;
+  for (int64_t k = threadIdx.x & 63; k < K; k += 64) acc = fmaf(x[k], w[k], acc);
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) y[row] = acc;
+}
+
 // Any K and any alignment: one wavefront per row, element accesses.
 __global__ void __launch_bounds__(256) gemv_scalar_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
                                                           const half_t* __restrict__ bias, half_t* __restrict__ y,
@@ -150,4 +205,40 @@ extern "C" int dtas_gemv_f16(const void* x, const void* W, const void* bias, voi
     case 8: hipLaunchKernelGGL(gemv_splitk_kernel<8>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
   }
   return check_launch("gemv");
+}
+
+extern "C" int dtas_gemv_f32(const void* x, const void* W, void* y, int64_t N, int64_t K, const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (N < 0 || K < 0) return fail("gemv_f32: negative extent N=%lld K=%lld", (long long)N, (long long)K);
+  if (N == 0) return 0;
+  if (K != 0 && N > INT64_MAX / 8 / K) return fail("gemv_f32: N*K overflows");
+  if (!y || (K > 0 && (!x || !W))) return fail("gemv_f32: NULL buffer");
+  if (overlaps(y, N * 4, W, N * K * 4) || overlaps(y, N * 4, x, K * 4)) return fail("gemv_f32: output overlaps an input");
+  // the fp16 table, read for a weight matrix of the same bytes (2K fp16 columns)
+  dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMV_F16, 1, N, 2 * K).cfg;
+  if (cfg.vec == 8) cfg.vec = 4;  // (a row of the fp16 table says 8 elements per access: 128 bits are 4 floats)
+  const bool vec_ok = K % 4 == 0 && aligned(x, 16) && aligned(W, 16);
+  if (cfg.vec == 4 && !vec_ok) cfg.vec = 1;
+  if (cfg.vec != 4 && cfg.vec != 1) return fail("gemv_f32: vector width must be 4 (128 bit) or 1, got %d", cfg.vec);
+  dtas_config shape = cfg;
+  shape.vec = cfg.vec == 4 ? 8 : 1;  // describe_gemv speaks of 128-bit accesses as vec 8
+  int64_t la[7];
+  if (describe_gemv(N, K, shape, la) != 0) return -1;
+  const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float* xp = static_cast<const float*>(x);
+  const float* wp = static_cast<const float*>(W);
+  float* yp = static_cast<float*>(y);
+  if (cfg.vec == 1) {
+    hipLaunchKernelGGL(gemv_f32_scalar_kernel, grid, block, 0, s, xp, wp, yp, N, K);
+    return check_launch("gemv_f32");
+  }
+  switch (cfg.tile[0]) {
+    case 1: hipLaunchKernelGGL(gemv_f32_kernel<1>, grid, block, 0, s, xp, wp, yp, N, K); break;
+    case 2: hipLaunchKernelGGL(gemv_f32_kernel<2>, grid, block, 0, s, xp, wp, yp, N, K); break;
+    case 4: hipLaunchKernelGGL(gemv_f32_kernel<4>, grid, block, 0, s, xp, wp, yp, N, K); break;
+    case 8: hipLaunchKernelGGL(gemv_f32_kernel<8>, grid, block, 0, s, xp, wp, yp, N, K); break;
+  }
+  return check_launch("gemv_f32");
 }

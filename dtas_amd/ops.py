@@ -149,6 +149,17 @@ def gemv(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], y: torc
     check(lib().dtas_gemv_f16(_p(x), _p(W), _p(bias), _p(y), N, K, _cfg(cfg), _stream()), "dtas_gemv_f16")
 
 
+def gemv_f32(x: torch.Tensor, W: torch.Tensor, y: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """y[N] = W[N,K] . x[K], all fp32: NT_matmul5 (dolly-v2-3b-q0f16/before_dl.py:8-19)."""
+    _dev(x, W, y)
+    N, K = W.shape
+    if x.numel() != K or y.numel() != N:
+        raise ValueError("gemv_f32: shape mismatch")
+    if any(t.dtype != torch.float32 for t in (x, W, y)):
+        raise ValueError("gemv_f32: expects fp32 tensors")
+    check(lib().dtas_gemv_f32(_p(x), _p(W), _p(y), N, K, _cfg(cfg), _stream()), "dtas_gemv_f32")
+
+
 def gemm(A: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], C: torch.Tensor,
          cfg: Optional[DtasConfig] = None, epilogue: int = 0, res1: Optional[torch.Tensor] = None,
          res2: Optional[torch.Tensor] = None) -> None:

@@ -105,6 +105,13 @@ def fused_NT_matmul_add_gemv(N: int = 2560, K: int = 10240, bias: bool = True,
                     attrs={"tir.noalias": True})
 
 
+def NT_matmul_f32(N: int = 50280, K: int = 2560, name: Optional[str] = None) -> PrimFunc:
+    """y(1,1,N) = x(1,1,K) . W(N,K)^T, all fp32: NT_matmul5 (the vocabulary projection), before_dl.py:8-19."""
+    params = [Buffer("A", (1, 1, K), "float32"), Buffer("B", (N, K), "float32"), Buffer("NT_matmul", (1, 1, N), "float32")]
+    blocks = [Block("NT_matmul", "SSSR", ["A", "B"], ["NT_matmul"])]
+    return PrimFunc(name or "NT_matmul5", params, blocks, op="gemv_f32", attrs={"tir.noalias": True})
+
+
 def fused_NT_matmul_add_gemm(N: int = 2560, K: int = 10240, bias: bool = True,
                              name: Optional[str] = None) -> PrimFunc:
     """C(1,n,N) = A(1,n,K) . W(N,K)^T (+ bias), n dynamic: fused_NT_matmul4_add1, before_dl.py:320-341."""

@@ -218,6 +218,12 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
 int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int64_t n, int64_t m,
                      int64_t d, const dtas_config* cfg, void* stream);
 
+/* ---- fp32 GEMV: NT_matmul5 (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:8-19), the 50280 x 2560
+ * vocabulary projection of the decode graph: y[N] = x[K] . W[N,K]^T, all fp32, no bias.  cfg, when given, is a
+ * DTAS_GEMV_SPLITK row with vec 4 (128-bit accesses) or 1. */
+int dtas_gemv_f32(const void* x, const void* W, void* y, int64_t N, int64_t K, const dtas_config* cfg,
+                  void* stream);
+
 /* ---- 8-bit weights with fp16 group scales (the q8f16_1 layout of
  * experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py) ----
  * Wq[N, K/4] uint32: element j of a row is byte j % 4 of word j / 4; scale[N, K/32] fp16; K % 32 == 0.

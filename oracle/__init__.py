@@ -68,6 +68,7 @@ class _C:
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
                 "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
                 "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
+                "oracle_gemv_f32": [vp, vp, vp, i64, i64, ci],
                 "oracle_decode_q8_f16": [vp, vp, vp, i64, i64, ci],
                 "oracle_gemv_q8_f16": [vp, vp, vp, vp, vp, i64, i64, ci, ci, ci],
             }
@@ -180,6 +181,14 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         assert v.shape == (heads, m, d) and p.dtype == np.float16 and v.dtype == np.float16
         out = np.empty((heads, n, d), dtype=np.float16)
         _C.lib().oracle_attn_pv_f16(_ptr(p), _ptr(v), _ptr(out), heads, n, m, d, int(acc_f16), threads)
+        return out
+
+    @staticmethod
+    def gemv_f32(x, w, threads: int = 1) -> np.ndarray:
+        """fp32 y[N] = x[K] . w[N,K]^T, fp32 running sum with k ascending."""
+        assert x.dtype == np.float32 and w.dtype == np.float32 and x.size == w.shape[1]
+        out = np.empty(x.shape[:-1] + (w.shape[0],), dtype=np.float32)
+        _C.lib().oracle_gemv_f32(_ptr(x), _ptr(w), _ptr(out), w.shape[0], w.shape[1], threads)
         return out
 
     @staticmethod

@@ -429,6 +429,21 @@ void oracle_gemv_q8_f16(const f16* x, const uint32_t* Wq, const f16* S, const f1
   }
 }
 
+/* ========================================================================
+ * fp32 GEMV: NT_matmul5 (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:8-19)
+ *   NT_matmul[0,0,i] = sum_k A[0,0,k] * B[i,k]     fp32 throughout, k ascending, no contraction
+ * Pinned by: float64 closed form (error bound from sum |x||w|), numpy's float32 dot on short rows,
+ * one-hot x (a column of W, exact), K = 1 (one rounded product), exactly representable integers.
+ * ======================================================================== */
+void oracle_gemv_f32(const float* x, const float* W, float* y, int64_t N, int64_t K, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < N; ++i) {
+    float acc = 0.f;
+    for (int64_t k = 0; k < K; ++k) acc = acc + x[k] * W[i * K + k];
+    y[i] = acc;
+  }
+}
+
 int oracle_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

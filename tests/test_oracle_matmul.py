@@ -86,3 +86,28 @@ def test_fp16_accumulate_follows_the_primfunc_text(oracle):
 def test_threads_do_not_change_bits(oracle):
     a, w = _inputs(7, 33, 100)
     assert np.array_equal(oracle.c.gemm(a, w, threads=1).view(np.uint16), oracle.c.gemm(a, w, threads=4).view(np.uint16))
+
+
+# ---- fp32 GEMV: NT_matmul5 (before_dl.py:8-19) ----------------------------------------------------------
+
+def test_gemv_f32_closed_forms_and_exact_cases(oracle):
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal(2560).astype(np.float32)
+    w = (rng.standard_normal((97, 2560)) * 0.02).astype(np.float32)
+    got = oracle.c.gemv_f32(x, w)
+    f64 = w.astype(np.float64) @ x.astype(np.float64)
+    bound = (np.abs(w.astype(np.float64)) @ np.abs(x.astype(np.float64))) * 2560 * 2.0 ** -24      # a running fp32 sum of K terms
+    assert got.dtype == np.float32 and (np.abs(got - f64) <= bound).all()
+    assert (np.abs(got - f64) <= 1e-5 * np.abs(f64) + 1e-5).all()
+    # short rows: numpy's float32 dot product has the same few roundings
+    assert np.allclose(oracle.c.gemv_f32(x[:8], np.ascontiguousarray(w[:, :8])), w[:, :8] @ x[:8], rtol=1e-6, atol=1e-7)
+    # one-hot x returns a column of W exactly; K = 1 is one rounded product; small integers are exact
+    for k in (0, 1, 2559):
+        e = np.zeros(2560, np.float32)
+        e[k] = 1
+        assert np.array_equal(oracle.c.gemv_f32(e, w), w[:, k])
+    assert np.array_equal(oracle.c.gemv_f32(np.float32([3.1]), np.float32([[0.7], [-2.0]])), np.float32([3.1]) * np.float32([0.7, -2.0]))
+    xi = rng.integers(-8, 9, 64).astype(np.float32)
+    wi = rng.integers(-8, 9, (5, 64)).astype(np.float32)
+    assert np.array_equal(oracle.c.gemv_f32(xi, wi), (wi.astype(np.int64) @ xi.astype(np.int64)).astype(np.float32))
+    assert np.array_equal(oracle.c.gemv_f32(x, w, threads=4), got)                               # rows are independent

@@ -323,3 +323,49 @@ def test_gelu_over_every_fp16_preactivation(oracle):
         assert np.abs(diff).max() <= 1
         assert (diff[:, 0] != 0).sum() <= 16, (diff[:, 0] != 0).sum()
     # the decode path (q8 GEMV) and the skinny kernel share the same steps
+
+
+@pytest.mark.parametrize("N,K", [(50280, 2560), (4096, 4096), (101, 36), (7, 4)])
+def test_gemv_f32(oracle, N, K):
+    """NT_matmul5: fp32 in, fp32 out.  The kernel's summation order differs from the oracle's running sum, so both
+    are held to the float64 product within the bound a K-term fp32 sum carries."""
+    rng = np.random.default_rng(N + K)
+    x = rng.standard_normal(K).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+    out = Guarded((1, 1, N), torch.float32)
+    ops.gemv_f32(dev(x).view(1, 1, K), dev(w), out.t)
+    got = out.check().reshape(N).astype(np.float64)
+    f64 = w.astype(np.float64) @ x.astype(np.float64)
+    mag = np.abs(w.astype(np.float64)) @ np.abs(x.astype(np.float64))
+    assert (np.abs(got - f64) <= mag * 64 * 2.0 ** -24 + 1e-30).all()          # far inside rtol 1e-2
+    want = oracle.c.gemv_f32(x, w, threads=8).astype(np.float64)
+    assert (np.abs(got - want) <= mag * K * 2.0 ** -24 + 1e-30).all()
+
+
+def test_gemv_f32_variants_exact_cases_and_errors(oracle):
+    rng = np.random.default_rng(77)
+    N, K = 203, 1028
+    w = rng.integers(-8, 9, (N, K)).astype(np.float32)                        # sums of small integers are exact in fp32
+    x = rng.integers(-8, 9, K).astype(np.float32)
+    want = (w.astype(np.int64) @ x.astype(np.int64)).astype(np.float32)
+    for rows in (1, 2, 4, 8):
+        for block in (64, 256, 512):
+            out = Guarded((N,), torch.float32)
+            ops.gemv_f32(dev(x), dev(w), out.t, cfg(variant=_lib.GEMV_SPLITK, block=block, vec=4, unroll=2, tile=[rows, 0, 0]))
+            assert np.array_equal(out.check(), want)
+    out = Guarded((N,), torch.float32)
+    ops.gemv_f32(dev(x), dev(w), out.t, cfg(variant=_lib.GEMV_SPLITK, block=256, vec=1, unroll=1, tile=[1, 0, 0]))
+    assert np.array_equal(out.check(), want)
+    # K % 4 != 0 and an odd x pointer take the element path
+    w3, x3 = np.ascontiguousarray(w[:, :1027]), np.ascontiguousarray(x[:1027])
+    out = Guarded((N,), torch.float32)
+    ops.gemv_f32(dev(x3), dev(w3), out.t)
+    assert np.array_equal(out.check(), (w3.astype(np.int64) @ x3.astype(np.int64)).astype(np.float32))
+    xb = torch.empty(K + 1, dtype=torch.float32, device="cuda")
+    xb[1:].copy_(dev(x))
+    out = Guarded((N,), torch.float32)
+    ops.gemv_f32(xb[1:], dev(w), out.t)
+    assert np.array_equal(out.check(), want)
+    with pytest.raises(_lib.DtasError, match="vector width"):
+        ops.gemv_f32(dev(x), dev(w), out.t, cfg(variant=_lib.GEMV_SPLITK, block=256, vec=2, unroll=1, tile=[1, 0, 0]))
+    assert _lib.lib().dtas_gemv_f32(None, None, None, 0, 8, None, None) == 0
