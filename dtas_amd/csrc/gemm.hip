@@ -1,5 +1,6 @@
 // Dynamic-M GEMM for gfx950: C[M,N] = A[M,K] . W[N,K]^T (+ bias[N]); fp16 in/out, fp32
-// accumulation on the MFMA matrix cores.
+// accumulation on the MFMA matrix cores.  The fused-epilogue GEMMs and the two batched
+// attention matmuls run on the same kernels.
 //
 // Replaces the kernels DTAS's WMMA rule generates (python/dtas/schedule/tir_wmma.py:20-222:
 // pad M to a tile multiple, block tile (i*micro_x*16) x (j*micro_y*16), k tile micro_k*16,
@@ -16,7 +17,8 @@
 //              ds_write): one wavefront instruction fills one 1 KiB block = 8 tile rows; which
 //              (row, chunk) a lane fetches is the inverse of the LDS swizzle.  Rows past M / N
 //              and chunks past K fall outside the buffer's range and arrive as zeros.
-//   LDS      : two stages of (BM + BN) x 128 B.  Chunk c of row r sits at a swizzled slot so
+//   LDS      : two to four stages of (BM + BN) x 128 B (256x256: a ring of five 32 KiB operand
+//              units).  Chunk c of row r sits at a swizzled slot so
 //              that the MFMA operand reads (a column of 32 rows per half-wavefront, 128 bit
 //              per lane) spread over all 64 banks.
 //   pipeline : 4-wavefront tiles: fragments of step s+1 are read from LDS while the MFMAs of step
@@ -33,9 +35,17 @@
 //              slots) -> 8-byte coalesced row stores with the bias added on the way out.
 //   launch   : workgroup ids are remapped so that each XCD (own L2) works on a compact patch of
 //              the tile grid.
+//   split K  : few output tiles -> several workgroups share a tile and meet in a workspace.
+//   epilogues: bias; bias + two residuals (optionally widened to fp32); bias + erf-GELU; the
+//              attention scores' scale / clamp / mask -- every step an fp16 value, as the fused
+//              PrimFuncs spell them.
+//   batches  : the attention matmuls run all heads in one launch (strides in GemmEpilogue).
+//   k-major W: for P.V the V tiles are transposed on their way into the LDS (template flag WT).
 // SKINNY kernel (M <= 64): the work is streaming W once; a workgroup owns 16 columns of C and
 //              all of M, its wavefronts split K, v_mfma_f32_16x16x32_f16 operands are loaded
 //              straight from global memory, partial tiles are folded through LDS.
+// Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles) and
+//              attn_pv_rows_kernel (P.V for a handful of query rows).
 #include "dtas_device.h"
 #include "dtas_host.h"
 
