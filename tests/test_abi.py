@@ -123,3 +123,32 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libdtas_gfx950.so")
     with pytest.raises(ImportError, match="no fallback"):
         _lib.lib()
+
+
+def test_header_is_plain_c_and_a_c_caller_links(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 (no C++ in it), and a C program that calls an
+    entry point through it must link against the library (no GPU needed: the call fails its argument check)."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None or not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("needs gcc and the built library")
+    src = tmp_path / "caller.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "dtas_abi.h"\n'
+        "int main(void) {\n"
+        "  struct dtas_config cfg; memset(&cfg, 0, sizeof cfg);\n"
+        "  if (dtas_abi_version() != DTAS_ABI_VERSION) return 1;\n"
+        "  if (dtas_add_f16(NULL, NULL, NULL, -1, 8, NULL, NULL) != -1) return 2;   /* negative extent */\n"
+        '  if (strstr(dtas_last_error(), "negative") == NULL) return 3;\n'
+        "  if (dtas_gemv_q8_f16(NULL, NULL, NULL, NULL, NULL, 4, 48, DTAS_EPI_BIAS, NULL, NULL) != -1) return 4;\n"
+        "  if (dtas_attn_pv_f16(NULL, NULL, NULL, 0, 0, 0, 80, NULL, NULL) != 0) return 5;     /* empty: no-op */\n"
+        '  puts("ok");\n  return 0;\n}\n')
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    exe = tmp_path / "caller"
+    subprocess.check_call([gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", include, str(src), "-o", str(exe),
+                           "-L", libdir, "-ldtas_gfx950", f"-Wl,-rpath,{libdir}"])
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", (out.returncode, out.stdout, out.stderr)
