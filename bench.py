@@ -138,6 +138,16 @@ def _workload(name: str, n: int, extra=None):
         make = lambda s: (uniform((heads, rows, m), s), normal((heads, m, d), s + 50), empty((heads, rows, d)))
         return (make, lambda b: call(L.dtas_attn_pv_f16, P(b[0]), P(b[1]), P(b[2]), heads, rows, m, d, None, stream),
                 2 * heads * (rows * m + m * d + rows * d), 2 * heads * rows * m * d)
+    if name == "gemm_q8_f16":
+        # fused_fused_decode2_fused_NT_matmul6_add4: 8-bit weights + fp16 group scales, bias epilogue, n rows
+        N, K = extra
+        g = torch.Generator(device="cuda").manual_seed(300)
+        wq = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device="cuda", generator=g)
+        sc, bias = uniform((N, K // 32), 301, 0.001, 0.02), uniform((N,), 302)
+        make = lambda s: (normal((n, K), s), wq, sc, bias, empty((n, N)))
+        return (make, lambda b: call(L.dtas_gemm_q8_f16_fused, P(b[0]), P(b[1]), P(b[2]), P(b[3]), None, None, P(b[4]), n, N, K, 0,
+                                     None, stream),
+                2 * n * K + N * K + 2 * N * (K // 32) + 2 * n * N + 2 * N, 2 * n * N * K)
     if name in ("gemm_add2_f16", "gemm_gelu_f16"):
         # fused_NT_matmul2_add1_add3_add3 at (N, K) = (2560, 2560); fused_NT_matmul3_add2_gelu at (10240, 2560)
         N, K = extra
@@ -214,7 +224,7 @@ def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool =
            "bytes": nbytes, "flops": flops, "pool": len(pool), "gbs": nbytes / per_launch / 1e9}
     if extra:
         out["NK"] = list(extra)
-    if flops and name in ("gemm_f16", "gemm_add2_f16", "gemm_gelu_f16", "attn_scores_f16_f32", "attn_pv_f16"):
+    if flops and name in ("gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16", "attn_scores_f16_f32", "attn_pv_f16"):
         out["tflops"] = flops / per_launch / 1e12
         hbm_bound_s = nbytes / (HBM_PEAK_GBS * 1e9)
         mfma_bound_s = flops / (MFMA_FP16_PEAK_TFLOPS * 1e12)
@@ -299,6 +309,7 @@ def sweep(steps: int, warmup: int) -> list:
     for m in (16, 256, 2048):
         rows.append(measure("gemm_add2_f16", m, (2560, 2560), max(10, steps // 2), max(2, warmup // 2)))
         rows.append(measure("gemm_gelu_f16", m, (10240, 2560), max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure("gemm_q8_f16", m, (7680, 2560), max(10, steps // 2), max(2, warmup // 2)))
     for n in (128, 1024, 2048):
         rows.append(measure("attn_scores_f16_f32", n, None, max(10, steps // 2), max(2, warmup // 2)))
         rows.append(measure("attn_pv_f16", n, None, max(10, steps // 2), max(2, warmup // 2)))
@@ -324,7 +335,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
-                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemm_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
+                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -349,7 +360,7 @@ def main() -> int:
         print(_lib.last_error(), file=sys.stderr)
         return 2
 
-    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemm_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
     info = None

@@ -58,20 +58,6 @@ def op_id_of(func: PrimFunc) -> int:
 # PrimFuncs the tuner does not search: the library picks their kernel and launch shape per call
 LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "gemv_q8", "gemm_q8", "gemv_f32")
 
-# fp16 copies of 8-bit weight matrices for the dynamic-n q8 PrimFuncs: one buffer per (device, N, K), reused by
-# every call (the C library itself allocates nothing; the PrimFunc has no parameter for the intermediate)
-_DEQUANT_SCRATCH: Dict[Tuple[int, int, int], object] = {}
-
-
-def _dequant_scratch(like, N: int, K: int):
-    import torch
-
-    key = (like.device.index or 0, N, K)
-    buf = _DEQUANT_SCRATCH.get(key)
-    if buf is None:
-        buf = _DEQUANT_SCRATCH[key] = torch.empty(N, K, dtype=torch.float16, device=like.device)
-    return buf
-
 
 def _concrete(shape, values: Dict[str, int]) -> Tuple[int, ...]:
     return tuple(values[e] if isinstance(e, str) else e for e in shape)
@@ -154,14 +140,7 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
     elif op == "decode_q8":                                                   # Wq, scale, W
         ops.decode_q8(tensors[0], tensors[1], tensors[2], abi)
     elif op == "gemm_q8":                                                     # Wq, scale, A, bias, out; n dynamic
-        N, K = tensors[0].shape[0], tensors[0].shape[1] * 4
-        epilogue = int(func.attrs.get("epilogue", 0))
-        if tensors[2].numel() == K and epilogue in (_lib.EPI_BIAS, _lib.EPI_BIAS_GELU):      # one row: the dequantising GEMV
-            ops.gemv_q8(tensors[2], tensors[0], tensors[1], tensors[3], tensors[4], None, epilogue)
-        else:
-            W = _dequant_scratch(tensors[2], N, K)
-            ops.decode_q8(tensors[0], tensors[1], W)
-            ops.gemm(tensors[2], W, tensors[3], tensors[4], abi, epilogue=epilogue)
+        ops.gemm_q8(tensors[2], tensors[0], tensors[1], tensors[3], tensors[4], abi, int(func.attrs.get("epilogue", 0)))
     elif op == "gemv_q8":                                                     # Wq, scale, x, bias, y
         ops.gemv_q8(tensors[2], tensors[0], tensors[1], tensors[3], tensors[4], abi, int(func.attrs.get("epilogue", 0)))
     elif op == "matmul":

@@ -130,6 +130,18 @@ __device__ __forceinline__ half_t gelu_erf_f16_steps(half_t t) {
   return static_cast<half_t>(x * static_cast<float>(a));
 }
 
+// ---- four 8-bit weights of a word as two packed fp16 pairs {W[4w], W[4w+1]}, {W[4w+2], W[4w+3]}:
+// W = (fp16(byte) - 127) * scale in fp16 arithmetic.  0x6400 | byte is the fp16 number 1024 + byte, so one byte
+// permute builds two such halves, a packed subtract of 1151 leaves byte - 127 exactly, the packed multiply rounds
+// as an fp16 product does.
+__device__ __forceinline__ void dequant_q8_word(unsigned word, f16x2 scale2, f16x2& lo, f16x2& hi) {
+  const f16x2 bias2 = {static_cast<half_t>(1151.f), static_cast<half_t>(1151.f)};
+  const unsigned plo = __builtin_amdgcn_perm(0x64646464u, word, 0x04010400u);  // bytes: b0, 0x64, b1, 0x64
+  const unsigned phi = __builtin_amdgcn_perm(0x64646464u, word, 0x04030402u);  // bytes: b2, 0x64, b3, 0x64
+  lo = (__builtin_bit_cast(f16x2, plo) - bias2) * scale2;
+  hi = (__builtin_bit_cast(f16x2, phi) - bias2) * scale2;
+}
+
 // ---- streaming (touch-once) global accesses ---------------------------------------
 template <typename V>
 __device__ __forceinline__ V load_stream(const V* p) { return __builtin_nontemporal_load(p); }

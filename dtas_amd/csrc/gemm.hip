@@ -90,6 +90,7 @@ struct GemmEpilogue {
   int64_t stride_a, stride_w, stride_c, stride_res;
   unsigned batches;
   unsigned tiles_pinned;  // batched launches: an XCD keeps its tiles and walks the problems (see the kernel)
+  const half_t* wscale;   // 8-bit W: the fp16 scales [N][K/32]
 };
 
 // Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):
@@ -156,7 +157,9 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // WT: W is given k-major ([K][N], N contiguous -- the V operand of attention's P.V); its tiles are
 // then transposed on the way into the LDS (two stages, 4 wavefronts only).
-template <int BM, int BN, int WM, int WN, int NS, bool WT = false>
+// WQ: W is 8-bit with an fp16 scale per 32 elements of a row (Wq bytes [N][K], ep.wscale [N][K/32]); its
+// tiles are dequantised on their way into the LDS by the same register path.
+template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ W,
                                                                  GemmEpilogue ep, void* __restrict__ C, int64_t M,
@@ -172,7 +175,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
   static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
-  static_assert(!WT || (NS <= 3 && NW == 4), "the transposing W path is written for two or three stages and 4 wavefronts");
+  constexpr bool WREG = WT || WQ;  // W tiles pass through registers (transposed or dequantised), not the direct-to-LDS path
+  static_assert(!WREG || (NS <= 3 && NW == 4), "the register W path is written for two or three stages and 4 wavefronts");
+  static_assert(!(WT && WQ), "k-major 8-bit weights are not served");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
   static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
   constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
@@ -260,7 +265,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
     for (int i = 0; i < LA; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, 0);
-    if constexpr (!WT) {
+    if constexpr (!WREG) {
 #pragma unroll
       for (int i = 0; i < LB; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
@@ -275,10 +280,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // chunks.  The pieces come through buffer loads (out of range -> zeros), so every lane issues the
   // same number of loads per tile whatever its columns: the waits below count them.  Columns past N
   // are never written: the W parts of all stages are zeroed once, up front.
-  constexpr int kWtItems = WT ? 4 * BN / (64 * NW) : 1;
-  constexpr int kWtSlots = WT ? NS - 1 : 1;  // register sets: one per tile in flight
-  u32x4 wt_reg[kWtSlots][kWtItems][2];
-  const __amdgpu_buffer_rsrc_t rv = make_rsrc(W, WT ? static_cast<unsigned>(K * N * 2) : 0u);
+  // 8-bit W: an item is 16 weights of a row (16 bytes -> two 16-byte chunks of fp16) and their scale; lane
+  // t takes piece t % 4 of row t / 4 (+ 64 rows per further item), so a wavefront reads 64 contiguous bytes
+  // of each of 16 rows.  Every row of the tile is written every time (rows past N as zeros): nothing to clear.
+  constexpr int kWtItems = WREG ? 4 * BN / (64 * NW) : 1;
+  constexpr int kWtSlots = WREG ? NS - 1 : 1;  // register sets: one per tile in flight
+  constexpr int kWtLoads = 2 * kWtItems;  // per lane and tile: k-major two pieces per item, 8-bit a piece and its scale
+  u32x4 wt_reg[kWtSlots][kWtItems][WQ ? 1 : 2];
+  unsigned short wq_scale[kWtSlots][kWtItems];
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(W, WT ? static_cast<unsigned>(K * N * 2) : WQ ? static_cast<unsigned>(K * N) : 0u);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(ep.wscale, WQ ? static_cast<unsigned>((K / 32) * N * 2) : 0u);
   auto wt_item = [&](int i, unsigned& cc, unsigned& kp) {
     const unsigned item = t + i * 64 * NW;
     cc = ((item >> 6) << 1) | (item & 1u);
@@ -286,30 +297,61 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   };
   auto wt_load = [&](int kt, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
+    if constexpr (WQ) {
 #pragma unroll
-    for (int i = 0; i < kWtItems; ++i) {
-      unsigned cc, kp;
-      wt_item(i, cc, kp);
-      const int64_t col = n0 + cc * 8, k = static_cast<int64_t>(kt0 + kt) * kBK + 2 * kp;
-      const unsigned at = static_cast<unsigned>((k * N + col) * 2), row = static_cast<unsigned>(N) * 2u;
-      wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k < K) ? at : kOob, 0, 0);
-      wt_reg[SLOT][i][1] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k + 1 < K) ? at + row : kOob, 0, 0);
+      for (int i = 0; i < kWtItems; ++i) {
+        const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
+        const int64_t row = n0 + r, k = static_cast<int64_t>(kt0 + kt) * kBK + c4 * 16;
+        const bool in = row < N && k < K;  // K % 32 == 0: a piece and its scale group are all-in or all-out
+        wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, in ? static_cast<unsigned>(row * K + k) : kOob, 0, 0);
+        wq_scale[SLOT][i] = __builtin_amdgcn_raw_buffer_load_b16(rs, in ? static_cast<unsigned>((row * (K >> 5) + (k >> 5)) * 2) : kOob, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kWtItems; ++i) {
+        unsigned cc, kp;
+        wt_item(i, cc, kp);
+        const int64_t col = n0 + cc * 8, k = static_cast<int64_t>(kt0 + kt) * kBK + 2 * kp;
+        const unsigned at = static_cast<unsigned>((k * N + col) * 2), row = static_cast<unsigned>(N) * 2u;
+        wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k < K) ? at : kOob, 0, 0);
+        wt_reg[SLOT][i][1] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k + 1 < K) ? at + row : kOob, 0, 0);
+      }
     }
   };
   auto wt_commit = [&](int kt, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     char* base = lds + (kt % NS) * kStage + kABytes;
+    if constexpr (WQ) {
 #pragma unroll
-    for (int i = 0; i < kWtItems; ++i) {
-      unsigned cc, kp;
-      wt_item(i, cc, kp);
-      if (n0 + cc * 8 >= N) continue;
+      for (int i = 0; i < kWtItems; ++i) {
+        const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
+        const half_t sc = __builtin_bit_cast(half_t, wq_scale[SLOT][i]);
+        const f16x2 s2 = {sc, sc};
+        u32x4 out[2];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const unsigned a = wt_reg[SLOT][i][0][j], b = wt_reg[SLOT][i][1][j];
-        const unsigned r = cc * 8 + 2 * j;
-        *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r, kp >> 2) + (kp & 3u) * 4u) = (a & 0xffffu) | (b << 16);
-        *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r + 1, kp >> 2) + (kp & 3u) * 4u) = (a >> 16) | (b & 0xffff0000u);
+        for (int w = 0; w < 4; ++w) {
+          f16x2 lo, hi;
+          const unsigned word = wt_reg[SLOT][i][0][w];
+          dequant_q8_word(word, s2, lo, hi);
+          out[w >> 1][(w & 1) * 2] = __builtin_bit_cast(unsigned, lo);
+          out[w >> 1][(w & 1) * 2 + 1] = __builtin_bit_cast(unsigned, hi);
+        }
+        *reinterpret_cast<u32x4*>(base + lds_chunk_offset(r, 2 * c4)) = out[0];
+        *reinterpret_cast<u32x4*>(base + lds_chunk_offset(r, 2 * c4 + 1)) = out[1];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kWtItems; ++i) {
+        unsigned cc, kp;
+        wt_item(i, cc, kp);
+        if (n0 + cc * 8 >= N) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned a = wt_reg[SLOT][i][0][j], b = wt_reg[SLOT][i][1][j];
+          const unsigned r = cc * 8 + 2 * j;
+          *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r, kp >> 2) + (kp & 3u) * 4u) = (a & 0xffffu) | (b << 16);
+          *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r + 1, kp >> 2) + (kp & 3u) * 4u) = (a >> 16) | (b & 0xffff0000u);
+        }
       }
     }
   };
@@ -349,12 +391,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     }
   };
 
-  if constexpr (WT) {
-    // ---- k-major W: NS stages, NS-1 tiles requested ahead (W pieces to registers, then the A blocks
+  if constexpr (WREG) {
+    // ---- W through registers (k-major or 8-bit): NS stages, NS-1 tiles requested ahead (W pieces to registers, then the A blocks
     // to the LDS, so the loads of a tile are contiguous in the order they complete in).  This path
     // is bound by the bytes of A in flight, not by MFMA issue: loads go out in one burst per tile.
     constexpr int AH = NS - 1;
-    constexpr int kTileLoads = LA + 2 * kWtItems;  // per lane and tile
+    constexpr int kTileLoads = LA + kWtLoads;  // per lane and tile
     static_assert((AH - 1) * kTileLoads <= 63, "outstanding loads must fit the vmcnt field");
     using Slot0 = std::integral_constant<int, 0>;
     using Slot1 = std::integral_constant<int, (AH > 1 ? 1 : 0)>;
@@ -1148,7 +1190,7 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
 }
 
 // Any K and alignment: one thread per element of C.  blockIdx.y = problem of a batched launch;
-// w_kmajor: W is [K][N] instead of [N][K].
+// w_kmajor: W is [K][N] instead of [N][K]; ep.wscale set: W is 8-bit with group scales.
 __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
                                                           GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
                                                           int64_t K, bool w_kmajor) {
@@ -1162,10 +1204,19 @@ __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restri
   for (int64_t ij = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; ij < total;
        ij += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const half_t* a = A + (ij / N) * K;
-    const half_t* w = w_kmajor ? W + ij % N : W + (ij % N) * K;
-    const int64_t wk = w_kmajor ? N : 1;
     float acc = 0.f;
-    for (int64_t k = 0; k < K; ++k) acc += static_cast<float>(a[k]) * static_cast<float>(w[k * wk]);
+    if (ep.wscale) {  // 8-bit W: bytes [N][K], one fp16 scale per 32
+      const unsigned char* wq = reinterpret_cast<const unsigned char*>(W) + (ij % N) * K;
+      const half_t* sc = ep.wscale + (ij % N) * (K >> 5);
+      for (int64_t k = 0; k < K; ++k) {
+        const half_t q = static_cast<half_t>(static_cast<float>(wq[k])) - static_cast<half_t>(127.f);
+        acc += static_cast<float>(a[k]) * static_cast<float>(q * sc[k >> 5]);
+      }
+    } else {
+      const half_t* w = w_kmajor ? W + ij % N : W + (ij % N) * K;
+      const int64_t wk = w_kmajor ? N : 1;
+      for (int64_t k = 0; k < K; ++k) acc += static_cast<float>(a[k]) * static_cast<float>(w[k * wk]);
+    }
     finish(acc, ep, C, ij / N, ij % N, N);
   }
 }
@@ -1276,7 +1327,38 @@ int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsign
   return 0;
 }
 
-template <int BM, int BN, int WM, int WN, int NS, bool WT = false>
+// fp16 copy of an 8-bit weight matrix for dtas_gemm_q8_f16_fused's two-pass route: one buffer per device,
+// allocated on first use and grown on demand like the split-K workspace, and like it shared by the launches
+// that use it (one stream).
+struct DequantWorkspace {
+  void* buf = nullptr;
+  size_t bytes = 0;
+};
+DequantWorkspace g_dequant_ws[kMaxDevices];
+
+int dequant_workspace(size_t bytes, void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("gemm_q8: cannot identify the current device");
+  std::lock_guard<std::mutex> lock(g_split_ws_mutex);
+  DequantWorkspace& w = g_dequant_ws[dev];
+  if (bytes > w.bytes) {
+    if (bytes > kMaxSplitWsBytes) return fail("gemm_q8: an fp16 copy of W needs %zu bytes (limit %zu)", bytes, kMaxSplitWsBytes);
+    // kernels of earlier launches may still use the old buffer: hipFree waits for the device
+    if (w.buf && hipFree(w.buf) != hipSuccess) return fail("gemm_q8: hipFree of the dequantised-weight buffer failed");
+    w.buf = nullptr;
+    w.bytes = 0;
+    const size_t want = bytes < (size_t{64} << 20) ? (size_t{64} << 20) : bytes;
+    if (hipMalloc(&w.buf, want) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail("gemm_q8: cannot allocate %zu bytes for the dequantised weights", want);
+    }
+    w.bytes = want;
+  }
+  *out = w.buf;
+  return 0;
+}
+
+template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
                 int64_t K, int nsplit, int batch = 1) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
@@ -1293,7 +1375,7 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   if (tiles * nsplit * batch > 0x7fffffffu) return fail("gemm: too many workgroups");
   GemmEpilogue batched = ep;
   batched.batches = static_cast<unsigned>(batch);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT>), dim3(static_cast<unsigned>(tiles * nsplit * batch)), dim3(64 * WM * WN), 0,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT, WQ>), dim3(static_cast<unsigned>(tiles * nsplit * batch)), dim3(64 * WM * WN), 0,
                      s, A, W, batched, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
@@ -1587,4 +1669,64 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
   if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
   return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
+}
+
+extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias, const void* res1,
+                                      const void* res2, void* C, int64_t M, int64_t N, int64_t K, int32_t epilogue,
+                                      const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (M < 0 || N < 0 || K < 0) return fail("gemm_q8: negative extent M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  if (K % 32 != 0) return fail("gemm_q8: K must be a multiple of the scale group, 32 (K=%lld)", (long long)K);
+  if (epilogue < DTAS_EPI_BIAS || epilogue > DTAS_EPI_BIAS_GELU) return fail("gemm_q8: unknown epilogue %d", epilogue);
+  if (M == 0 || N == 0) return 0;
+  if ((K != 0 && (M > INT64_MAX / 8 / K || N > INT64_MAX / 8 / K)) || M > INT64_MAX / 8 / N) return fail("gemm_q8: extents overflow");
+  const bool add2 = epilogue == DTAS_EPI_BIAS_ADD2 || epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  if (!A || !Wq || !scale || !C) {
+    if (K > 0 || !C) return fail("gemm_q8: NULL buffer");
+  }
+  if (add2 && (!res1 || !res2)) return fail("gemm_q8: epilogue %d needs both residuals", epilogue);
+  if (!add2 && (res1 || res2)) return fail("gemm_q8: epilogue %d takes no residuals", epilogue);
+  const int out_bytes = epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32 ? 4 : 2;
+  if (overlaps(C, M * N * out_bytes, A, M * K * 2) || overlaps(C, M * N * out_bytes, Wq, N * K) ||
+      overlaps(C, M * N * out_bytes, scale, N * (K / 32) * 2) ||
+      (add2 && (overlaps(C, M * N * out_bytes, res1, M * N * 2) || overlaps(C, M * N * out_bytes, res2, M * N * 2))))
+    return fail("gemm_q8: output overlaps an input");
+  // one row with a plain or GELU epilogue is the dequantising GEMV
+  if (!user && M == 1 && (epilogue == DTAS_EPI_BIAS || epilogue == DTAS_EPI_BIAS_GELU))
+    return dtas_gemv_q8_f16(A, Wq, scale, bias, C, N, K, epilogue, nullptr, stream);
+  GemmEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1), static_cast<const half_t*>(res2),
+                     epilogue, out_bytes == 4 ? 1 : 0, 0.f, 0, 0, 0, 0, 1, 0, static_cast<const half_t*>(scale)};
+  // Two routes.  Dequantising in the W path of the GEMM (no intermediate) runs on a plain burst pipeline without
+  // split K: measured at the model's shapes it wins for M <= 64 with K <= 4096 (18 against 24 us at 7680x2560)
+  // and loses beyond (M = 2048: 109 against 84 us; K = 10240: 2x or more).  Otherwise: the dequantiser into a
+  // library-owned fp16 buffer, then the fp16 GEMM with everything its table offers.  A cfg selects the first route.
+  if (!user && !(M <= 64 && K <= 4096)) {
+    void* wbuf = nullptr;
+    if (dequant_workspace(static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
+    if (dtas_decode_q8_f16(Wq, scale, wbuf, N, K, nullptr, stream) != 0) return -1;
+    return dtas_gemm_f16_fused(A, wbuf, bias, res1, res2, C, M, N, K, epilogue, nullptr, stream);
+  }
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, 64, kBK}, 1, 0};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const half_t* a = static_cast<const half_t*>(A);
+  const half_t* w = static_cast<const half_t*>(Wq);  // (bytes; the kernels take the pointer as they take fp16 W)
+  const bool vec_ok = aligned(A, 16) && aligned(Wq, 16) && aligned(scale, 2) && N * K < (int64_t{1} << 32) && K > 0;
+  if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;
+  if (cfg.vec == 1) {
+    int64_t grid = ceil_div(M * N, 256);
+    grid = grid > 65536 ? 65536 : grid;
+    hipLaunchKernelGGL(gemm_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, a, w, ep, C, M, N, K, false);
+    return check_launch("gemm_q8");
+  }
+  if (cfg.vec != 8) return fail("gemm_q8: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+  if (cfg.variant != DTAS_GEMM_MFMA) return fail("gemm_q8: only the MFMA kernels serve 8-bit weights");
+  if (cfg.split_k > 1) return fail("gemm_q8: K is not split for 8-bit weights");
+  int64_t la[7];
+  if (describe_gemm(M, N, K, cfg, la) != 0) return -1;
+  const int bm = cfg.tile[0], bn = cfg.tile[1];
+  if (bm == 256 && bn == 128 && cfg.unroll == 3) return launch_mfma<256, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, 1);
+  if (bm == 128 && bn == 128 && cfg.unroll == 3) return launch_mfma<128, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, 1);
+  if (bm == 64 && bn == 64 && cfg.unroll == 2) return launch_mfma<64, 64, 2, 2, 2, false, true>(s, a, w, ep, C, M, N, K, 1);
+  return fail("gemm_q8: 8-bit weights come with tiles 256x128 and 128x128 (three stages) and 64x64 (two), got %dx%d with %d", bm, bn, cfg.unroll);
 }

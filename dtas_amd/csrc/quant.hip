@@ -19,18 +19,12 @@
 namespace dtas {
 namespace {
 
-// the four weights of a word as two packed fp16 pairs: {W[4w], W[4w+1]}, {W[4w+2], W[4w+3]}
-__device__ __forceinline__ void dequant_word(unsigned word, f16x2 scale2, f16x2& lo, f16x2& hi) {
-  const f16x2 bias2 = {static_cast<half_t>(1151.f), static_cast<half_t>(1151.f)};
-  const unsigned plo = __builtin_amdgcn_perm(0x64646464u, word, 0x04010400u);  // bytes: b0, 0x64, b1, 0x64
-  const unsigned phi = __builtin_amdgcn_perm(0x64646464u, word, 0x04030402u);  // bytes: b2, 0x64, b3, 0x64
-  lo = (__builtin_bit_cast(f16x2, plo) - bias2) * scale2;
-  hi = (__builtin_bit_cast(f16x2, phi) - bias2) * scale2;
-}
-
 // One item = 8 weights: 8 bytes in, 16 bytes out, so that a wavefront's loads and stores are each one
 // contiguous span (512 bytes in, 1 KiB out).  A thread requests four items, a grid stride apart, before
 // it uses the first.  K % 32 == 0, so an item's weights share a scale and the flat scale index is (8 i) / 32.
+// STREAM: non-temporal stores (the output is larger than the Infinity Cache); otherwise plain stores, so that
+// the GEMM that reads the matrix next finds it in the cache.
+template <bool STREAM>
 __global__ void __launch_bounds__(256) decode_q8_kernel(const u32x2* __restrict__ Wq, const half_t* __restrict__ S,
                                                         u32x4* __restrict__ W, int64_t items) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -52,11 +46,12 @@ __global__ void __launch_bounds__(256) decode_q8_kernel(const u32x2* __restrict_
       const f16x2 s2 = {s[u], s[u]};
       f16x2 a, b, c, d;
       const unsigned w0 = q[u][0], w1 = q[u][1];
-      dequant_word(w0, s2, a, b);
-      dequant_word(w1, s2, c, d);
+      dequant_q8_word(w0, s2, a, b);
+      dequant_q8_word(w1, s2, c, d);
       const u32x4 out = {__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, c),
                          __builtin_bit_cast(unsigned, d)};
-      store_stream(out, W + i);
+      if (STREAM) store_stream(out, W + i);
+      else W[i] = out;
     }
   }
 }
@@ -118,7 +113,7 @@ __global__ void __launch_bounds__(512) gemv_q8_kernel(const half_t* __restrict__
       for (int w = 0; w < 4; ++w) {
         f16x2 lo, hi;
         const unsigned word = q[r][w];
-        dequant_word(word, s2, lo, hi);
+        dequant_q8_word(word, s2, lo, hi);
         const unsigned xa = w < 2 ? x0[2 * w] : x1[2 * w - 4], xb = w < 2 ? x0[2 * w + 1] : x1[2 * w - 3];
         acc[r] = __builtin_amdgcn_fdot2(lo, __builtin_bit_cast(f16x2, xa), acc[r], false);
         acc[r] = __builtin_amdgcn_fdot2(hi, __builtin_bit_cast(f16x2, xb), acc[r], false);
@@ -184,8 +179,12 @@ extern "C" int dtas_decode_q8_f16(const void* Wq, const void* scale, void* W, in
   int64_t grid = ceil_div(items, cfg.vec == 8 ? 4 * 256 : 256);
   const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
   grid = grid > cap ? cap : grid;
-  if (cfg.vec == 8)
-    hipLaunchKernelGGL(decode_q8_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x2*>(Wq),
+  const bool stream_out = N * K * 2 > (int64_t{128} << 20);  // half of the 256 MiB Infinity Cache
+  if (cfg.vec == 8 && stream_out)
+    hipLaunchKernelGGL(decode_q8_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x2*>(Wq),
+                       static_cast<const half_t*>(scale), static_cast<u32x4*>(W), items);
+  else if (cfg.vec == 8)
+    hipLaunchKernelGGL(decode_q8_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x2*>(Wq),
                        static_cast<const half_t*>(scale), static_cast<u32x4*>(W), items);
   else
     hipLaunchKernelGGL(decode_q8_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s,

@@ -253,3 +253,22 @@ def gemv_q8(x: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, bias: Option
         raise ValueError("gemv_q8: expects fp16 x, bias and y")
     check(lib().dtas_gemv_q8_f16(_p(x), _p(Wq), _p(scale), _p(bias), _p(y), N, K, epilogue, _cfg(cfg), _stream()),
           "dtas_gemv_q8_f16")
+
+
+def gemm_q8(A: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor], C: torch.Tensor,
+            cfg: Optional[DtasConfig] = None, epilogue: int = 0, res1: Optional[torch.Tensor] = None,
+            res2: Optional[torch.Tensor] = None) -> None:
+    """C[M,N] = epilogue(A[M,K] . decode_q8(Wq, scale)^T), the weights dequantised on their way into the LDS: the
+    dynamic-n q8f16_1 PrimFuncs (dolly-v2-3b-q8f16_1/before_dl.py:371-399, :504-581); epilogues as ``gemm``."""
+    _dev(A, Wq, scale, bias, C, res1, res2)
+    N, K = _q8_shapes("gemm_q8", Wq, scale)
+    if A.shape[-1] != K or C.shape[-1] != N:
+        raise ValueError("gemm_q8: inner extents differ")
+    M = A.numel() // K if K else C.numel() // max(N, 1)
+    want_out = torch.float32 if epilogue == _lib.EPI_BIAS_ADD2_CAST_F32 else torch.float16
+    if A.dtype != torch.float16 or C.dtype != want_out or any(t is not None and t.dtype != torch.float16 for t in (bias, res1, res2)):
+        raise ValueError("gemm_q8: expects fp16 A, bias and residuals (and an fp32 C for the cast epilogue)")
+    if C.numel() != M * N or (bias is not None and bias.numel() != N) or any(t is not None and t.numel() != M * N for t in (res1, res2)):
+        raise ValueError("gemm_q8: shape mismatch")
+    check(lib().dtas_gemm_q8_f16_fused(_p(A), _p(Wq), _p(scale), _p(bias), _p(res1), _p(res2), _p(C), M, N, K, epilogue,
+                                       _cfg(cfg), _stream()), "dtas_gemm_q8_f16_fused")

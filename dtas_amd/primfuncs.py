@@ -217,8 +217,7 @@ def fused_decode_NT_matmul_add(N: int = 7680, K: int = 2560, gelu: bool = False,
 def fused_decode_NT_matmul_add_dyn(N: int = 7680, K: int = 2560, gelu: bool = False, name: Optional[str] = None) -> PrimFunc:
     """out(1,n,N) = A(1,n,K) . decode(Wq, scale)^T + bias (then GELU), n dynamic: fused_fused_decode2_fused_NT_matmul6_add4
     (dolly-v2-3b-q8f16_1/before_dl.py:371-399) or, with ``gelu``, fused_fused_decode4_fused_NT_matmul9_add6_gelu1
-    (:504-581).  Parameters: Wq, scale, A, bias, out.  Served as the model's own graph serves fused_decode3: the
-    weights are dequantised into an fp16 matrix (held by the runtime module), then multiplied by the fp16 GEMM."""
+    (:504-581).  Parameters: Wq, scale, A, bias, out."""
     out = "T_multiply_intermediate_intermediate" if gelu else "T_add_intermediate_intermediate"
     params = [Buffer("lv780", (N, K // 4), "uint32"), Buffer("lv781", (N, K // 32), "float16"), Buffer("lv779", (1, "n", K), "float16"),
               Buffer("param_810", (N,), "float16"), Buffer(out, (1, "n", N), "float16")]

@@ -24,7 +24,8 @@
  *    when M x N yields few tiles) keeps fp32 partial tiles in a per-device workspace that the
  *    library allocates on first use and grows on demand (32 MiB at first, at most 1 GiB; growing
  *    waits for the device).  Launches that use it share it: enqueue them on one stream, or pass
- *    a cfg with split_k = 1 on the others;
+ *    a cfg with split_k = 1 on the others.  dtas_gemm_q8_f16_fused keeps a second buffer of that kind
+ *    (an fp16 copy of the weights it was given) under the same rules;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
  *    reference's call_table holds); NULL = use the library's built-in bucket table; either way a
  *    128-bit variant steps down to its element-access kernel for extents or pointers that do not
@@ -236,8 +237,17 @@ int dtas_gemv_f32(const void* x, const void* W, void* y, int64_t N, int64_t K, c
  *   fused_fused_decode4_fused_NT_matmul3_add2_gelu (:428-502; DTAS_EPI_BIAS_GELU); fp32 accumulation, then
  *   the fp16 steps of dtas_gemm_f16_fused.  cfg, when given, is a DTAS_GEMV_SPLITK row as for dtas_gemv_f16
  *   (vec 8 = 128-bit accesses); NULL = 256 threads and 2 (N >= 16384: 4) rows per workgroup.
- * The dynamic-n forms of these PrimFuncs (decode + GEMM, :371-399, :504-581) are served as the model's own
- * graph serves fused_decode3: dtas_decode_q8_f16 into a caller-owned fp16 W, then dtas_gemm_f16_fused. */
+ */
+/* dtas_gemm_q8_f16_fused: C[M,N] = epilogue(A[M,K] . W^T) with W dequantised on its way into the LDS, never
+ * written: the dynamic-n forms fused_fused_decode2_fused_NT_matmul6_add4 (:371-399), ..decode4.._matmul9_add6_gelu1
+ * (:504-581), ..decode5.._matmul4_add1; epilogues as dtas_gemm_f16_fused.  cfg, when given: a DTAS_GEMM_MFMA row
+ * with tile {256,128,64} or {128,128,64} and unroll 3, or {64,64,64} and unroll 2.  One row with a bias or GELU
+ * epilogue goes to dtas_gemv_q8_f16.  With cfg == NULL and M > 64 or K > 4096 the library takes the faster
+ * two-pass route: dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on
+ * demand, at most 1 GiB; same sharing rule as the split-K workspace), then dtas_gemm_f16_fused. */
+int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias,
+                           const void* res1, const void* res2, void* C, int64_t M, int64_t N, int64_t K,
+                           int32_t epilogue, const dtas_config* cfg, void* stream);
 int dtas_decode_q8_f16(const void* Wq, const void* scale, void* W, int64_t N, int64_t K,
                        const dtas_config* cfg, void* stream);
 int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale, const void* bias, void* y,

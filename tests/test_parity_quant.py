@@ -193,3 +193,88 @@ def test_q8_dynamic_n_primfuncs_through_the_module(oracle):
             want = oracle.c.gemm_fused(a[0], w, bias, None, None, kind, threads=8).astype(np.float64)
             got = out.cpu().numpy()[0].astype(np.float64)
             assert (np.abs(got - want) <= 4e-3 + 2.0 ** -8 * np.abs(want)).all(), (name, n)
+
+
+def _check_gemm_q8(got, a, wq, scale, bias, r1, r2, kind, oracle):
+    w = oracle.c.decode_q8(wq, scale, threads=8)
+    want = oracle.c.gemm_fused(a, w, bias, r1, r2, kind, threads=8).astype(np.float64)
+    w64 = w.astype(np.float64)
+    f64 = a.astype(np.float64) @ w64.T + (bias.astype(np.float64) if bias is not None else 0.0)
+    if kind in (1, 2):
+        f64 = r1.astype(np.float64) + f64 + r2.astype(np.float64)
+    elif kind == 3:
+        from scipy.special import erf
+        f64 = f64 * (0.5 + 0.5 * erf(f64 * 0.70710678118654757))
+    mag = np.abs(a.astype(np.float64)) @ np.abs(w64).T
+    if kind in (1, 2):
+        mag = mag + np.abs(r1.astype(np.float64)) + np.abs(r2.astype(np.float64))
+    got = got.astype(np.float64)
+    assert np.isfinite(got).all()
+    assert (np.abs(got - f64) <= 1e-2 * np.abs(f64) + mag * 2.0 ** -9 + 4e-3).all()
+    assert (np.abs(got - want) <= 2.0 ** -8 * np.maximum(np.abs(want), mag * 2.0 ** -3) + 4e-3).all()
+    assert (got == want).mean() > 0.9
+
+
+Q8_GEMM_CONFIGS = [None,
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64]),
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[128, 128, 64]),
+                   dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64])]
+
+
+@pytest.mark.parametrize("which", range(len(Q8_GEMM_CONFIGS)))
+@pytest.mark.parametrize("M,N,K", [(2, 40, 32), (77, 200, 96), (130, 257, 160), (300, 384, 1056), (520, 130, 64)])
+@pytest.mark.parametrize("kind", [0, 1, 3])
+def test_gemm_q8_every_tile_on_ragged_shapes(oracle, which, M, N, K, kind):
+    # K = 32 .. 1056: half a k tile, one and a half, two and a half, many (every prologue / drain case)
+    rng = np.random.default_rng(M + N + K + kind)
+    wq, scale = _weights(N, K, M * 3 + N)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    r1 = rng.standard_normal((M, N)).astype(np.float16) if kind == 1 else None
+    r2 = rng.standard_normal((M, N)).astype(np.float16) if kind == 1 else None
+    out = Guarded((M, N), torch.float16)
+    conf = Q8_GEMM_CONFIGS[which]
+    ops.gemm_q8(dev(a), _words(wq), dev(scale), dev(bias), out.t, cfg(**conf) if conf else None, kind,
+                dev(r1) if r1 is not None else None, dev(r2) if r2 is not None else None)
+    _check_gemm_q8(out.check(), a, wq, scale, bias, r1, r2, kind, oracle)
+
+
+@pytest.mark.parametrize("M", [1, 16, 256, 2048])
+@pytest.mark.parametrize("N,K,kind", [(7680, 2560, 0), (10240, 2560, 3), (2560, 10240, 0)])
+def test_gemm_q8_at_the_models_shapes(oracle, M, N, K, kind):
+    rng = np.random.default_rng(M + N + kind)
+    wq, scale = _weights(N, K, N + K)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    out = Guarded((1, M, N), torch.float16)
+    ops.gemm_q8(dev(a).view(1, M, K), _words(wq), dev(scale), dev(bias), out.t, None, kind)
+    rows = np.unique(np.concatenate([np.arange(min(M, 8)), [M // 2, M - 1]]))       # sampled rows against the oracle
+    _check_gemm_q8(out.check().reshape(M, N)[rows], np.ascontiguousarray(a[rows]), wq, scale, bias, None, None, kind, oracle)
+
+
+def test_gemm_q8_exact_cases_fallback_and_errors(oracle):
+    # A = rows of the identity returns columns... of W^T: C[i, :] = decoded W[:, k_i], bit for bit
+    wq, scale = _weights(96, 128, 3)
+    w = oracle.c.decode_q8(wq, scale)
+    a = np.zeros((5, 128), np.float16)
+    for i, k in enumerate((0, 7, 31, 32, 127)):
+        a[i, k] = 1
+    out = Guarded((5, 96), torch.float16)
+    ops.gemm_q8(dev(a), _words(wq), dev(scale), None, out.t)
+    assert np.array_equal(out.check().view(np.uint16), np.ascontiguousarray(w[:, [0, 7, 31, 32, 127]].T).view(np.uint16))
+    # an odd A pointer takes the element path
+    rng = np.random.default_rng(4)
+    a = rng.standard_normal((9, 128)).astype(np.float16)
+    abuf = torch.empty(9 * 128 + 1, dtype=torch.float16, device="cuda")
+    abuf[1:].copy_(dev(a).flatten())
+    out = Guarded((9, 96), torch.float16)
+    ops.gemm_q8(abuf[1:].view(9, 128), _words(wq), dev(scale), None, out.t)
+    _check_gemm_q8(out.check(), a, wq, scale, None, None, None, 0, oracle)
+    c = torch.empty(9, 96, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="8-bit weights come with tiles"):
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=0, block=256, vec=8, unroll=2, tile=[128, 128, 64]))
+    with pytest.raises(_lib.DtasError, match="not split"):
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=2))
+    with pytest.raises(_lib.DtasError, match="needs both residuals"):
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, None, _lib.EPI_BIAS_ADD2)
+    assert _lib.lib().dtas_gemm_q8_f16_fused(None, None, None, None, None, None, None, 0, 96, 128, 0, None, None) == 0
