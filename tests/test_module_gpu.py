@@ -117,3 +117,34 @@ def test_fused_epilogues_through_the_module(tuned, oracle):
             mod["fused_NT_matmul3_add2_gelu"](t(A), t(W), t(bias), out)
             want = oracle.np64.gemm_fused(A[0], W, bias, None, None, 3)
             assert (np.abs(out.cpu().numpy()[0].astype(np.float64) - want) <= 4e-3 + 1e-2 * np.abs(want)).all()
+
+
+def test_profile_sweep_writes_the_reference_file_format(tmp_path):
+    """tune -> reload from the work_dir -> sweep: latency.json / bandwidth.json as the reference's profile scripts
+    write them ({"<n>": us}, {"<n>": GiB/s}; experiment/dtas_tuned/elementwise/add/profile_add.py)."""
+    import json
+    import os
+
+    from dtas_amd import primfuncs as pf
+    from dtas_amd.arch import MI355X
+    from dtas_amd.codegen.runtime_packer import load_module_from_file
+    from dtas_amd.engine.tuner import Engine
+    from dtas_amd.tuning_test import profile_add
+
+    work_dir = str(tmp_path / "add_f16")
+    Engine(1, parallel_build=False, work_dir=work_dir).tune_module(
+        pf.module(pf.add("float16", 2560), upper_bound={"n": 1024}), arch=MI355X(0, require_device=True), range_div_factor=256)
+    rt_mod = load_module_from_file(work_dir)
+
+    def make(n):
+        a = torch.rand(1, n, 2560, device="cuda").half()
+        return a, torch.rand(1, n, 2560, device="cuda").half(), torch.empty_like(a)
+
+    latency, bandwidth = profile_add.sweep(rt_mod, "add", make, lambda n: n * 2560 * 3 * 2, (1, 300, 1024), number=3, min_repeat_ms=2)
+    profile_add.save_to_json(latency, os.path.join(work_dir, "latency.json"))
+    profile_add.save_to_json(bandwidth, os.path.join(work_dir, "bandwidth.json"))
+    lat = json.load(open(os.path.join(work_dir, "latency.json")))
+    bw = json.load(open(os.path.join(work_dir, "bandwidth.json")))
+    assert list(lat) == ["1", "300", "1024"] and all(0.5 < v < 1000 for v in lat.values())
+    assert bw["1024"] > bw["1"] > 0                       # the launch floor dominates n = 1
+    assert abs(bw["1024"] - 1024 * 2560 * 6 / 2 ** 30 / (lat["1024"] * 1e-6)) < 1e-6 * bw["1024"]
