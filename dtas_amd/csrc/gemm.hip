@@ -782,7 +782,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // compiler order every fragment read behind the outstanding direct-to-LDS loads)
     volatile unsigned* is_last = reinterpret_cast<volatile unsigned*>(lds);
     constexpr int kTilePairs = BM * BN / 2;  // 8-byte units per partial tile
-    unsigned long long* tile_ws = reinterpret_cast<unsigned long long*>(ws) + static_cast<size_t>(pid) * nsplit * kTilePairs;
+    const unsigned tile_g = batch_u * total + pid;  // this tile among all problems' tiles
+    unsigned long long* tile_ws = reinterpret_cast<unsigned long long*>(ws) + static_cast<size_t>(tile_g) * nsplit * kTilePairs;
     unsigned long long* mine = tile_ws + static_cast<size_t>(z) * kTilePairs + wv * (MT * NT * 8 * 64);
 #pragma unroll
     for (int i = 0; i < MT; ++i)
@@ -796,10 +797,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         }
     __syncthreads();  // every store of this workgroup has completed; nobody reads the stages any more
     if (t == 0) {
-      const unsigned before = __hip_atomic_fetch_add(arrivals + pid, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned before = __hip_atomic_fetch_add(arrivals + tile_g, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       *is_last = before == nsplit - 1 ? 1u : 0u;
       if (before == nsplit - 1)  // re-armed for the next launch
-        __hip_atomic_store(arrivals + pid, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(arrivals + tile_g, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     const bool last = *is_last != 0;
@@ -1365,13 +1366,12 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   const size_t tiles = static_cast<size_t>(tiles_m) * tiles_n;
   float* partials = nullptr;
   unsigned* arrivals = nullptr;
-  if (nsplit > 1) {
-    const size_t bytes = tiles * nsplit * BM * BN * sizeof(float);
-    if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
-    if (split_workspace(bytes, tiles, &partials, &arrivals) != 0) return -1;
-  }
-  if (batch > 1 && nsplit > 1) return fail("gemm: a batched launch cannot split K");
   if (batch < 1 || batch > 65535) return fail("gemm: batch must be in [1, 65535], got %d", batch);
+  if (nsplit > 1) {
+    const size_t bytes = tiles * batch * nsplit * BM * BN * sizeof(float);
+    if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
+    if (split_workspace(bytes, tiles * batch, &partials, &arrivals) != 0) return -1;
+  }
   if (tiles * nsplit * batch > 0x7fffffffu) return fail("gemm: too many workgroups");
   GemmEpilogue batched = ep;
   batched.batches = static_cast<unsigned>(batch);
@@ -1621,6 +1621,24 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
     else if (t128 > 2 * kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
     else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
+    // Fewer workgroups than CUs and many keys: the workgroups of a tile split m.  Fitted to measurements at
+    // 13 .. 256 rows against 512 .. 8192 keys: a k tile costs a workgroup ~0.8 us, combining S partial tiles
+    // ~3 / 5.5 / 10 us for S = 2 / 4 / 8 (16 loses everywhere).
+    const int64_t wgs = heads * ceil_div(n, cfg.tile[0]), ktiles = ceil_div(m, kBK);
+    if (wgs < kNumCU) {
+      const double combine[4] = {0.0, 3.0, 5.5, 10.0};
+      const double whole = 0.8 * static_cast<double>(ktiles);
+      double best = 0.8 * whole;  // (a split has to promise a fifth less: the fit is coarse)
+      for (int i = 1; i < 4; ++i) {
+        const int split = 1 << i;
+        if (wgs * split > 4 * kNumCU || ktiles < 2 * split) break;
+        const double t = 0.8 * static_cast<double>(ceil_div(ktiles, split)) + combine[i];
+        if (t < best) {
+          best = t;
+          cfg.split_k = split;
+        }
+      }
+    }
   }
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_SKINNY && !v_vec) cfg.vec = 1;
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && (!(v_vec && p_vec) || m == 0)) cfg.vec = 1;  // m == 0: zeros
@@ -1654,20 +1672,20 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     return check_launch("attn_pv");
   }
   if (cfg.variant != DTAS_GEMM_MFMA) return fail("attn_pv: unknown variant %d", cfg.variant);
-  if (cfg.split_k > 1) return fail("attn_pv: a batched launch cannot split K");
+  const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (cfg.unroll > 3) return fail("attn_pv: the transposing kernels hold two or three LDS stages, got %d", cfg.unroll);
   if (m * d >= (int64_t{1} << 31)) return fail("attn_pv: a head's V exceeds the 4 GiB a buffer descriptor spans");
   int64_t la[7];
   if (describe_gemm(n, d, m, cfg, la) != 0) return -1;
   const int bm = cfg.tile[0], bn = cfg.tile[1];
   const bool three = cfg.unroll == 3;
-  if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, 1, b);
-  if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, sk, b);
+  if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, sk, b);
   if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
-  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
-  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
-  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
-  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, 1, b);
+  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
+  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
+  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
+  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
   return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
 }
 

@@ -213,7 +213,8 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
  * P[heads,n,m] (the softmaxed scores), V[heads,m,d], out[heads,n,d], all fp16; n and m are the dynamic
  * extents.  V is k-major (its rows run along d), so its tiles are transposed on the way into the LDS.
  * fp32 accumulation, one rounding to fp16.  cfg, when given: a DTAS_GEMM_MFMA row for the per-head
- * (n, d, m) problem with tile {64|128, 64|128, 64} and two stages, or {128|256, 128, 64} and three, or a DTAS_GEMM_SKINNY row
+ * (n, d, m) problem with tile {64|128, 64|128, 64} and two stages, or {128|256, 128, 64} and three (split_k > 1:
+ * the workgroups of a (head, tile) split m and meet in the split-K workspace), or a DTAS_GEMM_SKINNY row
  * {block 256, tile {1|2|4|8, 8}} for the kernel that serves a handful of rows (decoding).  m % 8 != 0,
  * d % 8 != 0 or odd pointers fall back to the element-access kernel; m == 0 writes zeros. */
 int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int64_t n, int64_t m,

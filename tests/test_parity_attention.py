@@ -125,6 +125,23 @@ def test_pv_every_tile(oracle, tile, stages, heads, n, m, d):
     _check_pv(out.check(), p, v, oracle)
 
 
+@pytest.mark.parametrize("tile,stages,split", [((64, 128), 2, 2), ((64, 128), 2, 16), ((64, 64), 2, 3), ((128, 128), 3, 4), ((256, 128), 3, 2)])
+@pytest.mark.parametrize("heads,n,m,d", [(32, 16, 2048, 80), (3, 70, 1032, 80), (2, 5, 64, 64), (1, 130, 8192, 128)])
+def test_pv_split_over_workgroups(oracle, tile, stages, split, heads, n, m, d):
+    """Few query rows against many keys: the workgroups of a (head, tile) split m and meet in the workspace; the
+    partials are added in split order, so two runs give the same bits, and the counters re-arm themselves."""
+    p, v = _pv_inputs(heads, n, m, d, n + m + d + split)
+    row = cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=stages, tile=[tile[0], tile[1], 64], split_k=split)
+    first = None
+    for _ in range(2):
+        out = Guarded((heads, n, d), torch.float16)
+        ops.attn_pv(dev(p), dev(v), out.t, row)
+        got = out.check()
+        _check_pv(got, p, v, oracle)
+        assert first is None or np.array_equal(first, got)
+        first = got
+
+
 @pytest.mark.parametrize("rows", [1, 2, 4, 8])
 @pytest.mark.parametrize("heads,n,m,d", [(32, 1, 515, 80), (32, 1, 4096, 80), (3, 3, 64, 8), (2, 11, 1000, 128), (1, 8, 1, 16),
                                          (2, 5, 300, 264)])
@@ -165,8 +182,8 @@ def test_pv_selector_rows_are_exact_and_edge_cases(oracle):
 def test_pv_errors():
     p, v = _pv_inputs(2, 16, 16, 80, 1)
     out = torch.empty(2, 16, 80, dtype=torch.float16, device="cuda")
-    with pytest.raises(_lib.DtasError, match="split"):
-        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=2))
+    with pytest.raises(_lib.DtasError, match=r"split_k must be in \[1, 16\]"):
+        ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=17))
     with pytest.raises(_lib.DtasError, match="two or three LDS stages"):
         ops.attn_pv(dev(p), dev(v), out, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=4, tile=[64, 64, 64]))
     with pytest.raises(_lib.DtasError, match="three stages come with"):
