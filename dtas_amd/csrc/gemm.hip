@@ -811,21 +811,32 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       for (int j = 0; j < NT; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    for (unsigned k = 0; k < nsplit; ++k) {
-      const unsigned long long* part = tile_ws + static_cast<size_t>(k) * kTilePairs + wv * (MT * NT * 8 * 64);
+    // The partials are added in split order, but requested kGroup tiles at a time (up to 64 loads per lane):
+    // one tile per round trip made the combine cost ~1.2 us per split, which capped useful splits at 4.
+    constexpr int kPer = MT * NT * 8;  // 8-byte loads per lane and partial tile
+    constexpr int kGroup = kPer >= 64 ? 1 : 64 / kPer;
+    auto add_partials = [&](unsigned k0, auto count_tag) {
+      constexpr int COUNT = decltype(count_tag)::value;
+      unsigned long long raw[COUNT][kPer];
 #pragma unroll
-      for (int i = 0; i < MT; ++i)
+      for (int g = 0; g < COUNT; ++g) {
+        const unsigned long long* part = tile_ws + static_cast<size_t>(k0 + g) * kTilePairs + wv * (kPer * 64);
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
+        for (int q = 0; q < kPer; ++q)
+          raw[g][q] = __hip_atomic_load(part + q * 64 + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
 #pragma unroll
-          for (int h = 0; h < 8; ++h) {
-            const unsigned long long raw =
-                __hip_atomic_load(part + ((i * NT + j) * 8 + h) * 64 + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const f32x2v pr = __builtin_bit_cast(f32x2v, raw);
-            acc[i][j][2 * h] += pr[0];
-            acc[i][j][2 * h + 1] += pr[1];
-          }
-    }
+      for (int g = 0; g < COUNT; ++g)
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+          const f32x2v pr = __builtin_bit_cast(f32x2v, raw[g][q]);
+          acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8)] += pr[0];
+          acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8) + 1] += pr[1];
+        }
+    };
+    unsigned k = 0;
+    for (; k + kGroup <= nsplit; k += kGroup) add_partials(k, std::integral_constant<int, kGroup>{});
+    for (; k < nsplit; ++k) add_partials(k, std::integral_constant<int, 1>{});
   }
 
   constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots;
