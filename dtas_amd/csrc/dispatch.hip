@@ -123,10 +123,14 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
 // A candidate's time is (rounds of workgroups over the chip) x (time of one k tile) x (k tiles):
 //  * time of one k tile with every CU busy: 256x256 1.80 us, 256x128 (3 stages) 1.045 us, 128x128
 //    0.665 us with 4 stages (one workgroup per CU) or 1.14 us per round of two per CU with 2 stages;
-//  * a partly filled last round is faster than a full one: x (0.55 + 0.45 * fill);
-//  * 64x64 (two per CU): 0.33 us per k tile up to 256 workgroups, x 0.82 * workgroups / 256 beyond;
-//  * few tiles: K split over up to 4 workgroups per tile (128x128 and 64x64), each partial tile
-//    costing ~4 us / ~1 us for the last workgroup to add up;
+//  * a partly filled last round is faster than a full one: x (0.55 + 0.45 * fill); 128x128 with 4
+//    stages in a single round gains less: x (0.8 + 0.2 * fill);
+//  * 64x64: 0.33 us per k tile up to 256 workgroups, x 0.82 * (workgroups on the fullest CU) beyond;
+//  * 128x64 (4 stages, one workgroup per CU at most): 0.47 us per k tile whatever the fill;
+//  * few tiles: K split over up to 4 workgroups per tile, each partial tile costing the last
+//    workgroup ~4 us (128x128), ~2.5 us (128x64), ~1 us (64x64; 2 us with more than one per CU)
+//    to add up; 256x128 splits while its workgroups fit one round and each keeps 32 k tiles or
+//    more (~5 us per partial tile);
 //  * M <= 32: the W-streaming SKINNY kernel, whose time grows with N*K (about 3.5 TB/s of W).
 struct GemmChoice {
   double us;
@@ -156,8 +160,14 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     const double steps = static_cast<double>(ceil_div(ktiles, split));
     const double t128 = tiles_of(128, 128) * split, t64 = tiles_of(64, 64) * split;
     if (split == 1 || t128 <= kNumCU)
-      consider(gemm_rounds(t128, kNumCU) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 128, 128, 256, 4, split);
-    consider((t64 <= kNumCU ? 1.0 : 0.82 * t64 / kNumCU) * 0.33 * steps + (split > 1 ? 1.0 * split : 0.0), 64, 64, 256, 4, split);
+      consider((t128 <= kNumCU ? 0.8 + 0.2 * t128 / kNumCU : gemm_rounds(t128, kNumCU)) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 128, 128, 256, 4, split);
+    consider((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.0) * split : 0.0), 64, 64, 256, 4, split);
+    const double t256128 = tiles_of(256, 128) * split;
+    if (split > 1 && steps >= 32 && t256128 <= kNumCU)
+      consider(gemm_rounds(t256128, kNumCU) * 1.045 * steps + 5.0 * split, 256, 128, 256, 3, split);
+    const double t12864 = tiles_of(128, 64) * split;
+    if (t12864 <= kNumCU)
+      consider(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 128, 64, 256, 4, split);
   }
   if (M_hi <= 32) {
     const double skinny_us = static_cast<double>(n) * static_cast<double>(k) * 2.0 / 3.5e6 * (M_hi <= 8 ? 0.9 : M_hi <= 16 ? 0.95 : 1.35);

@@ -36,9 +36,13 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         one the library's built-in table uses): time = rounds of workgroups over the chip x time of one
         k tile x k tiles.  One k tile with every CU busy: 256x256 1.80 us, 256x128 (3 stages) 1.045 us,
         128x128 0.665 us (4 stages, one workgroup per CU) or 1.14 us per round of two per CU (2 stages);
-        a partly filled last round costs 0.55 + 0.45 * fill of a full one; 64x64 0.33 us per k tile up to
-        one workgroup per CU, x 0.82 * workgroups / CUs beyond; with few tiles K is split over up to 4
-        workgroups per tile at ~4 us (128x128) / ~1 us (64x64) per partial tile."""
+        a partly filled last round costs 0.55 + 0.45 * fill of a full one (0.8 + 0.2 * fill for 128x128 with 4 stages
+        in a single round); 64x64 0.33 us per k tile up to
+        one workgroup per CU, x 0.82 * (workgroups on the fullest CU) beyond; with few tiles K is split over up
+        to 4 workgroups per tile at ~4 us (128x128) / ~1 us (64x64; 2 us with more than one per CU) per partial
+        tile; 128x64 (4 stages, at most one workgroup per CU) 0.47 us per k tile whatever the fill and ~2.5 us
+        per partial tile; 256x128 splits too while its workgroups fit one round and each keeps 32 k tiles or
+        more (~5 us per partial tile)."""
         cdiv = lambda a, b: -(-a // b)
         cus = self.arch.num_sm
         ktiles = cdiv(K, 64)
@@ -57,9 +61,16 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             steps = cdiv(ktiles, split)
             t128, t64 = tiles(128, 128) * split, tiles(64, 64) * split
             if split == 1 or t128 <= cus:
-                cands.append((rounds(t128, cus) * 0.665 * steps + (4.0 * split if split > 1 else 0.0), (128, 128, 4, split)))
-            cands.append(((1.0 if t64 <= cus else 0.82 * t64 / cus) * 0.33 * steps + (1.0 * split if split > 1 else 0.0),
+                cands.append(((0.8 + 0.2 * t128 / cus if t128 <= cus else rounds(t128, cus)) * 0.665 * steps + (4.0 * split if split > 1 else 0.0), (128, 128, 4, split)))
+            cands.append(((1.0 if t64 <= cus else 0.82 * -(-int(t64) // cus)) * 0.33 * steps
+                          + ((1.0 if t64 <= cus else 2.0) * split if split > 1 else 0.0),
                           (64, 64, 4, split)))
+            t256128 = tiles(256, 128) * split
+            if split > 1 and steps >= 32 and t256128 <= cus:
+                cands.append((rounds(t256128, cus) * 1.045 * steps + 5.0 * split, (256, 128, 3, split)))
+            t12864 = tiles(128, 64) * split
+            if t12864 <= cus:
+                cands.append((0.47 * steps + (2.5 * split if split > 1 else 0.0), (128, 64, 4, split)))
         best = cands[0]
         for c in cands[1:]:          # first strict minimum, in the library's order of evaluation
             if c[0] < best[0]:
@@ -108,7 +119,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                     continue
                 tiles = -(-m_hi // tm) * -(-N // tn)
                 c.num_wave = -(-tiles // self.arch.num_sm)
-                splits = [1] + [sk for sk in (2, 3, 4) if tiles * sk <= 2 * self.arch.num_sm and -(-K // 64) // sk >= 8]
+                splits = [1] + [sk for sk in (2, 3, 4) if tiles * sk <= 4 * self.arch.num_sm and -(-K // 64) // sk >= 8]
                 for sk in splits:
                     cs = MFMAConfig().from_dict(c.to_dict())
                     cs.split_k, cs.num_wave = sk, -(-tiles * sk // self.arch.num_sm)
