@@ -306,9 +306,11 @@ def sweep(steps: int, warmup: int) -> list:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
     # the model's own fused shapes (dolly-v2-3b: hidden 2560, 32 heads of 80)
-    for m in (16, 256, 2048):
+    for m in (1, 16, 256, 2048):   # m = 1: the decode forms (fused_NT_matmul8_add5_add7_add7, ..9_add6_gelu1) on the GEMV kernel
         rows.append(measure("gemm_add2_f16", m, (2560, 2560), max(10, steps // 2), max(2, warmup // 2)))
         rows.append(measure("gemm_gelu_f16", m, (10240, 2560), max(10, steps // 2), max(2, warmup // 2)))
+        if m == 1:
+            continue
         rows.append(measure("gemm_q8_f16", m, (7680, 2560), max(10, steps // 2), max(2, warmup // 2)))
     for n in (128, 1024, 2048):
         rows.append(measure("attn_scores_f16_f32", n, None, max(10, steps // 2), max(2, warmup // 2)))

@@ -91,6 +91,7 @@ SIGNATURES = {
     "dtas_softmax_f32_f16": [_vp, _vp, _i64, _i64, _cfg, _vp],
     "dtas_softmax_f16": [_vp, _vp, _i64, _i64, _cfg, _vp],
     "dtas_gemv_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _cfg, _vp],
+    "dtas_gemv_f16_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _cfg, _vp],
     "dtas_gemm_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],
     "dtas_gemm_f16_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_int32, _cfg, _vp],
     "dtas_attn_scores_f16_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _cfg, _vp],

@@ -145,10 +145,11 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.gemv_q8(tensors[2], tensors[0], tensors[1], tensors[3], tensors[4], abi, int(func.attrs.get("epilogue", 0)))
     elif op == "matmul":
         epilogue = int(func.attrs.get("epilogue", 0))
+        mm = ops.gemv if FuncInfo(func).kind == FuncKind.kFunc_GEMV else ops.gemm   # one static row: the decode forms
         if epilogue in (_lib.EPI_BIAS_ADD2, _lib.EPI_BIAS_ADD2_CAST_F32):   # A, W, bias, res1, res2, out
-            ops.gemm(tensors[0], tensors[1], tensors[2], tensors[5], abi, epilogue=epilogue, res1=tensors[3], res2=tensors[4])
+            mm(tensors[0], tensors[1], tensors[2], tensors[5], abi, epilogue=epilogue, res1=tensors[3], res2=tensors[4])
         elif epilogue == _lib.EPI_BIAS_GELU:                                  # A, W, bias, out
-            ops.gemm(tensors[0], tensors[1], tensors[2], tensors[3], abi, epilogue=epilogue)
+            mm(tensors[0], tensors[1], tensors[2], tensors[3], abi, epilogue=epilogue)
         else:
             bias = tensors[2] if len(tensors) == 4 else None
             if FuncInfo(func).kind == FuncKind.kFunc_GEMV:

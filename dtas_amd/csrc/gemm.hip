@@ -1478,8 +1478,8 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   if (overlaps(C, M * N * out_bytes, A, M * K * 2) || overlaps(C, M * N * out_bytes, W, N * K * 2) ||
       (add2 && (overlaps(C, M * N * out_bytes, res1, M * N * 2) || overlaps(C, M * N * out_bytes, res2, M * N * 2))))
     return fail("gemm: output overlaps an input");
-  // one row of A with the plain epilogue is the decode GEMV: same PrimFunc shape, dedicated kernel
-  if (!user && M == 1 && epilogue == DTAS_EPI_BIAS) return dtas_gemv_f16(A, W, bias, C, N, K, nullptr, stream);
+  // one row of A is the decode GEMV: same PrimFunc shape, dedicated kernel (every epilogue)
+  if (!user && M == 1) return dtas_gemv_f16_fused(A, W, bias, res1, res2, C, N, K, epilogue, nullptr, stream);
   const GemmEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1),
                            static_cast<const half_t*>(res2), epilogue, out_bytes == 4 ? 1 : 0, 0.f, 0, 0, 0, 0};
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMM_F16, M, N, K).cfg;

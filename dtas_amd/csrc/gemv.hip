@@ -1,4 +1,5 @@
-// Decode GEMV for gfx950: y[N] = W[N,K] . x[K] (+ bias[N]), fp16 in/out, fp32 accumulate.
+// Decode GEMV for gfx950: y[N] = epilogue(W[N,K] . x[K]), fp16 in/out, fp32 accumulate; the epilogues are
+// those of the fused decode PrimFuncs (+ bias; + bias + two residuals, optionally widened; + bias, GELU).
 //
 // Replaces the kernel DTAS's GEMV rule generates (python/dtas/schedule/tir_gemv.py:33-249:
 // two-level rfactor split-K over TR lanes x VEC_C elements, weight to registers with vector
@@ -27,17 +28,33 @@ __device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float acc) {
   return acc;
 }
 
-__device__ __forceinline__ half_t finish(float acc, const half_t* bias, int64_t j) {
+// What follows the dot product in the fused decode PrimFuncs (one fp16 tensor per step, each step
+// rounded): + bias; then either nothing, or res1 + t, then + res2 (optionally widened to an fp32 y), or
+// the erf-GELU.  `kind` is a DTAS_EPI_* value.
+struct GemvEpilogue {
+  const half_t* bias;  // [N] or nullptr
+  const half_t* res1;  // [N]: the ADD2 kinds
+  const half_t* res2;  // [N]: the ADD2 kinds
+  int kind;
+};
+
+__device__ __forceinline__ void finish(float acc, const GemvEpilogue& ep, void* y, int64_t j) {
   // round the fp32 sum to fp16 first, then "+ bias" as the PrimFunc's separate fp16 T_add block
-  half_t r = static_cast<half_t>(acc);
-  if (bias) r = static_cast<half_t>(static_cast<float>(r) + static_cast<float>(bias[j]));
-  return r;
+  half_t t = static_cast<half_t>(acc);
+  if (ep.bias) t = static_cast<half_t>(static_cast<float>(t) + static_cast<float>(ep.bias[j]));
+  if (ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32) {
+    t = static_cast<half_t>(static_cast<float>(ep.res1[j]) + static_cast<float>(t));
+    t = static_cast<half_t>(static_cast<float>(t) + static_cast<float>(ep.res2[j]));
+  } else if (ep.kind == DTAS_EPI_BIAS_GELU) {
+    t = gelu_erf_f16_steps(t);
+  }
+  if (ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32) static_cast<float*>(y)[j] = static_cast<float>(t);
+  else static_cast<half_t*>(y)[j] = t;
 }
 
 template <int R>
 __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
-                                                          const half_t* __restrict__ bias, half_t* __restrict__ y,
-                                                          int64_t N, int64_t K) {
+                                                          GemvEpilogue ep, void* __restrict__ y, int64_t N, int64_t K) {
   __shared__ float part[8][R];
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
   const int64_t nvec = K >> 3;
@@ -73,7 +90,7 @@ __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restri
   if (threadIdx.x < R && row0 + threadIdx.x < N) {
     float s = 0.f;
     for (int w = 0; w < nwaves; ++w) s += part[w][threadIdx.x];
-    y[row0 + threadIdx.x] = finish(s, bias, row0 + threadIdx.x);
+    finish(s, ep, y, row0 + threadIdx.x);
   }
 }
 
@@ -134,15 +151,14 @@ __global__ void __launch_bounds__(256) gemv_f32_scalar_kernel(const float* __res
 
 // Any K and any alignment: one wavefront per row, element accesses.
 __global__ void __launch_bounds__(256) gemv_scalar_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
-                                                          const half_t* __restrict__ bias, half_t* __restrict__ y,
-                                                          int64_t N, int64_t K) {
+                                                          GemvEpilogue ep, void* __restrict__ y, int64_t N, int64_t K) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (row >= N) return;  // whole wavefronts leave together; no workgroup barrier below
   const half_t* w = W + row * K;
   float acc = 0.f;
   for (int64_t k = threadIdx.x & 63; k < K; k += 64) acc += static_cast<float>(x[k]) * static_cast<float>(w[k]);
   acc = wave_sum(acc);
-  if ((threadIdx.x & 63) == 0) y[row] = finish(acc, bias, row);
+  if ((threadIdx.x & 63) == 0) finish(acc, ep, y, row);
 }
 
 }  // namespace
@@ -174,15 +190,22 @@ int describe_gemv(int64_t N, int64_t K, const dtas_config& cfg, int64_t la[7]) {
 
 }  // namespace dtas
 
-extern "C" int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,
-                             const dtas_config* user, void* stream) {
+extern "C" int dtas_gemv_f16_fused(const void* x, const void* W, const void* bias, const void* res1, const void* res2,
+                                   void* y, int64_t N, int64_t K, int32_t epilogue, const dtas_config* user, void* stream) {
   using namespace dtas;
   clear_error();
+  if (epilogue < DTAS_EPI_BIAS || epilogue > DTAS_EPI_BIAS_GELU) return fail("gemv: unknown epilogue %d", epilogue);
+  const bool add2 = epilogue == DTAS_EPI_BIAS_ADD2 || epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const int out_bytes = epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32 ? 4 : 2;
   if (N < 0 || K < 0) return fail("gemv: negative extent N=%lld K=%lld", (long long)N, (long long)K);
   if (N == 0) return 0;
   if (K != 0 && N > INT64_MAX / 4 / K) return fail("gemv: N*K overflows");
   if (!y || (K > 0 && (!x || !W))) return fail("gemv: NULL buffer");
-  if (overlaps(y, N * 2, W, N * K * 2) || overlaps(y, N * 2, x, K * 2)) return fail("gemv: output overlaps an input");
+  if (add2 && (!res1 || !res2)) return fail("gemv: the add-add epilogue needs both residual buffers");
+  if (!add2 && (res1 || res2)) return fail("gemv: residual buffers given for an epilogue that takes none");
+  if (overlaps(y, N * out_bytes, W, N * K * 2) || overlaps(y, N * out_bytes, x, K * 2) ||
+      (add2 && (overlaps(y, N * out_bytes, res1, N * 2) || overlaps(y, N * out_bytes, res2, N * 2))))
+    return fail("gemv: output overlaps an input");
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMV_F16, 1, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(x, 16) && aligned(W, 16);
   if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
@@ -192,19 +215,24 @@ extern "C" int dtas_gemv_f16(const void* x, const void* W, const void* bias, voi
   hipStream_t s = static_cast<hipStream_t>(stream);
   const half_t* xp = static_cast<const half_t*>(x);
   const half_t* wp = static_cast<const half_t*>(W);
-  const half_t* bp = static_cast<const half_t*>(bias);
-  half_t* yp = static_cast<half_t*>(y);
+  const GemvEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1),
+                           static_cast<const half_t*>(res2), epilogue};
   if (cfg.vec == 1) {
-    hipLaunchKernelGGL(gemv_scalar_kernel, grid, block, 0, s, xp, wp, bp, yp, N, K);
+    hipLaunchKernelGGL(gemv_scalar_kernel, grid, block, 0, s, xp, wp, ep, y, N, K);
     return check_launch("gemv");
   }
   switch (cfg.tile[0]) {
-    case 1: hipLaunchKernelGGL(gemv_splitk_kernel<1>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
-    case 2: hipLaunchKernelGGL(gemv_splitk_kernel<2>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
-    case 4: hipLaunchKernelGGL(gemv_splitk_kernel<4>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
-    case 8: hipLaunchKernelGGL(gemv_splitk_kernel<8>, grid, block, 0, s, xp, wp, bp, yp, N, K); break;
+    case 1: hipLaunchKernelGGL(gemv_splitk_kernel<1>, grid, block, 0, s, xp, wp, ep, y, N, K); break;
+    case 2: hipLaunchKernelGGL(gemv_splitk_kernel<2>, grid, block, 0, s, xp, wp, ep, y, N, K); break;
+    case 4: hipLaunchKernelGGL(gemv_splitk_kernel<4>, grid, block, 0, s, xp, wp, ep, y, N, K); break;
+    case 8: hipLaunchKernelGGL(gemv_splitk_kernel<8>, grid, block, 0, s, xp, wp, ep, y, N, K); break;
   }
   return check_launch("gemv");
+}
+
+extern "C" int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,
+                             const dtas_config* user, void* stream) {
+  return dtas_gemv_f16_fused(x, W, bias, nullptr, nullptr, y, N, K, DTAS_EPI_BIAS, user, stream);
 }
 
 extern "C" int dtas_gemv_f32(const void* x, const void* W, void* y, int64_t N, int64_t K, const dtas_config* user, void* stream) {

@@ -138,15 +138,25 @@ def softmax(A: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None
 
 
 def gemv(x: torch.Tensor, W: torch.Tensor, bias: Optional[torch.Tensor], y: torch.Tensor,
-         cfg: Optional[DtasConfig] = None) -> None:
-    """y[N] = W[N,K] . x[K] (+ bias[N]); fp16, fp32 accumulate."""
-    _dev(x, W, bias, y)
+         cfg: Optional[DtasConfig] = None, epilogue: int = 0, res1: Optional[torch.Tensor] = None,
+         res2: Optional[torch.Tensor] = None) -> None:
+    """y[N] = epilogue(W[N,K] . x[K]); fp16, fp32 accumulate.  epilogue (``_lib.EPI_*``) as for gemm: 0 ``+ bias``
+    (fused_NT_matmul10_add5); 1 ``(res1 + (mm + bias)) + res2`` (fused_NT_matmul8_add5_add7_add7,
+    before_dl.py:408-439); 2 the same into an fp32 y (.._cast5, :442-480); 3 ``gelu(mm + bias)``
+    (fused_NT_matmul9_add6_gelu1, :483-549)."""
+    _dev(x, W, bias, y, res1, res2)
     N, K = W.shape
-    if x.numel() != K or y.numel() != N or (bias is not None and bias.numel() != N):
+    if x.numel() != K or y.numel() != N or any(t is not None and t.numel() != N for t in (bias, res1, res2)):
         raise ValueError("gemv: shape mismatch")
-    if any(t.dtype != torch.float16 for t in (x, W, y)) or (bias is not None and bias.dtype != torch.float16):
-        raise ValueError("gemv: expects fp16 tensors")
-    check(lib().dtas_gemv_f16(_p(x), _p(W), _p(bias), _p(y), N, K, _cfg(cfg), _stream()), "dtas_gemv_f16")
+    want_out = torch.float32 if epilogue == _lib.EPI_BIAS_ADD2_CAST_F32 else torch.float16
+    if any(t.dtype != torch.float16 for t in (x, W)) or y.dtype != want_out or \
+            any(t is not None and t.dtype != torch.float16 for t in (bias, res1, res2)):
+        raise ValueError("gemv: expects fp16 tensors (and an fp32 y for the cast epilogue)")
+    if epilogue == _lib.EPI_BIAS and res1 is None and res2 is None:
+        check(lib().dtas_gemv_f16(_p(x), _p(W), _p(bias), _p(y), N, K, _cfg(cfg), _stream()), "dtas_gemv_f16")
+    else:
+        check(lib().dtas_gemv_f16_fused(_p(x), _p(W), _p(bias), _p(res1), _p(res2), _p(y), N, K, epilogue, _cfg(cfg),
+                                        _stream()), "dtas_gemv_f16_fused")
 
 
 def gemv_f32(x: torch.Tensor, W: torch.Tensor, y: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:

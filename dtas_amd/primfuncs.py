@@ -126,31 +126,37 @@ def fused_NT_matmul_add_gemm(N: int = 2560, K: int = 10240, bias: bool = True,
 
 
 def fused_NT_matmul_add_add_add(N: int = 2560, K: int = 2560, cast: bool = False,
-                                name: Optional[str] = None) -> PrimFunc:
+                                name: Optional[str] = None, decode: bool = False) -> PrimFunc:
     """out(1,n,N) = (lv58 + (A(1,n,K) . W(N,K)^T + bias)) + lv2, every step an fp16 tensor; with ``cast`` the
     result is widened to fp32: fused_NT_matmul2_add1_add3_add3, before_dl.py:163-200, and
-    fused_NT_matmul2_add1_add3_add3_cast, :202-246.  Parameter order as there: A, W, bias, res1, res2, out."""
-    params = [Buffer("lv43", (1, "n", K), "float16"), Buffer("param_7", (N, K), "float16"),
-              Buffer("param_8", (N,), "float16"), Buffer("lv58", (1, "n", N), "float16"),
-              Buffer("lv2", (1, "n", N), "float16")]
+    fused_NT_matmul2_add1_add3_add3_cast, :202-246.  Parameter order as there: A, W, bias, res1, res2, out.
+    ``decode``: the static one-row forms of the decode graph, fused_NT_matmul8_add5_add7_add7 (:408-439) and
+    fused_NT_matmul8_add5_add7_add7_cast5 (:442-480)."""
+    n = 1 if decode else "n"
+    params = [Buffer("lv43", (1, n, K), "float16"), Buffer("param_7", (N, K), "float16"),
+              Buffer("param_8", (N,), "float16"), Buffer("lv58", (1, n, N), "float16"),
+              Buffer("lv2", (1, n, N), "float16")]
     blocks = [Block("NT_matmul", "SSSR", ["lv43", "param_7"], ["NT_matmul_intermediate"]),
               Block("T_add", "SSS", ["NT_matmul_intermediate", "param_8"], ["T_add_intermediate"]),
               Block("T_add_1", "SSS", ["lv58", "T_add_intermediate"], ["T_add_intermediate_1"]),
               Block("T_add_2", "SSS", ["T_add_intermediate_1", "lv2"], ["T_add_intermediate_1_2"])]
     if cast:
         blocks.append(Block("compute", "SSS", ["T_add_intermediate_1_2"], ["compute_intermediate"]))
-        params.append(Buffer("compute_intermediate", (1, "n", N), "float32"))
+        params.append(Buffer("compute_intermediate", (1, n, N), "float32"))
     else:
-        params.append(Buffer("T_add_intermediate_1_2", (1, "n", N), "float16"))
-    return PrimFunc(name or ("fused_NT_matmul2_add1_add3_add3_cast" if cast else "fused_NT_matmul2_add1_add3_add3"),
+        params.append(Buffer("T_add_intermediate_1_2", (1, n, N), "float16"))
+    stem = "fused_NT_matmul8_add5_add7_add7" if decode else "fused_NT_matmul2_add1_add3_add3"
+    return PrimFunc(name or (stem + (("_cast5" if decode else "_cast") if cast else "")),
                     params, blocks, op="matmul", attrs={"tir.noalias": True, "epilogue": 2 if cast else 1})
 
 
-def fused_NT_matmul_add_gelu(N: int = 10240, K: int = 2560, name: Optional[str] = None) -> PrimFunc:
+def fused_NT_matmul_add_gelu(N: int = 10240, K: int = 2560, name: Optional[str] = None, decode: bool = False) -> PrimFunc:
     """out(1,n,N) = gelu(A(1,n,K) . W(N,K)^T + bias) with the erf form and an fp16 tensor after every step:
-    fused_NT_matmul3_add2_gelu, before_dl.py:248-318.  Parameters: A, W, bias, out."""
-    params = [Buffer("lv50", (1, "n", K), "float16"), Buffer("param_9", (N, K), "float16"),
-              Buffer("param_10", (N,), "float16"), Buffer("T_multiply_intermediate", (1, "n", N), "float16")]
+    fused_NT_matmul3_add2_gelu, before_dl.py:248-318.  Parameters: A, W, bias, out.  ``decode``: the static
+    one-row form of the decode graph, fused_NT_matmul9_add6_gelu1 (:483-549)."""
+    n = 1 if decode else "n"
+    params = [Buffer("lv50", (1, n, K), "float16"), Buffer("param_9", (N, K), "float16"),
+              Buffer("param_10", (N,), "float16"), Buffer("T_multiply_intermediate", (1, n, N), "float16")]
     blocks = [Block("NT_matmul", "SSSR", ["lv50", "param_9"], ["NT_matmul_intermediate"]),
               Block("T_add", "SSS", ["NT_matmul_intermediate", "param_10"], ["T_add_intermediate"]),
               Block("T_multiply", "SSS", ["T_add_intermediate"], ["T_multiply"]),
@@ -160,8 +166,8 @@ def fused_NT_matmul_add_gelu(N: int = 10240, K: int = 2560, name: Optional[str] 
               Block("T_multiply_1", "SSS", ["compute_2"], ["T_multiply_1"]),
               Block("T_add_1", "SSS", ["T_multiply_1"], ["T_add"]),
               Block("T_multiply_2", "SSS", ["T_add_intermediate", "T_add"], ["T_multiply_intermediate"])]
-    return PrimFunc(name or "fused_NT_matmul3_add2_gelu", params, blocks, op="matmul",
-                    attrs={"tir.noalias": True, "epilogue": 3})
+    return PrimFunc(name or ("fused_NT_matmul9_add6_gelu1" if decode else "fused_NT_matmul3_add2_gelu"), params, blocks,
+                    op="matmul", attrs={"tir.noalias": True, "epilogue": 3})
 
 
 def fused_NT_matmul_divide_maximum_minimum_cast(heads: int = 32, head_dim: int = 80,

@@ -173,6 +173,13 @@ int dtas_softmax_f16(const void* A, void* out, int64_t rows, int64_t cols, const
  * y[N] = W[N,K] . x[K] (+ bias[N] when bias != NULL); fp16 in/out, fp32 accumulate. */
 int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,
                   const dtas_config* cfg, void* stream);
+/* The decode GEMVs with the epilogues of dtas_gemm_f16_fused (a DTAS_EPI_* value, defined below; the
+ * same fp16 steps): fused_NT_matmul8_add5_add7_add7 (before_dl.py:408-439; DTAS_EPI_BIAS_ADD2, res1
+ * and res2 are [N] fp16), .._cast5 (:442-480; DTAS_EPI_BIAS_ADD2_CAST_F32, y is fp32),
+ * fused_NT_matmul9_add6_gelu1 (:483-549; DTAS_EPI_BIAS_GELU).  res1 = res2 = NULL for the kinds without
+ * residuals.  dtas_gemm_f16_fused with M == 1 and cfg == NULL lands here. */
+int dtas_gemv_f16_fused(const void* x, const void* W, const void* bias, const void* res1, const void* res2,
+                        void* y, int64_t N, int64_t K, int32_t epilogue, const dtas_config* cfg, void* stream);
 
 /* ---- GEMM: fused_NT_matmul4_add1 (before_dl.py:320-341) -------------------
  * C[M,N] = A[M,K] . W[N,K]^T (+ bias[N] when bias != NULL); M is the dynamic extent;

@@ -115,6 +115,8 @@ def test_empty_extent_is_a_successful_no_op():
     assert _call("dtas_rms_norm_f16", None, None, None, 0, 4096, 1e-5, None, None) == 0
     assert _call("dtas_softmax_f16", None, None, 0, 0, None, None) == 0
     assert _call("dtas_gemv_f16", None, None, None, None, 0, 4096, None, None) == 0
+    assert _call("dtas_gemv_f16_fused", None, None, None, None, None, None, 0, 4096, 3, None, None) == 0
+    assert _call("dtas_gemv_f16_fused", None, None, None, None, None, None, 0, 4096, 9, None, None) == -1
     assert _call("dtas_gemm_f16", None, None, None, None, 0, 4096, 4096, None, None) == 0
 
 

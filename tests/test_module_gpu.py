@@ -119,6 +119,39 @@ def test_fused_epilogues_through_the_module(tuned, oracle):
             assert (np.abs(out.cpu().numpy()[0].astype(np.float64) - want) <= 4e-3 + 1e-2 * np.abs(want)).all()
 
 
+def test_decode_forms_of_the_fused_matmuls_go_through_the_gemv_rule(tmp_path, oracle):
+    """fused_NT_matmul8_add5_add7_add7(_cast5) and fused_NT_matmul9_add6_gelu1: one static row, tuned as GEMVs."""
+    from dtas_amd.common.analisys import FuncInfo, FuncKind
+
+    funcs = [pf.fused_NT_matmul_add_add_add(2560, 2560, decode=True), pf.fused_NT_matmul_add_add_add(2560, 2560, cast=True, decode=True),
+             pf.fused_NT_matmul_add_gelu(10240, 2560, decode=True)]
+    assert [f.name for f in funcs] == ["fused_NT_matmul8_add5_add7_add7", "fused_NT_matmul8_add5_add7_add7_cast5",
+                                       "fused_NT_matmul9_add6_gelu1"]
+    assert all(FuncInfo(f).kind == FuncKind.kFunc_GEMV for f in funcs)
+    work_dir = str(tmp_path / "decode")
+    rt = Engine(topk=3, parallel_build=False, work_dir=work_dir).tune_module(pf.module(*funcs), arch=MI355X(0, require_device=True))
+    rng = np.random.default_rng(9)
+    t = lambda a: torch.from_numpy(a).cuda()
+    x = rng.standard_normal((1, 1, 2560)).astype(np.float16)
+    W = (rng.standard_normal((2560, 2560)) * 0.02).astype(np.float16)
+    W2 = (rng.standard_normal((10240, 2560)) * 0.02).astype(np.float16)
+    bias, bias2 = rng.uniform(-1, 1, 2560).astype(np.float16), rng.uniform(-1, 1, 10240).astype(np.float16)
+    r1, r2 = rng.standard_normal((1, 1, 2560)).astype(np.float16), rng.standard_normal((1, 1, 2560)).astype(np.float16)
+    for mod in (rt, load_module_from_file(work_dir)):
+        out = torch.empty(1, 1, 2560, dtype=torch.float16, device="cuda")
+        mod["fused_NT_matmul8_add5_add7_add7"](t(x), t(W), t(bias), t(r1), t(r2), out)
+        want = oracle.c.gemm_fused(x[0], W, bias, r1[0], r2[0], 1)
+        got = out.cpu().numpy()[0]
+        assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 2e-3 + 2.0 ** -8 * np.maximum(np.abs(r1[0]), np.abs(r2[0]))).all()
+        out32 = torch.empty(1, 1, 2560, dtype=torch.float32, device="cuda")
+        mod["fused_NT_matmul8_add5_add7_add7_cast5"](t(x), t(W), t(bias), t(r1), t(r2), out32)
+        assert (np.abs(out32.cpu().numpy()[0].astype(np.float64) - want.astype(np.float64)) <= 2e-3 + 2.0 ** -8 * np.maximum(np.abs(r1[0]), np.abs(r2[0]))).all()
+        out2 = torch.empty(1, 1, 10240, dtype=torch.float16, device="cuda")
+        mod["fused_NT_matmul9_add6_gelu1"](t(x), t(W2), t(bias2), out2)
+        want = oracle.np64.gemm_fused(x[0], W2, bias2, None, None, 3)
+        assert (np.abs(out2.cpu().numpy()[0].astype(np.float64) - want) <= 4e-3 + 1e-2 * np.abs(want)).all()
+
+
 def test_profile_sweep_writes_the_reference_file_format(tmp_path):
     """tune -> reload from the work_dir -> sweep: latency.json / bandwidth.json as the reference's profile scripts
     write them ({"<n>": us}, {"<n>": GiB/s}; experiment/dtas_tuned/elementwise/add/profile_add.py)."""

@@ -291,6 +291,51 @@ def test_gemm_fused_at_the_models_shapes(oracle, kind, N, K):
     _check_fused(out.check().reshape(M, N), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
 
 
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("rows,block", [(None, None), (1, 64), (2, 256), (4, 512), (8, 256)])
+@pytest.mark.parametrize("N,K", [(2560, 2560), (10240, 2560), (1001, 520), (7, 8), (33, 1003)])
+def test_gemv_fused_epilogues(oracle, kind, rows, block, N, K):
+    # the decode forms fused_NT_matmul8_add5_add7_add7(_cast5) and fused_NT_matmul9_add6_gelu1 on every GEMV
+    # variant (K = 1003: the element-access kernel)
+    a, w, bias, r1, r2 = _fused_inputs(1, N, K, N + K + kind)
+    res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+    out = Guarded((1, 1, N), torch.float32 if kind == 2 else torch.float16)
+    c = None if rows is None else cfg(variant=_lib.GEMV_SPLITK, block=block, vec=8, unroll=2, tile=[rows, 0, 0])
+    ops.gemv(dev(a), dev(w), dev(bias), out.t, c, epilogue=kind, res1=res[0], res2=res[1])
+    want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind)
+    _check_fused(out.check().reshape(1, N), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+
+
+def test_gemv_fused_is_what_one_row_of_the_gemm_entry_runs_and_errors(oracle):
+    a, w, bias, r1, r2 = _fused_inputs(1, 2560, 2560, 11)
+    via_gemv = Guarded((1, 2560), torch.float16)
+    ops.gemv(dev(a), dev(w), dev(bias), via_gemv.t, None, epilogue=1, res1=dev(r1), res2=dev(r2))
+    via_gemm = Guarded((1, 2560), torch.float16)
+    ops.gemm(dev(a), dev(w), dev(bias), via_gemm.t, None, epilogue=1, res1=dev(r1), res2=dev(r2))
+    assert_bits_equal(via_gemv.check(), via_gemm.check())
+    # without a bias the epilogue still applies
+    out = Guarded((1, 2560), torch.float16)
+    ops.gemv(dev(a), dev(w), None, out.t, None, epilogue=3)
+    want = oracle.c.gemm_fused(a, w, None, None, None, 3)
+    _check_fused(out.check(), want, oracle.np64.gemm_fused(a, w, None, r1, r2, 3), 3)
+    y = torch.empty(2560, dtype=torch.float16, device="cuda")
+    L = _lib.lib()
+    with pytest.raises(_lib.DtasError, match="residual"):
+        _lib.check(L.dtas_gemv_f16_fused(dev(a).data_ptr(), dev(w).data_ptr(), None, None, None, y.data_ptr(), 2560, 2560,
+                                         _lib.EPI_BIAS_ADD2, None, None), "fused")
+    with pytest.raises(_lib.DtasError, match="residual"):
+        _lib.check(L.dtas_gemv_f16_fused(dev(a).data_ptr(), dev(w).data_ptr(), None, dev(r1).data_ptr(), None, y.data_ptr(),
+                                         2560, 2560, _lib.EPI_BIAS_GELU, None, None), "fused")
+    with pytest.raises(_lib.DtasError, match="epilogue"):
+        _lib.check(L.dtas_gemv_f16_fused(dev(a).data_ptr(), dev(w).data_ptr(), None, None, None, y.data_ptr(), 2560, 2560,
+                                         7, None, None), "fused")
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        _lib.check(L.dtas_gemv_f16_fused(dev(a).data_ptr(), dev(w).data_ptr(), None, y.data_ptr(), dev(r2).data_ptr(),
+                                         y.data_ptr(), 2560, 2560, _lib.EPI_BIAS_ADD2, None, None), "fused")
+    with pytest.raises(ValueError, match="fp32 y"):
+        ops.gemv(dev(a), dev(w), None, y, None, epilogue=_lib.EPI_BIAS_ADD2_CAST_F32, res1=dev(r1), res2=dev(r2))
+
+
 def test_gemm_fused_argument_errors():
     a, w, bias, r1, r2 = _fused_inputs(8, 16, 16, 1)
     out = torch.empty(8, 16, dtype=torch.float16, device="cuda")
