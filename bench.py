@@ -116,6 +116,26 @@ def _workload(name: str, n: int, extra=None):
             return normal((1, K), s), wq, uniform((N, K // 32), s + 100, 0.001, 0.02), empty((1, N))
         return (make, lambda b: call(L.dtas_gemv_q8_f16, P(b[0]), P(b[1]), P(b[2]), None, P(b[3]), N, K, 0, None, stream),
                 N * K + 2 * N * (K // 32) + 2 * K + 2 * N, 2 * N * K)
+    if name == "gemv_q8_f32":
+        # fused_fused_decode6_NT_matmul5: the 8-bit model's vocabulary projection (fp32 x, y and group scales)
+        N, K = extra
+        def make(s):
+            g = torch.Generator(device="cuda").manual_seed(s + 200)
+            wq = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device="cuda", generator=g)
+            return (normal((1, K), s, 1.0, torch.float32), wq, uniform((N, K // 32), s + 100, 0.001, 0.02).float(),
+                    empty((1, N), torch.float32))
+        return (make, lambda b: call(L.dtas_gemv_q8_f32, P(b[0]), P(b[1]), P(b[2]), P(b[3]), N, K, None, stream),
+                N * K + 4 * N * (K // 32) + 4 * K + 4 * N, 2 * N * K)
+    if name == "take_q8_f16":
+        # fused_fused_decode1_take1: n rows of the 50280 x 2560 embedding table, dequantised (1.0625 bytes in, 2 out per element)
+        V, K = extra
+        def make(s):
+            g = torch.Generator(device="cuda").manual_seed(s + 200)
+            wq = torch.randint(-2 ** 31, 2 ** 31 - 1, (V, K // 4), dtype=torch.int32, device="cuda", generator=g)
+            ids = torch.randint(0, V, (n,), dtype=torch.int32, device="cuda", generator=g)
+            return wq, uniform((V, K // 32), s + 100, 0.001, 0.02), ids, empty((n, K))
+        return (make, lambda b: call(L.dtas_take_q8_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, V, K, None, stream),
+                n * K + 2 * n * (K // 32) + 4 * n + 2 * n * K, 0)
     if name == "gemm_f16":
         N, K = extra
         wt = normal((N, K), 100, 0.02)
@@ -302,6 +322,9 @@ def sweep(steps: int, warmup: int) -> list:
     for nk in GEMV_SHAPES:
         rows.append(measure("gemv_q8_f16", 1, nk, steps, warmup))
     rows.append(measure("gemv_f32", 1, (50280, 2560), steps, warmup))
+    rows.append(measure("gemv_q8_f32", 1, (50280, 2560), steps, warmup))
+    for n in (1, 1024, 4096):
+        rows.append(measure("take_q8_f16", n, (50280, 2560), steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
@@ -337,7 +360,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
-                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
+                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -362,7 +385,7 @@ def main() -> int:
         print(_lib.last_error(), file=sys.stderr)
         return 2
 
-    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32", "take_q8_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
     info = None
@@ -382,7 +405,7 @@ def main() -> int:
         workload_key = f"{args.workload} [32 heads of 80, n=m={args.n}]"
     elif extra is None:
         workload_key = f"{args.workload} [n={args.n}, 4096]"
-    elif args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16"):
+    elif args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32"):
         workload_key = f"{args.workload} M=1 NxK={args.nk}"
     else:
         workload_key = f"{args.workload} M={args.n} NxK={args.nk}"

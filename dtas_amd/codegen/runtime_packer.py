@@ -32,7 +32,8 @@ def _torch_dtype(name: str):
     if _TORCH_DTYPES is None:
         import torch
 
-        _TORCH_DTYPES = {"float16": torch.float16, "float32": torch.float32, "int8": torch.int8, "uint32": torch.uint32}
+        _TORCH_DTYPES = {"float16": torch.float16, "float32": torch.float32, "int8": torch.int8, "uint32": torch.uint32,
+                         "int32": torch.int32}
     return _TORCH_DTYPES[name]
 
 
@@ -56,7 +57,7 @@ def op_id_of(func: PrimFunc) -> int:
 
 
 # PrimFuncs the tuner does not search: the library picks their kernel and launch shape per call
-LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "gemv_q8", "gemm_q8", "gemv_f32")
+LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "take_q8", "gemv_q8", "gemv_q8_f32", "gemm_q8", "gemv_f32")
 
 
 def _concrete(shape, values: Dict[str, int]) -> Tuple[int, ...]:
@@ -139,6 +140,10 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.gemv_f32(tensors[0], tensors[1], tensors[2], abi)
     elif op == "decode_q8":                                                   # Wq, scale, W
         ops.decode_q8(tensors[0], tensors[1], tensors[2], abi)
+    elif op == "take_q8":                                                     # Wq, scale, ids, out
+        ops.take_q8(tensors[0], tensors[1], tensors[2], tensors[3], abi)
+    elif op == "gemv_q8_f32":                                                 # Wq, scale, x, y
+        ops.gemv_q8_f32(tensors[2], tensors[0], tensors[1], tensors[3], abi)
     elif op == "gemm_q8":                                                     # Wq, scale, A, bias, out; n dynamic
         ops.gemm_q8(tensors[2], tensors[0], tensors[1], tensors[3], tensors[4], abi, int(func.attrs.get("epilogue", 0)))
     elif op == "gemv_q8":                                                     # Wq, scale, x, bias, y

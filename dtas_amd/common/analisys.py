@@ -112,7 +112,7 @@ class FuncInfo:
         b = red_blocks[0]
         if self.func.op in ("attn_scores", "attn_pv"):      # batched matmuls over the heads
             return FuncKind.kFunc_GEMM
-        if self.func.op in ("matmul", "gemv_q8", "gemm_q8", "gemv_f32") and len(b.reads) == 2:
+        if self.func.op in ("matmul", "gemv_q8", "gemv_q8_f32", "gemm_q8", "gemv_f32") and len(b.reads) == 2:
             lhs = next(p for p in self.func.params if p.name == b.reads[0])
             rows = 1
             for e in lhs.shape[:-1]:

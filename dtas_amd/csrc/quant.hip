@@ -1,5 +1,6 @@
-// 8-bit weights with fp16 group scales (the q8f16_1 layout) for gfx950: the standalone dequantiser
-// and the decode GEMV that dequantises in registers.
+// 8-bit weights with group scales (the q8f16_1 layout) for gfx950: the standalone dequantiser, the
+// dequantising row gather of the embedding, and the decode GEMVs that dequantise in registers (fp16 with
+// fp16 scales; fp32 with fp32 scales for the vocabulary projection).
 //
 // Layout and arithmetic, as the PrimFuncs spell them
 // (experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py:335-343 fused_decode3, :401-426
@@ -65,6 +66,121 @@ __global__ void __launch_bounds__(256) decode_q8_scalar_kernel(const unsigned ch
     const half_t q = static_cast<half_t>(static_cast<float>(Wq[j])) - static_cast<half_t>(127.f);  // little endian: byte j
     W[j] = q * S[j >> 5];
   }
+}
+
+// The embedding rows, dequantised: out[i, :] = decode(Wq, S)[ids[i], :].  Items of 8 weights as above; item t of
+// the output is item ids[t / per_row] * per_row + t % per_row of the table.  Ids outside [0, V) are clipped
+// to the nearest row (the PrimFunc reads whatever address they make).
+__global__ void __launch_bounds__(256) take_q8_kernel(const u32x2* __restrict__ Wq, const half_t* __restrict__ S,
+                                                      const int* __restrict__ ids, u32x4* __restrict__ out, int64_t items,
+                                                      int64_t per_row, int64_t V) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < items; t += stride) {
+    int64_t row = ids[t / per_row];
+    row = row < 0 ? 0 : row >= V ? V - 1 : row;
+    const int64_t src = row * per_row + t % per_row;
+    const u32x2 q = Wq[src];
+    const half_t s = S[src >> 2];
+    const f16x2 s2 = {s, s};
+    f16x2 a, b, c, d;
+    const unsigned w0 = q[0], w1 = q[1];
+    dequant_q8_word(w0, s2, a, b);
+    dequant_q8_word(w1, s2, c, d);
+    const u32x4 v = {__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, c),
+                     __builtin_bit_cast(unsigned, d)};
+    out[t] = v;
+  }
+}
+
+// any alignment: one thread per weight
+__global__ void __launch_bounds__(256) take_q8_scalar_kernel(const unsigned char* __restrict__ Wq, const half_t* __restrict__ S,
+                                                             const int* __restrict__ ids, half_t* __restrict__ out,
+                                                             int64_t total, int64_t K, int64_t V) {
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    int64_t row = ids[t / K];
+    row = row < 0 ? 0 : row >= V ? V - 1 : row;
+    const int64_t j = row * K + t % K;
+    const half_t q = static_cast<half_t>(static_cast<float>(Wq[j])) - static_cast<half_t>(127.f);
+    out[t] = q * S[j >> 5];
+  }
+}
+
+// fp32 scales, fp32 x and y (fused_fused_decode6_NT_matmul5, before_dl.py:640-657: the vocabulary projection
+// of the 8-bit model): W = float(byte - 127) * S32, one fp32 rounding, then fp32 multiply-adds against x.
+// Workgroup shape and weight stream as gemv_q8_kernel; a 16-byte chunk of weights meets 64 bytes of x.
+template <int R>
+__global__ void __launch_bounds__(512) gemv_q8_f32_kernel(const float* __restrict__ x, const unsigned* __restrict__ Wq,
+                                                          const float* __restrict__ S, float* __restrict__ y, int64_t N,
+                                                          int64_t K) {
+  __shared__ float part[8][R];
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * R;
+  const int64_t nchunk = K >> 4, ngroup = K >> 5;
+  const f32x4* xv = reinterpret_cast<const f32x4*>(x);
+  const u32x4* wv[R];
+  const float* sv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r < N ? row0 + r : N - 1;  // rows past N re-read the last row; never stored
+    wv[r] = reinterpret_cast<const u32x4*>(Wq + row * (K >> 2));
+    sv[r] = S + row * ngroup;
+  }
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+#pragma unroll 2
+  for (int64_t i = threadIdx.x; i < nchunk; i += blockDim.x) {
+    f32x4 xr[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) xr[w] = xv[4 * i + w];
+    u32x4 q[R];
+    float s[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      q[r] = load_stream(wv[r] + i);
+      s[r] = sv[r][i >> 1];
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const unsigned word = q[r][w];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float wt = (static_cast<float>((word >> (8 * e)) & 255u) - 127.f) * s[r];
+          acc[r] = fmaf(xr[w][e], wt, acc[r]);
+        }
+      }
+  }
+
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float sum = wave_sum(acc[r]);
+    if ((threadIdx.x & 63) == 0) part[wave][r] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x < R && row0 + threadIdx.x < N) {
+    float sum = 0.f;
+    for (int w = 0; w < nwaves; ++w) sum += part[w][threadIdx.x];
+    y[row0 + threadIdx.x] = sum;
+  }
+}
+
+// any alignment: one wavefront per row, byte accesses
+__global__ void __launch_bounds__(256) gemv_q8_f32_scalar_kernel(const float* __restrict__ x, const unsigned char* __restrict__ Wq,
+                                                                 const float* __restrict__ S, float* __restrict__ y, int64_t N,
+                                                                 int64_t K) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= N) return;  // whole wavefronts leave together; no workgroup barrier below
+  float acc = 0.f;
+  for (int64_t k = threadIdx.x & 63; k < K; k += 64) {
+    const float wt = (static_cast<float>(Wq[row * K + k]) - 127.f) * S[row * (K >> 5) + (k >> 5)];
+    acc = fmaf(x[k], wt, acc);
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0) y[row] = acc;
 }
 
 __device__ __forceinline__ half_t finish_q8(float acc, const half_t* bias, int64_t j, int kind) {
@@ -227,4 +343,67 @@ extern "C" int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale
     case 8: hipLaunchKernelGGL(gemv_q8_kernel<8>, grid, block, 0, s, xp, wp, sp, bp, yp, N, K, epilogue); break;
   }
   return check_launch("gemv_q8");
+}
+
+extern "C" int dtas_take_q8_f16(const void* Wq, const void* scale, const void* ids, void* out, int64_t n, int64_t V, int64_t K,
+                                const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (check_q8_shape("take_q8", V, K) != 0) return -1;
+  if (n < 0) return fail("take_q8: negative extent n=%lld", (long long)n);
+  if (K != 0 && n > INT64_MAX / 4 / K) return fail("take_q8: n*K overflows");
+  if (n == 0 || K == 0) return 0;
+  if (V == 0) return fail("take_q8: an empty table has no row to take");
+  if (!Wq || !scale || !ids || !out) return fail("take_q8: NULL buffer");
+  if (overlaps(out, n * K * 2, Wq, V * K) || overlaps(out, n * K * 2, scale, V * (K / 32) * 2) || overlaps(out, n * K * 2, ids, n * 4))
+    return fail("take_q8: output overlaps an input");
+  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, 256, 8, 1, {0, 0, 0}, 1, 0};
+  if (cfg.block != 256) return fail("take_q8: the kernels use 256 threads, got %d", cfg.block);
+  if (cfg.vec != 8 && cfg.vec != 1) return fail("take_q8: vector width must be 8 (128-bit stores) or 1, got %d", cfg.vec);
+  if (cfg.vec == 8 && !(aligned(Wq, 8) && aligned(out, 16))) cfg.vec = 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t items = cfg.vec == 8 ? n * K / 8 : n * K;
+  int64_t grid = ceil_div(items, 256);
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  grid = grid > cap ? cap : grid;
+  if (cfg.vec == 8)
+    hipLaunchKernelGGL(take_q8_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x2*>(Wq),
+                       static_cast<const half_t*>(scale), static_cast<const int*>(ids), static_cast<u32x4*>(out), items, K / 8, V);
+  else
+    hipLaunchKernelGGL(take_q8_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s,
+                       static_cast<const unsigned char*>(Wq), static_cast<const half_t*>(scale), static_cast<const int*>(ids),
+                       static_cast<half_t*>(out), items, K, V);
+  return check_launch("take_q8");
+}
+
+extern "C" int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, int64_t N, int64_t K,
+                                const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (check_q8_shape("gemv_q8_f32", N, K) != 0) return -1;
+  if (N == 0) return 0;
+  if (!y || (K > 0 && (!x || !Wq || !scale))) return fail("gemv_q8_f32: NULL buffer");
+  if (overlaps(y, N * 4, Wq, N * K) || overlaps(y, N * 4, x, K * 4) || overlaps(y, N * 4, scale, N * (K / 32) * 4))
+    return fail("gemv_q8_f32: output overlaps an input");
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 4 : 2, 0, 0}, 1, 0};
+  if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
+  int64_t la[7];
+  if (describe_gemv(N, K, cfg, la) != 0) return -1;
+  const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float* xp = static_cast<const float*>(x);
+  const float* sp = static_cast<const float*>(scale);
+  float* yp = static_cast<float*>(y);
+  if (cfg.vec == 1) {
+    hipLaunchKernelGGL(gemv_q8_f32_scalar_kernel, grid, block, 0, s, xp, static_cast<const unsigned char*>(Wq), sp, yp, N, K);
+    return check_launch("gemv_q8_f32");
+  }
+  const unsigned* wp = static_cast<const unsigned*>(Wq);
+  switch (cfg.tile[0]) {
+    case 1: hipLaunchKernelGGL(gemv_q8_f32_kernel<1>, grid, block, 0, s, xp, wp, sp, yp, N, K); break;
+    case 2: hipLaunchKernelGGL(gemv_q8_f32_kernel<2>, grid, block, 0, s, xp, wp, sp, yp, N, K); break;
+    case 4: hipLaunchKernelGGL(gemv_q8_f32_kernel<4>, grid, block, 0, s, xp, wp, sp, yp, N, K); break;
+    case 8: hipLaunchKernelGGL(gemv_q8_f32_kernel<8>, grid, block, 0, s, xp, wp, sp, yp, N, K); break;
+  }
+  return check_launch("gemv_q8_f32");
 }

@@ -231,9 +231,9 @@ def attn_pv(P: torch.Tensor, V: torch.Tensor, out: torch.Tensor, cfg: Optional[D
     check(lib().dtas_attn_pv_f16(_p(P), _p(V), _p(out), heads, n, m, d, _cfg(cfg), _stream()), "dtas_attn_pv_f16")
 
 
-def _q8_shapes(what: str, Wq: torch.Tensor, scale: torch.Tensor):
-    if Wq.dim() != 2 or Wq.dtype not in (torch.int32, torch.uint32) or scale.dtype != torch.float16:
-        raise ValueError(f"{what}: expects 32-bit words [N, K/4] and fp16 scales [N, K/32]")
+def _q8_shapes(what: str, Wq: torch.Tensor, scale: torch.Tensor, scale_dtype=torch.float16):
+    if Wq.dim() != 2 or Wq.dtype not in (torch.int32, torch.uint32) or scale.dtype != scale_dtype:
+        raise ValueError(f"{what}: expects 32-bit words [N, K/4] and {str(scale_dtype).split('.')[-1]} scales [N, K/32]")
     N, K = Wq.shape[0], Wq.shape[1] * 4
     if K % 32 != 0 or tuple(scale.shape) != (N, K // 32):
         raise ValueError(f"{what}: K = {K} and scales {tuple(scale.shape)} do not form groups of 32")
@@ -248,6 +248,30 @@ def decode_q8(Wq: torch.Tensor, scale: torch.Tensor, W: torch.Tensor, cfg: Optio
     if W.dtype != torch.float16 or W.numel() != N * K:
         raise ValueError("decode_q8: expects an fp16 output of N * K elements")
     check(lib().dtas_decode_q8_f16(_p(Wq), _p(scale), _p(W), N, K, _cfg(cfg), _stream()), "dtas_decode_q8_f16")
+
+
+def take_q8(Wq: torch.Tensor, scale: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """out[n,K] (fp16) = rows ids[i] of decode_q8(Wq, scale), the embedding lookup of the 8-bit model:
+    fused_fused_decode1_take1 (dolly-v2-3b-q8f16_1/before_dl.py:357-369) and, one row, fused_fused_decode1_take
+    (:346-355).  ids int32; values outside [0, V) are clipped to the nearest row."""
+    _dev(Wq, scale, ids, out)
+    V, K = _q8_shapes("take_q8", Wq, scale)
+    n = ids.numel()
+    if ids.dtype != torch.int32 or out.dtype != torch.float16 or out.numel() != n * K:
+        raise ValueError("take_q8: expects int32 ids[n] and an fp16 output of n * K elements")
+    check(lib().dtas_take_q8_f16(_p(Wq), _p(scale), _p(ids), _p(out), n, V, K, _cfg(cfg), _stream()), "dtas_take_q8_f16")
+
+
+def gemv_q8_f32(x: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, y: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """fp32 y[N] = x[K] . W^T with W = float32(byte - 127) * scale[N, K/32] (fp32 scales), never written: the vocabulary
+    projection of the 8-bit model, fused_fused_decode6_NT_matmul5 (dolly-v2-3b-q8f16_1/before_dl.py:640-657)."""
+    _dev(x, Wq, scale, y)
+    N, K = _q8_shapes("gemv_q8_f32", Wq, scale, torch.float32)
+    if x.numel() != K or y.numel() != N:
+        raise ValueError("gemv_q8_f32: shape mismatch")
+    if x.dtype != torch.float32 or y.dtype != torch.float32:
+        raise ValueError("gemv_q8_f32: expects fp32 x and y")
+    check(lib().dtas_gemv_q8_f32(_p(x), _p(Wq), _p(scale), _p(y), N, K, _cfg(cfg), _stream()), "dtas_gemv_q8_f32")
 
 
 def gemv_q8(x: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor], y: torch.Tensor,

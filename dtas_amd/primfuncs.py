@@ -204,6 +204,28 @@ def fused_decode(N: int = 2560, K: int = 2560, name: Optional[str] = None) -> Pr
     return PrimFunc(name or "fused_decode3", params, blocks, op="decode_q8", attrs={"tir.noalias": True})
 
 
+def fused_decode_take(V: int = 50280, K: int = 2560, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """out(n,K) fp16 = rows ids(n) of the dequantised table: fused_fused_decode1_take1
+    (dolly-v2-3b-q8f16_1/before_dl.py:357-369; n dynamic) or, with ``decode``, fused_fused_decode1_take (:346-355;
+    one row).  Parameters: Wq, scale, ids, out."""
+    n = 1 if decode else "n"
+    params = [Buffer("lv775", (V, K // 4), "uint32"), Buffer("lv776", (V, K // 32), "float16"), Buffer("lv", (n,), "int32"),
+              Buffer("T_take_intermediate", (n, K), "float16")]
+    blocks = [Block("T_take", "SS", ["lv", "lv775", "lv776"], ["T_take_intermediate"])]
+    return PrimFunc(name or ("fused_fused_decode1_take" if decode else "fused_fused_decode1_take1"), params, blocks,
+                    op="take_q8", attrs={"tir.noalias": True})
+
+
+def fused_decode_NT_matmul_f32(N: int = 50280, K: int = 2560, name: Optional[str] = None) -> PrimFunc:
+    """y(1,1,N) fp32 = x(1,1,K) fp32 . W^T with W = float32(byte - 127) * scale(N, K/32) fp32:
+    fused_fused_decode6_NT_matmul5, dolly-v2-3b-q8f16_1/before_dl.py:640-657.  Parameters: Wq, scale, x, out."""
+    params = [Buffer("lv772", (N, K // 4), "uint32"), Buffer("lv773", (N, K // 32), "float32"), Buffer("lv771", (1, 1, K), "float32"),
+              Buffer("NT_matmul_intermediate", (1, 1, N), "float32")]
+    blocks = [Block("decode", "SS", ["lv772", "lv773"], ["decode_intermediate_intermediate"]),
+              Block("NT_matmul", "SSSR", ["lv771", "decode_intermediate_intermediate"], ["NT_matmul_intermediate"])]
+    return PrimFunc(name or "fused_fused_decode6_NT_matmul5", params, blocks, op="gemv_q8_f32", attrs={"tir.noalias": True})
+
+
 def fused_decode_NT_matmul_add(N: int = 7680, K: int = 2560, gelu: bool = False, name: Optional[str] = None) -> PrimFunc:
     """y(1,1,N) = x(1,1,K) . decode(Wq, scale)^T + bias (then GELU): fused_fused_decode2_fused_NT_matmul_add
     (dolly-v2-3b-q8f16_1/before_dl.py:401-426) or, with ``gelu``, fused_fused_decode4_fused_NT_matmul3_add2_gelu

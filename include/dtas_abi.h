@@ -246,6 +246,16 @@ int dtas_gemv_f32(const void* x, const void* W, void* y, int64_t N, int64_t K, c
  *   the fp16 steps of dtas_gemm_f16_fused.  cfg, when given, is a DTAS_GEMV_SPLITK row as for dtas_gemv_f16
  *   (vec 8 = 128-bit accesses); NULL = 256 threads and 2 (N >= 16384: 4) rows per workgroup.
  */
+/* dtas_take_q8_f16: fused_fused_decode1_take1 (:357-369; one row: fused_fused_decode1_take, :346-355), the
+ *   embedding rows dequantised: out[n, K] fp16 = decode(Wq, scale)[ids[i], :], Wq[V, K/4], scale[V, K/32] fp16,
+ *   ids[n] int32.  Ids outside [0, V) are clipped to the nearest row.  cfg as dtas_decode_q8_f16.
+ * dtas_gemv_q8_f32: fused_fused_decode6_NT_matmul5 (:640-657), the vocabulary projection of the 8-bit model:
+ *   x[K], y[N] and scale[N, K/32] are fp32; W = float32(fp16(byte) - fp16(127)) * scale (one fp32 rounding);
+ *   y = x . W^T in fp32.  cfg as dtas_gemv_q8_f16. */
+int dtas_take_q8_f16(const void* Wq, const void* scale, const void* ids, void* out, int64_t n, int64_t V, int64_t K,
+                     const dtas_config* cfg, void* stream);
+int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, int64_t N, int64_t K,
+                     const dtas_config* cfg, void* stream);
 /* dtas_gemm_q8_f16_fused: C[M,N] = epilogue(A[M,K] . W^T) with W dequantised on its way into the LDS, never
  * written: the dynamic-n forms fused_fused_decode2_fused_NT_matmul6_add4 (:371-399), ..decode4.._matmul9_add6_gelu1
  * (:504-581), ..decode5.._matmul4_add1; epilogues as dtas_gemm_f16_fused.  cfg, when given: a DTAS_GEMM_MFMA row

@@ -69,6 +69,8 @@ class _C:
                 "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
                 "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
                 "oracle_gemv_f32": [vp, vp, vp, i64, i64, ci],
+                "oracle_take_q8_f16": [vp, vp, vp, vp, i64, i64, ci],
+                "oracle_gemv_q8_f32": [vp, vp, vp, vp, i64, i64, ci],
                 "oracle_decode_q8_f16": [vp, vp, vp, i64, i64, ci],
                 "oracle_gemv_q8_f16": [vp, vp, vp, vp, vp, i64, i64, ci, ci, ci],
             }
@@ -208,6 +210,26 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         out = np.empty(x.shape[:-1] + (N,), dtype=np.float16)
         bp = _ptr(bias) if bias is not None else None
         _C.lib().oracle_gemv_q8_f16(_ptr(x), _ptr(wq), _ptr(scale), bp, _ptr(out), N, K, kind, int(acc_f16), threads)
+        return out
+
+    @staticmethod
+    def take_q8(wq, scale, ids, threads: int = 1) -> np.ndarray:
+        """fp16 out[n,K]: rows ids[i] of decode_q8(wq, scale)."""
+        V, K = wq.shape[0], wq.shape[1] * 4
+        assert wq.dtype == np.uint32 and scale.dtype == np.float16 and scale.shape == (V, K // 32) and ids.dtype == np.int32
+        assert ids.size == 0 or (0 <= ids.min() and ids.max() < V)
+        out = np.empty((ids.size, K), dtype=np.float16)
+        _C.lib().oracle_take_q8_f16(_ptr(wq), _ptr(scale), _ptr(ids), _ptr(out), ids.size, K, threads)
+        return out
+
+    @staticmethod
+    def gemv_q8_f32(x, wq, scale, threads: int = 1) -> np.ndarray:
+        """fp32 y[N] = x[K] . W^T with W = float32(byte - 127) * fp32 scale[N,K/32]."""
+        N, K = wq.shape[0], wq.shape[1] * 4
+        assert x.dtype == np.float32 and x.size == K and wq.dtype == np.uint32
+        assert scale.dtype == np.float32 and scale.shape == (N, K // 32)
+        out = np.empty(x.shape[:-1] + (N,), dtype=np.float32)
+        _C.lib().oracle_gemv_q8_f32(_ptr(x), _ptr(wq), _ptr(scale), _ptr(out), N, K, threads)
         return out
 
     @staticmethod

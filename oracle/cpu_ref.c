@@ -444,6 +444,35 @@ void oracle_gemv_f32(const float* x, const float* W, float* y, int64_t N, int64_
   }
 }
 
+/* ========================================================================
+ * The other q8 forms of the same model file (experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py):
+ *  fused_fused_decode1_take1 (:357-369; the one-row form fused_fused_decode1_take :346-355):
+ *      out[i, j] = decode(Wq, S)[ids[i], j]                      -- the embedding rows, dequantised
+ *  fused_fused_decode6_NT_matmul5 (:640-657): fp32 scales, fp32 x and y
+ *      W[i, j] = float32(fp16(byte) - fp16(127)) * S32[i, j/32]   -- one fp32 rounding (the product)
+ *      y[i]    = sum_k x[k] * W[i, k]                             -- fp32, k ascending, no contraction
+ * Pinned by: rows of the pinned dequantiser picked with numpy indexing (bit-exact); numpy float32 arithmetic on the
+ * bytes (bit-exact W), the pinned fp32 GEMV on that W (bit-exact y), float64 closed form, one-hot x.
+ * ======================================================================== */
+void oracle_take_q8_f16(const uint32_t* Wq, const f16* S, const int32_t* ids, f16* out, int64_t n, int64_t K, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t ij = 0; ij < n * K; ++ij) out[ij] = decode_q8(Wq, S, K, ids[ij / K], ij % K);
+}
+
+void oracle_gemv_q8_f32(const float* x, const uint32_t* Wq, const float* S, float* y, int64_t N, int64_t K, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t i = 0; i < N; ++i) {
+    float acc = 0.f;
+    for (int64_t k = 0; k < K; ++k) {
+      const uint32_t byte = (Wq[i * (K / 4) + k / 4] >> (8 * (k % 4))) & 255u;
+      const float q = h2f(f2h(h2f(f2h((float)byte)) - 127.f));
+      const float w = q * S[i * (K / 32) + k / 32];
+      acc = acc + x[k] * w;
+    }
+    y[i] = acc;
+  }
+}
+
 int oracle_max_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

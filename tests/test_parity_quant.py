@@ -278,3 +278,126 @@ def test_gemm_q8_exact_cases_fallback_and_errors(oracle):
     with pytest.raises(_lib.DtasError, match="needs both residuals"):
         ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, None, _lib.EPI_BIAS_ADD2)
     assert _lib.lib().dtas_gemm_q8_f16_fused(None, None, None, None, None, None, None, 0, 96, 128, 0, None, None) == 0
+
+
+# ---- the embedding gather and the fp32-scale vocabulary projection (before_dl.py:346-369, :640-657) ----------
+
+@pytest.mark.parametrize("V,K,n", [(50280, 2560, 1), (50280, 2560, 300), (50280, 2560, 4096), (7, 32, 19), (100, 96, 1)])
+def test_take_is_bit_exact(oracle, V, K, n):
+    wq, scale = _weights(V, K, V + n)
+    ids = np.random.default_rng(n).integers(0, V, n).astype(np.int32)
+    ids[0], ids[-1] = V - 1, 0
+    out = Guarded((n, K), torch.float16)
+    ops.take_q8(_words(wq), dev(scale), dev(ids), out.t)
+    assert np.array_equal(out.check().view(np.uint16), oracle.c.take_q8(wq, scale, ids, threads=8).view(np.uint16))
+
+
+def test_take_clips_ids_scalar_path_and_errors(oracle):
+    wq, scale = _weights(10, 64, 3)
+    ids = np.array([-5, 0, 9, 10, 2 ** 31 - 1, -2 ** 31], np.int32)
+    want = oracle.c.take_q8(wq, scale, np.clip(ids, 0, 9).astype(np.int32))
+    for vec in (8, 1):
+        out = Guarded((6, 64), torch.float16)
+        ops.take_q8(_words(wq), dev(scale), dev(ids), out.t, cfg(variant=_lib.ELT_VECTOR, block=256, vec=vec))
+        assert np.array_equal(out.check().view(np.uint16), want.view(np.uint16))
+    buf = torch.empty(6 * 64 + 1, dtype=torch.float16, device="cuda")            # 2-byte aligned output: element path
+    ops.take_q8(_words(wq), dev(scale), dev(ids), buf[1:].view(6, 64))
+    torch.cuda.synchronize()
+    assert np.array_equal(buf[1:].cpu().numpy().reshape(6, 64).view(np.uint16), want.view(np.uint16))
+    L = _lib.lib()
+    assert L.dtas_take_q8_f16(None, None, None, None, 0, 10, 64, None, None) == 0
+    assert L.dtas_take_q8_f16(None, None, None, None, 3, 10, 64, None, None) == -1 and b"NULL" in L.dtas_last_error()
+    assert L.dtas_take_q8_f16(None, None, None, None, 3, 0, 64, None, None) == -1 and b"empty table" in L.dtas_last_error()
+    assert L.dtas_take_q8_f16(None, None, None, None, -1, 10, 64, None, None) == -1
+    with pytest.raises(ValueError, match="int32 ids"):
+        ops.take_q8(_words(wq), dev(scale), torch.zeros(6, dtype=torch.int64, device="cuda"), torch.empty(6, 64, dtype=torch.float16, device="cuda"))
+
+
+def _weights_f32(N, K, seed):
+    rng = np.random.default_rng(seed)
+    wq = rng.integers(0, 2 ** 32, (N, K // 4), dtype=np.uint32)
+    return wq, (rng.random((N, K // 32)) * 0.02 + 0.001).astype(np.float32)
+
+
+def _check_gemv_f32(got, x, wq, scale, oracle):
+    N, K = wq.shape[0], wq.shape[1] * 4
+    want = oracle.c.gemv_q8_f32(x, wq, scale, threads=8)
+    w64 = (wq.view(np.uint8).reshape(N, K).astype(np.float64) - 127) * np.repeat(scale.astype(np.float64), 32, axis=1)
+    f64 = w64 @ x.astype(np.float64)
+    mag = np.abs(w64) @ np.abs(x.astype(np.float64))
+    assert np.isfinite(got).all()
+    assert (np.abs(got.astype(np.float64) - f64) <= 1e-2 * np.abs(f64) + 1e-5 * mag).all()          # rtol 1e-2 where the sum does not cancel
+    assert (np.abs(got.astype(np.float64) - f64) <= (K + 2) * 2.0 ** -24 * mag).all()                # fp32 summation, any order
+    assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 2 * (K + 2) * 2.0 ** -24 * mag).all()
+
+
+@pytest.mark.parametrize("N,K", [(50280, 2560), (2560, 10240), (33, 64), (5, 32)])
+def test_gemv_f32_scales_builtin_config(oracle, N, K):
+    wq, scale = _weights_f32(N, K, N + K)
+    x = np.random.default_rng(1).standard_normal(K).astype(np.float32)
+    out = Guarded((1, 1, N), torch.float32)
+    ops.gemv_q8_f32(dev(x), _words(wq), dev(scale), out.t)
+    _check_gemv_f32(out.check().reshape(N), x, wq, scale, oracle)
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 8])
+@pytest.mark.parametrize("block", [64, 256, 512])
+def test_gemv_f32_scales_every_row_count_and_block(oracle, rows, block):
+    N, K = 1001, 2560
+    wq, scale = _weights_f32(N, K, rows + block)
+    x = np.random.default_rng(2).standard_normal(K).astype(np.float32)
+    out = Guarded((N,), torch.float32)
+    ops.gemv_q8_f32(dev(x), _words(wq), dev(scale), out.t, cfg(variant=_lib.GEMV_SPLITK, block=block, vec=8, unroll=2, tile=[rows, 0, 0]))
+    _check_gemv_f32(out.check(), x, wq, scale, oracle)
+
+
+def test_gemv_f32_scales_exact_cases_scalar_path_and_errors(oracle):
+    wq, scale = _weights_f32(40, 96, 5)
+    w32 = (wq.view(np.uint8).reshape(40, 96).astype(np.float32) - np.float32(127)) * np.repeat(scale, 32, axis=1)
+    for k in (0, 31, 32, 95):                       # one-hot x returns a column of W: the rounded fp32 product, exactly
+        e = np.zeros(96, np.float32)
+        e[k] = 1
+        for c in (None, cfg(variant=_lib.GEMV_SPLITK, block=256, vec=1, unroll=2, tile=[1, 0, 0])):
+            out = Guarded((40,), torch.float32)
+            ops.gemv_q8_f32(dev(e), _words(wq), dev(scale), out.t, c)
+            assert np.array_equal(out.check().view(np.uint32), w32[:, k].view(np.uint32))
+    x = np.random.default_rng(3).standard_normal(96).astype(np.float32)
+    buf = torch.empty(97, dtype=torch.float32, device="cuda")                       # x only 4-byte aligned: element path
+    buf[1:] = dev(x)
+    out = Guarded((40,), torch.float32)
+    ops.gemv_q8_f32(buf[1:], _words(wq), dev(scale), out.t)
+    _check_gemv_f32(out.check(), x, wq, scale, oracle)
+    L = _lib.lib()
+    assert L.dtas_gemv_q8_f32(None, None, None, None, 0, 64, None, None) == 0
+    assert L.dtas_gemv_q8_f32(None, None, None, None, 4, 48, None, None) == -1 and b"multiple of the scale group" in L.dtas_last_error()
+    assert L.dtas_gemv_q8_f32(None, None, None, None, 4, 64, None, None) == -1 and b"NULL" in L.dtas_last_error()
+    with pytest.raises(ValueError, match="float32 scales"):
+        ops.gemv_q8_f32(dev(x), _words(wq), dev(scale.astype(np.float16)), torch.empty(40, dtype=torch.float32, device="cuda"))
+
+
+def test_take_and_vocabulary_projection_through_the_primfunc_descriptors(oracle):
+    from dtas_amd import primfuncs as pf
+    from dtas_amd.arch import MI355X
+    from dtas_amd.common.analisys import FuncInfo, FuncKind
+    from dtas_amd.engine.tuner import Engine
+
+    V, K = 50280, 2560
+    funcs = [pf.fused_decode_take(V, K), pf.fused_decode_take(V, K, decode=True), pf.fused_decode_NT_matmul_f32(V, K)]
+    assert [f.name for f in funcs] == ["fused_fused_decode1_take1", "fused_fused_decode1_take", "fused_fused_decode6_NT_matmul5"]
+    assert FuncInfo(funcs[0]).kind == FuncKind.kFunc_Elementwise and FuncInfo(funcs[2]).kind == FuncKind.kFunc_GEMV
+    rt = Engine(topk=2, parallel_build=False).tune_module(pf.module(*funcs, upper_bound={"n": 1024}), MI355X())
+    wq, scale = _weights(V, K, 12)
+    ids = np.random.default_rng(4).integers(0, V, 77).astype(np.int32)
+    out = torch.empty(77, K, dtype=torch.float16, device="cuda")
+    rt["fused_fused_decode1_take1"](_words(wq), dev(scale), dev(ids), out)
+    one = torch.empty(1, K, dtype=torch.float16, device="cuda")
+    rt["fused_fused_decode1_take"](_words(wq), dev(scale), dev(ids[:1]), one)
+    s32 = scale.astype(np.float32)
+    x = np.random.default_rng(5).standard_normal(K).astype(np.float32)
+    y = torch.empty(1, 1, V, dtype=torch.float32, device="cuda")
+    rt["fused_fused_decode6_NT_matmul5"](_words(wq), dev(s32), dev(x).view(1, 1, K), y)
+    torch.cuda.synchronize()
+    want = oracle.c.take_q8(wq, scale, ids, threads=8)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    assert np.array_equal(one.cpu().numpy().view(np.uint16), want[:1].view(np.uint16))
+    _check_gemv_f32(y.cpu().numpy().reshape(V), x, wq, s32, oracle)
