@@ -1623,20 +1623,21 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : 2, 8, 0}, 1, 0};
   } else {
     // what this op moves is P (2*n*m bytes per head).  Measured over n = m = 128 .. 4096 with 32 heads of 80:
-    // 64-row tiles while 128-row tiles would leave most CUs idle; three stages when a CU holds one
-    // workgroup anyway (up to one 128-row tile per CU, or 256-row tiles once there are two rounds of
-    // them); in between, two workgroups of two stages per CU
+    // 64-row tiles while 128-row tiles would leave most CUs idle; 128-row tiles with three stages up to
+    // one per CU; 256-row tiles with three stages beyond (n = m = 1280: 37 us against 44 for 128x128
+    // with three stages and 61 with two; 2048: 74 / 79 / 98).  Head dimensions up to 64 keep the
+    // 64-column tiles: two workgroups of two stages per CU
     const int64_t t128 = heads * ceil_div(n, 128);
     const int bn = d <= 64 ? 64 : 128;
     if (t128 <= kNumCU / 4) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, bn, kBK}, 1, 0};
     else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
-    else if (t128 > 2 * kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
+    else if (bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
     else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
     // Fewer workgroups than CUs and many keys: the workgroups of a tile split m.  Fitted to measurements at
     // 13 .. 256 rows against 512 .. 8192 keys: a k tile costs a workgroup ~0.8 us, combining S partial tiles
     // ~3 / 5.5 / 10 us for S = 2 / 4 / 8 (16 loses everywhere).
     const int64_t wgs = heads * ceil_div(n, cfg.tile[0]), ktiles = ceil_div(m, kBK);
-    if (wgs < kNumCU) {
+    if (wgs < kNumCU && cfg.tile[0] <= 128) {  // (partial tiles of 256 rows cost more to combine than a split saves)
       const double combine[4] = {0.0, 3.0, 5.5, 10.0};
       const double whole = 0.8 * static_cast<double>(ktiles);
       double best = 0.8 * whole;  // (a split has to promise a fifth less: the fit is coarse)
