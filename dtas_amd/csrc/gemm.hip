@@ -1549,10 +1549,13 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   if (overlaps(out, heads * n * m * 4, Q, heads * n * d * 2) || overlaps(out, heads * n * m * 4, Kmat, heads * m * d * 2) ||
       overlaps(out, heads * n * m * 4, mask, n * m * 2))
     return fail("attn_scores: output overlaps an input");
-  if (!user && d <= 2 * kBK) {
-    // the walking kernel: 128x64 tiles, at most three workgroups per CU (their LDS allows no more)
-    const unsigned tm = static_cast<unsigned>(ceil_div(n, 128)), tn = static_cast<unsigned>(ceil_div(m, 64));
-    const int64_t total = static_cast<int64_t>(tm) * tn * heads;
+  // the walking kernel: 128x64 tiles, at most three workgroups per CU (their LDS allows no more).  Up to 64 query
+  // rows half of such a tile would be idle, and fewer tiles than CUs leave CUs idle: 64x64 tiles of the general
+  // kernel then (n = 64 against 2048 keys: 6.9 us against 10.3)
+  const unsigned tm = static_cast<unsigned>(ceil_div(n, 128)), tn = static_cast<unsigned>(ceil_div(m, 64));
+  const int64_t total = static_cast<int64_t>(tm) * tn * heads;
+  const bool small = n <= 64 || total < kNumCU;
+  if (!user && d <= 2 * kBK && !small) {
     if (total > 0x7fffffff) return fail("attn_scores: too many tiles");
     const int64_t grid = total < 3 * kNumCU ? total : 3 * kNumCU;
     hipLaunchKernelGGL((attn_scores_kernel<128, 64>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, static_cast<hipStream_t>(stream),
@@ -1569,7 +1572,7 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
     // is mostly latency: measured best are 64x64 while 128x128 tiles do not give every CU a
     // workgroup, 128x128 up to ~1M scores per head, 128x64 (three workgroups per CU) beyond
     const int64_t t128 = heads * ceil_div(n, 128) * ceil_div(m, 128);
-    const int bm = t128 >= kNumCU ? 128 : 64, bn = t128 < kNumCU ? 64 : (n * m >= (int64_t{1} << 20) ? 64 : 128);
+    const int bm = t128 >= kNumCU && !small ? 128 : 64, bn = t128 < kNumCU || small ? 64 : (n * m >= (int64_t{1} << 20) ? 64 : 128);
     cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {bm, bn, kBK}, 1, 0};
   }
   if (cfg.variant != DTAS_GEMM_MFMA || cfg.vec != 8) return fail("attn_scores: only the MFMA kernels (vec 8) serve this op");
@@ -1637,13 +1640,17 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     // 13 .. 256 rows against 512 .. 8192 keys: a k tile costs a workgroup ~0.8 us, combining S partial tiles
     // ~3 / 5.5 / 10 us for S = 2 / 4 / 8 (16 loses everywhere).
     const int64_t wgs = heads * ceil_div(n, cfg.tile[0]), ktiles = ceil_div(m, kBK);
-    if (wgs < kNumCU && cfg.tile[0] <= 128) {  // (partial tiles of 256 rows cost more to combine than a split saves)
+    // 128-row tiles (one workgroup per CU) gain only while all parts run at once: 512 rows against 4096 keys
+    // take 47 us in two parts, 58 whole, 80 in eight.  Partial tiles of 256 rows cost more to combine than a
+    // split saves.
+    const int64_t wg_limit = cfg.tile[0] <= 64 ? 4 * kNumCU : kNumCU;
+    if (wgs < kNumCU && cfg.tile[0] <= 128) {
       const double combine[4] = {0.0, 3.0, 5.5, 10.0};
       const double whole = 0.8 * static_cast<double>(ktiles);
       double best = 0.8 * whole;  // (a split has to promise a fifth less: the fit is coarse)
       for (int i = 1; i < 4; ++i) {
         const int split = 1 << i;
-        if (wgs * split > 4 * kNumCU || ktiles < 2 * split) break;
+        if (wgs * split > wg_limit || ktiles < 2 * split) break;
         const double t = 0.8 * static_cast<double>(ceil_div(ktiles, split)) + combine[i];
         if (t < best) {
           best = t;
