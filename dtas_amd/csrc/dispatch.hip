@@ -131,6 +131,7 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
 //    workgroup ~4 us (128x128), ~2.5 us (128x64), ~1 us (64x64; 2 us with more than one per CU)
 //    to add up; 256x128 splits while its workgroups fit one round and each keeps 32 k tiles or
 //    more (~5 us per partial tile);
+//  * a floor: W (2NK bytes) streams at 3.1 .. 4.1 TB/s depending on the tile (few rows against a very wide W);
 //  * M <= 32: the W-streaming SKINNY kernel, whose time grows with N*K (about 3.5 TB/s of W).
 struct GemmChoice {
   double us;
@@ -152,22 +153,25 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   };
   auto tiles_of = [&](int bm, int bn) { return static_cast<double>(ceil_div(M_hi, bm) * ceil_div(n, bn)); };
   const double kt = static_cast<double>(ktiles);
-  consider(gemm_rounds(tiles_of(256, 256), kNumCU) * 1.80 * kt, 256, 256, 512, 2, 1);
-  consider(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.045 * kt, 256, 128, 256, 3, 1);
-  consider(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 128, 128, 256, 2, 1);
+  // no candidate is faster than it streams W: TB/s measured at M = 64 against a 50280 x 2560 W
+  const double w_mb = 2.0 * static_cast<double>(n) * static_cast<double>(k) * 1e-6;
+  auto floored = [&](double us, double tbs) { return us > w_mb / tbs ? us : w_mb / tbs; };
+  consider(floored(gemm_rounds(tiles_of(256, 256), kNumCU) * 1.80 * kt, 3.5), 256, 256, 512, 2, 1);
+  consider(floored(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.045 * kt, 3.5), 256, 128, 256, 3, 1);
+  consider(floored(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 3.1), 128, 128, 256, 2, 1);
   for (int split = 1; split <= 4; ++split) {
     if (split > 1 && ktiles / split < 8) continue;
     const double steps = static_cast<double>(ceil_div(ktiles, split));
     const double t128 = tiles_of(128, 128) * split, t64 = tiles_of(64, 64) * split;
     if (split == 1 || t128 <= kNumCU)
-      consider((t128 <= kNumCU ? 0.8 + 0.2 * t128 / kNumCU : gemm_rounds(t128, kNumCU)) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 128, 128, 256, 4, split);
-    consider((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.0) * split : 0.0), 64, 64, 256, 4, split);
+      consider(floored((t128 <= kNumCU ? 0.8 + 0.2 * t128 / kNumCU : gemm_rounds(t128, kNumCU)) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 4.1), 128, 128, 256, 4, split);
+    consider(floored((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.0) * split : 0.0), 3.9), 64, 64, 256, 4, split);
     const double t256128 = tiles_of(256, 128) * split;
     if (split > 1 && steps >= 32 && t256128 <= kNumCU)
-      consider(gemm_rounds(t256128, kNumCU) * 1.045 * steps + 5.0 * split, 256, 128, 256, 3, split);
+      consider(floored(gemm_rounds(t256128, kNumCU) * 1.045 * steps + 5.0 * split, 3.5), 256, 128, 256, 3, split);
     const double t12864 = tiles_of(128, 64) * split;
     if (t12864 <= kNumCU)
-      consider(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 128, 64, 256, 4, split);
+      consider(floored(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 3.4), 128, 64, 256, 4, split);
   }
   if (M_hi <= 32) {
     const double skinny_us = static_cast<double>(n) * static_cast<double>(k) * 2.0 / 3.5e6 * (M_hi <= 8 ? 0.9 : M_hi <= 16 ? 0.95 : 1.35);

@@ -42,7 +42,8 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         to 4 workgroups per tile at ~4 us (128x128) / ~1 us (64x64; 2 us with more than one per CU) per partial
         tile; 128x64 (4 stages, at most one workgroup per CU) 0.47 us per k tile whatever the fill and ~2.5 us
         per partial tile; 256x128 splits too while its workgroups fit one round and each keeps 32 k tiles or
-        more (~5 us per partial tile)."""
+        more (~5 us per partial tile).  No candidate is faster than W (2NK bytes) streams through it: 3.1 .. 4.1 TB/s
+        by tile, measured with 64 rows against a 50280 x 2560 W."""
         cdiv = lambda a, b: -(-a // b)
         cus = self.arch.num_sm
         ktiles = cdiv(K, 64)
@@ -52,25 +53,28 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             return full + ((0.55 + 0.45 * rem / slots) if rem else 0.0)
 
         tiles = lambda bm, bn: cdiv(m_hi, bm) * cdiv(N, bn)
-        cands = [(rounds(tiles(256, 256), cus) * 1.80 * ktiles, (256, 256, 2, 1)),
-                 (rounds(tiles(256, 128), cus) * 1.045 * ktiles, (256, 128, 3, 1)),
-                 (rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, (128, 128, 2, 1))]
+        w_mb = 2.0 * float(N) * float(K) * 1e-6
+        floored = lambda us, tbs: us if us > w_mb / tbs else w_mb / tbs     # W streams at 3.1 .. 4.1 TB/s, by tile
+        cands = [(floored(rounds(tiles(256, 256), cus) * 1.80 * ktiles, 3.5), (256, 256, 2, 1)),
+                 (floored(rounds(tiles(256, 128), cus) * 1.045 * ktiles, 3.5), (256, 128, 3, 1)),
+                 (floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1))]
         for split in (1, 2, 3, 4):
             if split > 1 and ktiles // split < 8:
                 continue
             steps = cdiv(ktiles, split)
             t128, t64 = tiles(128, 128) * split, tiles(64, 64) * split
             if split == 1 or t128 <= cus:
-                cands.append(((0.8 + 0.2 * t128 / cus if t128 <= cus else rounds(t128, cus)) * 0.665 * steps + (4.0 * split if split > 1 else 0.0), (128, 128, 4, split)))
-            cands.append(((1.0 if t64 <= cus else 0.82 * -(-int(t64) // cus)) * 0.33 * steps
-                          + ((1.0 if t64 <= cus else 2.0) * split if split > 1 else 0.0),
+                cands.append((floored((0.8 + 0.2 * t128 / cus if t128 <= cus else rounds(t128, cus)) * 0.665 * steps
+                                      + (4.0 * split if split > 1 else 0.0), 4.1), (128, 128, 4, split)))
+            cands.append((floored((1.0 if t64 <= cus else 0.82 * -(-int(t64) // cus)) * 0.33 * steps
+                                  + ((1.0 if t64 <= cus else 2.0) * split if split > 1 else 0.0), 3.9),
                           (64, 64, 4, split)))
             t256128 = tiles(256, 128) * split
             if split > 1 and steps >= 32 and t256128 <= cus:
-                cands.append((rounds(t256128, cus) * 1.045 * steps + 5.0 * split, (256, 128, 3, split)))
+                cands.append((floored(rounds(t256128, cus) * 1.045 * steps + 5.0 * split, 3.5), (256, 128, 3, split)))
             t12864 = tiles(128, 64) * split
             if t12864 <= cus:
-                cands.append((0.47 * steps + (2.5 * split if split > 1 else 0.0), (128, 64, 4, split)))
+                cands.append((floored(0.47 * steps + (2.5 * split if split > 1 else 0.0), 3.4), (128, 64, 4, split)))
         best = cands[0]
         for c in cands[1:]:          # first strict minimum, in the library's order of evaluation
             if c[0] < best[0]:
