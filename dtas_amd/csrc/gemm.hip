@@ -1201,6 +1201,97 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
   }
 }
 
+// A few rows of A (M <= MV <= 4) against a W that is streamed once: R rows of W per wavefront, lane l
+// takes the 16-byte chunks l, l + 64, ... of each (a wavefront access is 1 KiB of one W row, non-temporal,
+// as in the GEMV kernel), multiplies each with the matching chunks of the MV rows of A (re-read per
+// wavefront; they stay in L1 / L2) by v_dot2_f32_f16, and holds R * MV fp32 sums.  At the end the sums are
+// added across the lanes by a reduce-scatter: in each of the first log2(R * MV) butterfly steps a lane hands
+// half of its values to its partner and keeps the other half, so the fold costs R * MV - 1 exchanges in all
+// instead of six per value; lane l ends with value l >> (6 - log2(R * MV)).  No LDS, no barrier: wavefronts
+// are independent.  This pays for two rows of A only (8.1 against 10.1 us at 4096 x 4096, 40 against 60 at
+// 32000 x 4096): every 16 bytes of W meet MV * 16 bytes of A from the L1, whose 64 bytes per clock bound
+// the kernel from four rows on (16 rows: 3x slower than the MFMA tiles), so the instantiations stop at MV = 4.
+template <int R, int MV>
+__global__ void __launch_bounds__(256) gemm_rows_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
+                                                        GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
+                                                        int64_t K) {
+  constexpr int NV = R * MV;
+  static_assert(NV >= 2 && NV <= 64 && (NV & (NV - 1)) == 0, "R * MV must be a power of two in [2, 64]");
+  const unsigned l = threadIdx.x & 63u;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * R;
+  if (row0 >= N) return;  // whole wavefronts leave together; nothing below synchronises across wavefronts
+  const int64_t chunks = K >> 3;
+  const u32x4* wv[R];
+  const u32x4* av[MV];
+#pragma unroll
+  for (int r = 0; r < R; ++r) wv[r] = reinterpret_cast<const u32x4*>(W + (row0 + r < N ? row0 + r : N - 1) * K);  // rows past N: re-read, never stored
+#pragma unroll
+  for (int m = 0; m < MV; ++m) av[m] = reinterpret_cast<const u32x4*>(A + (m < M ? m : M - 1) * K);                // likewise rows past M
+  float v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = 0.f;
+  auto dot8 = [](u32x4 a, u32x4 b, float acc) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned ai = a[i], bi = b[i];
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, ai), __builtin_bit_cast(f16x2, bi), acc, false);
+    }
+    return acc;
+  };
+  constexpr int U = R >= 4 ? 2 : 4;  // steps requested together: U * R KiB of W per wavefront in flight
+  int64_t i = l;
+  for (; i + (U - 1) * 64 < chunks; i += U * 64) {
+    u32x4 wr[U][R];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < R; ++r) wr[u][r] = load_stream(wv[r] + i + u * 64);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int m = 0; m < MV; ++m) {
+        const u32x4 xr = av[m][i + u * 64];
+#pragma unroll
+        for (int r = 0; r < R; ++r) v[r * MV + m] = dot8(xr, wr[u][r], v[r * MV + m]);
+      }
+  }
+  for (; i < chunks; i += 64) {
+    u32x4 wr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wr[r] = load_stream(wv[r] + i);
+#pragma unroll
+    for (int m = 0; m < MV; ++m) {
+      const u32x4 xr = av[m][i];
+#pragma unroll
+      for (int r = 0; r < R; ++r) v[r * MV + m] = dot8(xr, wr[r], v[r * MV + m]);
+    }
+  }
+  // reduce-scatter over the 64 lanes
+  int n = NV;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    if (n > 1) {
+      const int half = n >> 1;
+      const bool upper = (l & d) != 0;
+#pragma unroll
+      for (int j = 0; j < half; ++j) {
+        const float send = upper ? v[j] : v[j + half];
+        const float keep = upper ? v[j + half] : v[j];
+        v[j] = keep + __shfl_xor(send, d, 64);
+      }
+      n = half;
+    } else {
+      v[0] += __shfl_xor(v[0], d, 64);
+    }
+  }
+  constexpr int kShift = NV == 64 ? 0 : NV == 32 ? 1 : NV == 16 ? 2 : NV == 8 ? 3 : NV == 4 ? 4 : 5;
+  if ((l & ((1u << kShift) - 1u)) == 0) {
+    const unsigned idx = l >> kShift;  // = r * MV + m
+    const int64_t row = row0 + idx / MV, m = idx % MV;
+    if (row < N && m < M) finish(v[0], ep, C, m, row, N);
+  }
+}
+
 // Any K and alignment: one thread per element of C.  blockIdx.y = problem of a batched launch;
 // w_kmajor: W is [K][N] instead of [N][K]; ep.wscale set: W is 8-bit with group scales.
 __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
@@ -1437,6 +1528,19 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     la[6] = tn;
     return 0;
   }
+  if (cfg.variant == DTAS_GEMM_ROWS) {
+    const int mv = cfg.tile[0], r = cfg.tile[1];
+    if ((mv != 2 && mv != 4) || (r != 1 && r != 2 && r != 4))
+      return fail("gemm: the row kernel takes tile {2,4} rows of A x {1,2,4} rows of W, got %dx%d", mv, r);
+    if (M > mv) return fail("gemm: a row tile of %d rows cannot hold M=%lld", mv, (long long)M);
+    if (cfg.block != 64 && cfg.block != 128 && cfg.block != 256) return fail("gemm: the row kernel uses 64, 128 or 256 threads, got %d", cfg.block);
+    la[0] = ceil_div(N, static_cast<int64_t>(r) * (cfg.block / 64));
+    la[3] = cfg.block;
+    la[5] = 1;
+    la[6] = la[0];
+    if (la[0] > 0x7fffffff) return fail("gemm: too many workgroups");
+    return 0;
+  }
   if (cfg.variant == DTAS_GEMM_SKINNY) {
     const int mt = cfg.tile[0] / 16;
     if (cfg.tile[0] % 16 != 0 || mt < 1 || mt > 5 || cfg.tile[1] != 16)
@@ -1484,6 +1588,8 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
                            static_cast<const half_t*>(res2), epilogue, out_bytes == 4 ? 1 : 0, 0.f, 0, 0, 0, 0};
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMM_F16, M, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(A, 16) && aligned(W, 16);
+  // two rows of A (the first bucket's table row is sized for 16): W streamed in whole rows, as the GEMV does
+  if (!user && M == 2 && vec_ok) cfg = dtas_config{DTAS_GEMM_ROWS, 64, 8, 1, {2, 2, 8}, 1, 0};
   if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
   int64_t la[7];
   if (describe_gemm(M, N, K, cfg, la) != 0) return -1;
@@ -1494,6 +1600,15 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   void* c = C;
   if (cfg.vec == 1) {
     hipLaunchKernelGGL(gemm_scalar_kernel, dim3(static_cast<unsigned>(la[0])), dim3(256), 0, s, a, w, b, c, M, N, K, false);
+    return check_launch("gemm");
+  }
+  if (cfg.variant == DTAS_GEMM_ROWS) {
+    const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));
+#define DTAS_ROWS_CASE(MV_, R_) \
+  if (cfg.tile[0] == MV_ && cfg.tile[1] == R_) hipLaunchKernelGGL((gemm_rows_kernel<R_, MV_>), grid, block, 0, s, a, w, b, c, M, N, K)
+    DTAS_ROWS_CASE(2, 1); DTAS_ROWS_CASE(2, 2); DTAS_ROWS_CASE(2, 4);
+    DTAS_ROWS_CASE(4, 1); DTAS_ROWS_CASE(4, 2); DTAS_ROWS_CASE(4, 4);
+#undef DTAS_ROWS_CASE
     return check_launch("gemm");
   }
   if (cfg.variant == DTAS_GEMM_SKINNY) {

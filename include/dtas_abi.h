@@ -86,7 +86,9 @@ enum dtas_variant {
   DTAS_GEMV_SPLITK = 0,   /* K split over the lanes and wavefronts of a workgroup */
   /* GEMM (python/dtas/schedule/tir_wmma.py:20-222) */
   DTAS_GEMM_MFMA = 0,     /* LDS-tiled MFMA, tile = tile[0] x tile[1] x tile[2] */
-  DTAS_GEMM_SKINNY = 1    /* small M: weight-streaming MFMA 16x16x32, split over N and K */
+  DTAS_GEMM_SKINNY = 1,   /* small M: weight-streaming MFMA 16x16x32, split over N and K */
+  DTAS_GEMM_ROWS = 2      /* M <= 4: W streamed once in whole rows (tile[1] per wavefront) against tile[0] >= M
+                             rows of A on the vector ALU; tile = {2|4, 1|2|4, 8}, block 64 / 128 / 256 */
 };
 
 /* One row of a call table: the launch-relevant part of the reference's *Config classes

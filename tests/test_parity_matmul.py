@@ -139,6 +139,45 @@ def test_gemm_every_skinny_tile(oracle, rows, block, N, K):
         _check(out.check(), oracle.c.gemm(a, w, threads=8), oracle.np64.gemm(a, w))
 
 
+@pytest.mark.parametrize("mv,r", [(2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4)])
+@pytest.mark.parametrize("block", [64, 128, 256])
+@pytest.mark.parametrize("N,K", [(64, 64), (101, 520), (4096, 4096), (33, 8 * 64 * 5 + 8)])
+def test_gemm_row_kernel_every_variant(oracle, mv, r, block, N, K):
+    # W streamed in whole rows against up to four rows of A: every M the tile holds, ragged N, K with a tail
+    for M in range(1, mv + 1):
+        a, w = _inputs(M, N, K, M + N + K)
+        bias = np.random.default_rng(M).uniform(-1, 1, N).astype(np.float16)
+        out = Guarded((M, N), torch.float16)
+        ops.gemm(dev(a), dev(w), dev(bias), out.t, cfg(variant=_lib.GEMM_ROWS, block=block, vec=8, tile=[mv, r, 8]))
+        _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+
+
+def test_gemm_two_rows_take_the_row_kernel_with_every_epilogue_and_errors(oracle):
+    for kind, N, K in ((0, 4096, 4096), (1, 2560, 2560), (2, 2560, 2560), (3, 10240, 2560)):
+        a, w, bias, r1, r2 = _fused_inputs(2, N, K, 40 + kind)
+        res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+        out = Guarded((1, 2, N), torch.float32 if kind == 2 else torch.float16)
+        ops.gemm(dev(a), dev(w), dev(bias), out.t, None, epilogue=kind, res1=res[0], res2=res[1])
+        want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+        _check_fused(out.check().reshape(2, N), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+    a, w = _inputs(2, 96, 64, 3)
+    x = np.zeros((2, 64), np.float16)
+    x[0, 5], x[1, 63] = 1, 1
+    out = Guarded((2, 96), torch.float16)
+    ops.gemm(dev(x), dev(w), None, out.t)
+    got = out.check()
+    assert_bits_equal(got[0], w[:, 5].copy())          # one-hot rows of A select columns of W exactly
+    assert_bits_equal(got[1], w[:, 63].copy())
+    out = torch.empty(5, 96, dtype=torch.float16, device="cuda")
+    a5, _ = _inputs(5, 96, 64, 4)
+    with pytest.raises(_lib.DtasError, match="cannot hold M=5"):
+        ops.gemm(dev(a5), dev(w), None, out, cfg(variant=_lib.GEMM_ROWS, block=64, vec=8, tile=[4, 2, 8]))
+    with pytest.raises(_lib.DtasError, match="row kernel takes tile"):
+        ops.gemm(dev(a), dev(w), None, out[:2], cfg(variant=_lib.GEMM_ROWS, block=64, vec=8, tile=[8, 2, 8]))
+    with pytest.raises(_lib.DtasError, match="64, 128 or 256 threads"):
+        ops.gemm(dev(a), dev(w), None, out[:2], cfg(variant=_lib.GEMM_ROWS, block=512, vec=8, tile=[2, 2, 8]))
+
+
 def test_gemm_exact_cases(oracle):
     rng = np.random.default_rng(7)
     a = rng.standard_normal((300, 256)).astype(np.float16)
