@@ -128,10 +128,10 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
 //  * 64x64: 0.33 us per k tile up to 256 workgroups, x 0.82 * (workgroups on the fullest CU) beyond;
 //  * 128x64 (4 stages, one workgroup per CU at most): 0.47 us per k tile whatever the fill;
 //  * few tiles: K split over up to 4 workgroups per tile, each partial tile costing the last
-//    workgroup ~4 us (128x128), ~2.5 us (128x64), ~1 us (64x64; 2 us with more than one per CU)
+//    workgroup ~4 us (128x128), ~2.5 us (128x64), ~1 us (64x64; 2.5 us with more than one per CU)
 //    to add up; 256x128 splits while its workgroups fit one round and each keeps 32 k tiles or
 //    more (~5 us per partial tile);
-//  * a floor: W (2NK bytes) streams at 3.1 .. 4.1 TB/s depending on the tile (few rows against a very wide W);
+//  * a floor: W (2NK bytes) streams at 3.1 .. 4.3 TB/s depending on the tile (few rows against a very wide W);
 //  * M <= 32: the W-streaming SKINNY kernel, whose time grows with N*K (about 3.5 TB/s of W).
 struct GemmChoice {
   double us;
@@ -165,7 +165,7 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     const double t128 = tiles_of(128, 128) * split, t64 = tiles_of(64, 64) * split;
     if (split == 1 || t128 <= kNumCU)
       consider(floored((t128 <= kNumCU ? 0.8 + 0.2 * t128 / kNumCU : gemm_rounds(t128, kNumCU)) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 4.1), 128, 128, 256, 4, split);
-    consider(floored((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.0) * split : 0.0), 3.9), 64, 64, 256, 4, split);
+    consider(floored((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.5) * split : 0.0), 4.3), 64, 64, 256, 4, split);
     const double t256128 = tiles_of(256, 128) * split;
     if (split > 1 && steps >= 32 && t256128 <= kNumCU)
       consider(floored(gemm_rounds(t256128, kNumCU) * 1.045 * steps + 5.0 * split, 3.5), 256, 128, 256, 3, split);
@@ -174,7 +174,10 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
       consider(floored(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 3.4), 128, 64, 256, 4, split);
   }
   if (M_hi <= 32) {
-    const double skinny_us = static_cast<double>(n) * static_cast<double>(k) * 2.0 / 3.5e6 * (M_hi <= 8 ? 0.9 : M_hi <= 16 ? 0.95 : 1.35);
+    // (one workgroup per 16 rows of W: fewer than one per CU leave CUs idle)
+    const double skinny_wgs = static_cast<double>(ceil_div(n, 16));
+    const double skinny_us = static_cast<double>(n) * static_cast<double>(k) * 2.0 / 3.5e6 * (M_hi <= 8 ? 0.9 : M_hi <= 16 ? 0.95 : 1.35) *
+                             (skinny_wgs < kNumCU ? kNumCU / skinny_wgs : 1.0);
     if (skinny_us <= best.us) return make(DTAS_GEMM_SKINNY, 512, 8, 4, static_cast<int>((M_hi + 15) / 16 * 16), 16, 32);
   }
   return make(DTAS_GEMM_MFMA, best.block, 8, best.stages, best.bm, best.bn, 64, best.split);

@@ -39,10 +39,10 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         a partly filled last round costs 0.55 + 0.45 * fill of a full one (0.8 + 0.2 * fill for 128x128 with 4 stages
         in a single round); 64x64 0.33 us per k tile up to
         one workgroup per CU, x 0.82 * (workgroups on the fullest CU) beyond; with few tiles K is split over up
-        to 4 workgroups per tile at ~4 us (128x128) / ~1 us (64x64; 2 us with more than one per CU) per partial
+        to 4 workgroups per tile at ~4 us (128x128) / ~1 us (64x64; 2.5 us with more than one per CU) per partial
         tile; 128x64 (4 stages, at most one workgroup per CU) 0.47 us per k tile whatever the fill and ~2.5 us
         per partial tile; 256x128 splits too while its workgroups fit one round and each keeps 32 k tiles or
-        more (~5 us per partial tile).  No candidate is faster than W (2NK bytes) streams through it: 3.1 .. 4.1 TB/s
+        more (~5 us per partial tile).  No candidate is faster than W (2NK bytes) streams through it: 3.1 .. 4.3 TB/s
         by tile, measured with 64 rows against a 50280 x 2560 W."""
         cdiv = lambda a, b: -(-a // b)
         cus = self.arch.num_sm
@@ -54,7 +54,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
 
         tiles = lambda bm, bn: cdiv(m_hi, bm) * cdiv(N, bn)
         w_mb = 2.0 * float(N) * float(K) * 1e-6
-        floored = lambda us, tbs: us if us > w_mb / tbs else w_mb / tbs     # W streams at 3.1 .. 4.1 TB/s, by tile
+        floored = lambda us, tbs: us if us > w_mb / tbs else w_mb / tbs     # W streams at 3.1 .. 4.3 TB/s, by tile
         cands = [(floored(rounds(tiles(256, 256), cus) * 1.80 * ktiles, 3.5), (256, 256, 2, 1)),
                  (floored(rounds(tiles(256, 128), cus) * 1.045 * ktiles, 3.5), (256, 128, 3, 1)),
                  (floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1))]
@@ -67,7 +67,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 cands.append((floored((0.8 + 0.2 * t128 / cus if t128 <= cus else rounds(t128, cus)) * 0.665 * steps
                                       + (4.0 * split if split > 1 else 0.0), 4.1), (128, 128, 4, split)))
             cands.append((floored((1.0 if t64 <= cus else 0.82 * -(-int(t64) // cus)) * 0.33 * steps
-                                  + ((1.0 if t64 <= cus else 2.0) * split if split > 1 else 0.0), 3.9),
+                                  + ((1.0 if t64 <= cus else 2.5) * split if split > 1 else 0.0), 4.3),
                           (64, 64, 4, split)))
             t256128 = tiles(256, 128) * split
             if split > 1 and steps >= 32 and t256128 <= cus:
@@ -88,6 +88,9 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         if m_hi > 32:
             return False
         us = N * K * 2.0 / 3.5e6 * (0.9 if m_hi <= 8 else 0.95 if m_hi <= 16 else 1.35)
+        wgs = -(-N // 16)               # one workgroup per 16 rows of W: fewer than one per CU leave CUs idle
+        if wgs < self.arch.num_sm:
+            us *= self.arch.num_sm / wgs
         return us <= self._model_us
 
     def emit_config(self, range_tuple: Tuple[Range, ...], topk: int = 20) -> List[MFMAConfig]:
