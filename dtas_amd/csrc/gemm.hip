@@ -56,6 +56,11 @@ namespace dtas {
 namespace {
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
+// The same vectors at the alignment of their elements: rows of a dynamic length start anywhere (the scores'
+// m, the residuals' N), the hardware runs in its unaligned access mode and the compiler emits one access for
+// these types as it does for the aligned ones.
+typedef f32x4v __attribute__((aligned(4))) f32x4v_a4;
+typedef f16x4 __attribute__((aligned(2))) f16x4_a2;
 typedef float f32x2v __attribute__((ext_vector_type(2)));
 
 constexpr int kBK = 64;             // k extent of a tile: 128 bytes of fp16
@@ -91,6 +96,7 @@ struct GemmEpilogue {
   unsigned batches;
   unsigned tiles_pinned;  // batched launches: an XCD keeps its tiles and walks the problems (see the kernel)
   const half_t* wscale;   // 8-bit W: the fp16 scales [N][K/32]
+  int64_t lda;            // k-major W only (P.V): row stride of A in elements when its rows are padded; 0 = K
 };
 
 // Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):
@@ -227,8 +233,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // the (row, chunk) that lds_chunk_offset places there; the block index of wavefront w's i-th
   // load is i*NW + w, whose parity is w's (NW is even).
   const int64_t rows_a = M - m0 < BM ? M - m0 : BM, rows_w = N - n0 < BN ? N - n0 : BN;
-  const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(A + m0 * K, static_cast<unsigned>(rows_a) * row_bytes);
+  const int64_t lda = WT && ep.lda ? ep.lda : K;  // (with a row-major W both operands' rows are K long)
+  const unsigned row_bytes = static_cast<unsigned>(lda) * 2u;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(A + m0 * lda, static_cast<unsigned>(rows_a) * row_bytes);
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
   const unsigned r_in = 2u * (l >> 4) + (((l >> 3) & 1u) ^ (wv & 1u));  // row inside the 8-row block
   const unsigned c_in = (l & 7u) ^ r_in;                                // chunk of that row
@@ -861,11 +868,11 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const int64_t col = n0 + wn * WTN + slot * 4;
   const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
   const bool use_r1 = add2 || ep.kind == kEpiScores;
-  // 8-byte accesses to C and the residuals (16-byte to an fp32 C) where extents and pointers allow
-  const bool vec_store = (N % 4 == 0) && col + 3 < N &&
-                         (reinterpret_cast<uintptr_t>(C) & (ep.out_f32 ? 15u : 7u)) == 0 &&
-                         (!use_r1 || (reinterpret_cast<uintptr_t>(ep.res1) & 7u) == 0) &&
-                         (!add2 || (reinterpret_cast<uintptr_t>(ep.res2) & 7u) == 0);
+  // 8-byte accesses to C and the residuals (16-byte to an fp32 C) for every slot that lies inside the row, at
+  // whatever alignment the row has
+  const bool vec_store = col + 3 < N;
+  (void)use_r1;
+  (void)add2;
   float bv[4] = {0.f, 0.f, 0.f, 0.f};
   if (ep.bias) {
 #pragma unroll
@@ -895,8 +902,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           if (row >= M) continue;
           const int64_t at = row * N + col;
           if (vec_store) {
-            r1v[u] = *reinterpret_cast<const f16x4*>(ep.res1 + at);
-            if (kAdd2) r2v[u] = *reinterpret_cast<const f16x4*>(ep.res2 + at);
+            r1v[u] = *reinterpret_cast<const f16x4_a2*>(ep.res1 + at);
+            if (kAdd2) r2v[u] = *reinterpret_cast<const f16x4_a2*>(ep.res2 + at);
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -925,8 +932,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           if (vec_store) {
             const f32x4v wide = {static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]),
                                  static_cast<float>(hv[3])};
-            if (KIND == kEpiScores) __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));  // 4*heads*n*m bytes: streamed
-            else *reinterpret_cast<f32x4v*>(dst) = wide;
+            if (KIND == kEpiScores && N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 63u) == 0)
+              __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));  // 4*heads*n*m bytes: streamed (rows of whole sectors)
+            else
+              *reinterpret_cast<f32x4v_a4*>(dst) = wide;
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -935,7 +944,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         } else {
           half_t* dst = static_cast<half_t*>(C) + at;
           if (vec_store) {
-            *reinterpret_cast<f16x4*>(dst) = hv;
+            *reinterpret_cast<f16x4_a2*>(dst) = hv;
           } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -989,7 +998,8 @@ __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restri
   constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots, kPasses = WTM / kRowsPerPass;
   const unsigned slot = l % kSlots, rsub = l / kSlots;
   char* region = lds + wv * (WTM * kRowB);
-  const bool ptr_ok = (m % 4 == 0) && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
+  const bool ptr_ok = true;  // rows of any length: vector accesses at the rows' own alignment
+  const bool stream_out = m % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 63u) == 0;  // (then every access is 16-byte aligned)
 
   const unsigned per_batch = tiles_m * tiles_n, total = per_batch * heads;
   for (unsigned tix = blockIdx.x; tix < total; tix += gridDim.x) {
@@ -1030,7 +1040,7 @@ __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restri
       mk[p] = zero;
       if (row >= n) continue;
       if (vec_ok) {
-        mk[p] = *reinterpret_cast<const f16x4*>(mask + row * m + col);
+        mk[p] = *reinterpret_cast<const f16x4_a2*>(mask + row * m + col);
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -1093,7 +1103,10 @@ __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restri
       float* dst = out + (static_cast<int64_t>(batch) * n + row) * m + col;
       if (vec_ok) {
         const f32x4v wide = {static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]), static_cast<float>(hv[3])};
-        __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));  // 4*heads*n*m bytes: streamed
+        // 4*heads*n*m bytes: streamed -- unless a row is not a whole number of 64-byte sectors: then the tiles
+        // left and right of a column boundary each write part of a sector, and only the cache can join the parts
+        if (stream_out) __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));
+        else *reinterpret_cast<f32x4v_a4*>(dst) = wide;
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -1292,6 +1305,32 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(const half_t* __restrict
   }
 }
 
+// P.V with a key count that is not a multiple of 8 (or a P that is not 16-byte aligned): the rows of P are
+// copied once into rows of m_pad = 8 * slots elements, zero-filled, which the direct-to-LDS loads can fetch.
+// Whole 8-element pieces are read with one access at the row's alignment, the piece across the end of a row
+// element by element.
+typedef u32x4 __attribute__((aligned(2))) u32x4_a2;
+__global__ void __launch_bounds__(256) pad_rows_kernel(const half_t* __restrict__ P, u32x4* __restrict__ out, int64_t rows,
+                                                       int64_t m, int64_t slots) {
+  const int64_t total = rows * slots;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t row = t / slots, at = (t % slots) * 8, left = m - at;
+    const half_t* p = P + row * m + at;
+    u32x4 v;
+    if (left >= 8) {
+      v = *reinterpret_cast<const u32x4_a2*>(p);
+    } else {
+      unsigned short h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) h[e] = e < left ? reinterpret_cast<const unsigned short*>(p)[e] : 0u;
+      v = u32x4{h[0] | (static_cast<unsigned>(h[1]) << 16), h[2] | (static_cast<unsigned>(h[3]) << 16),
+                h[4] | (static_cast<unsigned>(h[5]) << 16), h[6] | (static_cast<unsigned>(h[7]) << 16)};
+    }
+    out[t] = v;
+  }
+}
+
 // Any K and alignment: one thread per element of C.  blockIdx.y = problem of a batched launch;
 // w_kmajor: W is [K][N] instead of [N][K]; ep.wscale set: W is 8-bit with group scales.
 __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
@@ -1430,7 +1469,8 @@ int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsign
   return 0;
 }
 
-// fp16 copy of an 8-bit weight matrix for dtas_gemm_q8_f16_fused's two-pass route: one buffer per device,
+// A rewritten operand: the fp16 copy of an 8-bit weight matrix (dtas_gemm_q8_f16_fused's two-pass route) or the
+// padded copy of P (dtas_attn_pv_f16 with a key count that is not a multiple of 8).  One buffer per device,
 // allocated on first use and grown on demand like the split-K workspace, and like it shared by the launches
 // that use it (one stream).
 struct DequantWorkspace {
@@ -1441,19 +1481,19 @@ DequantWorkspace g_dequant_ws[kMaxDevices];
 
 int dequant_workspace(size_t bytes, void** out) {
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("gemm_q8: cannot identify the current device");
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("operand buffer: cannot identify the current device");
   std::lock_guard<std::mutex> lock(g_split_ws_mutex);
   DequantWorkspace& w = g_dequant_ws[dev];
   if (bytes > w.bytes) {
-    if (bytes > kMaxSplitWsBytes) return fail("gemm_q8: an fp16 copy of W needs %zu bytes (limit %zu)", bytes, kMaxSplitWsBytes);
+    if (bytes > kMaxSplitWsBytes) return fail("operand buffer: a rewritten operand needs %zu bytes (limit %zu)", bytes, kMaxSplitWsBytes);
     // kernels of earlier launches may still use the old buffer: hipFree waits for the device
-    if (w.buf && hipFree(w.buf) != hipSuccess) return fail("gemm_q8: hipFree of the dequantised-weight buffer failed");
+    if (w.buf && hipFree(w.buf) != hipSuccess) return fail("operand buffer: hipFree failed");
     w.buf = nullptr;
     w.bytes = 0;
     const size_t want = bytes < (size_t{64} << 20) ? (size_t{64} << 20) : bytes;
     if (hipMalloc(&w.buf, want) != hipSuccess) {
       (void)hipGetLastError();
-      return fail("gemm_q8: cannot allocate %zu bytes for the dequantised weights", want);
+      return fail("operand buffer: cannot allocate %zu bytes", want);
     }
     w.bytes = want;
   }
@@ -1731,7 +1771,7 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   if (overlaps(out, heads * n * d * 2, P, heads * n * m * 2) || overlaps(out, heads * n * d * 2, V, heads * m * d * 2))
     return fail("attn_pv: output overlaps an input");
   const bool v_vec = d % 8 == 0 && aligned(V, 16);                  // 16-byte pieces of V's rows
-  const bool p_vec = m % 8 == 0 && aligned(P, 16) && aligned(out, 8);  // 16-byte pieces of P's rows
+  const bool p_vec = m % 8 == 0 && aligned(P, 16);                  // 16-byte pieces of P's rows
   dtas_config cfg;
   if (user) {
     cfg = *user;
@@ -1775,13 +1815,33 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     }
   }
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_SKINNY && !v_vec) cfg.vec = 1;
-  if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && (!(v_vec && p_vec) || m == 0)) cfg.vec = 1;  // m == 0: zeros
+  if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && (!v_vec || m == 0)) cfg.vec = 1;  // m == 0: zeros
   hipStream_t s = static_cast<hipStream_t>(stream);
   const half_t* a = static_cast<const half_t*>(P);
   const half_t* w = static_cast<const half_t*>(V);
   half_t* c = static_cast<half_t*>(out);
   const int b = static_cast<int>(heads);
   GemmEpilogue ep = {nullptr, nullptr, nullptr, DTAS_EPI_BIAS, 0, 1.f, n * m, m * d, n * d, 0};
+  if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && !p_vec) {
+    // rows of P that the 16-byte loads cannot fetch where they lie: a padded copy in the library's buffer
+    const int64_t m_pad = (m + 7) / 8 * 8;
+    const size_t bytes = static_cast<size_t>(heads) * n * m_pad * 2;
+    void* buf = nullptr;
+    if (!aligned(P, 2) || bytes > kMaxSplitWsBytes) {
+      cfg.vec = 1;  // (the element-access kernel: correct, slow)
+    } else {
+      if (dequant_workspace(bytes, &buf) != 0) return -1;
+      const int64_t items = heads * n * (m_pad / 8);
+      int64_t grid = ceil_div(items, 256);
+      grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+      hipLaunchKernelGGL(pad_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, a, static_cast<u32x4*>(buf), heads * n, m,
+                         m_pad / 8);
+      if (check_launch("attn_pv") != 0) return -1;
+      a = static_cast<const half_t*>(buf);
+      ep.stride_a = n * m_pad;
+      ep.lda = m_pad;
+    }
+  }
   if (cfg.vec == 1) {
     int64_t grid = ceil_div(n * d, 256);
     grid = grid > 4096 ? 4096 : grid;

@@ -82,6 +82,56 @@ __device__ __forceinline__ void store_half_vec(half_t* dst, const float (&v)[VEC
   }
 }
 
+// ---- rows whose length is not a multiple of the vector width, or whose buffers are only element-aligned
+// (softmax over a dynamic row length: (1,32,n,m) with any m).  Vector slots that lie wholly inside a row are
+// moved with the same 16-byte accesses at the row's own alignment (2 or 4 bytes: the hardware runs in its
+// unaligned access mode, and the compiler emits one dwordx4 for these under-aligned types); the one slot that
+// straddles the end of a row is moved element by element, its missing elements set to -inf, which max and
+// exp-sum ignore.
+typedef u32x4 __attribute__((aligned(2))) u32x4_a2;
+typedef u32x4 __attribute__((aligned(4))) u32x4_a4;
+typedef u32x2 __attribute__((aligned(2))) u32x2_a2;
+
+template <typename In, int VEC>
+__device__ __forceinline__ u32x4 load_ragged(const In* p, int64_t left) {  // left = elements of the row from p on
+  if (left >= VEC) {
+    if (sizeof(In) == 2) return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a2*>(p));
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(p));
+  }
+  if (sizeof(In) == 2) {
+    unsigned short h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = e < left ? reinterpret_cast<const unsigned short*>(p)[e] : 0xFC00u;  // -inf
+    return u32x4{h[0] | (static_cast<unsigned>(h[1]) << 16), h[2] | (static_cast<unsigned>(h[3]) << 16),
+                 h[4] | (static_cast<unsigned>(h[5]) << 16), h[6] | (static_cast<unsigned>(h[7]) << 16)};
+  }
+  u32x4 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = e < left ? reinterpret_cast<const unsigned*>(p)[e] : 0xFF800000u;  // -inf
+  return r;
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_half_ragged(half_t* dst, const float (&v)[VEC], int64_t left) {
+  if (left >= VEC) {
+    if (VEC == 8) {
+      f16x8 h;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) h[e] = static_cast<half_t>(v[e]);
+      __builtin_nontemporal_store(__builtin_bit_cast(u32x4, h), reinterpret_cast<u32x4_a2*>(dst));
+    } else {
+      f16x4 h;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h[e] = static_cast<half_t>(v[e]);
+      __builtin_nontemporal_store(__builtin_bit_cast(u32x2, h), reinterpret_cast<u32x2_a2*>(dst));
+    }
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+    if (e < left) dst[e] = static_cast<half_t>(v[e]);
+}
+
 // N independent reductions at once: DPP inside each wavefront, then (BLOCK) one LDS slot per
 // wavefront and value, joined in wavefront order by every thread.  Consecutive calls alternate
 // between two banks of N x 16 slots (`phase` counts them), so a bank is rewritten only after a
@@ -113,7 +163,8 @@ __device__ __forceinline__ void group_reduce(float (&a)[N], float* slots, int& p
 // are in flight together, the R rows share each barrier, and the per-column parameters
 // (w, or gamma and beta) are fetched once for the R rows.
 // More than 8 vectors per lane need more registers than a 1024-thread workgroup leaves each lane.
-template <int OP, int ITERS, bool BLOCK, int R>
+// RAGGED (softmax): cols is any length and the buffers are element-aligned (see load_ragged).
+template <int OP, int ITERS, bool BLOCK, int R, bool RAGGED = false>
 __global__ void __launch_bounds__(ITERS * R > 8 ? 512 : 1024) row_reg_kernel(
     const void* __restrict__ xin, const void* __restrict__ p1, const void* __restrict__ p2, void* __restrict__ outp,
     int64_t rows, int64_t cols, float eps) {
@@ -126,7 +177,8 @@ __global__ void __launch_bounds__(ITERS * R > 8 ? 512 : 1024) row_reg_kernel(
   const int lane = BLOCK ? threadIdx.x : (threadIdx.x & 63);
   const int width = BLOCK ? blockDim.x : 64;
   const int64_t trip_rows = static_cast<int64_t>(R) * (BLOCK ? 1 : (blockDim.x >> 6));
-  const int64_t nvec = cols / VEC;
+  static_assert(!RAGGED || OP == kSoftmaxF32 || OP == kSoftmaxF16, "ragged rows: softmax only");
+  const int64_t nvec = RAGGED ? (cols + VEC - 1) / VEC : cols / VEC;
   const float inv_cols = 1.0f / static_cast<float>(cols);
   half_t* out = static_cast<half_t*>(outp);
   bool has[ITERS];  // which of this lane's vector slots lie inside the row
@@ -163,15 +215,22 @@ __global__ void __launch_bounds__(ITERS * R > 8 ? 512 : 1024) row_reg_kernel(
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       live[r] = base + r < rows;
-      const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const In*>(xin) + (base + r) * cols);
+      const In* row_in = static_cast<const In*>(xin) + (base + r) * cols;
+      const u32x4* src = reinterpret_cast<const u32x4*>(row_in);
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
         v[r][it].raw = u32x4{0u, 0u, 0u, 0u};
-        if (live[r] && has[it]) v[r][it].raw = load_stream(src + lane + it * width);
+        if (live[r] && has[it]) {
+          const int64_t at = (lane + static_cast<int64_t>(it) * width) * VEC;
+          if (RAGGED) v[r][it].raw = load_ragged<In, VEC>(row_in + at, cols - at);
+          else v[r][it].raw = load_stream(src + lane + it * width);
+        }
       }
     }
     auto store_row = [&](int r, int it, const float (&res)[VEC]) {
-      store_half_vec<VEC>(out + (base + r) * cols + (lane + static_cast<int64_t>(it) * width) * VEC, res);
+      const int64_t at = (lane + static_cast<int64_t>(it) * width) * VEC;
+      if (RAGGED) store_half_ragged<VEC>(out + (base + r) * cols + at, res, cols - at);
+      else store_half_vec<VEC>(out + (base + r) * cols + at, res);
     };
 
     if (OP == kRms) {
@@ -341,12 +400,12 @@ __global__ void __launch_bounds__(1024) row_stream_kernel(const void* __restrict
 }
 
 // instantiated (vectors per lane, rows per trip) pairs: ITERS * R <= 16
-template <int OP, bool BLOCK>
+template <int OP, bool BLOCK, bool RAGGED = false>
 int launch_reg(int iters, int rpt, dim3 grid, dim3 block, hipStream_t s, const void* x, const void* p1,
                const void* p2, void* out, int64_t rows, int64_t cols, float eps) {
-#define DTAS_ROW_CASE(I, R)                                                                                      \
-  case I * 8 + R:                                                                                                \
-    hipLaunchKernelGGL((row_reg_kernel<OP, I, BLOCK, R>), grid, block, 0, s, x, p1, p2, out, rows, cols, eps);   \
+#define DTAS_ROW_CASE(I, R)                                                                                              \
+  case I * 8 + R:                                                                                                        \
+    hipLaunchKernelGGL((row_reg_kernel<OP, I, BLOCK, R, RAGGED>), grid, block, 0, s, x, p1, p2, out, rows, cols, eps);   \
     break;
   switch (iters * 8 + rpt) {
     DTAS_ROW_CASE(1, 1) DTAS_ROW_CASE(1, 2) DTAS_ROW_CASE(1, 4)
@@ -394,13 +453,19 @@ int rows_per_trip(const dtas_config& cfg) { return cfg.unroll <= 1 ? 1 : cfg.unr
 
 template <int OP>
 int launch_rows(const dtas_config& cfg, const int64_t la[7], hipStream_t s, const void* x, const void* p1,
-                const void* p2, void* out, int64_t rows, int64_t cols, float eps) {
+                const void* p2, void* out, int64_t rows, int64_t cols, float eps, bool ragged) {
   const dim3 grid(static_cast<unsigned>(la[0])), block(static_cast<unsigned>(la[3]));
   if (cfg.variant == DTAS_RED_STREAM_ROW) {
     hipLaunchKernelGGL((row_stream_kernel<OP>), grid, block, 0, s, x, p1, p2, out, rows, cols, eps);
     return check_launch("reduction");
   }
   const int iters = static_cast<int>(la[5]), rpt = rows_per_trip(cfg);
+  if constexpr (OP == kSoftmaxF32 || OP == kSoftmaxF16) {
+    if (ragged) {
+      if (cfg.variant == DTAS_RED_WAVE_ROW) return launch_reg<OP, false, true>(iters, rpt, grid, block, s, x, p1, p2, out, rows, cols, eps);
+      return launch_reg<OP, true, true>(iters, rpt, grid, block, s, x, p1, p2, out, rows, cols, eps);
+    }
+  }
   if (cfg.variant == DTAS_RED_WAVE_ROW) return launch_reg<OP, false>(iters, rpt, grid, block, s, x, p1, p2, out, rows, cols, eps);
   return launch_reg<OP, true>(iters, rpt, grid, block, s, x, p1, p2, out, rows, cols, eps);
 }
@@ -423,9 +488,11 @@ int run_reduction(int op, const void* x, const void* p1, const void* p2, void* o
   // dynamic extent: the row count for the norms, the row length for softmax
   const bool softmax = r.kind == kSoftmaxF32 || r.kind == kSoftmaxF16;
   dtas_config cfg = user ? *user : builtin_config(op, softmax ? cols : rows, softmax ? rows : cols, softmax ? cols : 0).cfg;
-  // 128-bit row accesses need cols % vec == 0 and 16-byte aligned buffers; other rows take the
-  // element-access kernel (a bucket's config must serve every n in the bucket)
-  if (cfg.variant != DTAS_RED_STREAM_ROW && !vec_ok) {
+  // 128-bit row accesses at 16-byte alignment need cols % vec == 0 and aligned buffers.  Softmax rows of any
+  // other length (the row length is its dynamic extent) keep the register kernels, with accesses at the rows'
+  // own alignment; the norms take the element-access kernel (a bucket's config must serve every n in the bucket)
+  const bool ragged = softmax && !vec_ok && aligned(x, r.in_bytes) && aligned(out, 2);
+  if (cfg.variant != DTAS_RED_STREAM_ROW && !vec_ok && !ragged) {
     cfg.variant = DTAS_RED_STREAM_ROW;
     if (!user) cfg.block = cols >= 4096 ? 1024 : cols >= 1024 ? 512 : 256;
     cfg.vec = 1;
@@ -434,10 +501,10 @@ int run_reduction(int op, const void* x, const void* p1, const void* p2, void* o
   if (describe_reduction(op, rows, cols, cfg, la) != 0) return -1;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (r.kind) {
-    case kRms: return launch_rows<kRms>(cfg, la, s, x, p1, p2, out, rows, cols, eps);
-    case kLayerNorm: return launch_rows<kLayerNorm>(cfg, la, s, x, p1, p2, out, rows, cols, eps);
-    case kSoftmaxF32: return launch_rows<kSoftmaxF32>(cfg, la, s, x, p1, p2, out, rows, cols, eps);
-    case kSoftmaxF16: return launch_rows<kSoftmaxF16>(cfg, la, s, x, p1, p2, out, rows, cols, eps);
+    case kRms: return launch_rows<kRms>(cfg, la, s, x, p1, p2, out, rows, cols, eps, false);
+    case kLayerNorm: return launch_rows<kLayerNorm>(cfg, la, s, x, p1, p2, out, rows, cols, eps, false);
+    case kSoftmaxF32: return launch_rows<kSoftmaxF32>(cfg, la, s, x, p1, p2, out, rows, cols, eps, ragged);
+    case kSoftmaxF16: return launch_rows<kSoftmaxF16>(cfg, la, s, x, p1, p2, out, rows, cols, eps, ragged);
   }
   return fail("reduction: unknown op %d", op);
 }

@@ -179,6 +179,37 @@ def test_pv_selector_rows_are_exact_and_edge_cases(oracle):
     assert _lib.lib().dtas_attn_pv_f16(None, None, None, 32, 0, 16, 80, None, None) == 0
 
 
+@pytest.mark.parametrize("n,m", [(13, 1025), (64, 77), (130, 1027), (300, 1028), (257, 513), (1024, 1032), (515, 7)])
+def test_scores_and_pv_with_key_counts_off_the_vector_width(oracle, n, m):
+    # rows of m floats / halves start anywhere: the scores keep their vector stores (at the rows' alignment), P.V
+    # pads the rows of P into the library's buffer and keeps the MFMA kernel
+    heads, d = 4, 80
+    q, k, mask = _inputs(heads, n, m, d, n + m)
+    out = Guarded((heads, n, m), torch.float32)
+    ops.attn_scores(dev(q), dev(k), dev(mask), out.t, SCALE)
+    _check(out.check(), q, k, mask, oracle)
+    p, v = _pv_inputs(heads, n, m, d, n * m)
+    o = Guarded((heads, n, d), torch.float16)
+    ops.attn_pv(dev(p), dev(v), o.t)
+    _check_pv(o.check(), p, v, oracle)
+    # an explicit tile on the same shapes, and a split over the keys
+    for c in (cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=2, tile=[64, 128, 64]),
+              cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=3, tile=[128, 128, 64], split_k=2 if m >= 256 else 1)):
+        o = Guarded((heads, n, d), torch.float16)
+        ops.attn_pv(dev(p), dev(v), o.t, c)
+        _check_pv(o.check(), p, v, oracle)
+
+
+def test_pv_with_a_p_that_is_not_16_byte_aligned(oracle):
+    heads, n, m, d = 2, 70, 136, 80
+    p, v = _pv_inputs(heads, n, m, d, 5)
+    buf = torch.empty(heads * n * m + 1, dtype=torch.float16, device="cuda")
+    buf[1:] = dev(p).reshape(-1)
+    o = Guarded((heads, n, d), torch.float16)
+    ops.attn_pv(buf[1:].view(heads, n, m), dev(v), o.t)
+    _check_pv(o.check(), p, v, oracle)
+
+
 def test_pv_errors():
     p, v = _pv_inputs(2, 16, 16, 80, 1)
     out = torch.empty(2, 16, 80, dtype=torch.float16, device="cuda")

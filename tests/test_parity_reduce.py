@@ -167,8 +167,8 @@ def test_softmax_special_rows(oracle):
 
 
 def test_register_variants_step_down_on_ragged_rows(oracle):
-    # a bucket's config must serve every n in it: rows that are not a multiple of the vector width
-    # take the element-access kernel even when the config names a register variant
+    # a bucket's config must serve every n in it: norm rows that are not a multiple of the vector width take
+    # the element-access kernel even when the config names a register variant (softmax rows stay in it)
     rng = np.random.default_rng(21)
     x = rng.standard_normal((4, 100)).astype(np.float16)
     w = rng.uniform(0.5, 1.5, 100).astype(np.float16)
@@ -180,6 +180,60 @@ def test_register_variants_step_down_on_ragged_rows(oracle):
     out = Guarded(s.shape, torch.float16)
     ops.softmax(dev(s), out.t, cfg=cfg(variant=_lib.RED_WAVE_ROW, block=64, vec=8))
     _check(out.check(), oracle.c.softmax(s), oracle.np64.softmax(s))
+
+
+@pytest.mark.parametrize("variant,block", [v for v in RED_VARIANTS if v[0] != _lib.RED_STREAM_ROW])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("rows,cols", [(19, 2047), (19, 2049), (33, 1026), (7, 9), (64, 33), (5, 3), (40, 1)])
+def test_softmax_rows_of_any_length_keep_the_register_kernels(oracle, variant, block, dtype, rows, cols):
+    # the row length is softmax's dynamic extent: lengths that are not a multiple of the vector width, and rows
+    # that start at any element, run in the register kernels with accesses at the rows' own alignment
+    if variant == _lib.RED_WAVE_ROW and cols > 64 * 16 * (8 if dtype == np.float16 else 4):
+        pytest.skip("row does not fit one wavefront's registers")
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2).astype(dtype)
+    out = Guarded(x.shape, torch.float16)
+    ops.softmax(dev(x), out.t, cfg=cfg(variant=variant, block=block, vec=8 if dtype == np.float16 else 4))
+    _check(out.check(), oracle.c.softmax(x), oracle.np64.softmax(x))
+
+
+@pytest.mark.parametrize("n", [9, 33, 257, 1025, 1026, 2047])
+def test_softmax_builtin_on_unaligned_lengths_and_buffers(oracle, n):
+    rng = np.random.default_rng(n)
+    for dtype, tdt in ((np.float16, torch.float16), (np.float32, torch.float32)):
+        x = (rng.standard_normal((32 * min(n, 64), n)) * 2).astype(dtype)
+        out = Guarded(x.shape, torch.float16)
+        ops.softmax(dev(x), out.t)
+        _check(out.check(), oracle.c.softmax(x, threads=8), oracle.np64.softmax(x))
+        # aligned length, buffers that start one element off a 16-byte boundary
+        y = (rng.standard_normal((16, 1024)) * 2).astype(dtype)
+        src = torch.empty(16 * 1024 + 1, dtype=tdt, device="cuda")
+        src[1:] = dev(y).reshape(-1)
+        dst = torch.full((16 * 1024 + 2,), 3.0, dtype=torch.float16, device="cuda")
+        ops.softmax(src[1:].view(16, 1024), dst[1:-1].view(16, 1024))
+        torch.cuda.synchronize()
+        assert dst[0] == 3.0 and dst[-1] == 3.0
+        _check(dst[1:-1].view(16, 1024).cpu().numpy(), oracle.c.softmax(y), oracle.np64.softmax(y))
+
+
+def test_softmax_ragged_special_rows(oracle):
+    # the slot across the end of a row is filled with -inf: constant rows at the fp16 minimum, a row whose
+    # maximum sits in the last, partial slot, and -inf entries all come out as in the oracle
+    x = np.zeros((5, 67), np.float16)
+    x[0] = -65504.0                  # the attention mask's value in every position -> 1/67
+    x[1, 66] = 30000                 # the dominant entry is the row's last element
+    x[2] = np.linspace(-60000, 60000, 67).astype(np.float16)
+    x[3, :] = -np.inf
+    x[3, 64] = 0
+    x[4] = 5.0
+    for variant, block in ((_lib.RED_WAVE_ROW, 64), (_lib.RED_BLOCK_ROW, 64), (_lib.RED_BLOCK_ROW, 256)):
+        out = Guarded(x.shape, torch.float16)
+        ops.softmax(dev(x), out.t, cfg=cfg(variant=variant, block=block, vec=8))
+        got = out.check()
+        assert (got[0] == np.float16(1 / 67)).all() and (got[4] == np.float16(1 / 67)).all()
+        assert got[1, 66] == 1 and got[1].sum() == 1
+        assert got[3, 64] == 1 and got[3].sum() == 1
+        assert np.abs(got.astype(np.float64) - oracle.c.softmax(x).astype(np.float64)).max() < 2e-3
 
 
 def test_reduction_errors():
