@@ -25,11 +25,14 @@
  *    library allocates on first use and grows on demand (32 MiB at first, at most 1 GiB; growing
  *    waits for the device).  Launches that use it share it: enqueue them on one stream, or pass
  *    a cfg with split_k = 1 on the others.  dtas_gemm_q8_f16_fused keeps a second buffer of that kind
- *    (an fp16 copy of the weights it was given) under the same rules;
+ *    (an fp16 copy of the weights it was given) under the same rules, and dtas_attn_pv_f16 uses that
+ *    buffer for a padded copy of P when m is not a multiple of 8;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
  *    reference's call_table holds); NULL = use the library's built-in bucket table; either way a
  *    128-bit variant steps down to its element-access kernel for extents or pointers that do not
- *    allow 128-bit accesses (a bucket's row must serve every n and buffer that falls in it);
+ *    allow 128-bit accesses (a bucket's row must serve every n and buffer that falls in it).  The
+ *    dynamic row lengths are exempt: softmax rows and attention's key count m may be any number and
+ *    keep the vector kernels (accesses at the rows' own alignment);
  *  - returns 0 on success, -1 on error (the reference's host functions do the same,
  *    host.cc:75-83,133-143); dtas_last_error() gives the thread-local message;
  *  - n == 0 (an empty dynamic extent) is a no-op that returns 0; negative extents, NULL
@@ -224,8 +227,9 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
  * fp32 accumulation, one rounding to fp16.  cfg, when given: a DTAS_GEMM_MFMA row for the per-head
  * (n, d, m) problem with tile {64|128, 64|128, 64} and two stages, or {128|256, 128, 64} and three (split_k > 1:
  * the workgroups of a (head, tile) split m and meet in the split-K workspace), or a DTAS_GEMM_SKINNY row
- * {block 256, tile {1|2|4|8, 8}} for the kernel that serves a handful of rows (decoding).  m % 8 != 0,
- * d % 8 != 0 or odd pointers fall back to the element-access kernel; m == 0 writes zeros. */
+ * {block 256, tile {1|2|4|8, 8}} for the kernel that serves a handful of rows (decoding).  With m % 8 != 0
+ * or a P off a 16-byte boundary the rows of P are first copied, padded, into the library's operand buffer;
+ * d % 8 != 0 or a V off 16 bytes fall back to the element-access kernel; m == 0 writes zeros. */
 int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int64_t n, int64_t m,
                      int64_t d, const dtas_config* cfg, void* stream);
 
