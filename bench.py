@@ -339,6 +339,9 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("attn_scores_f16_f32", n, None, max(10, steps // 2), max(2, warmup // 2)))
         rows.append(measure("attn_pv_f16", n, None, max(10, steps // 2), max(2, warmup // 2)))
     rows.append(measure("attn_pv_f16", 1, (1, 2048), steps, warmup))      # matmul10: decoding against 2048 keys
+    # a sequence length off every vector width: rows that start at any element
+    for op in ("softmax_f16", "attn_scores_f16_f32", "attn_pv_f16"):
+        rows.append(measure(op, 1025, None, max(10, steps // 2), max(2, warmup // 2)))
     return rows
 
 
