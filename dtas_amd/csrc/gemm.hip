@@ -1822,24 +1822,17 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   half_t* c = static_cast<half_t*>(out);
   const int b = static_cast<int>(heads);
   GemmEpilogue ep = {nullptr, nullptr, nullptr, DTAS_EPI_BIAS, 0, 1.f, n * m, m * d, n * d, 0};
+  // rows of P that the 16-byte loads cannot fetch where they lie: a padded copy in the library's buffer, as many
+  // heads at a time as the buffer may hold
+  const int64_t m_pad = (m + 7) / 8 * 8;
+  int64_t pad_heads = 0;  // heads per padded launch; 0 = P is used where it lies
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && !p_vec) {
-    // rows of P that the 16-byte loads cannot fetch where they lie: a padded copy in the library's buffer
-    const int64_t m_pad = (m + 7) / 8 * 8;
-    const size_t bytes = static_cast<size_t>(heads) * n * m_pad * 2;
-    void* buf = nullptr;
-    if (!aligned(P, 2) || bytes > kMaxSplitWsBytes) {
+    const int64_t per_head = n * m_pad * 2;
+    pad_heads = static_cast<int64_t>(kMaxSplitWsBytes) / per_head;
+    if (pad_heads > heads) pad_heads = heads;
+    if (!aligned(P, 2) || pad_heads == 0) {
       cfg.vec = 1;  // (the element-access kernel: correct, slow)
-    } else {
-      if (dequant_workspace(bytes, &buf) != 0) return -1;
-      const int64_t items = heads * n * (m_pad / 8);
-      int64_t grid = ceil_div(items, 256);
-      grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
-      hipLaunchKernelGGL(pad_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, a, static_cast<u32x4*>(buf), heads * n, m,
-                         m_pad / 8);
-      if (check_launch("attn_pv") != 0) return -1;
-      a = static_cast<const half_t*>(buf);
-      ep.stride_a = n * m_pad;
-      ep.lda = m_pad;
+      pad_heads = 0;
     }
   }
   if (cfg.vec == 1) {
@@ -1873,14 +1866,33 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   if (describe_gemm(n, d, m, cfg, la) != 0) return -1;
   const int bm = cfg.tile[0], bn = cfg.tile[1];
   const bool three = cfg.unroll == 3;
-  if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, sk, b);
-  if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m, sk, b);
-  if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
-  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
-  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
-  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
-  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m, sk, b);
-  return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
+  // `hb` heads from P `pa` (row stride in ep), V `pw`, into `po`
+  auto launch = [&](const half_t* pa, const half_t* pw, void* po, int hb) -> int {
+    if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
+    if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
+    if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
+    if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
+    if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
+    if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
+    if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
+    return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
+  };
+  if (pad_heads == 0) return launch(a, w, out, b);
+  void* buf = nullptr;
+  if (dequant_workspace(static_cast<size_t>(pad_heads) * n * m_pad * 2, &buf) != 0) return -1;
+  ep.stride_a = n * m_pad;
+  ep.lda = m_pad;
+  for (int64_t h0 = 0; h0 < heads; h0 += pad_heads) {
+    const int64_t hb = heads - h0 < pad_heads ? heads - h0 : pad_heads;
+    const int64_t items = hb * n * (m_pad / 8);
+    int64_t grid = ceil_div(items, 256);
+    grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+    hipLaunchKernelGGL(pad_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, a + h0 * n * m, static_cast<u32x4*>(buf), hb * n, m,
+                       m_pad / 8);
+    if (check_launch("attn_pv") != 0) return -1;
+    if (launch(static_cast<const half_t*>(buf), w + h0 * m * d, c + h0 * n * d, static_cast<int>(hb)) != 0) return -1;
+  }
+  return 0;
 }
 
 extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias, const void* res1,
