@@ -1473,17 +1473,17 @@ int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsign
 // padded copy of P (dtas_attn_pv_f16 with a key count that is not a multiple of 8).  One buffer per device,
 // allocated on first use and grown on demand like the split-K workspace, and like it shared by the launches
 // that use it (one stream).
-struct DequantWorkspace {
+struct OperandWorkspace {
   void* buf = nullptr;
   size_t bytes = 0;
 };
-DequantWorkspace g_dequant_ws[kMaxDevices];
+OperandWorkspace g_operand_ws[kMaxDevices];
 
-int dequant_workspace(size_t bytes, void** out) {
+int operand_workspace(size_t bytes, void** out) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("operand buffer: cannot identify the current device");
   std::lock_guard<std::mutex> lock(g_split_ws_mutex);
-  DequantWorkspace& w = g_dequant_ws[dev];
+  OperandWorkspace& w = g_operand_ws[dev];
   if (bytes > w.bytes) {
     if (bytes > kMaxSplitWsBytes) return fail("operand buffer: a rewritten operand needs %zu bytes (limit %zu)", bytes, kMaxSplitWsBytes);
     // kernels of earlier launches may still use the old buffer: hipFree waits for the device
@@ -1879,7 +1879,7 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   };
   if (pad_heads == 0) return launch(a, w, out, b);
   void* buf = nullptr;
-  if (dequant_workspace(static_cast<size_t>(pad_heads) * n * m_pad * 2, &buf) != 0) return -1;
+  if (operand_workspace(static_cast<size_t>(pad_heads) * n * m_pad * 2, &buf) != 0) return -1;
   ep.stride_a = n * m_pad;
   ep.lda = m_pad;
   for (int64_t h0 = 0; h0 < heads; h0 += pad_heads) {
@@ -1927,7 +1927,7 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
   // library-owned fp16 buffer, then the fp16 GEMM with everything its table offers.  A cfg selects the first route.
   if (!user && !(M <= 64 && K <= 4096)) {
     void* wbuf = nullptr;
-    if (dequant_workspace(static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
+    if (operand_workspace(static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
     if (dtas_decode_q8_f16(Wq, scale, wbuf, N, K, nullptr, stream) != 0) return -1;
     return dtas_gemm_f16_fused(A, wbuf, bias, res1, res2, C, M, N, K, epilogue, nullptr, stream);
   }
