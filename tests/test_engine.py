@@ -152,3 +152,32 @@ def test_reduction_emitters_lead_with_the_librarys_builtin_choice():
             got = _first_candidate(func, (Range("n", n_hi - 15, n_hi),))
             for k in ("variant", "block", "vec", "unroll"):
                 assert got[k] == want[k], (func.name, n_hi, got, want)
+
+
+def test_builtin_tables_name_a_launchable_kernel_for_every_bucket_and_shape():
+    # whatever the extents, the row the built-in table returns must be one its own launch description accepts
+    # (no GPU needed: both are host code), with a tile the kernels exist for and a split that keeps 8 k tiles
+    for N in (1, 7, 64, 100, 2560, 4096, 7680, 11008, 32000, 50280, 250000):
+        for K in (8, 64, 80, 520, 2560, 4096, 11008, 32768):
+            for M in (1, 2, 15, 16, 17, 64, 100, 256, 257, 1000, 2048, 4096, 4097, 10 ** 5):
+                info = _lib.select_bucket(_lib.OP_GEMM_F16, M, N, K)
+                c = info.config
+                again = _lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c)
+                assert list(again.launch_args) == list(info.launch_args), (M, N, K)
+                assert info.bucket_lo <= max(M, 1) and (M <= info.bucket_hi or info.index == 511), (M, N, K, info.bucket_lo, info.bucket_hi)
+                if c.variant == _lib.GEMM_MFMA:
+                    assert (c.tile[0], c.tile[1]) in {(256, 256), (256, 128), (128, 128), (128, 64), (64, 64)} and c.tile[2] == 64
+                    assert 1 <= c.split_k <= 4 and (c.split_k == 1 or -(-K // 64) // c.split_k >= 8), (M, N, K, c.split_k)
+                else:
+                    assert c.variant == _lib.GEMM_SKINNY and M <= 32 and c.tile[0] >= min(M, 32)
+            info = _lib.select_bucket(_lib.OP_GEMV_F16, 1, N, K)
+            assert list(_lib.describe_launch(_lib.OP_GEMV_F16, 1, N, K, info.config).launch_args) == list(info.launch_args)
+    for op, H in ((_lib.OP_ADD_F16, 4096), (_lib.OP_CAST_F32_F16, 2560), (_lib.OP_COPY_I8, 4096), (_lib.OP_RMS_NORM_F16, 4096),
+                  (_lib.OP_LAYER_NORM_F32_F16, 2560)):
+        for n in (1, 16, 17, 255, 256, 257, 4096, 4097, 10 ** 6):
+            info = _lib.select_bucket(op, n, H, 0)
+            assert list(_lib.describe_launch(op, n, H, 0, info.config).launch_args) == list(info.launch_args), (op, n)
+    for op in (_lib.OP_SOFTMAX_F16, _lib.OP_SOFTMAX_F32_F16):
+        for n in (1, 7, 8, 33, 256, 257, 1025, 2047, 4096, 4097, 20000):
+            info = _lib.select_bucket(op, n, 32 * n, n)
+            assert list(_lib.describe_launch(op, n, 32 * n, n, info.config).launch_args) == list(info.launch_args), (op, n)
