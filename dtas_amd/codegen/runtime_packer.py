@@ -57,7 +57,7 @@ def op_id_of(func: PrimFunc) -> int:
 
 
 # PrimFuncs the tuner does not search: the library picks their kernel and launch shape per call
-LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "take_q8", "gemv_q8", "gemv_q8_f32", "gemm_q8", "gemv_f32")
+LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "take", "take_q8", "gemv_q8", "gemv_q8_f32", "gemm_q8", "gemv_f32")
 
 
 def _concrete(shape, values: Dict[str, int]) -> Tuple[int, ...]:
@@ -140,6 +140,8 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.gemv_f32(tensors[0], tensors[1], tensors[2], abi)
     elif op == "decode_q8":                                                   # Wq, scale, W
         ops.decode_q8(tensors[0], tensors[1], tensors[2], abi)
+    elif op == "take":                                                        # A, ids, out
+        ops.take(tensors[0], tensors[1], tensors[2], abi)
     elif op == "take_q8":                                                     # Wq, scale, ids, out
         ops.take_q8(tensors[0], tensors[1], tensors[2], tensors[3], abi)
     elif op == "gemv_q8_f32":                                                 # Wq, scale, x, y

@@ -254,6 +254,29 @@ int run_eltwise(int op, const void* a, const void* b, void* out, int64_t n, int6
   return fail("elementwise: unknown op %d", op);
 }
 
+// The embedding rows (take, experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1151-1163; one row: take1,
+// :1166-1174): out[i, :] = A[ids[i], :].  16-byte pieces, piece t of the output is piece t % per_row of row
+// ids[t / per_row]; ids outside [0, V) are clipped to the nearest row (the PrimFunc reads whatever address
+// they make).  `scalar`: one element per thread, any alignment.
+__global__ void __launch_bounds__(kBlock) take_f16_kernel(const u32x4* __restrict__ A, const int* __restrict__ ids,
+                                                          u32x4* __restrict__ out, int64_t pieces, int64_t per_row, int64_t V) {
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < pieces;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    int64_t row = ids[t / per_row];
+    row = row < 0 ? 0 : row >= V ? V - 1 : row;
+    out[t] = A[row * per_row + t % per_row];
+  }
+}
+__global__ void __launch_bounds__(kBlock) take_f16_scalar_kernel(const half_t* __restrict__ A, const int* __restrict__ ids,
+                                                                 half_t* __restrict__ out, int64_t total, int64_t H, int64_t V) {
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    int64_t row = ids[t / H];
+    row = row < 0 ? 0 : row >= V ? V - 1 : row;
+    out[t] = A[row * H + t % H];
+  }
+}
+
 }  // namespace
 
 // grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
@@ -308,5 +331,32 @@ int dtas_cast_f16_f32(const void* A, void* C, int64_t n, int64_t H, const dtas_c
 }
 int dtas_cast_f32_f16(const void* A, void* C, int64_t n, int64_t H, const dtas_config* cfg, void* stream) {
   return dtas::run_eltwise(DTAS_OP_CAST_F32_F16, A, nullptr, C, n, H, cfg, stream);
+}
+int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t V, int64_t H, const dtas_config* user,
+                  void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (n < 0 || V < 0 || H < 0) return fail("take: negative extent n=%lld V=%lld H=%lld", (long long)n, (long long)V, (long long)H);
+  if (H != 0 && (n > INT64_MAX / 4 / H || V > INT64_MAX / 4 / H)) return fail("take: extents overflow");
+  if (n == 0 || H == 0) return 0;
+  if (V == 0) return fail("take: an empty table has no row to take");
+  if (!A || !ids || !out) return fail("take: NULL buffer");
+  if (overlaps(out, n * H * 2, A, V * H * 2) || overlaps(out, n * H * 2, ids, n * 4)) return fail("take: output overlaps an input");
+  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, kBlock, 8, 1, {0, 0, 0}, 1, 0};
+  if (cfg.block != kBlock) return fail("take: the kernels use %d threads, got %d", kBlock, cfg.block);
+  if (cfg.vec != 8 && cfg.vec != 1) return fail("take: vector width must be 8 (128-bit accesses) or 1, got %d", cfg.vec);
+  if (cfg.vec == 8 && !(H % 8 == 0 && aligned(A, 16) && aligned(out, 16))) cfg.vec = 1;
+  const int64_t items = cfg.vec == 8 ? n * (H / 8) : n * H;
+  int64_t grid = ceil_div(items, kBlock);
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  grid = grid > cap ? cap : grid;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (cfg.vec == 8)
+    hipLaunchKernelGGL(take_f16_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, s, static_cast<const u32x4*>(A),
+                       static_cast<const int*>(ids), static_cast<u32x4*>(out), items, H / 8, V);
+  else
+    hipLaunchKernelGGL(take_f16_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, s, static_cast<const half_t*>(A),
+                       static_cast<const int*>(ids), static_cast<half_t*>(out), items, H, V);
+  return check_launch("take");
 }
 }

@@ -250,6 +250,19 @@ def decode_q8(Wq: torch.Tensor, scale: torch.Tensor, W: torch.Tensor, cfg: Optio
     check(lib().dtas_decode_q8_f16(_p(Wq), _p(scale), _p(W), N, K, _cfg(cfg), _stream()), "dtas_decode_q8_f16")
 
 
+def take(A: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
+    """out[n,H] = A[ids[i], :], the fp16 embedding lookup: take (dolly-v2-3b-q0f16/before_dl.py:1151-1163) and, one row,
+    take1 (:1166-1174).  ids int32; values outside [0, V) are clipped to the nearest row."""
+    _dev(A, ids, out)
+    if A.dim() != 2 or A.dtype != torch.float16 or ids.dtype != torch.int32 or out.dtype != torch.float16:
+        raise ValueError("take: expects an fp16 table [V, H], int32 ids[n] and an fp16 output")
+    V, H = A.shape
+    n = ids.numel()
+    if out.numel() != n * H:
+        raise ValueError("take: the output holds n * H elements")
+    check(lib().dtas_take_f16(_p(A), _p(ids), _p(out), n, V, H, _cfg(cfg), _stream()), "dtas_take_f16")
+
+
 def take_q8(Wq: torch.Tensor, scale: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
     """out[n,K] (fp16) = rows ids[i] of decode_q8(Wq, scale), the embedding lookup of the 8-bit model:
     fused_fused_decode1_take1 (dolly-v2-3b-q8f16_1/before_dl.py:357-369) and, one row, fused_fused_decode1_take

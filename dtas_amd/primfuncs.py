@@ -204,6 +204,15 @@ def fused_decode(N: int = 2560, K: int = 2560, name: Optional[str] = None) -> Pr
     return PrimFunc(name or "fused_decode3", params, blocks, op="decode_q8", attrs={"tir.noalias": True})
 
 
+def take(V: int = 50280, H: int = 2560, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """T_take(n,H) = A(V,H)[B(n), :], the fp16 embedding lookup: take (dolly-v2-3b-q0f16/before_dl.py:1151-1163; n dynamic)
+    or, with ``decode``, take1 (:1166-1174; one row).  Parameters: A, B, T_take."""
+    n = 1 if decode else "n"
+    params = [Buffer("A", (V, H), "float16"), Buffer("B", (n,), "int32"), Buffer("T_take", (n, H), "float16")]
+    blocks = [Block("T_take", "SS", ["A", "B"], ["T_take"])]
+    return PrimFunc(name or ("take1" if decode else "take"), params, blocks, op="take", attrs={"tir.noalias": True})
+
+
 def fused_decode_take(V: int = 50280, K: int = 2560, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
     """out(n,K) fp16 = rows ids(n) of the dequantised table: fused_fused_decode1_take1
     (dolly-v2-3b-q8f16_1/before_dl.py:357-369; n dynamic) or, with ``decode``, fused_fused_decode1_take (:346-355;

@@ -174,6 +174,12 @@ int dtas_softmax_f32_f16(const void* A, void* out, int64_t rows, int64_t cols,
 int dtas_softmax_f16(const void* A, void* out, int64_t rows, int64_t cols, const dtas_config* cfg,
                      void* stream);
 
+/* take (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1151-1163; one row: take1, :1166-1174), the
+ * embedding lookup: out[n, H] = A[ids[i], :] for a table A[V, H] fp16 and ids[n] int32 (n dynamic).  Ids
+ * outside [0, V) are clipped to the nearest row.  cfg, when given: {DTAS_ELT_VECTOR, block 256, vec 8 | 1}. */
+int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t V, int64_t H,
+                  const dtas_config* cfg, void* stream);
+
 /* ---- GEMV: fused_NT_matmul10_add5 (before_dl.py:96-113) ------------------
  * y[N] = W[N,K] . x[K] (+ bias[N] when bias != NULL); fp16 in/out, fp32 accumulate. */
 int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,

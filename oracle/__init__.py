@@ -69,6 +69,7 @@ class _C:
                 "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
                 "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
                 "oracle_gemv_f32": [vp, vp, vp, i64, i64, ci],
+                "oracle_take_f16": [vp, vp, vp, i64, i64, ci],
                 "oracle_take_q8_f16": [vp, vp, vp, vp, i64, i64, ci],
                 "oracle_gemv_q8_f32": [vp, vp, vp, vp, i64, i64, ci],
                 "oracle_decode_q8_f16": [vp, vp, vp, i64, i64, ci],
@@ -210,6 +211,15 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         out = np.empty(x.shape[:-1] + (N,), dtype=np.float16)
         bp = _ptr(bias) if bias is not None else None
         _C.lib().oracle_gemv_q8_f16(_ptr(x), _ptr(wq), _ptr(scale), bp, _ptr(out), N, K, kind, int(acc_f16), threads)
+        return out
+
+    @staticmethod
+    def take(a, ids, threads: int = 1) -> np.ndarray:
+        """fp16 out[n,H]: rows ids[i] of a[V,H]."""
+        assert a.dtype == np.float16 and a.ndim == 2 and ids.dtype == np.int32
+        assert ids.size == 0 or (0 <= ids.min() and ids.max() < a.shape[0])
+        out = np.empty((ids.size, a.shape[1]), dtype=np.float16)
+        _C.lib().oracle_take_f16(_ptr(a), _ptr(ids), _ptr(out), ids.size, a.shape[1], threads)
         return out
 
     @staticmethod

@@ -454,6 +454,13 @@ void oracle_gemv_f32(const float* x, const float* W, float* y, int64_t N, int64_
  * Pinned by: rows of the pinned dequantiser picked with numpy indexing (bit-exact); numpy float32 arithmetic on the
  * bytes (bit-exact W), the pinned fp32 GEMV on that W (bit-exact y), float64 closed form, one-hot x.
  * ======================================================================== */
+/* take (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1151-1163): T_take[i, j] = A[B[i], j].
+ * Pinned by: numpy indexing (bit-exact). */
+void oracle_take_f16(const f16* A, const int32_t* ids, f16* out, int64_t n, int64_t H, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t ij = 0; ij < n * H; ++ij) out[ij] = A[(int64_t)ids[ij / H] * H + ij % H];
+}
+
 void oracle_take_q8_f16(const uint32_t* Wq, const f16* S, const int32_t* ids, f16* out, int64_t n, int64_t K, int nthreads) {
   OMP_FOR(nthreads)
   for (int64_t ij = 0; ij < n * K; ++ij) out[ij] = decode_q8(Wq, S, K, ids[ij / K], ij % K);

@@ -125,3 +125,12 @@ def test_threads_do_not_change_bits(oracle):
     b = rng.uniform(-1, 1, (37, 4096)).astype(np.float16)
     assert np.array_equal(oracle.c.add(a, b, threads=1).view(np.uint16), oracle.c.add(a, b, threads=4).view(np.uint16))
     assert oracle.c.add(a[:0], b[:0]).size == 0  # empty extent
+
+
+def test_take_is_numpy_row_indexing(oracle):
+    # take (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1151-1163): T_take[i, :] = A[B[i], :], bit for bit
+    rng = np.random.default_rng(31)
+    a = rng.integers(0, 2 ** 16, (37, 24), dtype=np.uint16).view(np.float16)      # every bit pattern, NaN payloads included
+    ids = np.array([0, 36, 5, 5, 17, 36, 0, 1], np.int32)
+    assert np.array_equal(oracle.c.take(a, ids).view(np.uint16), a[ids].view(np.uint16))
+    assert oracle.c.take(a, np.zeros(0, np.int32)).shape == (0, 24)

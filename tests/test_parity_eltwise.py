@@ -203,3 +203,50 @@ def test_full_size_properties():
     assert torch.equal(back.view(torch.int16), a.view(torch.int16))
     # checksum of the sum against an independent fp64 accumulation on the device
     assert abs(ab.double().sum().item() - a.double().sum().item()) == 0
+
+
+@pytest.mark.parametrize("V,H,n", [(50280, 2560, 1), (50280, 2560, 300), (50280, 2560, 4096), (9, 8, 33), (100, 20, 7)])
+def test_take_is_bit_exact(oracle, V, H, n):
+    # the fp16 embedding lookup (take / take1): rows of bit patterns, copied untouched
+    rng = np.random.default_rng(V + n)
+    a = rng.integers(0, 2 ** 16, (V, H), dtype=np.uint16).view(np.float16)
+    ids = rng.integers(0, V, n).astype(np.int32)
+    ids[0], ids[-1] = V - 1, 0
+    out = Guarded((n, H), torch.float16)
+    ops.take(dev(a), dev(ids), out.t)
+    assert_bits_equal(out.check(), oracle.c.take(a, ids, threads=8))
+
+
+def test_take_clips_ids_scalar_path_descriptor_and_errors(oracle):
+    from dtas_amd import primfuncs as pf
+    from dtas_amd.arch import MI355X
+    from dtas_amd.engine.tuner import Engine
+
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((10, 64)).astype(np.float16)
+    ids = np.array([-5, 0, 9, 10, 2 ** 31 - 1, -2 ** 31], np.int32)
+    want = oracle.c.take(a, np.clip(ids, 0, 9).astype(np.int32))
+    for vec in (8, 1):
+        out = Guarded((6, 64), torch.float16)
+        ops.take(dev(a), dev(ids), out.t, cfg(variant=_lib.ELT_VECTOR, block=256, vec=vec))
+        assert_bits_equal(out.check(), want)
+    buf = torch.empty(6 * 64 + 1, dtype=torch.float16, device="cuda")            # 2-byte aligned output: element path
+    ops.take(dev(a), dev(ids), buf[1:].view(6, 64))
+    torch.cuda.synchronize()
+    assert_bits_equal(buf[1:].cpu().numpy().reshape(6, 64), want)
+    funcs = [pf.take(10, 64), pf.take(10, 64, decode=True)]
+    assert [f.name for f in funcs] == ["take", "take1"]
+    rt = Engine(topk=2, parallel_build=False).tune_module(pf.module(*funcs, upper_bound={"n": 512}), MI355X())
+    o = torch.empty(6, 64, dtype=torch.float16, device="cuda")
+    rt["take"](dev(a), dev(np.clip(ids, 0, 9).astype(np.int32)), o)
+    o1 = torch.empty(1, 64, dtype=torch.float16, device="cuda")
+    rt["take1"](dev(a), dev(np.array([9], np.int32)), o1)
+    torch.cuda.synchronize()
+    assert_bits_equal(o.cpu().numpy(), want)
+    assert_bits_equal(o1.cpu().numpy(), a[9:10])
+    L = _lib.lib()
+    assert L.dtas_take_f16(None, None, None, 0, 10, 64, None, None) == 0
+    assert L.dtas_take_f16(None, None, None, 3, 10, 64, None, None) == -1 and b"NULL" in L.dtas_last_error()
+    assert L.dtas_take_f16(None, None, None, 3, 0, 64, None, None) == -1 and b"empty table" in L.dtas_last_error()
+    with pytest.raises(ValueError, match="int32 ids"):
+        ops.take(dev(a), torch.zeros(6, dtype=torch.int64, device="cuda"), torch.empty(6, 64, dtype=torch.float16, device="cuda"))
