@@ -277,6 +277,42 @@ __global__ void __launch_bounds__(kBlock) take_f16_scalar_kernel(const half_t* _
   }
 }
 
+// rotary_embedding (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1023-1035; one row: rotary_embedding1,
+// :1038-1047): the first `rot` of the d elements of every (position, head) row are rotated, every step an fp16
+// value as the PrimFunc spells it,
+//   out[j] = j < rot ? cos[pos, j] * A[j] + sin[pos, j] * (j < rot/2 ? A[j + rot/2] * -1 : A[j - rot/2]) : A[j]
+// with pos = m + s - n.  A thread takes 8 consecutive elements; those past `rot` are a 16-byte copy.
+__global__ void __launch_bounds__(kBlock) rotary_f16_kernel(const half_t* __restrict__ A, const half_t* __restrict__ cs,
+                                                            const half_t* __restrict__ sn, half_t* __restrict__ out,
+                                                            int64_t pieces, int64_t heads, int64_t d, int64_t rot, int64_t pos0) {
+  // (the two products and the sum are three fp16 tensor ops in the PrimFunc: no fused multiply-add, which the
+  // compiler would otherwise form once it has narrowed them to fp16 instructions)
+#pragma clang fp contract(off)
+  const int64_t per_row = d >> 3, half_rot = rot >> 1;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < pieces;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t row = t / per_row, j0 = (t % per_row) << 3;
+    const half_t* a = A + row * d;
+    u32x4 raw = *reinterpret_cast<const u32x4*>(a + j0);
+    if (j0 < rot) {
+      const int64_t pos = pos0 + row / heads;
+      f16x8 v = __builtin_bit_cast(f16x8, raw);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int64_t j = j0 + e;
+        if (j < rot) {
+          const half_t partner = j < half_rot ? static_cast<half_t>(static_cast<float>(a[j + half_rot]) * -1.f) : a[j - half_rot];
+          const half_t t1 = static_cast<half_t>(static_cast<float>(cs[pos * rot + j]) * static_cast<float>(v[e]));
+          const half_t t2 = static_cast<half_t>(static_cast<float>(sn[pos * rot + j]) * static_cast<float>(partner));
+          v[e] = static_cast<half_t>(static_cast<float>(t1) + static_cast<float>(t2));
+        }
+      }
+      raw = __builtin_bit_cast(u32x4, v);
+    }
+    *reinterpret_cast<u32x4*>(out + row * d + j0) = raw;
+  }
+}
+
 }  // namespace
 
 // grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
@@ -358,5 +394,33 @@ int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t 
     hipLaunchKernelGGL(take_f16_scalar_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, s, static_cast<const half_t*>(A),
                        static_cast<const int*>(ids), static_cast<half_t*>(out), items, H, V);
   return check_launch("take");
+}
+int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* out, int64_t n, int64_t m, int64_t heads,
+                    int64_t d, int64_t rot, int64_t max_pos, const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (n < 0 || m < 0 || heads < 0 || d < 0 || rot < 0 || max_pos < 0)
+    return fail("rotary: negative extent n=%lld m=%lld heads=%lld d=%lld rot=%lld", (long long)n, (long long)m, (long long)heads, (long long)d, (long long)rot);
+  if (rot > d || rot % 2 != 0) return fail("rotary: the rotated part (%lld) must be even and at most d (%lld)", (long long)rot, (long long)d);
+  if (d % 8 != 0) return fail("rotary: the head dimension must be a multiple of 8 (d=%lld)", (long long)d);
+  if (n == 0 || heads == 0 || d == 0) return 0;
+  if (heads > INT64_MAX / 4 / d || n > INT64_MAX / 4 / (heads * d)) return fail("rotary: extents overflow");
+  // positions m - n .. m - 1 of the tables
+  if (m < n || m > max_pos) return fail("rotary: positions %lld .. %lld lie outside the tables' %lld rows", (long long)(m - n), (long long)(m - 1), (long long)max_pos);
+  if (!A || !out || (rot > 0 && (!cos_t || !sin_t))) return fail("rotary: NULL buffer");
+  if (!aligned(A, 16) || !aligned(out, 16)) return fail("rotary: A and the output must be 16-byte aligned");
+  const int64_t bytes = n * heads * d * 2;
+  if (overlaps(out, bytes, A, bytes) || overlaps(out, bytes, cos_t, max_pos * rot * 2) || overlaps(out, bytes, sin_t, max_pos * rot * 2))
+    return fail("rotary: output overlaps an input");
+  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, kBlock, 8, 1, {0, 0, 0}, 1, 0};
+  if (cfg.block != kBlock || cfg.vec != 8) return fail("rotary: the kernel uses %d threads and 8 elements per thread", kBlock);
+  const int64_t pieces = n * heads * (d / 8);
+  int64_t grid = ceil_div(pieces, kBlock);
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  grid = grid > cap ? cap : grid;
+  hipLaunchKernelGGL(rotary_f16_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const half_t*>(A), static_cast<const half_t*>(cos_t), static_cast<const half_t*>(sin_t),
+                     static_cast<half_t*>(out), pieces, heads, d, rot, m - n);
+  return check_launch("rotary");
 }
 }

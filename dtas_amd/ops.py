@@ -250,6 +250,21 @@ def decode_q8(Wq: torch.Tensor, scale: torch.Tensor, W: torch.Tensor, cfg: Optio
     check(lib().dtas_decode_q8_f16(_p(Wq), _p(scale), _p(W), N, K, _cfg(cfg), _stream()), "dtas_decode_q8_f16")
 
 
+def rotary(A: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, out: torch.Tensor, m: int,
+           cfg: Optional[DtasConfig] = None) -> None:
+    """rotary_embedding (dolly-v2-3b-q0f16/before_dl.py:1023-1035; rotary_embedding1 :1038-1047): A and out
+    (..., n, heads, d) fp16 with leading extents of 1, cos / sin [max_pos, rot] fp16; position s of A takes the
+    tables' row m + s - n (m = length of the whole sequence)."""
+    _dev(A, cos, sin, out)
+    if any(t.dtype != torch.float16 for t in (A, cos, sin, out)) or cos.dim() != 2 or cos.shape != sin.shape or A.dim() < 3:
+        raise ValueError("rotary: expects fp16 A (..., n, heads, d) and fp16 tables [max_pos, rot]")
+    n, heads, d = A.shape[-3:]
+    if A.numel() != n * heads * d or out.shape != A.shape:
+        raise ValueError("rotary: leading extents must be 1 and out must have A's shape")
+    check(lib().dtas_rotary_f16(_p(A), _p(cos), _p(sin), _p(out), n, int(m), heads, d, cos.shape[1], cos.shape[0], _cfg(cfg),
+                                _stream()), "dtas_rotary_f16")
+
+
 def take(A: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, cfg: Optional[DtasConfig] = None) -> None:
     """out[n,H] = A[ids[i], :], the fp16 embedding lookup: take (dolly-v2-3b-q0f16/before_dl.py:1151-1163) and, one row,
     take1 (:1166-1174).  ids int32; values outside [0, V) are clipped to the nearest row."""

@@ -180,6 +180,14 @@ int dtas_softmax_f16(const void* A, void* out, int64_t rows, int64_t cols, const
 int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t V, int64_t H,
                   const dtas_config* cfg, void* stream);
 
+/* rotary_embedding (before_dl.py:1023-1035; one row: rotary_embedding1, :1038-1047), applied to the queries
+ * and keys before the scores: A and out are [n, heads, d] fp16 (n dynamic), cos and sin [max_pos, rot] fp16;
+ * the first rot elements of every row are rotated with the tables' row m + s - n for position s (m = the
+ * length of the whole sequence, m >= n), each step an fp16 value:
+ *   out[j] = cos[j] * A[j] + sin[j] * (j < rot/2 ? A[j + rot/2] * -1 : A[j - rot/2])   (j < rot);  A[j] else. */
+int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* out, int64_t n, int64_t m,
+                    int64_t heads, int64_t d, int64_t rot, int64_t max_pos, const dtas_config* cfg, void* stream);
+
 /* ---- GEMV: fused_NT_matmul10_add5 (before_dl.py:96-113) ------------------
  * y[N] = W[N,K] . x[K] (+ bias[N] when bias != NULL); fp16 in/out, fp32 accumulate. */
 int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,

@@ -70,6 +70,7 @@ class _C:
                 "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
                 "oracle_gemv_f32": [vp, vp, vp, i64, i64, ci],
                 "oracle_take_f16": [vp, vp, vp, i64, i64, ci],
+                "oracle_rotary_f16": [vp, vp, vp, vp, i64, i64, i64, i64, i64, ci],
                 "oracle_take_q8_f16": [vp, vp, vp, vp, i64, i64, ci],
                 "oracle_gemv_q8_f32": [vp, vp, vp, vp, i64, i64, ci],
                 "oracle_decode_q8_f16": [vp, vp, vp, i64, i64, ci],
@@ -211,6 +212,16 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         out = np.empty(x.shape[:-1] + (N,), dtype=np.float16)
         bp = _ptr(bias) if bias is not None else None
         _C.lib().oracle_gemv_q8_f16(_ptr(x), _ptr(wq), _ptr(scale), bp, _ptr(out), N, K, kind, int(acc_f16), threads)
+        return out
+
+    @staticmethod
+    def rotary(a, cos, sin, m: int, threads: int = 1) -> np.ndarray:
+        """fp16 rotary embedding of a[n, heads, d] with tables cos/sin[max_pos, rot] at positions m - n .. m - 1."""
+        n, heads, d = a.shape[-3:]
+        rot = cos.shape[1]
+        assert a.dtype == cos.dtype == sin.dtype == np.float16 and cos.shape == sin.shape and n <= m <= cos.shape[0]
+        out = np.empty_like(a)
+        _C.lib().oracle_rotary_f16(_ptr(a), _ptr(cos), _ptr(sin), _ptr(out), n, m, heads, d, rot, threads)
         return out
 
     @staticmethod

@@ -454,6 +454,26 @@ void oracle_gemv_f32(const float* x, const float* W, float* y, int64_t N, int64_
  * Pinned by: rows of the pinned dequantiser picked with numpy indexing (bit-exact); numpy float32 arithmetic on the
  * bytes (bit-exact W), the pinned fp32 GEMV on that W (bit-exact y), float64 closed form, one-hot x.
  * ======================================================================== */
+/* rotary_embedding (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1023-1035), every step an fp16 tensor op:
+ *   rotary[s,h,j] = j < rot ? B[pos,j] * A[s,h,j] + C[pos,j] * (j < rot/2 ? A[s,h,j+rot/2] * -1 : A[s,h,j-rot/2]) : A[s,h,j]
+ * with pos = m + s - n.  Pinned by: numpy float16 arithmetic step by step (bit-exact), cos = 1 / sin = 0 (identity),
+ * the float64 rotation (tolerance), preserved pair norms for cos^2 + sin^2 = 1. */
+void oracle_rotary_f16(const f16* A, const f16* B, const f16* C, f16* out, int64_t n, int64_t m, int64_t heads, int64_t d,
+                       int64_t rot, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t sh = 0; sh < n * heads; ++sh) {
+    const int64_t pos = m + sh / heads - n;
+    const f16* a = A + sh * d;
+    for (int64_t j = 0; j < d; ++j) {
+      if (j >= rot) { out[sh * d + j] = a[j]; continue; }
+      const f16 partner = j < rot / 2 ? f2h(h2f(a[j + rot / 2]) * -1.f) : a[j - rot / 2];
+      const f16 t1 = f2h(h2f(B[pos * rot + j]) * h2f(a[j]));
+      const f16 t2 = f2h(h2f(C[pos * rot + j]) * h2f(partner));
+      out[sh * d + j] = f2h(h2f(t1) + h2f(t2));
+    }
+  }
+}
+
 /* take (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1151-1163): T_take[i, j] = A[B[i], j].
  * Pinned by: numpy indexing (bit-exact). */
 void oracle_take_f16(const f16* A, const int32_t* ids, f16* out, int64_t n, int64_t H, int nthreads) {

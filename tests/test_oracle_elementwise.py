@@ -134,3 +134,39 @@ def test_take_is_numpy_row_indexing(oracle):
     ids = np.array([0, 36, 5, 5, 17, 36, 0, 1], np.int32)
     assert np.array_equal(oracle.c.take(a, ids).view(np.uint16), a[ids].view(np.uint16))
     assert oracle.c.take(a, np.zeros(0, np.int32)).shape == (0, 24)
+
+
+def _rotary_inputs(n, heads, d, rot, max_pos, seed):
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((1, n, heads, d)).astype(np.float16)
+    ang = rng.uniform(0, 6.28, (max_pos, rot))
+    return a, np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+
+
+def test_rotary_matches_numpy_float16_step_by_step(oracle):
+    # rotary_embedding (before_dl.py:1023-1035): B * A + C * (j < 10 ? A[j + 10] * -1 : A[j - 10]) for j < 20, A beyond
+    n, heads, d, rot, m = 5, 3, 80, 20, 9
+    a, cos, sin = _rotary_inputs(n, heads, d, rot, 16, 1)
+    got = oracle.c.rotary(a, cos, sin, m)
+    pos = m + np.arange(n) - n
+    b, c = cos[pos][:, None, :], sin[pos][:, None, :]                        # [n, 1, rot]
+    x = a[0]
+    partner = np.concatenate([x[..., 10:20] * np.float16(-1), x[..., 0:10]], axis=-1)      # numpy rounds each fp16 op
+    want = x.copy()
+    want[..., :rot] = b * x[..., :rot] + c * partner
+    assert want.dtype == np.float16 and np.array_equal(got[0].view(np.uint16), want.view(np.uint16))
+    # float64 rotation of the pairs (j, j + 10): tolerance, and the pair norms survive when cos^2 + sin^2 = 1
+    x64, b64, c64 = x.astype(np.float64), b.astype(np.float64), c.astype(np.float64)
+    lo = b64[..., :10] * x64[..., :10] - c64[..., :10] * x64[..., 10:20]
+    hi = b64[..., 10:] * x64[..., 10:20] + c64[..., 10:] * x64[..., :10]
+    assert np.abs(got[0][..., :10].astype(np.float64) - lo).max() < 4e-3 and np.abs(got[0][..., 10:20].astype(np.float64) - hi).max() < 4e-3
+    # a swapped partner or a missing sign fails this: rotating by a quarter turn maps (x, y) to (-y, x)
+    q_cos, q_sin = np.zeros((16, rot), np.float16), np.ones((16, rot), np.float16)
+    quarter = oracle.c.rotary(a, q_cos, q_sin, m)[0]
+    assert np.array_equal(quarter[..., :10], -x[..., 10:20]) and np.array_equal(quarter[..., 10:20], x[..., :10])
+    # cos = 1, sin = 0: the identity, bit for bit; the positions are m - n .. m - 1
+    ident = oracle.c.rotary(a, np.ones((16, rot), np.float16), np.zeros((16, rot), np.float16), m)
+    assert np.array_equal(ident.view(np.uint16), a.view(np.uint16))
+    marked = np.ones((16, rot), np.float16)
+    marked[m - n] = 2
+    assert np.array_equal(oracle.c.rotary(a, marked, np.zeros((16, rot), np.float16), m)[0, 0, :, :rot], x[0, :, :rot] * np.float16(2))

@@ -250,3 +250,29 @@ def test_take_clips_ids_scalar_path_descriptor_and_errors(oracle):
     assert L.dtas_take_f16(None, None, None, 3, 0, 64, None, None) == -1 and b"empty table" in L.dtas_last_error()
     with pytest.raises(ValueError, match="int32 ids"):
         ops.take(dev(a), torch.zeros(6, dtype=torch.int64, device="cuda"), torch.empty(6, 64, dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.parametrize("n,m,heads,d,rot", [(1, 1, 32, 80, 20), (1, 2048, 32, 80, 20), (300, 300, 32, 80, 20), (257, 4096, 32, 80, 20),
+                                             (7, 9, 3, 64, 64), (5, 5, 2, 16, 0), (33, 40, 4, 128, 32)])
+def test_rotary_is_bit_exact(oracle, n, m, heads, d, rot):
+    rng = np.random.default_rng(n + m + d)
+    a = rng.standard_normal((1, n, heads, d)).astype(np.float16)
+    ang = rng.uniform(0, 6.28, (4096, rot))
+    cos, sin = np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
+    out = Guarded(a.shape, torch.float16)
+    ops.rotary(dev(a), dev(cos), dev(sin), out.t, m)
+    assert_bits_equal(out.check(), oracle.c.rotary(a, cos, sin, m, threads=8))
+
+
+def test_rotary_errors():
+    a = torch.zeros(1, 4, 2, 80, dtype=torch.float16, device="cuda")
+    t = torch.zeros(16, 20, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="outside the tables"):
+        ops.rotary(a, t, t, torch.empty_like(a), 3)          # m < n
+    with pytest.raises(_lib.DtasError, match="outside the tables"):
+        ops.rotary(a, t, t, torch.empty_like(a), 17)         # m > max_pos
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        ops.rotary(a, t, t, a, 4)
+    with pytest.raises(_lib.DtasError, match="must be even"):
+        ops.rotary(a, torch.zeros(16, 21, dtype=torch.float16, device="cuda"), torch.zeros(16, 21, dtype=torch.float16, device="cuda"),
+                   torch.empty_like(a), 4)
