@@ -136,6 +136,18 @@ def _workload(name: str, n: int, extra=None):
             return wq, uniform((V, K // 32), s + 100, 0.001, 0.02), ids, empty((n, K))
         return (make, lambda b: call(L.dtas_take_q8_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, V, K, None, stream),
                 n * K + 2 * n * (K // 32) + 4 * n + 2 * n * K, 0)
+    if name == "take_f16":
+        # take: n rows of the 50280 x 2560 fp16 embedding table
+        V, K = extra
+        def make(s):
+            g = torch.Generator(device="cuda").manual_seed(s + 200)
+            return normal((V, K), s), torch.randint(0, V, (n,), dtype=torch.int32, device="cuda", generator=g), empty((n, K))
+        return (make, lambda b: call(L.dtas_take_f16, P(b[0]), P(b[1]), P(b[2]), n, V, K, None, stream), 4 * n * K + 4 * n, 0)
+    if name == "rotary_f16":
+        # rotary_embedding: [n, 32, 80] with the first 20 of every 80 rotated, tables [4096, 20]
+        make = lambda s: (normal((n, 32, 80), s), uniform((4096, 20), s + 1), uniform((4096, 20), s + 2), empty((n, 32, 80)))
+        return (make, lambda b: call(L.dtas_rotary_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, n, 32, 80, 20, 4096, None, stream),
+                4 * n * 2560 + 2 * 2 * n * 20, 0)
     if name == "gemm_f16":
         N, K = extra
         wt = normal((N, K), 100, 0.02)
@@ -325,6 +337,8 @@ def sweep(steps: int, warmup: int) -> list:
     rows.append(measure("gemv_q8_f32", 1, (50280, 2560), steps, warmup))
     for n in (1, 1024, 4096):
         rows.append(measure("take_q8_f16", n, (50280, 2560), steps, warmup))
+        rows.append(measure("take_f16", n, (50280, 2560), steps, warmup))
+        rows.append(measure("rotary_f16", n, None, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
@@ -363,7 +377,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
-                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
+                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")
@@ -388,7 +402,7 @@ def main() -> int:
         print(_lib.last_error(), file=sys.stderr)
         return 2
 
-    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32", "take_q8_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
+    extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32", "take_q8_f16", "take_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
     info = None

@@ -313,6 +313,53 @@ __global__ void __launch_bounds__(kBlock) rotary_f16_kernel(const half_t* __rest
   }
 }
 
+// The same for the model's shape (20 of the d elements rotated): every thread takes one 16-byte piece, and a
+// piece of the rotated part finds its partners with one or two more 16-byte loads at the elements' alignment
+// (piece 0: elements 10..17 negated; piece 1: 18, 19 negated, then 0..5; piece 2: 6..9) and its part of the
+// tables' row with 8-byte loads (a table row is 40 bytes).
+__global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restrict__ A, const half_t* __restrict__ cs,
+                                                          const half_t* __restrict__ sn, half_t* __restrict__ out,
+                                                          int64_t pieces, int64_t heads, int64_t d, int64_t pos0) {
+#pragma clang fp contract(off)
+  typedef u32x4 __attribute__((aligned(2))) u32x4_a2;
+  const int64_t per_row = d >> 3;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < pieces;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t row = t / per_row, v = t % per_row;
+    const half_t* a = A + row * d;
+    u32x4 raw = *reinterpret_cast<const u32x4*>(a + 8 * v);
+    if (v < 3) {
+      const f16x8 x = __builtin_bit_cast(f16x8, raw);
+      // partners: p[e] for element j = 8 v + e
+      const f16x8 far = __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4_a2*>(a + (v == 0 ? 10 : v == 1 ? 18 : 6)));
+      const f16x8 low = __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(a));   // elements 0..7 (piece 1 needs 0..5)
+      const half_t* cr = cs + (pos0 + row / heads) * 20 + 8 * v;
+      const half_t* sr = sn + (pos0 + row / heads) * 20 + 8 * v;
+      f16x4 c0 = __builtin_bit_cast(f16x4, *reinterpret_cast<const u32x2*>(cr)), s0 = __builtin_bit_cast(f16x4, *reinterpret_cast<const u32x2*>(sr));
+      f16x4 c1 = {}, s1 = {};
+      if (v < 2) {  // (piece 2 holds the tables' elements 16..19 only)
+        c1 = __builtin_bit_cast(f16x4, *reinterpret_cast<const u32x2*>(cr + 4));
+        s1 = __builtin_bit_cast(f16x4, *reinterpret_cast<const u32x2*>(sr + 4));
+      }
+      f16x8 r = x;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (v == 2 && e >= 4) continue;  // elements 20..23 are not rotated
+        half_t partner;
+        if (v == 0) partner = static_cast<half_t>(static_cast<float>(far[e]) * -1.f);
+        else if (v == 1) partner = e < 2 ? static_cast<half_t>(static_cast<float>(far[e]) * -1.f) : low[e >= 2 ? e - 2 : 0];
+        else partner = far[e];
+        const half_t cj = e < 4 ? c0[e] : c1[e - 4 < 0 ? 0 : e - 4], sj = e < 4 ? s0[e] : s1[e - 4 < 0 ? 0 : e - 4];
+        const half_t t1 = static_cast<half_t>(static_cast<float>(cj) * static_cast<float>(x[e]));
+        const half_t t2 = static_cast<half_t>(static_cast<float>(sj) * static_cast<float>(partner));
+        r[e] = static_cast<half_t>(static_cast<float>(t1) + static_cast<float>(t2));
+      }
+      raw = __builtin_bit_cast(u32x4, r);
+    }
+    *reinterpret_cast<u32x4*>(out + row * d + 8 * v) = raw;
+  }
+}
+
 }  // namespace
 
 // grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
@@ -414,9 +461,18 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
     return fail("rotary: output overlaps an input");
   dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, kBlock, 8, 1, {0, 0, 0}, 1, 0};
   if (cfg.block != kBlock || cfg.vec != 8) return fail("rotary: the kernel uses %d threads and 8 elements per thread", kBlock);
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  if (rot == 20 && d >= 32 && cfg.unroll <= 1 && aligned(cos_t, 8) && aligned(sin_t, 8)) {  // the model's shape (cfg.unroll = 2 forces the general kernel)
+    const int64_t pieces20 = n * heads * (d / 8);
+    int64_t grid = ceil_div(pieces20, kBlock);
+    grid = grid > cap ? cap : grid;
+    hipLaunchKernelGGL(rotary20_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const half_t*>(A), static_cast<const half_t*>(cos_t), static_cast<const half_t*>(sin_t),
+                       static_cast<half_t*>(out), pieces20, heads, d, m - n);
+    return check_launch("rotary");
+  }
   const int64_t pieces = n * heads * (d / 8);
   int64_t grid = ceil_div(pieces, kBlock);
-  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
   grid = grid > cap ? cap : grid;
   hipLaunchKernelGGL(rotary_f16_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
                      static_cast<const half_t*>(A), static_cast<const half_t*>(cos_t), static_cast<const half_t*>(sin_t),

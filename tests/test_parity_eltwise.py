@@ -261,7 +261,11 @@ def test_rotary_is_bit_exact(oracle, n, m, heads, d, rot):
     cos, sin = np.cos(ang).astype(np.float16), np.sin(ang).astype(np.float16)
     out = Guarded(a.shape, torch.float16)
     ops.rotary(dev(a), dev(cos), dev(sin), out.t, m)
-    assert_bits_equal(out.check(), oracle.c.rotary(a, cos, sin, m, threads=8))
+    want = oracle.c.rotary(a, cos, sin, m, threads=8)
+    assert_bits_equal(out.check(), want)
+    out = Guarded(a.shape, torch.float16)      # the kernel for any rotated width, also where the model's has its own
+    ops.rotary(dev(a), dev(cos), dev(sin), out.t, m, cfg(variant=_lib.ELT_VECTOR, block=256, vec=8, unroll=2))
+    assert_bits_equal(out.check(), want)
 
 
 def test_rotary_errors():
