@@ -360,6 +360,49 @@ __global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restri
   }
 }
 
+// The attention mask of the prefill and decode graphs in one pass: fused_min_max_triu_te_broadcast_to
+// (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:642-658: [n, n], -65504 above the diagonal, 65504 elsewhere),
+// extended to m >= n key positions by extend_te (:68-80: 65504 for the m - n positions already cached, the
+// triangle after them) -- and, with n = 1, full (:83-93).  out[i, j] = (j - (m - n) > i) ? -65504 : 65504.
+// A thread writes 8 consecutive elements of the flat [n * m] array (16-byte stores whatever m is).
+__global__ void __launch_bounds__(kBlock) attn_mask_kernel(half_t* __restrict__ out, int64_t n, int64_t m) {
+  const int64_t total = n * m, shift = m - n;
+  for (int64_t t = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8; t < total;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x * 8) {
+    int64_t i = t / m, jj = t % m;
+    f16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = static_cast<half_t>(jj - shift > i ? -65504.f : 65504.f);
+      if (++jj == m) {
+        jj = 0;
+        ++i;
+      }
+    }
+    if (t + 8 <= total) {
+      *reinterpret_cast<u32x4*>(out + t) = __builtin_bit_cast(u32x4, v);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (t + e < total) out[t + e] = v[e];
+    }
+  }
+}
+
+// transpose6 / transpose7 (before_dl.py:1177-1203): [a, b, d] -> [b, a, d], rows of d elements moved whole
+// (queries, keys and values between the projection's [n, heads, d] and attention's [heads, n, d]).  A thread
+// moves one 16-byte piece; the stores are the contiguous side.
+__global__ void __launch_bounds__(kBlock) swap_axes_kernel(const u32x4* __restrict__ A, u32x4* __restrict__ out, int64_t a,
+                                                           int64_t b, int64_t per_row) {
+  const int64_t total = a * b * per_row;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t p = t % per_row, r = t / per_row;   // output row r = ib * a + ia
+    const int64_t ib = r / a, ia = r % a;
+    out[t] = A[(ia * b + ib) * per_row + p];
+  }
+}
+
 }  // namespace
 
 // grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
@@ -478,5 +521,36 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
                      static_cast<const half_t*>(A), static_cast<const half_t*>(cos_t), static_cast<const half_t*>(sin_t),
                      static_cast<half_t*>(out), pieces, heads, d, rot, m - n);
   return check_launch("rotary");
+}
+int dtas_attn_mask_f16(void* out, int64_t n, int64_t m, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (n < 0 || m < 0) return fail("attn_mask: negative extent n=%lld m=%lld", (long long)n, (long long)m);
+  if (m < n) return fail("attn_mask: m (%lld key positions) must be at least n (%lld query positions)", (long long)m, (long long)n);
+  if (n == 0 || m == 0) return 0;
+  if (n > INT64_MAX / 4 / m) return fail("attn_mask: n*m overflows");
+  if (!out) return fail("attn_mask: NULL buffer");
+  if (!aligned(out, 16)) return fail("attn_mask: the output must be 16-byte aligned");
+  int64_t grid = ceil_div(ceil_div(n * m, 8), kBlock);
+  grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+  hipLaunchKernelGGL(attn_mask_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                     static_cast<half_t*>(out), n, m);
+  return check_launch("attn_mask");
+}
+int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (a < 0 || b < 0 || d < 0) return fail("swap_axes: negative extent a=%lld b=%lld d=%lld", (long long)a, (long long)b, (long long)d);
+  if (a == 0 || b == 0 || d == 0) return 0;
+  if (d % 8 != 0) return fail("swap_axes: rows must be a multiple of 8 elements (d=%lld)", (long long)d);
+  if (a > INT64_MAX / 4 / d || b > INT64_MAX / 4 / (a * d)) return fail("swap_axes: extents overflow");
+  if (!A || !out) return fail("swap_axes: NULL buffer");
+  if (!aligned(A, 16) || !aligned(out, 16)) return fail("swap_axes: buffers must be 16-byte aligned");
+  if (overlaps(out, a * b * d * 2, A, a * b * d * 2)) return fail("swap_axes: output overlaps the input");
+  int64_t grid = ceil_div(a * b * (d / 8), kBlock);
+  grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+  hipLaunchKernelGGL(swap_axes_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const u32x4*>(A), static_cast<u32x4*>(out), a, b, d / 8);
+  return check_launch("swap_axes");
 }
 }

@@ -250,6 +250,28 @@ def decode_q8(Wq: torch.Tensor, scale: torch.Tensor, W: torch.Tensor, cfg: Optio
     check(lib().dtas_decode_q8_f16(_p(Wq), _p(scale), _p(W), N, K, _cfg(cfg), _stream()), "dtas_decode_q8_f16")
 
 
+def attn_mask(out: torch.Tensor) -> None:
+    """out (..., n, m) fp16 = the causal mask of n query positions against m >= n key positions (65504 where a key
+    may be seen, -65504 where not): fused_min_max_triu_te_broadcast_to + extend_te, and full for n = 1
+    (dolly-v2-3b-q0f16/before_dl.py:642-658, :68-80, :83-93)."""
+    _dev(out)
+    n, m = out.shape[-2:]
+    if out.dtype != torch.float16 or out.numel() != n * m:
+        raise ValueError("attn_mask: expects an fp16 output (..., n, m) with leading extents of 1")
+    check(lib().dtas_attn_mask_f16(_p(out), n, m, _stream()), "dtas_attn_mask_f16")
+
+
+def swap_axes(A: torch.Tensor, out: torch.Tensor) -> None:
+    """out (..., b, a, d) = A (..., a, b, d) with leading extents of 1, fp16: transpose6 / transpose7
+    (dolly-v2-3b-q0f16/before_dl.py:1177-1203)."""
+    _dev(A, out)
+    a, b, d = A.shape[-3:]
+    if A.dtype != torch.float16 or out.dtype != torch.float16 or A.numel() != a * b * d or tuple(out.shape[-3:]) != (b, a, d) \
+            or out.numel() != a * b * d:
+        raise ValueError("swap_axes: expects fp16 A (..., a, b, d) and out (..., b, a, d) with leading extents of 1")
+    check(lib().dtas_swap_axes_f16(_p(A), _p(out), a, b, d, _stream()), "dtas_swap_axes_f16")
+
+
 def rotary(A: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, out: torch.Tensor, m: int,
            cfg: Optional[DtasConfig] = None) -> None:
     """rotary_embedding (dolly-v2-3b-q0f16/before_dl.py:1023-1035; rotary_embedding1 :1038-1047): A and out

@@ -188,6 +188,14 @@ int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t 
 int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* out, int64_t n, int64_t m,
                     int64_t heads, int64_t d, int64_t rot, int64_t max_pos, const dtas_config* cfg, void* stream);
 
+/* The attention mask: fused_min_max_triu_te_broadcast_to (before_dl.py:642-658) followed by extend_te (:68-80),
+ * and full (:83-93) when n = 1.  out[n, m] fp16 (n query positions, m >= n key positions, both dynamic):
+ *   out[i, j] = j - (m - n) > i ? -65504 : 65504. */
+int dtas_attn_mask_f16(void* out, int64_t n, int64_t m, void* stream);
+/* transpose6 / transpose7 (before_dl.py:1177-1203): A[a, b, d] -> out[b, a, d] fp16, rows of d elements
+ * (d % 8 == 0) moved whole: [n, heads, d] <-> [heads, n, d] around the attention kernels. */
+int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d, void* stream);
+
 /* ---- GEMV: fused_NT_matmul10_add5 (before_dl.py:96-113) ------------------
  * y[N] = W[N,K] . x[K] (+ bias[N] when bias != NULL); fp16 in/out, fp32 accumulate. */
 int dtas_gemv_f16(const void* x, const void* W, const void* bias, void* y, int64_t N, int64_t K,

@@ -270,6 +270,23 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         return int(_C.lib().oracle_soft_f2h(ctypes.c_float(v)))
 
 
+class layout:
+    """The index-only PrimFuncs around attention, in numpy (bit-exact by construction)."""
+
+    @staticmethod
+    def attn_mask(n: int, m: int) -> np.ndarray:
+        """fused_min_max_triu_te_broadcast_to (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:642-658) followed by
+        extend_te (:68-80), in one expression: -65504 where key j lies after query i (of the last n positions), 65504
+        elsewhere; n = 1 is full (:83-93)."""
+        i, j = np.arange(n)[:, None], np.arange(m)[None, :]
+        return np.where(j - (m - n) > i, np.float16(-65504), np.float16(65504)).astype(np.float16)
+
+    @staticmethod
+    def swap_axes(a: np.ndarray) -> np.ndarray:
+        """transpose6 / transpose7 (before_dl.py:1177-1203): T[.., i1, i2, :] = A[.., i2, i1, :]."""
+        return np.ascontiguousarray(np.swapaxes(a, -3, -2))
+
+
 class np64:  # noqa: N801
     """Closed forms in float64 -- independent of cpu_ref.c; the tolerance anchor."""
 

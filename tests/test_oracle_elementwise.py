@@ -170,3 +170,26 @@ def test_rotary_matches_numpy_float16_step_by_step(oracle):
     marked = np.ones((16, rot), np.float16)
     marked[m - n] = 2
     assert np.array_equal(oracle.c.rotary(a, marked, np.zeros((16, rot), np.float16), m)[0, 0, :, :rot], x[0, :, :rot] * np.float16(2))
+
+
+def test_attn_mask_is_the_two_primfuncs_in_sequence(oracle):
+    # make_diag_mask_te: Select(i < j, -65504, 65504) on [n, n]; extend_te: j < m - n ? 65504 : A[i, j + n - m] on [n, m]
+    for n, m in ((1, 1), (1, 7), (5, 5), (5, 9), (64, 200)):
+        diag = np.where(np.arange(n)[:, None] < np.arange(n)[None, :], np.float16(-65504), np.float16(65504)).astype(np.float16)
+        ext = np.full((n, m), np.float16(65504), np.float16)
+        ext[:, m - n:] = diag
+        got = oracle.layout.attn_mask(n, m)
+        assert got.dtype == np.float16 and np.array_equal(got, ext)
+    assert np.array_equal(oracle.layout.attn_mask(1, 9), np.full((1, 9), 65504, np.float16))      # full: nothing hidden from the last position
+    last = oracle.layout.attn_mask(4, 6)
+    assert (last[0] == [65504, 65504, 65504, -65504, -65504, -65504]).all() and (last[3] == 65504).all()
+
+
+def test_swap_axes_follows_the_index_expression(oracle):
+    rng = np.random.default_rng(3)
+    a = rng.integers(0, 2 ** 16, (1, 5, 3, 8), dtype=np.uint16).view(np.float16)
+    t = oracle.layout.swap_axes(a)
+    assert t.shape == (1, 3, 5, 8)
+    for i1 in range(3):
+        for i2 in range(5):
+            assert np.array_equal(t[0, i1, i2].view(np.uint16), a[0, i2, i1].view(np.uint16))

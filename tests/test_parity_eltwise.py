@@ -280,3 +280,30 @@ def test_rotary_errors():
     with pytest.raises(_lib.DtasError, match="must be even"):
         ops.rotary(a, torch.zeros(16, 21, dtype=torch.float16, device="cuda"), torch.zeros(16, 21, dtype=torch.float16, device="cuda"),
                    torch.empty_like(a), 4)
+
+
+@pytest.mark.parametrize("n,m", [(1, 1), (1, 2049), (7, 7), (33, 77), (300, 1025), (1024, 1024), (2047, 2047)])
+def test_attn_mask_is_exact(oracle, n, m):
+    out = Guarded((1, 1, n, m), torch.float16)
+    ops.attn_mask(out.t)
+    assert_bits_equal(out.check().reshape(n, m), oracle.layout.attn_mask(n, m))
+
+
+@pytest.mark.parametrize("a,b,d", [(1, 32, 80), (300, 32, 80), (32, 300, 80), (4096, 32, 80), (5, 3, 8)])
+def test_swap_axes_is_exact(oracle, a, b, d):
+    rng = np.random.default_rng(a + b)
+    x = rng.integers(0, 2 ** 16, (1, a, b, d), dtype=np.uint16).view(np.float16)
+    out = Guarded((1, b, a, d), torch.float16)
+    ops.swap_axes(dev(x), out.t)
+    assert_bits_equal(out.check(), oracle.layout.swap_axes(x))
+
+
+def test_mask_and_swap_errors():
+    L = _lib.lib()
+    assert L.dtas_attn_mask_f16(None, 0, 5, None) == 0 and L.dtas_swap_axes_f16(None, None, 0, 3, 8, None) == 0
+    assert L.dtas_attn_mask_f16(None, 5, 3, None) == -1 and b"at least n" in L.dtas_last_error()
+    assert L.dtas_attn_mask_f16(None, 3, 5, None) == -1 and b"NULL" in L.dtas_last_error()
+    assert L.dtas_swap_axes_f16(None, None, 2, 3, 7, None) == -1 and b"multiple of 8" in L.dtas_last_error()
+    x = torch.zeros(2, 3, 8, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        _lib.check(L.dtas_swap_axes_f16(x.data_ptr(), x.data_ptr(), 2, 3, 8, None), "swap")
