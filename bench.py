@@ -148,6 +148,26 @@ def _workload(name: str, n: int, extra=None):
         make = lambda s: (normal((n, 32, 80), s), uniform((4096, 20), s + 1), uniform((4096, 20), s + 2), empty((n, 32, 80)))
         return (make, lambda b: call(L.dtas_rotary_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, n, 32, 80, 20, 4096, None, stream),
                 4 * n * 2560 + 2 * 2 * n * 20, 0)
+    if name == "attn_mask_f16":
+        # fused_min_max_triu_te_broadcast_to + extend_te: the [n, n] causal mask, written only
+        make = lambda s: (empty((n, n)),)
+        return make, lambda b: call(L.dtas_attn_mask_f16, P(b[0]), n, n, stream), 2 * n * n, 0
+    if name == "swap_axes_f16":
+        # transpose6: [n, 32, 80] -> [32, n, 80]
+        make = lambda s: (normal((n, 32, 80), s), empty((32, n, 80)))
+        return make, lambda b: call(L.dtas_swap_axes_f16, P(b[0]), P(b[1]), n, 32, 80, stream), 4 * n * 2560, 0
+    if name == "split3_f16":
+        # split: the fused projection [n, 32, 240] into queries, keys and values [n, 32, 80]
+        make = lambda s: (normal((n * 32, 240), s), empty((n * 32, 80)), empty((n * 32, 80)), empty((n * 32, 80)))
+        return (make, lambda b: call(L.dtas_split3_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n * 32, 80, stream),
+                4 * n * 7680, 0)
+    if name == "softmax_temperature_f32":
+        # softmax_with_temperature: n rows (the model has 1) of 50280 fp32 logits
+        V = 50280
+        temp = torch.tensor(0.7, dtype=torch.float32, device="cuda")
+        make = lambda s: (normal((n, V), s, 4.0, torch.float32), temp, empty((n, V), torch.float32))
+        return (make, lambda b: call(L.dtas_softmax_temperature_f32, P(b[0]), P(b[1]), P(b[2]), n, V, stream),
+                8 * n * V + 4, 0)
     if name == "gemm_f16":
         N, K = extra
         wt = normal((N, K), 100, 0.02)
@@ -339,6 +359,10 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("take_q8_f16", n, (50280, 2560), steps, warmup))
         rows.append(measure("take_f16", n, (50280, 2560), steps, warmup))
         rows.append(measure("rotary_f16", n, None, steps, warmup))
+        rows.append(measure("split3_f16", n, None, steps, warmup))
+        rows.append(measure("swap_axes_f16", n, None, steps, warmup))
+        rows.append(measure("attn_mask_f16", n, None, steps, warmup))
+    rows.append(measure("softmax_temperature_f32", 1, None, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
@@ -377,7 +401,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
                     help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
-                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
+                         "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | split3_f16 | swap_axes_f16 | attn_mask_f16 | softmax_temperature_f32 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
     ap.add_argument("--no-sweep", action="store_true")

@@ -403,6 +403,23 @@ __global__ void __launch_bounds__(kBlock) swap_axes_kernel(const u32x4* __restri
   }
 }
 
+// split (before_dl.py:1099-1125) and fused_reshape7_split1 (:661-688): the fused query / key / value projection
+// A[rows, 3 d] (rows = positions x heads, d = 80) cut into three [rows, d] buffers, section s = columns
+// [s d, (s + 1) d).  T is a 16-byte piece (d % 8 == 0, aligned buffers) or one element; the loads run
+// through A in order, the stores are runs of d elements.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) split3_kernel(const T* __restrict__ A, T* __restrict__ o0, T* __restrict__ o1,
+                                                        T* __restrict__ o2, int64_t rows, int64_t per_sec) {
+  const int64_t total = rows * 3 * per_sec;
+  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = t / (3 * per_sec), c = t % (3 * per_sec);
+    const int64_t sec = c / per_sec, j = c % per_sec;
+    T* o = sec == 0 ? o0 : sec == 1 ? o1 : o2;
+    o[r * per_sec + j] = A[t];
+  }
+}
+
 }  // namespace
 
 // grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
@@ -552,5 +569,34 @@ int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d
   hipLaunchKernelGGL(swap_axes_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4*>(A), static_cast<u32x4*>(out), a, b, d / 8);
   return check_launch("swap_axes");
+}
+int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t rows, int64_t d, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (rows < 0 || d < 0) return fail("split3: negative extent rows=%lld d=%lld", (long long)rows, (long long)d);
+  if (rows == 0 || d == 0) return 0;
+  if (rows > INT64_MAX / 8 / d) return fail("split3: rows*d overflows");
+  if (!A || !out0 || !out1 || !out2) return fail("split3: NULL buffer");
+  void* outs[3] = {out0, out1, out2};
+  const int64_t sec_bytes = rows * d * 2;
+  for (int i = 0; i < 3; ++i) {
+    if (!aligned(outs[i], 2)) return fail("split3: buffers must be 2-byte aligned");
+    if (overlaps(outs[i], sec_bytes, A, 3 * sec_bytes)) return fail("split3: an output overlaps the input");
+    for (int j = 0; j < i; ++j)
+      if (overlaps(outs[i], sec_bytes, outs[j], sec_bytes)) return fail("split3: two outputs overlap");
+  }
+  if (!aligned(A, 2)) return fail("split3: buffers must be 2-byte aligned");
+  const bool vec = d % 8 == 0 && aligned(A, 16) && aligned(out0, 16) && aligned(out1, 16) && aligned(out2, 16);
+  const int64_t per_sec = vec ? d / 8 : d;
+  int64_t grid = ceil_div(rows * 3 * per_sec, kBlock);
+  grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (vec)
+    hipLaunchKernelGGL(split3_kernel<u32x4>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const u32x4*>(A),
+                       static_cast<u32x4*>(out0), static_cast<u32x4*>(out1), static_cast<u32x4*>(out2), rows, per_sec);
+  else
+    hipLaunchKernelGGL(split3_kernel<half_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const half_t*>(A),
+                       static_cast<half_t*>(out0), static_cast<half_t*>(out1), static_cast<half_t*>(out2), rows, per_sec);
+  return check_launch("split3");
 }
 }

@@ -563,9 +563,166 @@ int describe_reduction(int op, int64_t rows, int64_t cols, const dtas_config& cf
   return 0;
 }
 
+// softmax_with_temperature (before_dl.py:4154-4161): divide2 (:57-65, logits / temperature, the temperature a
+// device scalar) then softmax2 (:1062-1096), fp32 in and out, over the vocabulary.  One workgroup of 1024 per
+// row; ITERS > 0 keeps the divided row in registers (cols <= 4096 ITERS, cols % 4 == 0, 16-byte aligned rows),
+// ITERS == 0 walks the row three times with element accesses.  exp is the library's (the result stays fp32).
+template <int ITERS>
+__global__ void __launch_bounds__(1024) softmax_temp_kernel(const float* __restrict__ A, const float* __restrict__ temp,
+                                                            float* __restrict__ out, int64_t rows, int64_t cols) {
+  __shared__ float slots[64];
+  int phase = 0;
+  const float t = *temp;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const float* x = A + row * cols;
+    float* o = out + row * cols;
+    if constexpr (ITERS > 0) {
+      f32x4 v[ITERS];
+      float mx = kNegMax;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {   // every load issued before the first use (slots past the row reread its start)
+        const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
+        v[it] = *reinterpret_cast<const f32x4*>(x + (k < cols ? k : 0));
+      }
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
+        if (k < cols) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[it][e] = v[it][e] / t;
+            mx = fmaxf(mx, v[it][e]);
+          }
+        } else {
+          v[it] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        }
+      }
+      mx = block_reduce<MaxOp>(mx, slots, phase);
+      float s = 0.f;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[it][e] = expf(v[it][e] - mx);
+          s += v[it][e];
+        }
+      }
+      s = block_reduce<SumOp>(s, slots, phase);
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
+        if (k < cols) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[it][e] = v[it][e] / s;
+          *reinterpret_cast<f32x4*>(o + k) = v[it];
+        }
+      }
+    } else {
+      float mx = kNegMax;
+      for (int64_t k = threadIdx.x; k < cols; k += blockDim.x) mx = fmaxf(mx, x[k] / t);
+      mx = block_reduce<MaxOp>(mx, slots, phase);
+      float s = 0.f;
+      for (int64_t k = threadIdx.x; k < cols; k += blockDim.x) s += expf(x[k] / t - mx);
+      s = block_reduce<SumOp>(s, slots, phase);
+      for (int64_t k = threadIdx.x; k < cols; k += blockDim.x) o[k] = expf(x[k] / t - mx) / s;
+    }
+  }
+}
+
+// The same result for a few long rows (the model has one row of 50280): a single workgroup spends its time on
+// the two divisions and the exp of every element, so a row is shared by `parts` workgroups of 4096 elements.
+// Every workgroup needs the row's maximum and sum; rather than exchange them it derives them again from the
+// whole row with cheap arithmetic -- max_k(x_k / t) = (max_k x_k) / t for t > 0 ((min_k x_k) / t for t < 0:
+// a correctly rounded division is monotone), and the sum of exp((x_k - x_max) / t) through the hardware's
+// reciprocal and exp2 -- and pays the exact division and the library's exp only on its own 4096 elements.
+// No scratch memory, one launch, the same bits on every run.  cols % 4 == 0, cols <= 4096 ITERS, 16-byte rows.
+template <int ITERS>
+__global__ void __launch_bounds__(1024) softmax_temp_split_kernel(const float* __restrict__ A, const float* __restrict__ temp,
+                                                                  float* __restrict__ out, int64_t cols, int parts) {
+  __shared__ float slots[64];
+  int phase = 0;
+  const float t = *temp;
+  const int64_t row = blockIdx.x / parts;
+  const int part = blockIdx.x % parts;
+  const float* x = A + row * cols;
+  f32x4 v[ITERS];
+  float hi = kNegMax, lo = -kNegMax;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {   // every load issued before the first use (slots past the row reread its start)
+    const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
+    v[it] = *reinterpret_cast<const f32x4*>(x + (k < cols ? k : 0));
+  }
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
+    if (k < cols) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        hi = fmaxf(hi, v[it][e]);
+        lo = fminf(lo, v[it][e]);
+      }
+    }
+  }
+  hi = block_reduce<MaxOp>(hi, slots, phase);
+  lo = -block_reduce<MaxOp>(-lo, slots, phase);
+  const float xm = t < 0.f ? lo : hi;
+  const float mx = fmaxf(kNegMax, xm / t);
+  const float rt = kLog2e * __builtin_amdgcn_rcpf(t);
+  float s = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
+    if (k < cols) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s += __builtin_amdgcn_exp2f((v[it][e] - xm) * rt);
+    }
+  }
+  s = block_reduce<SumOp>(s, slots, phase);
+  const int64_t k = (static_cast<int64_t>(part) * 1024 + threadIdx.x) * 4;
+  if (k < cols) {
+    f32x4 w = *reinterpret_cast<const f32x4*>(x + k);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = expf(w[e] / t - mx) / s;
+    *reinterpret_cast<f32x4*>(out + row * cols + k) = w;
+  }
+}
+
 }  // namespace dtas
 
 extern "C" {
+int dtas_softmax_temperature_f32(const void* logits, const void* temperature, void* out, int64_t rows, int64_t cols,
+                                 void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (rows < 0 || cols < 0) return fail("softmax_temperature: negative extent rows=%lld cols=%lld", (long long)rows, (long long)cols);
+  if (rows == 0 || cols == 0) return 0;
+  if (rows > INT64_MAX / 8 / cols) return fail("softmax_temperature: rows*cols overflows");
+  if (!logits || !temperature || !out) return fail("softmax_temperature: NULL buffer");
+  if (!aligned(logits, 4) || !aligned(temperature, 4) || !aligned(out, 4)) return fail("softmax_temperature: buffers must be 4-byte aligned");
+  if (overlaps(out, rows * cols * 4, logits, rows * cols * 4)) return fail("softmax_temperature: output overlaps the input");
+  const bool vec = cols % 4 == 0 && aligned(logits, 16) && aligned(out, 16) && cols <= 4096 * 16;
+  const unsigned grid = static_cast<unsigned>(rows > int64_t{kNumCU} * 8 ? int64_t{kNumCU} * 8 : rows);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float* x = static_cast<const float*>(logits);
+  const float* t = static_cast<const float*>(temperature);
+  float* o = static_cast<float*>(out);
+  const int64_t parts = ceil_div(cols, 4096);
+  if (vec && parts > 1 && rows * parts <= 2 * kNumCU) {
+    const unsigned wgs = static_cast<unsigned>(rows * parts);
+    if (parts <= 4)
+      hipLaunchKernelGGL(softmax_temp_split_kernel<4>, dim3(wgs), dim3(1024), 0, st, x, t, o, cols, static_cast<int>(parts));
+    else
+      hipLaunchKernelGGL(softmax_temp_split_kernel<16>, dim3(wgs), dim3(1024), 0, st, x, t, o, cols, static_cast<int>(parts));
+  } else if (vec && cols <= 4096)
+    hipLaunchKernelGGL(softmax_temp_kernel<1>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
+  else if (vec && cols <= 4096 * 4)
+    hipLaunchKernelGGL(softmax_temp_kernel<4>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
+  else if (vec)
+    hipLaunchKernelGGL(softmax_temp_kernel<16>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
+  else
+    hipLaunchKernelGGL(softmax_temp_kernel<0>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
+  return check_launch("softmax_temperature");
+}
 int dtas_layer_norm_f32_f16(const void* x, const void* gamma, const void* beta, void* out, int64_t n, int64_t H,
                             float eps, const dtas_config* cfg, void* stream) {
   return dtas::run_reduction(DTAS_OP_LAYER_NORM_F32_F16, x, gamma, beta, out, n, H, eps, cfg, stream);

@@ -261,6 +261,36 @@ def attn_mask(out: torch.Tensor) -> None:
     check(lib().dtas_attn_mask_f16(_p(out), n, m, _stream()), "dtas_attn_mask_f16")
 
 
+def softmax_temperature(logits: torch.Tensor, temperature: torch.Tensor, out: torch.Tensor) -> None:
+    """softmax_with_temperature (dolly-v2-3b-q0f16/before_dl.py:4154-4161): out = softmax(logits / temperature) over
+    the last axis, fp32 in and out; `temperature` is a 0-d (or one-element) fp32 device tensor."""
+    _dev(logits, temperature, out)
+    if logits.dtype != torch.float32 or out.dtype != torch.float32 or temperature.dtype != torch.float32:
+        raise ValueError("softmax_temperature: logits, temperature and out must be fp32")
+    if out.shape != logits.shape or temperature.numel() != 1:
+        raise ValueError("softmax_temperature: out must have the logits' shape and temperature one element")
+    rows, cols = _rows_cols(logits)
+    check(lib().dtas_softmax_temperature_f32(_p(logits), _p(temperature), _p(out), rows, cols, _stream()),
+          "dtas_softmax_temperature_f32")
+
+
+def split3(A: torch.Tensor, out0: torch.Tensor, out1: torch.Tensor, out2: torch.Tensor) -> None:
+    """split / fused_reshape7_split1 (dolly-v2-3b-q0f16/before_dl.py:1099-1125, :661-688): A (..., 3 d) fp16 cut into
+    three (..., d) buffers along the last axis."""
+    _dev(A, out0, out1, out2)
+    d3 = A.shape[-1]
+    if d3 % 3 != 0:
+        raise ValueError("split3: the last extent must be a multiple of 3")
+    d = d3 // 3
+    rows = A.numel() // d3 if d3 else 0
+    for o in (out0, out1, out2):
+        if o.dtype != torch.float16 or o.shape[-1] != d or o.numel() != rows * d:
+            raise ValueError("split3: each output must be fp16 (..., d) with A's leading extents")
+    if A.dtype != torch.float16:
+        raise ValueError("split3: A must be fp16")
+    check(lib().dtas_split3_f16(_p(A), _p(out0), _p(out1), _p(out2), rows, d, _stream()), "dtas_split3_f16")
+
+
 def swap_axes(A: torch.Tensor, out: torch.Tensor) -> None:
     """out (..., b, a, d) = A (..., a, b, d) with leading extents of 1, fp16: transpose6 / transpose7
     (dolly-v2-3b-q0f16/before_dl.py:1177-1203)."""

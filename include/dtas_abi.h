@@ -173,6 +173,11 @@ int dtas_softmax_f32_f16(const void* A, void* out, int64_t rows, int64_t cols,
                          const dtas_config* cfg, void* stream);
 int dtas_softmax_f16(const void* A, void* out, int64_t rows, int64_t cols, const dtas_config* cfg,
                      void* stream);
+/* softmax_with_temperature (before_dl.py:4154-4161): divide2 (:57-65) then softmax2 (:1062-1096).
+ * out[rows, cols] fp32 = softmax over each row of logits[rows, cols] / *temperature; `temperature` points at
+ * one fp32 in device memory (the PrimFunc's 0-d buffer B). */
+int dtas_softmax_temperature_f32(const void* logits, const void* temperature, void* out, int64_t rows,
+                                 int64_t cols, void* stream);
 
 /* take (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:1151-1163; one row: take1, :1166-1174), the
  * embedding lookup: out[n, H] = A[ids[i], :] for a table A[V, H] fp16 and ids[n] int32 (n dynamic).  Ids
@@ -195,6 +200,9 @@ int dtas_attn_mask_f16(void* out, int64_t n, int64_t m, void* stream);
 /* transpose6 / transpose7 (before_dl.py:1177-1203): A[a, b, d] -> out[b, a, d] fp16, rows of d elements
  * (d % 8 == 0) moved whole: [n, heads, d] <-> [heads, n, d] around the attention kernels. */
 int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d, void* stream);
+/* split (before_dl.py:1099-1125) and fused_reshape7_split1 (:661-688): the fused projection A[rows, 3 d] fp16
+ * (rows = positions x heads) cut into out0 / out1 / out2 [rows, d], section s = columns [s d, (s + 1) d). */
+int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t rows, int64_t d, void* stream);
 
 /* ---- GEMV: fused_NT_matmul10_add5 (before_dl.py:96-113) ------------------
  * y[N] = W[N,K] . x[K] (+ bias[N] when bias != NULL); fp16 in/out, fp32 accumulate. */

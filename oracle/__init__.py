@@ -63,6 +63,7 @@ class _C:
                 "oracle_rms_norm_f16": [vp, vp, vp, i64, i64, f32, ci],
                 "oracle_softmax_f32_f16": [vp, vp, i64, i64, ci],
                 "oracle_softmax_f16_f16": [vp, vp, i64, i64, ci],
+                "oracle_softmax_temperature_f32": [vp, vp, vp, i64, i64, ci],
                 "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
@@ -141,6 +142,15 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         out = np.empty(x.shape, dtype=np.float16)
         fn = {"float16": "oracle_softmax_f16_f16", "float32": "oracle_softmax_f32_f16"}[x.dtype.name]
         getattr(_C.lib(), fn)(_ptr(x), _ptr(out), x.size // max(cols, 1), cols, threads)
+        return out
+
+    @staticmethod
+    def softmax_temperature(x, temperature: float, threads: int = 1) -> np.ndarray:
+        assert x.dtype == np.float32
+        cols = x.shape[-1]
+        t = np.array([temperature], dtype=np.float32)
+        out = np.empty(x.shape, dtype=np.float32)
+        _C.lib().oracle_softmax_temperature_f32(_ptr(x), _ptr(t), _ptr(out), x.size // max(cols, 1), cols, threads)
         return out
 
     @staticmethod
@@ -280,6 +290,13 @@ class layout:
         elsewhere; n = 1 is full (:83-93)."""
         i, j = np.arange(n)[:, None], np.arange(m)[None, :]
         return np.where(j - (m - n) > i, np.float16(-65504), np.float16(65504)).astype(np.float16)
+
+    @staticmethod
+    def split3(a: np.ndarray):
+        """split (before_dl.py:1099-1125) / fused_reshape7_split1 (:661-688): section s of the last axis is
+        A[..., s d : (s + 1) d]."""
+        d = a.shape[-1] // 3
+        return tuple(np.ascontiguousarray(a[..., s_ * d:(s_ + 1) * d]) for s_ in range(3))
 
     @staticmethod
     def swap_axes(a: np.ndarray) -> np.ndarray:

@@ -198,6 +198,32 @@ void oracle_softmax_f32_f16(const float* x, f16* out, int64_t rows, int64_t cols
   }
 }
 
+/* softmax_with_temperature: experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:4154-4161 = divide2 (:57-65,
+ * A / B[()] in fp32) then softmax2 (:1062-1096: max from -FLT_MAX, exp(x - max), sequential sum, exp / sum;
+ * fp32 throughout).
+ * Pinned by: fp64 numpy softmax(x / t), rows sum to 1, temperature 1 equals the plain softmax of the row,
+ * a single column gives exactly 1.0. */
+void oracle_softmax_temperature_f32(const float* x, const float* temperature, float* out, int64_t rows, int64_t cols,
+                                    int nthreads) {
+  const float t = *temperature;
+  OMP_FOR(nthreads)
+  for (int64_t r = 0; r < rows; ++r) {
+    const float* xr = x + r * cols;
+    float* o = out + r * cols;
+    float mx = -3.4028234663852886e+38f;
+    for (int64_t k = 0; k < cols; ++k) {
+      o[k] = xr[k] / t;
+      mx = o[k] > mx ? o[k] : mx;
+    }
+    float s = 0.f;
+    for (int64_t k = 0; k < cols; ++k) {
+      o[k] = expf(o[k] - mx);
+      s = s + o[k];
+    }
+    for (int64_t k = 0; k < cols; ++k) o[k] = o[k] / s;
+  }
+}
+
 /* Same PrimFunc with an fp16 input buffer (the [32n, n] attention-score form):
  * the values are widened to fp32 first, then the identical fp32 pipeline. */
 void oracle_softmax_f16_f16(const f16* x, f16* out, int64_t rows, int64_t cols, int nthreads) {

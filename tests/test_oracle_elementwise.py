@@ -193,3 +193,17 @@ def test_swap_axes_follows_the_index_expression(oracle):
     for i1 in range(3):
         for i2 in range(5):
             assert np.array_equal(t[0, i1, i2].view(np.uint16), a[0, i2, i1].view(np.uint16))
+
+
+def test_split3_follows_the_index_expression(oracle):
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 2 ** 16, (1, 4, 32, 240), dtype=np.uint16).view(np.float16)
+    outs = oracle.layout.split3(a)
+    assert all(o.shape == (1, 4, 32, 80) and o.flags.c_contiguous for o in outs)
+    for sec, off in enumerate((0, 80, 160)):                 # T_split_sections_s[.., ax3] = A[.., ax3 + 80 s]
+        for ax3 in (0, 1, 79):
+            assert np.array_equal(outs[sec][..., ax3].view(np.uint16), a[..., ax3 + off].view(np.uint16))
+    # the decode form reads the flat [1, 1, 7680] projection: same bytes, reshaped to heads x 240 first
+    flat = a[:, :1].reshape(1, 1, 7680)
+    again = oracle.layout.split3(flat.reshape(1, 1, 32, 240))
+    assert np.array_equal(again[1].view(np.uint16), outs[1][:, :1].view(np.uint16))

@@ -99,3 +99,29 @@ def test_softmax_invariants(oracle):
     assert np.isfinite(out).all() and abs(out[0, 0] - 1 / (1 + np.exp(-1))) < 1e-3 and out[0, 2] == 0
     # rows are independent: permuting rows permutes outputs
     assert np.array_equal(oracle.c.softmax(x[::-1].copy()), oracle.c.softmax(x)[::-1])
+
+
+@pytest.mark.parametrize("cols,t", [(1, 0.7), (5, 1.0), (1000, 0.7), (50280, 0.7), (50280, 1.3)])
+def test_softmax_temperature_closed_form_and_scipy(oracle, cols, t):
+    rng = np.random.default_rng(cols)
+    x = (rng.standard_normal((2, cols)) * 4).astype(np.float32)
+    got = oracle.c.softmax_temperature(x, t)
+    assert got.dtype == np.float32
+    want = scipy_softmax(x.astype(np.float64) / float(np.float32(t)), axis=-1)
+    # the sum runs in fp32 in the PrimFunc's order: its rounding (a common factor of each row) grows with the row length
+    assert np.abs(got - want).max() < 1e-4 and np.abs(got / want - 1).max() < 1e-3
+    assert np.abs(got.astype(np.float64).sum(-1) - 1).max() < 1e-3
+
+
+def test_softmax_temperature_invariants(oracle):
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((3, 777)) * 3).astype(np.float32)
+    # temperature 1 divides by exactly 1: the plain fp32 softmax, whose fp16 rounding is the other oracle function
+    one = oracle.c.softmax_temperature(x, 1.0)
+    assert np.array_equal(one.astype(np.float16), oracle.c.softmax(x))
+    # a division, not a product: t = 0.5 doubles the logits exactly
+    assert np.array_equal(oracle.c.softmax_temperature(x, 0.5), oracle.c.softmax_temperature(x * np.float32(2), 1.0))
+    # a lower temperature sharpens: the largest probability grows
+    assert (oracle.c.softmax_temperature(x, 0.5).max(-1) > one.max(-1)).all()
+    assert (oracle.c.softmax_temperature(np.array([[2.5]], np.float32), 0.3) == np.float32(1)).all()
+    assert np.array_equal(np.argmax(one, -1), np.argmax(x, -1))

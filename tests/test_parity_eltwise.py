@@ -307,3 +307,33 @@ def test_mask_and_swap_errors():
     x = torch.zeros(2, 3, 8, dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.DtasError, match="overlaps"):
         _lib.check(L.dtas_swap_axes_f16(x.data_ptr(), x.data_ptr(), 2, 3, 8, None), "swap")
+
+
+@pytest.mark.parametrize("lead,d", [((1, 1, 32), 80), ((1, 300, 32), 80), ((1, 4096, 32), 80), ((7,), 3), ((33, 5), 12)])
+def test_split3_is_exact(oracle, lead, d):
+    rng = np.random.default_rng(d + len(lead))
+    x = rng.integers(0, 2 ** 16, lead + (3 * d,), dtype=np.uint16).view(np.float16)
+    outs = [Guarded(lead + (d,), torch.float16) for _ in range(3)]
+    ops.split3(dev(x), *[o.t for o in outs])
+    for o, want in zip(outs, oracle.layout.split3(x)):
+        assert_bits_equal(o.check(), want)
+
+
+def test_split3_misaligned_and_errors(oracle):
+    rng = np.random.default_rng(9)
+    x = rng.integers(0, 2 ** 16, (50, 240), dtype=np.uint16).view(np.float16)
+    raw = torch.empty(50 * 240 + 1, dtype=torch.float16, device="cuda")
+    xd = raw[1:].view(50, 240)                                               # 2-byte aligned: element accesses
+    xd.copy_(dev(x))
+    outs = [Guarded((50, 80), torch.float16) for _ in range(3)]
+    ops.split3(xd, *[o.t for o in outs])
+    for o, want in zip(outs, oracle.layout.split3(x)):
+        assert_bits_equal(o.check(), want)
+    L = _lib.lib()
+    assert L.dtas_split3_f16(None, None, None, None, 0, 80, None) == 0
+    assert L.dtas_split3_f16(None, None, None, None, 4, 80, None) == -1 and b"NULL" in L.dtas_last_error()
+    o = outs[0].t
+    with pytest.raises(_lib.DtasError, match="overlap"):
+        _lib.check(L.dtas_split3_f16(xd.data_ptr(), o.data_ptr(), o.data_ptr(), outs[2].t.data_ptr(), 50, 80, None), "split3")
+    with pytest.raises(ValueError):
+        ops.split3(xd[:, :239], *[o.t for o in outs])

@@ -243,3 +243,38 @@ def test_reduction_errors():
         ops.rms_norm(x, w, x)
     with pytest.raises(_lib.DtasError, match="block must be"):
         ops.rms_norm(x, w, torch.empty_like(x), cfg=cfg(variant=_lib.RED_STREAM_ROW, block=100, vec=1))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 50280), (1, 1), (3, 4096), (2, 4100), (5, 16384), (2, 50281), (1, 65540), (4, 100000),
+                                       (700, 64)])
+@pytest.mark.parametrize("t", [0.7, 1.0, -0.8])
+def test_softmax_temperature(oracle, rows, cols, t):
+    rng = np.random.default_rng(rows * 7 + cols)
+    x = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
+    out = Guarded(x.shape, torch.float32)
+    ops.softmax_temperature(dev(x), torch.tensor(t, dtype=torch.float32, device="cuda"), out.t)
+    got = out.check().astype(np.float64)
+    want = oracle.c.softmax_temperature(x, t, threads=8).astype(np.float64)
+    assert np.abs(got - want).max() < 1e-2                                   # the stated tolerance of the reductions
+    # the oracle sums the row in fp32 in index order, the kernel as a tree: both within fp32 summation error of the fp64 row
+    assert np.abs(got / np.maximum(want, 1e-300) - 1)[want > 1e-30].max() < 1e-3
+    want64 = oracle.np64.softmax(x.astype(np.float64) / float(np.float32(t)))
+    assert np.abs(got / want64 - 1)[want64 > 1e-30].max() < 3e-5
+    assert np.abs(got.sum(-1) - 1).max() < 1e-4
+    assert np.array_equal(got.argmax(-1), (x if t > 0 else -x).argmax(-1))
+
+
+def test_softmax_temperature_unaligned_and_errors(oracle):
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal(50280 + 1) * 4).astype(np.float32)
+    xd = dev(x)[1:]                                                          # 4-byte aligned only: the element path
+    out = Guarded((50280,), torch.float32)
+    ops.softmax_temperature(xd, torch.tensor([0.9], dtype=torch.float32, device="cuda"), out.t)
+    want = oracle.c.softmax_temperature(x[1:].copy(), 0.9)
+    assert np.abs(out.check() - want).max() < 1e-4
+    L = _lib.lib()
+    assert L.dtas_softmax_temperature_f32(None, None, None, 0, 9, None) == 0
+    assert L.dtas_softmax_temperature_f32(None, None, None, 1, 9, None) == -1 and b"NULL" in L.dtas_last_error()
+    assert L.dtas_softmax_temperature_f32(None, None, None, -1, 9, None) == -1 and b"negative" in L.dtas_last_error()
+    with pytest.raises(ValueError):
+        ops.softmax_temperature(xd, torch.tensor(0.9, dtype=torch.float16, device="cuda"), out.t)
