@@ -365,27 +365,30 @@ __global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restri
 // extended to m >= n key positions by extend_te (:68-80: 65504 for the m - n positions already cached, the
 // triangle after them) -- and, with n = 1, full (:83-93).  out[i, j] = (j - (m - n) > i) ? -65504 : 65504.
 // A thread writes 8 consecutive elements of the flat [n * m] array (16-byte stores whatever m is).
-__global__ void __launch_bounds__(kBlock) attn_mask_kernel(half_t* __restrict__ out, int64_t n, int64_t m) {
-  const int64_t total = n * m, shift = m - n;
-  for (int64_t t = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 8; t < total;
-       t += static_cast<int64_t>(gridDim.x) * blockDim.x * 8) {
-    int64_t i = t / m, jj = t % m;
+// I = the index type: 32-bit while n * m fits (a 64-bit division costs more than the eight stores it places).
+template <typename I>
+__global__ void __launch_bounds__(kBlock) attn_mask_kernel(half_t* __restrict__ out, I n, I m, I total) {
+  const I shift = m - n;
+  const I step = static_cast<I>(gridDim.x) * kBlock * 8;
+  for (I t = (static_cast<I>(blockIdx.x) * kBlock + threadIdx.x) * 8; t < total; t += step) {
+    I i = t / m, jj = t - i * m;
     f16x8 v;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      v[e] = static_cast<half_t>(jj - shift > i ? -65504.f : 65504.f);
+      v[e] = static_cast<half_t>(jj > i + shift ? -65504.f : 65504.f);
       if (++jj == m) {
         jj = 0;
         ++i;
       }
     }
-    if (t + 8 <= total) {
-      *reinterpret_cast<u32x4*>(out + t) = __builtin_bit_cast(u32x4, v);
+    if (total - t >= 8) {
+      __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(out + t));
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        if (t + e < total) out[t + e] = v[e];
+        if (e < total - t) out[t + e] = v[e];
     }
+    if (total - t <= step) break;   // t + step would pass total (and, in 32 bits, might wrap)
   }
 }
 
@@ -550,8 +553,13 @@ int dtas_attn_mask_f16(void* out, int64_t n, int64_t m, void* stream) {
   if (!aligned(out, 16)) return fail("attn_mask: the output must be 16-byte aligned");
   int64_t grid = ceil_div(ceil_div(n * m, 8), kBlock);
   grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
-  hipLaunchKernelGGL(attn_mask_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
-                     static_cast<half_t*>(out), n, m);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n * m + 8 < (int64_t{1} << 31))   // + 8: the last thread's t stays below 2^31 as well
+    hipLaunchKernelGGL(attn_mask_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<half_t*>(out),
+                       static_cast<uint32_t>(n), static_cast<uint32_t>(m), static_cast<uint32_t>(n * m));
+  else
+    hipLaunchKernelGGL(attn_mask_kernel<int64_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<half_t*>(out),
+                       n, m, n * m);
   return check_launch("attn_mask");
 }
 int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d, void* stream) {

@@ -289,6 +289,20 @@ def test_attn_mask_is_exact(oracle, n, m):
     assert_bits_equal(out.check().reshape(n, m), oracle.layout.attn_mask(n, m))
 
 
+def test_attn_mask_beyond_32_bit_indices():
+    # n * m >= 2^31: the 64-bit index path, checked on the device block of rows by block of rows (the property
+    # out[i, j] == (j - (m - n) > i ? -65504 : 65504) itself, evaluated by torch)
+    n, m = 32768, 65537
+    out = torch.empty(n, m, dtype=torch.float16, device="cuda")
+    ops.attn_mask(out.view(1, 1, n, m))
+    j = torch.arange(m, device="cuda")[None, :]
+    for lo in range(0, n, 4096):
+        i = torch.arange(lo, lo + 4096, device="cuda")[:, None]
+        want = torch.where(j - (m - n) > i, -65504.0, 65504.0).half()
+        assert torch.equal(out[lo:lo + 4096], want), f"rows {lo}.."
+    del out
+
+
 @pytest.mark.parametrize("a,b,d", [(1, 32, 80), (300, 32, 80), (32, 300, 80), (4096, 32, 80), (5, 3, 8)])
 def test_swap_axes_is_exact(oracle, a, b, d):
     rng = np.random.default_rng(a + b)
