@@ -213,6 +213,42 @@ def take(V: int = 50280, H: int = 2560, decode: bool = False, name: Optional[str
     return PrimFunc(name or ("take1" if decode else "take"), params, blocks, op="take", attrs={"tir.noalias": True})
 
 
+def split(heads: int = 32, d: int = 80, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """The fused projection cut into queries, keys and values, section s = columns [s d, (s + 1) d) of every head:
+    split (dolly-v2-3b-q0f16/before_dl.py:1099-1125; A (1, n, heads, 3 d), n dynamic) or, with ``decode``,
+    fused_reshape7_split1 (:661-688; A (1, 1, heads * 3 d), reshaped first).  Parameters: A and the three sections."""
+    n = 1 if decode else "n"
+    a_shape = (1, 1, heads * 3 * d) if decode else (1, n, heads, 3 * d)
+    outs = ["T_split_sections", "T_split_sections_1", "T_split_sections_2"]
+    params = [Buffer("A", a_shape, "float16")] + [Buffer(o, (1, n, heads, d), "float16") for o in outs]
+    blocks = [Block(o, "SSSS", ["A"], [o]) for o in outs]
+    return PrimFunc(name or ("fused_reshape7_split1" if decode else "split"), params, blocks, op="split3",
+                    attrs={"tir.noalias": True, "heads": heads, "d": d})
+
+
+def transpose(heads: int = 32, d: int = 80, back: bool = False, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
+    """T_transpose(1, heads, n, d) = A(1, n, heads, d): transpose6 (dolly-v2-3b-q0f16/before_dl.py:1177-1189) or, with
+    ``back``, transpose7 (:1192-1203; (1, heads, n, d) -> (1, n, heads, d)); ``decode``: transpose8 (:1205-1213, n = 1)."""
+    n = 1 if decode else "n"
+    src, dst = ((1, heads, n, d), (1, n, heads, d)) if back else ((1, n, heads, d), (1, heads, n, d))
+    params = [Buffer("A", src, "float16"), Buffer("T_transpose", dst, "float16")]
+    blocks = [Block("T_transpose", "SSSS", ["A"], ["T_transpose"])]
+    return PrimFunc(name or ("transpose8" if decode else "transpose7" if back else "transpose6"), params, blocks, op="swap_axes",
+                    attrs={"tir.noalias": True})
+
+
+def softmax_with_temperature(V: int = 50280, name: Optional[str] = None) -> PrimFunc:
+    """T_softmax_norm(1, 1, V) = softmax(A(1, 1, V) / B()), fp32: divide2 (dolly-v2-3b-q0f16/before_dl.py:57-65) and
+    softmax2 (:1062-1096) as the graph's softmax_with_temperature chains them (:4154-4161).  Parameters: A (the
+    logits), B (the temperature, a 0-d buffer), T_softmax_norm."""
+    params = [Buffer("A", (1, 1, V), "float32"), Buffer("B", (), "float32"), Buffer("T_softmax_norm", (1, 1, V), "float32")]
+    blocks = [Block("T_divide", "SSS", ["A", "B"], ["T_divide"]), Block("T_softmax_maxelem", "SSR", ["T_divide"], ["T_softmax_maxelem"]),
+              Block("T_softmax_exp", "SSS", ["T_divide", "T_softmax_maxelem"], ["T_softmax_exp"]),
+              Block("T_softmax_expsum", "SSR", ["T_softmax_exp"], ["T_softmax_expsum"]),
+              Block("T_softmax_norm", "SSS", ["T_softmax_exp", "T_softmax_expsum"], ["T_softmax_norm"])]
+    return PrimFunc(name or "softmax_with_temperature", params, blocks, op="softmax_temperature", attrs={"tir.noalias": True})
+
+
 def fused_decode_take(V: int = 50280, K: int = 2560, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
     """out(n,K) fp16 = rows ids(n) of the dequantised table: fused_fused_decode1_take1
     (dolly-v2-3b-q8f16_1/before_dl.py:357-369; n dynamic) or, with ``decode``, fused_fused_decode1_take (:346-355;

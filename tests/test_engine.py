@@ -118,6 +118,25 @@ def test_bind_extents_checks_the_signature():
         bind_extents(f, [a, a, torch.zeros(1, 6, 64, dtype=torch.float16)])
 
 
+def test_layout_and_sampling_descriptors_follow_the_graph_signatures():
+    from dtas_amd.codegen.runtime_packer import LIBRARY_CHOSEN_OPS
+
+    sp = pf.split()
+    assert sp.name == "split" and [p.shape for p in sp.params] == [(1, "n", 32, 240)] + [(1, "n", 32, 80)] * 3
+    a, o = torch.zeros(1, 6, 32, 240, dtype=torch.float16), torch.zeros(1, 6, 32, 80, dtype=torch.float16)
+    assert bind_extents(sp, [a, o, o, o]) == {"n": 6}
+    dec = pf.split(decode=True)
+    assert dec.name == "fused_reshape7_split1" and dec.params[0].shape == (1, 1, 7680) and dec.params[1].shape == (1, 1, 32, 80)
+    t6, t7, t8 = pf.transpose(), pf.transpose(back=True), pf.transpose(decode=True)
+    assert (t6.name, t7.name, t8.name) == ("transpose6", "transpose7", "transpose8")
+    assert t6.params[0].shape == t7.params[1].shape == (1, "n", 32, 80) and t6.params[1].shape == t7.params[0].shape == (1, 32, "n", 80)
+    assert t8.params[0].shape == (1, 1, 32, 80) and t8.params[1].shape == (1, 32, 1, 80)
+    sm = pf.softmax_with_temperature()
+    assert [p.shape for p in sm.params] == [(1, 1, 50280), (), (1, 1, 50280)] and all(p.dtype == "float32" for p in sm.params)
+    assert bind_extents(sm, [torch.zeros(1, 1, 50280), torch.tensor(0.7), torch.zeros(1, 1, 50280)]) == {}
+    assert all(f.op in LIBRARY_CHOSEN_OPS for f in (sp, dec, t6, t7, t8, sm))
+
+
 def test_cpu_tensors_are_refused_not_computed_elsewhere():
     from dtas_amd import ops
 

@@ -152,6 +152,39 @@ def test_decode_forms_of_the_fused_matmuls_go_through_the_gemv_rule(tmp_path, or
         assert (np.abs(out2.cpu().numpy()[0].astype(np.float64) - want) <= 4e-3 + 1e-2 * np.abs(want)).all()
 
 
+def test_layout_and_sampling_primfuncs_through_the_module(tmp_path, oracle):
+    """split / fused_reshape7_split1, transpose6 / 7 / 8 and softmax_with_temperature: served by the library's own choice."""
+    funcs = [pf.split(), pf.split(decode=True), pf.transpose(), pf.transpose(back=True), pf.transpose(decode=True),
+             pf.softmax_with_temperature()]
+    work_dir = str(tmp_path / "layout")
+    rt = Engine(topk=2, parallel_build=False, work_dir=work_dir).tune_module(pf.module(*funcs), arch=MI355X(0, require_device=True))
+    rng = np.random.default_rng(12)
+    t = lambda a: torch.from_numpy(a).cuda()
+    bits = lambda x: x.cpu().numpy().view(np.uint16)
+    for mod in (rt, load_module_from_file(work_dir)):
+        for name, n in (("split", 37), ("fused_reshape7_split1", 1)):
+            a = rng.integers(0, 2 ** 16, (1, n, 32, 240), dtype=np.uint16).view(np.float16)
+            outs = [torch.empty(1, n, 32, 80, dtype=torch.float16, device="cuda") for _ in range(3)]
+            mod[name](t(a if n > 1 else a.reshape(1, 1, 7680)), *outs)
+            for got, want in zip(outs, oracle.layout.split3(a)):
+                assert np.array_equal(bits(got), want.view(np.uint16))
+        a = rng.integers(0, 2 ** 16, (1, 21, 32, 80), dtype=np.uint16).view(np.float16)
+        out = torch.empty(1, 32, 21, 80, dtype=torch.float16, device="cuda")
+        mod["transpose6"](t(a), out)
+        assert np.array_equal(bits(out), oracle.layout.swap_axes(a).view(np.uint16))
+        back = torch.empty(1, 21, 32, 80, dtype=torch.float16, device="cuda")
+        mod["transpose7"](out, back)
+        assert np.array_equal(bits(back), a.view(np.uint16))
+        one = torch.empty(1, 32, 1, 80, dtype=torch.float16, device="cuda")
+        mod["transpose8"](t(a[:, :1].copy()), one)
+        assert np.array_equal(bits(one).reshape(32, 80), a[0, 0].view(np.uint16))
+        logits = (rng.standard_normal((1, 1, 50280)) * 4).astype(np.float32)
+        probs = torch.empty(1, 1, 50280, dtype=torch.float32, device="cuda")
+        mod["softmax_with_temperature"](t(logits), torch.tensor(0.8, dtype=torch.float32, device="cuda"), probs)
+        want = oracle.c.softmax_temperature(logits, 0.8)
+        assert np.abs(probs.cpu().numpy() - want).max() < 1e-2 and np.abs(probs.cpu().numpy() / want - 1).max() < 1e-3
+
+
 def test_profile_sweep_writes_the_reference_file_format(tmp_path):
     """tune -> reload from the work_dir -> sweep: latency.json / bandwidth.json as the reference's profile scripts
     write them ({"<n>": us}, {"<n>": GiB/s}; experiment/dtas_tuned/elementwise/add/profile_add.py)."""
