@@ -646,26 +646,22 @@ __global__ void __launch_bounds__(1024) softmax_temp_split_kernel(const float* _
   const int part = blockIdx.x % parts;
   const float* x = A + row * cols;
   f32x4 v[ITERS];
-  float hi = kNegMax, lo = -kNegMax;
+  float hi = kNegMax;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {   // every load issued before the first use (slots past the row reread its start)
     const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
     v[it] = *reinterpret_cast<const f32x4*>(x + (k < cols ? k : 0));
   }
+  const float sign = t < 0.f ? -1.f : 1.f;   // the extreme that the division turns into the maximum: max x for t > 0, min x for t < 0
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int64_t k = (static_cast<int64_t>(it) * 1024 + threadIdx.x) * 4;
     if (k < cols) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        hi = fmaxf(hi, v[it][e]);
-        lo = fminf(lo, v[it][e]);
-      }
+      for (int e = 0; e < 4; ++e) hi = fmaxf(hi, sign * v[it][e]);
     }
   }
-  hi = block_reduce<MaxOp>(hi, slots, phase);
-  lo = -block_reduce<MaxOp>(-lo, slots, phase);
-  const float xm = t < 0.f ? lo : hi;
+  const float xm = sign * block_reduce<MaxOp>(hi, slots, phase);
   const float mx = fmaxf(kNegMax, xm / t);
   const float rt = kLog2e * __builtin_amdgcn_rcpf(t);
   float s = 0.f;
