@@ -1775,43 +1775,63 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   dtas_config cfg;
   if (user) {
     cfg = *user;
-  } else if (n <= 12 && v_vec) {
-    // a handful of rows (decoding): the row kernel, two rows per workgroup (measured best for 2..8
-    // rows: more rows per workgroup mean fewer workgroups than the 256 CUs want)
-    cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : 2, 8, 0}, 1, 0};
   } else {
-    // what this op moves is P (2*n*m bytes per head).  Measured over n = m = 128 .. 4096 with 32 heads of 80:
-    // 64-row tiles while 128-row tiles would leave most CUs idle; 128-row tiles with three stages up to
-    // one per CU; 256-row tiles with three stages beyond (n = m = 1280: 37 us against 44 for 128x128
-    // with three stages and 61 with two; 2048: 74 / 79 / 98).  Head dimensions up to 64 keep the
-    // 64-column tiles: two workgroups of two stages per CU
-    const int64_t t128 = heads * ceil_div(n, 128);
-    const int bn = d <= 64 ? 64 : 128;
-    if (t128 <= kNumCU / 4) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, bn, kBK}, 1, 0};
-    else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
-    else if (bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
-    else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
     // Fewer workgroups than CUs and many keys: the workgroups of a tile split m.  Fitted to measurements at
     // 13 .. 256 rows against 512 .. 8192 keys: a k tile costs a workgroup ~0.8 us, combining S partial tiles
-    // ~3 / 5.5 / 10 us for S = 2 / 4 / 8 (16 loses everywhere).
-    const int64_t wgs = heads * ceil_div(n, cfg.tile[0]), ktiles = ceil_div(m, kBK);
-    // 128-row tiles (one workgroup per CU) gain only while all parts run at once: 512 rows against 4096 keys
-    // take 47 us in two parts, 58 whole, 80 in eight.  Partial tiles of 256 rows cost more to combine than a
-    // split saves.
-    const int64_t wg_limit = cfg.tile[0] <= 64 ? 4 * kNumCU : kNumCU;
-    if (wgs < kNumCU && cfg.tile[0] <= 128) {
+    // ~3 / 5.5 / 10 us for S = 2 / 4 / 8 (16 loses everywhere).  Returns the split and its estimate in us.
+    auto key_split = [](int64_t wgs, int64_t wg_limit, int64_t ktiles, double* us) {
       const double combine[4] = {0.0, 3.0, 5.5, 10.0};
       const double whole = 0.8 * static_cast<double>(ktiles);
       double best = 0.8 * whole;  // (a split has to promise a fifth less: the fit is coarse)
+      int chosen = 1;
       for (int i = 1; i < 4; ++i) {
         const int split = 1 << i;
         if (wgs * split > wg_limit || ktiles < 2 * split) break;
         const double t = 0.8 * static_cast<double>(ceil_div(ktiles, split)) + combine[i];
         if (t < best) {
           best = t;
-          cfg.split_k = split;
+          chosen = split;
         }
       }
+      *us = chosen == 1 ? whole : best;
+      return chosen;
+    };
+    const int64_t ktiles = ceil_div(m, kBK);
+    const int bn = d <= 64 ? 64 : 128;
+    bool rows = false;
+    if (n <= 12 && v_vec) {
+      // a handful of rows (decoding, short continuations): the row kernel (two rows per workgroup, four when the
+      // keys are many: ~4.5 + 0.7 n m / 1000 us and ~6 + 0.4 n m / 1000 us, measured at n = 2 .. 12 against 512 ..
+      // 4096 keys) unless the 64-row MFMA tiles with their keys split come out ahead (from ~8 rows against 4096
+      // keys, ~12 against 512: 15 us against 25 at n = 8, m = 4096); P's rows must be fetchable in 16-byte pieces
+      const double nm = 1e-3 * static_cast<double>(n) * static_cast<double>(m);
+      const double r2 = 4.5 + 0.7 * nm, r4 = n >= 4 ? 6.0 + 0.4 * nm : 1e30;
+      double mfma_us = 1e30;
+      if (n >= 2 && p_vec) {
+        key_split(heads, 4 * kNumCU, ktiles, &mfma_us);
+        mfma_us += 1.5;
+      }
+      rows = mfma_us >= (r2 < r4 ? r2 : r4);
+      if (rows) cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : r4 < r2 ? 4 : 2, 8, 0}, 1, 0};
+    }
+    if (!rows) {
+      // what this op moves is P (2*n*m bytes per head).  Measured over n = m = 128 .. 4096 with 32 heads of 80:
+      // 64-row tiles while 128-row tiles would leave most CUs idle; 128-row tiles with three stages up to
+      // one per CU; 256-row tiles with three stages beyond (n = m = 1280: 37 us against 44 for 128x128
+      // with three stages and 61 with two; 2048: 74 / 79 / 98).  Head dimensions up to 64 keep the
+      // 64-column tiles: two workgroups of two stages per CU
+      const int64_t t128 = heads * ceil_div(n, 128);
+      if (t128 <= kNumCU / 4) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, bn, kBK}, 1, 0};
+      else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
+      else if (bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
+      else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
+      // 128-row tiles (one workgroup per CU) gain only while all parts run at once: 512 rows against 4096 keys
+      // take 47 us in two parts, 58 whole, 80 in eight.  Partial tiles of 256 rows cost more to combine than a
+      // split saves.
+      const int64_t wgs = heads * ceil_div(n, cfg.tile[0]);
+      const int64_t wg_limit = cfg.tile[0] <= 64 ? 4 * kNumCU : kNumCU;
+      double us;
+      if (wgs < kNumCU && cfg.tile[0] <= 128) cfg.split_k = key_split(wgs, wg_limit, ktiles, &us);
     }
   }
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_SKINNY && !v_vec) cfg.vec = 1;

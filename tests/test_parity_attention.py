@@ -152,6 +152,17 @@ def test_pv_row_kernel(oracle, rows, heads, n, m, d):
     _check_pv(out.check(), p, v, oracle)
 
 
+@pytest.mark.parametrize("n", [2, 4, 5, 8, 12])
+@pytest.mark.parametrize("m", [512, 1024, 4096, 4097])
+def test_pv_few_rows_builtin_choice(oracle, n, m):
+    # 2 .. 12 query rows: two- or four-row workgroups of the row kernel, or 64-row MFMA tiles with the keys split
+    # (m = 4097: P's rows are not fetchable in 16-byte pieces, which keeps the row kernel)
+    p, v = _pv_inputs(32, n, m, 80, n + m)
+    out = Guarded((32, n, 80), torch.float16)
+    ops.attn_pv(dev(p), dev(v), out.t)
+    _check_pv(out.check(), p, v, oracle)
+
+
 def test_pv_selector_rows_are_exact_and_edge_cases(oracle):
     # P = identity picks the rows of V: any operand mix-up (a transposed V, a shifted k) shows as wrong bits
     rng = np.random.default_rng(5)
