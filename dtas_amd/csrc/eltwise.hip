@@ -317,24 +317,27 @@ __global__ void __launch_bounds__(kBlock) rotary_f16_kernel(const half_t* __rest
 // piece of the rotated part finds its partners with one or two more 16-byte loads at the elements' alignment
 // (piece 0: elements 10..17 negated; piece 1: 18, 19 negated, then 0..5; piece 2: 6..9) and its part of the
 // tables' row with 8-byte loads (a table row is 40 bytes).
+// I = the index type: 32-bit while the piece count fits (shorter index arithmetic; the time is the same at n = 4096).
+template <typename I>
 __global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restrict__ A, const half_t* __restrict__ cs,
                                                           const half_t* __restrict__ sn, half_t* __restrict__ out,
-                                                          int64_t pieces, int64_t heads, int64_t d, int64_t pos0) {
+                                                          I pieces, I heads, I d, int64_t pos0) {
 #pragma clang fp contract(off)
   typedef u32x4 __attribute__((aligned(2))) u32x4_a2;
-  const int64_t per_row = d >> 3;
-  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < pieces;
-       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int64_t row = t / per_row, v = t % per_row;
-    const half_t* a = A + row * d;
+  const I per_row = d >> 3;
+  const I step = static_cast<I>(gridDim.x) * kBlock;
+  for (I t = static_cast<I>(blockIdx.x) * kBlock + threadIdx.x; t < pieces; t += step) {
+    const I row = t / per_row, v = t - row * per_row;
+    const half_t* a = A + static_cast<int64_t>(row) * d;
     u32x4 raw = *reinterpret_cast<const u32x4*>(a + 8 * v);
     if (v < 3) {
       const f16x8 x = __builtin_bit_cast(f16x8, raw);
       // partners: p[e] for element j = 8 v + e
       const f16x8 far = __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4_a2*>(a + (v == 0 ? 10 : v == 1 ? 18 : 6)));
       const f16x8 low = __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(a));   // elements 0..7 (piece 1 needs 0..5)
-      const half_t* cr = cs + (pos0 + row / heads) * 20 + 8 * v;
-      const half_t* sr = sn + (pos0 + row / heads) * 20 + 8 * v;
+      const int64_t pos = pos0 + row / heads;
+      const half_t* cr = cs + pos * 20 + 8 * v;
+      const half_t* sr = sn + pos * 20 + 8 * v;
       f16x4 c0 = __builtin_bit_cast(f16x4, *reinterpret_cast<const u32x2*>(cr)), s0 = __builtin_bit_cast(f16x4, *reinterpret_cast<const u32x2*>(sr));
       f16x4 c1 = {}, s1 = {};
       if (v < 2) {  // (piece 2 holds the tables' elements 16..19 only)
@@ -356,7 +359,8 @@ __global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restri
       }
       raw = __builtin_bit_cast(u32x4, r);
     }
-    *reinterpret_cast<u32x4*>(out + row * d + 8 * v) = raw;
+    *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row) * d + 8 * v) = raw;
+    if (pieces - t <= step) break;   // (t + step might wrap in 32 bits)
   }
 }
 
@@ -365,7 +369,7 @@ __global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restri
 // extended to m >= n key positions by extend_te (:68-80: 65504 for the m - n positions already cached, the
 // triangle after them) -- and, with n = 1, full (:83-93).  out[i, j] = (j - (m - n) > i) ? -65504 : 65504.
 // A thread writes 8 consecutive elements of the flat [n * m] array (16-byte stores whatever m is).
-// I = the index type: 32-bit while n * m fits (a 64-bit division costs more than the eight stores it places).
+// I = the index type: 32-bit while n * m fits.
 template <typename I>
 __global__ void __launch_bounds__(kBlock) attn_mask_kernel(half_t* __restrict__ out, I n, I m, I total) {
   const I shift = m - n;
@@ -395,14 +399,16 @@ __global__ void __launch_bounds__(kBlock) attn_mask_kernel(half_t* __restrict__ 
 // transpose6 / transpose7 (before_dl.py:1177-1203): [a, b, d] -> [b, a, d], rows of d elements moved whole
 // (queries, keys and values between the projection's [n, heads, d] and attention's [heads, n, d]).  A thread
 // moves one 16-byte piece; the stores are the contiguous side.
-__global__ void __launch_bounds__(kBlock) swap_axes_kernel(const u32x4* __restrict__ A, u32x4* __restrict__ out, int64_t a,
-                                                           int64_t b, int64_t per_row) {
-  const int64_t total = a * b * per_row;
-  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
-       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int64_t p = t % per_row, r = t / per_row;   // output row r = ib * a + ia
-    const int64_t ib = r / a, ia = r % a;
-    out[t] = A[(ia * b + ib) * per_row + p];
+// I = the index type: 32-bit while the piece count fits.
+template <typename I>
+__global__ void __launch_bounds__(kBlock) swap_axes_kernel(const u32x4* __restrict__ A, u32x4* __restrict__ out, I a, I b,
+                                                           I per_row, I total) {
+  const I step = static_cast<I>(gridDim.x) * kBlock;
+  for (I t = static_cast<I>(blockIdx.x) * kBlock + threadIdx.x; t < total; t += step) {
+    const I r = t / per_row, p = t - r * per_row;   // output row r = ib * a + ia
+    const I ib = r / a, ia = r - ib * a;
+    out[t] = A[(static_cast<int64_t>(ia) * b + ib) * per_row + p];
+    if (total - t <= step) break;   // (t + step might wrap in 32 bits)
   }
 }
 
@@ -410,16 +416,16 @@ __global__ void __launch_bounds__(kBlock) swap_axes_kernel(const u32x4* __restri
 // A[rows, 3 d] (rows = positions x heads, d = 80) cut into three [rows, d] buffers, section s = columns
 // [s d, (s + 1) d).  T is a 16-byte piece (d % 8 == 0, aligned buffers) or one element; the loads run
 // through A in order, the stores are runs of d elements.
-template <typename T>
+template <typename T, typename I>
 __global__ void __launch_bounds__(kBlock) split3_kernel(const T* __restrict__ A, T* __restrict__ o0, T* __restrict__ o1,
-                                                        T* __restrict__ o2, int64_t rows, int64_t per_sec) {
-  const int64_t total = rows * 3 * per_sec;
-  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
-       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int64_t r = t / (3 * per_sec), c = t % (3 * per_sec);
-    const int64_t sec = c / per_sec, j = c % per_sec;
+                                                        T* __restrict__ o2, I per_sec, I total) {
+  const I step = static_cast<I>(gridDim.x) * kBlock;
+  for (I t = static_cast<I>(blockIdx.x) * kBlock + threadIdx.x; t < total; t += step) {
+    const I r = t / (3 * per_sec), c = t - r * (3 * per_sec);
+    const I sec = c / per_sec, j = c - sec * per_sec;
     T* o = sec == 0 ? o0 : sec == 1 ? o1 : o2;
-    o[r * per_sec + j] = A[t];
+    o[static_cast<int64_t>(r) * per_sec + j] = A[t];
+    if (total - t <= step) break;   // (t + step might wrap in 32 bits)
   }
 }
 
@@ -529,9 +535,16 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
     const int64_t pieces20 = n * heads * (d / 8);
     int64_t grid = ceil_div(pieces20, kBlock);
     grid = grid > cap ? cap : grid;
-    hipLaunchKernelGGL(rotary20_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const half_t*>(A), static_cast<const half_t*>(cos_t), static_cast<const half_t*>(sin_t),
-                       static_cast<half_t*>(out), pieces20, heads, d, m - n);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half_t* a = static_cast<const half_t*>(A);
+    const half_t* c = static_cast<const half_t*>(cos_t);
+    const half_t* sn = static_cast<const half_t*>(sin_t);
+    if (pieces20 < (int64_t{1} << 31) && heads < (int64_t{1} << 31) && d < (int64_t{1} << 31))
+      hipLaunchKernelGGL(rotary20_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
+                         static_cast<uint32_t>(pieces20), static_cast<uint32_t>(heads), static_cast<uint32_t>(d), m - n);
+    else
+      hipLaunchKernelGGL(rotary20_kernel<int64_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
+                         pieces20, heads, d, m - n);
     return check_launch("rotary");
   }
   const int64_t pieces = n * heads * (d / 8);
@@ -574,8 +587,15 @@ int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d
   if (overlaps(out, a * b * d * 2, A, a * b * d * 2)) return fail("swap_axes: output overlaps the input");
   int64_t grid = ceil_div(a * b * (d / 8), kBlock);
   grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
-  hipLaunchKernelGGL(swap_axes_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const u32x4*>(A), static_cast<u32x4*>(out), a, b, d / 8);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total = a * b * (d / 8);
+  if (total < (int64_t{1} << 31))
+    hipLaunchKernelGGL(swap_axes_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const u32x4*>(A),
+                       static_cast<u32x4*>(out), static_cast<uint32_t>(a), static_cast<uint32_t>(b), static_cast<uint32_t>(d / 8),
+                       static_cast<uint32_t>(total));
+  else
+    hipLaunchKernelGGL(swap_axes_kernel<int64_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const u32x4*>(A),
+                       static_cast<u32x4*>(out), a, b, d / 8, total);
   return check_launch("swap_axes");
 }
 int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t rows, int64_t d, void* stream) {
@@ -599,12 +619,20 @@ int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t r
   int64_t grid = ceil_div(rows * 3 * per_sec, kBlock);
   grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (vec)
-    hipLaunchKernelGGL(split3_kernel<u32x4>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const u32x4*>(A),
-                       static_cast<u32x4*>(out0), static_cast<u32x4*>(out1), static_cast<u32x4*>(out2), rows, per_sec);
-  else
-    hipLaunchKernelGGL(split3_kernel<half_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const half_t*>(A),
-                       static_cast<half_t*>(out0), static_cast<half_t*>(out1), static_cast<half_t*>(out2), rows, per_sec);
+  const int64_t total = rows * 3 * per_sec;
+  const bool narrow = total < (int64_t{1} << 31);   // 32-bit indices while they fit
+  const dim3 g(static_cast<unsigned>(grid)), blk(kBlock);
+  if (vec) {
+    const u32x4* a = static_cast<const u32x4*>(A);
+    u32x4 *p0 = static_cast<u32x4*>(out0), *p1 = static_cast<u32x4*>(out1), *p2 = static_cast<u32x4*>(out2);
+    if (narrow) hipLaunchKernelGGL((split3_kernel<u32x4, uint32_t>), g, blk, 0, st, a, p0, p1, p2, static_cast<uint32_t>(per_sec), static_cast<uint32_t>(total));
+    else hipLaunchKernelGGL((split3_kernel<u32x4, int64_t>), g, blk, 0, st, a, p0, p1, p2, per_sec, total);
+  } else {
+    const half_t* a = static_cast<const half_t*>(A);
+    half_t *p0 = static_cast<half_t*>(out0), *p1 = static_cast<half_t*>(out1), *p2 = static_cast<half_t*>(out2);
+    if (narrow) hipLaunchKernelGGL((split3_kernel<half_t, uint32_t>), g, blk, 0, st, a, p0, p1, p2, static_cast<uint32_t>(per_sec), static_cast<uint32_t>(total));
+    else hipLaunchKernelGGL((split3_kernel<half_t, int64_t>), g, blk, 0, st, a, p0, p1, p2, per_sec, total);
+  }
   return check_launch("split3");
 }
 }

@@ -351,3 +351,21 @@ def test_split3_misaligned_and_errors(oracle):
         _lib.check(L.dtas_split3_f16(xd.data_ptr(), o.data_ptr(), o.data_ptr(), outs[2].t.data_ptr(), 50, 80, None), "split3")
     with pytest.raises(ValueError):
         ops.split3(xd[:, :239], *[o.t for o in outs])
+
+
+def test_swap_and_split_beyond_32_bit_indices():
+    # 2^31 pieces and more: the 64-bit index instantiations, checked on the device against torch's own views
+    a, b = 65536, 32768
+    g = torch.Generator(device="cuda").manual_seed(3)
+    A = torch.randint(-2 ** 15, 2 ** 15, (a, b, 8), dtype=torch.int16, device="cuda", generator=g).view(torch.float16)
+    out = torch.empty(b, a, 8, dtype=torch.float16, device="cuda")
+    ops.swap_axes(A, out)
+    for lo in range(0, b, 4096):
+        assert torch.equal(out[lo:lo + 4096].view(torch.int16), A[:, lo:lo + 4096].transpose(0, 1).view(torch.int16)), f"rows {lo}.."
+    del A, out
+    rows, d = 2 ** 20, 683                                                      # 3 * rows * d elements > 2^31, one element per access
+    A = torch.randint(-2 ** 15, 2 ** 15, (rows, 3 * d), dtype=torch.int16, device="cuda", generator=g).view(torch.float16)
+    outs = [torch.empty(rows, d, dtype=torch.float16, device="cuda") for _ in range(3)]
+    ops.split3(A, *outs)
+    for sec, o in enumerate(outs):
+        assert torch.equal(o.view(torch.int16), A[:, sec * d:(sec + 1) * d].view(torch.int16)), f"section {sec}"
