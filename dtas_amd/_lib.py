@@ -103,6 +103,8 @@ SIGNATURES = {
     "dtas_swap_axes_f16": [_vp, _vp, _i64, _i64, _i64, _vp],
     "dtas_split3_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
     "dtas_softmax_temperature_f32": [_vp, _vp, _vp, _i64, _i64, _vp],
+    "dtas_divide_f32": [_vp, _vp, _vp, _i64, _vp],
+    "dtas_softmax_f32": [_vp, _vp, _i64, _i64, _vp],
     "dtas_rotary_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _cfg, _vp],
     "dtas_take_f16": [_vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],
     "dtas_take_q8_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],

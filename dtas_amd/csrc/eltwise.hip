@@ -429,6 +429,27 @@ __global__ void __launch_bounds__(kBlock) split3_kernel(const T* __restrict__ A,
   }
 }
 
+// divide2 (before_dl.py:57-65): T_divide[k] = A[k] / B[()], fp32, the divisor one device scalar (the sampling
+// temperature).  The division is the correctly rounded one (no reciprocal shortcut): the result is bit-exact.
+__global__ void __launch_bounds__(kBlock) divide_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                            float* __restrict__ out, int64_t count, bool vec) {
+  const float b = *B;
+  const int64_t step = static_cast<int64_t>(gridDim.x) * kBlock;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (vec) {
+    const int64_t nvec = count >> 2;
+    for (int64_t t = t0; t < nvec; t += step) {
+      f32x4 v = reinterpret_cast<const f32x4*>(A)[t];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = v[e] / b;
+      reinterpret_cast<f32x4*>(out)[t] = v;
+    }
+    for (int64_t k = (nvec << 2) + t0; k < count; k += step) out[k] = A[k] / b;
+  } else {
+    for (int64_t k = t0; k < count; k += step) out[k] = A[k] / b;
+  }
+}
+
 }  // namespace
 
 // grid = min(ceil(nvec / (256 * unroll)), grid_cap): the reference's
@@ -634,5 +655,21 @@ int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t r
     else hipLaunchKernelGGL((split3_kernel<half_t, int64_t>), g, blk, 0, st, a, p0, p1, p2, per_sec, total);
   }
   return check_launch("split3");
+}
+int dtas_divide_f32(const void* A, const void* B, void* out, int64_t count, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (count < 0) return fail("divide: negative extent %lld", (long long)count);
+  if (count == 0) return 0;
+  if (count > INT64_MAX / 8) return fail("divide: extent overflows");
+  if (!A || !B || !out) return fail("divide: NULL buffer");
+  if (!aligned(A, 4) || !aligned(B, 4) || !aligned(out, 4)) return fail("divide: buffers must be 4-byte aligned");
+  if (overlaps(out, count * 4, A, count * 4) || overlaps(out, count * 4, B, 4)) return fail("divide: output overlaps an input");
+  const bool vec = aligned(A, 16) && aligned(out, 16);
+  int64_t grid = ceil_div(vec ? ceil_div(count, 4) : count, kBlock);
+  grid = grid > int64_t{kNumCU} * 32 ? int64_t{kNumCU} * 32 : grid;
+  hipLaunchKernelGGL(divide_f32_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const float*>(A), static_cast<const float*>(B), static_cast<float*>(out), count, vec);
+  return check_launch("divide");
 }
 }

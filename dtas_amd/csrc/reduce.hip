@@ -572,7 +572,7 @@ __global__ void __launch_bounds__(1024) softmax_temp_kernel(const float* __restr
                                                             float* __restrict__ out, int64_t rows, int64_t cols) {
   __shared__ float slots[64];
   int phase = 0;
-  const float t = *temp;
+  const float t = temp ? *temp : 1.f;   // no temperature: softmax2 alone (x / 1 is x)
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const float* x = A + row * cols;
     float* o = out + row * cols;
@@ -641,7 +641,7 @@ __global__ void __launch_bounds__(1024) softmax_temp_split_kernel(const float* _
                                                                   float* __restrict__ out, int64_t cols, int parts) {
   __shared__ float slots[64];
   int phase = 0;
-  const float t = *temp;
+  const float t = temp ? *temp : 1.f;   // no temperature: softmax2 alone (x / 1 is x)
   const int64_t row = blockIdx.x / parts;
   const int part = blockIdx.x % parts;
   const float* x = A + row * cols;
@@ -686,16 +686,16 @@ __global__ void __launch_bounds__(1024) softmax_temp_split_kernel(const float* _
 }  // namespace dtas
 
 extern "C" {
-int dtas_softmax_temperature_f32(const void* logits, const void* temperature, void* out, int64_t rows, int64_t cols,
-                                 void* stream) {
+static int run_softmax_f32(const char* what, const void* logits, const void* temperature, bool with_temperature, void* out,
+                           int64_t rows, int64_t cols, void* stream) {
   using namespace dtas;
   clear_error();
-  if (rows < 0 || cols < 0) return fail("softmax_temperature: negative extent rows=%lld cols=%lld", (long long)rows, (long long)cols);
+  if (rows < 0 || cols < 0) return fail("%s: negative extent rows=%lld cols=%lld", what, (long long)rows, (long long)cols);
   if (rows == 0 || cols == 0) return 0;
-  if (rows > INT64_MAX / 8 / cols) return fail("softmax_temperature: rows*cols overflows");
-  if (!logits || !temperature || !out) return fail("softmax_temperature: NULL buffer");
-  if (!aligned(logits, 4) || !aligned(temperature, 4) || !aligned(out, 4)) return fail("softmax_temperature: buffers must be 4-byte aligned");
-  if (overlaps(out, rows * cols * 4, logits, rows * cols * 4)) return fail("softmax_temperature: output overlaps the input");
+  if (rows > INT64_MAX / 8 / cols) return fail("%s: rows*cols overflows", what);
+  if (!logits || (with_temperature && !temperature) || !out) return fail("%s: NULL buffer", what);
+  if (!aligned(logits, 4) || (with_temperature && !aligned(temperature, 4)) || !aligned(out, 4)) return fail("%s: buffers must be 4-byte aligned", what);
+  if (overlaps(out, rows * cols * 4, logits, rows * cols * 4)) return fail("%s: output overlaps the input", what);
   const bool vec = cols % 4 == 0 && aligned(logits, 16) && aligned(out, 16) && cols <= 4096 * 16;
   const unsigned grid = static_cast<unsigned>(rows > int64_t{kNumCU} * 8 ? int64_t{kNumCU} * 8 : rows);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -717,7 +717,14 @@ int dtas_softmax_temperature_f32(const void* logits, const void* temperature, vo
     hipLaunchKernelGGL(softmax_temp_kernel<16>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
   else
     hipLaunchKernelGGL(softmax_temp_kernel<0>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
-  return check_launch("softmax_temperature");
+  return check_launch(what);
+}
+int dtas_softmax_temperature_f32(const void* logits, const void* temperature, void* out, int64_t rows, int64_t cols,
+                                 void* stream) {
+  return run_softmax_f32("softmax_temperature", logits, temperature, true, out, rows, cols, stream);
+}
+int dtas_softmax_f32(const void* A, void* out, int64_t rows, int64_t cols, void* stream) {
+  return run_softmax_f32("softmax_f32", A, nullptr, false, out, rows, cols, stream);
 }
 int dtas_layer_norm_f32_f16(const void* x, const void* gamma, const void* beta, void* out, int64_t n, int64_t H,
                             float eps, const dtas_config* cfg, void* stream) {

@@ -274,6 +274,23 @@ def softmax_temperature(logits: torch.Tensor, temperature: torch.Tensor, out: to
           "dtas_softmax_temperature_f32")
 
 
+def divide(A: torch.Tensor, B: torch.Tensor, out: torch.Tensor) -> None:
+    """divide2 (dolly-v2-3b-q0f16/before_dl.py:57-65): out = A / B, fp32, B a 0-d (one-element) device tensor."""
+    _dev(A, B, out)
+    if any(t.dtype != torch.float32 for t in (A, B, out)) or out.shape != A.shape or B.numel() != 1:
+        raise ValueError("divide: expects fp32 A and out of one shape and a one-element fp32 B")
+    check(lib().dtas_divide_f32(_p(A), _p(B), _p(out), A.numel(), _stream()), "dtas_divide_f32")
+
+
+def softmax_f32(A: torch.Tensor, out: torch.Tensor) -> None:
+    """softmax2 (dolly-v2-3b-q0f16/before_dl.py:1062-1096): softmax over the last axis, fp32 in and out."""
+    _dev(A, out)
+    if A.dtype != torch.float32 or out.dtype != torch.float32 or out.shape != A.shape:
+        raise ValueError("softmax_f32: expects fp32 A and out of one shape")
+    rows, cols = _rows_cols(A)
+    check(lib().dtas_softmax_f32(_p(A), _p(out), rows, cols, _stream()), "dtas_softmax_f32")
+
+
 def split3(A: torch.Tensor, out0: torch.Tensor, out1: torch.Tensor, out2: torch.Tensor) -> None:
     """split / fused_reshape7_split1 (dolly-v2-3b-q0f16/before_dl.py:1099-1125, :661-688): A (..., 3 d) fp16 cut into
     three (..., d) buffers along the last axis."""

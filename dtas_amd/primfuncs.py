@@ -237,6 +237,23 @@ def transpose(heads: int = 32, d: int = 80, back: bool = False, decode: bool = F
                     attrs={"tir.noalias": True})
 
 
+def divide(V: int = 50280, name: Optional[str] = None) -> PrimFunc:
+    """T_divide(1, 1, V) = A(1, 1, V) / B(), fp32: divide2 (dolly-v2-3b-q0f16/before_dl.py:57-65)."""
+    params = [Buffer("A", (1, 1, V), "float32"), Buffer("B", (), "float32"), Buffer("T_divide", (1, 1, V), "float32")]
+    return PrimFunc(name or "divide2", params, [Block("T_divide", "SSS", ["A", "B"], ["T_divide"])], op="divide",
+                    attrs={"tir.noalias": True})
+
+
+def softmax2(V: int = 50280, name: Optional[str] = None) -> PrimFunc:
+    """T_softmax_norm(1, 1, V) = softmax(A(1, 1, V)), fp32 in and out: softmax2 (dolly-v2-3b-q0f16/before_dl.py:1062-1096)."""
+    params = [Buffer("A", (1, 1, V), "float32"), Buffer("T_softmax_norm", (1, 1, V), "float32")]
+    blocks = [Block("T_softmax_maxelem", "SSR", ["A"], ["T_softmax_maxelem"]),
+              Block("T_softmax_exp", "SSS", ["A", "T_softmax_maxelem"], ["T_softmax_exp"]),
+              Block("T_softmax_expsum", "SSR", ["T_softmax_exp"], ["T_softmax_expsum"]),
+              Block("T_softmax_norm", "SSS", ["T_softmax_exp", "T_softmax_expsum"], ["T_softmax_norm"])]
+    return PrimFunc(name or "softmax2", params, blocks, op="softmax_f32", attrs={"tir.noalias": True})
+
+
 def softmax_with_temperature(V: int = 50280, name: Optional[str] = None) -> PrimFunc:
     """T_softmax_norm(1, 1, V) = softmax(A(1, 1, V) / B()), fp32: divide2 (dolly-v2-3b-q0f16/before_dl.py:57-65) and
     softmax2 (:1062-1096) as the graph's softmax_with_temperature chains them (:4154-4161).  Parameters: A (the

@@ -173,6 +173,10 @@ int dtas_softmax_f32_f16(const void* A, void* out, int64_t rows, int64_t cols,
                          const dtas_config* cfg, void* stream);
 int dtas_softmax_f16(const void* A, void* out, int64_t rows, int64_t cols, const dtas_config* cfg,
                      void* stream);
+/* divide2 (before_dl.py:57-65): out[count] = A[count] / *B, fp32, B one value in device memory (the PrimFunc's
+ * 0-d buffer); the correctly rounded division.  softmax2 (:1062-1096): fp32 softmax over each row, fp32 out. */
+int dtas_divide_f32(const void* A, const void* B, void* out, int64_t count, void* stream);
+int dtas_softmax_f32(const void* A, void* out, int64_t rows, int64_t cols, void* stream);
 /* softmax_with_temperature (before_dl.py:4154-4161): divide2 (:57-65) then softmax2 (:1062-1096).
  * out[rows, cols] fp32 = softmax over each row of logits[rows, cols] / *temperature; `temperature` points at
  * one fp32 in device memory (the PrimFunc's 0-d buffer B). */

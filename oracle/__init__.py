@@ -64,6 +64,7 @@ class _C:
                 "oracle_softmax_f32_f16": [vp, vp, i64, i64, ci],
                 "oracle_softmax_f16_f16": [vp, vp, i64, i64, ci],
                 "oracle_softmax_temperature_f32": [vp, vp, vp, i64, i64, ci],
+                "oracle_divide_f32": [vp, vp, vp, i64],
                 "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
@@ -143,6 +144,19 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         fn = {"float16": "oracle_softmax_f16_f16", "float32": "oracle_softmax_f32_f16"}[x.dtype.name]
         getattr(_C.lib(), fn)(_ptr(x), _ptr(out), x.size // max(cols, 1), cols, threads)
         return out
+
+    @staticmethod
+    def divide(a, b: float) -> np.ndarray:
+        assert a.dtype == np.float32
+        bb = np.array([b], dtype=np.float32)
+        out = np.empty_like(a)
+        _C.lib().oracle_divide_f32(_ptr(a), _ptr(bb), _ptr(out), a.size)
+        return out
+
+    @staticmethod
+    def softmax_f32(x, threads: int = 1) -> np.ndarray:
+        """softmax2 (before_dl.py:1062-1096): the fp32 pipeline of softmax_temperature with nothing divided (x / 1 is x)."""
+        return c.softmax_temperature(x, 1.0, threads)
 
     @staticmethod
     def softmax_temperature(x, temperature: float, threads: int = 1) -> np.ndarray:

@@ -198,6 +198,12 @@ void oracle_softmax_f32_f16(const float* x, f16* out, int64_t rows, int64_t cols
   }
 }
 
+/* divide2: experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:57-65, T_divide[k] = A[k] / B[()] in fp32.
+ * Pinned by: numpy float32 division (bit-exact), the float64 quotient rounded once, B = 1 is the identity. */
+void oracle_divide_f32(const float* a, const float* b, float* out, int64_t count) {
+  for (int64_t k = 0; k < count; ++k) out[k] = a[k] / *b;
+}
+
 /* softmax_with_temperature: experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:4154-4161 = divide2 (:57-65,
  * A / B[()] in fp32) then softmax2 (:1062-1096: max from -FLT_MAX, exp(x - max), sequential sum, exp / sum;
  * fp32 throughout).

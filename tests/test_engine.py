@@ -134,7 +134,10 @@ def test_layout_and_sampling_descriptors_follow_the_graph_signatures():
     sm = pf.softmax_with_temperature()
     assert [p.shape for p in sm.params] == [(1, 1, 50280), (), (1, 1, 50280)] and all(p.dtype == "float32" for p in sm.params)
     assert bind_extents(sm, [torch.zeros(1, 1, 50280), torch.tensor(0.7), torch.zeros(1, 1, 50280)]) == {}
-    assert all(f.op in LIBRARY_CHOSEN_OPS for f in (sp, dec, t6, t7, t8, sm))
+    dv, s2 = pf.divide(), pf.softmax2()
+    assert (dv.name, s2.name) == ("divide2", "softmax2") and [p.shape for p in dv.params] == [(1, 1, 50280), (), (1, 1, 50280)]
+    assert [p.shape for p in s2.params] == [(1, 1, 50280)] * 2 and s2.params[1].dtype == "float32"
+    assert all(f.op in LIBRARY_CHOSEN_OPS for f in (sp, dec, t6, t7, t8, sm, dv, s2))
 
 
 def test_cpu_tensors_are_refused_not_computed_elsewhere():

@@ -207,3 +207,17 @@ def test_split3_follows_the_index_expression(oracle):
     flat = a[:, :1].reshape(1, 1, 7680)
     again = oracle.layout.split3(flat.reshape(1, 1, 32, 240))
     assert np.array_equal(again[1].view(np.uint16), outs[1][:, :1].view(np.uint16))
+
+
+def test_divide_is_numpy_float32_division(oracle):
+    rng = np.random.default_rng(6)
+    a = np.concatenate([(rng.standard_normal(5000) * 10).astype(np.float32), np.array([0.0, -0.0, np.inf, -np.inf, 1e-45, 3.4e38], np.float32)])
+    with np.errstate(over="ignore"):                                                    # 3.4e38 / 1e-30 is meant to overflow
+        for b in (0.7, 1.0, -0.3, 3.0, 1e-30):
+            got = oracle.c.divide(a, b)
+            want = a / np.float32(b)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            finite = np.isfinite(want) & (np.abs(want) > 1e-30)
+            exact = (a.astype(np.float64) / float(np.float32(b))).astype(np.float32)    # one rounding of the exact quotient
+            assert np.array_equal(got[finite], exact[finite])
+    assert np.array_equal(oracle.c.divide(a, 1.0).view(np.uint32), a.view(np.uint32))

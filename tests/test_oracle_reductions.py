@@ -125,3 +125,13 @@ def test_softmax_temperature_invariants(oracle):
     assert (oracle.c.softmax_temperature(x, 0.5).max(-1) > one.max(-1)).all()
     assert (oracle.c.softmax_temperature(np.array([[2.5]], np.float32), 0.3) == np.float32(1)).all()
     assert np.array_equal(np.argmax(one, -1), np.argmax(x, -1))
+
+
+def test_softmax_f32_is_the_temperature_form_with_nothing_divided(oracle):
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal((2, 3000)) * 3).astype(np.float32)
+    got = oracle.c.softmax_f32(x)
+    assert got.dtype == np.float32 and np.array_equal(got.astype(np.float16), oracle.c.softmax(x))
+    assert np.abs(got / scipy_softmax(x.astype(np.float64), axis=-1) - 1).max() < 1e-4
+    # divide2 then softmax2 is softmax_with_temperature, bit for bit
+    assert np.array_equal(oracle.c.softmax_f32(oracle.c.divide(x, 0.7)), oracle.c.softmax_temperature(x, 0.7))

@@ -369,3 +369,30 @@ def test_swap_and_split_beyond_32_bit_indices():
     ops.split3(A, *outs)
     for sec, o in enumerate(outs):
         assert torch.equal(o.view(torch.int16), A[:, sec * d:(sec + 1) * d].view(torch.int16)), f"section {sec}"
+
+
+@pytest.mark.parametrize("count", [1, 3, 4, 1023, 50280, 50281, 1 << 22])
+@pytest.mark.parametrize("b", [0.7, -3.0])
+def test_divide_is_exact(oracle, count, b):
+    rng = np.random.default_rng(count)
+    a = (rng.standard_normal(count) * 10).astype(np.float32)
+    special = np.array([0.0, np.inf, -np.inf, 1e-45, 3.4e38, -0.0, 1.0], np.float32)[:count]
+    a[:special.size] = special
+    out = Guarded((count,), torch.float32)
+    ops.divide(dev(a), torch.tensor(b, dtype=torch.float32, device="cuda"), out.t)
+    assert_bits_equal(out.check(), oracle.c.divide(a, b))
+    if count > 8:                                                                # 4-byte alignment only: element accesses
+        raw = dev(np.concatenate([[0.0], a]).astype(np.float32))
+        out = Guarded((count,), torch.float32)
+        ops.divide(raw[1:], torch.tensor([b], dtype=torch.float32, device="cuda"), out.t)
+        assert_bits_equal(out.check(), oracle.c.divide(a, b))
+
+
+def test_divide_errors():
+    L = _lib.lib()
+    assert L.dtas_divide_f32(None, None, None, 0, None) == 0
+    assert L.dtas_divide_f32(None, None, None, 5, None) == -1 and b"NULL" in L.dtas_last_error()
+    assert L.dtas_divide_f32(None, None, None, -5, None) == -1 and b"negative" in L.dtas_last_error()
+    x = torch.zeros(8, dtype=torch.float32, device="cuda")
+    with pytest.raises(_lib.DtasError, match="overlaps"):
+        _lib.check(L.dtas_divide_f32(x.data_ptr(), x.data_ptr() + 16, x.data_ptr(), 4, None), "divide")

@@ -278,3 +278,22 @@ def test_softmax_temperature_unaligned_and_errors(oracle):
     assert L.dtas_softmax_temperature_f32(None, None, None, -1, 9, None) == -1 and b"negative" in L.dtas_last_error()
     with pytest.raises(ValueError):
         ops.softmax_temperature(xd, torch.tensor(0.9, dtype=torch.float16, device="cuda"), out.t)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 50280), (3, 4096), (2, 50281), (300, 1000)])
+def test_softmax_f32(oracle, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
+    out = Guarded(x.shape, torch.float32)
+    ops.softmax_f32(dev(x), out.t)
+    got = out.check().astype(np.float64)
+    assert np.abs(got - oracle.c.softmax_f32(x, threads=8)).max() < 1e-2
+    assert np.abs(got / oracle.np64.softmax(x) - 1).max() < 3e-5 and np.abs(got.sum(-1) - 1).max() < 1e-4
+    # divide2 then softmax2 on the device against softmax_with_temperature on the device (the shared-row kernel sums
+    # exp2((x - max) * log2e / t) in one, exp2((x / t - max) * log2e) in the other: last-place differences)
+    t = torch.tensor(0.7, dtype=torch.float32, device="cuda")
+    div, two, one = torch.empty_like(out.t), torch.empty_like(out.t), torch.empty_like(out.t)
+    ops.divide(dev(x), t, div)
+    ops.softmax_f32(div, two)
+    ops.softmax_temperature(dev(x), t, one)
+    assert float(((one - two).abs() / one.clamp_min(1e-30)).max()) < 1e-5
