@@ -92,6 +92,13 @@ def _workload(name: str, n: int, extra=None):
         make = lambda s: (normal((n, Hr), s, 1.0, torch.float32), gm, bt, empty((n, Hr)))
         return (make, lambda b: call(L.dtas_layer_norm_f32_f16, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, Hr, 1e-5, None, stream),
                 (4 + 2) * n * Hr + 8 * Hr, 0)
+    if name == "layer_norm_f32":
+        # layer_norm: the graph's last layer norm, fp32 in and out
+        Hr = 2560
+        gm, bt = uniform((Hr,), 3, 0.5, 1.5, torch.float32), uniform((Hr,), 4, -1, 1, torch.float32)
+        make = lambda s: (normal((n, Hr), s, 1.0, torch.float32), gm, bt, empty((n, Hr), torch.float32))
+        return (make, lambda b: call(L.dtas_layer_norm_f32, P(b[0]), P(b[1]), P(b[2]), P(b[3]), n, Hr, 1e-5, stream),
+                8 * n * Hr + 8 * Hr, 0)
     if name == "softmax_f16":
         R = 32 * n
         make = lambda s: (normal((R, n), s, 2.0), empty((R, n)))
@@ -363,6 +370,8 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("swap_axes_f16", n, None, steps, warmup))
         rows.append(measure("attn_mask_f16", n, None, steps, warmup))
     rows.append(measure("softmax_temperature_f32", 1, None, steps, warmup))
+    for n in (1, 4096):
+        rows.append(measure("layer_norm_f32", n, None, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
             rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
@@ -400,7 +409,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
-                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
+                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | layer_norm_f32 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
                          "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | split3_f16 | swap_axes_f16 | attn_mask_f16 | softmax_temperature_f32 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")

@@ -104,6 +104,7 @@ SIGNATURES = {
     "dtas_split3_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
     "dtas_softmax_temperature_f32": [_vp, _vp, _vp, _i64, _i64, _vp],
     "dtas_divide_f32": [_vp, _vp, _vp, _i64, _vp],
+    "dtas_layer_norm_f32": [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_float, _vp],
     "dtas_softmax_f32": [_vp, _vp, _i64, _i64, _vp],
     "dtas_rotary_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _cfg, _vp],
     "dtas_take_f16": [_vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],

@@ -58,7 +58,7 @@ def op_id_of(func: PrimFunc) -> int:
 
 # PrimFuncs the tuner does not search: the library picks their kernel and launch shape per call
 LIBRARY_CHOSEN_OPS = ("attn_scores", "attn_pv", "decode_q8", "take", "take_q8", "gemv_q8", "gemv_q8_f32", "gemm_q8", "gemv_f32",
-                      "split3", "swap_axes", "softmax_temperature", "divide", "softmax_f32")
+                      "split3", "swap_axes", "softmax_temperature", "divide", "softmax_f32", "layer_norm_f32")
 
 
 def _concrete(shape, values: Dict[str, int]) -> Tuple[int, ...]:
@@ -148,6 +148,8 @@ def call_primfunc(func: PrimFunc, tensors: Sequence, abi: Optional[_lib.DtasConf
         ops.split3(tensors[0].view(-1, heads, 3 * d), tensors[1], tensors[2], tensors[3])
     elif op == "swap_axes":                                                   # A, out
         ops.swap_axes(tensors[0], tensors[1])
+    elif op == "layer_norm_f32":                                              # A, gamma, beta, out
+        ops.layer_norm_f32(tensors[0], tensors[1], tensors[2], tensors[3], func.attrs.get("eps", 1e-5))
     elif op == "divide":                                                      # A, B (0-d), out
         ops.divide(tensors[0], tensors[1], tensors[2])
     elif op == "softmax_f32":                                                 # A, out

@@ -563,6 +563,112 @@ int describe_reduction(int op, int64_t rows, int64_t cols, const dtas_config& cf
   return 0;
 }
 
+// layer_norm / layer_norm1 (before_dl.py:846-896): the final layer norm, fp32 in and fp32 out (the fused forms
+// above round to fp16).  One workgroup of 256 per row; ITERS > 0 holds the row in registers (H % 4 == 0,
+// H <= 1024 ITERS, 16-byte aligned rows), ITERS == 0 walks it twice with element accesses.
+template <int ITERS>
+__global__ void __launch_bounds__(256) layer_norm_f32_kernel(const float* __restrict__ x, const float* __restrict__ g,
+                                                             const float* __restrict__ b, float* __restrict__ out,
+                                                             int64_t rows, int64_t H, float eps) {
+  __shared__ float slots[64];
+  int phase = 0;
+  const float inv = 1.0f / static_cast<float>(H);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const float* xr = x + row * H;
+    float* o = out + row * H;
+    float s0 = 0.f, s1 = 0.f;
+    if constexpr (ITERS > 0) {
+      f32x4 v[ITERS];
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int64_t k = (static_cast<int64_t>(it) * 256 + threadIdx.x) * 4;   // every load issued before the first use
+        v[it] = *reinterpret_cast<const f32x4*>(xr + (k < H ? k : 0));
+      }
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int64_t k = (static_cast<int64_t>(it) * 256 + threadIdx.x) * 4;
+        if (k < H) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            s0 += v[it][e];
+            s1 += v[it][e] * v[it][e];
+          }
+        }
+      }
+      block_sum2(s0, s1, slots, phase);
+      const float mean = s0 * inv;
+      const float rstd = 1.0f / sqrtf(s1 * inv - mean * mean + eps);
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int64_t k = (static_cast<int64_t>(it) * 256 + threadIdx.x) * 4;
+        if (k < H) {
+          const f32x4 gv = *reinterpret_cast<const f32x4*>(g + k), bv = *reinterpret_cast<const f32x4*>(b + k);
+          f32x4 r;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r[e] = (v[it][e] - mean) * rstd * gv[e] + bv[e];
+          *reinterpret_cast<f32x4*>(o + k) = r;
+        }
+      }
+    } else {
+      for (int64_t k = threadIdx.x; k < H; k += blockDim.x) {
+        s0 += xr[k];
+        s1 += xr[k] * xr[k];
+      }
+      block_sum2(s0, s1, slots, phase);
+      const float mean = s0 * inv;
+      const float rstd = 1.0f / sqrtf(s1 * inv - mean * mean + eps);
+      for (int64_t k = threadIdx.x; k < H; k += blockDim.x) o[k] = (xr[k] - mean) * rstd * g[k] + b[k];
+    }
+  }
+}
+
+// The same with a wavefront per row (four rows per workgroup, no barrier): for many rows.  H % 4 == 0,
+// H <= 256 ITERS, 16-byte aligned rows.
+template <int ITERS>
+__global__ void __launch_bounds__(256) layer_norm_f32_wave_kernel(const float* __restrict__ x, const float* __restrict__ g,
+                                                                  const float* __restrict__ b, float* __restrict__ out,
+                                                                  int64_t rows, int64_t H, float eps) {
+  const float inv = 1.0f / static_cast<float>(H);
+  const int lane = threadIdx.x & 63;
+  for (int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6); row < rows; row += static_cast<int64_t>(gridDim.x) * 4) {
+    const float* xr = x + row * H;
+    float* o = out + row * H;
+    f32x4 v[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {   // every load issued before the first use
+      const int64_t k = (it * 64 + lane) * 4;
+      v[it] = *reinterpret_cast<const f32x4*>(xr + (k < H ? k : 0));
+    }
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int64_t k = (it * 64 + lane) * 4;
+      if (k < H) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s0 += v[it][e];
+          s1 += v[it][e] * v[it][e];
+        }
+      }
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    const float mean = s0 * inv;
+    const float rstd = 1.0f / sqrtf(s1 * inv - mean * mean + eps);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int64_t k = (it * 64 + lane) * 4;
+      if (k < H) {
+        const f32x4 gv = *reinterpret_cast<const f32x4*>(g + k), bv = *reinterpret_cast<const f32x4*>(b + k);
+        f32x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = (v[it][e] - mean) * rstd * gv[e] + bv[e];
+        __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(o + k));
+      }
+    }
+  }
+}
+
 // softmax_with_temperature (before_dl.py:4154-4161): divide2 (:57-65, logits / temperature, the temperature a
 // device scalar) then softmax2 (:1062-1096), fp32 in and out, over the vocabulary.  One workgroup of 1024 per
 // row; ITERS > 0 keeps the divided row in registers (cols <= 4096 ITERS, cols % 4 == 0, 16-byte aligned rows),
@@ -686,6 +792,38 @@ __global__ void __launch_bounds__(1024) softmax_temp_split_kernel(const float* _
 }  // namespace dtas
 
 extern "C" {
+int dtas_layer_norm_f32(const void* x, const void* gamma, const void* beta, void* out, int64_t n, int64_t H, float eps,
+                        void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (n < 0 || H < 0) return fail("layer_norm_f32: negative extent n=%lld H=%lld", (long long)n, (long long)H);
+  if (n == 0 || H == 0) return 0;
+  if (n > INT64_MAX / 8 / H) return fail("layer_norm_f32: n*H overflows");
+  if (!x || !gamma || !beta || !out) return fail("layer_norm_f32: NULL buffer");
+  if (!aligned(x, 4) || !aligned(gamma, 4) || !aligned(beta, 4) || !aligned(out, 4)) return fail("layer_norm_f32: buffers must be 4-byte aligned");
+  if (overlaps(out, n * H * 4, x, n * H * 4) || overlaps(out, n * H * 4, gamma, H * 4) || overlaps(out, n * H * 4, beta, H * 4))
+    return fail("layer_norm_f32: output overlaps an input");
+  const bool vec = H % 4 == 0 && H <= 4096 && aligned(x, 16) && aligned(out, 16) && aligned(gamma, 16) && aligned(beta, 16);
+  const unsigned grid = static_cast<unsigned>(n > int64_t{kNumCU} * 32 ? int64_t{kNumCU} * 32 : n);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float* xp = static_cast<const float*>(x);
+  const float* gp = static_cast<const float*>(gamma);
+  const float* bp = static_cast<const float*>(beta);
+  float* op = static_cast<float*>(out);
+  if (vec && n >= 2 * kNumCU) {   // many rows: a wavefront each
+    const unsigned wgrid = static_cast<unsigned>(ceil_div(n, 4) > int64_t{kNumCU} * 32 ? int64_t{kNumCU} * 32 : ceil_div(n, 4));
+    if (H <= 1024) hipLaunchKernelGGL(layer_norm_f32_wave_kernel<4>, dim3(wgrid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+    else if (H <= 2560) hipLaunchKernelGGL(layer_norm_f32_wave_kernel<10>, dim3(wgrid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+    else hipLaunchKernelGGL(layer_norm_f32_wave_kernel<16>, dim3(wgrid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+    return check_launch("layer_norm_f32");
+  }
+  if (vec && H <= 1024) hipLaunchKernelGGL(layer_norm_f32_kernel<1>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  else if (vec && H <= 2048) hipLaunchKernelGGL(layer_norm_f32_kernel<2>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  else if (vec && H <= 3072) hipLaunchKernelGGL(layer_norm_f32_kernel<3>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  else if (vec) hipLaunchKernelGGL(layer_norm_f32_kernel<4>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  else hipLaunchKernelGGL(layer_norm_f32_kernel<0>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  return check_launch("layer_norm_f32");
+}
 static int run_softmax_f32(const char* what, const void* logits, const void* temperature, bool with_temperature, void* out,
                            int64_t rows, int64_t cols, void* stream) {
   using namespace dtas;

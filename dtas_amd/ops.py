@@ -110,6 +110,17 @@ def layer_norm(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, out: to
           "dtas_layer_norm_f32_f16")
 
 
+def layer_norm_f32(x: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, out: torch.Tensor, eps: float = 1e-5) -> None:
+    """layer_norm / layer_norm1 (dolly-v2-3b-q0f16/before_dl.py:846-896): layer norm over the last axis, fp32 in and out."""
+    _dev(x, gamma, beta, out)
+    if any(t.dtype != torch.float32 for t in (x, gamma, beta, out)) or out.shape != x.shape:
+        raise ValueError("layer_norm_f32: expects fp32 tensors and an output of x's shape")
+    n, H = _rows_cols(x)
+    if gamma.numel() != H or beta.numel() != H:
+        raise ValueError("layer_norm_f32: gamma and beta hold one value per column")
+    check(lib().dtas_layer_norm_f32(_p(x), _p(gamma), _p(beta), _p(out), n, H, eps, _stream()), "dtas_layer_norm_f32")
+
+
 def rms_norm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float = 1e-5,
              cfg: Optional[DtasConfig] = None) -> None:
     """out = x * rsqrt(mean(x^2) + eps) * w over the last axis; fp16 in/out, fp32 arithmetic."""

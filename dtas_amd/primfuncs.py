@@ -48,6 +48,19 @@ def fused_layer_norm_cast1(hidden: int = 2560) -> PrimFunc:
         op="layer_norm", attrs={"tir.noalias": True, "eps": 1e-5})
 
 
+def layer_norm(hidden: int = 2560, decode: bool = False) -> PrimFunc:
+    """LayerNorm fp32 -> fp32 (the graph's last one): layer_norm (dolly-v2-3b-q0f16/before_dl.py:846-872; n dynamic) or,
+    with ``decode``, layer_norm1 (:874-896; one row).  Parameters: A, B (gamma), C (beta), T_layer_norm."""
+    n = 1 if decode else "n"
+    return PrimFunc(
+        "layer_norm1" if decode else "layer_norm",
+        [Buffer("A", (1, n, hidden), "float32"), Buffer("B", (hidden,), "float32"), Buffer("C", (hidden,), "float32"),
+         Buffer("T_layer_norm", (1, n, hidden), "float32")],
+        [Block("A_red_temp", "SSR", ["A"], ["A_red_temp_v0", "A_red_temp_v1"]),
+         Block("T_layer_norm", "SSS", ["A", "A_red_temp_v0", "A_red_temp_v1", "B", "C"], ["T_layer_norm"])],
+        op="layer_norm_f32", attrs={"tir.noalias": True, "eps": 1e-5})
+
+
 def rms_norm(hidden: int = 4096, eps: float = 1e-5) -> PrimFunc:
     """RMSNorm fp16 with fp16 weight; no counterpart in the reference (the benchmark's norm)."""
     return PrimFunc(

@@ -162,6 +162,10 @@ int dtas_cast_f32_f16(const void* A, void* compute, int64_t n, int64_t H, const 
  * x fp32 [n,H], gamma/beta fp32 [H] -> out fp16 [n,H]; eps is 1e-5 in the PrimFunc. */
 int dtas_layer_norm_f32_f16(const void* x, const void* gamma, const void* beta, void* out,
                             int64_t n, int64_t H, float eps, const dtas_config* cfg, void* stream);
+/* layer_norm / layer_norm1 (before_dl.py:846-896): the same normalisation with an fp32 output (the graph's last
+ * layer norm, in front of the vocabulary projection). */
+int dtas_layer_norm_f32(const void* x, const void* gamma, const void* beta, void* out, int64_t n, int64_t H,
+                        float eps, void* stream);
 /* RMSNorm (no PrimFunc in the reference; the benchmark's norm): x fp16 [n,H], w fp16 [H]
  * -> out fp16 [n,H] = x * rsqrt(mean(x^2) + eps) * w, fp32 arithmetic. */
 int dtas_rms_norm_f16(const void* x, const void* w, void* out, int64_t n, int64_t H, float eps,

@@ -65,6 +65,7 @@ class _C:
                 "oracle_softmax_f16_f16": [vp, vp, i64, i64, ci],
                 "oracle_softmax_temperature_f32": [vp, vp, vp, i64, i64, ci],
                 "oracle_divide_f32": [vp, vp, vp, i64],
+                "oracle_layer_norm_f32": [vp, vp, vp, vp, i64, i64, ctypes.c_float, ci],
                 "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
@@ -127,6 +128,14 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         H = x.shape[-1]
         out = np.empty(x.shape, dtype=np.float16)
         _C.lib().oracle_layer_norm_f32_f16(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.size // H, H, eps, threads)
+        return out
+
+    @staticmethod
+    def layer_norm_f32(x, gamma, beta, eps: float = 1e-5, threads: int = 1) -> np.ndarray:
+        assert x.dtype == gamma.dtype == beta.dtype == np.float32
+        H = x.shape[-1]
+        out = np.empty(x.shape, dtype=np.float32)
+        _C.lib().oracle_layer_norm_f32(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.size // max(H, 1), H, eps, threads)
         return out
 
     @staticmethod

@@ -158,6 +158,26 @@ void oracle_layer_norm_f32_f16(const float* x, const float* gamma, const float* 
   }
 }
 
+/* layer_norm / layer_norm1: experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:846-896, the same arithmetic
+ * with the result left in fp32.
+ * Pinned by: rounds to the fused function's fp16 result bit for bit; fp64 closed form (1e-4); torch.layer_norm. */
+void oracle_layer_norm_f32(const float* x, const float* gamma, const float* beta, float* out, int64_t n, int64_t H,
+                           float eps, int nthreads) {
+  const float inv = (float)(1.0 / (double)H);
+  OMP_FOR(nthreads)
+  for (int64_t r = 0; r < n; ++r) {
+    const float* xr = x + r * H;
+    float s0 = 0.f, s1 = 0.f;
+    for (int64_t k = 0; k < H; ++k) {
+      s0 = s0 + xr[k];
+      s1 = s1 + xr[k] * xr[k];
+    }
+    const float mean = s0 * inv;
+    const float rstd = 1.0f / sqrtf(s1 * inv - mean * mean + eps);
+    for (int64_t k = 0; k < H; ++k) out[r * H + k] = (xr[k] - mean) * rstd * gamma[k] + beta[k];
+  }
+}
+
 /* rms_norm: no counterpart in the reference (PARITY UNPINNED by the
  * reference).  Closed form: ss = sum f32(x)^2 in fp32;
  * out = f16(f32(x) * rsqrt(ss/H + eps) * f32(w)), one final rounding.

@@ -155,7 +155,7 @@ def test_decode_forms_of_the_fused_matmuls_go_through_the_gemv_rule(tmp_path, or
 def test_layout_and_sampling_primfuncs_through_the_module(tmp_path, oracle):
     """split / fused_reshape7_split1, transpose6 / 7 / 8 and softmax_with_temperature: served by the library's own choice."""
     funcs = [pf.split(), pf.split(decode=True), pf.transpose(), pf.transpose(back=True), pf.transpose(decode=True),
-             pf.softmax_with_temperature(), pf.divide(), pf.softmax2()]
+             pf.softmax_with_temperature(), pf.divide(), pf.softmax2(), pf.layer_norm(), pf.layer_norm(decode=True)]
     work_dir = str(tmp_path / "layout")
     rt = Engine(topk=2, parallel_build=False, work_dir=work_dir).tune_module(pf.module(*funcs), arch=MI355X(0, require_device=True))
     rng = np.random.default_rng(12)
@@ -183,6 +183,12 @@ def test_layout_and_sampling_primfuncs_through_the_module(tmp_path, oracle):
         mod["softmax_with_temperature"](t(logits), torch.tensor(0.8, dtype=torch.float32, device="cuda"), probs)
         want = oracle.c.softmax_temperature(logits, 0.8)
         assert np.abs(probs.cpu().numpy() - want).max() < 1e-2 and np.abs(probs.cpu().numpy() / want - 1).max() < 1e-3
+        for name, n in (("layer_norm", 9), ("layer_norm1", 1)):
+            x = rng.standard_normal((1, n, 2560)).astype(np.float32)
+            gm, bt = rng.uniform(0.5, 1.5, 2560).astype(np.float32), rng.uniform(-1, 1, 2560).astype(np.float32)
+            y = torch.empty(1, n, 2560, dtype=torch.float32, device="cuda")
+            mod[name](t(x), t(gm), t(bt), y)
+            assert np.abs(y.cpu().numpy() - oracle.c.layer_norm_f32(x, gm, bt)).max() < 1e-4
         div, two = torch.empty_like(probs), torch.empty_like(probs)
         mod["divide2"](t(logits), torch.tensor(0.8, dtype=torch.float32, device="cuda"), div)
         assert np.array_equal(div.cpu().numpy().view(np.uint32), oracle.c.divide(logits, 0.8).view(np.uint32))

@@ -135,3 +135,14 @@ def test_softmax_f32_is_the_temperature_form_with_nothing_divided(oracle):
     assert np.abs(got / scipy_softmax(x.astype(np.float64), axis=-1) - 1).max() < 1e-4
     # divide2 then softmax2 is softmax_with_temperature, bit for bit
     assert np.array_equal(oracle.c.softmax_f32(oracle.c.divide(x, 0.7)), oracle.c.softmax_temperature(x, 0.7))
+
+
+def test_layer_norm_f32_rounds_to_the_fused_form_and_matches_the_closed_form(oracle):
+    x, g, b = _ln_inputs()
+    got = oracle.c.layer_norm_f32(x, g, b)
+    assert got.dtype == np.float32 and np.array_equal(got.astype(np.float16), oracle.c.layer_norm(x, g, b))
+    assert np.abs(got - oracle.np64.layer_norm(x, g, b)).max() < 1e-4
+    want = torch.layer_norm(torch.from_numpy(x), (x.shape[-1],), torch.from_numpy(g), torch.from_numpy(b), 1e-5).numpy()
+    assert np.abs(got - want).max() < 1e-4
+    short = x[:, :777].copy()                                                   # 1/H follows the row length
+    assert np.abs(oracle.c.layer_norm_f32(short, g[:777].copy(), b[:777].copy()) - oracle.np64.layer_norm(short, g[:777], b[:777])).max() < 1e-4

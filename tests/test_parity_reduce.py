@@ -297,3 +297,31 @@ def test_softmax_f32(oracle, rows, cols):
     ops.softmax_f32(div, two)
     ops.softmax_temperature(dev(x), t, one)
     assert float(((one - two).abs() / one.clamp_min(1e-30)).max()) < 1e-5
+
+
+@pytest.mark.parametrize("n,H", [(1, 2560), (37, 2560), (4096, 2560), (5, 1024), (3, 4096), (7, 4100), (6, 777), (2, 10000),
+                                 (600, 1024), (520, 4096), (513, 1028), (515, 8), (2049, 2564)])   # from 512 rows: a wavefront per row
+def test_layer_norm_f32(oracle, n, H):
+    rng = np.random.default_rng(n + H)
+    x = (rng.standard_normal((n, H)) * 2 + 0.5).astype(np.float32)
+    g, b = rng.uniform(0.5, 1.5, H).astype(np.float32), rng.uniform(-1, 1, H).astype(np.float32)
+    out = Guarded((n, H), torch.float32)
+    ops.layer_norm_f32(dev(x), dev(g), dev(b), out.t)
+    got = out.check()
+    assert np.abs(got - oracle.c.layer_norm_f32(x, g, b, threads=8)).max() < 1e-2       # the stated tolerance
+    assert np.abs(got - oracle.np64.layer_norm(x, g, b)).max() < 2e-5                    # what fp32 gives
+
+
+def test_layer_norm_f32_unaligned_and_errors(oracle):
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((3, 2560))).astype(np.float32)
+    g, b = rng.uniform(0.5, 1.5, 2560).astype(np.float32), rng.uniform(-1, 1, 2560).astype(np.float32)
+    raw = dev(np.concatenate([[0.0], x.ravel()]).astype(np.float32))
+    out = Guarded((3, 2560), torch.float32)
+    ops.layer_norm_f32(raw[1:].view(3, 2560), dev(g), dev(b), out.t)                       # 4-byte aligned rows: element accesses
+    assert np.abs(out.check() - oracle.np64.layer_norm(x, g, b)).max() < 2e-5
+    L = _lib.lib()
+    assert L.dtas_layer_norm_f32(None, None, None, None, 0, 2560, 1e-5, None) == 0
+    assert L.dtas_layer_norm_f32(None, None, None, None, 2, 2560, 1e-5, None) == -1 and b"NULL" in L.dtas_last_error()
+    with pytest.raises(ValueError):
+        ops.layer_norm_f32(dev(x), dev(g[:100]), dev(b), out.t)
