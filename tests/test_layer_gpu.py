@@ -132,22 +132,26 @@ def test_one_layer_call_by_call(oracle, n, past):
 
 
 def test_sampling_head(oracle):
-    """slice + fused_slice1_cast4 (the last position, fp32), NT_matmul5 (the vocabulary projection) and
-    softmax_with_temperature (before_dl.py:2677-2679, :4154-4161)."""
+    """layer_norm (the last one, fp32), slice + fused_slice1_cast4 (the last position), NT_matmul5 (the vocabulary
+    projection) and softmax_with_temperature (before_dl.py:4144, :2677-2679, :4154-4161)."""
     rng = np.random.default_rng(5)
     n = 9
     hidden = rng.standard_normal((n, H)).astype(np.float32)
+    g, b = rng.uniform(0.5, 1.5, H).astype(np.float32), rng.uniform(-0.2, 0.2, H).astype(np.float32)
     emb = (rng.standard_normal((VOCAB, H)) * 0.05).astype(np.float32)
-    hd, ed = dev(hidden), dev(emb)
+    normed = torch.empty(n, H, dtype=torch.float32, device="cuda")
+    ops.layer_norm_f32(dev(hidden), dev(g), dev(b), normed)
     last = torch.empty(1, H, dtype=torch.float32, device="cuda")
-    ops.copy(hd[n - 1:], last)
+    ops.copy(normed[n - 1:], last)
     logits = torch.empty(1, VOCAB, dtype=torch.float32, device="cuda")
-    ops.gemv_f32(last, ed, logits)
+    ops.gemv_f32(last, dev(emb), logits)
     probs = torch.empty_like(logits)
     ops.softmax_temperature(logits, torch.tensor(0.7, dtype=torch.float32, device="cuda"), probs)
     torch.cuda.synchronize()
-    assert np.array_equal(last.cpu().numpy(), hidden[n - 1:])
-    want_logits = oracle.c.gemv_f32(hidden[n - 1], emb, threads=8).reshape(1, VOCAB)
+    want_normed = oracle.c.layer_norm_f32(hidden, g, b)
+    assert np.abs(normed.cpu().numpy() - want_normed).max() < 1e-4
+    assert torch.equal(last[0], normed[n - 1])
+    want_logits = oracle.c.gemv_f32(want_normed[n - 1], emb, threads=8).reshape(1, VOCAB)
     _close(logits.cpu().numpy(), want_logits, "logits", atol=1e-3)
     want = oracle.c.softmax_temperature(want_logits, 0.7)
     got = probs.cpu().numpy()
