@@ -241,7 +241,7 @@ def split(heads: int = 32, d: int = 80, decode: bool = False, name: Optional[str
 
 def transpose(heads: int = 32, d: int = 80, back: bool = False, decode: bool = False, name: Optional[str] = None) -> PrimFunc:
     """T_transpose(1, heads, n, d) = A(1, n, heads, d): transpose6 (dolly-v2-3b-q0f16/before_dl.py:1177-1189) or, with
-    ``back``, transpose7 (:1192-1203; (1, heads, n, d) -> (1, n, heads, d)); ``decode``: transpose8 (:1205-1213, n = 1)."""
+    ``back``, transpose7 (:1191-1203; (1, heads, n, d) -> (1, n, heads, d)); ``decode``: transpose8 (:1205-1213, n = 1)."""
     n = 1 if decode else "n"
     src, dst = ((1, heads, n, d), (1, n, heads, d)) if back else ((1, n, heads, d), (1, heads, n, d))
     params = [Buffer("A", src, "float16"), Buffer("T_transpose", dst, "float16")]
