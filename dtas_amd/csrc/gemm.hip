@@ -165,7 +165,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // then transposed on the way into the LDS (two stages, 4 wavefronts only).
 // WQ: W is 8-bit with an fp16 scale per 32 elements of a row (Wq bytes [N][K], ep.wscale [N][K/32]); its
 // tiles are dequantised on their way into the LDS by the same register path.
-template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false>
+// M16: the 8-wavefront 256x256 tile on v_mfma_f32_16x16x32_f16 with one barrier per k tile (see the main loop).
+template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ W,
                                                                  GemmEpilogue ep, void* __restrict__ C, int64_t M,
@@ -184,6 +185,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   constexpr bool WREG = WT || WQ;  // W tiles pass through registers (transposed or dequantised), not the direct-to-LDS path
   static_assert(!WREG || (NS <= 3 && NW == 4), "the register W path is written for two or three stages and 4 wavefronts");
   static_assert(!(WT && WQ), "k-major 8-bit weights are not served");
+  static_assert(!M16 || (NW == 8 && BM == 256 && BN == 256 && !WREG), "the 16x16x32 loop is written for the 8-wavefront 256x256 tile");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
   static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
   constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
@@ -255,6 +257,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     for (int j = 0; j < NT; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  // M16: 16x16 blocks, 4 accumulator registers each
+  constexpr int MT16 = M16 ? WTM / 16 : 1, NT16 = M16 ? WTN / 16 : 1;
+  f32x4 acc16[MT16][NT16];
+#pragma unroll
+  for (int i = 0; i < MT16; ++i)
+#pragma unroll
+    for (int j = 0; j < NT16; ++j) acc16[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // this workgroup's k tiles: kt0 .. kt0 + ktiles - 1 of the matrix (none, if the split runs out)
   const int ktiles_all = static_cast<int>((K + kBK - 1) / kBK);
@@ -457,6 +466,106 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       k_tile(kt, Slot0{}, Slot1{}, std::false_type{});
       if (AH > 1 && kt + 1 < ktiles) k_tile(kt + 1, Slot1{}, Slot0{}, std::false_type{});
     }
+  } else if constexpr (M16) {
+    // ---- 8 wavefronts, v_mfma_f32_16x16x32_f16, one barrier per k tile.
+    // What the measurements on MI355X said, and what this loop is built around:
+    //  * with random operands the card is power-limited, and the 16x16x32 instruction holds ~15 % more flops per
+    //    watt than 32x32x16 (half the accumulator traffic per flop): 1.94 against 1.68 PFLOP/s for bare MFMA loops;
+    //  * a wavefront that issues a direct-to-LDS load stalls until the texture addresser takes it (tens of
+    //    cycles per instruction while data comes from the L2), and cannot issue its MFMAs behind it; of the two
+    //    wavefronts of a SIMD the older one wins the MFMA pipe, so between two barriers w multiplies first and w+4
+    //    second.  Each therefore issues its loads while the other one multiplies: w+4 (W units) right after the
+    //    barrier, w (A units) after its own MFMAs;
+    //  * loads are whole 128-byte lines (half lines cost the L2 path twice the requests), and the barrier sits
+    //    where every wavefront holds all fragments of the tile in registers, so both units of tile kt are free
+    //    from that barrier on.
+    // Ring of five 32 KiB units as in the ping-pong loop: A(0) W(0) A(1) W(1) A(2) ...; k tile = two k32 steps.
+    static_assert(BM == BN, "ring units are one operand's rows of a k tile");
+    constexpr int kUnit = BM * kRowBytes;
+    static_assert(5 * kUnit <= kLdsAlloc, "ring exceeds the LDS");
+    auto wrap5 = [](int v) { return v >= 5 ? v - 5 : v; };
+    const bool hi = wv >= 4;
+    if (hi) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(2);
+    // wavefronts 0-3 load A units, 4-7 W units; block b (8 rows) of a unit goes to wavefront b % 4 of the group,
+    // whose parity is the block's (the lane -> (row, chunk) map depends on it)
+    const unsigned r16 = 2u * (l >> 4) + (((l >> 3) & 1u) ^ (wv & 1u));
+    const unsigned c16 = (l & 7u) ^ r16;
+    const unsigned g16 = (8u * (wv & 3u) + r16) * row_bytes + c16 * 16u;
+    const unsigned g16_step = 32u * row_bytes;
+    auto lane_off16 = [&](int kt) -> unsigned {
+      return (static_cast<int64_t>(kt0 + kt) * kBK + c16 * 8 < K && kt < ktiles) ? g16 + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+    };
+    auto fetch16 = [&](int slot, unsigned voff) {
+      char* base = lds + slot * kUnit + (wv & 3u) * 1024;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        if (hi) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
+      }
+    };
+    // fragment of 16 rows x 32 k: lane l supplies row (l & 15), chunk 4 ks + (l >> 4)
+    unsigned rd16[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) rd16[ks] = lds_chunk_offset(l & 15u, 4u * ks + (l >> 4));
+    const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
+    f16x8 ga[2][MT16], gb[2][NT16];
+    if (hi) {
+      fetch16(1, lane_off16(0));
+      fetch16(3, lane_off16(1));
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(8));
+    } else {
+      fetch16(0, lane_off16(0));
+      fetch16(2, lane_off16(1));
+      fetch16(4, lane_off16(2));
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(16));
+    }
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+#pragma unroll
+    for (int j = 0; j < NT16; ++j) gb[0][j] = *reinterpret_cast<const f16x8*>(lds + kUnit + b_frag + j * 2048 + rd16[0]);
+#pragma unroll
+    for (int i = 0; i < MT16; ++i) ga[0][i] = *reinterpret_cast<const f16x8*>(lds + a_frag + i * 2048 + rd16[0]);
+    DTAS_SCHED_FENCE();
+    // the MFMAs of fragment set `set`; the fragment reads of (pa, pw, ks) into the other set, one before every
+    // other MFMA (a burst of reads backs up the LDS queue, and the wavefront's MFMAs wait behind it)
+    auto step16 = [&](int set, const char* pa, const char* pw, int ks) {
+      constexpr int kReads = MT16 + NT16;
+#pragma unroll
+      for (int i = 0; i < MT16; ++i)
+#pragma unroll
+        for (int j = 0; j < NT16; ++j) {
+          const int q = i * NT16 + j;
+          if (q % 2 == 0 && q / 2 < kReads) {
+            const int r = q / 2;
+            if (r < NT16) gb[set ^ 1][r] = *reinterpret_cast<const f16x8*>(pw + b_frag + r * 2048 + rd16[ks]);
+            else ga[set ^ 1][r - NT16] = *reinterpret_cast<const f16x8*>(pa + a_frag + (r - NT16) * 2048 + rd16[ks]);
+          }
+          acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(gb[set][j], ga[set][i], acc16[i][j], 0, 0, 0);
+          DTAS_SCHED_FENCE();
+        }
+    };
+    static_assert(2 * (MT16 + NT16) <= MT16 * NT16, "fragment reads must fit between the MFMAs of a step");
+    int slot_a = 0, slot_w = 1;  // slots of A(kt), W(kt)
+    for (int kt = 0; kt < ktiles; ++kt) {
+      const char* pa = lds + slot_a * kUnit;
+      const char* pw = lds + slot_w * kUnit;
+      const int next_a = wrap5(slot_a + 2), next_w = wrap5(slot_w + 2);
+      step16(0, pa, pw, 1);
+      // wavefronts 0-3: A(kt+2) into the slot W(kt-1) left at the previous barrier
+      if (!hi && kt > 0) fetch16(wrap5(slot_w + 3), lane_off16(kt + 2));
+      // every fragment of tile kt is in registers and tile kt+1 has landed (0-3: all but the unit just requested)
+      if (hi) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(8));
+      DTAS_SCHED_FENCE();
+      __builtin_amdgcn_s_barrier();
+      DTAS_SCHED_FENCE();
+      if (hi) fetch16(slot_a, lane_off16(kt + 2));  // W(kt+2) into the slot of A(kt)
+      DTAS_SCHED_FENCE();
+      step16(1, lds + next_a * kUnit, lds + next_w * kUnit, 0);
+      slot_a = next_a;
+      slot_w = next_w;
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));  // (loads past the last tile are out of range: zeros, but they do write the LDS)
+    __builtin_amdgcn_s_setprio(0);
   } else if constexpr (NW == 8) {
     // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD).
     // The LDS is a ring of five 32 KiB units, filled in the order A(0) W(0) A(1) W(1) ...: unit u
@@ -784,7 +893,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // therefore moved with device-scope accesses (they pass the L2), ordered by the barriers' waits,
   // rather than with device-scope fences, which write back and invalidate a whole L2 on every use
   // (measured: that made a two-way split slower than no split).
-  if (nsplit > 1) {
+  if (!M16 && nsplit > 1) {
     // (the flag lives in the operand stages, free by now: a second LDS object would make the
     // compiler order every fragment read behind the outstanding direct-to-LDS loads)
     volatile unsigned* is_last = reinterpret_cast<volatile unsigned*>(lds);
@@ -849,6 +958,21 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots;
   char* region = lds + wv * (WTM * kRowB);
   __syncthreads();  // every wavefront is done with the operand stages
+  if constexpr (M16) {
+    // acc16[i][j][v] of lane l is C row i*16 + (l & 15), column j*16 + 4*(l >> 4) + v of the wavefront tile
+#pragma unroll
+    for (int i = 0; i < MT16; ++i) {
+      const unsigned m = i * 16 + (l & 15u);
+#pragma unroll
+      for (int j = 0; j < NT16; ++j) {
+        f16x4 hv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(acc16[i][j][e]);
+        const unsigned slot = j * 4 + (l >> 4);
+        *reinterpret_cast<f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8)) = hv;
+      }
+    }
+  } else {
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
     const unsigned m = i * 32 + (l & 31u);
@@ -862,6 +986,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         const unsigned slot = j * 8 + g * 2 + (l >> 5);
         *reinterpret_cast<f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8)) = hv;
       }
+  }
   }
   // no barrier: a wavefront reads back only what it wrote itself
   const unsigned slot = l % kSlots, rsub = l / kSlots;
@@ -1501,7 +1626,7 @@ int operand_workspace(size_t bytes, void** out) {
   return 0;
 }
 
-template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false>
+template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
                 int64_t K, int nsplit, int batch = 1) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
@@ -1517,7 +1642,7 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   if (tiles * nsplit * batch > 0x7fffffffu) return fail("gemm: too many workgroups");
   GemmEpilogue batched = ep;
   batched.batches = static_cast<unsigned>(batch);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT, WQ>), dim3(static_cast<unsigned>(tiles * nsplit * batch)), dim3(64 * WM * WN), 0,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT, WQ, M16>), dim3(static_cast<unsigned>(tiles * nsplit * batch)), dim3(64 * WM * WN), 0,
                      s, A, W, batched, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
@@ -1667,7 +1792,8 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (bm == 256 && bn == 256)
     return cfg.block == 256 ? launch_mfma<256, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
-                            : launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K, sk);
+           : sk == 1        ? launch_mfma<256, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, 1)
+                            : launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K, sk);  // (K split: the ping-pong loop)
   if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
                                              : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk);
   if (bm == 128 && bn == 256) return ns == 2 ? launch_mfma<128, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
@@ -1745,7 +1871,7 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   const int bm = cfg.tile[0], bn = cfg.tile[1], ns = cfg.unroll >= 2 ? cfg.unroll : 2, b = static_cast<int>(heads);
   if (bm == 256 && bn == 256)
     return cfg.block == 256 ? launch_mfma<256, 256, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b)
-                            : launch_mfma<256, 256, 2, 4, 2>(s, a, w, ep, out, n, m, d, 1, b);
+                            : launch_mfma<256, 256, 2, 4, 2, false, false, true>(s, a, w, ep, out, n, m, d, 1, b);
   if (bm == 256 && bn == 128) return launch_mfma<256, 128, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
   if (bm == 128 && bn == 256) return launch_mfma<128, 256, 2, 2, 2>(s, a, w, ep, out, n, m, d, 1, b);
   if (bm == 128 && bn == 128)
