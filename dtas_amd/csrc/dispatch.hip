@@ -156,7 +156,26 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   // no candidate is faster than it streams W: TB/s measured at M = 64 against a 50280 x 2560 W
   const double w_mb = 2.0 * static_cast<double>(n) * static_cast<double>(k) * 1e-6;
   auto floored = [&](double us, double tbs) { return us > w_mb / tbs ? us : w_mb / tbs; };
-  consider(floored(gemm_rounds(tiles_of(256, 256), kNumCU) * 1.80 * kt, 3.5), 256, 256, 512, 2, 1);
+  {
+    // 256x256 on 8 wavefronts (16x16x32 MFMA): a round of the chip costs ~8 us plus 1.50 us per k tile with every CU
+    // busy; with half of the CUs or fewer busy the card clocks higher and a k tile takes 0.63 of that, linearly in
+    // between.  split_k = 0: the tiles of a partly filled last round are shared by 2..4 workgroups each
+    // (tail_split_256), which costs ~15 / 18 / 21 us to combine the partial tiles.
+    const int64_t tiles = static_cast<int64_t>(tiles_of(256, 256));
+    const int64_t full = tiles / kNumCU, rem = tiles % kNumCU;
+    auto relief = [](double fill) { return fill <= 0.5 ? 0.63 : 0.63 + 0.74 * (fill - 0.5); };
+    double us = static_cast<double>(full) * (8.0 + 1.50 * kt);
+    if (rem > 0) {
+      int split = 1;
+      unsigned unsplit = 0;
+      tail_split_256(M_hi, n, k, &split, &unsplit);
+      if (split >= 2)
+        us += 8.0 + 1.50 * static_cast<double>(ceil_div(ktiles, split)) * relief(static_cast<double>(rem * split) / kNumCU) + 12.0 + 3.0 * (split - 1);
+      else
+        us += 8.0 + 1.50 * kt * relief(static_cast<double>(rem) / kNumCU);
+    }
+    consider(floored(us, 3.5), 256, 256, 512, 2, 0);
+  }
   consider(floored(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.045 * kt, 3.5), 256, 128, 256, 3, 1);
   consider(floored(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 3.1), 128, 128, 256, 2, 1);
   for (int split = 1; split <= 4; ++split) {

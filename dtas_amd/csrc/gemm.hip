@@ -97,6 +97,7 @@ struct GemmEpilogue {
   unsigned tiles_pinned;  // batched launches: an XCD keeps its tiles and walks the problems (see the kernel)
   const half_t* wscale;   // 8-bit W: the fp16 scales [N][K/32]
   int64_t lda;            // k-major W only (P.V): row stride of A in elements when its rows are padded; 0 = K
+  unsigned tiles_unsplit; // one problem only: tiles [0, tiles_unsplit) are computed whole, only the rest is split over nsplit workgroups
 };
 
 // Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):
@@ -199,12 +200,21 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // one problem (which share its W -- the keys or values of an attention head) meet in one L2.
   // With ep.tiles_pinned (the scores: every problem reads the same mask) an XCD instead keeps one
   // span of tiles and walks the problems, so its part of the shared operand stays in its L2.
-  const unsigned total = tiles_m * tiles_n, per_batch = total * nsplit;
+  // With ep.tiles_unsplit (one problem): the first tiles_unsplit tiles -- whole rounds of the chip -- are computed by
+  // one workgroup each; only the tiles of the last, partly filled round are shared by nsplit workgroups, which are
+  // launched after the whole ones.
+  const unsigned total = tiles_m * tiles_n, unsplit = ep.tiles_unsplit;
+  const unsigned per_batch = unsplit + (total - unsplit) * nsplit;
   // (divisions run on the vector ALU; pinning the results to scalar registers keeps every address
   // and buffer descriptor derived from them scalar -- a descriptor left in vector registers turns
   // each load into a loop over its distinct values)
   unsigned batch_u, wgid;
-  if (ep.tiles_pinned && per_batch % kNumXCD == 0) {
+  bool whole = false;
+  if (unsplit > 0) {
+    batch_u = 0;
+    whole = blockIdx.x < unsplit;
+    wgid = whole ? xcd_contiguous_id(blockIdx.x, unsplit) : unsplit * nsplit + xcd_contiguous_id(blockIdx.x - unsplit, per_batch - unsplit);
+  } else if (ep.tiles_pinned && per_batch % kNumXCD == 0) {
     const unsigned span = per_batch / kNumXCD, xcd = blockIdx.x % kNumXCD, local = blockIdx.x / kNumXCD;
     batch_u = __builtin_amdgcn_readfirstlane(local / span);
     wgid = xcd * span + local % span;
@@ -222,7 +232,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 
   // ---- tiles in groups of 8 tile rows walked column-wise
   // nsplit > 1: nsplit consecutive workgroups (same XCD) share a tile and split its k tiles
-  const unsigned pid = __builtin_amdgcn_readfirstlane(wgid / nsplit), z = __builtin_amdgcn_readfirstlane(wgid % nsplit);
+  const unsigned my_split = __builtin_amdgcn_readfirstlane(whole ? 1u : nsplit);
+  const unsigned pid = __builtin_amdgcn_readfirstlane(whole ? wgid : wgid / nsplit), z = __builtin_amdgcn_readfirstlane(whole ? 0u : wgid % nsplit);
   constexpr unsigned kGroup = 8;
   const unsigned width = kGroup * tiles_n;
   const unsigned first_m = (pid / width) * kGroup;
@@ -267,7 +278,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 
   // this workgroup's k tiles: kt0 .. kt0 + ktiles - 1 of the matrix (none, if the split runs out)
   const int ktiles_all = static_cast<int>((K + kBK - 1) / kBK);
-  const int kt_per = (ktiles_all + static_cast<int>(nsplit) - 1) / static_cast<int>(nsplit);
+  const int kt_per = (ktiles_all + static_cast<int>(my_split) - 1) / static_cast<int>(my_split);
   const int kt0 = static_cast<int>(z) * kt_per;
   const int ktiles = ktiles_all - kt0 < kt_per ? (ktiles_all - kt0 > 0 ? ktiles_all - kt0 : 0) : kt_per;
 
@@ -893,43 +904,46 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // therefore moved with device-scope accesses (they pass the L2), ordered by the barriers' waits,
   // rather than with device-scope fences, which write back and invalidate a whole L2 on every use
   // (measured: that made a two-way split slower than no split).
-  if (!M16 && nsplit > 1) {
+  if (my_split > 1) {
     // (the flag lives in the operand stages, free by now: a second LDS object would make the
     // compiler order every fragment read behind the outstanding direct-to-LDS loads)
     volatile unsigned* is_last = reinterpret_cast<volatile unsigned*>(lds);
     constexpr int kTilePairs = BM * BN / 2;  // 8-byte units per partial tile
-    const unsigned tile_g = batch_u * total + pid;  // this tile among all problems' tiles
+    const unsigned tile_g = batch_u * total + pid - unsplit;  // this tile among all problems' tiles
     unsigned long long* tile_ws = reinterpret_cast<unsigned long long*>(ws) + static_cast<size_t>(tile_g) * nsplit * kTilePairs;
     unsigned long long* mine = tile_ws + static_cast<size_t>(z) * kTilePairs + wv * (MT * NT * 8 * 64);
+    // pair q of a lane's accumulators (in whatever order the main loop keeps them)
+    constexpr int kPer = MT * NT * 8;  // 8-byte units per lane and partial tile
+    auto pair_get = [&](int q, int e) -> float {
+      if constexpr (M16) return acc16[q / (NT16 * 2)][(q / 2) % NT16][2 * (q % 2) + e];
+      else return acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8) + e];
+    };
+    auto pair_set = [&](int q, int e, float v) {
+      if constexpr (M16) acc16[q / (NT16 * 2)][(q / 2) % NT16][2 * (q % 2) + e] = v;
+      else acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8) + e] = v;
+    };
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int h = 0; h < 8; ++h) {
-          const f32x2v pr = {acc[i][j][2 * h], acc[i][j][2 * h + 1]};
-          __hip_atomic_store(mine + ((i * NT + j) * 8 + h) * 64 + l, __builtin_bit_cast(unsigned long long, pr),
-                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+    for (int q = 0; q < kPer; ++q) {
+      const f32x2v pr = {pair_get(q, 0), pair_get(q, 1)};
+      __hip_atomic_store(mine + q * 64 + l, __builtin_bit_cast(unsigned long long, pr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     __syncthreads();  // every store of this workgroup has completed; nobody reads the stages any more
     if (t == 0) {
       const unsigned before = __hip_atomic_fetch_add(arrivals + tile_g, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      *is_last = before == nsplit - 1 ? 1u : 0u;
-      if (before == nsplit - 1)  // re-armed for the next launch
+      *is_last = before == my_split - 1 ? 1u : 0u;
+      if (before == my_split - 1)  // re-armed for the next launch
         __hip_atomic_store(arrivals + tile_g, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     const bool last = *is_last != 0;
     if (!last) return;
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    for (int q = 0; q < kPer; ++q) {
+      pair_set(q, 0, 0.f);
+      pair_set(q, 1, 0.f);
+    }
     // The partials are added in split order, but requested kGroup tiles at a time (up to 64 loads per lane):
     // one tile per round trip made the combine cost ~1.2 us per split, which capped useful splits at 4.
-    constexpr int kPer = MT * NT * 8;  // 8-byte loads per lane and partial tile
     constexpr int kGroup = kPer >= 64 ? 1 : 64 / kPer;
     auto add_partials = [&](unsigned k0, auto count_tag) {
       constexpr int COUNT = decltype(count_tag)::value;
@@ -946,13 +960,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
         for (int q = 0; q < kPer; ++q) {
           const f32x2v pr = __builtin_bit_cast(f32x2v, raw[g][q]);
-          acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8)] += pr[0];
-          acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8) + 1] += pr[1];
+          pair_set(q, 0, pair_get(q, 0) + pr[0]);
+          pair_set(q, 1, pair_get(q, 1) + pr[1]);
         }
     };
     unsigned k = 0;
-    for (; k + kGroup <= nsplit; k += kGroup) add_partials(k, std::integral_constant<int, kGroup>{});
-    for (; k < nsplit; ++k) add_partials(k, std::integral_constant<int, 1>{});
+    for (; k + kGroup <= my_split; k += kGroup) add_partials(k, std::integral_constant<int, kGroup>{});
+    for (; k < my_split; ++k) add_partials(k, std::integral_constant<int, 1>{});
   }
 
   constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots;
@@ -1545,104 +1559,148 @@ __global__ void __launch_bounds__(256) attn_pv_rows_kernel(const half_t* __restr
   }
 }
 
-// Split-K workspace of the current device: nsplit fp32 partial tiles per output tile and one
-// arrival counter per tile.  Allocated on first use and grown on demand (the only allocation in
-// the library); the counters are zero between launches (the last arriver of a tile re-arms it).
-// Launches that split K share it, so they must be ordered by one stream.
+// Library-owned scratch memory, one set per (device, stream):
+//  * the split-K workspace: nsplit fp32 partial tiles per shared output tile and one arrival counter per tile
+//    (zero between launches: the last arriver of a tile re-arms it);
+//  * the operand buffer: the fp16 copy of an 8-bit weight matrix (dtas_gemm_q8_f16_fused's two-pass route) or the
+//    padded copy of P (dtas_attn_pv_f16 with a key count that is not a multiple of 8).
+// Allocated on first use by a stream and grown on demand -- the only allocations in the library.  Launches on one
+// stream are ordered by it and share its set; launches on different streams use different sets, so they may overlap.
+// g_ws_mutex is held from the lookup until the launches that use the set are enqueued: a set is never grown (freed
+// and re-allocated: hipFree waits for the device, hence for every launch that may still use it) between a lookup
+// and its launch, also with several host threads.  At most kMaxWsStreams streams per device hold a set; beyond
+// that the set used longest ago is released first.
 constexpr size_t kMaxSplitWsBytes = size_t{1} << 30;
 constexpr int kMaxDevices = 64;
-struct SplitWorkspace {
+constexpr int kMaxWsStreams = 16;
+struct StreamWorkspace {
+  bool used = false;
+  hipStream_t stream = nullptr;
+  uint64_t stamp = 0;
   float* partials = nullptr;
   size_t partial_bytes = 0;
   unsigned* arrivals = nullptr;
   size_t tiles = 0;
+  void* operand = nullptr;
+  size_t operand_bytes = 0;
 };
-SplitWorkspace g_split_ws[kMaxDevices];
-std::mutex g_split_ws_mutex;
+struct DeviceWorkspaces {
+  StreamWorkspace slot[kMaxWsStreams];
+  uint64_t clock = 0;
+};
+DeviceWorkspaces g_ws[kMaxDevices];
+std::recursive_mutex g_ws_mutex;
 
-int split_workspace(size_t partial_bytes, size_t tiles, float** partials, unsigned** arrivals) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("gemm: cannot identify the current device");
-  std::lock_guard<std::mutex> lock(g_split_ws_mutex);
-  SplitWorkspace& w = g_split_ws[dev];
-  if (partial_bytes > w.partial_bytes) {
-    // kernels of earlier launches may still use the old buffer: hipFree waits for the device
-    if (w.partials && hipFree(w.partials) != hipSuccess) return fail("gemm: hipFree of the split-K workspace failed");
-    w.partials = nullptr;
-    w.partial_bytes = 0;
-    const size_t want = partial_bytes < (size_t{32} << 20) ? (size_t{32} << 20) : partial_bytes;
-    if (hipMalloc(reinterpret_cast<void**>(&w.partials), want) != hipSuccess) {
-      (void)hipGetLastError();
-      return fail("gemm: cannot allocate %zu bytes of split-K workspace", want);
-    }
-    w.partial_bytes = want;
-  }
-  if (tiles > w.tiles) {
-    if (w.arrivals && hipFree(w.arrivals) != hipSuccess) return fail("gemm: hipFree of the split-K counters failed");
-    w.arrivals = nullptr;
-    w.tiles = 0;
-    const size_t want = tiles < 4096 ? 4096 : tiles;
-    if (hipMalloc(reinterpret_cast<void**>(&w.arrivals), want * sizeof(unsigned)) != hipSuccess ||
-        hipMemset(w.arrivals, 0, want * sizeof(unsigned)) != hipSuccess) {
-      (void)hipGetLastError();
-      return fail("gemm: cannot allocate the split-K arrival counters");
-    }
-    w.tiles = want;
-  }
-  *partials = w.partials;
-  *arrivals = w.arrivals;
+int release_workspace(StreamWorkspace& w) {
+  // kernels of earlier launches may still use the buffers: hipFree waits for the device
+  if (w.partials && hipFree(w.partials) != hipSuccess) return fail("workspace: hipFree of the split-K partials failed");
+  if (w.arrivals && hipFree(w.arrivals) != hipSuccess) return fail("workspace: hipFree of the split-K counters failed");
+  if (w.operand && hipFree(w.operand) != hipSuccess) return fail("workspace: hipFree of the operand buffer failed");
+  w = StreamWorkspace{};
   return 0;
 }
 
-// A rewritten operand: the fp16 copy of an 8-bit weight matrix (dtas_gemm_q8_f16_fused's two-pass route) or the
-// padded copy of P (dtas_attn_pv_f16 with a key count that is not a multiple of 8).  One buffer per device,
-// allocated on first use and grown on demand like the split-K workspace, and like it shared by the launches
-// that use it (one stream).
-struct OperandWorkspace {
-  void* buf = nullptr;
-  size_t bytes = 0;
-};
-OperandWorkspace g_operand_ws[kMaxDevices];
-
-int operand_workspace(size_t bytes, void** out) {
+// The set of `stream` on the current device (g_ws_mutex held by the caller).
+int stream_workspace(hipStream_t stream, StreamWorkspace** out) {
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("operand buffer: cannot identify the current device");
-  std::lock_guard<std::mutex> lock(g_split_ws_mutex);
-  OperandWorkspace& w = g_operand_ws[dev];
-  if (bytes > w.bytes) {
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("workspace: cannot identify the current device");
+  DeviceWorkspaces& d = g_ws[dev];
+  StreamWorkspace* free_slot = nullptr;
+  StreamWorkspace* oldest = nullptr;
+  for (StreamWorkspace& w : d.slot) {
+    if (w.used && w.stream == stream) {
+      w.stamp = ++d.clock;
+      *out = &w;
+      return 0;
+    }
+    if (!w.used && !free_slot) free_slot = &w;
+    if (w.used && (!oldest || w.stamp < oldest->stamp)) oldest = &w;
+  }
+  if (!free_slot) {
+    if (release_workspace(*oldest) != 0) return -1;
+    free_slot = oldest;
+  }
+  free_slot->used = true;
+  free_slot->stream = stream;
+  free_slot->stamp = ++d.clock;
+  *out = free_slot;
+  return 0;
+}
+
+int split_workspace(hipStream_t stream, size_t partial_bytes, size_t tiles, float** partials, unsigned** arrivals) {
+  StreamWorkspace* w = nullptr;
+  if (stream_workspace(stream, &w) != 0) return -1;
+  if (partial_bytes > w->partial_bytes) {
+    if (w->partials && hipFree(w->partials) != hipSuccess) return fail("gemm: hipFree of the split-K workspace failed");
+    w->partials = nullptr;
+    w->partial_bytes = 0;
+    const size_t want = partial_bytes < (size_t{32} << 20) ? (size_t{32} << 20) : partial_bytes;
+    if (hipMalloc(reinterpret_cast<void**>(&w->partials), want) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail("gemm: cannot allocate %zu bytes of split-K workspace", want);
+    }
+    w->partial_bytes = want;
+  }
+  if (tiles > w->tiles) {
+    if (w->arrivals && hipFree(w->arrivals) != hipSuccess) return fail("gemm: hipFree of the split-K counters failed");
+    w->arrivals = nullptr;
+    w->tiles = 0;
+    const size_t want = tiles < 4096 ? 4096 : tiles;
+    // (cleared on the stream that will use them: a memset on the default stream is not ordered with a non-blocking stream)
+    if (hipMalloc(reinterpret_cast<void**>(&w->arrivals), want * sizeof(unsigned)) != hipSuccess ||
+        hipMemsetAsync(w->arrivals, 0, want * sizeof(unsigned), stream) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail("gemm: cannot allocate the split-K arrival counters");
+    }
+    w->tiles = want;
+  }
+  *partials = w->partials;
+  *arrivals = w->arrivals;
+  return 0;
+}
+
+int operand_workspace(hipStream_t stream, size_t bytes, void** out) {
+  StreamWorkspace* w = nullptr;
+  if (stream_workspace(stream, &w) != 0) return -1;
+  if (bytes > w->operand_bytes) {
     if (bytes > kMaxSplitWsBytes) return fail("operand buffer: a rewritten operand needs %zu bytes (limit %zu)", bytes, kMaxSplitWsBytes);
-    // kernels of earlier launches may still use the old buffer: hipFree waits for the device
-    if (w.buf && hipFree(w.buf) != hipSuccess) return fail("operand buffer: hipFree failed");
-    w.buf = nullptr;
-    w.bytes = 0;
+    if (w->operand && hipFree(w->operand) != hipSuccess) return fail("operand buffer: hipFree failed");
+    w->operand = nullptr;
+    w->operand_bytes = 0;
     const size_t want = bytes < (size_t{64} << 20) ? (size_t{64} << 20) : bytes;
-    if (hipMalloc(&w.buf, want) != hipSuccess) {
+    if (hipMalloc(&w->operand, want) != hipSuccess) {
       (void)hipGetLastError();
       return fail("operand buffer: cannot allocate %zu bytes", want);
     }
-    w.bytes = want;
+    w->operand_bytes = want;
   }
-  *out = w.buf;
+  *out = w->operand;
   return 0;
 }
 
 template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
-                int64_t K, int nsplit, int batch = 1) {
+                int64_t K, int nsplit, int batch = 1, unsigned unsplit = 0) {
   const unsigned tiles_m = static_cast<unsigned>(ceil_div(M, BM)), tiles_n = static_cast<unsigned>(ceil_div(N, BN));
   const size_t tiles = static_cast<size_t>(tiles_m) * tiles_n;
   float* partials = nullptr;
   unsigned* arrivals = nullptr;
   if (batch < 1 || batch > 65535) return fail("gemm: batch must be in [1, 65535], got %d", batch);
+  if (unsplit > 0 && (batch != 1 || unsplit >= tiles || nsplit < 2)) return fail("gemm: a partly split launch takes one problem and a split");
+  const size_t split_tiles = (tiles - unsplit) * batch;  // tiles shared by nsplit workgroups
+  std::unique_lock<std::recursive_mutex> ws_lock;  // held until the launch is enqueued
   if (nsplit > 1) {
-    const size_t bytes = tiles * batch * nsplit * BM * BN * sizeof(float);
+    const size_t bytes = split_tiles * nsplit * BM * BN * sizeof(float);
     if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
-    if (split_workspace(bytes, tiles * batch, &partials, &arrivals) != 0) return -1;
+    ws_lock = std::unique_lock<std::recursive_mutex>(g_ws_mutex);
+    if (split_workspace(s, bytes, split_tiles, &partials, &arrivals) != 0) return -1;
   }
-  if (tiles * nsplit * batch > 0x7fffffffu) return fail("gemm: too many workgroups");
+  const size_t wgs = unsplit + split_tiles * nsplit;
+  if (wgs > 0x7fffffffu) return fail("gemm: too many workgroups");
   GemmEpilogue batched = ep;
   batched.batches = static_cast<unsigned>(batch);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT, WQ, M16>), dim3(static_cast<unsigned>(tiles * nsplit * batch)), dim3(64 * WM * WN), 0,
+  batched.tiles_unsplit = unsplit;
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, NS, WT, WQ, M16>), dim3(static_cast<unsigned>(wgs)), dim3(64 * WM * WN), 0,
                      s, A, W, batched, C, M, N, K, tiles_m, tiles_n, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
@@ -1653,6 +1711,27 @@ inline int mfma_threads(int bm, int bn) { return bm == 256 && bn == 256 ? 512 : 
 inline int mfma_max_stages(int bm, int bn) { return bm + bn >= 512 ? 2 : bm + bn >= 384 ? 3 : 4; }
 
 }  // namespace
+
+// The 8-wavefront 256x256 tile when the library chooses: whole rounds of the chip run one workgroup per tile; the
+// tiles of a last, partly filled round are shared by 2..4 workgroups each (as many as still fit the chip at once),
+// which split K and meet in the workspace -- a round of half or a third the length instead of a whole one.
+// Fewer tiles than CUs in all: every tile is split that way.
+void tail_split_256(int64_t M, int64_t N, int64_t K, int* nsplit, unsigned* unsplit) {
+  const int64_t tiles = ceil_div(M, 256) * ceil_div(N, 256), ktiles = ceil_div(K, kBK);
+  const int64_t rem = tiles % kNumCU;
+  *nsplit = 1;
+  *unsplit = 0;
+  if (rem == 0) return;
+  int64_t split = kNumCU / rem;
+  if (split > 4) split = 4;
+  while (split >= 2 && ktiles / split < 8) --split;  // (a part should still be long against its prologue and the combine)
+  // a round that fills only part of the chip runs at a higher clock; against that, parts that fill it again gain
+  // only when K is long (measured: 128 tiles in two parts each break even at K = 4096 and win 20 % at K = 11008)
+  if (split >= 2 && rem * split > 3 * kNumCU / 4 && ktiles < 128) return;
+  if (split < 2) return;
+  *nsplit = static_cast<int>(split);
+  *unsplit = static_cast<unsigned>(tiles - rem);
+}
 
 // launch_args: {grid, 1, 1, block, static LDS bytes, tiles along M, tiles along N}
 int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64_t la[7]) {
@@ -1681,10 +1760,13 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     // cfg.unroll = LDS stages (the depth of the load pipeline); 0 or 1 = as many as fit
     if (cfg.unroll < 0 || cfg.unroll > mfma_max_stages(bm, bn))
       return fail("gemm: the %dx%d tile holds at most %d LDS stages, got %d", bm, bn, mfma_max_stages(bm, bn), cfg.unroll);
-    const int nsplit = cfg.split_k < 1 ? 1 : cfg.split_k;
+    int nsplit = cfg.split_k < 1 ? 1 : cfg.split_k;
     if (nsplit > 16) return fail("gemm: split_k must be in [1, 16], got %d", cfg.split_k);
+    // split_k = 0 on the 8-wavefront 256x256 tile: only the tiles of a last, partly filled round are split
+    unsigned unsplit = 0;
+    if (cfg.split_k == 0 && bm == 256 && bn == 256 && !four_waves) tail_split_256(M, N, K, &nsplit, &unsplit);
     if (tm * tn * nsplit > 0x7fffffff) return fail("gemm: too many workgroups");
-    la[0] = tm * tn * nsplit;
+    la[0] = unsplit + (tm * tn - unsplit) * nsplit;
     la[3] = four_waves ? 256 : mfma_threads(bm, bn);
     // 256x256: a ring of five 32 KiB operand units; else whole-tile stages
     la[4] = bm == 256 && bn == 256 ? 5 * 256 * kRowBytes
@@ -1791,9 +1873,13 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   const int ns = cfg.unroll >= 2 ? cfg.unroll : 0;
   const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (bm == 256 && bn == 256)
-    return cfg.block == 256 ? launch_mfma<256, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
-           : sk == 1        ? launch_mfma<256, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, 1)
-                            : launch_mfma<256, 256, 2, 4, 2>(s, a, w, b, c, M, N, K, sk);  // (K split: the ping-pong loop)
+  {
+    if (cfg.block == 256) return launch_mfma<256, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk);
+    int split = sk;
+    unsigned unsplit = 0;
+    if (cfg.split_k == 0) tail_split_256(M, N, K, &split, &unsplit);  // (split_k >= 1: that split for every tile)
+    return launch_mfma<256, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, split, 1, unsplit);
+  }
   if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
                                              : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk);
   if (bm == 128 && bn == 256) return ns == 2 ? launch_mfma<128, 256, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
@@ -2025,7 +2111,8 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   };
   if (pad_heads == 0) return launch(a, w, out, b);
   void* buf = nullptr;
-  if (operand_workspace(static_cast<size_t>(pad_heads) * n * m_pad * 2, &buf) != 0) return -1;
+  std::lock_guard<std::recursive_mutex> ws_lock(g_ws_mutex);  // until every launch that uses the buffer is enqueued
+  if (operand_workspace(s, static_cast<size_t>(pad_heads) * n * m_pad * 2, &buf) != 0) return -1;
   ep.stride_a = n * m_pad;
   ep.lda = m_pad;
   for (int64_t h0 = 0; h0 < heads; h0 += pad_heads) {
@@ -2073,7 +2160,8 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
   // library-owned fp16 buffer, then the fp16 GEMM with everything its table offers.  A cfg selects the first route.
   if (!user && !(M <= 64 && K <= 4096)) {
     void* wbuf = nullptr;
-    if (operand_workspace(static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
+    std::lock_guard<std::recursive_mutex> ws_lock(g_ws_mutex);  // until both launches are enqueued
+    if (operand_workspace(static_cast<hipStream_t>(stream), static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
     if (dtas_decode_q8_f16(Wq, scale, wbuf, N, K, nullptr, stream) != 0) return -1;
     return dtas_gemm_f16_fused(A, wbuf, bias, res1, res2, C, M, N, K, epilogue, nullptr, stream);
   }

@@ -5,7 +5,7 @@ enumerate block tiles as i x j wavefronts of micro_x x micro_y matrix-core block
 those that do not fit shared memory / registers (:46-70) and rank by a roofline estimate in which a
 tile's throughput is min(matrix-core peak, bandwidth * flops-per-byte of the tile) and the job costs
 ceil(tiles / SMs) rounds (:148-262).  The candidate set is what libdtas_gfx950.so has kernels for:
-32x32x16 MFMA tiles from 64x64 to 256x256 with 2 to 4 LDS stages, with K split over up to 4 workgroups
+MFMA tiles from 64x64 to 256x256 (16x16x32 on the largest, 32x32x16 below) with 2 to 4 LDS stages, with K split over up to 4 workgroups
 per tile when M x N yields few tiles, plus, for M <= 64, the weight-streaming 16x16x32 kernel whose
 wavefronts split K.  The order is the one on-GPU sweeps favoured;
 with a GPU present the Engine times the top-k anyway.
@@ -34,7 +34,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
     def preferred(self, m_hi: int, N: int, K: int = 4096):
         """(tile_m, tile_n, stages, split_k) under the cost model fitted to sweeps on an MI355X (the same
         one the library's built-in table uses): time = rounds of workgroups over the chip x time of one
-        k tile x k tiles.  One k tile with every CU busy: 256x256 1.80 us, 256x128 (3 stages) 1.045 us,
+        k tile x k tiles.  One k tile with every CU busy: 256x256 see below, 256x128 (3 stages) 1.045 us,
         128x128 0.665 us (4 stages, one workgroup per CU) or 1.14 us per round of two per CU (2 stages);
         a partly filled last round costs 0.55 + 0.45 * fill of a full one (0.8 + 0.2 * fill for 128x128 with 4 stages
         in a single round); 64x64 0.33 us per k tile up to
@@ -55,7 +55,20 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         tiles = lambda bm, bn: cdiv(m_hi, bm) * cdiv(N, bn)
         w_mb = 2.0 * float(N) * float(K) * 1e-6
         floored = lambda us, tbs: us if us > w_mb / tbs else w_mb / tbs     # W streams at 3.1 .. 4.3 TB/s, by tile
-        cands = [(floored(rounds(tiles(256, 256), cus) * 1.80 * ktiles, 3.5), (256, 256, 2, 1)),
+        # 256x256 on 8 wavefronts: ~8 us per round of the chip plus 1.50 us per k tile with every CU busy, 0.63 of that
+        # with half of the CUs or fewer busy (the card clocks higher), linear in between; split_k = 0: the tiles of
+        # a partly filled last round are shared by 2..4 workgroups each (~15 / 18 / 21 us to combine)
+        t256 = tiles(256, 256)
+        full, rem = divmod(t256, cus)
+        relief = lambda fill: 0.63 if fill <= 0.5 else 0.63 + 0.74 * (fill - 0.5)
+        us256 = full * (8.0 + 1.50 * ktiles)
+        if rem:
+            split, _ = self.tail_split_256(m_hi, N, K)
+            if split >= 2:
+                us256 += 8.0 + 1.50 * cdiv(ktiles, split) * relief(rem * split / cus) + 12.0 + 3.0 * (split - 1)
+            else:
+                us256 += 8.0 + 1.50 * ktiles * relief(rem / cus)
+        cands = [(floored(us256, 3.5), (256, 256, 2, 0)),
                  (floored(rounds(tiles(256, 128), cus) * 1.045 * ktiles, 3.5), (256, 128, 3, 1)),
                  (floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1))]
         for split in (1, 2, 3, 4):
@@ -81,6 +94,26 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 best = c
         self._model_us = best[0]
         return best[1]
+
+    def tail_split_256(self, M: int, N: int, K: int):
+        """(parts, tiles left whole) for split_k = 0 on the 8-wavefront 256x256 tile: whole rounds of the chip
+        run one workgroup per tile, the tiles of a last, partly filled round are shared by 2..4 workgroups each
+        (as many as still fit the chip at once, each keeping 8 k tiles or more) -- unless the parts would fill more
+        than three quarters of the chip and K is short (a partly filled round clocks higher; libdtas: tail_split_256)."""
+        cdiv = lambda a, b: -(-a // b)
+        cus = self.arch.num_sm
+        tiles, ktiles = cdiv(M, 256) * cdiv(N, 256), cdiv(K, 64)
+        rem = tiles % cus
+        if rem == 0:
+            return 1, 0
+        split = min(cus // rem, 4)
+        while split >= 2 and ktiles // split < 8:
+            split -= 1
+        if split >= 2 and rem * split > 3 * cus // 4 and ktiles < 128:
+            return 1, 0
+        if split < 2:
+            return 1, 0
+        return split, tiles - rem
 
     def prefers_skinny(self, m_hi: int, N: int, K: int) -> bool:
         """M <= 32: the W-streaming kernel (about 3.5 TB/s of W, slower as M grows) against the model's
@@ -120,13 +153,15 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 c = MFMAConfig()
                 c.micro_shape_x, c.micro_shape_y, c.stages = mx, my, stages
                 if (mx, my) == (4, 4):
-                    # the 256x256 kernel runs 2x4 wavefronts of 128x64 (two per SIMD, alternating phases)
+                    # the 256x256 kernel runs 2x4 wavefronts of 128x64 (two per SIMD)
                     c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 2, 4, 4, 2, 512
                 if not self.check_valid(c):
                     continue
                 tiles = -(-m_hi // tm) * -(-N // tn)
                 c.num_wave = -(-tiles // self.arch.num_sm)
                 splits = [1] + [sk for sk in (2, 3, 4) if tiles * sk <= 4 * self.arch.num_sm and -(-K // 64) // sk >= 8]
+                if c.block_threads == 512:
+                    splits = [0] + splits   # 0: only the tiles of a partly filled last round are split
                 for sk in splits:
                     cs = MFMAConfig().from_dict(c.to_dict())
                     cs.split_k, cs.num_wave = sk, -(-tiles * sk // self.arch.num_sm)

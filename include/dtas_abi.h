@@ -105,7 +105,9 @@ typedef struct dtas_config {
   int32_t unroll;   /* elementwise/GEMV: independent vector accesses in flight per thread; row
                        reductions: rows a lane group takes per trip (1, 2, 4); GEMM: LDS stages (0 = max) */
   int32_t tile[3];  /* GEMM: workgroup tile M, N, K; GEMV: rows per workgroup, -, - */
-  int32_t split_k;  /* GEMM (MFMA): workgroups that share a tile and split its K extent, 1..16 (1 = none) */
+  int32_t split_k;  /* GEMM (MFMA): workgroups that share a tile and split its K extent, 1..16 (1 = none).
+                     * 0 on the 256x256 tile with 512 threads: whole rounds of the chip are not split, the tiles of a
+                     * last, partly filled round are shared by 2..4 workgroups each (elsewhere 0 means 1) */
   int64_t grid_cap; /* upper limit on workgroups (then the kernel loops); 0 = no limit */
 } dtas_config;
 

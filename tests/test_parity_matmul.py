@@ -264,6 +264,54 @@ def test_gemm_split_k_many_launches_back_to_back():
     assert float((outs[0].float() - ref).abs().max()) < 2e-2
 
 
+def test_gemm_split_k_on_two_streams_at_once():
+    # each stream has its own partial tiles and arrival counters: launches that split K may overlap.
+    # Two streams of the default priority take turns launching different problems without any
+    # synchronisation in between; every result must equal the bits of the same launch made alone.
+    g = torch.Generator(device="cuda").manual_seed(11)
+    probs = []
+    for (M, N, K) in ((64, 4096, 4096), (48, 2048, 8192)):
+        a = torch.randn(M, K, device="cuda", generator=g).half()
+        w = (torch.randn(N, K, device="cuda", generator=g) * 0.02).half()
+        alone = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        ops.gemm(a, w, None, alone)                     # the built-in row: 64x64 tiles, K split over workgroups
+        assert _lib.select_bucket(_lib.OP_GEMM_F16, M, N, K).config.split_k > 1
+        probs.append((a, w, alone))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.empty_like(probs[i][2]) for _ in range(40)] for i in range(2)]
+    for rep in range(40):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                ops.gemm(probs[i][0], probs[i][1], None, outs[i][rep])
+    torch.cuda.synchronize()
+    for i in range(2):
+        for o in outs[i]:
+            assert torch.equal(o, probs[i][2])
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 1000, 4096), (1536, 4096, 2048), (1100, 5000, 1024), (8192 + 256, 4096, 512)])
+def test_gemm_256_tile_splits_only_its_last_round(oracle, M, N, K):
+    # split_k = 0 on the 8-wavefront tile: whole rounds of the chip one workgroup per tile, the tiles of the
+    # partly filled last round shared by several; the launch description tells how many
+    a, w = _inputs(M, N, K, M + N)
+    bias = np.random.default_rng(5).uniform(-1, 1, N).astype(np.float16)
+    c = cfg(variant=_lib.GEMM_MFMA, block=512, vec=8, unroll=2, tile=[256, 256, 64], split_k=0)
+    tiles, ktiles = -(-M // 256) * -(-N // 256), -(-K // 64)
+    info = _lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c)
+    rem = tiles % 256
+    assert rem > 0
+    split, rest = divmod(info.launch_args[0] - (tiles - rem), rem)
+    assert rest == 0 and 1 <= split <= 4 and rem * split <= 256 and (split == 1 or ktiles // split >= 8)
+    out = Guarded((M, N), torch.float16)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c)
+    got = out.check()
+    _check(got, oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+    again = Guarded((M, N), torch.float16)
+    ops.gemm(dev(a), dev(w), dev(bias), again.t, c)
+    assert_bits_equal(again.check(), got)
+
+
 def test_gemm_split_k_errors():
     a, w = _inputs(64, 64, 64, 1)
     with pytest.raises(_lib.DtasError, match="split_k"):
