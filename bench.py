@@ -3,11 +3,12 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-sweep] [--no-cpu]
 
-A "step" is one call of the workload's kernel through the C ABI on synthetic, seeded inputs that are
-already resident in device memory.  The headline workload is the elementwise fp32 -> fp16 cast over
-[4096, 4096] (the largest n of the elementwise sweep); buffers rotate through a pool larger than the
-256 MiB Infinity Cache so that every step streams from HBM.  W warm-up steps, then exactly K timed
-steps between two device synchronisations; `value` = algorithmic bytes * K / that time.
+A "step" is one pass of the workload's kernel over its whole pool of synthetic, seeded inputs, all
+resident in device memory: one call through the C ABI per buffer set of the pool (`launches_per_step` in
+`config`).  The headline workload is the elementwise fp32 -> fp16 cast over [4096, 4096] (the largest n
+of the elementwise sweep); the pool is larger than 3x the 256 MiB Infinity Cache so that every launch
+streams from HBM.  W warm-up steps, then exactly K timed steps between two device synchronisations;
+`value` = algorithmic bytes of those launches / that time.
 
 The same JSON line also carries
   roofline     : the workload's kernel against MI355X's published peak (HBM 8 TB/s, or dense fp16
@@ -15,8 +16,12 @@ The same JSON line also carries
                  duration measured with HIP events on the launch stream inside the timed region;
   cpu_baseline : the CPU oracle (a port of the PrimFunc loop nest, oracle/cpu_ref.c) on a bounded
                  sample of the same workload, on this machine's host cores;
+  roofline.families : the other families of the metric in short -- the large-n fraction of the HBM roof for
+                 add / copy / casts / RMSNorm / layer norm / softmax / each GEMV shape, TFLOP/s and the fraction
+                 of the MFMA roof for the GEMM at M = 2048 / 4096 / 8192 per (N, K);
+  cpu_baseline.families : the oracle on bounded samples of a GEMV and a GEMM point;
   sweep        : every op family over the dynamic extent n (GB/s or TFLOP/s and roofline fraction),
-                 HBM-streaming (rotating buffers) unless marked cache-resident.
+                 all of them HBM-streaming (rotating buffer sets, the GEMM's W included).
 One GPU only: `--gpus N` with N > 1 exits with a message.
 """
 from __future__ import annotations
@@ -103,6 +108,12 @@ def _workload(name: str, n: int, extra=None):
         R = 32 * n
         make = lambda s: (normal((R, n), s, 2.0), empty((R, n)))
         return make, lambda b: call(L.dtas_softmax_f16, P(b[0]), P(b[1]), R, n, None, stream), 2 * 2 * R * n, 0
+    if name == "softmax_f32_f16":
+        # the reference's published softmax sweep: fp32 in, fp16 out, 12800 rows x n
+        # (experiment/dtas_tuned/general_reduction/softmax/row_12800/top10_256_10_nounroll/latency.json)
+        R = 12800
+        make = lambda s: (normal((R, n), s, 2.0, torch.float32), empty((R, n)))
+        return make, lambda b: call(L.dtas_softmax_f32_f16, P(b[0]), P(b[1]), R, n, None, stream), (4 + 2) * R * n, 0
     if name == "gemv_f16":
         N, K = extra
         make = lambda s: (normal((1, K), s), normal((N, K), s + 100, 0.02), empty((1, N)))
@@ -177,8 +188,7 @@ def _workload(name: str, n: int, extra=None):
                 8 * n * V + 4, 0)
     if name == "gemm_f16":
         N, K = extra
-        wt = normal((N, K), 100, 0.02)
-        make = lambda s: (normal((n, K), s), wt, empty((n, N)))
+        make = lambda s: (normal((n, K), s), normal((N, K), 100 + s, 0.02), empty((n, N)))
         return (make, lambda b: call(L.dtas_gemm_f16, P(b[0]), P(b[1]), None, P(b[2]), n, N, K, None, stream),
                 2 * (n * K + N * K + n * N), 2 * n * N * K)
     if name == "attn_scores_f16_f32":
@@ -245,15 +255,15 @@ def make_pool(make, streaming: bool, max_bytes: int = 6 << 30):
 
 
 def time_kernel(calls, steps: int, warmup: int, min_warm_s: float = 0.2):
-    """(wall seconds for `steps` calls between two synchronisations, device seconds per call from a
+    """(wall seconds for `steps` steps between two synchronisations, device seconds per launch from a
     pair of HIP events recorded on the launch stream before the first and after the last call).
-    Launches are issued back to back, so device seconds / steps is the average launch duration
-    (kernel time plus the inter-kernel gap, which is what a caller sees).  Warm-up runs at least
-    `warmup` calls and at least `min_warm_s` of them: clocks take a moment to settle."""
+    A step is one pass over the pool: len(calls) launches, issued back to back, so device seconds / launches
+    is the average launch duration (kernel time plus the inter-kernel gap, which is what a caller sees).
+    Warm-up runs at least `warmup` steps and at least `min_warm_s`: clocks take a moment to settle."""
     import torch
 
     t0, i = time.perf_counter(), 0
-    while i < warmup or time.perf_counter() - t0 < min_warm_s:
+    while i < warmup * len(calls) or time.perf_counter() - t0 < min_warm_s:
         calls[i % len(calls)]()
         i += 1
         if i % 64 == 0:
@@ -262,12 +272,13 @@ def time_kernel(calls, steps: int, warmup: int, min_warm_s: float = 0.2):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     start.record()
-    for k in range(steps):
-        calls[(i + k) % len(calls)]()
+    for _ in range(steps):
+        for c in calls:
+            c()
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, start.elapsed_time(stop) * 1e-3 / steps
+    return wall, start.elapsed_time(stop) * 1e-3 / (steps * len(calls))
 
 
 def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool = True, min_region_s: float = 2e-3) -> dict:
@@ -275,10 +286,10 @@ def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool =
     pool = make_pool(make, streaming)
     calls = [bind(b) for b in pool]
     wall, per_launch = time_kernel(calls, steps, warmup)
-    # short kernels: lengthen the timed region so that event and synchronisation costs vanish
-    if per_launch * steps < min_region_s:
-        steps2 = min(20000, int(min_region_s / max(per_launch, 1e-7)) + 1)
-        wall2, per_launch = time_kernel(calls, steps2, 0, 0.0)
+    # short regions: lengthen the timed region so that event and synchronisation costs vanish
+    if per_launch * steps * len(calls) < min_region_s:
+        steps2 = min(20000, int(min_region_s / max(per_launch * len(calls), 1e-7)) + 1)
+        _, per_launch = time_kernel(calls, steps2, 0, 0.0)
     out = {"op": name, "n": n, "us": round(per_launch * 1e6, 3), "ms_per_step": wall * 1e3 / steps,
            "bytes": nbytes, "flops": flops, "pool": len(pool), "gbs": nbytes / per_launch / 1e9}
     if extra:
@@ -356,6 +367,8 @@ def sweep(steps: int, warmup: int) -> list:
     for op in ("add_f16", "copy_f16", "cast_f32_f16", "cast_f16_f32", "rms_norm_f16", "layer_norm_f32_f16", "softmax_f16"):
         for n in SWEEP_N:
             rows.append(measure(op, n, None, steps, warmup))
+    for n in (1024, 2048, 4096):   # the reference's published softmax form: fp32 in, 12800 rows x n
+        rows.append(measure("softmax_f32_f16", n, None, steps, warmup))
     for nk in GEMV_SHAPES:
         rows.append(measure("gemv_f16", 1, nk, steps, warmup))
     for nk in GEMV_SHAPES:
@@ -374,22 +387,81 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("layer_norm_f32", n, None, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
-            rows.append(measure("gemm_f16", m, nk, max(10, steps // 2), max(2, warmup // 2), streaming=m < 2048))
+            rows.append(measure("gemm_f16", m, nk, steps, warmup))
     # the model's own fused shapes (dolly-v2-3b: hidden 2560, 32 heads of 80)
     for m in (1, 16, 256, 2048):   # m = 1: the decode forms (fused_NT_matmul8_add5_add7_add7, ..9_add6_gelu1) on the GEMV kernel
-        rows.append(measure("gemm_add2_f16", m, (2560, 2560), max(10, steps // 2), max(2, warmup // 2)))
-        rows.append(measure("gemm_gelu_f16", m, (10240, 2560), max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure("gemm_add2_f16", m, (2560, 2560), steps, warmup))
+        rows.append(measure("gemm_gelu_f16", m, (10240, 2560), steps, warmup))
         if m == 1:
             continue
-        rows.append(measure("gemm_q8_f16", m, (7680, 2560), max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure("gemm_q8_f16", m, (7680, 2560), steps, warmup))
     for n in (128, 1024, 2048):
-        rows.append(measure("attn_scores_f16_f32", n, None, max(10, steps // 2), max(2, warmup // 2)))
-        rows.append(measure("attn_pv_f16", n, None, max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure("attn_scores_f16_f32", n, None, steps, warmup))
+        rows.append(measure("attn_pv_f16", n, None, steps, warmup))
     rows.append(measure("attn_pv_f16", 1, (1, 2048), steps, warmup))      # matmul10: decoding against 2048 keys
     # a sequence length off every vector width: rows that start at any element
     for op in ("softmax_f16", "attn_scores_f16_f32", "attn_pv_f16"):
-        rows.append(measure(op, 1025, None, max(10, steps // 2), max(2, warmup // 2)))
+        rows.append(measure(op, 1025, None, steps, warmup))
     return rows
+
+
+def families(rows: list) -> dict:
+    """The metric's families in short, from the sweep rows: fraction of the HBM roof at the largest n of the
+    memory-bound ops, TFLOP/s and fraction of the MFMA roof of the GEMM at M >= 2048."""
+    out = {}
+    for op in ("add_f16", "copy_f16", "cast_f32_f16", "cast_f16_f32", "rms_norm_f16", "layer_norm_f32_f16", "softmax_f16"):
+        big = [r for r in rows if r["op"] == op and r["n"] == 4096 and "NK" not in r]
+        if big:
+            out[f"{op} n=4096"] = {"GB/s": round(big[0]["gbs"], 1), "frac": round(big[0]["frac"], 3)}
+    for r in rows:
+        if r["op"] == "softmax_f32_f16":
+            out[f"softmax_f32_f16 12800x{r['n']}"] = {"GB/s": round(r["gbs"], 1), "frac": round(r["frac"], 3), "us": r["us"]}
+        if r["op"] == "gemv_f16":
+            out[f"gemv_f16 {r['NK'][0]}x{r['NK'][1]}"] = {"GB/s": round(r["gbs"], 1), "frac": round(r["frac"], 3)}
+        if r["op"] == "gemm_f16" and r["n"] >= 2048:
+            out[f"gemm_f16 M={r['n']} {r['NK'][0]}x{r['NK'][1]}"] = {"TFLOP/s": round(r["tflops"], 1), "frac": round(r["frac"], 3)}
+        if r["op"] == "gemm_f16" and r["n"] in (16, 64, 256):
+            out[f"gemm_f16 M={r['n']} {r['NK'][0]}x{r['NK'][1]}"] = {"us": r["us"], "W TB/s": round(2e-12 * r["NK"][0] * r["NK"][1] / (r["us"] * 1e-6), 2),
+                                                                    "bound": r["bound"], "frac": round(r["frac"], 3)}
+    return out
+
+
+def cpu_families(budget_s: float = 6.0) -> dict:
+    """The oracle on bounded samples of a GEMV and a GEMM point (one thread and all host cores)."""
+    import numpy as np
+
+    import oracle
+
+    oracle.build()
+    rng = np.random.default_rng(5)
+    cores = min(oracle.c.max_threads(), len(os.sched_getaffinity(0)))
+
+    def rate(fn, work, budget):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            el = time.perf_counter() - t0
+            if el > budget or reps >= 50:
+                return work * reps / el, reps
+
+    N, K = 4096, 4096
+    x = rng.standard_normal((1, K)).astype(np.float16)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    gemv_bytes = 2 * N * K + 2 * K + 2 * N
+    g1, r1 = rate(lambda: oracle.c.gemm(x, w, threads=1), gemv_bytes, budget_s * 0.2)
+    gn, rn = rate(lambda: oracle.c.gemm(x, w, threads=cores), gemv_bytes, budget_s * 0.1)
+    M = 64   # 64 of the rows of the M-sweep's problems against the whole W
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    flops = 2.0 * M * N * K
+    f1, q1 = rate(lambda: oracle.c.gemm(a, w, threads=1), flops, budget_s * 0.4)
+    fn_, qn = rate(lambda: oracle.c.gemm(a, w, threads=cores), flops, budget_s * 0.3)
+    return {"gemv_f16 4096x4096": {"value": round(g1 / 1e9, 3), "unit": "GB/s", "cores": 1, "passes": r1,
+                                   "all_cores": {"value": round(gn / 1e9, 3), "cores": cores, "passes": rn}},
+            "gemm_f16 N=K=4096": {"value": round(f1 / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "passes": q1,
+                                  "sample": f"{M} rows of A against the whole W (the oracle is row-parallel: the rate does not depend on M)",
+                                  "all_cores": {"value": round(fn_ / 1e12, 5), "cores": cores, "passes": qn}}}
 
 
 def recorded_traffic(workload_key: str):
@@ -409,7 +481,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cast_f32_f16",
-                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | layer_norm_f32 | softmax_f16 | attn_scores_f16_f32 | attn_pv_f16 | "
+                    help="cast_f32_f16 | cast_f16_f32 | add_f16 | copy_f16 | rms_norm_f16 | layer_norm_f32_f16 | layer_norm_f32 | softmax_f16 | softmax_f32_f16 (12800 rows x n) | attn_scores_f16_f32 | attn_pv_f16 | "
                          "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | split3_f16 | swap_axes_f16 | attn_mask_f16 | softmax_temperature_f32 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
@@ -451,6 +523,8 @@ def main() -> int:
         workload_key = f"{args.workload} [n={args.n}, 2560]"
     elif args.workload == "softmax_f16":
         workload_key = f"{args.workload} [{32 * args.n}, n={args.n}]"
+    elif args.workload == "softmax_f32_f16":
+        workload_key = f"{args.workload} [12800, n={args.n}]"
     elif args.workload in ("attn_scores_f16_f32", "attn_pv_f16"):
         workload_key = f"{args.workload} [32 heads of 80, n=m={args.n}]"
     elif extra is None:
@@ -461,8 +535,9 @@ def main() -> int:
         workload_key = f"{args.workload} M={args.n} NxK={args.nk}"
     line = {
         "metric": METRIC,
-        "value": round(head["flops"] * args.steps / (head["ms_per_step"] * 1e-3 * args.steps) / 1e12, 3) if is_gemm
-        else round(head["bytes"] / (head["ms_per_step"] * 1e-3) / 1e9, 3),
+        # one step = one launch per buffer set of the pool
+        "value": round(head["flops"] * head["pool"] / (head["ms_per_step"] * 1e-3) / 1e12, 3) if is_gemm
+        else round(head["bytes"] * head["pool"] / (head["ms_per_step"] * 1e-3) / 1e9, 3),
         "unit": "TFLOP/s" if is_gemm else "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(head["ms_per_step"], 6),
@@ -470,7 +545,7 @@ def main() -> int:
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": workload_key,
                    "buffers": "rotating pool > 3x Infinity Cache" if not args.cache_resident else "single set (cache-resident)",
-                   "pool_sets": head["pool"],
+                   "pool_sets": head["pool"], "launches_per_step": head["pool"],
                    "kernel": info.name.decode() if info is not None else args.workload,
                    "launch": list(info.launch_args)[:5] if info is not None else None},
         "roofline": {
@@ -490,7 +565,10 @@ def main() -> int:
     else:
         line["cpu_baseline"] = None
     if not args.no_sweep:
-        rows = sweep(max(20, args.steps // 4), max(3, args.warmup // 4))
+        rows = sweep(max(3, args.steps // 40), 1)
+        line["roofline"]["families"] = families(rows)
+        if line["cpu_baseline"] is not None:
+            line["cpu_baseline"]["families"] = cpu_families()
         line["sweep"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
                           if k in ("op", "n", "NK", "us", "gbs", "tflops", "bound", "frac")} for r in rows]
         if args.out:

@@ -10,8 +10,8 @@
 //
 // MFMA kernel (M > 64)
 //   tile     : BM x BN x 64 per workgroup; WM x WN wavefronts (8 for 256x256, else 4), each owning
-//              (BM/WM) x (BN/WN) as 32x32 blocks of v_mfma_f32_32x32x16_f16, fp32 accumulators
-//              in registers.  Both operands are K-contiguous, so a tile row is one 128-byte
+//              (BM/WM) x (BN/WN) as 32x32 blocks of v_mfma_f32_32x32x16_f16 (16x16 blocks of
+//              v_mfma_f32_16x16x32_f16 on the 8-wavefront tile), fp32 accumulators in registers.  Both operands are K-contiguous, so a tile row is one 128-byte
 //              line = 8 chunks of 16 bytes.
 //   global   : 128-bit buffer loads that write LDS directly (no register staging, no
 //              ds_write): one wavefront instruction fills one 1 KiB block = 8 tile rows; which
@@ -26,11 +26,11 @@
 //              tile, the loads of tile k+2 are issued right after it into the stage just
 //              vacated, and the first fragments of tile k+1 are read under the last MFMAs of
 //              tile k.  The interleaving is pinned with scheduling barriers.
-//              8-wavefront tile (256x256): wavefronts w and w+4 share a SIMD and alternate
-//              roles ("ping-pong"): while one issues the 8 MFMAs of a step, the other reads its
-//              next fragments and issues its share of the next tile's loads; a workgroup
-//              barrier separates the phases, group 1 runs one phase behind group 0, so the MFMA
-//              pipe of every SIMD always has exactly one wavefront feeding it.
+//              8-wavefront tile (256x256): v_mfma_f32_16x16x32_f16 (more flops per watt than 32x32x16,
+//              and the card is power-limited on random operands), a whole k32 step of fragments in
+//              registers, one barrier per k tile; wavefronts w and w+4 share a SIMD, the older one
+//              wins the MFMA pipe, and each requests its share of the next units while the other
+//              multiplies (a wavefront that issues a load stalls until the load path takes it).
 //   epilogue : accumulators -> fp16 -> wavefront-private LDS region (xor-swizzled 8-byte
 //              slots) -> 8-byte coalesced row stores with the bias added on the way out.
 //   launch   : workgroup ids are remapped so that each XCD (own L2) works on a compact patch of
@@ -186,7 +186,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   constexpr bool WREG = WT || WQ;  // W tiles pass through registers (transposed or dequantised), not the direct-to-LDS path
   static_assert(!WREG || (NS <= 3 && NW == 4), "the register W path is written for two or three stages and 4 wavefronts");
   static_assert(!(WT && WQ), "k-major 8-bit weights are not served");
-  static_assert(!M16 || (NW == 8 && BM == 256 && BN == 256 && !WREG), "the 16x16x32 loop is written for the 8-wavefront 256x256 tile");
+  static_assert(M16 == (NW == 8) && (!M16 || (BM == 256 && BN == 256 && !WREG)), "8 wavefronts: the 256x256 tile on the 16x16x32 loop, and only it");
   static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
   static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
   constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
@@ -490,7 +490,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     //  * loads are whole 128-byte lines (half lines cost the L2 path twice the requests), and the barrier sits
     //    where every wavefront holds all fragments of the tile in registers, so both units of tile kt are free
     //    from that barrier on.
-    // Ring of five 32 KiB units as in the ping-pong loop: A(0) W(0) A(1) W(1) A(2) ...; k tile = two k32 steps.
+    // The whole LDS is a ring of five 32 KiB operand units, A(0) W(0) A(1) W(1) A(2) ...: unit u sits in slot u % 5;
+    // a k tile is two k32 steps.
     static_assert(BM == BN, "ring units are one operand's rows of a k tile");
     constexpr int kUnit = BM * kRowBytes;
     static_assert(5 * kUnit <= kLdsAlloc, "ring exceeds the LDS");
@@ -514,10 +515,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
       }
     };
-    // fragment of 16 rows x 32 k: lane l supplies row (l & 15), chunk 4 ks + (l >> 4)
+    // fragment of 16 rows x 32 k: lane l supplies row (l & 15) and the 8 k of lane group l >> 4.  Which chunk of the
+    // step a lane group holds is free as long as both operands agree: groups 0..3 take chunks 0, 2, 1, 3, so that
+    // lanes l and l + 32, which the LDS serves together, read neighbouring chunks -- the pairing the swizzle keeps
+    // free of bank conflicts (chunks 0 and 2 of the same rows collide: measured, half of the LDS cycles)
     unsigned rd16[2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) rd16[ks] = lds_chunk_offset(l & 15u, 4u * ks + (l >> 4));
+    for (int ks = 0; ks < 2; ++ks) rd16[ks] = lds_chunk_offset(l & 15u, 4u * ks + (((l >> 4) & 1u) << 1 | (l >> 5)));
     const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
     f16x8 ga[2][MT16], gb[2][NT16];
     if (hi) {
@@ -577,99 +581,6 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));  // (loads past the last tile are out of range: zeros, but they do write the LDS)
     __builtin_amdgcn_s_setprio(0);
-  } else if constexpr (NW == 8) {
-    // ---- ping-pong: group = wv >> 2 (wavefronts w and w + 4 sit on the same SIMD).
-    // The LDS is a ring of five 32 KiB units, filled in the order A(0) W(0) A(1) W(1) ...: unit u
-    // sits in slot u % 5.  While tile kt (two units) is multiplied, up to three more units are in
-    // flight or landed -- W(kt+1) and A(kt+2) are requested during tile kt, A(kt+1) was during tile
-    // kt-1 -- against one tile (two units) with two whole-tile stages: the global->LDS stream is
-    // what bounds this kernel, and it needs ~96 KiB per CU in flight to run at the L2's rate.
-    static_assert(BM == BN, "ring units are one operand's rows of a k tile");
-    constexpr int kUnit = BM * kRowBytes;
-    static_assert(5 * kUnit <= kLdsAlloc, "ring exceeds the LDS");
-    auto wrap5 = [](int v) { return v >= 5 ? v - 5 : v; };
-    // per-lane byte offset of this lane's chunk in k tile kt of either operand (out of range past K)
-    auto lane_off = [&](int kt) -> unsigned {
-      return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
-    };
-    // this wavefront's LA block loads of one unit; the block's row offset rides in the scalar offset
-    auto fetch_unit = [&](bool is_w, unsigned voff, int slot) {
-      char* base = lds + slot * kUnit + wv * 1024;
-#pragma unroll
-      for (int i = 0; i < LA; ++i) {
-        if (is_w) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + i * NW * 1024), 16, voff, i * g_step, 0, 0);
-        else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, voff, i * g_step, 0, 0);
-      }
-    };
-    const unsigned group = wv >> 2;
-    const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
-    if (ktiles > 0) {
-      const unsigned v0 = lane_off(0);
-      fetch_unit(false, v0, 0);
-      fetch_unit(true, v0, 1);
-    }
-    if (ktiles > 1) {
-      fetch_unit(false, lane_off(1), 2);
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA));  // tile 0 has landed, A(1) may be in flight
-    } else {
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
-    }
-    __builtin_amdgcn_s_barrier();
-    DTAS_SCHED_FENCE();
-    if (group == 1) {  // one phase behind group 0; group 0 makes up the barrier after the loop
-      __builtin_amdgcn_s_barrier();
-      DTAS_SCHED_FENCE();
-    }
-    int slot_a = 0, slot_w = 1;  // slots of A(kt) and W(kt)
-    // one k tile; `steady`: tiles kt+1 and kt+2 exist (no conditions in the instruction stream)
-    auto pp_tile = [&](int kt, bool steady) {
-      const char* cur_a = lds + slot_a * kUnit + a_frag;
-      const char* cur_w = lds + slot_w * kUnit + b_frag;
-      const bool w1 = steady || kt + 1 < ktiles, a2 = steady || kt + 2 < ktiles;
-      const unsigned vw = lane_off(kt + 1), va = lane_off(kt + 2);
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int set = ks & 1;
-        // memory phase: this step's fragments; in step 0 the requests for W(kt+1), in step 1 those
-        // for A(kt+2), into the slots of A(kt-1) and W(kt-1), which every wavefront finished reading
-        // two phases ago at the latest
-#pragma unroll
-        for (int i = 0; i < MT; ++i) fa[set][i] = *reinterpret_cast<const f16x8*>(cur_a + i * 4096 + lds_rd[ks]);
-#pragma unroll
-        for (int j = 0; j < NT; ++j) fb[set][j] = *reinterpret_cast<const f16x8*>(cur_w + j * 4096 + lds_rd[ks]);
-        if (ks == 0 && w1) fetch_unit(true, vw, wrap5(slot_w + 2));
-        if (ks == 1 && a2) fetch_unit(false, va, wrap5(slot_a + 4));
-        // fragments in registers before the barrier (after a tile's last step the other group may
-        // overwrite the slots); at the last step also this wavefront's loads of tile kt+1: all
-        // but the newest unit's, A(kt+2), if that was requested
-        if (ks == 3) {
-          if (a2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LA)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
-        } else {
-          __builtin_amdgcn_s_waitcnt(0xC07F);
-        }
-        DTAS_SCHED_FENCE();
-        __builtin_amdgcn_s_barrier();
-        DTAS_SCHED_FENCE();
-        // MFMA phase
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);
-        DTAS_SCHED_FENCE();
-        __builtin_amdgcn_s_barrier();
-        DTAS_SCHED_FENCE();
-      }
-      slot_a = wrap5(slot_a + 2);
-      slot_w = wrap5(slot_w + 2);
-    };
-    int kt = 0;
-    for (; kt + 2 < ktiles; ++kt) pp_tile(kt, true);
-    for (; kt < ktiles; ++kt) pp_tile(kt, false);
-    if (group == 0) {
-      __builtin_amdgcn_s_barrier();
-      DTAS_SCHED_FENCE();
-    }
   } else if constexpr (MT * NT == 16) {
     // ---- four wavefronts with 128x128 tiles each (256 accumulator registers): every k step reads
     // 8 KiB of fragments per wavefront for 16 MFMAs, two thirds of the LDS traffic per flop of the
@@ -1750,7 +1661,7 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
                        (bm == 128 && bn == 128) || (bm == 64 && bn == 128) || (bm == 128 && bn == 64) ||
                        (bm == 64 && bn == 64);
     if (!known || cfg.tile[2] != kBK) return fail("gemm: no MFMA kernel for tile %dx%dx%d", bm, bn, cfg.tile[2]);
-    // 256x256 comes as 8 wavefronts (two per SIMD, alternating phases) or 4 (one per SIMD, 128x128 each)
+    // 256x256 comes as 8 wavefronts (two per SIMD, 128x64 each) or 4 (one per SIMD, 128x128 each)
     const bool four_waves = bm == 256 && bn == 256 && cfg.block == 256;
     if (cfg.block != mfma_threads(bm, bn) && !four_waves)
       return fail("gemm: the %dx%d MFMA kernel uses %d threads, got %d", bm, bn, mfma_threads(bm, bn), cfg.block);
