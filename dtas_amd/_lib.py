@@ -93,6 +93,7 @@ SIGNATURES = {
     "dtas_gemv_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _cfg, _vp],
     "dtas_gemv_f16_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _cfg, _vp],
     "dtas_gemm_f16": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],
+    "dtas_gemm_f16_static": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _cfg, _vp],
     "dtas_gemm_f16_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, ctypes.c_int32, _cfg, _vp],
     "dtas_attn_scores_f16_f32": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, ctypes.c_float, _cfg, _vp],
     "dtas_attn_pv_f16": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _cfg, _vp],

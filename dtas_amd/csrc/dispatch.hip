@@ -293,7 +293,8 @@ int dtas_init(void) {
   if (e != hipSuccess) return fail("dtas_init: hipGetDeviceProperties: %s", hipGetErrorString(e));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail("dtas_init: device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
-  return 0;
+  // loads the code object on this device and looks up the static scratch array of dtas_gemm_f16_static
+  return resolve_static_scratch(nullptr);
 }
 
 int dtas_select_bucket(int op, int64_t n, int64_t d0, int64_t d1, dtas_launch_info* out) {

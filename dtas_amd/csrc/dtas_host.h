@@ -54,6 +54,9 @@ int describe_reduction(int op, int64_t rows, int64_t cols, const dtas_config& cf
 int describe_gemv(int64_t N, int64_t K, const dtas_config& cfg, int64_t launch_args[7]);
 int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64_t launch_args[7]);
 
+// Resolves (once per device) the device address of the scratch array behind dtas_gemm_f16_static; *out may be NULL.
+int resolve_static_scratch(void** out);
+
 // split_k = 0 on the 8-wavefront 256x256 GEMM tile: how the tiles of a last, partly filled round are shared.
 // *unsplit tiles (whole rounds of the chip) get one workgroup each, the rest *nsplit workgroups each (1 = none).
 void tail_split_256(int64_t M, int64_t N, int64_t K, int* nsplit, unsigned* unsplit);

@@ -52,6 +52,12 @@
 #include <mutex>
 #include <type_traits>
 
+// Scratch memory of dtas_gemm_f16_static, the entry point that allocates nothing: arrival counters first, fp32
+// partial tiles behind them.  Every device the library runs on holds its own copy of this array from the moment
+// the code object is loaded until the process ends.  In host code the array's name is not a device address:
+// resolve_static_scratch() asks the runtime for the address, once per device, and everything below uses that pointer.
+static __device__ __align__(256) unsigned char scratch[DTAS_STATIC_SCRATCH_COUNTERS * 4 + DTAS_STATIC_SCRATCH_PARTIAL_BYTES];
+
 namespace dtas {
 namespace {
 
@@ -1589,6 +1595,24 @@ int operand_workspace(hipStream_t stream, size_t bytes, void** out) {
   return 0;
 }
 
+// Where a launch that splits K keeps its partial tiles when the caller must not allocate: set (per host thread) by
+// dtas_gemm_f16_static around its call into the common code, read by launch_mfma.
+struct FixedScratch {
+  float* partials;
+  size_t partial_bytes;
+  unsigned* arrivals;
+  size_t tiles;
+};
+thread_local const FixedScratch* t_fixed_scratch = nullptr;
+
+void* g_static_scratch[kMaxDevices];  // device address of `scratch` on each device, once resolved
+std::mutex g_static_scratch_mutex;
+
+__global__ void zero_u32_kernel(unsigned* p, size_t count) {
+  const size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+  if (i < count) p[i] = 0u;
+}
+
 template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
                 int64_t K, int nsplit, int batch = 1, unsigned unsplit = 0) {
@@ -1602,9 +1626,23 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   std::unique_lock<std::recursive_mutex> ws_lock;  // held until the launch is enqueued
   if (nsplit > 1) {
     const size_t bytes = split_tiles * nsplit * BM * BN * sizeof(float);
-    if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
-    ws_lock = std::unique_lock<std::recursive_mutex>(g_ws_mutex);
-    if (split_workspace(s, bytes, split_tiles, &partials, &arrivals) != 0) return -1;
+    if (t_fixed_scratch) {
+      const FixedScratch& f = *t_fixed_scratch;
+      if (bytes > f.partial_bytes || split_tiles > f.tiles)
+        return fail("gemm: K split over %d workgroups needs %zu bytes of partial tiles and %zu counters; the static scratch "
+                    "holds %zu bytes and %zu counters (a cfg with split_k = 1 needs none)", nsplit, bytes, split_tiles, f.partial_bytes, f.tiles);
+      partials = f.partials;
+      arrivals = f.arrivals;
+      // every call on this device shares the array and finds what the last one left: the counters of this launch are
+      // cleared first (by a kernel, not a memset node: the caller may be capturing a graph)
+      hipLaunchKernelGGL(zero_u32_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(split_tiles), 256))), dim3(256), 0, s, arrivals,
+                         split_tiles);
+      if (check_launch("gemm") != 0) return -1;
+    } else {
+      if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
+      ws_lock = std::unique_lock<std::recursive_mutex>(g_ws_mutex);
+      if (split_workspace(s, bytes, split_tiles, &partials, &arrivals) != 0) return -1;
+    }
   }
   const size_t wgs = unsplit + split_tiles * nsplit;
   if (wgs > 0x7fffffffu) return fail("gemm: too many workgroups");
@@ -1622,6 +1660,25 @@ inline int mfma_threads(int bm, int bn) { return bm == 256 && bn == 256 ? 512 : 
 inline int mfma_max_stages(int bm, int bn) { return bm + bn >= 512 ? 2 : bm + bn >= 384 ? 3 : 4; }
 
 }  // namespace
+
+// The device address of the static scratch array on the current device.  hipGetSymbolAddress is asked once per
+// device, with that device current (each GPU holds its own copy of the array at its own address).
+int resolve_static_scratch(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail("static scratch: cannot identify the current device");
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+  if (!g_static_scratch[dev]) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return fail("static scratch: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    }
+    g_static_scratch[dev] = ptr;
+  }
+  if (out) *out = g_static_scratch[dev];
+  return 0;
+}
 
 // The 8-wavefront 256x256 tile when the library chooses: whole rounds of the chip run one workgroup per tile; the
 // tiles of a last, partly filled round are shared by 2..4 workgroups each (as many as still fit the chip at once),
@@ -1720,6 +1777,21 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
 
 extern "C" int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
                              const dtas_config* user, void* stream) {
+  return dtas_gemm_f16_fused(A, W, bias, nullptr, nullptr, C, M, N, K, DTAS_EPI_BIAS, user, stream);
+}
+
+extern "C" int dtas_gemm_f16_static(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N, int64_t K,
+                                    const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  void* base = nullptr;
+  if (resolve_static_scratch(&base) != 0) return -1;  // (a table lookup after the first call on a device, or after dtas_init)
+  const FixedScratch fixed = {reinterpret_cast<float*>(static_cast<unsigned char*>(base) + DTAS_STATIC_SCRATCH_COUNTERS * 4),
+                              DTAS_STATIC_SCRATCH_PARTIAL_BYTES, static_cast<unsigned*>(base), DTAS_STATIC_SCRATCH_COUNTERS};
+  struct Scope {
+    explicit Scope(const FixedScratch* f) { t_fixed_scratch = f; }
+    ~Scope() { t_fixed_scratch = nullptr; }
+  } scope(&fixed);
   return dtas_gemm_f16_fused(A, W, bias, nullptr, nullptr, C, M, N, K, DTAS_EPI_BIAS, user, stream);
 }
 

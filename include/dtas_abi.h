@@ -20,11 +20,15 @@
  *    host.cc:64-69); the leading batch-1 dim of (1, n, H) is not passed;
  *  - `stream` is a hipStream_t (NULL = the default stream); nothing synchronises, the kernel is
  *    enqueued on `stream` on the current device.  Nothing is allocated, with one exception:
- *    dtas_gemm_f16 with K split over workgroups (split_k > 1, which the built-in table chooses
- *    when M x N yields few tiles) keeps fp32 partial tiles in a per-device workspace that the
+ *    dtas_gemm_f16 with K split over workgroups (split_k > 1, or 0 on the 256x256 tile; the built-in
+ *    table chooses either when M x N leaves CUs idle) keeps fp32 partial tiles in a workspace that the
  *    library allocates on first use and grows on demand (32 MiB at first, at most 1 GiB; growing
- *    waits for the device).  Launches that use it share it: enqueue them on one stream, or pass
- *    a cfg with split_k = 1 on the others.  dtas_gemm_q8_f16_fused keeps a second buffer of that kind
+ *    waits for the device).  There is one workspace per (device, stream): launches on one stream are
+ *    ordered by it, launches on different streams use different workspaces and may overlap; the
+ *    library holds its lock from looking a workspace up to enqueueing the launch, so host threads may
+ *    share a stream.  At most 16 streams per device hold one (the one used longest ago is released
+ *    first, which waits for the device).  A cfg with split_k = 1 uses none; dtas_gemm_f16_static
+ *    never allocates.  dtas_gemm_q8_f16_fused keeps a second buffer of that kind
  *    (an fp16 copy of the weights it was given) under the same rules, and dtas_attn_pv_f16 uses that
  *    buffer for a padded copy of P when m is not a multiple of 8;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
@@ -231,6 +235,23 @@ int dtas_gemv_f16_fused(const void* x, const void* W, const void* bias, const vo
  * fp16 in/out, fp32 accumulate on MFMA. */
 int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N,
                   int64_t K, const dtas_config* cfg, void* stream);
+
+/* ---- GEMM that allocates nothing ------------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory where they call: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  dtas_gemm_f16 in every respect (same
+ * kernels, same results bit for bit), except that a launch which splits K keeps its fp32 partial tiles and arrival
+ * counters in a static device array of the library -- DTAS_STATIC_SCRATCH_PARTIAL_BYTES of partial tiles and
+ * DTAS_STATIC_SCRATCH_COUNTERS counters (tiles that are split), held by every GPU the library runs on from the
+ * first use of the library on it until the process ends -- instead of the workspace dtas_gemm_f16 allocates.  It
+ * calls no hipMalloc, no hipFree and no other allocating routine; a launch that needs more scratch than the array
+ * holds returns -1 and says how much (pass a cfg with split_k = 1, or a smaller split).  All calls on one GPU share
+ * the array, whatever their streams: calls that overlap in time on one GPU race -- order them (one stream, or
+ * events).  dtas_init() resolves the array's address on the current device; otherwise the first call on a
+ * device does. */
+#define DTAS_STATIC_SCRATCH_PARTIAL_BYTES (32u << 20)
+#define DTAS_STATIC_SCRATCH_COUNTERS 4096u
+int dtas_gemm_f16_static(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N,
+                         int64_t K, const dtas_config* cfg, void* stream);
 
 /* ---- GEMM with the model's fused epilogues ------------------------------------
  * The PrimFuncs keep every intermediate as an fp16 tensor, so each step rounds to fp16:
