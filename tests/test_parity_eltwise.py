@@ -10,6 +10,8 @@ from gpu_util import Guarded, assert_bits_equal, cfg, dev
 pytestmark = pytest.mark.gpu
 
 N_SWEEP = [1, 16, 128, 1024, 4096]
+# beyond the sweep: the buckets above 4096, the table's upper bound 8192 and the last bucket's own sizing past it
+N_BEYOND = [4097, 8192, 8193, 20000]
 ALL_F16 = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(np.float16)
 
 
@@ -96,8 +98,29 @@ def test_cast_f16_to_f32_all_patterns(oracle):
     assert np.array_equal(got[~np.isnan(got)], h.astype(np.float32)[~np.isnan(got)])
 
 
+@pytest.mark.parametrize("n", N_BEYOND)
+def test_add_cast_copy_beyond_the_sweep(oracle, n):
+    H = 4096 if n <= 8193 else 2560
+    rng = np.random.default_rng(n)
+    a, b = rng.uniform(-1, 1, (n, H)).astype(np.float16), rng.uniform(-1, 1, (n, H)).astype(np.float16)
+    out = Guarded(a.shape, torch.float16)
+    ops.add(dev(a), dev(b), out.t)
+    assert_bits_equal(out.check(), oracle.c.add(a, b, threads=8))
+    x = (rng.standard_normal((n, H)) * 100).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    ops.cast(dev(x), out.t)
+    assert_bits_equal(out.check(), oracle.c.cast(x, "float16", threads=8), nan_ok=True)
+    h = x.astype(np.float16)
+    out32 = Guarded(h.shape, torch.float32)
+    ops.cast(dev(h), out32.t)
+    assert_bits_equal(out32.check(), oracle.c.cast(h, "float32", threads=8), nan_ok=True)
+    outc = Guarded(h.shape, torch.float16)
+    ops.copy(dev(h), outc.t)
+    assert np.array_equal(outc.check().view(np.uint16), oracle.c.copy(h, threads=8).view(np.uint16))
+
+
 @pytest.mark.parametrize("dtype", [np.float16, np.float32, np.int8])
-@pytest.mark.parametrize("n", [1, 16, 1024])
+@pytest.mark.parametrize("n", [1, 16, 128, 1024, 4096])
 def test_copy_is_identity_on_bits(oracle, dtype, n):
     rng = np.random.default_rng(3)
     raw = rng.integers(0, 256, size=n * 4096 * np.dtype(dtype).itemsize, dtype=np.uint8)

@@ -22,7 +22,7 @@ def _check(got, oracle_out, f64):
     assert (np.abs(got - want) <= ATOL_ORACLE + RTOL_ORACLE * np.abs(want)).all()
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 7, 16, 128, 257, 513, 1024, 4096])
+@pytest.mark.parametrize("n", [1, 2, 3, 7, 16, 128, 257, 513, 1024, 4096, 4097, 8192, 8193, 20000])
 def test_rms_norm_benchmark_config(oracle, n):
     rng = np.random.default_rng(3)
     x = rng.standard_normal((n, 4096)).astype(np.float16)
@@ -70,7 +70,7 @@ def test_rms_norm_grid_cap_and_invariants(oracle):
         assert np.abs(np.sqrt((got.astype(np.float64) ** 2).mean(-1)) - 1).max() < 2e-3   # unit rms with w = 1
 
 
-@pytest.mark.parametrize("n", [1, 3, 100, 257, 1024, 4096])
+@pytest.mark.parametrize("n", [1, 3, 100, 257, 1024, 4096, 4097, 8192, 8193, 20000])
 def test_layer_norm_reference_signature(oracle, n):
     rng = np.random.default_rng(13)
     x = (rng.standard_normal((1, n, 2560)) * 2 + 0.5).astype(np.float32)
