@@ -260,7 +260,14 @@ class FunctionTable:
         return f"  int64_t index = {expr} > {last} ? {last} : {expr};\n"
 
     def select(self, values: Dict[str, int]) -> Optional[KernelEntryInfo]:
+        """The row for these extents, or None where the library sizes the launch itself: a
+        function without tuned rows, and any extent above its upper bound.  The reference runs the
+        last bucket's predicated kernel there (python/dtas/engine/tuner.py:166-208 clamps the
+        index); a row here was validated only up to its bucket's end and may not fit a larger
+        extent (rows per wavefront, a skinny tile), while the library's own choice fits any."""
         if not self.call_table:      # a function whose launch shape the library chooses itself
+            return None
+        if any(values[a] > self.upper_bound[a] for a in self.dynamic_args if a in self.upper_bound):
             return None
         if not self.index_table:
             return self.call_table[0]

@@ -104,7 +104,7 @@ enum dtas_variant {
  * WMMAConfig{i, j, micro_shape}). */
 typedef struct dtas_config {
   int32_t variant;  /* enum dtas_variant of the op's family */
-  int32_t block;    /* threads per workgroup = launch_args[1] */
+  int32_t block;    /* threads per workgroup = launch_args[3] */
   int32_t vec;      /* elements per vector access */
   int32_t unroll;   /* elementwise/GEMV: independent vector accesses in flight per thread; row
                        reductions: rows a lane group takes per trip (1, 2, 4); GEMM: LDS stages (0 = max) */
@@ -119,7 +119,10 @@ typedef struct dtas_config {
  * `kernel_entry_info info = call_table[index_table[index]]` (host.cc:105-125,
  * python/dtas/codegen/runtime_packer.py:32-40). */
 typedef struct dtas_launch_info {
-  int64_t launch_args[7]; /* grid.x, grid.y, grid.z, block.x, dynamic LDS bytes, 0, 0 */
+  int64_t launch_args[7]; /* grid.x, grid.y, grid.z, block.x, dynamic LDS bytes, then two figures of the family:
+                           * row reductions: register iterations per row, rows per workgroup trip; GEMV: rows per
+                           * workgroup, 0; GEMM (MFMA): tiles along M, tiles along N; other GEMM kernels: 1, grid.x;
+                           * elementwise: 0, 0 */
   int64_t bucket_lo;      /* the merged bucket [lo, hi] of the dynamic extent that n fell in */
   int64_t bucket_hi;
   int32_t index;          /* min((n - 1) / range_div, last): position in the index table */
@@ -132,7 +135,8 @@ typedef struct dtas_launch_info {
 int dtas_abi_version(void);
 /* Thread-local text of the last error on this thread ("" if none). */
 const char* dtas_last_error(void);
-/* Checks that the current device is a gfx950 part and warms the kernel images. */
+/* Checks that the current device is a gfx950 part, loads the library's code object on it and looks up the
+ * static scratch array of dtas_gemm_f16_static there.  Optional: every entry point works without it. */
 int dtas_init(void);
 
 /* The built-in bucket table: which config a call with these extents uses.

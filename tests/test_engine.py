@@ -81,6 +81,26 @@ def test_index_statement_semantics(tmp_path):
             assert rn.start <= a * 256 + 1 <= rn.end and rm.start <= b * 256 + 1 <= rm.end
 
 
+def test_past_the_upper_bound_the_library_sizes_the_launch(tmp_path):
+    """A row is validated up to its bucket's end only: above the table's bound select() hands the
+    choice to the library, whose own config is launchable for any extent."""
+    rt = Engine(3, work_dir=str(tmp_path)).tune_module(_module(), MI355X(), 256)
+    for name, table in rt.tables.items():
+        if not table.dynamic_args:
+            continue
+        ub = table.upper_bound
+        inside = {a: ub[a] for a in table.dynamic_args}
+        assert table.select(inside) is not None
+        for factor_plus in ((1, 1), (8, 0)):
+            for a in table.dynamic_args:
+                beyond = dict(inside)
+                beyond[a] = ub[a] * factor_plus[0] + factor_plus[1]
+                assert table.select(beyond) is None, (name, beyond)
+                ext = extents_of(table.func, beyond)
+                info = _lib.select_bucket(op_id_of(table.func), *ext)   # the library's own config fits
+                assert info.launch_args[0] >= 1 and info.launch_args[3] >= 64
+
+
 def test_merge_two_dynamic_extents(tmp_path):
     from dtas_amd.codegen.compile_result import CompileResult
     from dtas_amd.common.config import ReductionConfig
