@@ -232,6 +232,7 @@ class MFMAConfig(Config):
         self.micro_shape_k = 4
         self.mfma_m, self.mfma_n, self.mfma_k = 32, 32, 16
         self.skinny = False      # small M: weight-streaming 16x16x32 kernel, K split over wavefronts
+        self.stream = False      # M <= 64: W streamed through the LDS in 1 KiB row pieces, K sliced over workgroups
         self.block_threads = 256
         self.stages = 0          # LDS stages of the load pipeline (0 = as many as the tile allows)
         self.split_k = 1         # workgroups that share a tile and split its K extent
@@ -257,7 +258,7 @@ class MFMAConfig(Config):
         return {"tile_shape": (self.tile_size_m, self.tile_size_n, self.tile_size_k),
                 "mfma_shape": (self.mfma_m, self.mfma_n, self.mfma_k), "i": self.i, "j": self.j,
                 "micro_shape": (self.micro_shape_x, self.micro_shape_y, self.micro_shape_k),
-                "skinny": self.skinny, "block_threads": self.block_threads, "stages": self.stages,
+                "skinny": self.skinny, "stream": self.stream, "block_threads": self.block_threads, "stages": self.stages,
                 "split_k": self.split_k, "in_vec_len_a": self.in_vec_len_a, "in_vec_len_b": self.in_vec_len_b}
 
     def from_dict(self, dic: Dict) -> "MFMAConfig":
@@ -266,6 +267,7 @@ class MFMAConfig(Config):
         self.i, self.j = dic["i"], dic["j"]
         self.micro_shape_x, self.micro_shape_y, self.micro_shape_k = dic["micro_shape"]
         self.skinny = dic.get("skinny", False)
+        self.stream = dic.get("stream", False)
         self.block_threads = dic.get("block_threads", 256)
         self.stages = dic.get("stages", 0)
         self.split_k = dic.get("split_k", 1)
@@ -273,11 +275,11 @@ class MFMAConfig(Config):
 
     def to_abi(self):
         c = _lib.DtasConfig()
-        c.variant = _lib.GEMM_SKINNY if self.skinny else _lib.GEMM_MFMA
+        c.variant = _lib.GEMM_SKINNY if self.skinny else _lib.GEMM_STREAM if self.stream else _lib.GEMM_MFMA
         c.block, c.vec = self.block_threads, 8
-        c.unroll = 4 if self.skinny else self.stages
+        c.unroll = 4 if self.skinny else 1 if self.stream else self.stages
         c.tile[0], c.tile[1], c.tile[2] = self.tile_size_m, self.tile_size_n, self.tile_size_k
-        c.split_k = 1 if self.skinny else self.split_k
+        c.split_k = 1 if self.skinny or self.stream else self.split_k
         return c
 
 

@@ -121,7 +121,7 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
 
 // GEMM: a cost model fitted to sweeps of every tile x stage count x K split over M on an MI355X.
 // A candidate's time is (rounds of workgroups over the chip) x (time of one k tile) x (k tiles):
-//  * time of one k tile with every CU busy: 256x256 1.80 us, 256x128 (3 stages) 1.045 us, 128x128
+//  * time of one k tile with every CU busy: 256x256 1.50 us, 256x128 (8 wavefronts) 1.00 us, 128x128
 //    0.665 us with 4 stages (one workgroup per CU) or 1.14 us per round of two per CU with 2 stages;
 //  * a partly filled last round is faster than a full one: x (0.55 + 0.45 * fill); 128x128 with 4
 //    stages in a single round gains less: x (0.8 + 0.2 * fill);
@@ -176,7 +176,8 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     }
     consider(floored(us, 3.5), 256, 256, 512, 2, 0);
   }
-  consider(floored(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.045 * kt, 3.5), 256, 128, 256, 3, 1);
+  // 256x128 on 8 wavefronts (64x64 each, the 16x16x32 ring loop): 1.00 us per k tile against 1.045 us on 4 wavefronts
+  consider(floored(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.0 * kt, 3.5), 256, 128, 512, 2, 1);
   consider(floored(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 3.1), 128, 128, 256, 2, 1);
   for (int split = 1; split <= 4; ++split) {
     if (split > 1 && ktiles / split < 8) continue;
@@ -187,11 +188,15 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     consider(floored((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.5) * split : 0.0), 4.3), 64, 64, 256, 4, split);
     const double t256128 = tiles_of(256, 128) * split;
     if (split > 1 && steps >= 32 && t256128 <= kNumCU)
-      consider(floored(gemm_rounds(t256128, kNumCU) * 1.045 * steps + 5.0 * split, 3.5), 256, 128, 256, 3, split);
+      consider(floored(gemm_rounds(t256128, kNumCU) * 1.0 * steps + 5.0 * split, 3.5), 256, 128, 512, 2, split);
     const double t12864 = tiles_of(128, 64) * split;
     if (t12864 <= kNumCU)
       consider(floored(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 3.4), 128, 64, 256, 4, split);
   }
+  // M <= 16 and at most one workgroup per CU of the W-streaming kernel (64 columns x 1024 of K each): 10.9 against
+  // 12.8 us at 4096 x 4096, 7.2 against 10.2 at 2560 x 2560; with more workgroups than CUs a workgroup's loads,
+  // MFMAs and the hand-over of its partial sums are no longer hidden behind another's, and the tiles win again
+  if (M_hi <= 16 && ceil_div(n, 64) * ceil_div(k, 1024) <= kNumCU) return make(DTAS_GEMM_STREAM, 256, 8, 1, 16, 64, 1024);
   if (M_hi <= 32) {
     // (one workgroup per 16 rows of W: fewer than one per CU leave CUs idle)
     const double skinny_wgs = static_cast<double>(ceil_div(n, 16));

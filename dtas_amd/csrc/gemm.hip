@@ -168,6 +168,18 @@ constexpr int waitcnt_imm(int v) { return 0x0070 | (v & 15) | ((v >> 4) << 14); 
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// Waits until at most min(n, MAX) whole tiles' loads (KL per lane each) are outstanding (n <= 0: none).  The
+// wait count is an immediate, hence the chain of comparisons.
+template <int KL, int MAX>
+__device__ __forceinline__ void wait_whole_tiles(int n) {
+  if constexpr (MAX <= 0) {
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+  } else {
+    if (n >= MAX) __builtin_amdgcn_s_waitcnt(waitcnt_imm(MAX * KL));
+    else wait_whole_tiles<KL, MAX - 1>(n);
+  }
+}
+
 // WT: W is given k-major ([K][N], N contiguous -- the V operand of attention's P.V); its tiles are
 // then transposed on the way into the LDS (two stages, 4 wavefronts only).
 // WQ: W is 8-bit with an fp16 scale per 32 elements of a row (Wq bytes [N][K], ep.wscale [N][K/32]); its
@@ -188,14 +200,17 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   constexpr int kABytes = BM * kRowBytes, kStage = (BM + BN) * kRowBytes;
   static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
-  static_assert((NS - 2) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
+  static_assert((NS - 1) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
   constexpr bool WREG = WT || WQ;  // W tiles pass through registers (transposed or dequantised), not the direct-to-LDS path
   static_assert(!WREG || (NS <= 3 && NW == 4), "the register W path is written for two or three stages and 4 wavefronts");
   static_assert(!(WT && WQ), "k-major 8-bit weights are not served");
-  static_assert(M16 == (NW == 8) && (!M16 || (BM == 256 && BN == 256 && !WREG)), "8 wavefronts: the 256x256 tile on the 16x16x32 loop, and only it");
-  static_assert(BM * BN * 2 <= NS * kStage, "epilogue staging must fit the operand stages");
-  static_assert(NS * kStage <= kLdsBytes && (BM + BN != 512 || 5 * BM * kRowBytes <= kLdsBytes), "stages exceed the LDS");
-  constexpr int kLdsAlloc = BM + BN == 512 ? 5 * BM * kRowBytes : NS * kStage;  // 256x256: a ring of 5 operand units
+  static_assert(M16 == (NW == 8) && (!M16 || !WREG), "8 wavefronts run the 16x16x32 loop, and only they");
+  // 256x256 and every 8-wavefront tile: a ring of 5 operand units, each the larger operand's rows of a k tile
+  constexpr bool kRing = BM + BN == 512 || M16;
+  constexpr int kRingUnit = (BM > BN ? BM : BN) * kRowBytes;
+  constexpr int kLdsAlloc = kRing ? 5 * kRingUnit : NS * kStage;
+  static_assert(BM * BN * 2 <= kLdsAlloc, "epilogue staging must fit the operand stages");
+  static_assert(kLdsAlloc <= kLdsBytes, "stages exceed the LDS");
   __shared__ __attribute__((aligned(1024))) char lds[kLdsAlloc];
 
   const unsigned t = threadIdx.x, l = t & 63u;
@@ -498,9 +513,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     //    from that barrier on.
     // The whole LDS is a ring of five 32 KiB operand units, A(0) W(0) A(1) W(1) A(2) ...: unit u sits in slot u % 5;
     // a k tile is two k32 steps.
-    static_assert(BM == BN, "ring units are one operand's rows of a k tile");
-    constexpr int kUnit = BM * kRowBytes;
-    static_assert(5 * kUnit <= kLdsAlloc, "ring exceeds the LDS");
+    // (a 256x128 or 128x256 tile leaves half of every other slot unused)
+    constexpr int kUnit = kRingUnit;
+    constexpr int kLoadsA = BM / 32, kLoadsW = BN / 32;  // 1 KiB block loads per wavefront and unit
+    static_assert(5 * kUnit <= kLdsAlloc && BM % 32 == 0 && BN % 32 == 0, "ring exceeds the LDS");
     auto wrap5 = [](int v) { return v >= 5 ? v - 5 : v; };
     const bool hi = wv >= 4;
     if (hi) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(2);
@@ -515,10 +531,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     };
     auto fetch16 = [&](int slot, unsigned voff) {
       char* base = lds + slot * kUnit + (wv & 3u) * 1024;
+      if (hi) {
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        if (hi) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
-        else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
+        for (int q = 0; q < kLoadsW; ++q) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
+      } else {
+#pragma unroll
+        for (int q = 0; q < kLoadsA; ++q) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
       }
     };
     // fragment of 16 rows x 32 k: lane l supplies row (l & 15) and the 8 k of lane group l >> 4.  Which chunk of the
@@ -533,12 +551,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     if (hi) {
       fetch16(1, lane_off16(0));
       fetch16(3, lane_off16(1));
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(8));
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoadsW));
     } else {
       fetch16(0, lane_off16(0));
       fetch16(2, lane_off16(1));
       fetch16(4, lane_off16(2));
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(16));
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * kLoadsA));
     }
     __builtin_amdgcn_s_barrier();
     DTAS_SCHED_FENCE();
@@ -549,6 +567,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     DTAS_SCHED_FENCE();
     // the MFMAs of fragment set `set`; the fragment reads of (pa, pw, ks) into the other set, one before every
     // other MFMA (a burst of reads backs up the LDS queue, and the wavefront's MFMAs wait behind it)
+    // (a 64x32 wavefront tile has 8 MFMAs for 6 reads: then one before every MFMA)
+    constexpr int kReadEvery = 2 * (MT16 + NT16) <= MT16 * NT16 ? 2 : 1;
     auto step16 = [&](int set, const char* pa, const char* pw, int ks) {
       constexpr int kReads = MT16 + NT16;
 #pragma unroll
@@ -556,8 +576,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
         for (int j = 0; j < NT16; ++j) {
           const int q = i * NT16 + j;
-          if (q % 2 == 0 && q / 2 < kReads) {
-            const int r = q / 2;
+          if (q % kReadEvery == 0 && q / kReadEvery < kReads) {
+            const int r = q / kReadEvery;
             if (r < NT16) gb[set ^ 1][r] = *reinterpret_cast<const f16x8*>(pw + b_frag + r * 2048 + rd16[ks]);
             else ga[set ^ 1][r - NT16] = *reinterpret_cast<const f16x8*>(pa + a_frag + (r - NT16) * 2048 + rd16[ks]);
           }
@@ -565,7 +585,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           DTAS_SCHED_FENCE();
         }
     };
-    static_assert(2 * (MT16 + NT16) <= MT16 * NT16, "fragment reads must fit between the MFMAs of a step");
+    static_assert(kReadEvery * (MT16 + NT16) <= MT16 * NT16, "fragment reads must fit between the MFMAs of a step");
     int slot_a = 0, slot_w = 1;  // slots of A(kt), W(kt)
     for (int kt = 0; kt < ktiles; ++kt) {
       const char* pa = lds + slot_a * kUnit;
@@ -575,7 +595,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       // wavefronts 0-3: A(kt+2) into the slot W(kt-1) left at the previous barrier
       if (!hi && kt > 0) fetch16(wrap5(slot_w + 3), lane_off16(kt + 2));
       // every fragment of tile kt is in registers and tile kt+1 has landed (0-3: all but the unit just requested)
-      if (hi) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(8));
+      if (hi) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0)); else __builtin_amdgcn_s_waitcnt(waitcnt_imm(kLoadsA));
       DTAS_SCHED_FENCE();
       __builtin_amdgcn_s_barrier();
       DTAS_SCHED_FENCE();
@@ -720,15 +740,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         DTAS_SCHED_FENCE();
       }
     };
+    // every stage is free: tile 0, tiles 1 .. NS-2 whole and part 0 of tile NS-1 are requested together, and only
+    // tile 0 is waited for (loads complete in order: whole tiles requested after it may stay outstanding)
     if (ktiles > 0) {
       const unsigned v0 = lane_off(0);
 #pragma unroll
       for (int l_ = 0; l_ < kL; ++l_) fetch_one(l_, v0, lds);
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
-    __builtin_amdgcn_s_barrier();
-    DTAS_SCHED_FENCE();
-    // tiles 1 .. NS-2 whole, part 0 of tile NS-1
 #pragma unroll
     for (int p = 1; p < NS; ++p) {
       if (p < ktiles) {
@@ -737,6 +755,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         for (int l_ = 0; l_ < (p < NS - 1 ? kL : kL / 4); ++l_) fetch_one(l_, vp, lds + p * kStage);
       }
     }
+    wait_whole_tiles<kL, NS - 2>(ktiles - 1);
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
     if (ktiles > 0) {
 #pragma unroll
       for (int i = 0; i < MT; ++i) read_a(0, i, lds, 0);
@@ -760,10 +781,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       if (steady) {
         __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * kL));
       } else {
-        const int ahead = ktiles - 2 - kt;  // tiles after kt+1 that have been requested
-        if (NS >= 4 && ahead >= 2) __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * kL));
-        else if (ahead >= 1) __builtin_amdgcn_s_waitcnt(waitcnt_imm(kL));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+        wait_whole_tiles<kL, NS - 2>(ktiles - 2 - kt);  // tiles after kt+1 that have been requested
       }
       __builtin_amdgcn_s_barrier();  // ... and every wavefront has finished reading tile kt
       DTAS_SCHED_FENCE();
@@ -818,9 +836,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // last adds the nsplit partials in split order, so the sum does not depend on who was last, and
   // goes on to the epilogue.  Nobody waits for anybody.
   // The XCDs' L2 caches are not coherent with each other.  Partials and the arrival counter are
-  // therefore moved with device-scope accesses (they pass the L2), ordered by the barriers' waits,
-  // rather than with device-scope fences, which write back and invalidate a whole L2 on every use
-  // (measured: that made a two-way split slower than no split).
+  // therefore moved with device-scope accesses (they pass the L2), ordered by explicit waits for the
+  // store count plus the barriers, rather than with device-scope fences, which write back and
+  // invalidate a whole L2 on every use (measured: that made a two-way split slower than no split).
   if (my_split > 1) {
     // (the flag lives in the operand stages, free by now: a second LDS object would make the
     // compiler order every fragment read behind the outstanding direct-to-LDS loads)
@@ -844,6 +862,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       const f32x2v pr = {pair_get(q, 0), pair_get(q, 1)};
       __hip_atomic_store(mine + q * 64 + l, __builtin_bit_cast(unsigned long long, pr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    // The partials are device-scope stores (write-through): once a wavefront's store count has drained they are
+    // visible to every XCD.  The barrier alone does not wait for that (a workgroup-scope barrier lets stores stay
+    // in flight), and the counter below must not be seen before the partials it announces.
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
     __syncthreads();  // every store of this workgroup has completed; nobody reads the stages any more
     if (t == 0) {
       const unsigned before = __hip_atomic_fetch_add(arrivals + tile_g, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1270,6 +1292,152 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
   }
 }
 
+// M <= 16 * MT against a W that is streamed once: with few rows of A the launch is a read of W from HBM, and what
+// the measurements on MI355X say about that read decides the shape.  A wavefront access of 1 KiB of one row
+// sustains 7.0 TB/s over the chip; 4 rows x 256 bytes 6.0; 8 rows x 128 bytes -- the block loads of the MFMA
+// tiles -- 4.5; 16 rows x 64 bytes -- operands loaded in MFMA layout, as gemm_skinny_kernel does -- 5.0, and A
+// fetched per wavefront from the L2 in that layout costs a further quarter.  Deeper LDS pipelines of the tile
+// kernel (up to all of a workgroup's k tiles in flight) changed nothing: the access shape is the limit.
+// So here a workgroup of WAVES wavefronts owns 16 * WAVES columns of C and a K slice of SEG x 512 elements;
+// wavefront w brings in its own 16 rows of W, each row's slice as SEG direct-to-LDS loads of 1 KiB, and its share
+// of the slice's A rows (1 KiB accesses as well, from the L2), all requested before anything is waited for.  Only
+// the A rows are shared, so one barrier, after they have landed; W is waited for per 512-element segment.
+// In the LDS the 16-byte chunk c of row r sits in slot c ^ f(r), f(r) = 2 * (r & 7) + ((r >> 3) & 1), and lane
+// groups 0..3 of a fragment read take chunks 0, 2, 1, 3 of the k step: the 16 rows of a lane group land in 16
+// different 16-byte bank groups, and so do the 8 rows x 2 chunks of lanes l, l + 32, which the LDS serves together.
+// K slices meet in the workspace as in the tile kernel: partials in accumulator layout, added in slice order by
+// the workgroup that arrives last.  Result register v of lane l is row 4 * (l >> 4) + v, column l & 15 of a 16x16
+// block (A is the first MFMA operand).
+__device__ __forceinline__ unsigned stream_swizzle(unsigned r) { return ((r & 7u) << 1) | ((r >> 3) & 1u); }
+
+template <int MT, int SEG, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
+                                                                GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
+                                                                int64_t K, unsigned nsplit, float* __restrict__ ws,
+                                                                unsigned* __restrict__ arrivals) {
+  constexpr int kCols = 16 * WAVES, kRowsA = 16 * MT, kSegBytes = 1024, kRowLds = SEG * kSegBytes;
+  constexpr int kALoads = kRowsA / WAVES * SEG, kWLoads = 16 * SEG;
+  static_assert(kRowsA % WAVES == 0 && (kCols + kRowsA) * kRowLds <= kLdsBytes && kALoads + kWLoads <= 63, "slab / LDS / vmcnt");
+  __shared__ __attribute__((aligned(1024))) char lds[(kCols + kRowsA) * kRowLds];
+  const unsigned t = threadIdx.x, l = t & 63u;
+  const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6);
+  const unsigned tn = __builtin_amdgcn_readfirstlane(blockIdx.x / nsplit), z = __builtin_amdgcn_readfirstlane(blockIdx.x % nsplit);
+  const int64_t n0 = static_cast<int64_t>(tn) * kCols;
+  const int64_t rows_w = N - n0 < kCols ? N - n0 : kCols;
+  const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, static_cast<unsigned>(M) * row_bytes);
+  // lane l of the load of (row, segment s) fetches the chunk that belongs in slot l: chunk l ^ f(row); past K: out of range
+  auto voff = [&](unsigned row, int s) -> unsigned {
+    const unsigned c = l ^ stream_swizzle(row);
+    const int64_t k = (static_cast<int64_t>(z) * SEG + s) * 512 + c * 8;
+    return k < K ? row * row_bytes + static_cast<unsigned>(k) * 2u : kOob;
+  };
+  char* lds_a = lds + kCols * kRowLds;
+#pragma unroll
+  for (int i = 0; i < kRowsA / WAVES; ++i) {
+    const unsigned a = i * WAVES + wv;
+#pragma unroll
+    for (int s = 0; s < SEG; ++s) {
+      const unsigned at = voff(a, s);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds_a + a * kRowLds + s * kSegBytes), 16, at, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < SEG; ++s)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const unsigned row = wv * 16u + r, at = voff(row, s);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(lds + row * kRowLds + s * kSegBytes), 16, at, 0, 0, 0);
+    }
+  f32x4v acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(kWLoads));  // this wavefront's A rows have landed
+  __builtin_amdgcn_s_barrier();                       // ... and everybody's
+  DTAS_SCHED_FENCE();
+  // fragment reads: row l & 15 of a 16-row block, chunk 4 * ks + perm(l >> 4) -> slot (4 * ks) ^ x, x = perm ^ f(row)
+  const unsigned i16 = l & 15u, g = l >> 4;
+  const unsigned x16 = ((((g & 1u) << 1) | (g >> 1)) ^ stream_swizzle(i16)) * 16u;
+  const char* w_lane = lds + (wv * 16u + i16) * kRowLds;
+  const char* a_lane = lds_a + i16 * kRowLds;
+#pragma unroll
+  for (int s = 0; s < SEG; ++s) {
+    if (s == 0) __builtin_amdgcn_s_waitcnt(waitcnt_imm(16 * (SEG - 1)));
+    else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
+    DTAS_SCHED_FENCE();
+#pragma unroll
+    for (int ks = 0; ks < 16; ++ks) {
+      const unsigned at = s * kSegBytes + (x16 ^ (ks * 64u));
+      const f16x8 fw = *reinterpret_cast<const f16x8*>(w_lane + at);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const f16x8*>(a_lane + i * 16 * kRowLds + at), fw, acc[i], 0, 0, 0);
+    }
+    DTAS_SCHED_FENCE();
+  }
+  static_assert(SEG <= 2, "the waits above are written for one or two segments");
+
+  if (nsplit > 1) {
+    __syncthreads();  // nobody reads the slab any more: its first word becomes the flag
+    volatile unsigned* is_last = reinterpret_cast<volatile unsigned*>(lds);
+    constexpr int kPer = 2 * MT;                    // 8-byte units per lane
+    constexpr int kPartial = kPer * 64 * WAVES;     // ... per workgroup
+    unsigned long long* tile_ws = reinterpret_cast<unsigned long long*>(ws) + static_cast<size_t>(tn) * nsplit * kPartial;
+    unsigned long long* mine = tile_ws + static_cast<size_t>(z) * kPartial + wv * (kPer * 64);
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+      const f32x2v pr = {acc[q / 2][2 * (q % 2)], acc[q / 2][2 * (q % 2) + 1]};
+      __hip_atomic_store(mine + q * 64 + l, __builtin_bit_cast(unsigned long long, pr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));  // (device-scope stores: drained = visible to every XCD; the barrier does not wait for them)
+    __syncthreads();  // every store of this workgroup has completed
+    if (t == 0) {
+      const unsigned before = __hip_atomic_fetch_add(arrivals + tn, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *is_last = before == nsplit - 1 ? 1u : 0u;
+      if (before == nsplit - 1)  // re-armed for the next launch
+        __hip_atomic_store(arrivals + tn, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (*is_last == 0) return;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    // slices are added in slice order whoever arrived last, up to 8 of them requested per round trip
+    constexpr int kGroup = MT <= 2 ? 8 : 4;
+    for (unsigned k0 = 0; k0 < nsplit; k0 += kGroup) {
+      unsigned long long raw[kGroup][kPer];
+#pragma unroll
+      for (int gk = 0; gk < kGroup; ++gk) {
+        const unsigned k = k0 + gk < nsplit ? k0 + gk : nsplit - 1;  // (past the last slice: re-read it, not added)
+        const unsigned long long* part = tile_ws + static_cast<size_t>(k) * kPartial + wv * (kPer * 64);
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) raw[gk][q] = __hip_atomic_load(part + q * 64 + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+      for (int gk = 0; gk < kGroup; ++gk) {
+        if (k0 + gk < nsplit) {
+#pragma unroll
+          for (int q = 0; q < kPer; ++q) {
+            const f32x2v pr = __builtin_bit_cast(f32x2v, raw[gk][q]);
+            acc[q / 2][2 * (q % 2)] += pr[0];
+            acc[q / 2][2 * (q % 2) + 1] += pr[1];
+          }
+        }
+      }
+    }
+  }
+  const int64_t col = n0 + wv * 16u + i16;
+  if (col < N) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int64_t row = i * 16 + 4 * g + v;
+        if (row < M) finish(acc[i][v], ep, C, row, col, N);
+      }
+  }
+}
+
 // A few rows of A (M <= MV <= 4) against a W that is streamed once: R rows of W per wavefront, lane l
 // takes the 16-byte chunks l, l + 64, ... of each (a wavefront access is 1 KiB of one W row, non-temporal,
 // as in the GEMV kernel), multiplies each with the matching chunks of the MV rows of A (re-read per
@@ -1613,6 +1781,29 @@ __global__ void zero_u32_kernel(unsigned* p, size_t count) {
   if (i < count) p[i] = 0u;
 }
 
+// Partial tiles and arrival counters of a launch that splits K over `nsplit` workgroups per tile: the static scratch
+// if the calling thread is inside dtas_gemm_f16_static, else the stream's workspace, whose lock `lock` then holds
+// (the caller keeps it until its kernel is enqueued).
+int split_scratch(hipStream_t s, size_t bytes, size_t split_tiles, int nsplit, float** partials, unsigned** arrivals,
+                  std::unique_lock<std::recursive_mutex>* lock) {
+  if (t_fixed_scratch) {
+    const FixedScratch& f = *t_fixed_scratch;
+    if (bytes > f.partial_bytes || split_tiles > f.tiles)
+      return fail("gemm: K split over %d workgroups needs %zu bytes of partial tiles and %zu counters; the static scratch "
+                  "holds %zu bytes and %zu counters (a cfg with split_k = 1 needs none)", nsplit, bytes, split_tiles, f.partial_bytes, f.tiles);
+    *partials = f.partials;
+    *arrivals = f.arrivals;
+    // every call on this device shares the array and finds what the last one left: the counters of this launch are
+    // cleared first (by a kernel, not a memset node: the caller may be capturing a graph)
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(split_tiles), 256))), dim3(256), 0, s, *arrivals,
+                       split_tiles);
+    return check_launch("gemm");
+  }
+  if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
+  *lock = std::unique_lock<std::recursive_mutex>(g_ws_mutex);
+  return split_workspace(s, bytes, split_tiles, partials, arrivals);
+}
+
 template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N,
                 int64_t K, int nsplit, int batch = 1, unsigned unsplit = 0) {
@@ -1624,26 +1815,8 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   if (unsplit > 0 && (batch != 1 || unsplit >= tiles || nsplit < 2)) return fail("gemm: a partly split launch takes one problem and a split");
   const size_t split_tiles = (tiles - unsplit) * batch;  // tiles shared by nsplit workgroups
   std::unique_lock<std::recursive_mutex> ws_lock;  // held until the launch is enqueued
-  if (nsplit > 1) {
-    const size_t bytes = split_tiles * nsplit * BM * BN * sizeof(float);
-    if (t_fixed_scratch) {
-      const FixedScratch& f = *t_fixed_scratch;
-      if (bytes > f.partial_bytes || split_tiles > f.tiles)
-        return fail("gemm: K split over %d workgroups needs %zu bytes of partial tiles and %zu counters; the static scratch "
-                    "holds %zu bytes and %zu counters (a cfg with split_k = 1 needs none)", nsplit, bytes, split_tiles, f.partial_bytes, f.tiles);
-      partials = f.partials;
-      arrivals = f.arrivals;
-      // every call on this device shares the array and finds what the last one left: the counters of this launch are
-      // cleared first (by a kernel, not a memset node: the caller may be capturing a graph)
-      hipLaunchKernelGGL(zero_u32_kernel, dim3(static_cast<unsigned>(ceil_div(static_cast<int64_t>(split_tiles), 256))), dim3(256), 0, s, arrivals,
-                         split_tiles);
-      if (check_launch("gemm") != 0) return -1;
-    } else {
-      if (bytes > kMaxSplitWsBytes) return fail("gemm: split_k %d needs %zu bytes of workspace (limit %zu)", nsplit, bytes, kMaxSplitWsBytes);
-      ws_lock = std::unique_lock<std::recursive_mutex>(g_ws_mutex);
-      if (split_workspace(s, bytes, split_tiles, &partials, &arrivals) != 0) return -1;
-    }
-  }
+  if (nsplit > 1 && split_scratch(s, split_tiles * nsplit * BM * BN * sizeof(float), split_tiles, nsplit, &partials, &arrivals, &ws_lock) != 0)
+    return -1;
   const size_t wgs = unsplit + split_tiles * nsplit;
   if (wgs > 0x7fffffffu) return fail("gemm: too many workgroups");
   GemmEpilogue batched = ep;
@@ -1654,9 +1827,31 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
   return check_launch("gemm");
 }
 
+// The W-streaming kernel: 16 * WAVES columns and SEG * 512 elements of K per workgroup, K slices met in the workspace.
+template <int MT, int SEG, int WAVES>
+int launch_stream(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N, int64_t K) {
+  const size_t tiles = static_cast<size_t>(ceil_div(N, 16 * WAVES));
+  const int nsplit = static_cast<int>(ceil_div(K, SEG * 512));
+  float* partials = nullptr;
+  unsigned* arrivals = nullptr;
+  std::unique_lock<std::recursive_mutex> ws_lock;  // held until the launch is enqueued
+  if (nsplit > 1 && split_scratch(s, tiles * nsplit * (16 * MT) * (16 * WAVES) * sizeof(float), tiles, nsplit, &partials, &arrivals, &ws_lock) != 0)
+    return -1;
+  if (tiles * nsplit > 0x7fffffffu) return fail("gemm: too many workgroups");
+  hipLaunchKernelGGL((gemm_stream_kernel<MT, SEG, WAVES>), dim3(static_cast<unsigned>(tiles * nsplit)), dim3(64 * WAVES), 0, s, A, W, ep,
+                     C, M, N, K, static_cast<unsigned>(nsplit), partials, arrivals);
+  return check_launch("gemm");
+}
+
+// the instantiated W-streaming shapes: rows of A x columns x K slice
+inline bool stream_shape_ok(int bm, int bn, int bk) {
+  if ((bm != 16 && bm != 32 && bm != 64) || (bn != 64 && bn != 128) || (bk != 512 && bk != 1024)) return false;
+  return (bm + bn) * bk * 2 <= kLdsBytes;
+}
+
 // threads per workgroup of the MFMA kernel for a tile: 8 wavefronts for 256x256, else 4
 inline int mfma_threads(int bm, int bn) { return bm == 256 && bn == 256 ? 512 : 256; }
-// LDS stages a tile can hold (160 KiB): 2 for 256x256, 3 for 256x128, 4 below that
+// LDS stages a launch uses unless told otherwise: 2 for 256x256, 3 for 256x128, 4 below that
 inline int mfma_max_stages(int bm, int bn) { return bm + bn >= 512 ? 2 : bm + bn >= 384 ? 3 : 4; }
 
 }  // namespace
@@ -1718,9 +1913,12 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
                        (bm == 128 && bn == 128) || (bm == 64 && bn == 128) || (bm == 128 && bn == 64) ||
                        (bm == 64 && bn == 64);
     if (!known || cfg.tile[2] != kBK) return fail("gemm: no MFMA kernel for tile %dx%dx%d", bm, bn, cfg.tile[2]);
-    // 256x256 comes as 8 wavefronts (two per SIMD, 128x64 each) or 4 (one per SIMD, 128x128 each)
+    // 256x256 comes as 8 wavefronts (two per SIMD, 128x64 each) or 4 (one per SIMD, 128x128 each); 256x128 and
+    // 128x256 as 4 wavefronts on whole-tile stages or 8 (64x64 each) on the 16x16x32 ring loop (128x128 on that
+    // loop, 64x32 per wavefront, measured slower than on 4 wavefronts at every M: not instantiated)
     const bool four_waves = bm == 256 && bn == 256 && cfg.block == 256;
-    if (cfg.block != mfma_threads(bm, bn) && !four_waves)
+    const bool eight_waves = bm + bn == 384 && cfg.block == 512;
+    if (cfg.block != mfma_threads(bm, bn) && !four_waves && !eight_waves)
       return fail("gemm: the %dx%d MFMA kernel uses %d threads, got %d", bm, bn, mfma_threads(bm, bn), cfg.block);
     if (K * 2 * (bm > bn ? bm : bn) >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
     const int64_t tm = ceil_div(M, bm), tn = ceil_div(N, bn);
@@ -1735,10 +1933,10 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     if (cfg.split_k == 0 && bm == 256 && bn == 256 && !four_waves) tail_split_256(M, N, K, &nsplit, &unsplit);
     if (tm * tn * nsplit > 0x7fffffff) return fail("gemm: too many workgroups");
     la[0] = unsplit + (tm * tn - unsplit) * nsplit;
-    la[3] = four_waves ? 256 : mfma_threads(bm, bn);
-    // 256x256: a ring of five 32 KiB operand units; else whole-tile stages
-    la[4] = bm == 256 && bn == 256 ? 5 * 256 * kRowBytes
-                                   : (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
+    la[3] = four_waves ? 256 : eight_waves ? 512 : mfma_threads(bm, bn);
+    // 256x256 and the 8-wavefront tiles: a ring of five operand units; else whole-tile stages
+    la[4] = (bm == 256 && bn == 256) || eight_waves ? 5 * (bm > bn ? bm : bn) * kRowBytes
+                                                    : (cfg.unroll >= 2 ? cfg.unroll : mfma_max_stages(bm, bn)) * (bm + bn) * kRowBytes;
     la[5] = tm;
     la[6] = tn;
     return 0;
@@ -1768,6 +1966,23 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     la[4] = 16 * mt * 64 * 16;
     la[5] = 1;
     la[6] = la[0];
+    return 0;
+  }
+  if (cfg.variant == DTAS_GEMM_STREAM) {
+    const int mt = cfg.tile[0] / 16, waves = cfg.tile[1] / 16, seg = cfg.tile[2] / 512;
+    if (!stream_shape_ok(cfg.tile[0], cfg.tile[1], cfg.tile[2]))
+      return fail("gemm: the W-streaming kernel takes tiles {16,32,64}x{64,128}x{512,1024} that fit the LDS, got %dx%dx%d", cfg.tile[0],
+                  cfg.tile[1], cfg.tile[2]);
+    if (M > cfg.tile[0]) return fail("gemm: a streaming tile of %d rows cannot hold M=%lld", cfg.tile[0], (long long)M);
+    if (cfg.block != 64 * waves) return fail("gemm: the %d-column streaming tile uses %d threads, got %d", cfg.tile[1], 64 * waves, cfg.block);
+    if (K * 2 * cfg.tile[1] >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
+    const int64_t tn = ceil_div(N, cfg.tile[1]), slices = ceil_div(K, cfg.tile[2]);
+    if (slices < 1 || tn * slices > 0x7fffffff) return fail("gemm: too many workgroups");
+    la[0] = tn * slices;
+    la[3] = cfg.block;
+    la[4] = (16 * mt + 16 * waves) * seg * 1024;
+    la[5] = 1;
+    la[6] = tn;
     return 0;
   }
   return fail("gemm: unknown variant %d", cfg.variant);
@@ -1852,6 +2067,15 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
     }
     return check_launch("gemm");
   }
+  if (cfg.variant == DTAS_GEMM_STREAM) {
+#define DTAS_STREAM_CASE(BM_, BN_, BK_) \
+  if (cfg.tile[0] == BM_ && cfg.tile[1] == BN_ && cfg.tile[2] == BK_) return launch_stream<BM_ / 16, BK_ / 512, BN_ / 16>(s, a, w, b, c, M, N, K)
+    DTAS_STREAM_CASE(16, 64, 512); DTAS_STREAM_CASE(16, 64, 1024); DTAS_STREAM_CASE(16, 128, 512);
+    DTAS_STREAM_CASE(32, 64, 512); DTAS_STREAM_CASE(32, 128, 512);
+    DTAS_STREAM_CASE(64, 64, 512);
+#undef DTAS_STREAM_CASE
+    return fail("gemm: no W-streaming kernel for tile %dx%dx%d", cfg.tile[0], cfg.tile[1], cfg.tile[2]);
+  }
   const int bm = cfg.tile[0], bn = cfg.tile[1];
   const int ns = cfg.unroll >= 2 ? cfg.unroll : 0;
   const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
@@ -1862,6 +2086,10 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
     unsigned unsplit = 0;
     if (cfg.split_k == 0) tail_split_256(M, N, K, &split, &unsplit);  // (split_k >= 1: that split for every tile)
     return launch_mfma<256, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, split, 1, unsplit);
+  }
+  if (cfg.block == 512) {  // 8 wavefronts on the 16x16x32 ring loop
+    if (bm == 256 && bn == 128) return launch_mfma<256, 128, 4, 2, 2, false, false, true>(s, a, w, b, c, M, N, K, sk);
+    if (bm == 128 && bn == 256) return launch_mfma<128, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, sk);
   }
   if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
                                              : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk);
@@ -1876,9 +2104,9 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   if (bm == 128 && bn == 64) return ns == 2   ? launch_mfma<128, 64, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
                                     : ns == 3 ? launch_mfma<128, 64, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
                                               : launch_mfma<128, 64, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
-  if (bm == 64 && bn == 64) return ns == 2   ? launch_mfma<64, 64, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
-                                   : ns == 3 ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
-                                             : launch_mfma<64, 64, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
+  if (bm == 64 && bn == 64) return ns == 2    ? launch_mfma<64, 64, 2, 2, 2>(s, a, w, b, c, M, N, K, sk)
+                                   : ns == 3  ? launch_mfma<64, 64, 2, 2, 3>(s, a, w, b, c, M, N, K, sk)
+                                              : launch_mfma<64, 64, 2, 2, 4>(s, a, w, b, c, M, N, K, sk);
   return fail("gemm: no MFMA kernel for tile %dx%d", bm, bn);
 }
 

@@ -34,7 +34,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
     def preferred(self, m_hi: int, N: int, K: int = 4096):
         """(tile_m, tile_n, stages, split_k) under the cost model fitted to sweeps on an MI355X (the same
         one the library's built-in table uses): time = rounds of workgroups over the chip x time of one
-        k tile x k tiles.  One k tile with every CU busy: 256x256 see below, 256x128 (3 stages) 1.045 us,
+        k tile x k tiles.  One k tile with every CU busy: 256x256 see below, 256x128 (8 wavefronts of 64x64) 1.00 us,
         128x128 0.665 us (4 stages, one workgroup per CU) or 1.14 us per round of two per CU (2 stages);
         a partly filled last round costs 0.55 + 0.45 * fill of a full one (0.8 + 0.2 * fill for 128x128 with 4 stages
         in a single round); 64x64 0.33 us per k tile up to
@@ -69,7 +69,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             else:
                 us256 += 8.0 + 1.50 * ktiles * relief(rem / cus)
         cands = [(floored(us256, 3.5), (256, 256, 2, 0)),
-                 (floored(rounds(tiles(256, 128), cus) * 1.045 * ktiles, 3.5), (256, 128, 3, 1)),
+                 (floored(rounds(tiles(256, 128), cus) * 1.0 * ktiles, 3.5), (256, 128, 2, 1)),
                  (floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1))]
         for split in (1, 2, 3, 4):
             if split > 1 and ktiles // split < 8:
@@ -84,7 +84,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                           (64, 64, 4, split)))
             t256128 = tiles(256, 128) * split
             if split > 1 and steps >= 32 and t256128 <= cus:
-                cands.append((floored(rounds(t256128, cus) * 1.045 * steps + 5.0 * split, 3.5), (256, 128, 3, split)))
+                cands.append((floored(rounds(t256128, cus) * 1.0 * steps + 5.0 * split, 3.5), (256, 128, 2, split)))
             t12864 = tiles(128, 64) * split
             if t12864 <= cus:
                 cands.append((floored(0.47 * steps + (2.5 * split if split > 1 else 0.0), 3.4), (128, 64, 4, split)))
@@ -115,6 +115,12 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             return 1, 0
         return split, tiles - rem
 
+    def prefers_stream(self, m_hi: int, N: int, K: int) -> bool:
+        """M <= 16 and at most one workgroup per CU of the W-streaming kernel (64 columns x 1024 of K each):
+        measured 10.9 against 12.8 us at 4096 x 4096, 7.2 against 10.2 at 2560 x 2560; beyond one round of
+        workgroups the tiles win again (libdtas: gemm_policy)."""
+        return m_hi <= 16 and -(-N // 64) * -(-K // 1024) <= self.arch.num_sm
+
     def prefers_skinny(self, m_hi: int, N: int, K: int) -> bool:
         """M <= 32: the W-streaming kernel (about 3.5 TB/s of W, slower as M grows) against the model's
         best MFMA candidate; call after preferred()."""
@@ -136,6 +142,18 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             for e in params[0].shape[:-1]:
                 m_hi *= e
         out: List[MFMAConfig] = []
+        stream: List[MFMAConfig] = []
+        if m_hi <= 64:
+            # the W-streaming kernel: rows of A x columns x K slice, (rows + columns) * slice * 2 bytes of LDS
+            for cols, kslice in ((64, 1024), (64, 512), (128, 512)):
+                rows = 16 if m_hi <= 16 else 32 if m_hi <= 32 else 64
+                if (rows + cols) * kslice * 2 > _LDS or (rows == 64 and cols == 128):
+                    continue
+                c = MFMAConfig()
+                c.stream, c.block_threads = True, 4 * cols
+                c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.micro_shape_k = 1, cols // 16, rows // 16, 1, kslice // 32
+                c.mfma_m, c.mfma_n, c.mfma_k = 16, 16, 32
+                stream.append(c)
         if m_hi <= 64:
             for threads in (512, 256):
                 c = MFMAConfig()
@@ -155,12 +173,15 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 if (mx, my) == (4, 4):
                     # the 256x256 kernel runs 2x4 wavefronts of 128x64 (two per SIMD)
                     c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 2, 4, 4, 2, 512
+                if (mx, my) == (4, 2) and stages == 2:
+                    # 256x128 with two "stages": 4x2 wavefronts of 64x64 on the ring loop of the 256x256 kernel
+                    c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 4, 2, 2, 2, 512
                 if not self.check_valid(c):
                     continue
                 tiles = -(-m_hi // tm) * -(-N // tn)
                 c.num_wave = -(-tiles // self.arch.num_sm)
                 splits = [1] + [sk for sk in (2, 3, 4) if tiles * sk <= 4 * self.arch.num_sm and -(-K // 64) // sk >= 8]
-                if c.block_threads == 512:
+                if c.block_threads == 512 and (tm, tn) == (256, 256):
                     splits = [0] + splits   # 0: only the tiles of a partly filled last round are split
                 for sk in splits:
                     cs = MFMAConfig().from_dict(c.to_dict())
@@ -172,4 +193,5 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         mfma = [c for _, c in sorted(scored, key=lambda t: t[0])]
         # the W-streaming kernel leads only where it beats the best MFMA candidate under the model
         out = (out + mfma) if self.prefers_skinny(m_hi, N, K) else (mfma[:1] + out + mfma[1:])
+        out = (stream + out) if self.prefers_stream(m_hi, N, K) else (out[:1] + stream + out[1:])
         return out[:topk]

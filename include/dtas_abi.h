@@ -94,8 +94,12 @@ enum dtas_variant {
   /* GEMM (python/dtas/schedule/tir_wmma.py:20-222) */
   DTAS_GEMM_MFMA = 0,     /* LDS-tiled MFMA, tile = tile[0] x tile[1] x tile[2] */
   DTAS_GEMM_SKINNY = 1,   /* small M: weight-streaming MFMA 16x16x32, split over N and K */
-  DTAS_GEMM_ROWS = 2      /* M <= 4: W streamed once in whole rows (tile[1] per wavefront) against tile[0] >= M
+  DTAS_GEMM_ROWS = 2,     /* M <= 4: W streamed once in whole rows (tile[1] per wavefront) against tile[0] >= M
                              rows of A on the vector ALU; tile = {2|4, 1|2|4, 8}, block 64 / 128 / 256 */
+  DTAS_GEMM_STREAM = 3    /* M <= tile[0] in {16, 32, 64}: W streamed once, 1 KiB of a row per access, through the LDS to
+                             MFMA 16x16x32; a workgroup of tile[1] / 16 wavefronts owns tile[1] in {64, 128} columns and
+                             tile[2] in {512, 1024} elements of K, the K slices are added up in the workspace;
+                             (tile[0] + tile[1]) * tile[2] * 2 bytes of LDS, block = 4 * tile[1] */
 };
 
 /* One row of a call table: the launch-relevant part of the reference's *Config classes

@@ -39,7 +39,11 @@ def test_select_bucket_uses_labelled_ranges():
     b = _lib.select_bucket(_lib.OP_GEMM_F16, 17, 4096, 4096)
     assert (a.index, b.index) == (0, 1)
     assert a.name == b"fused_NT_matmul4_add1_n_1_to_16__kernel"
-    assert a.config.variant == _lib.GEMM_SKINNY and list(a.config.tile) == [16, 16, 32]
+    # 16 rows against 4096 x 4096: the W-streaming kernel, 64 columns x 1024 of K per workgroup, one workgroup per CU
+    assert a.config.variant == _lib.GEMM_STREAM and list(a.config.tile) == [16, 64, 1024]
+    assert list(a.launch_args)[:5] == [256, 1, 1, 256, (16 + 64) * 1024 * 2]
+    wide = _lib.select_bucket(_lib.OP_GEMM_F16, 16, 32000, 4096)   # more workgroups than CUs: the tiles
+    assert wide.config.variant == _lib.GEMM_MFMA
     big = _lib.select_bucket(_lib.OP_GEMM_F16, 4096, 4096, 4096)
     assert big.config.variant == _lib.GEMM_MFMA and list(big.config.tile) == [256, 256, 64]
     assert list(big.launch_args)[:4] == [256, 1, 1, 512] and big.launch_args[4] == 5 * 256 * 128  # a ring of five operand units

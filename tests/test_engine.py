@@ -183,6 +183,8 @@ def test_gemm_emitter_leads_with_the_librarys_builtin_choice(N, K):
         want = _lib.select_bucket(_lib.OP_GEMM_F16, m_hi, N, K).config.to_dict()
         got = _first_candidate(func, (Range("n", m_hi - 15, m_hi),))
         keys = ("variant", "tile", "split_k") if want["variant"] == _lib.GEMM_SKINNY else ("variant", "block", "tile", "unroll", "split_k")
+        if want["variant"] == _lib.GEMM_MFMA and want["block"] == 512:
+            keys = ("variant", "block", "tile", "split_k")   # the 8-wavefront ring loops have no stage count
         assert {k: got[k] for k in keys} == {k: want[k] for k in keys}, (m_hi, got, want)
 
 
@@ -212,6 +214,9 @@ def test_builtin_tables_name_a_launchable_kernel_for_every_bucket_and_shape():
                     # (split_k = 0, the 8-wavefront 256x256 tile only: the library splits just the tiles of a partly filled last round)
                     assert (c.split_k == 0 and tuple(c.tile[:2]) == (256, 256) and c.block == 512) or \
                         (1 <= c.split_k <= 4 and (c.split_k == 1 or -(-K // 64) // c.split_k >= 8)), (M, N, K, c.split_k)
+                elif c.variant == _lib.GEMM_STREAM:
+                    # at most one workgroup per CU, 64 columns x 1024 of K each
+                    assert M <= 16 and list(c.tile) == [16, 64, 1024] and c.block == 256 and info.launch_args[0] <= 256
                 else:
                     assert c.variant == _lib.GEMM_SKINNY and M <= 32 and c.tile[0] >= min(M, 32)
             info = _lib.select_bucket(_lib.OP_GEMV_F16, 1, N, K)

@@ -139,6 +139,64 @@ def test_gemm_every_skinny_tile(oracle, rows, block, N, K):
         _check(out.check(), oracle.c.gemm(a, w, threads=8), oracle.np64.gemm(a, w))
 
 
+STREAM_TILES = [(16, 64, 512), (16, 64, 1024), (16, 128, 512), (32, 64, 512), (32, 128, 512), (64, 64, 512)]
+
+
+@pytest.mark.parametrize("rows,cols,kslice", STREAM_TILES)
+@pytest.mark.parametrize("N,K", [(64, 64), (100, 520), (1000, 2560), (4096, 4096), (33, 40), (2560, 8 * 1000)])
+def test_gemm_every_streaming_tile(oracle, rows, cols, kslice, N, K):
+    # the W-streaming kernel: one K slice (K <= the slice) up to 16 of them, ragged N, K and M, with and without bias
+    for M in (rows, rows - 3, 1):
+        a, w = _inputs(M, N, K, M + N + K)
+        bias = np.random.default_rng(2).uniform(-1, 1, N).astype(np.float16) if M != 1 else None
+        out = Guarded((M, N), torch.float16)
+        c = cfg(variant=_lib.GEMM_STREAM, block=4 * cols, vec=8, unroll=1, tile=[rows, cols, kslice])
+        ops.gemm(dev(a), dev(w), None if bias is None else dev(bias), out.t, c)
+        _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+        info = _lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c)
+        assert list(info.launch_args)[:5] == [-(-N // cols) * -(-K // kslice), 1, 1, 4 * cols, (rows + cols) * kslice * 2]
+
+
+def test_gemm_streaming_tile_is_reproducible_exact_and_refuses_what_it_cannot_hold(oracle):
+    M, N, K = 16, 4096, 4096
+    a, w = _inputs(M, N, K, 5)
+    assert _lib.select_bucket(_lib.OP_GEMM_F16, M, N, K).config.variant == _lib.GEMM_STREAM   # what cfg = NULL runs here
+    runs = []
+    for _ in range(3):
+        out = Guarded((M, N), torch.float16)
+        ops.gemm(dev(a), dev(w), None, out.t)
+        runs.append(out.check())
+    assert all(np.array_equal(r.view(np.uint16), runs[0].view(np.uint16)) for r in runs)   # slices are added in slice order
+    _check(runs[0], oracle.c.gemm(a, w, threads=8), oracle.np64.gemm(a, w))
+    # small integers: every sum is exact in fp32 and fp16, whatever the order
+    rng = np.random.default_rng(6)
+    ai, wi = rng.integers(-2, 3, (13, 2048)).astype(np.float16), rng.integers(-2, 3, (200, 2048)).astype(np.float16)
+    out = Guarded((13, 200), torch.float16)
+    ops.gemm(dev(ai), dev(wi), None, out.t, cfg(variant=_lib.GEMM_STREAM, block=256, vec=8, unroll=1, tile=[16, 64, 512]))
+    assert np.array_equal(out.check().astype(np.float64), ai.astype(np.float64) @ wi.astype(np.float64).T)
+    big = dev(np.zeros((17, 64), np.float16))
+    with pytest.raises(_lib.DtasError, match="cannot hold M=17"):
+        ops.gemm(big, dev(np.zeros((8, 64), np.float16)), None, torch.empty(17, 8, dtype=torch.float16, device="cuda"),
+                 cfg(variant=_lib.GEMM_STREAM, block=256, vec=8, unroll=1, tile=[16, 64, 512]))
+    for tile, block in (([64, 128, 512], 512), ([16, 64, 2048], 256), ([48, 64, 512], 256), ([16, 64, 512], 512)):
+        with pytest.raises(_lib.DtasError, match="streaming"):
+            _lib.describe_launch(_lib.OP_GEMM_F16, 8, 64, 64, cfg(variant=_lib.GEMM_STREAM, block=block, vec=8, unroll=1, tile=tile))
+
+
+@pytest.mark.parametrize("bm,bn", [(256, 128), (128, 256)])
+@pytest.mark.parametrize("split", [1, 2, 3])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 8), (300, 260, 200), (257, 513, 1096), (512, 512, 64), (256, 256, 4096), (700, 300, 4104)])
+def test_gemm_rectangular_tiles_with_eight_wavefronts(oracle, bm, bn, split, M, N, K):
+    # block = 512 on 256x128 / 128x256: 64x64 per wavefront on the ring loop of the 256x256 kernel
+    a, w = _inputs(M, N, K, M + N + K)
+    bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
+    out = Guarded((M, N), torch.float16)
+    c = cfg(variant=_lib.GEMM_MFMA, block=512, vec=8, unroll=2, tile=[bm, bn, 64], split_k=split)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c)
+    _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+    assert list(_lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c).launch_args)[3:5] == [512, 5 * 256 * 128]
+
+
 @pytest.mark.parametrize("mv,r", [(2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4)])
 @pytest.mark.parametrize("block", [64, 128, 256])
 @pytest.mark.parametrize("N,K", [(64, 64), (101, 520), (4096, 4096), (33, 8 * 64 * 5 + 8)])
@@ -264,6 +322,26 @@ def test_gemm_split_k_many_launches_back_to_back():
     assert float((outs[0].float() - ref).abs().max()) < 2e-2
 
 
+@pytest.mark.parametrize("c", [dict(variant=3, block=256, vec=8, unroll=1, tile=[32, 64, 512]),
+                               dict(variant=3, block=256, vec=8, unroll=1, tile=[16, 64, 512]),
+                               dict(variant=0, block=256, vec=8, unroll=4, tile=[64, 64, 64], split_k=4)])
+def test_gemm_split_k_hands_over_fresh_partials(c):
+    # launches alternate between two problems in one workspace: a partial sum read before its writer's stores have
+    # landed would be the other problem's (small partials and a short hand-over are where that shows)
+    M, N, K = 32 if c["tile"][0] >= 32 else 16, 4096, 4096
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a = [torch.randn(M, K, device="cuda", generator=g).half() for _ in range(2)]
+    w = [(torch.randn(N, K, device="cuda", generator=g) * 0.02).half() for _ in range(2)]
+    outs = [torch.empty(M, N, dtype=torch.float16, device="cuda") for _ in range(120)]
+    for i, o in enumerate(outs):
+        ops.gemm(a[i % 2], w[i % 2], None, o, cfg(**c))
+    torch.cuda.synchronize()
+    for i, o in enumerate(outs):
+        assert torch.equal(o, outs[i % 2]), i
+    for i in range(2):
+        assert float((outs[i].float() - a[i].float() @ w[i].float().T).abs().max()) < 2e-2
+
+
 def test_gemm_split_k_on_two_streams_at_once():
     # each stream has its own partial tiles and arrival counters: launches that split K may overlap.
     # Two streams of the default priority take turns launching different problems without any
@@ -350,7 +428,8 @@ FUSED_CONFIGS = [None,
                  dict(variant=0, block=256, vec=8, tile=[256, 256, 64]),
                  dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64]),
                  dict(variant=0, block=256, vec=8, unroll=4, tile=[64, 64, 64], split_k=3),
-                 dict(variant=1, block=512, vec=8, unroll=4, tile=[80, 16, 32])]
+                 dict(variant=1, block=512, vec=8, unroll=4, tile=[80, 16, 32]),
+                 dict(variant=0, block=512, vec=8, unroll=2, tile=[256, 128, 64], split_k=2)]
 
 
 @pytest.mark.parametrize("kind", [1, 2, 3])
@@ -362,6 +441,19 @@ def test_gemm_fused_epilogues(oracle, kind, which, M, N, K):
     res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
     out = Guarded((M, N), torch.float32 if kind == 2 else torch.float16)
     c = None if FUSED_CONFIGS[which] is None else cfg(**FUSED_CONFIGS[which])
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c, epilogue=kind, res1=res[0], res2=res[1])
+    want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+    _check_fused(out.check(), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3])
+@pytest.mark.parametrize("rows,cols,kslice", [(16, 64, 1024), (32, 128, 512), (64, 64, 512)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 7, 8), (16, 130, 1096), (13, 2560, 2560)])
+def test_gemm_fused_epilogues_streaming_tile(oracle, kind, rows, cols, kslice, M, N, K):
+    a, w, bias, r1, r2 = _fused_inputs(M, N, K, M + N + K + kind)
+    res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+    out = Guarded((M, N), torch.float32 if kind == 2 else torch.float16)
+    c = cfg(variant=_lib.GEMM_STREAM, block=4 * cols, vec=8, unroll=1, tile=[rows, cols, kslice])
     ops.gemm(dev(a), dev(w), dev(bias), out.t, c, epilogue=kind, res1=res[0], res2=res[1])
     want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
     _check_fused(out.check(), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
