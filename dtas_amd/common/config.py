@@ -197,9 +197,12 @@ class GEMVConfig(Config):
         self.LOAD_V_SHARED = False
         self.LOAD_V_VEC = 8
         self.UNROLL = 2
+        # every sum in fp16, in the order of the reference's scheduled kernel (TS x TR = 16 x 32 threads there:
+        # 32 threads x 8 chains per row, experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:11-92)
+        self.ACC_F16 = False
 
     def to_dict(self) -> Dict:
-        return {"sapctial_thread": self.TS, "sapctial_tile": self.TILE_S, "reduction_thread": self.TR,
+        return {"acc_f16": self.ACC_F16, "sapctial_thread": self.TS, "sapctial_tile": self.TILE_S, "reduction_thread": self.TR,
                 "reduction_tile": self.TILE_R, "vec_c": self.VEC_C, "tag_s": self.TAG_S, "tag_r": self.TAG_R,
                 "load_v_shared": self.LOAD_V_SHARED, "load_v_vec": self.LOAD_V_VEC, "unroll_factor": self.UNROLL}
 
@@ -208,12 +211,15 @@ class GEMVConfig(Config):
         self.TS, self.TILE_S = dic["sapctial_thread"], dic["sapctial_tile"]
         self.TR, self.TILE_R, self.VEC_C = dic["reduction_thread"], dic["reduction_tile"], dic["vec_c"]
         self.UNROLL = dic.get("unroll_factor", 2)
+        self.ACC_F16 = dic.get("acc_f16", False)
         return self
 
     def to_abi(self):
         c = _lib.DtasConfig()
         c.variant, c.block, c.vec, c.unroll = _lib.GEMV_SPLITK, self.TR, self.VEC_C, self.UNROLL
         c.tile[0] = self.TILE_S
+        if self.ACC_F16:   # half a wavefront per row, 8 rows per workgroup of 256
+            c.variant, c.block, c.tile[0] = _lib.GEMV_RF16, 256, 8
         c.split_k = 1
         return c
 

@@ -94,6 +94,53 @@ __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restri
   }
 }
 
+// The same product with every sum in fp16, in the order of the reference's own scheduled kernel
+// (experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:11-92: rfactor over 256 strided chains per row, held 8 per
+// thread by 32 threads; the 8 folded in order; the 32 threads joined by the shuffle tree TVM lowers a
+// cross-thread reduction to, strides 16, 8, 4, 2, 1 as in .../layernorm/top1_256/tvm_device_kernels.cu:184-203).
+// Half a wavefront plays the 32 threads of a row: lane t owns chains j = 8t .. 8t+7, i.e. the 16-byte chunk t of
+// every 256-element step, so a step is 512 contiguous bytes of the row.  Products are rounded to fp16 before they
+// are added (no fused multiply-add: the PrimFunc has two fp16 operations).  Bit-identical to the CPU restatement.
+template <bool VEC>
+__global__ void __launch_bounds__(256) gemv_rf16_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
+                                                        GemvEpilogue ep, void* __restrict__ y, int64_t N, int64_t K) {
+#pragma clang fp contract(off)
+  const int t = threadIdx.x & 31;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 8 + (threadIdx.x >> 5);
+  const half_t* w = W + (row < N ? row : N - 1) * K;  // rows past N re-read the last row; never stored
+  half_t rf[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) rf[i] = static_cast<half_t>(0.f);
+  for (int64_t k0 = 8 * t; k0 < K; k0 += 256) {
+    if (VEC) {  // K % 8 == 0: a chunk is all inside the row
+      const f16x8 xv = __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(x + k0));
+      const f16x8 wv = __builtin_bit_cast(f16x8, load_stream(reinterpret_cast<const u32x4*>(w + k0)));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const half_t p = xv[i] * wv[i];
+        rf[i] = rf[i] + p;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (k0 + i < K) {
+          const half_t p = x[k0 + i] * w[k0 + i];
+          rf[i] = rf[i] + p;
+        }
+    }
+  }
+  half_t acc = static_cast<half_t>(0.f);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc = acc + rf[i];
+#pragma unroll
+  for (int d = 16; d >= 1; d >>= 1) {
+    // lane t adds lane t + d of its group of 32 (past the group: its own value, which lane 0's chain never reads)
+    const half_t other = __builtin_bit_cast(half_t, static_cast<unsigned short>(__shfl_down(static_cast<int>(__builtin_bit_cast(unsigned short, acc)), d, 32)));
+    acc = acc + other;
+  }
+  if (t == 0 && row < N) finish(static_cast<float>(acc), ep, y, row);
+}
+
 // fp32 operands and result (NT_matmul5, experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:8-19: the
 // 50280 x 2560 vocabulary projection of the decode graph): the same workgroup shape, 4 elements per
 // 128-bit access, fused multiply-adds in fp32.
@@ -168,6 +215,15 @@ int describe_gemv(int64_t N, int64_t K, const dtas_config& cfg, int64_t la[7]) {
   (void)K;
   for (int i = 0; i < 7; ++i) la[i] = 0;
   la[1] = la[2] = 1;
+  if (cfg.variant == DTAS_GEMV_RF16) {  // half a wavefront per row, 8 rows per workgroup
+    if (cfg.block != 256) return fail("gemv: the fp16-accumulate kernel uses 256 threads, got %d", cfg.block);
+    if (cfg.vec != 8 && cfg.vec != 1) return fail("gemv: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+    la[0] = ceil_div(N, 8);
+    la[3] = 256;
+    la[5] = 8;
+    if (la[0] > 0x7fffffff) return fail("gemv: N=%lld needs too many workgroups", (long long)N);
+    return 0;
+  }
   if (cfg.variant != DTAS_GEMV_SPLITK) return fail("gemv: unknown variant %d", cfg.variant);
   if (cfg.block < 64 || cfg.block > 512 || cfg.block % 64 != 0)
     return fail("gemv: block must be a multiple of 64 in [64, 512], got %d", cfg.block);
@@ -217,6 +273,11 @@ extern "C" int dtas_gemv_f16_fused(const void* x, const void* W, const void* bia
   const half_t* wp = static_cast<const half_t*>(W);
   const GemvEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1),
                            static_cast<const half_t*>(res2), epilogue};
+  if (cfg.variant == DTAS_GEMV_RF16) {
+    if (cfg.vec == 8) hipLaunchKernelGGL(gemv_rf16_kernel<true>, grid, block, 0, s, xp, wp, ep, y, N, K);
+    else hipLaunchKernelGGL(gemv_rf16_kernel<false>, grid, block, 0, s, xp, wp, ep, y, N, K);
+    return check_launch("gemv");
+  }
   if (cfg.vec == 1) {
     hipLaunchKernelGGL(gemv_scalar_kernel, grid, block, 0, s, xp, wp, ep, y, N, K);
     return check_launch("gemv");

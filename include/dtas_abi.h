@@ -90,7 +90,10 @@ enum dtas_variant {
   DTAS_RED_BLOCK_ROW = 1, /* one workgroup per row, row in registers, DPP + LDS staging */
   DTAS_RED_STREAM_ROW = 2,/* one workgroup per row, row re-read per pass: any length / alignment */
   /* GEMV (python/dtas/schedule/tir_gemv.py:33-249) */
-  DTAS_GEMV_SPLITK = 0,   /* K split over the lanes and wavefronts of a workgroup */
+  DTAS_GEMV_SPLITK = 0,   /* K split over the lanes and wavefronts of a workgroup; fp32 sums */
+  DTAS_GEMV_RF16 = 1,     /* every sum in fp16, in the order of the reference's scheduled kernel
+                             (experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:11-92): for results bit-identical to
+                             that kernel's arithmetic; block 256 (8 rows per workgroup), vec 8 or 1 */
   /* GEMM (python/dtas/schedule/tir_wmma.py:20-222) */
   DTAS_GEMM_MFMA = 0,     /* LDS-tiled MFMA, tile = tile[0] x tile[1] x tile[2] */
   DTAS_GEMM_SKINNY = 1,   /* small M: weight-streaming MFMA 16x16x32, split over N and K */

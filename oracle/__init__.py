@@ -68,6 +68,7 @@ class _C:
                 "oracle_layer_norm_f32": [vp, vp, vp, vp, i64, i64, ctypes.c_float, ci],
                 "oracle_gemm_f16": [vp, vp, vp, vp, i64, i64, i64, ci, ci],
                 "oracle_gemm_f16_f32out": [vp, vp, vp, i64, i64, i64, ci],
+                "oracle_gemv_f16_rf": [vp, vp, vp, vp, i64, i64, ci],
                 "oracle_gemm_f16_fused": [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, ci, ci],
                 "oracle_attn_scores_f16_f32": [vp, vp, vp, vp, i64, i64, i64, i64, f32, ci, ci],
                 "oracle_attn_pv_f16": [vp, vp, vp, i64, i64, i64, i64, ci, ci],
@@ -186,6 +187,16 @@ class c:  # noqa: N801  (namespace, mirrors the C file)
         out = np.empty(a.shape[:-1] + (N,), dtype=np.float16)
         bp = _ptr(bias) if bias is not None else None
         _C.lib().oracle_gemm_f16(_ptr(a), _ptr(w), bp, _ptr(out), M, N, K, int(acc_f16), threads)
+        return out
+
+    @staticmethod
+    def gemv_rf(x, w, bias=None, threads: int = 1) -> np.ndarray:
+        """y[N] = W[N,K] . x[K] (+ bias), every sum in fp16 in the order of the reference's scheduled GEMV kernel
+        (256 strided partial sums per row, folded 8 at a time, then the 32-lane shuffle tree)."""
+        assert x.dtype == np.float16 and w.dtype == np.float16 and x.size == w.shape[1]
+        N, K = w.shape
+        out = np.empty(N, dtype=np.float16)
+        _C.lib().oracle_gemv_f16_rf(_ptr(x), _ptr(w), _ptr(bias) if bias is not None else None, _ptr(out), N, K, threads)
         return out
 
     @staticmethod

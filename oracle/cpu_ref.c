@@ -302,6 +302,42 @@ void oracle_gemm_f16(const f16* A, const f16* W, const f16* bias, f16* C, int64_
   }
 }
 
+/* GEMV in the order of the reference's own scheduled kernel
+ * (experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:11-92: the GEMV rule's two-level rfactor, every buffer fp16):
+ *   rf[j], j < 256 (:12, :35-56): for o ascending, rf[j] = f16(rf[j] + f16(x[256 o + j] * W[row][256 o + j]))
+ *   rf1[t], t < 32 (:13, :57-73): from 0, + rf[8 t], + rf[8 t + 1], ..., + rf[8 t + 7], each step rounded
+ *   the 32 rf1 over threadIdx.x (:74-84): a cross-thread reduction, which TVM lowers to the shuffle tree that
+ *     the reference's committed kernels show (experiment/dtas_tuned/general_reduction/layernorm/top1_256/
+ *     tvm_device_kernels.cu:184-203): v[t] = f16(v[t] + v[t + d]) for d = 16, 8, 4, 2, 1; lane 0 holds the sum
+ *   y = f16(sum + bias[row]) (:85-91)
+ * The schedule is written for K = 10240; k past K contributes nothing here (the rule predicates it).
+ * Pinned by: hand-built inputs whose result depends on each of the three stages' order (tests/
+ * test_oracle_matmul.py), exactness on small integers, and agreement with the fp64 product within fp16 error. */
+void oracle_gemv_f16_rf(const f16* x, const f16* W, const f16* bias, f16* y, int64_t N, int64_t K, int nthreads) {
+  OMP_FOR(nthreads)
+  for (int64_t row = 0; row < N; ++row) {
+    const f16* w = W + row * K;
+    f16 rf[256];
+    for (int j = 0; j < 256; ++j) rf[j] = 0;
+    for (int64_t o = 0; o * 256 < K; ++o)
+      for (int j = 0; j < 256; ++j) {
+        const int64_t k = o * 256 + j;
+        if (k < K) rf[j] = f2h(h2f(rf[j]) + h2f(f2h(h2f(x[k]) * h2f(w[k]))));
+      }
+    f16 v[32];
+    for (int t = 0; t < 32; ++t) {
+      f16 acc = 0;
+      for (int i = 0; i < 8; ++i) acc = f2h(h2f(acc) + h2f(rf[8 * t + i]));
+      v[t] = acc;
+    }
+    for (int d = 16; d >= 1; d >>= 1)
+      for (int t = 0; t < d; ++t) v[t] = f2h(h2f(v[t]) + h2f(v[t + d]));
+    f16 r = v[0];
+    if (bias) r = f2h(h2f(r) + h2f(bias[row]));
+    y[row] = r;
+  }
+}
+
 /* The same sum with the fp32 accumulator returned unrounded; the parity tests
  * use it to bound the GPU's fp32 partial-sum reordering separately from the
  * final fp16 rounding. */

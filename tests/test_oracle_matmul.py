@@ -83,6 +83,47 @@ def test_fp16_accumulate_follows_the_primfunc_text(oracle):
     assert not np.array_equal(oracle.c.gemm(a, w, acc_f16=True), oracle.c.gemm(a, w))
 
 
+def test_gemv_rf_follows_the_order_of_the_reference_schedule(oracle):
+    """oracle.c.gemv_rf restates experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:11-92.  Each case below has a result
+    that one stage's order fixes: 2048 + 1 is a tie in fp16 (spacing 2) and rounds back to 2048, so ones added one at
+    a time vanish, ones added to each other first survive."""
+    def run(K, entries, x_entries=()):
+        w = np.zeros((1, K), np.float16)
+        x = np.ones(K, np.float16)
+        for k, v in entries:
+            w[0, k] = v
+        for k, v in x_entries:
+            x[k] = v
+        return float(oracle.c.gemv_rf(x, w)[0])
+    # stage 1, one strided chain (k = j, 256 + j, 512 + j), ascending: (2048 + 1) + 1 = 2048; descending would give 2050
+    assert run(768, [(0, 2048), (256, 1), (512, 1)]) == 2048.0
+    assert run(768, [(0, 1), (256, 1), (512, 2048)]) == 2050.0
+    # stage 2, the 8 chains of one lane, ascending from 0: ones after 2048 vanish; a pairwise fold would keep two of them
+    assert run(256, [(0, 2048), (1, 1), (2, 1), (3, 1), (4, 1)]) == 2048.0
+    assert run(256, [(0, 1), (1, 1), (2, 1), (3, 1), (4, 2048)]) == 2052.0
+    # stage 3, the 32 lanes (lane t owns k = 8t .. 8t+7), shuffle tree with strides 16, 8, 4, 2, 1:
+    # lanes 0..3 = 2048, 1, 1, 1: stride 2 gives lane 0 = 2048 + 1 = 2048 and lane 1 = 1 + 1, stride 1 adds them: 2050
+    # (a left-to-right sum would give 2048)
+    assert run(256, [(0, 2048), (8, 1), (16, 1), (24, 1)]) == 2050.0
+    # lanes 0, 16, 17 = 2048, 1, 1: stride 16 comes first, lane 0 = 2048 + 1 = 2048, lane 1 = 0 + 1, then 2048 + 1 = 2048
+    # (strides 1, 2, ..., 16 would join lanes 16 and 17 first: 2050)
+    assert run(256, [(0, 2048), (128, 1), (136, 1)]) == 2048.0
+    # the product is rounded before it is added: (1 + 2^-10)(1 - 2^-11) = 1.000488 rounds to 1, and 2048 + 1 = 2048;
+    # a fused multiply-add would see 2049.000488 and give 2050
+    assert run(512, [(0, 2048), (256, 1 - 2.0 ** -11)], [(256, 1 + 2.0 ** -10)]) == 2048.0
+    # small integers: exact whatever the order; bias added last, in fp16; K that is no multiple of 256
+    rng = np.random.default_rng(12)
+    xi, wi = rng.integers(-2, 3, 1000).astype(np.float16), rng.integers(-2, 3, (37, 1000)).astype(np.float16)
+    bi = rng.integers(-4, 5, 37).astype(np.float16)
+    assert np.array_equal(oracle.c.gemv_rf(xi, wi, bi).astype(np.float64), wi.astype(np.float64) @ xi.astype(np.float64) + bi)
+    # random data: within fp16 accumulation error of the exact product, and not the fp32-accumulated result
+    x, w = (rng.standard_normal(10240) * 0.5).astype(np.float16), (rng.standard_normal((64, 10240)) * 0.05).astype(np.float16)
+    got, f64 = oracle.c.gemv_rf(x, w, threads=4).astype(np.float64), w.astype(np.float64) @ x.astype(np.float64)
+    assert np.abs(got - f64).max() < 0.05
+    assert not np.array_equal(oracle.c.gemv_rf(x, w), oracle.c.gemm(x[None, :], w)[0])
+    assert np.array_equal(oracle.c.gemv_rf(x, w, threads=1).view(np.uint16), oracle.c.gemv_rf(x, w, threads=4).view(np.uint16))
+
+
 def test_threads_do_not_change_bits(oracle):
     a, w = _inputs(7, 33, 100)
     assert np.array_equal(oracle.c.gemm(a, w, threads=1).view(np.uint16), oracle.c.gemm(a, w, threads=4).view(np.uint16))

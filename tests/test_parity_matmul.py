@@ -49,6 +49,49 @@ def test_gemv_every_variant_and_bias(oracle, rows, block, N, K):
     _check(out.check().reshape(1, N), oracle.c.gemm(x, w, bias), oracle.np64.gemm(x, w, bias))
 
 
+@pytest.mark.parametrize("N,K", [(2560, 10240), (4096, 4096), (33, 1003), (7, 8), (1001, 2560), (64, 256), (5, 250)])
+def test_gemv_fp16_accumulate_in_the_reference_schedules_order(oracle, N, K):
+    # variant RF16: every sum in fp16 in the order of the reference's scheduled kernel -> the same bits as its CPU restatement
+    rng = np.random.default_rng(N + K)
+    x = (rng.standard_normal(K) * 0.5).astype(np.float16)
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    bias = rng.uniform(-1, 1, N).astype(np.float16)
+    c = cfg(variant=_lib.GEMV_RF16, block=256, vec=8, tile=[8, 0, 0])
+    for b in (bias, None):
+        out = Guarded((N,), torch.float16)
+        ops.gemv(dev(x), dev(w), None if b is None else dev(b), out.t, c)
+        assert_bits_equal(out.check(), oracle.c.gemv_rf(x, w, b, threads=8))
+    assert list(_lib.describe_launch(_lib.OP_GEMV_F16, 1, N, K, c).launch_args)[:4] == [-(-N // 8), 1, 1, 256]
+    # the fused epilogues act on the fp16 sum as they do on the rounded fp32 one
+    r1, r2 = rng.standard_normal(N).astype(np.float16), rng.standard_normal(N).astype(np.float16)
+    out = Guarded((N,), torch.float16)
+    ops.gemv(dev(x), dev(w), dev(bias), out.t, c, epilogue=1, res1=dev(r1), res2=dev(r2))
+    mm = oracle.c.gemv_rf(x, w, bias, threads=8)
+    assert_bits_equal(out.check(), ((r1 + mm).astype(np.float16) + r2).astype(np.float16))
+
+
+def test_gemv_fp16_accumulate_order_cases_and_errors(oracle):
+    # the hand-built cases that pin each stage's order in the oracle, through the kernel: 2048 + 1 ties back to 2048
+    def run(K, entries, x_entries=()):
+        w, x = np.zeros((3, K), np.float16), np.ones(K, np.float16)
+        for k, v in entries:
+            w[1, k] = v
+        for k, v in x_entries:
+            x[k] = v
+        out = Guarded((3,), torch.float16)
+        ops.gemv(dev(x), dev(w), None, out.t, cfg(variant=_lib.GEMV_RF16, block=256, vec=8, tile=[8, 0, 0]))
+        got = out.check()
+        assert_bits_equal(got, oracle.c.gemv_rf(x, w))
+        return float(got[1])
+    assert run(768, [(0, 2048), (256, 1), (512, 1)]) == 2048.0                      # a chain, ascending
+    assert run(256, [(0, 2048), (1, 1), (2, 1), (3, 1), (4, 1)]) == 2048.0          # a lane's 8 chains, ascending
+    assert run(256, [(0, 2048), (8, 1), (16, 1), (24, 1)]) == 2050.0                # the tree: strides 2 then 1
+    assert run(256, [(0, 2048), (128, 1), (136, 1)]) == 2048.0                      # ... after stride 16
+    assert run(512, [(0, 2048), (256, 1 - 2.0 ** -11)], [(256, 1 + 2.0 ** -10)]) == 2048.0   # product rounded before the add
+    with pytest.raises(_lib.DtasError, match="256 threads"):
+        _lib.describe_launch(_lib.OP_GEMV_F16, 1, 64, 64, cfg(variant=_lib.GEMV_RF16, block=128, vec=8, tile=[8, 0, 0]))
+
+
 def test_gemv_exact_and_ragged(oracle):
     rng = np.random.default_rng(2)
     w = (rng.standard_normal((96, 64)) * 0.02).astype(np.float16)
