@@ -40,6 +40,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # dense fp16 -> fp32 MFMA
 INFINITY_CACHE_BYTES = 256 << 20
 METRIC = "achieved HBM GB/s (eltwise/reduce/GEMV) + GEMM TFLOP/s, swept over dynamic n"
+OPERANDS = "normal"            # --operands: what the gemm_f16 workload multiplies
 
 
 # ---------------------------------------------------------------------------------------------
@@ -188,7 +189,18 @@ def _workload(name: str, n: int, extra=None):
                 8 * n * V + 4, 0)
     if name == "gemm_f16":
         N, K = extra
-        make = lambda s: (normal((n, K), s), normal((N, K), 100 + s, 0.02), empty((n, N)))
+        # OPERANDS != "normal" (--operands): the same launches on operands whose bits hardly toggle -- how far the
+        # card's power limit, not the kernel, sets the rate on the benchmark's random operands
+        def operand(shape, s, std):
+            if OPERANDS == "zeros":
+                return torch.zeros(shape, dtype=torch.float16, device="cuda")
+            if OPERANDS == "ones":
+                return torch.ones(shape, dtype=torch.float16, device="cuda")
+            if OPERANDS == "ints":
+                g.manual_seed(s)
+                return torch.randint(-2, 3, shape, device="cuda", generator=g).to(torch.float16)
+            return normal(shape, s, std)
+        make = lambda s: (operand((n, K), s, 1.0), operand((N, K), 100 + s, 0.02), empty((n, N)))
         return (make, lambda b: call(L.dtas_gemm_f16, P(b[0]), P(b[1]), None, P(b[2]), n, N, K, None, stream),
                 2 * (n * K + N * K + n * N), 2 * n * N * K)
     if name == "attn_scores_f16_f32":
@@ -485,11 +497,16 @@ def main() -> int:
                          "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | split3_f16 | swap_axes_f16 | attn_mask_f16 | softmax_temperature_f32 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
+    ap.add_argument("--operands", default="normal", choices=["normal", "zeros", "ones", "ints"],
+                    help="gemm_f16 only: normal = the benchmark's A ~ N(0,1), W ~ N(0,0.02); zeros / ones / ints (-2..2) "
+                         "run the same launches on operands that draw less power")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="time on one buffer set (no rotation)")
     ap.add_argument("--out", default=None, help="also write the sweep rows to this JSON file")
     args = ap.parse_args()
+    global OPERANDS
+    OPERANDS = args.operands
     if args.gpus != 1:
         print(f"bench.py measures one GPU: every kernel here runs on a single device and no collective exists "
               f"(--gpus {args.gpus} is not supported)", file=sys.stderr)
@@ -542,7 +559,7 @@ def main() -> int:
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(head["ms_per_step"], 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic" if OPERANDS == "normal" else f"synthetic ({OPERANDS}: not the benchmark's operands)",
         "config": {"workload": workload_key,
                    "buffers": "rotating pool > 3x Infinity Cache" if not args.cache_resident else "single set (cache-resident)",
                    "pool_sets": head["pool"], "launches_per_step": head["pool"],
