@@ -9,10 +9,11 @@
 // store; example output experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py).
 //
 // MFMA kernel (M > 64)
-//   tile     : BM x BN x 64 per workgroup; WM x WN wavefronts (8 for 256x256, else 4), each owning
-//              (BM/WM) x (BN/WN) as 32x32 blocks of v_mfma_f32_32x32x16_f16 (16x16 blocks of
-//              v_mfma_f32_16x16x32_f16 on the 8-wavefront tile), fp32 accumulators in registers.  Both operands are K-contiguous, so a tile row is one 128-byte
-//              line = 8 chunks of 16 bytes.
+//   tile     : BM x BN x 64 per workgroup; WM x WN wavefronts (8 for 256x256 and, on request, 256x128 /
+//              128x256; else 4), each owning (BM/WM) x (BN/WN) as 32x32 blocks of
+//              v_mfma_f32_32x32x16_f16 (16x16 blocks of v_mfma_f32_16x16x32_f16 on the 8-wavefront
+//              tiles), fp32 accumulators in registers.  Both operands are K-contiguous, so a tile row
+//              is one 128-byte line = 8 chunks of 16 bytes.
 //   global   : 128-bit buffer loads that write LDS directly (no register staging, no
 //              ds_write): one wavefront instruction fills one 1 KiB block = 8 tile rows; which
 //              (row, chunk) a lane fetches is the inverse of the LDS swizzle.  Rows past M / N
@@ -26,7 +27,7 @@
 //              tile, the loads of tile k+2 are issued right after it into the stage just
 //              vacated, and the first fragments of tile k+1 are read under the last MFMAs of
 //              tile k.  The interleaving is pinned with scheduling barriers.
-//              8-wavefront tile (256x256): v_mfma_f32_16x16x32_f16 (more flops per watt than 32x32x16,
+//              8-wavefront tiles: v_mfma_f32_16x16x32_f16 (more flops per watt than 32x32x16,
 //              and the card is power-limited on random operands), a whole k32 step of fragments in
 //              registers, one barrier per k tile; wavefronts w and w+4 share a SIMD, the older one
 //              wins the MFMA pipe, and each requests its share of the next units while the other
@@ -41,9 +42,12 @@
 //              PrimFuncs spell them.
 //   batches  : the attention matmuls run all heads in one launch (strides in GemmEpilogue).
 //   k-major W: for P.V the V tiles are transposed on their way into the LDS (template flag WT).
-// SKINNY kernel (M <= 64): the work is streaming W once; a workgroup owns 16 columns of C and
+// SKINNY kernel (M <= 80): the work is streaming W once; a workgroup owns 16 columns of C and
 //              all of M, its wavefronts split K, v_mfma_f32_16x16x32_f16 operands are loaded
 //              straight from global memory, partial tiles are folded through LDS.
+// STREAM kernel (M <= 64; the built-in choice for M <= 16): W rows come in as 1 KiB direct-to-LDS
+//              loads, everything a workgroup needs requested at once; K slices meet in the workspace.
+// ROWS kernel (M <= 4; the built-in choice for M = 2): W streamed in whole rows on the vector ALU.
 // Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles) and
 //              attn_pv_rows_kernel (P.V for a handful of query rows).
 #include "dtas_device.h"
@@ -184,7 +188,7 @@ __device__ __forceinline__ void wait_whole_tiles(int n) {
 // then transposed on the way into the LDS (two stages, 4 wavefronts only).
 // WQ: W is 8-bit with an fp16 scale per 32 elements of a row (Wq bytes [N][K], ep.wscale [N][K/32]); its
 // tiles are dequantised on their way into the LDS by the same register path.
-// M16: the 8-wavefront 256x256 tile on v_mfma_f32_16x16x32_f16 with one barrier per k tile (see the main loop).
+// M16: 8 wavefronts (256x256, 256x128, 128x256) on v_mfma_f32_16x16x32_f16 with one barrier per k tile (see the main loop).
 template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ W,
