@@ -293,10 +293,18 @@ def time_kernel(calls, steps: int, warmup: int, min_warm_s: float = 0.2):
     return wall, start.elapsed_time(stop) * 1e-3 / (steps * len(calls))
 
 
-def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool = True, min_region_s: float = 2e-3) -> dict:
+def measure(name: str, n: int, extra, steps: int, warmup: int, streaming: bool = True, min_region_s: float = 2e-3,
+            library: bool = False) -> dict:
+    """`library` (gemm_f16 only): the same pool, same order, same timing, through torch.matmul -- the vendor's GEMM
+    library -- instead of the C-ABI entry point: a yardstick measured on the same card, never part of `value`."""
     make, bind, nbytes, flops = _workload(name, n, extra)
     pool = make_pool(make, streaming)
-    calls = [bind(b) for b in pool]
+    if library:
+        import torch
+        assert name == "gemm_f16"
+        calls = [(lambda b: (lambda: torch.matmul(b[0], b[1].t(), out=b[2])))(b) for b in pool]
+    else:
+        calls = [bind(b) for b in pool]
     wall, per_launch = time_kernel(calls, steps, warmup)
     # short regions: lengthen the timed region so that event and synchronisation costs vanish
     if per_launch * steps * len(calls) < min_region_s:
@@ -500,6 +508,9 @@ def main() -> int:
     ap.add_argument("--operands", default="normal", choices=["normal", "zeros", "ones", "ints"],
                     help="gemm_f16 only: normal = the benchmark's A ~ N(0,1), W ~ N(0,0.02); zeros / ones / ints (-2..2) "
                          "run the same launches on operands that draw less power")
+    ap.add_argument("--beside-library", action="store_true",
+                    help="gemm_f16 only: also time torch.matmul (the vendor GEMM library) on the same operand pool and "
+                         "report it as `library_gemm`")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cache-resident", action="store_true", help="time on one buffer set (no rotation)")
@@ -576,6 +587,12 @@ def main() -> int:
             "algorithmic_bytes_per_launch": head["bytes"],
         },
     }
+    if args.beside_library and args.workload == "gemm_f16":
+        lib_row = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident, library=True)
+        again = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
+        line["library_gemm"] = {"call": "torch.matmul(A, W.t(), out=C), fp16", "launch_us_mean": lib_row["us"],
+                                "tflops": round(lib_row["tflops"], 3), "frac": round(lib_row["tflops"] / MFMA_FP16_PEAK_TFLOPS, 4),
+                                "this_kernel_after_it_us": again["us"]}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.workload if args.workload in ("cast_f32_f16", "add_f16", "copy_f16") else "rms_norm_f16",
                                             min(args.n, 4096))

@@ -912,7 +912,19 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     for (; k < my_split; ++k) add_partials(k, std::integral_constant<int, 1>{});
   }
 
-  constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots;
+  // The sums go through the LDS so that the stores are whole rows of the wavefront tile: staged as 8-byte slots of
+  // 4 columns (what a lane holds), read back kVecC columns per lane.  With 8 wavefronts a lane takes 16 bytes: half
+  // the store instructions for the same lines.
+  constexpr int kVecC = M16 ? 8 : 4;
+  constexpr int kSlots = WTN / 4, kLaneSlots = WTN / kVecC, kRowB = WTN * 2, kRowsPerPass = 64 / kLaneSlots;
+  using cvec_t = std::conditional_t<kVecC == 8, f16x8, f16x4>;
+  typedef cvec_t __attribute__((aligned(2))) cvec_a2;
+  // staging offset of 8-byte slot `s` of row m: the xor keeps a wavefront's writes (16 or 32 rows of one slot) and
+  // its reads (whole rows) on distinct banks; with 16-byte reads it leaves slot pairs together
+  auto stage_off = [](unsigned m, unsigned s) -> unsigned {
+    const unsigned x = M16 ? ((m >> 1) & (kSlots / 2 - 1)) << 1 : m & (kSlots - 1);
+    return m * kRowB + ((s ^ x) * 8);
+  };
   char* region = lds + wv * (WTM * kRowB);
   __syncthreads();  // every wavefront is done with the operand stages
   if constexpr (M16) {
@@ -925,8 +937,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         f16x4 hv;
 #pragma unroll
         for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(acc16[i][j][e]);
-        const unsigned slot = j * 4 + (l >> 4);
-        *reinterpret_cast<f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8)) = hv;
+        *reinterpret_cast<f16x4*>(region + stage_off(m, j * 4 + (l >> 4))) = hv;
       }
     }
   } else {
@@ -940,27 +951,19 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         f16x4 hv;
 #pragma unroll
         for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(acc[i][j][g * 4 + e]);
-        const unsigned slot = j * 8 + g * 2 + (l >> 5);
-        *reinterpret_cast<f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8)) = hv;
+        *reinterpret_cast<f16x4*>(region + stage_off(m, j * 8 + g * 2 + (l >> 5))) = hv;
       }
   }
   }
   // no barrier: a wavefront reads back only what it wrote itself
-  const unsigned slot = l % kSlots, rsub = l / kSlots;
-  const int64_t col = n0 + wn * WTN + slot * 4;
-  const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
-  const bool use_r1 = add2 || ep.kind == kEpiScores;
-  // 8-byte accesses to C and the residuals (16-byte to an fp32 C) for every slot that lies inside the row, at
-  // whatever alignment the row has
-  const bool vec_store = col + 3 < N;
-  (void)use_r1;
-  (void)add2;
-  float bv[4] = {0.f, 0.f, 0.f, 0.f};
-  if (ep.bias) {
+  const unsigned slot = l % kLaneSlots, rsub = l / kLaneSlots;
+  const int64_t col = n0 + wn * WTN + slot * kVecC;
+  // one access per lane to C and the residuals for every lane whose columns lie inside the row, at whatever
+  // alignment the row has
+  const bool vec_store = col + kVecC - 1 < N;
+  float bv[kVecC];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      if (col + e < N) bv[e] = static_cast<float>(ep.bias[col + e]);
-  }
+  for (int e = 0; e < kVecC; ++e) bv[e] = ep.bias && col + e < N ? static_cast<float>(ep.bias[col + e]) : 0.f;
   // one store loop per epilogue kind, chosen once (kind is uniform)
   auto store_tile = [&](auto kind_tag) {
     constexpr int KIND = decltype(kind_tag)::value;
@@ -971,12 +974,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // passes in groups of G: the group's residual / mask vectors are requested together, before the
     // first of them is needed (one at a time, every pass would wait out a memory round trip)
     constexpr int kPasses = WTM / kRowsPerPass;
-    // as many as the registers hold (two per vector): all 32 for one operand, 16 for two
-    constexpr int kWant = KIND == DTAS_EPI_BIAS_GELU ? 4 : kAdd2 ? 16 : kUseR1 ? 32 : 4;
-    constexpr int G = kPasses <= kWant ? kPasses : kPasses % kWant == 0 ? kWant : (kPasses % 8 == 0 ? 8 : (kPasses % 4 == 0 ? 4 : 1));
+    // as many as the registers hold (kVecC / 2 per vector): 128 registers for one operand, 64 each for two
+    constexpr int kWant = (KIND == DTAS_EPI_BIAS_GELU ? 16 : kAdd2 ? 64 : kUseR1 ? 128 : 16) / kVecC;
+    constexpr int G = kPasses <= kWant ? kPasses : kPasses % kWant == 0 ? kWant : (kPasses % 8 == 0 && kWant >= 8 ? 8 : (kPasses % 4 == 0 && kWant >= 4 ? 4 : 1));
 #pragma unroll 1
     for (int p0 = 0; p0 < kPasses; p0 += G) {
-      f16x4 r1v[G] = {}, r2v[G] = {};
+      cvec_t r1v[G] = {}, r2v[G] = {};
       if (kUseR1) {
 #pragma unroll
         for (int u = 0; u < G; ++u) {
@@ -984,11 +987,11 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           if (row >= M) continue;
           const int64_t at = row * N + col;
           if (vec_store) {
-            r1v[u] = *reinterpret_cast<const f16x4_a2*>(ep.res1 + at);
-            if (kAdd2) r2v[u] = *reinterpret_cast<const f16x4_a2*>(ep.res2 + at);
+            r1v[u] = *reinterpret_cast<const cvec_a2*>(ep.res1 + at);
+            if (kAdd2) r2v[u] = *reinterpret_cast<const cvec_a2*>(ep.res2 + at);
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+            for (int e = 0; e < kVecC; ++e)
               if (col + e < N) {
                 r1v[u][e] = ep.res1[at + e];
                 if (kAdd2) r2v[u][e] = ep.res2[at + e];
@@ -999,37 +1002,40 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
       for (int u = 0; u < G; ++u) {
         const unsigned m = (p0 + u) * kRowsPerPass + rsub;
-        f16x4 hv = *reinterpret_cast<const f16x4*>(region + m * kRowB + ((slot ^ (m & (kSlots - 1))) * 8));
+        cvec_t hv = *reinterpret_cast<const cvec_t*>(region + stage_off(m, slot * (kVecC / 4)));
         const int64_t row = m0 + wm * WTM + m;
         if (row >= M) continue;
         const int64_t at = row * N + col;
         if (KIND != DTAS_EPI_BIAS || has_bias) {  // "+ bias" etc. act on the sum already rounded to fp16
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
+          for (int e = 0; e < kVecC; ++e)
             hv[e] = epilogue_value_k<KIND>(hv[e], has_bias, ep.scale, bv[e], static_cast<float>(r1v[u][e]),
                                            static_cast<float>(r2v[u][e]));
         }
         if (kOutF32) {
           float* dst = static_cast<float*>(C) + at;
           if (vec_store) {
-            const f32x4v wide = {static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]),
-                                 static_cast<float>(hv[3])};
-            if (KIND == kEpiScores && N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 63u) == 0)
-              __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst));  // 4*heads*n*m bytes: streamed (rows of whole sectors)
-            else
-              *reinterpret_cast<f32x4v_a4*>(dst) = wide;
+            // 4*heads*n*m bytes of scores: streamed (rows of whole sectors)
+            const bool stream = KIND == kEpiScores && N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 63u) == 0;
+#pragma unroll
+            for (int h = 0; h < kVecC / 4; ++h) {
+              const f32x4v wide = {static_cast<float>(hv[4 * h]), static_cast<float>(hv[4 * h + 1]), static_cast<float>(hv[4 * h + 2]),
+                                   static_cast<float>(hv[4 * h + 3])};
+              if (stream) __builtin_nontemporal_store(wide, reinterpret_cast<f32x4v*>(dst + 4 * h));
+              else *reinterpret_cast<f32x4v_a4*>(dst + 4 * h) = wide;
+            }
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+            for (int e = 0; e < kVecC; ++e)
               if (col + e < N) dst[e] = static_cast<float>(hv[e]);
           }
         } else {
           half_t* dst = static_cast<half_t*>(C) + at;
           if (vec_store) {
-            *reinterpret_cast<f16x4_a2*>(dst) = hv;
+            *reinterpret_cast<cvec_a2*>(dst) = hv;
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+            for (int e = 0; e < kVecC; ++e)
               if (col + e < N) dst[e] = hv[e];
           }
         }
@@ -1314,22 +1320,32 @@ __global__ void __launch_bounds__(1024) gemm_skinny_kernel(const half_t* __restr
 // block (A is the first MFMA operand).
 __device__ __forceinline__ unsigned stream_swizzle(unsigned r) { return ((r & 7u) << 1) | ((r >> 3) & 1u); }
 
-template <int MT, int SEG, int WAVES>
+//
+// Q8: W is 8-bit with an fp16 scale per 32 elements of a row (bytes [N][K], ep.wscale [N][K/32], K % 256 == 0).  A
+// 512-element segment of a row is 512 bytes, so a 1 KiB load brings in two rows; the bytes sit in the LDS per
+// (wavefront, segment) as 16 rows of 512 bytes, 16-byte chunk c of row r in slot c ^ f(r) as above; a wavefront's
+// 16 x SEG x 16 scales arrive with one more load.  A lane's 8 weights of a k step are 8 consecutive bytes (lane
+// groups 0..3 take bytes 0-7, 16-23, 8-15, 24-31 of the step, matching the chunk order of the A fragments: lanes l
+// and l + 32 then read the two halves of one chunk) and are widened and scaled in registers, rounded as the
+// dequantiser rounds them.
+template <int MT, int SEG, int WAVES, bool Q8 = false>
 __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
                                                                 GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
                                                                 int64_t K, unsigned nsplit, float* __restrict__ ws,
                                                                 unsigned* __restrict__ arrivals) {
   constexpr int kCols = 16 * WAVES, kRowsA = 16 * MT, kSegBytes = 1024, kRowLds = SEG * kSegBytes;
-  constexpr int kALoads = kRowsA / WAVES * SEG, kWLoads = 16 * SEG;
-  static_assert(kRowsA % WAVES == 0 && (kCols + kRowsA) * kRowLds <= kLdsBytes && kALoads + kWLoads <= 63, "slab / LDS / vmcnt");
-  __shared__ __attribute__((aligned(1024))) char lds[(kCols + kRowsA) * kRowLds];
+  constexpr int kWSlab = Q8 ? kCols * SEG * 512 : kCols * kRowLds, kScaleSlab = Q8 ? WAVES * 1024 : 0;
+  constexpr int kALoads = kRowsA / WAVES * SEG, kWLoads = Q8 ? 8 * SEG + 1 : 16 * SEG;
+  static_assert(kRowsA % WAVES == 0 && kWSlab + kRowsA * kRowLds + kScaleSlab <= kLdsBytes && kALoads + kWLoads <= 63, "slab / LDS / vmcnt");
+  __shared__ __attribute__((aligned(1024))) char lds[kWSlab + kRowsA * kRowLds + kScaleSlab];
   const unsigned t = threadIdx.x, l = t & 63u;
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6);
   const unsigned tn = __builtin_amdgcn_readfirstlane(blockIdx.x / nsplit), z = __builtin_amdgcn_readfirstlane(blockIdx.x % nsplit);
   const int64_t n0 = static_cast<int64_t>(tn) * kCols;
   const int64_t rows_w = N - n0 < kCols ? N - n0 : kCols;
   const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
+  const unsigned w_row_bytes = Q8 ? static_cast<unsigned>(K) : row_bytes;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(reinterpret_cast<const char*>(W) + n0 * w_row_bytes, static_cast<unsigned>(rows_w) * w_row_bytes);
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, static_cast<unsigned>(M) * row_bytes);
   // lane l of the load of (row, segment s) fetches the chunk that belongs in slot l: chunk l ^ f(row); past K: out of range
   auto voff = [&](unsigned row, int s) -> unsigned {
@@ -1337,7 +1353,7 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
     const int64_t k = (static_cast<int64_t>(z) * SEG + s) * 512 + c * 8;
     return k < K ? row * row_bytes + static_cast<unsigned>(k) * 2u : kOob;
   };
-  char* lds_a = lds + kCols * kRowLds;
+  char* lds_a = lds + kWSlab;
 #pragma unroll
   for (int i = 0; i < kRowsA / WAVES; ++i) {
     const unsigned a = i * WAVES + wv;
@@ -1347,6 +1363,27 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(lds_a + a * kRowLds + s * kSegBytes), 16, at, 0, 0, 0);
     }
   }
+  char* lds_w8 = lds + wv * (SEG * 8192);          // Q8: this wavefront's bytes, [segment][row][512]
+  char* lds_sc = lds + kWSlab + kRowsA * kRowLds + wv * 1024;  // Q8: ... and scales, [row][16 * SEG]
+  if constexpr (Q8) {
+    {  // scales: lane l takes 8 of row l / (2 SEG)
+      const unsigned r = l / (2 * SEG), part = l % (2 * SEG);
+      const unsigned sc_row_bytes = static_cast<unsigned>(K >> 5) * 2u;
+      const __amdgpu_buffer_rsrc_t rs = make_rsrc(reinterpret_cast<const char*>(ep.wscale) + n0 * sc_row_bytes, static_cast<unsigned>(rows_w) * sc_row_bytes);
+      const int64_t k = static_cast<int64_t>(z) * (SEG * 512) + part * 256;
+      const unsigned at = (l < 32u * SEG && k < K) ? (wv * 16u + r) * sc_row_bytes + static_cast<unsigned>(k >> 5) * 2u : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)lds_sc, 16, at, 0, 0, 0);
+    }
+#pragma unroll
+    for (int s = 0; s < SEG; ++s)
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const unsigned r = 2u * q + (l >> 5), c = (l & 31u) ^ stream_swizzle(r);
+        const int64_t k = (static_cast<int64_t>(z) * SEG + s) * 512 + c * 16;
+        const unsigned at = k < K ? (wv * 16u + r) * w_row_bytes + static_cast<unsigned>(k) : kOob;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(lds_w8 + s * 8192 + q * 1024), 16, at, 0, 0, 0);
+      }
+  } else {
 #pragma unroll
   for (int s = 0; s < SEG; ++s)
 #pragma unroll
@@ -1354,6 +1391,7 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
       const unsigned row = wv * 16u + r, at = voff(row, s);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(lds + row * kRowLds + s * kSegBytes), 16, at, 0, 0, 0);
     }
+  }
   f32x4v acc[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) acc[i] = f32x4v{0.f, 0.f, 0.f, 0.f};
@@ -1365,15 +1403,39 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
   const unsigned x16 = ((((g & 1u) << 1) | (g >> 1)) ^ stream_swizzle(i16)) * 16u;
   const char* w_lane = lds + (wv * 16u + i16) * kRowLds;
   const char* a_lane = lds_a + i16 * kRowLds;
+  // Q8: bytes 8 p .. 8 p + 7 of the step, p = 0, 2, 1, 3 for lane groups 0..3: chunk 2 ks + (p >> 1), half p & 1
+  const unsigned p8 = ((g & 1u) << 1) | (g >> 1);
+  const unsigned x8 = (((p8 >> 1) ^ stream_swizzle(i16)) * 16u);
+  const char* w8_lane = lds_w8 + i16 * 512u + (p8 & 1u) * 8u;
+  f16x8 scales[Q8 ? 2 * SEG : 1];
 #pragma unroll
   for (int s = 0; s < SEG; ++s) {
-    if (s == 0) __builtin_amdgcn_s_waitcnt(waitcnt_imm(16 * (SEG - 1)));
+    if (s == 0) __builtin_amdgcn_s_waitcnt(waitcnt_imm((Q8 ? 8 : 16) * (SEG - 1)));
     else __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));
     DTAS_SCHED_FENCE();
+    if constexpr (Q8) {
+      if (s == 0) {
+#pragma unroll
+        for (int h = 0; h < 2 * SEG; ++h) scales[h] = *reinterpret_cast<const f16x8*>(lds_sc + i16 * (32 * SEG) + h * 16);
+      }
+    }
 #pragma unroll
     for (int ks = 0; ks < 16; ++ks) {
       const unsigned at = s * kSegBytes + (x16 ^ (ks * 64u));
-      const f16x8 fw = *reinterpret_cast<const f16x8*>(w_lane + at);
+      f16x8 fw;
+      if constexpr (Q8) {
+        const u32x2 raw = *reinterpret_cast<const u32x2*>(w8_lane + s * 8192 + (x8 ^ (ks * 32u)));
+        // (a step past K multiplies zeros of A: its scale is made zero too, whatever lies behind the row's scales)
+        const bool in = (static_cast<int64_t>(z) * SEG + s) * 512 + ks * 32 < K;
+        const half_t sc = in ? scales[2 * s + ks / 8][ks % 8] : static_cast<half_t>(0.f);
+        const f16x2 s2 = {sc, sc};
+        f16x2 d0, d1, d2, d3;
+        dequant_q8_word(raw[0], s2, d0, d1);
+        dequant_q8_word(raw[1], s2, d2, d3);
+        fw = f16x8{d0[0], d0[1], d1[0], d1[1], d2[0], d2[1], d3[0], d3[1]};
+      } else {
+        fw = *reinterpret_cast<const f16x8*>(w_lane + at);
+      }
 #pragma unroll
       for (int i = 0; i < MT; ++i)
         acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const f16x8*>(a_lane + i * 16 * kRowLds + at), fw, acc[i], 0, 0, 0);
@@ -1832,7 +1894,7 @@ int launch_mfma(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilo
 }
 
 // The W-streaming kernel: 16 * WAVES columns and SEG * 512 elements of K per workgroup, K slices met in the workspace.
-template <int MT, int SEG, int WAVES>
+template <int MT, int SEG, int WAVES, bool Q8 = false>
 int launch_stream(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N, int64_t K) {
   const size_t tiles = static_cast<size_t>(ceil_div(N, 16 * WAVES));
   const int nsplit = static_cast<int>(ceil_div(K, SEG * 512));
@@ -1842,7 +1904,7 @@ int launch_stream(hipStream_t s, const half_t* A, const half_t* W, const GemmEpi
   if (nsplit > 1 && split_scratch(s, tiles * nsplit * (16 * MT) * (16 * WAVES) * sizeof(float), tiles, nsplit, &partials, &arrivals, &ws_lock) != 0)
     return -1;
   if (tiles * nsplit > 0x7fffffffu) return fail("gemm: too many workgroups");
-  hipLaunchKernelGGL((gemm_stream_kernel<MT, SEG, WAVES>), dim3(static_cast<unsigned>(tiles * nsplit)), dim3(64 * WAVES), 0, s, A, W, ep,
+  hipLaunchKernelGGL((gemm_stream_kernel<MT, SEG, WAVES, Q8>), dim3(static_cast<unsigned>(tiles * nsplit)), dim3(64 * WAVES), 0, s, A, W, ep,
                      C, M, N, K, static_cast<unsigned>(nsplit), partials, arrivals);
   return check_launch("gemm");
 }
@@ -2369,6 +2431,33 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
     return dtas_gemv_q8_f16(A, Wq, scale, bias, C, N, K, epilogue, nullptr, stream);
   GemmEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1), static_cast<const half_t*>(res2),
                      epilogue, out_bytes == 4 ? 1 : 0, 0.f, 0, 0, 0, 0, 1, 0, static_cast<const half_t*>(scale)};
+  // Few rows of A: the launch is one read of the bytes of W.  The W-streaming kernel widens them on their way
+  // from the LDS into the MFMA (cfg: DTAS_GEMM_STREAM with tile 16x64x512, 16x64x1024 or 32x64x512).
+  {
+    const bool stream_ok = K > 0 && K % 256 == 0 && aligned(A, 16) && aligned(Wq, 16) && aligned(scale, 16) && K < (int64_t{1} << 24);
+    const half_t* a = static_cast<const half_t*>(A);
+    const half_t* w = static_cast<const half_t*>(Wq);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (user && user->variant == DTAS_GEMM_STREAM) {
+      const int bm = user->tile[0], bn = user->tile[1], bk = user->tile[2];
+      if (!((bm == 16 && bn == 64 && (bk == 512 || bk == 1024)) || ((bm == 32 || bm == 64) && bn == 64 && bk == 512)))
+        return fail("gemm_q8: the W-streaming kernel takes tiles 16x64x512, 16x64x1024, 32x64x512 and 64x64x512 for 8-bit weights, got %dx%dx%d", bm, bn, bk);
+      if (user->block != 256) return fail("gemm_q8: the 64-column streaming tile uses 256 threads, got %d", user->block);
+      if (M > bm) return fail("gemm_q8: a streaming tile of %d rows cannot hold M=%lld", bm, (long long)M);
+      if (!stream_ok) return fail("gemm_q8: the W-streaming kernel needs K %% 256 == 0 and 16-byte aligned A, W and scales");
+      if (bm == 64) return launch_stream<4, 1, 4, true>(s, a, w, ep, C, M, N, K);
+      if (bm == 32) return launch_stream<2, 1, 4, true>(s, a, w, ep, C, M, N, K);
+      return bk == 512 ? launch_stream<1, 1, 4, true>(s, a, w, ep, C, M, N, K) : launch_stream<1, 2, 4, true>(s, a, w, ep, C, M, N, K);
+    }
+    if (!user && stream_ok && M <= 32) {
+      // measured at the model's shapes (M = 16: 10.1 against 25.6 us at 7680x2560, 14.9 against 92 at 2560x10240;
+      // M = 32: 14.0 against 26.3 and 20.5 against 33.8).  512-element slices (three workgroups per CU) unless K is
+      // long: from 16 slices on the hand-over of the partial sums costs more than the second workgroup hides
+      if (M > 16) return launch_stream<2, 1, 4, true>(s, a, w, ep, C, M, N, K);
+      if (K >= 8192) return launch_stream<1, 2, 4, true>(s, a, w, ep, C, M, N, K);
+      return launch_stream<1, 1, 4, true>(s, a, w, ep, C, M, N, K);
+    }
+  }
   // Two routes.  Dequantising in the W path of the GEMM (no intermediate) runs on a plain burst pipeline without
   // split K: measured at the model's shapes it wins for M <= 64 with K <= 4096 (18 against 24 us at 7680x2560)
   // and loses beyond (M = 2048: 109 against 84 us; K = 10240: 2x or more).  Otherwise: the dequantiser into a

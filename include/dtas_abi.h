@@ -20,8 +20,9 @@
  *    host.cc:64-69); the leading batch-1 dim of (1, n, H) is not passed;
  *  - `stream` is a hipStream_t (NULL = the default stream); nothing synchronises, the kernel is
  *    enqueued on `stream` on the current device.  Nothing is allocated, with one exception:
- *    dtas_gemm_f16 with K split over workgroups (split_k > 1, or 0 on the 256x256 tile; the built-in
- *    table chooses either when M x N leaves CUs idle) keeps fp32 partial tiles in a workspace that the
+ *    dtas_gemm_f16 with K split over workgroups (split_k > 1, 0 on the 256x256 tile, or the
+ *    W-streaming kernel, also behind dtas_gemm_q8_f16_fused for M <= 32; the built-in table chooses
+ *    these when M x N leaves CUs idle) keeps fp32 partial tiles in a workspace that the
  *    library allocates on first use and grows on demand (32 MiB at first, at most 1 GiB; growing
  *    waits for the device).  There is one workspace per (device, stream): launches on one stream are
  *    ordered by it, launches on different streams use different workspaces and may overlap; the
@@ -340,8 +341,11 @@ int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, 
 /* dtas_gemm_q8_f16_fused: C[M,N] = epilogue(A[M,K] . W^T) with W dequantised on its way into the LDS, never
  * written: the dynamic-n forms fused_fused_decode2_fused_NT_matmul6_add4 (:371-399), ..decode4.._matmul9_add6_gelu1
  * (:504-581), ..decode5.._matmul4_add1; epilogues as dtas_gemm_f16_fused.  cfg, when given: a DTAS_GEMM_MFMA row
- * with tile {256,128,64} or {128,128,64} and unroll 3, or {64,64,64} and unroll 2.  One row with a bias or GELU
- * epilogue goes to dtas_gemv_q8_f16.  With cfg == NULL and M > 64 or K > 4096 the library takes the faster
+ * with tile {256,128,64} or {128,128,64} and unroll 3, or {64,64,64} and unroll 2; or a DTAS_GEMM_STREAM row
+ * (block 256, tile {16,64,512}, {16,64,1024}, {32,64,512} or {64,64,512}; M <= tile[0]; K % 256 == 0; 16-byte
+ * aligned A, Wq and scale): the W-streaming kernel on the bytes of W, widened between the LDS and the MFMA; its K
+ * slices meet in the split-K workspace.  One row with a bias or GELU epilogue goes to dtas_gemv_q8_f16.  With
+ * cfg == NULL: M <= 32 takes the W-streaming kernel where it applies; otherwise M > 64 or K > 4096 take the
  * two-pass route: dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on
  * demand, at most 1 GiB; same sharing rule as the split-K workspace), then dtas_gemm_f16_fused. */
 int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias,

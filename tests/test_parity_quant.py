@@ -252,6 +252,66 @@ def test_gemm_q8_at_the_models_shapes(oracle, M, N, K, kind):
     _check_gemm_q8(out.check().reshape(M, N)[rows], np.ascontiguousarray(a[rows]), wq, scale, bias, None, None, kind, oracle)
 
 
+Q8_STREAM_TILES = [(16, 64, 512), (16, 64, 1024), (32, 64, 512), (64, 64, 512)]
+
+
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("rows,cols,kslice", Q8_STREAM_TILES)
+@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (5, 7, 512), (16, 130, 768), (13, 200, 1280), (16, 2560, 2560), (9, 333, 4096)])
+def test_gemm_q8_streaming_tiles(oracle, kind, rows, cols, kslice, M, N, K):
+    M = M if M < 16 else rows                                  # a full tile of rows where the case asks for one
+    # the W-streaming kernel on bytes: K of one slice, a slice and a half, several; ragged N; every epilogue
+    rng = np.random.default_rng(M + N + K + kind)
+    wq, scale = _weights(N, K, M * 5 + N)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    r1 = rng.standard_normal((M, N)).astype(np.float16) if kind in (1, 2) else None
+    r2 = rng.standard_normal((M, N)).astype(np.float16) if kind in (1, 2) else None
+    out = Guarded((M, N), torch.float32 if kind == 2 else torch.float16)
+    c = cfg(variant=_lib.GEMM_STREAM, block=256, vec=8, unroll=1, tile=[rows, cols, kslice])
+    ops.gemm_q8(dev(a), _words(wq), dev(scale), dev(bias), out.t, c, kind,
+                dev(r1) if r1 is not None else None, dev(r2) if r2 is not None else None)
+    _check_gemm_q8(out.check(), a, wq, scale, bias, r1, r2, kind, oracle)
+
+
+def test_gemm_q8_streaming_is_the_choice_for_few_rows_exact_and_reproducible(oracle):
+    # one-hot rows of A return decoded columns of W bit for bit, through the route cfg = NULL takes for M <= 16
+    wq, scale = _weights(200, 1280, 3)
+    w = oracle.c.decode_q8(wq, scale)
+    ks = (0, 7, 31, 32, 511, 512, 1279)
+    a = np.zeros((len(ks), 1280), np.float16)
+    for i, k in enumerate(ks):
+        a[i, k] = 1
+    out = Guarded((len(ks), 200), torch.float16)
+    ops.gemm_q8(dev(a), _words(wq), dev(scale), None, out.t)
+    assert np.array_equal(out.check().view(np.uint16), np.ascontiguousarray(w[:, list(ks)].T).view(np.uint16))
+    # K slices are added in slice order whoever arrives last: three launches agree bit for bit
+    rng = np.random.default_rng(8)
+    wq, scale = _weights(2560, 2560, 9)
+    a = rng.standard_normal((16, 2560)).astype(np.float16)
+    runs = []
+    for _ in range(3):
+        out = Guarded((16, 2560), torch.float16)
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, out.t)
+        runs.append(out.check())
+    assert all(np.array_equal(r.view(np.uint16), runs[0].view(np.uint16)) for r in runs)
+    _check_gemm_q8(runs[0], a, wq, scale, None, None, None, 0, oracle)
+    # K off 256: the tiles take over
+    wq, scale = _weights(96, 160, 5)
+    a = rng.standard_normal((4, 160)).astype(np.float16)
+    out = Guarded((4, 96), torch.float16)
+    ops.gemm_q8(dev(a), _words(wq), dev(scale), None, out.t)
+    _check_gemm_q8(out.check(), a, wq, scale, None, None, None, 0, oracle)
+    c = torch.empty(4, 96, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.DtasError, match="K % 256"):
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=_lib.GEMM_STREAM, block=256, vec=8, unroll=1, tile=[16, 64, 512]))
+    with pytest.raises(_lib.DtasError, match="cannot hold M=17"):
+        ops.gemm_q8(dev(np.zeros((17, 256), np.float16)), _words(_weights(8, 256, 1)[0]), dev(_weights(8, 256, 1)[1]), None,
+                    torch.empty(17, 8, dtype=torch.float16, device="cuda"), cfg(variant=_lib.GEMM_STREAM, block=256, vec=8, unroll=1, tile=[16, 64, 512]))
+    with pytest.raises(_lib.DtasError, match="16x64x512, 16x64x1024, 32x64x512 and 64x64x512"):
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=_lib.GEMM_STREAM, block=512, vec=8, unroll=1, tile=[16, 128, 512]))
+
+
 def test_gemm_q8_exact_cases_fallback_and_errors(oracle):
     # A = rows of the identity returns columns... of W^T: C[i, :] = decoded W[:, k_i], bit for bit
     wq, scale = _weights(96, 128, 3)
