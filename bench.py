@@ -222,10 +222,13 @@ def _workload(name: str, n: int, extra=None):
     if name == "gemm_q8_f16":
         # fused_fused_decode2_fused_NT_matmul6_add4: 8-bit weights + fp16 group scales, bias epilogue, n rows
         N, K = extra
-        g = torch.Generator(device="cuda").manual_seed(300)
-        wq = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device="cuda", generator=g)
-        sc, bias = uniform((N, K // 32), 301, 0.001, 0.02), uniform((N,), 302)
-        make = lambda s: (normal((n, K), s), wq, sc, bias, empty((n, N)))
+        bias = uniform((N,), 302)
+
+        def make(s):
+            # the weights rotate with the rest: with few rows the launch is a read of them
+            g.manual_seed(300 + s)
+            wq = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device="cuda", generator=g)
+            return (normal((n, K), s), wq, uniform((N, K // 32), 301 + s, 0.001, 0.02), bias, empty((n, N)))
         return (make, lambda b: call(L.dtas_gemm_q8_f16_fused, P(b[0]), P(b[1]), P(b[2]), P(b[3]), None, None, P(b[4]), n, N, K, 0,
                                      None, stream),
                 2 * n * K + N * K + 2 * N * (K // 32) + 2 * n * N + 2 * N, 2 * n * N * K)

@@ -1340,7 +1340,9 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
   __shared__ __attribute__((aligned(1024))) char lds[kWSlab + kRowsA * kRowLds + kScaleSlab];
   const unsigned t = threadIdx.x, l = t & 63u;
   const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6);
-  const unsigned tn = __builtin_amdgcn_readfirstlane(blockIdx.x / nsplit), z = __builtin_amdgcn_readfirstlane(blockIdx.x % nsplit);
+  // (the K slices of a column tile, which share lines of the scales, run on one XCD)
+  const unsigned item = Q8 ? xcd_contiguous_id(blockIdx.x, gridDim.x) : blockIdx.x;
+  const unsigned tn = __builtin_amdgcn_readfirstlane(item / nsplit), z = __builtin_amdgcn_readfirstlane(item % nsplit);
   const int64_t n0 = static_cast<int64_t>(tn) * kCols;
   const int64_t rows_w = N - n0 < kCols ? N - n0 : kCols;
   const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
