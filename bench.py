@@ -235,13 +235,13 @@ def _workload(name: str, n: int, extra=None):
     if name in ("gemm_add2_f16", "gemm_gelu_f16"):
         # fused_NT_matmul2_add1_add3_add3 at (N, K) = (2560, 2560); fused_NT_matmul3_add2_gelu at (10240, 2560)
         N, K = extra
-        wt, bias = normal((N, K), 100, 0.02), uniform((N,), 101)
+        bias = uniform((N,), 101)
         if name == "gemm_add2_f16":
-            make = lambda s: (normal((n, K), s), wt, bias, normal((n, N), s + 1), normal((n, N), s + 2), empty((n, N)))
+            make = lambda s: (normal((n, K), s), normal((N, K), 100 + s, 0.02), bias, normal((n, N), s + 1), normal((n, N), s + 2), empty((n, N)))
             return (make, lambda b: call(L.dtas_gemm_f16_fused, P(b[0]), P(b[1]), P(b[2]), P(b[3]), P(b[4]), P(b[5]), n, N, K,
                                          _lib.EPI_BIAS_ADD2, None, stream),
                     2 * (n * K + N * K + 3 * n * N + N), 2 * n * N * K)
-        make = lambda s: (normal((n, K), s), wt, bias, empty((n, N)))
+        make = lambda s: (normal((n, K), s), normal((N, K), 100 + s, 0.02), bias, empty((n, N)))
         return (make, lambda b: call(L.dtas_gemm_f16_fused, P(b[0]), P(b[1]), P(b[2]), None, None, P(b[3]), n, N, K,
                                      _lib.EPI_BIAS_GELU, None, stream),
                 2 * (n * K + N * K + n * N + N), 2 * n * N * K)

@@ -962,8 +962,12 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // alignment the row has
   const bool vec_store = col + kVecC - 1 < N;
   float bv[kVecC];
+  cvec_t bvh;
 #pragma unroll
-  for (int e = 0; e < kVecC; ++e) bv[e] = ep.bias && col + e < N ? static_cast<float>(ep.bias[col + e]) : 0.f;
+  for (int e = 0; e < kVecC; ++e) {
+    bvh[e] = ep.bias && col + e < N ? ep.bias[col + e] : static_cast<half_t>(0.f);
+    bv[e] = static_cast<float>(bvh[e]);
+  }
   // one store loop per epilogue kind, chosen once (kind is uniform)
   auto store_tile = [&](auto kind_tag) {
     constexpr int KIND = decltype(kind_tag)::value;
@@ -1006,7 +1010,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         const int64_t row = m0 + wm * WTM + m;
         if (row >= M) continue;
         const int64_t at = row * N + col;
-        if (KIND != DTAS_EPI_BIAS || has_bias) {  // "+ bias" etc. act on the sum already rounded to fp16
+        if constexpr (KIND == DTAS_EPI_BIAS_GELU) {
+          hv = gelu_erf_f16_steps_vec<cvec_t, kVecC>(hv, has_bias, bvh);
+        } else if (KIND != DTAS_EPI_BIAS || has_bias) {  // "+ bias" etc. act on the sum already rounded to fp16
 #pragma unroll
           for (int e = 0; e < kVecC; ++e)
             hv[e] = epilogue_value_k<KIND>(hv[e], has_bias, ep.scale, bv[e], static_cast<float>(r1v[u][e]),
