@@ -33,7 +33,8 @@
 //              wins the MFMA pipe, and each requests its share of the next units while the other
 //              multiplies (a wavefront that issues a load stalls until the load path takes it).
 //   epilogue : accumulators -> fp16 -> wavefront-private LDS region (xor-swizzled 8-byte
-//              slots) -> 8-byte coalesced row stores with the bias added on the way out.
+//              slots) -> coalesced stores of whole tile rows (8 bytes per lane, 16 on the
+//              8-wavefront tiles) with the bias added on the way out.
 //   launch   : workgroup ids are remapped so that each XCD (own L2) works on a compact patch of
 //              the tile grid.
 //   split K  : few output tiles -> several workgroups share a tile and meet in a workspace.
@@ -47,6 +48,8 @@
 //              straight from global memory, partial tiles are folded through LDS.
 // STREAM kernel (M <= 64; the built-in choice for M <= 16): W rows come in as 1 KiB direct-to-LDS
 //              loads, everything a workgroup needs requested at once; K slices meet in the workspace.
+//              With 8-bit weights (M <= 32) the bytes ride the same loads and are widened between
+//              the LDS and the MFMA.
 // ROWS kernel (M <= 4; the built-in choice for M = 2): W streamed in whole rows on the vector ALU.
 // Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles) and
 //              attn_pv_rows_kernel (P.V for a handful of query rows).
