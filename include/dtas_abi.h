@@ -21,7 +21,7 @@
  *  - `stream` is a hipStream_t (NULL = the default stream); nothing synchronises, the kernel is
  *    enqueued on `stream` on the current device.  Nothing is allocated, with one exception:
  *    dtas_gemm_f16 with K split over workgroups (split_k > 1, 0 on the 256x256 tile, or the
- *    W-streaming kernel, also behind dtas_gemm_q8_f16_fused for M <= 32; the built-in table chooses
+ *    W-streaming kernel, also behind dtas_gemm_q8_f16_fused for few rows; the built-in table chooses
  *    these when M x N leaves CUs idle) keeps fp32 partial tiles in a workspace that the
  *    library allocates on first use and grows on demand (32 MiB at first, at most 1 GiB; growing
  *    waits for the device).  There is one workspace per (device, stream): launches on one stream are
@@ -345,8 +345,8 @@ int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, 
  * (block 256, tile {16,64,512}, {16,64,1024}, {32,64,512} or {64,64,512}; M <= tile[0]; K % 256 == 0; 16-byte
  * aligned A, Wq and scale): the W-streaming kernel on the bytes of W, widened between the LDS and the MFMA; its K
  * slices meet in the split-K workspace.  One row with a bias or GELU epilogue goes to dtas_gemv_q8_f16.  With
- * cfg == NULL: M <= 32 takes the W-streaming kernel where it applies; otherwise M > 64 or K > 4096 take the
- * two-pass route: dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on
+ * cfg == NULL: M <= 32 (M <= 64 with N, K <= 4096) takes the W-streaming kernel where it applies; otherwise
+ * M > 64 or K > 4096 take the two-pass route: dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on
  * demand, at most 1 GiB; same sharing rule as the split-K workspace), then dtas_gemm_f16_fused. */
 int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias,
                            const void* res1, const void* res2, void* C, int64_t M, int64_t N, int64_t K,

@@ -239,17 +239,21 @@ def test_gemm_q8_every_tile_on_ragged_shapes(oracle, which, M, N, K, kind):
     _check_gemm_q8(out.check(), a, wq, scale, bias, r1, r2, kind, oracle)
 
 
-@pytest.mark.parametrize("M", [1, 16, 256, 2048])
-@pytest.mark.parametrize("N,K,kind", [(7680, 2560, 0), (10240, 2560, 3), (2560, 10240, 0)])
+@pytest.mark.parametrize("M", [1, 16, 32, 64, 256, 2048])
+@pytest.mark.parametrize("N,K,kind", [(7680, 2560, 0), (10240, 2560, 3), (2560, 10240, 0), (2560, 2560, 1)])
 def test_gemm_q8_at_the_models_shapes(oracle, M, N, K, kind):
     rng = np.random.default_rng(M + N + kind)
     wq, scale = _weights(N, K, N + K)
     a = rng.standard_normal((M, K)).astype(np.float16)
     bias = rng.standard_normal(N).astype(np.float16)
+    r1 = rng.standard_normal((M, N)).astype(np.float16) if kind == 1 else None
+    r2 = rng.standard_normal((M, N)).astype(np.float16) if kind == 1 else None
     out = Guarded((1, M, N), torch.float16)
-    ops.gemm_q8(dev(a).view(1, M, K), _words(wq), dev(scale), dev(bias), out.t, None, kind)
+    ops.gemm_q8(dev(a).view(1, M, K), _words(wq), dev(scale), dev(bias), out.t, None, kind,
+                dev(r1) if kind == 1 else None, dev(r2) if kind == 1 else None)
     rows = np.unique(np.concatenate([np.arange(min(M, 8)), [M // 2, M - 1]]))       # sampled rows against the oracle
-    _check_gemm_q8(out.check().reshape(M, N)[rows], np.ascontiguousarray(a[rows]), wq, scale, bias, None, None, kind, oracle)
+    _check_gemm_q8(out.check().reshape(M, N)[rows], np.ascontiguousarray(a[rows]), wq, scale, bias,
+                   None if r1 is None else np.ascontiguousarray(r1[rows]), None if r2 is None else np.ascontiguousarray(r2[rows]), kind, oracle)
 
 
 Q8_STREAM_TILES = [(16, 64, 512), (16, 64, 1024), (32, 64, 512), (64, 64, 512)]
