@@ -540,7 +540,7 @@ def main() -> int:
 
     extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32", "take_q8_f16", "take_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
-    is_gemm = args.workload == "gemm_f16" and head["bound"] == "mfma"
+    is_gemm = args.workload in ("gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") and head["bound"] == "mfma"
     info = None
     try:
         op = {"cast_f32_f16": _lib.OP_CAST_F32_F16, "add_f16": _lib.OP_ADD_F16, "copy_f16": _lib.OP_COPY_F16,
