@@ -22,6 +22,10 @@ The same JSON line also carries
   cpu_baseline.families : the oracle on bounded samples of a GEMV and a GEMM point;
   sweep        : every op family over the dynamic extent n (GB/s or TFLOP/s and roofline fraction),
                  all of them HBM-streaming (rotating buffer sets, the GEMM's W included).
+For the gemm_f16 workload two more switches: `--operands zeros|ones|ints` runs the same launches on operands whose
+bits hardly toggle (how far the card's power limit sets the rate on the benchmark's random operands), and
+`--beside-library` times torch.matmul -- the vendor's GEMM library -- on the same operand pool and reports it as
+`library_gemm`, a yardstick that is never part of `value`.
 One GPU only: `--gpus N` with N > 1 exits with a message.
 """
 from __future__ import annotations
