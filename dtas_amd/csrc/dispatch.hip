@@ -197,6 +197,15 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   // 12.8 us at 4096 x 4096, 7.2 against 10.2 at 2560 x 2560; with more workgroups than CUs a workgroup's loads,
   // MFMAs and the hand-over of its partial sums are no longer hidden behind another's, and the tiles win again
   if (M_hi <= 16 && ceil_div(n, 64) * ceil_div(k, 1024) <= kNumCU) return make(DTAS_GEMM_STREAM, 256, 8, 1, 16, 64, 1024);
+  // M <= 16 against more rows of W: the looping form (the whole of K per workgroup, nothing handed over) while its
+  // workgroups run in one round -- 16 columns each (one wavefront, two workgroups per CU) for 4096 < N <= 8192, 64
+  // columns (one per CU) for 8192 <= N <= 16384 -- and K is short enough for a round to be worth its start:
+  // 15.9 against 20.2 us at 8192 x 4096, 10.6 / 13.5 at 7680 x 2560, 20.4 / 24.5 at 11008 x 4096, 13.0 / 16.4 at
+  // 10240 x 2560; level at K = 8192 and from two rounds on (32000 x 4096), behind at N <= 4096
+  if (M_hi <= 16 && k <= 4096) {
+    if (ceil_div(n, 16) > kNumCU && ceil_div(n, 16) <= 2 * kNumCU) return make(DTAS_GEMM_STREAM, 64, 8, 1, 16, 16, 256);
+    if (ceil_div(n, 64) >= kNumCU / 2 && ceil_div(n, 64) <= kNumCU) return make(DTAS_GEMM_STREAM, 256, 8, 1, 16, 64, 256);
+  }
   if (M_hi <= 32) {
     // (one workgroup per 16 rows of W: fewer than one per CU leave CUs idle)
     const double skinny_wgs = static_cast<double>(ceil_div(n, 16));

@@ -1515,6 +1515,92 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
   }
 }
 
+// The W-streaming kernel with a loop over K instead of K slices: for a W with many rows (enough column tiles to fill the
+// chip without splitting K) a workgroup of WAVES wavefronts owns 16 * WAVES columns of C over the whole of K and walks it
+// in segments of 256 elements through a ring of NSTG LDS stages, NSTG - 1 segments requested ahead; the sums stay in
+// registers, nothing is handed over.  A segment of a row is 512 bytes, so every 1 KiB load brings in two rows (a
+// wavefront its own 16 rows of W with 8 loads, and its share of the 16 * MT rows of A); layout, swizzle and fragment
+// order as in gemm_stream_kernel.  One barrier per segment: it makes the segment's A rows visible and says that
+// everybody has read the stage that the next request overwrites.
+template <int MT, int WAVES, int NSTG>
+__global__ void __launch_bounds__(64 * WAVES) gemm_stream_loop_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
+                                                                     GemmEpilogue ep, void* __restrict__ C, int64_t M, int64_t N,
+                                                                     int64_t K) {
+  constexpr int kCols = 16 * WAVES, kRowsA = 16 * MT, kSegK = 256, kRowLds = 2 * kSegK;
+  constexpr int kStage = (kCols + kRowsA) * kRowLds;
+  constexpr int kALoads = kRowsA / 2 / WAVES;  // 1 KiB loads (two rows each) per wavefront and segment
+  constexpr int kL = 8 + kALoads;
+  static_assert((kRowsA / 2) % WAVES == 0 && NSTG >= 2 && NSTG * kStage <= kLdsBytes && (NSTG - 1) * kL <= 63, "stages / LDS / vmcnt");
+  __shared__ __attribute__((aligned(1024))) char lds[NSTG * kStage];
+  const unsigned t = threadIdx.x, l = t & 63u;
+  const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * kCols;
+  const int64_t rows_w = N - n0 < kCols ? N - n0 : kCols;
+  const unsigned row_bytes = static_cast<unsigned>(K) * 2u;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, static_cast<unsigned>(M) * row_bytes);
+  const int nseg = static_cast<int>((K + kSegK - 1) / kSegK);
+  // lane l of load q of a 16-row group fills slot l & 31 of row 2 q + (l >> 5): it fetches chunk (l & 31) ^ f(row)
+  const unsigned lr = l >> 5;
+  auto request = [&](int seg, char* stage) {
+#pragma unroll
+    for (int i = 0; i < kALoads; ++i) {
+      const unsigned q = wv * kALoads + i, r = 2u * q + lr, c = (l & 31u) ^ stream_swizzle(r);
+      const int64_t k = static_cast<int64_t>(seg) * kSegK + c * 8;
+      const unsigned at = k < K ? r * row_bytes + static_cast<unsigned>(k) * 2u : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(stage + kCols * kRowLds + q * 1024), 16, at, 0, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const unsigned r = 2u * q + lr, c = (l & 31u) ^ stream_swizzle(r);
+      const int64_t k = static_cast<int64_t>(seg) * kSegK + c * 8;
+      const unsigned at = k < K ? (wv * 16u + r) * row_bytes + static_cast<unsigned>(k) * 2u : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(stage + wv * (16 * kRowLds) + q * 1024), 16, at, 0, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int p = 0; p < NSTG - 1; ++p)
+    if (p < nseg) request(p, lds + p * kStage);
+  f32x4v acc[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) acc[i] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  const unsigned i16 = l & 15u, g = l >> 4;
+  const unsigned x16 = ((((g & 1u) << 1) | (g >> 1)) ^ stream_swizzle(i16)) * 16u;
+  int cur = 0;  // stage of segment s
+  for (int s = 0; s < nseg; ++s) {
+    // segment s has landed; later ones (at most NSTG - 2 of those requested) may stay in flight
+    wait_whole_tiles<kL, NSTG - 2>(nseg - 1 - s);
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    const int into = cur == 0 ? NSTG - 1 : cur - 1;  // the stage of segment s - 1, read by everybody before this barrier
+    if (s + NSTG - 1 < nseg) request(s + NSTG - 1, lds + into * kStage);
+    DTAS_SCHED_FENCE();
+    const char* w_lane = lds + cur * kStage + (wv * 16u + i16) * kRowLds;
+    const char* a_lane = lds + cur * kStage + (kCols + i16) * kRowLds;
+#pragma unroll
+    for (int ks = 0; ks < kSegK / 32; ++ks) {
+      const unsigned at = x16 ^ (ks * 64u);
+      const f16x8 fw = *reinterpret_cast<const f16x8*>(w_lane + at);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(*reinterpret_cast<const f16x8*>(a_lane + i * 16 * kRowLds + at), fw, acc[i], 0, 0, 0);
+    }
+    DTAS_SCHED_FENCE();
+    cur = cur + 1 == NSTG ? 0 : cur + 1;
+  }
+  // result register v of lane l: row 4 * (l >> 4) + v, column l & 15 of a 16x16 block
+  const int64_t col = n0 + wv * 16u + i16;
+  if (col < N) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int64_t row = i * 16 + 4 * g + v;
+        if (row < M) finish(acc[i][v], ep, C, row, col, N);
+      }
+  }
+}
+
 // A few rows of A (M <= MV <= 4) against a W that is streamed once: R rows of W per wavefront, lane l
 // takes the 16-byte chunks l, l + 64, ... of each (a wavefront access is 1 KiB of one W row, non-temporal,
 // as in the GEMV kernel), multiplies each with the matching chunks of the MV rows of A (re-read per
@@ -1920,6 +2006,21 @@ int launch_stream(hipStream_t s, const half_t* A, const half_t* W, const GemmEpi
   return check_launch("gemm");
 }
 
+template <int MT, int WAVES, int NSTG>
+int launch_stream_loop(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = ceil_div(N, 16 * WAVES);
+  if (tiles > 0x7fffffff) return fail("gemm: too many workgroups");
+  hipLaunchKernelGGL((gemm_stream_loop_kernel<MT, WAVES, NSTG>), dim3(static_cast<unsigned>(tiles)), dim3(64 * WAVES), 0, s, A, W, ep, C, M, N, K);
+  return check_launch("gemm");
+}
+
+// the looping form of the W-streaming kernel (tile[2] == 256): rows of A x columns, and the stages it runs with
+inline int stream_loop_stages(int bm, int bn) {
+  if (bm == 16 && bn == 64) return 4;  // 160 KiB: one workgroup per CU
+  if (bm == 16 && bn == 16) return 4;  // 64 KiB: two one-wavefront workgroups per CU
+  return 0;
+}
+
 // the instantiated W-streaming shapes: rows of A x columns x K slice
 inline bool stream_shape_ok(int bm, int bn, int bk) {
   if ((bm != 16 && bm != 32 && bm != 64) || (bn != 64 && bn != 128) || (bk != 512 && bk != 1024)) return false;
@@ -2045,6 +2146,23 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
     la[6] = la[0];
     return 0;
   }
+  if (cfg.variant == DTAS_GEMM_STREAM && cfg.tile[2] == 256) {  // the looping form: the whole of K per workgroup
+    const int stages = stream_loop_stages(cfg.tile[0], cfg.tile[1]);
+    if (stages == 0)
+      return fail("gemm: the looping W-streaming kernel takes tiles 16x64x256 and 16x16x256, got %dx%dx%d", cfg.tile[0], cfg.tile[1],
+                  cfg.tile[2]);
+    if (M > cfg.tile[0]) return fail("gemm: a streaming tile of %d rows cannot hold M=%lld", cfg.tile[0], (long long)M);
+    if (cfg.block != 4 * cfg.tile[1]) return fail("gemm: the %d-column streaming tile uses %d threads, got %d", cfg.tile[1], 4 * cfg.tile[1], cfg.block);
+    if (K * 2 * cfg.tile[1] >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
+    const int64_t tn = ceil_div(N, cfg.tile[1]);
+    if (tn > 0x7fffffff) return fail("gemm: too many workgroups");
+    la[0] = tn;
+    la[3] = cfg.block;
+    la[4] = stages * (cfg.tile[0] + cfg.tile[1]) * 512;
+    la[5] = 1;
+    la[6] = tn;
+    return 0;
+  }
   if (cfg.variant == DTAS_GEMM_STREAM) {
     const int mt = cfg.tile[0] / 16, waves = cfg.tile[1] / 16, seg = cfg.tile[2] / 512;
     if (!stream_shape_ok(cfg.tile[0], cfg.tile[1], cfg.tile[2]))
@@ -2143,6 +2261,11 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
       case 80: hipLaunchKernelGGL(gemm_skinny_kernel<5>, grid, block, 0, s, a, w, b, c, M, N, K); break;
     }
     return check_launch("gemm");
+  }
+  if (cfg.variant == DTAS_GEMM_STREAM && cfg.tile[2] == 256) {
+    if (cfg.tile[0] == 16 && cfg.tile[1] == 64) return launch_stream_loop<1, 4, 4>(s, a, w, b, c, M, N, K);
+    if (cfg.tile[0] == 16 && cfg.tile[1] == 16) return launch_stream_loop<1, 1, 4>(s, a, w, b, c, M, N, K);
+    return fail("gemm: no looping W-streaming kernel for tile %dx%d", cfg.tile[0], cfg.tile[1]);
   }
   if (cfg.variant == DTAS_GEMM_STREAM) {
 #define DTAS_STREAM_CASE(BM_, BN_, BK_) \

@@ -121,6 +121,20 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         workgroups the tiles win again (libdtas: gemm_policy)."""
         return m_hi <= 16 and -(-N // 64) * -(-K // 1024) <= self.arch.num_sm
 
+    def prefers_stream_loop(self, m_hi: int, N: int, K: int) -> int:
+        """Columns per workgroup (16 or 64) of the looping W-streaming kernel where it leads, else 0: M <= 16, K <= 4096
+        and its workgroups fill one round of the chip -- two one-wavefront workgroups per CU for 4096 < N <= 8192, one
+        4-wavefront workgroup per CU for 8192 <= N <= 16384 (15.9 against 20.2 us at 8192 x 4096, 20.4 / 24.5 at
+        11008 x 4096; libdtas: gemm_policy)."""
+        if m_hi > 16 or K > 4096 or self.prefers_stream(m_hi, N, K):
+            return 0
+        cu = self.arch.num_sm
+        if cu < -(-N // 16) <= 2 * cu:
+            return 16
+        if cu // 2 <= -(-N // 64) <= cu:
+            return 64
+        return 0
+
     def prefers_skinny(self, m_hi: int, N: int, K: int) -> bool:
         """M <= 32: the W-streaming kernel (about 3.5 TB/s of W, slower as M grows) against the model's
         best MFMA candidate; call after preferred()."""
@@ -154,6 +168,17 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.micro_shape_k = 1, cols // 16, rows // 16, 1, kslice // 32
                 c.mfma_m, c.mfma_n, c.mfma_k = 16, 16, 32
                 stream.append(c)
+        loop: List[MFMAConfig] = []
+        if m_hi <= 16:
+            # its looping form (K slice 256 = the segment of the LDS ring; the whole of K per workgroup)
+            for cols in (64, 16):
+                c = MFMAConfig()
+                c.stream, c.block_threads = True, 4 * cols
+                c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.micro_shape_k = 1, cols // 16, 1, 1, 8
+                c.mfma_m, c.mfma_n, c.mfma_k = 16, 16, 32
+                loop.append(c)
+            lead = self.prefers_stream_loop(m_hi, N, K)
+            loop.sort(key=lambda c: c.tile_size_n != lead)
         if m_hi <= 64:
             for threads in (512, 256):
                 c = MFMAConfig()
@@ -194,4 +219,5 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         # the W-streaming kernel leads only where it beats the best MFMA candidate under the model
         out = (out + mfma) if self.prefers_skinny(m_hi, N, K) else (mfma[:1] + out + mfma[1:])
         out = (stream + out) if self.prefers_stream(m_hi, N, K) else (out[:1] + stream + out[1:])
+        out = (loop + out) if m_hi <= 16 and self.prefers_stream_loop(m_hi, N, K) else (out[:2] + loop + out[2:])
         return out[:topk]

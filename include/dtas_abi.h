@@ -106,7 +106,10 @@ enum dtas_variant {
   DTAS_GEMM_STREAM = 3    /* M <= tile[0] in {16, 32, 64}: W streamed once, 1 KiB of a row per access, through the LDS to
                              MFMA 16x16x32; a workgroup of tile[1] / 16 wavefronts owns tile[1] in {64, 128} columns and
                              tile[2] in {512, 1024} elements of K, the K slices are added up in the workspace;
-                             (tile[0] + tile[1]) * tile[2] * 2 bytes of LDS, block = 4 * tile[1] */
+                             (tile[0] + tile[1]) * tile[2] * 2 bytes of LDS, block = 4 * tile[1].
+                             tile[2] = 256 is the looping form for a W with many rows: tile = {16, 16 | 64, 256}, a
+                             workgroup owns its columns over the whole of K and walks it in segments of 256 through a
+                             ring of four LDS stages; no workspace */
 };
 
 /* One row of a call table: the launch-relevant part of the reference's *Config classes

@@ -214,6 +214,10 @@ def test_builtin_tables_name_a_launchable_kernel_for_every_bucket_and_shape():
                     # (split_k = 0, the 8-wavefront 256x256 tile only: the library splits just the tiles of a partly filled last round)
                     assert (c.split_k == 0 and tuple(c.tile[:2]) == (256, 256) and c.block == 512) or \
                         (1 <= c.split_k <= 4 and (c.split_k == 1 or -(-K // 64) // c.split_k >= 8)), (M, N, K, c.split_k)
+                elif c.variant == _lib.GEMM_STREAM and c.tile[2] == 256:
+                    # the looping form: one round of the chip, two one-wavefront workgroups or one of four wavefronts per CU
+                    assert M <= 16 and K <= 4096 and (list(c.tile[:2]), c.block) in (([16, 16], 64), ([16, 64], 256))
+                    assert (256 < info.launch_args[0] <= 512) if c.tile[1] == 16 else (128 <= info.launch_args[0] <= 256)
                 elif c.variant == _lib.GEMM_STREAM:
                     # at most one workgroup per CU, 64 columns x 1024 of K each
                     assert M <= 16 and list(c.tile) == [16, 64, 1024] and c.block == 256 and info.launch_args[0] <= 256

@@ -200,6 +200,61 @@ def test_gemm_every_streaming_tile(oracle, rows, cols, kslice, N, K):
         assert list(info.launch_args)[:5] == [-(-N // cols) * -(-K // kslice), 1, 1, 4 * cols, (rows + cols) * kslice * 2]
 
 
+@pytest.mark.parametrize("cols", [16, 64])
+@pytest.mark.parametrize("N,K", [(64, 64), (100, 520), (1000, 2560), (7680, 2560), (33, 40), (300, 256 * 9 + 8), (11008, 4096)])
+def test_gemm_looping_streaming_tiles(oracle, cols, N, K):
+    # the looping form (tile[2] = 256: the whole of K per workgroup through a ring of four LDS stages): fewer segments
+    # than stages, exactly as many, many, a ragged last one; ragged N and M; with and without bias
+    for M in (16, 13, 1):
+        a, w = _inputs(M, N, K, M + N + K + cols)
+        bias = np.random.default_rng(3).uniform(-1, 1, N).astype(np.float16) if M != 1 else None
+        out = Guarded((M, N), torch.float16)
+        c = cfg(variant=_lib.GEMM_STREAM, block=4 * cols, vec=8, unroll=1, tile=[16, cols, 256])
+        ops.gemm(dev(a), dev(w), None if bias is None else dev(bias), out.t, c)
+        _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
+        info = _lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c)
+        assert list(info.launch_args)[:5] == [-(-N // cols), 1, 1, 4 * cols, 4 * (16 + cols) * 512]
+
+
+def test_gemm_looping_streaming_tile_is_the_choice_for_many_rows_of_w_exact_and_refuses_what_it_cannot_hold(oracle):
+    # what cfg = NULL runs for M <= 16 against 4096 < N <= 16384 rows of W with K <= 4096
+    for N, K, tile, block in ((7680, 2560, [16, 16, 256], 64), (8192, 4096, [16, 16, 256], 64), (11008, 4096, [16, 64, 256], 256),
+                              (10240, 2560, [16, 64, 256], 256)):
+        got = _lib.select_bucket(_lib.OP_GEMM_F16, 16, N, K).config
+        assert (got.variant, list(got.tile), got.block) == (_lib.GEMM_STREAM, tile, block), (N, K)
+    for N, K in ((4096, 4096), (4096, 11008), (32000, 4096), (11008, 8192)):
+        got = _lib.select_bucket(_lib.OP_GEMM_F16, 16, N, K).config
+        assert not (got.variant == _lib.GEMM_STREAM and got.tile[2] == 256), (N, K)
+    assert _lib.select_bucket(_lib.OP_GEMM_F16, 17, 11008, 4096).config.variant == _lib.GEMM_MFMA
+    # small integers: every sum is exact in fp32 and fp16, whatever the order
+    rng = np.random.default_rng(7)
+    ai, wi = rng.integers(-2, 3, (13, 2048)).astype(np.float16), rng.integers(-2, 3, (200, 2048)).astype(np.float16)
+    for cols in (16, 64):
+        out = Guarded((13, 200), torch.float16)
+        ops.gemm(dev(ai), dev(wi), None, out.t, cfg(variant=_lib.GEMM_STREAM, block=4 * cols, vec=8, unroll=1, tile=[16, cols, 256]))
+        assert np.array_equal(out.check().astype(np.float64), ai.astype(np.float64) @ wi.astype(np.float64).T)
+    big = dev(np.zeros((17, 64), np.float16))
+    with pytest.raises(_lib.DtasError, match="cannot hold M=17"):
+        ops.gemm(big, dev(np.zeros((8, 64), np.float16)), None, torch.empty(17, 8, dtype=torch.float16, device="cuda"),
+                 cfg(variant=_lib.GEMM_STREAM, block=256, vec=8, unroll=1, tile=[16, 64, 256]))
+    for tile, block in (([32, 64, 256], 256), ([16, 32, 256], 128), ([16, 64, 256], 512)):
+        with pytest.raises(_lib.DtasError, match="streaming"):
+            _lib.describe_launch(_lib.OP_GEMM_F16, 8, 64, 64, cfg(variant=_lib.GEMM_STREAM, block=block, vec=8, unroll=1, tile=tile))
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3])
+@pytest.mark.parametrize("cols", [16, 64])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 7, 8), (16, 130, 1096), (13, 2560, 2560)])
+def test_gemm_fused_epilogues_looping_streaming_tile(oracle, kind, cols, M, N, K):
+    a, w, bias, r1, r2 = _fused_inputs(M, N, K, M + N + K + kind)
+    res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+    out = Guarded((M, N), torch.float32 if kind == 2 else torch.float16)
+    c = cfg(variant=_lib.GEMM_STREAM, block=4 * cols, vec=8, unroll=1, tile=[16, cols, 256])
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c, epilogue=kind, res1=res[0], res2=res[1])
+    want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+    _check_fused(out.check(), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+
+
 def test_gemm_streaming_tile_is_reproducible_exact_and_refuses_what_it_cannot_hold(oracle):
     M, N, K = 16, 4096, 4096
     a, w = _inputs(M, N, K, 5)
