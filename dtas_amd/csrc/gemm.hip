@@ -49,7 +49,8 @@
 // STREAM kernel (M <= 64; the built-in choice for M <= 16): W rows come in as 1 KiB direct-to-LDS
 //              loads, everything a workgroup needs requested at once; K slices meet in the workspace.
 //              With 8-bit weights (M <= 32) the bytes ride the same loads and are widened between
-//              the LDS and the MFMA.
+//              the LDS and the MFMA.  For a W with many rows (4096 < N <= 16384, K <= 4096) the looping
+//              form: a workgroup keeps its columns over the whole of K, walked through a ring of LDS stages.
 // ROWS kernel (M <= 4; the built-in choice for M = 2): W streamed in whole rows on the vector ALU.
 // Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles) and
 //              attn_pv_rows_kernel (P.V for a handful of query rows).
