@@ -161,6 +161,58 @@ __device__ __forceinline__ void finish(float acc, const GemmEpilogue& ep, void* 
   else static_cast<half_t*>(C)[row * N + col] = r;
 }
 
+// The 4 * MT sums a lane of the W-streaming kernels holds for column `col` (register v of block i: row i * 16 + 4 * g + v).
+// Bias and residuals are few and scattered (2 bytes per lane and row) and come from memory nobody has touched: they are
+// requested when the kernel starts, ahead of the operands, and wait in registers, instead of costing a round trip of
+// their own after the last MFMA (and one per row, behind the store before it, if they were read element by element).
+template <int MT>
+struct ColumnOperands {
+  half_t bias, r1[MT][4], r2[MT][4];  // as loaded: widening them here would make the wavefront wait for each load where it is issued
+};
+template <int MT>
+__device__ __forceinline__ void load_column_operands(ColumnOperands<MT>& o, const GemmEpilogue& ep, unsigned g, int64_t col, int64_t M,
+                                                     int64_t N) {
+  const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const bool use_r1 = add2 || ep.kind == kEpiScores;
+  const half_t zero = static_cast<half_t>(0.f);
+  o.bias = ep.bias && col < N ? ep.bias[col] : zero;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int64_t row = i * 16 + 4 * g + v;
+      const bool in = row < M && col < N;
+      o.r1[i][v] = use_r1 && in ? ep.res1[row * N + col] : zero;
+      o.r2[i][v] = add2 && in ? ep.res2[row * N + col] : zero;
+    }
+}
+// Called where the operands are known to have arrived (behind a wait for younger loads): the values must exist here,
+// so the compiler cannot move their loads down to their only use, behind the main loop and the hand-over.
+template <int MT>
+__device__ __forceinline__ void pin_column_operands(const ColumnOperands<MT>& o) {
+  asm volatile("" ::"v"(o.bias));
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+    asm volatile("" ::"v"(o.r1[i][0]), "v"(o.r1[i][1]), "v"(o.r1[i][2]), "v"(o.r1[i][3]), "v"(o.r2[i][0]), "v"(o.r2[i][1]), "v"(o.r2[i][2]),
+                 "v"(o.r2[i][3]));
+}
+template <int MT>
+__device__ __forceinline__ void finish_column(const f32x4v (&acc)[MT], const ColumnOperands<MT>& o, const GemmEpilogue& ep, void* C,
+                                              unsigned g, int64_t col, int64_t M, int64_t N) {
+  if (col >= N) return;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int64_t row = i * 16 + 4 * g + v;
+      if (row >= M) continue;
+      const half_t r = epilogue_value(round_h(acc[i][v]), ep, static_cast<float>(o.bias), static_cast<float>(o.r1[i][v]),
+                                      static_cast<float>(o.r2[i][v]));
+      if (ep.out_f32) static_cast<float*>(C)[row * N + col] = static_cast<float>(r);
+      else static_cast<half_t*>(C)[row * N + col] = r;
+    }
+}
+
 // Position of workgroup `wg` in a tile order in which each XCD gets a contiguous span:
 // the hardware deals consecutive workgroup ids round-robin over the 8 XCDs.
 __device__ __forceinline__ unsigned xcd_contiguous_id(unsigned wg, unsigned total) {
@@ -1365,6 +1417,8 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
     const int64_t k = (static_cast<int64_t>(z) * SEG + s) * 512 + c * 8;
     return k < K ? row * row_bytes + static_cast<unsigned>(k) * 2u : kOob;
   };
+  ColumnOperands<MT> colop;
+  load_column_operands<MT>(colop, ep, l >> 4, n0 + wv * 16u + (l & 15u), M, N);
   char* lds_a = lds + kWSlab;
 #pragma unroll
   for (int i = 0; i < kRowsA / WAVES; ++i) {
@@ -1409,6 +1463,7 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
   for (int i = 0; i < MT; ++i) acc[i] = f32x4v{0.f, 0.f, 0.f, 0.f};
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(kWLoads));  // this wavefront's A rows have landed
   __builtin_amdgcn_s_barrier();                       // ... and everybody's
+  pin_column_operands<MT>(colop);
   DTAS_SCHED_FENCE();
   // fragment reads: row l & 15 of a 16-row block, chunk 4 * ks + perm(l >> 4) -> slot (4 * ks) ^ x, x = perm ^ f(row)
   const unsigned i16 = l & 15u, g = l >> 4;
@@ -1504,16 +1559,7 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_kernel(const half_t* _
       }
     }
   }
-  const int64_t col = n0 + wv * 16u + i16;
-  if (col < N) {
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int64_t row = i * 16 + 4 * g + v;
-        if (row < M) finish(acc[i][v], ep, C, row, col, N);
-      }
-  }
+  finish_column<MT>(acc, colop, ep, C, g, n0 + wv * 16u + i16, M, N);
 }
 
 // The W-streaming kernel with a loop over K instead of K slices: for a W with many rows (enough column tiles to fill the
@@ -1541,6 +1587,8 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_loop_kernel(const half
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(A, static_cast<unsigned>(M) * row_bytes);
   const int nseg = static_cast<int>((K + kSegK - 1) / kSegK);
+  ColumnOperands<MT> colop;
+  load_column_operands<MT>(colop, ep, l >> 4, n0 + wv * 16u + (l & 15u), M, N);
   // lane l of load q of a 16-row group fills slot l & 31 of row 2 q + (l >> 5): it fetches chunk (l & 31) ^ f(row)
   const unsigned lr = l >> 5;
   auto request = [&](int seg, char* stage) {
@@ -1572,6 +1620,7 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_loop_kernel(const half
     // segment s has landed; later ones (at most NSTG - 2 of those requested) may stay in flight
     wait_whole_tiles<kL, NSTG - 2>(nseg - 1 - s);
     __builtin_amdgcn_s_barrier();
+    if (s == 0) pin_column_operands<MT>(colop);
     DTAS_SCHED_FENCE();
     const int into = cur == 0 ? NSTG - 1 : cur - 1;  // the stage of segment s - 1, read by everybody before this barrier
     if (s + NSTG - 1 < nseg) request(s + NSTG - 1, lds + into * kStage);
@@ -1590,16 +1639,7 @@ __global__ void __launch_bounds__(64 * WAVES) gemm_stream_loop_kernel(const half
     cur = cur + 1 == NSTG ? 0 : cur + 1;
   }
   // result register v of lane l: row 4 * (l >> 4) + v, column l & 15 of a 16x16 block
-  const int64_t col = n0 + wv * 16u + i16;
-  if (col < N) {
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int64_t row = i * 16 + 4 * g + v;
-        if (row < M) finish(acc[i][v], ep, C, row, col, N);
-      }
-  }
+  finish_column<MT>(acc, colop, ep, C, g, n0 + wv * 16u + i16, M, N);
 }
 
 // A few rows of A (M <= MV <= 4) against a W that is streamed once: R rows of W per wavefront, lane l
