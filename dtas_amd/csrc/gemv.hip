@@ -52,6 +52,21 @@ __device__ __forceinline__ void finish(float acc, const GemvEpilogue& ep, void* 
   else static_cast<half_t*>(y)[j] = t;
 }
 
+// The same with the operands already in registers (the split-K kernel requests them before it streams W: read at the
+// end, each would cost the launch a round trip to memory of its own).
+__device__ __forceinline__ void finish_with(float acc, int kind, bool has_bias, half_t bias, half_t r1, half_t r2, void* y, int64_t j) {
+  half_t t = static_cast<half_t>(acc);
+  if (has_bias) t = static_cast<half_t>(static_cast<float>(t) + static_cast<float>(bias));
+  if (kind == DTAS_EPI_BIAS_ADD2 || kind == DTAS_EPI_BIAS_ADD2_CAST_F32) {
+    t = static_cast<half_t>(static_cast<float>(r1) + static_cast<float>(t));
+    t = static_cast<half_t>(static_cast<float>(t) + static_cast<float>(r2));
+  } else if (kind == DTAS_EPI_BIAS_GELU) {
+    t = gelu_erf_f16_steps(t);
+  }
+  if (kind == DTAS_EPI_BIAS_ADD2_CAST_F32) static_cast<float*>(y)[j] = static_cast<float>(t);
+  else static_cast<half_t*>(y)[j] = t;
+}
+
 template <int R>
 __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restrict__ x, const half_t* __restrict__ W,
                                                           GemvEpilogue ep, void* __restrict__ y, int64_t N, int64_t K) {
@@ -69,6 +84,13 @@ __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restri
   float acc[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  // thread r < R stores row row0 + r: its bias and residual elements, requested now and kept as loaded
+  const bool stores = threadIdx.x < R && row0 + threadIdx.x < N;
+  const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const half_t zero = static_cast<half_t>(0.f);
+  const half_t e_bias = stores && ep.bias ? ep.bias[row0 + threadIdx.x] : zero;
+  const half_t e_r1 = stores && add2 ? ep.res1[row0 + threadIdx.x] : zero;
+  const half_t e_r2 = stores && add2 ? ep.res2[row0 + threadIdx.x] : zero;
 
 #pragma unroll 2
   for (int64_t i = threadIdx.x; i < nvec; i += blockDim.x) {
@@ -79,6 +101,7 @@ __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restri
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = dot8(xr, wr[r], acc[r]);
   }
+  asm volatile("" ::"v"(e_bias), "v"(e_r1), "v"(e_r2));  // (they exist by now: their loads stay where they were written)
 
   const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
 #pragma unroll
@@ -90,7 +113,7 @@ __global__ void __launch_bounds__(512) gemv_splitk_kernel(const half_t* __restri
   if (threadIdx.x < R && row0 + threadIdx.x < N) {
     float s = 0.f;
     for (int w = 0; w < nwaves; ++w) s += part[w][threadIdx.x];
-    finish(s, ep, y, row0 + threadIdx.x);
+    finish_with(s, ep.kind, ep.bias != nullptr, e_bias, e_r1, e_r2, y, row0 + threadIdx.x);
   }
 }
 
