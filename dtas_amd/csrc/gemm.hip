@@ -112,6 +112,8 @@ struct GemmEpilogue {
   const half_t* wscale;   // 8-bit W: the fp16 scales [N][K/32]
   int64_t lda;            // k-major W only (P.V): row stride of A in elements when its rows are padded; 0 = K
   unsigned tiles_unsplit; // one problem only: tiles [0, tiles_unsplit) are computed whole, only the rest is split over nsplit workgroups
+  unsigned k_tail;        // k-major W only (P.V): A's rows and W hold k_tail (< 8) more k than K, which the MFMA loop leaves out and
+                          // the epilogue adds (A's rows are then fetched at whatever alignment lda gives them)
 };
 
 // Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):
@@ -899,6 +901,34 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // therefore moved with device-scope accesses (they pass the L2), ordered by explicit waits for the
   // store count plus the barriers, rather than with device-scope fences, which write back and
   // invalidate a whole L2 on every use (measured: that made a two-way split slower than no split).
+  if constexpr (WT) {
+    // the last k_tail k: 16-byte pieces of A's rows end at K (a piece across the end of a row would bring in the next
+    // row's elements), so these few products are added here, element by element, in fp32
+    if (ep.k_tail > 0 && z == 0) {
+      const int64_t lda_t = ep.lda ? ep.lda : K;
+      for (unsigned e = 0; e < ep.k_tail; ++e) {
+        float pa[MT];
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const int64_t row = m0 + wm * WTM + i * 32 + (l & 31u);
+          pa[i] = row < M ? static_cast<float>(A[row * lda_t + K + e]) : 0.f;
+        }
+        const half_t* vrow = W + (K + e) * N;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int64_t col = n0 + wn * WTN + j * 32 + 8 * g + 4 * (l >> 5);
+            if (col >= N) continue;  // (N % 8 == 0: four columns are all-in or all-out)
+            const f16x4 vv = *reinterpret_cast<const f16x4*>(vrow + col);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+              for (int c = 0; c < 4; ++c) acc[i][j][g * 4 + c] += pa[i] * static_cast<float>(vv[c]);
+          }
+      }
+    }
+  }
   if (my_split > 1) {
     // (the flag lives in the operand stages, free by now: a second LDS object would make the
     // compiler order every fragment read behind the outstanding direct-to-LDS loads)
@@ -1733,32 +1763,6 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(const half_t* __restrict
   }
 }
 
-// P.V with a key count that is not a multiple of 8 (or a P that is not 16-byte aligned): the rows of P are
-// copied once into rows of m_pad = 8 * slots elements, zero-filled, which the direct-to-LDS loads can fetch.
-// Whole 8-element pieces are read with one access at the row's alignment, the piece across the end of a row
-// element by element.
-typedef u32x4 __attribute__((aligned(2))) u32x4_a2;
-__global__ void __launch_bounds__(256) pad_rows_kernel(const half_t* __restrict__ P, u32x4* __restrict__ out, int64_t rows,
-                                                       int64_t m, int64_t slots) {
-  const int64_t total = rows * slots;
-  for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
-       t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int64_t row = t / slots, at = (t % slots) * 8, left = m - at;
-    const half_t* p = P + row * m + at;
-    u32x4 v;
-    if (left >= 8) {
-      v = *reinterpret_cast<const u32x4_a2*>(p);
-    } else {
-      unsigned short h[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) h[e] = e < left ? reinterpret_cast<const unsigned short*>(p)[e] : 0u;
-      v = u32x4{h[0] | (static_cast<unsigned>(h[1]) << 16), h[2] | (static_cast<unsigned>(h[3]) << 16),
-                h[4] | (static_cast<unsigned>(h[5]) << 16), h[6] | (static_cast<unsigned>(h[7]) << 16)};
-    }
-    out[t] = v;
-  }
-}
-
 // Any K and alignment: one thread per element of C.  blockIdx.y = problem of a batched launch;
 // w_kmajor: W is [K][N] instead of [N][K]; ep.wscale set: W is 8-bit with group scales.
 __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W,
@@ -1851,8 +1855,7 @@ __global__ void __launch_bounds__(256) attn_pv_rows_kernel(const half_t* __restr
 // Library-owned scratch memory, one set per (device, stream):
 //  * the split-K workspace: nsplit fp32 partial tiles per shared output tile and one arrival counter per tile
 //    (zero between launches: the last arriver of a tile re-arms it);
-//  * the operand buffer: the fp16 copy of an 8-bit weight matrix (dtas_gemm_q8_f16_fused's two-pass route) or the
-//    padded copy of P (dtas_attn_pv_f16 with a key count that is not a multiple of 8).
+//  * the operand buffer: the fp16 copy of an 8-bit weight matrix (dtas_gemm_q8_f16_fused's two-pass route).
 // Allocated on first use by a stream and grown on demand -- the only allocations in the library.  Launches on one
 // stream are ordered by it and share its set; launches on different streams use different sets, so they may overlap.
 // g_ws_mutex is held from the lookup until the launches that use the set are enqueued: a set is never grown (freed
@@ -2506,18 +2509,13 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   half_t* c = static_cast<half_t*>(out);
   const int b = static_cast<int>(heads);
   GemmEpilogue ep = {nullptr, nullptr, nullptr, DTAS_EPI_BIAS, 0, 1.f, n * m, m * d, n * d, 0};
-  // rows of P that the 16-byte loads cannot fetch where they lie: a padded copy in the library's buffer, as many
-  // heads at a time as the buffer may hold
-  const int64_t m_pad = (m + 7) / 8 * 8;
-  int64_t pad_heads = 0;  // heads per padded launch; 0 = P is used where it lies
+  // A key count that is not a multiple of 8 (or a P that is not 16-byte aligned): the direct-to-LDS loads fetch the
+  // 16-byte pieces of P's rows at the rows' own 2-byte alignment, the MFMA loop covers the whole pieces (m_main keys)
+  // and the epilogue adds the last m % 8
+  int64_t m_main = m;
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_MFMA && !p_vec) {
-    const int64_t per_head = n * m_pad * 2;
-    pad_heads = static_cast<int64_t>(kMaxSplitWsBytes) / per_head;
-    if (pad_heads > heads) pad_heads = heads;
-    if (!aligned(P, 2) || pad_heads == 0) {
-      cfg.vec = 1;  // (the element-access kernel: correct, slow)
-      pad_heads = 0;
-    }
+    m_main = m - m % 8;
+    if (!aligned(P, 2) || m_main == 0) cfg.vec = 1;  // (the element-access kernel: correct, slow)
   }
   if (cfg.vec == 1) {
     int64_t grid = ceil_div(n * d, 256);
@@ -2550,34 +2548,16 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   if (describe_gemm(n, d, m, cfg, la) != 0) return -1;
   const int bm = cfg.tile[0], bn = cfg.tile[1];
   const bool three = cfg.unroll == 3;
-  // `hb` heads from P `pa` (row stride in ep), V `pw`, into `po`
-  auto launch = [&](const half_t* pa, const half_t* pw, void* po, int hb) -> int {
-    if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
-    if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
-    if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
-    if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
-    if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
-    if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
-    if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, pa, pw, ep, po, n, d, m, sk, hb);
-    return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
-  };
-  if (pad_heads == 0) return launch(a, w, out, b);
-  void* buf = nullptr;
-  std::lock_guard<std::recursive_mutex> ws_lock(g_ws_mutex);  // until every launch that uses the buffer is enqueued
-  if (operand_workspace(s, static_cast<size_t>(pad_heads) * n * m_pad * 2, &buf) != 0) return -1;
-  ep.stride_a = n * m_pad;
-  ep.lda = m_pad;
-  for (int64_t h0 = 0; h0 < heads; h0 += pad_heads) {
-    const int64_t hb = heads - h0 < pad_heads ? heads - h0 : pad_heads;
-    const int64_t items = hb * n * (m_pad / 8);
-    int64_t grid = ceil_div(items, 256);
-    grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
-    hipLaunchKernelGGL(pad_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, a + h0 * n * m, static_cast<u32x4*>(buf), hb * n, m,
-                       m_pad / 8);
-    if (check_launch("attn_pv") != 0) return -1;
-    if (launch(static_cast<const half_t*>(buf), w + h0 * m * d, c + h0 * n * d, static_cast<int>(hb)) != 0) return -1;
-  }
-  return 0;
+  ep.lda = m;
+  ep.k_tail = static_cast<unsigned>(m - m_main);
+  if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+  if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+  if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
+  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+  return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
 }
 
 extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias, const void* res1,

@@ -30,8 +30,7 @@
  *    share a stream.  At most 16 streams per device hold one (the one used longest ago is released
  *    first, which waits for the device).  A cfg with split_k = 1 uses none; dtas_gemm_f16_static
  *    never allocates.  dtas_gemm_q8_f16_fused keeps a second buffer of that kind
- *    (an fp16 copy of the weights it was given) under the same rules, and dtas_attn_pv_f16 uses that
- *    buffer for a padded copy of P when m is not a multiple of 8;
+ *    (an fp16 copy of the weights it was given) under the same rules;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the
  *    reference's call_table holds); NULL = use the library's built-in bucket table; either way a
  *    128-bit variant steps down to its element-access kernel for extents or pointers that do not
@@ -307,7 +306,8 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
  * (n, d, m) problem with tile {64|128, 64|128, 64} and two stages, or {128|256, 128, 64} and three (split_k > 1:
  * the workgroups of a (head, tile) split m and meet in the split-K workspace), or a DTAS_GEMM_SKINNY row
  * {block 256, tile {1|2|4|8, 8}} for the kernel that serves a handful of rows (decoding).  With m % 8 != 0
- * or a P off a 16-byte boundary the rows of P are first copied, padded, into the library's operand buffer;
+ * or a P off a 16-byte boundary the MFMA kernels read the rows of P where they lie (16-byte pieces at 2-byte
+ * alignment; the last m % 8 keys are added in the epilogue, in fp32, before the one rounding);
  * d % 8 != 0 or a V off 16 bytes fall back to the element-access kernel; m == 0 writes zeros. */
 int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t heads, int64_t n, int64_t m,
                      int64_t d, const dtas_config* cfg, void* stream);

@@ -193,7 +193,7 @@ def test_pv_selector_rows_are_exact_and_edge_cases(oracle):
 @pytest.mark.parametrize("n,m", [(13, 1025), (64, 77), (130, 1027), (300, 1028), (257, 513), (1024, 1032), (515, 7)])
 def test_scores_and_pv_with_key_counts_off_the_vector_width(oracle, n, m):
     # rows of m floats / halves start anywhere: the scores keep their vector stores (at the rows' alignment), P.V
-    # pads the rows of P into the library's buffer and keeps the MFMA kernel
+    # fetches the 16-byte pieces of P's rows where they lie and adds the last m % 8 keys in its epilogue
     heads, d = 4, 80
     q, k, mask = _inputs(heads, n, m, d, n + m)
     out = Guarded((heads, n, m), torch.float32)
@@ -209,6 +209,22 @@ def test_scores_and_pv_with_key_counts_off_the_vector_width(oracle, n, m):
         o = Guarded((heads, n, d), torch.float16)
         ops.attn_pv(dev(p), dev(v), o.t, c)
         _check_pv(o.check(), p, v, oracle)
+
+
+@pytest.mark.parametrize("n,m", [(70, 1025), (130, 71), (33, 15)])
+def test_pv_row_is_untouched_by_its_neighbours_with_key_counts_off_the_vector_width(oracle, n, m):
+    # the 16-byte piece that would straddle the end of a row of P is never fetched: a row of Inf next to a finite row
+    # leaves the finite row's result as it is (and exact, on small integers)
+    heads, d = 3, 80
+    rng = np.random.default_rng(n + m)
+    p = rng.integers(0, 3, size=(heads, n, m)).astype(np.float16)
+    v = rng.integers(-3, 4, size=(heads, m, d)).astype(np.float16)
+    want = np.einsum("hnm,hmd->hnd", p.astype(np.float64), v.astype(np.float64))
+    p[:, 1::2, :] = np.inf
+    o = Guarded((heads, n, d), torch.float16)
+    ops.attn_pv(dev(p), dev(v), o.t)
+    got = o.check()
+    assert np.array_equal(got[:, 0::2].astype(np.float64), want[:, 0::2])
 
 
 def test_pv_with_a_p_that_is_not_16_byte_aligned(oracle):
