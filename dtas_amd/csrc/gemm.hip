@@ -1149,8 +1149,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 // off the CU.  Here a workgroup walks tiles (stride = grid): it requests the whole Q and K tiles and
 // its part of the mask at once, multiplies, stages the result through the LDS and issues the stores;
 // the next tile's loads are then in flight together with those stores.  Tiles are numbered as the
-// batched launches of gemm_mfma_kernel number their workgroups (an XCD keeps one span of tiles when
-// `pinned`, so its part of the mask stays in its L2); operand layout in the LDS as there.
+// batched launches of gemm_mfma_kernel number their workgroups; with `pinned` an XCD keeps one span of
+// tiles (spans differ by at most one tile) and walks the heads, so its part of the mask stays in its L2.
+// Operand layout in the LDS as there.
 template <int BM, int BN>
 __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kmat,
                                                           const half_t* __restrict__ mask, float* __restrict__ out,
@@ -1182,12 +1183,16 @@ __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restri
   const bool stream_out = m % 16 == 0 && (reinterpret_cast<uintptr_t>(out) & 63u) == 0;  // (then every access is 16-byte aligned)
 
   const unsigned per_batch = tiles_m * tiles_n, total = per_batch * heads;
-  for (unsigned tix = blockIdx.x; tix < total; tix += gridDim.x) {
+  const unsigned span_base = per_batch / kNumXCD, span_rem = per_batch % kNumXCD;
+  const unsigned walk_end = pinned ? kNumXCD * heads * (span_base + (span_rem ? 1u : 0u)) : total;
+  for (unsigned tix = blockIdx.x; tix < walk_end; tix += gridDim.x) {
     unsigned batch, pid;
-    if (pinned && per_batch % kNumXCD == 0) {
-      const unsigned span = per_batch / kNumXCD, xcd = tix % kNumXCD, local = tix / kNumXCD;
+    if (pinned) {
+      const unsigned xcd = tix % kNumXCD, local = tix / kNumXCD;
+      const unsigned span = span_base + (xcd < span_rem ? 1u : 0u), first = xcd * span_base + (xcd < span_rem ? xcd : span_rem);
+      if (local >= span * heads) continue;  // (the shorter spans end earlier; uniform over the workgroup)
       batch = __builtin_amdgcn_readfirstlane(local / span);
-      pid = __builtin_amdgcn_readfirstlane(xcd * span + local % span);
+      pid = __builtin_amdgcn_readfirstlane(first + local % span);
     } else {
       const unsigned gid = xcd_contiguous_id(tix, total);
       batch = __builtin_amdgcn_readfirstlane(gid / per_batch);
@@ -2379,7 +2384,12 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   const bool small = n <= 64 || total < kNumCU;
   if (!user && d <= 2 * kBK && !small) {
     if (total > 0x7fffffff) return fail("attn_scores: too many tiles");
-    const int64_t grid = total < 3 * kNumCU ? total : 3 * kNumCU;
+    // Rows that are not whole 64-byte sectors (m % 16 != 0): neighbouring tiles each write part of the sector on their
+    // common boundary, and the parts only meet in the L2 if they are written close together -- one workgroup per
+    // tile, started in tile order, keeps them closer than workgroups that walk (n = m = 4097: 0.79 against 1.05 ms,
+    // 3001: 0.43 / 0.53; whole sectors: walking is ahead, 122 against 135 us at 2048)
+    const bool whole_sectors = m % 16 == 0 && aligned(out, 64);
+    const int64_t grid = !whole_sectors || total < 3 * kNumCU ? total : 3 * kNumCU;
     hipLaunchKernelGGL((attn_scores_kernel<128, 64>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const half_t*>(Q), static_cast<const half_t*>(Kmat), static_cast<const half_t*>(mask),
                        static_cast<float*>(out), n, m, d, static_cast<float>(static_cast<half_t>(scale)), tm, tn,
