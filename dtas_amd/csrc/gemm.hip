@@ -2480,11 +2480,11 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       // a handful of rows (decoding, short continuations): the row kernel (two rows per workgroup, four when the
       // keys are many: ~4.5 + 0.7 n m / 1000 us and ~6 + 0.4 n m / 1000 us, measured at n = 2 .. 12 against 512 ..
       // 4096 keys) unless the 64-row MFMA tiles with their keys split come out ahead (from ~8 rows against 4096
-      // keys, ~12 against 512: 15 us against 25 at n = 8, m = 4096); P's rows must be fetchable in 16-byte pieces
+      // keys, ~12 against 512: 15 us against 25 at n = 8, m = 4096)
       const double nm = 1e-3 * static_cast<double>(n) * static_cast<double>(m);
       const double r2 = 4.5 + 0.7 * nm, r4 = n >= 4 ? 6.0 + 0.4 * nm : 1e30;
       double mfma_us = 1e30;
-      if (n >= 2 && p_vec) {
+      if (n >= 2 && (p_vec || (aligned(P, 2) && m >= 8))) {  // (any key count: P is read where it lies)
         key_split(heads, 4 * kNumCU, ktiles, &mfma_us);
         mfma_us += 1.5;
       }
