@@ -906,26 +906,41 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // row's elements), so these few products are added here, element by element, in fp32
     if (ep.k_tail > 0 && z == 0) {
       const int64_t lda_t = ep.lda ? ep.lda : K;
-      for (unsigned e = 0; e < ep.k_tail; ++e) {
-        float pa[MT];
+      // kTB k at a time (four; two on the small tiles, whose register count decides how many workgroups a CU holds), every
+      // element of A and piece of W requested before the first is used: one round trip to memory per kTB k instead of one per k
+      constexpr int kTB = MT * NT >= 4 ? 4 : 2;
+      for (unsigned e0 = 0; e0 < ep.k_tail; e0 += kTB) {
+        half_t pa[kTB][MT];
+        f16x4 vv[kTB][NT][4];
+        const half_t hz = static_cast<half_t>(0.f);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          const int64_t row = m0 + wm * WTM + i * 32 + (l & 31u);
-          pa[i] = row < M ? static_cast<float>(A[row * lda_t + K + e]) : 0.f;
-        }
-        const half_t* vrow = W + (K + e) * N;
+        for (int e = 0; e < kTB; ++e) {
+          const bool k_in = e0 + e < ep.k_tail;
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int64_t col = n0 + wn * WTN + j * 32 + 8 * g + 4 * (l >> 5);
-            if (col >= N) continue;  // (N % 8 == 0: four columns are all-in or all-out)
-            const f16x4 vv = *reinterpret_cast<const f16x4*>(vrow + col);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-              for (int c = 0; c < 4; ++c) acc[i][j][g * 4 + c] += pa[i] * static_cast<float>(vv[c]);
+          for (int i = 0; i < MT; ++i) {
+            const int64_t row = m0 + wm * WTM + i * 32 + (l & 31u);
+            pa[e][i] = k_in && row < M ? A[row * lda_t + K + e0 + e] : hz;
           }
+          const half_t* vrow = W + (K + e0 + e) * N;
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const int64_t col = n0 + wn * WTN + j * 32 + 8 * g + 4 * (l >> 5);
+              const f16x4 none = {hz, hz, hz, hz};
+              vv[e][j][g] = k_in && col < N ? *reinterpret_cast<const f16x4*>(vrow + col) : none;  // (N % 8 == 0: four columns are all-in or all-out)
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < kTB; ++e)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+              for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[i][j][g * 4 + c] += static_cast<float>(pa[e][i]) * static_cast<float>(vv[e][j][g][c]);
       }
     }
   }
@@ -1857,6 +1872,65 @@ __global__ void __launch_bounds__(256) attn_pv_rows_kernel(const half_t* __restr
   }
 }
 
+// P.V for one query row per workgroup, the whole of V's head read in one sweep (decoding: n = 1, a few heads' worth of
+// workgroups on the chip).  A head's V is m rows of d fp16 = d / 8 16-byte pieces each, contiguous in memory: thread t of
+// 1024 takes piece t % (d / 8) of the rows t / (d / 8), + rows-per-pass, ... -- consecutive threads read consecutive
+// 16 bytes, a wavefront 1 KiB, eight passes in flight -- and multiplies each piece with its row's P.  The 8 sums of a
+// thread are those of its 8 columns; threads with the same piece index meet in the LDS and are added in thread order.
+__global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* __restrict__ P, const half_t* __restrict__ V,
+                                                                half_t* __restrict__ out, int64_t n, int64_t m, int64_t d) {
+  __shared__ float red[1024][8];
+  const unsigned chunks = static_cast<unsigned>(d / 8), per_pass = 1024u / chunks, t = threadIdx.x;
+  const int64_t h = blockIdx.x, r = blockIdx.y;
+  const half_t* p = P + (h * n + r) * m;
+  const u32x4* v = reinterpret_cast<const u32x4*>(V + h * m * d);
+  const bool active = t < per_pass * chunks;
+  const unsigned row0 = t / chunks;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  if (active) {
+    constexpr int kU = 8;
+    for (int64_t k0 = row0; k0 < m; k0 += static_cast<int64_t>(kU) * per_pass) {
+      u32x4 vraw[kU];
+      half_t pk[kU];
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int64_t k = k0 + static_cast<int64_t>(u) * per_pass;
+        // (piece index of thread t in pass u: t + u * per_pass * chunks -- the passes continue where the last thread stopped)
+        // (one row: V is read this once and streamed past the caches; more rows: their workgroups share it)
+        vraw[u] = k >= m ? zero : n == 1 ? load_stream(v + k * chunks + (t - row0 * chunks)) : v[k * chunks + (t - row0 * chunks)];
+        pk[u] = k < m ? p[k] : static_cast<half_t>(0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const f16x8 vv = __builtin_bit_cast(f16x8, vraw[u]);
+        const float pf = static_cast<float>(pk[u]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += pf * static_cast<float>(vv[e]);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[t][e] = active ? acc[e] : 0.f;
+  __syncthreads();
+  // column j of the row: piece j / 8, element j % 8, summed over the per_pass threads that hold that piece
+  if (t < chunks * 8u) {
+    const unsigned c = t >> 3, e = t & 7u;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    unsigned q = 0;
+    for (; q + 3 < per_pass; q += 4) {
+      s0 += red[(q + 0) * chunks + c][e];
+      s1 += red[(q + 1) * chunks + c][e];
+      s2 += red[(q + 2) * chunks + c][e];
+      s3 += red[(q + 3) * chunks + c][e];
+    }
+    for (; q < per_pass; ++q) s0 += red[q * chunks + c][e];
+    out[(h * n + r) * d + t] = static_cast<half_t>((s0 + s1) + (s2 + s3));
+  }
+}
+
 // Library-owned scratch memory, one set per (device, stream):
 //  * the split-K workspace: nsplit fp32 partial tiles per shared output tile and one arrival counter per tile
 //    (zero between launches: the last arriver of a tile re-arms it);
@@ -2484,12 +2558,25 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       const double nm = 1e-3 * static_cast<double>(n) * static_cast<double>(m);
       const double r2 = 4.5 + 0.7 * nm, r4 = n >= 4 ? 6.0 + 0.4 * nm : 1e30;
       double mfma_us = 1e30;
-      if (n >= 2 && (p_vec || (aligned(P, 2) && m >= 8))) {  // (any key count: P is read where it lies)
+      const bool mfma_ok = n >= 2 && (p_vec || (aligned(P, 2) && m >= 8));  // (any key count: P is read where it lies)
+      if (mfma_ok) {
         key_split(heads, 4 * kNumCU, ktiles, &mfma_us);
-        mfma_us += 1.5;
+        mfma_us = mfma_us + 1.5 < 5.5 ? 5.5 : mfma_us + 1.5;  // (no launch of the tiles takes less: 2 rows against 77 keys 7.5 us, the row kernel 4.6)
       }
-      rows = mfma_us >= (r2 < r4 ? r2 : r4);
-      if (rows) cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : r4 < r2 ? 4 : 2, 8, 0}, 1, 0};
+      // 3 .. 8 rows, one workgroup per (head, row) while these fit the chip at once: a head's V in one contiguous sweep
+      // per row (measured with V from memory, 32 heads of 80: 4 rows against 1024 / 2048 / 4096 keys 7.1 / 9.8 / 21.5 us
+      // where the row kernel takes 8.0 / 14.2 / 33.4; 8 rows 7.2 / 9.9 / 21.1 where the choices below take 12.4 / 16.7 / 19.4)
+      // -- up to ~3000 keys; beyond, the key-split MFMA tiles lead.  One and two rows: the row kernel (7.1 against 9.8
+      // us at 2048 keys: 32 workgroups are too few to pull V in)
+      if (n >= 3 && n <= 8 && heads * n <= kNumCU && d / 8 <= 128 && (m < 3072 || !mfma_ok)) {
+        rows = true;
+        cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, 0}, 1, 0};
+      } else if (n >= 2 && n <= 8 && m >= 3072 && heads * n <= kNumCU && mfma_ok) {
+        rows = false;  // (4 rows against 4096 / 8192 keys with V from memory: the row kernel 33 / 61 us, one sweep per row 22 / 39, the tiles 19 / 28)
+      } else {
+        rows = mfma_us >= (r2 < r4 ? r2 : r4);
+        if (rows) cfg = dtas_config{DTAS_GEMM_SKINNY, 256, 8, 1, {n <= 1 ? 1 : r4 < r2 ? 4 : 2, 8, 0}, 1, 0};
+      }
     }
     if (!rows) {
       // what this op moves is P (2*n*m bytes per head).  Measured over n = m = 128 .. 4096 with 32 heads of 80:
@@ -2534,6 +2621,14 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     return check_launch("attn_pv");
   }
   if (cfg.vec != 8) return fail("attn_pv: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+  if (cfg.variant == DTAS_GEMM_SKINNY && cfg.block == 1024) {  // one row per workgroup, V's head in one sweep
+    if (cfg.tile[0] != 1 || cfg.tile[1] != 8) return fail("attn_pv: the whole-row kernel takes one row per workgroup and 8-column pieces");
+    if (d / 8 > 128) return fail("attn_pv: the whole-row kernel holds head dimensions up to 1024, got %lld", (long long)d);
+    if (cfg.split_k > 1) return fail("attn_pv: the row kernels do not split K");
+    if (n > 65535) return fail("attn_pv: too many workgroups for the row kernel");
+    hipLaunchKernelGGL(attn_pv_whole_row_kernel, dim3(static_cast<unsigned>(heads), static_cast<unsigned>(n)), dim3(1024), 0, s, a, w, c, n, m, d);
+    return check_launch("attn_pv");
+  }
   if (cfg.variant == DTAS_GEMM_SKINNY) {
     const int R = cfg.tile[0];
     if (cfg.block != 256 || cfg.tile[1] != 8) return fail("attn_pv: the row kernel uses 256 threads and 8-column pieces");

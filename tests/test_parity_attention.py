@@ -153,11 +153,29 @@ def test_pv_row_kernel(oracle, rows, heads, n, m, d):
     _check_pv(out.check(), p, v, oracle)
 
 
-@pytest.mark.parametrize("n", [2, 4, 5, 8, 12])
-@pytest.mark.parametrize("m", [512, 1024, 4096, 4097])
+@pytest.mark.parametrize("heads,n,m,d", [(32, 1, 515, 80), (32, 4, 2048, 80), (3, 3, 64, 8), (2, 8, 1000, 128), (1, 5, 1, 16), (2, 2, 77, 136),
+                                         (2, 3, 9000, 64), (1, 7, 300, 1024)])
+def test_pv_whole_row_kernel(oracle, heads, n, m, d):
+    # one workgroup of 1024 threads per (head, query row): the head's V read as one contiguous run of 16-byte pieces,
+    # d / 8 of them per key (1 .. 128: every thread count per key, idle threads at the end of the workgroup included)
+    p, v = _pv_inputs(heads, n, m, d, heads + n + m + d)
+    out = Guarded((heads, n, d), torch.float16)
+    ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[1, 8, 0]))
+    _check_pv(out.check(), p, v, oracle)
+    rng = np.random.default_rng(m)
+    pi = rng.integers(0, 3, size=(heads, n, m)).astype(np.float16)
+    vi = rng.integers(-3, 4, size=(heads, m, d)).astype(np.float16)
+    ops.attn_pv(dev(pi), dev(vi), out.t, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[1, 8, 0]))
+    assert np.array_equal(out.check().astype(np.float64), np.einsum("hnm,hmd->hnd", pi.astype(np.float64), vi.astype(np.float64)))
+    with pytest.raises(_lib.DtasError):
+        ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[2, 8, 0]))
+
+
+@pytest.mark.parametrize("n", [2, 3, 4, 5, 8, 12])
+@pytest.mark.parametrize("m", [77, 512, 1024, 4096, 4097])
 def test_pv_few_rows_builtin_choice(oracle, n, m):
-    # 2 .. 12 query rows: two- or four-row workgroups of the row kernel, or 64-row MFMA tiles with the keys split
-    # (m = 4097: P's rows are not fetchable in 16-byte pieces, which keeps the row kernel)
+    # 2 .. 12 query rows: two- or four-row workgroups of the row kernel, one workgroup per row sweeping the head's V
+    # (3 .. 8 rows, up to ~3000 keys), or 64-row MFMA tiles with the keys split (any key count: P is read where it lies)
     p, v = _pv_inputs(32, n, m, 80, n + m)
     out = Guarded((32, n, 80), torch.float16)
     ops.attn_pv(dev(p), dev(v), out.t)
