@@ -1878,12 +1878,15 @@ __global__ void __launch_bounds__(256) attn_pv_rows_kernel(const half_t* __restr
 // 16 bytes, a wavefront 1 KiB, eight passes in flight -- and multiplies each piece with its row's P.  The 8 sums of a
 // thread are those of its 8 columns; threads with the same piece index meet in the LDS and are added in thread order.
 __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* __restrict__ P, const half_t* __restrict__ V,
-                                                                half_t* __restrict__ out, int64_t n, int64_t m, int64_t d) {
+                                                                half_t* __restrict__ out, int64_t n, int64_t m, int64_t d, unsigned cols) {
   __shared__ float red[1024][8];
-  const unsigned chunks = static_cast<unsigned>(d / 8), per_pass = 1024u / chunks, t = threadIdx.x;
-  const int64_t h = blockIdx.x, r = blockIdx.y;
+  // (cols < d: the workgroups of a (head, row) share the pieces of a key, cols / 8 consecutive ones each)
+  const unsigned row_chunks = static_cast<unsigned>(d / 8), chunks = cols / 8, groups = row_chunks / chunks;
+  const unsigned per_pass = blockDim.x / chunks, t = threadIdx.x;
+  const int64_t h = blockIdx.x / groups, r = blockIdx.y;
+  const unsigned first = (blockIdx.x % groups) * chunks;
   const half_t* p = P + (h * n + r) * m;
-  const u32x4* v = reinterpret_cast<const u32x4*>(V + h * m * d);
+  const u32x4* v = reinterpret_cast<const u32x4*>(V + h * m * d) + first;
   const bool active = t < per_pass * chunks;
   const unsigned row0 = t / chunks;
   float acc[8];
@@ -1900,7 +1903,7 @@ __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* _
         const int64_t k = k0 + static_cast<int64_t>(u) * per_pass;
         // (piece index of thread t in pass u: t + u * per_pass * chunks -- the passes continue where the last thread stopped)
         // (one row: V is read this once and streamed past the caches; more rows: their workgroups share it)
-        vraw[u] = k >= m ? zero : n == 1 ? load_stream(v + k * chunks + (t - row0 * chunks)) : v[k * chunks + (t - row0 * chunks)];
+        vraw[u] = k >= m ? zero : n == 1 ? load_stream(v + k * row_chunks + (t - row0 * chunks)) : v[k * row_chunks + (t - row0 * chunks)];
         pk[u] = k < m ? p[k] : static_cast<half_t>(0.f);
       }
 #pragma unroll
@@ -1927,7 +1930,7 @@ __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* _
       s3 += red[(q + 3) * chunks + c][e];
     }
     for (; q < per_pass; ++q) s0 += red[q * chunks + c][e];
-    out[(h * n + r) * d + t] = static_cast<half_t>((s0 + s1) + (s2 + s3));
+    out[(h * n + r) * d + first * 8u + t] = static_cast<half_t>((s0 + s1) + (s2 + s3));
   }
 }
 
@@ -2563,14 +2566,18 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
         key_split(heads, 4 * kNumCU, ktiles, &mfma_us);
         mfma_us = mfma_us + 1.5 < 5.5 ? 5.5 : mfma_us + 1.5;  // (no launch of the tiles takes less: 2 rows against 77 keys 7.5 us, the row kernel 4.6)
       }
-      // 3 .. 8 rows, one workgroup per (head, row) while these fit the chip at once: a head's V in one contiguous sweep
-      // per row (measured with V from memory, 32 heads of 80: 4 rows against 1024 / 2048 / 4096 keys 7.1 / 9.8 / 21.5 us
-      // where the row kernel takes 8.0 / 14.2 / 33.4; 8 rows 7.2 / 9.9 / 21.1 where the choices below take 12.4 / 16.7 / 19.4)
-      // -- up to ~3000 keys; beyond, the key-split MFMA tiles lead.  One and two rows: the row kernel (7.1 against 9.8
-      // us at 2048 keys: 32 workgroups are too few to pull V in)
-      if (n >= 3 && n <= 8 && heads * n <= kNumCU && d / 8 <= 128 && (m < 3072 || !mfma_ok)) {
+      // 2 .. 8 rows, one workgroup per (head, row) while these fit the chip at once: a head's V in one contiguous sweep
+      // per row -- or two workgroups, each with half of the pieces of a key, while those fit as well (measured with V
+      // from memory, 32 heads of 80, us: 4 rows against 1024 / 2048 / 4096 keys 6.5 / 8.4 / 16.0 in halves, 7.1 / 9.6 /
+      // 21.4 whole, where the row kernel takes 8.0 / 14.2 / 33.4 and the key-split tiles 19.3 at 4096; 8 rows, whole:
+      // 7.2 / 9.9 / 21.1 against 12.4 / 16.7 for the tiles up to 2048 keys and 19.4 at 4096; 2 rows in halves 6.3 / 8.3 /
+      // 16.2, the row kernel 6.7 / 9.1 / 19.1).  One row: the row kernel (7.0 against 8.3 us at 2048 keys: 64 workgroups
+      // are too few to pull V in)
+      const int64_t pieces = d / 8;
+      const int halves = pieces % 2 == 0 && heads * n * 2 <= kNumCU ? 2 : 1;
+      if (n >= 2 && n <= 8 && heads * n <= kNumCU && pieces <= 128 && (m < (halves == 2 ? 6144 : 3072) || !mfma_ok)) {
         rows = true;
-        cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, 0}, 1, 0};
+        cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, static_cast<int32_t>(d / halves)}, 1, 0};
       } else if (n >= 2 && n <= 8 && m >= 3072 && heads * n <= kNumCU && mfma_ok) {
         rows = false;  // (4 rows against 4096 / 8192 keys with V from memory: the row kernel 33 / 61 us, one sweep per row 22 / 39, the tiles 19 / 28)
       } else {
@@ -2621,12 +2628,16 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     return check_launch("attn_pv");
   }
   if (cfg.vec != 8) return fail("attn_pv: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
-  if (cfg.variant == DTAS_GEMM_SKINNY && cfg.block == 1024) {  // one row per workgroup, V's head in one sweep
+  if (cfg.variant == DTAS_GEMM_SKINNY && (cfg.block == 1024 || cfg.tile[2] > 0)) {  // one row per workgroup, V's head in one sweep
+    // tile[2] = columns per workgroup (0: all d), a multiple of 8 that divides d
+    const int64_t cols = cfg.tile[2] > 0 ? cfg.tile[2] : d;
     if (cfg.tile[0] != 1 || cfg.tile[1] != 8) return fail("attn_pv: the whole-row kernel takes one row per workgroup and 8-column pieces");
-    if (d / 8 > 128) return fail("attn_pv: the whole-row kernel holds head dimensions up to 1024, got %lld", (long long)d);
+    if (cfg.block != 256 && cfg.block != 512 && cfg.block != 1024) return fail("attn_pv: the whole-row kernel uses 256, 512 or 1024 threads, got %d", cfg.block);
+    if (cols % 8 != 0 || d % cols != 0 || cols / 8 > 128) return fail("attn_pv: the whole-row kernel takes columns per workgroup that divide d, in pieces of 8, at most 1024 (d=%lld, %lld)", (long long)d, (long long)cols);
     if (cfg.split_k > 1) return fail("attn_pv: the row kernels do not split K");
-    if (n > 65535) return fail("attn_pv: too many workgroups for the row kernel");
-    hipLaunchKernelGGL(attn_pv_whole_row_kernel, dim3(static_cast<unsigned>(heads), static_cast<unsigned>(n)), dim3(1024), 0, s, a, w, c, n, m, d);
+    if (n > 65535 || heads * (d / cols) > 0x7fffffff) return fail("attn_pv: too many workgroups for the row kernel");
+    hipLaunchKernelGGL(attn_pv_whole_row_kernel, dim3(static_cast<unsigned>(heads * (d / cols)), static_cast<unsigned>(n)), dim3(cfg.block), 0, s, a, w, c, n, m, d,
+                       static_cast<unsigned>(cols));
     return check_launch("attn_pv");
   }
   if (cfg.variant == DTAS_GEMM_SKINNY) {

@@ -157,18 +157,25 @@ def test_pv_row_kernel(oracle, rows, heads, n, m, d):
                                          (2, 3, 9000, 64), (1, 7, 300, 1024)])
 def test_pv_whole_row_kernel(oracle, heads, n, m, d):
     # one workgroup of 1024 threads per (head, query row): the head's V read as one contiguous run of 16-byte pieces,
-    # d / 8 of them per key (1 .. 128: every thread count per key, idle threads at the end of the workgroup included)
+    # d / 8 of them per key (1 .. 128: every thread count per key, idle threads at the end of the workgroup included);
+    # or several workgroups per (head, row), each with an equal share of a key's pieces (tile[2] columns), 256 .. 1024 threads
     p, v = _pv_inputs(heads, n, m, d, heads + n + m + d)
-    out = Guarded((heads, n, d), torch.float16)
-    ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[1, 8, 0]))
-    _check_pv(out.check(), p, v, oracle)
     rng = np.random.default_rng(m)
     pi = rng.integers(0, 3, size=(heads, n, m)).astype(np.float16)
     vi = rng.integers(-3, 4, size=(heads, m, d)).astype(np.float16)
-    ops.attn_pv(dev(pi), dev(vi), out.t, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[1, 8, 0]))
-    assert np.array_equal(out.check().astype(np.float64), np.einsum("hnm,hmd->hnd", pi.astype(np.float64), vi.astype(np.float64)))
-    with pytest.raises(_lib.DtasError):
-        ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[2, 8, 0]))
+    want_i = np.einsum("hnm,hmd->hnd", pi.astype(np.float64), vi.astype(np.float64))
+    shares = [(1024, 0), (1024, d)] + [(block, d // parts) for block, parts in ((1024, 2), (512, 2), (256, d // 8)) if (d // 8) % parts == 0]
+    for block, cols in shares:
+        c = cfg(variant=_lib.GEMM_SKINNY, block=block, vec=8, tile=[1, 8, cols])
+        out = Guarded((heads, n, d), torch.float16)
+        ops.attn_pv(dev(p), dev(v), out.t, c)
+        _check_pv(out.check(), p, v, oracle)
+        ops.attn_pv(dev(pi), dev(vi), out.t, c)
+        assert np.array_equal(out.check().astype(np.float64), want_i)
+    out = Guarded((heads, n, d), torch.float16)
+    for bad in (dict(block=1024, tile=[2, 8, 0]), dict(block=1024, tile=[1, 8, 12]), dict(block=128, tile=[1, 8, d]), dict(block=1024, tile=[1, 8, 2 * d])):
+        with pytest.raises(_lib.DtasError):
+            ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, vec=8, **bad))
 
 
 @pytest.mark.parametrize("n", [2, 3, 4, 5, 8, 12])
