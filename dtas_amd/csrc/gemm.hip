@@ -1872,6 +1872,67 @@ __global__ void __launch_bounds__(256) attn_pv_rows_kernel(const half_t* __restr
   }
 }
 
+// Scores for a handful of query rows (decoding): out[h, r, k] = epilogue(Q[h, r] . K[h, k]).  What the op moves is the
+// head's K, m rows of d fp16 = d / 8 16-byte pieces each, contiguous in memory; a workgroup of 1024 threads takes a run of
+// keys and sweeps it as attn_pv_whole_row_kernel sweeps V: thread t holds piece t % (d / 8) of the R query rows and
+// multiplies it with that piece of keys t / (d / 8), + per-pass, ... (consecutive threads, consecutive 16 bytes, kU
+// passes in flight), 8 products per row; the d / 8 threads of a key are neighbours, their sums meet in the LDS and the
+// first R * per-pass threads add them in piece order, apply the epilogue and store a row's scores side by side.
+template <int R>
+__global__ void __launch_bounds__(1024) attn_scores_rows_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kmat,
+                                                               const half_t* __restrict__ mask, float* __restrict__ out, int64_t n,
+                                                               int64_t m, int64_t d, float scale, unsigned keys_per_wg) {
+  constexpr int kU = 4;
+  __shared__ float part[R][1024];
+  const unsigned chunks = static_cast<unsigned>(d / 8), per_pass = 1024u / chunks, t = threadIdx.x;
+  const int64_t h = blockIdx.y, r0 = static_cast<int64_t>(blockIdx.z) * R;
+  const int64_t k_lo = static_cast<int64_t>(blockIdx.x) * keys_per_wg;
+  const int64_t k_hi = k_lo + keys_per_wg < m ? k_lo + keys_per_wg : m;
+  const bool active = t < per_pass * chunks;
+  const unsigned key0 = t / chunks, c = t - key0 * chunks;
+  const u32x4* kp = reinterpret_cast<const u32x4*>(Kmat + h * m * d);
+  f16x8 q[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    q[r] = __builtin_bit_cast(f16x8, active && r0 + r < n ? *(reinterpret_cast<const u32x4*>(Q + (h * n + r0 + r) * d) + c) : zero);
+  }
+  for (int64_t kb = k_lo; kb < k_hi; kb += static_cast<int64_t>(kU) * per_pass) {
+    u32x4 raw[kU];
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const int64_t k = kb + static_cast<int64_t>(u) * per_pass + key0;
+      // (K is read this once and streamed past the caches, unless further blocks of rows come for it)
+      raw[u] = !(active && k < k_hi) ? zero : n <= R ? load_stream(kp + k * chunks + c) : kp[k * chunks + c];
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      if (kb + static_cast<int64_t>(u) * per_pass >= k_hi) break;  // (uniform)
+      const f16x8 kv = __builtin_bit_cast(f16x8, raw[u]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += static_cast<float>(q[r][e]) * static_cast<float>(kv[e]);
+        part[r][t] = sum;
+      }
+      __syncthreads();
+      for (unsigned idx = t; idx < R * per_pass; idx += 1024u) {
+        const unsigned r = idx / per_pass, j = idx - r * per_pass;
+        const int64_t k = kb + static_cast<int64_t>(u) * per_pass + j, row = r0 + r;
+        if (k < k_hi && row < n) {
+          float sum = 0.f;
+          for (unsigned cc = 0; cc < chunks; ++cc) sum += part[r][j * chunks + cc];
+          const half_t v = epilogue_value_k<kEpiScores>(round_h(sum), false, scale, 0.f, static_cast<float>(mask[row * m + k]), 0.f);
+          out[(h * n + row) * m + k] = static_cast<float>(v);
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
 // P.V for one query row per workgroup, the whole of V's head read in one sweep (decoding: n = 1, a few heads' worth of
 // workgroups on the chip).  A head's V is m rows of d fp16 = d / 8 16-byte pieces each, contiguous in memory: thread t of
 // 1024 takes piece t % (d / 8) of the rows t / (d / 8), + rows-per-pass, ... -- consecutive threads read consecutive
@@ -2456,6 +2517,46 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   // the walking kernel: 128x64 tiles, at most three workgroups per CU (their LDS allows no more).  Up to 64 query
   // rows half of such a tile would be idle, and fewer tiles than CUs leave CUs idle: 64x64 tiles of the general
   // kernel then (n = 64 against 2048 keys: 6.9 us against 10.3)
+  // a handful of query rows (decoding): the head's K in one sweep, R rows per workgroup (cfg: DTAS_GEMM_SKINNY, block 1024,
+  // tile {1|2|4|8, 8, keys per workgroup or 0})
+  auto launch_rows = [&](int R, int64_t keys_per_wg) -> int {
+    const int64_t per_pass = 1024 / (d / 8);
+    if (keys_per_wg <= 0) {
+      // whole passes; enough workgroups to fill the chip twice, at least two passes each
+      const int64_t want = ceil_div(m * heads * ceil_div(n, R), 2 * kNumCU);
+      keys_per_wg = ceil_div(want < 2 * per_pass ? 2 * per_pass : want, per_pass) * per_pass;
+    }
+    const int64_t gx = ceil_div(m, keys_per_wg), gz = ceil_div(n, R);
+    if (gx > 0x7fffffff || gz > 65535) return fail("attn_scores: too many workgroups for the row kernel");
+    const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(heads), static_cast<unsigned>(gz));
+    const half_t* q_ = static_cast<const half_t*>(Q);
+    const half_t* k_ = static_cast<const half_t*>(Kmat);
+    const half_t* m_ = static_cast<const half_t*>(mask);
+    float* o_ = static_cast<float*>(out);
+    const float sc = static_cast<float>(static_cast<half_t>(scale));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const unsigned kw = static_cast<unsigned>(keys_per_wg);
+    switch (R) {
+      case 1: hipLaunchKernelGGL(attn_scores_rows_kernel<1>, grid, dim3(1024), 0, st, q_, k_, m_, o_, n, m, d, sc, kw); break;
+      case 2: hipLaunchKernelGGL(attn_scores_rows_kernel<2>, grid, dim3(1024), 0, st, q_, k_, m_, o_, n, m, d, sc, kw); break;
+      case 4: hipLaunchKernelGGL(attn_scores_rows_kernel<4>, grid, dim3(1024), 0, st, q_, k_, m_, o_, n, m, d, sc, kw); break;
+      default: hipLaunchKernelGGL(attn_scores_rows_kernel<8>, grid, dim3(1024), 0, st, q_, k_, m_, o_, n, m, d, sc, kw); break;
+    }
+    return check_launch("attn_scores");
+  };
+  if (user && user->variant == DTAS_GEMM_SKINNY) {
+    const int R = user->tile[0];
+    if (user->block != 1024 || user->vec != 8 || user->tile[1] != 8 || (R != 1 && R != 2 && R != 4 && R != 8))
+      return fail("attn_scores: the row kernel takes block 1024, vec 8 and tile {1|2|4|8, 8, keys per workgroup}");
+    if (d / 8 > 128) return fail("attn_scores: the row kernel holds head dimensions up to 1024, got %lld", (long long)d);
+    if (user->tile[2] < 0 || user->tile[2] % (1024 / (d / 8)) != 0)
+      return fail("attn_scores: keys per workgroup must be a multiple of the %lld keys a pass covers", (long long)(1024 / (d / 8)));
+    return launch_rows(R, user->tile[2]);
+  }
+  // one or two rows always, three or four against many keys (with K from memory, 32 heads of 80, us: 1 row against 2048 /
+  // 4096 / 8192 keys 4.7 / 7.0 / 11.6 where the 64x64 tiles take 6.0 / 10.5 / 18.8; 2 rows 5.6 / 8.3 / 14.5 against 6.1 /
+  // 10.6 / 18.8; 4 rows 6.7 / 9.3 / 16.4 against 6.1 / 10.6 / 19.2; 8 rows lose: 11.1 against 6.2 at 2048)
+  if (!user && d / 8 <= 128 && (n <= 2 || (n <= 4 && m >= 3072))) return launch_rows(n <= 1 ? 1 : n <= 2 ? 2 : 4, 0);
   const unsigned tm = static_cast<unsigned>(ceil_div(n, 128)), tn = static_cast<unsigned>(ceil_div(m, 64));
   const int64_t total = static_cast<int64_t>(tm) * tn * heads;
   const bool small = n <= 64 || total < kNumCU;

@@ -293,7 +293,9 @@ int dtas_gemm_f16_fused(const void* A, const void* W, const void* bias, const vo
  * out[h,i,j] = fp32(min(max(fp16(fp16(Q[h,i,:] . K[h,j,:]) * fp16(scale)), -65504), mask[i,j]))
  * Q[heads,n,d], K[heads,m,d], mask[n,m] fp16 (shared by the heads), out[heads,n,m] fp32; n and m are the
  * dynamic extents, d (80 in the model) a multiple of 8.  One batched launch over the heads on the MFMA
- * kernels; cfg, when given, is a DTAS_GEMM_MFMA row for the per-head (n, m, d) problem. */
+ * kernels; cfg, when given, is a DTAS_GEMM_MFMA row for the per-head (n, m, d) problem, or a DTAS_GEMM_SKINNY row
+ * {block 1024, vec 8, tile {1|2|4|8, 8, k}} for the kernel that serves a handful of query rows (decoding): that many
+ * rows per workgroup, k keys per workgroup (a multiple of 1024 / (d / 8); 0: chosen), d <= 1024. */
 int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, void* out, int64_t heads,
                              int64_t n, int64_t m, int64_t d, float scale, const dtas_config* cfg,
                              void* stream);

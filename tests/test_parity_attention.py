@@ -61,6 +61,31 @@ def test_scores_every_tile(oracle, tile, block, stages, heads, n, m, d):
     _check(out.check(), q, k, mask, oracle)
 
 
+@pytest.mark.parametrize("rows", [1, 2, 4, 8])
+@pytest.mark.parametrize("heads,n,m,d,keys", [(32, 1, 2048, 80, 0), (3, 1, 515, 80, 102), (2, 3, 77, 64, 0), (2, 8, 1000, 128, 128), (1, 5, 1, 16, 0),
+                                              (2, 2, 300, 136, 60), (1, 9, 4100, 8, 1024), (1, 2, 260, 1024, 8)])
+def test_scores_row_kernel(oracle, rows, heads, n, m, d, keys):
+    # a workgroup of 1024 threads sweeps a run of the head's keys for 1, 2, 4 or 8 query rows (d / 8 = 1 .. 128 threads
+    # per key; keys per workgroup given or chosen; more query rows than a workgroup takes: further workgroups)
+    q, k, mask = _inputs(heads, n, m, d, rows + n + m + d)
+    out = Guarded((heads, n, m), torch.float32)
+    ops.attn_scores(dev(q), dev(k), dev(mask), out.t, SCALE, cfg(variant=_lib.GEMM_SKINNY, block=1024, vec=8, tile=[rows, 8, keys]))
+    _check(out.check(), q, k, mask, oracle)
+
+
+def test_scores_row_kernel_is_the_choice_for_one_and_two_rows_and_refuses_what_it_cannot_hold(oracle):
+    for n, m in ((1, 2048), (2, 700), (3, 3100), (4, 3072)):
+        q, k, mask = _inputs(32, n, m, 80, n + m)
+        out = Guarded((32, n, m), torch.float32)
+        ops.attn_scores(dev(q), dev(k), dev(mask), out.t, SCALE)
+        _check(out.check(), q, k, mask, oracle)
+    q, k, mask = _inputs(2, 2, 64, 80, 1)
+    out = Guarded((2, 2, 64), torch.float32)
+    for bad in (dict(block=256, tile=[1, 8, 0]), dict(block=1024, tile=[3, 8, 0]), dict(block=1024, tile=[2, 8, 50]), dict(block=1024, tile=[2, 16, 0])):
+        with pytest.raises(_lib.DtasError):
+            ops.attn_scores(dev(q), dev(k), dev(mask), out.t, SCALE, cfg(variant=_lib.GEMM_SKINNY, vec=8, **bad))
+
+
 def test_scores_errors():
     q, k, mask = _inputs(2, 8, 8, 80, 1)
     out = torch.empty(2, 8, 8, dtype=torch.float32, device="cuda")
