@@ -1939,8 +1939,10 @@ __global__ void __launch_bounds__(1024) attn_scores_rows_kernel(const half_t* __
 // 16 bytes, a wavefront 1 KiB, eight passes in flight -- and multiplies each piece with its row's P.  The 8 sums of a
 // thread are those of its 8 columns; threads with the same piece index meet in the LDS and are added in thread order.
 __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* __restrict__ P, const half_t* __restrict__ V,
-                                                                half_t* __restrict__ out, int64_t n, int64_t m, int64_t d, unsigned cols) {
+                                                                half_t* __restrict__ out, int64_t n, int64_t m, int64_t d, unsigned cols,
+                                                                unsigned nsplit, float* __restrict__ ws, unsigned* __restrict__ arrivals) {
   __shared__ float red[1024][8];
+  __shared__ unsigned is_last;
   // (cols < d: the workgroups of a (head, row) share the pieces of a key, cols / 8 consecutive ones each)
   const unsigned row_chunks = static_cast<unsigned>(d / 8), chunks = cols / 8, groups = row_chunks / chunks;
   const unsigned per_pass = blockDim.x / chunks, t = threadIdx.x;
@@ -1953,9 +1955,13 @@ __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* _
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  // nsplit > 1: the workgroups blockIdx.z = 0 .. nsplit - 1 of a (head, row) share the keys, a run each, and meet in the
+  // split-K workspace as the GEMM kernels' K slices do (partials added in run order by whoever arrives last)
+  const int64_t run = (m + nsplit - 1) / nsplit;
+  const int64_t k_lo = static_cast<int64_t>(blockIdx.z) * run, k_hi = k_lo + run < m ? k_lo + run : m;
   if (active) {
     constexpr int kU = 8;
-    for (int64_t k0 = row0; k0 < m; k0 += static_cast<int64_t>(kU) * per_pass) {
+    for (int64_t k0 = k_lo + row0; k0 < k_hi; k0 += static_cast<int64_t>(kU) * per_pass) {
       u32x4 vraw[kU];
       half_t pk[kU];
       const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -1964,8 +1970,8 @@ __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* _
         const int64_t k = k0 + static_cast<int64_t>(u) * per_pass;
         // (piece index of thread t in pass u: t + u * per_pass * chunks -- the passes continue where the last thread stopped)
         // (one row: V is read this once and streamed past the caches; more rows: their workgroups share it)
-        vraw[u] = k >= m ? zero : n == 1 ? load_stream(v + k * row_chunks + (t - row0 * chunks)) : v[k * row_chunks + (t - row0 * chunks)];
-        pk[u] = k < m ? p[k] : static_cast<half_t>(0.f);
+        vraw[u] = k >= k_hi ? zero : n == 1 ? load_stream(v + k * row_chunks + (t - row0 * chunks)) : v[k * row_chunks + (t - row0 * chunks)];
+        pk[u] = k < k_hi ? p[k] : static_cast<half_t>(0.f);
       }
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
@@ -1980,7 +1986,9 @@ __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* _
   for (int e = 0; e < 8; ++e) red[t][e] = active ? acc[e] : 0.f;
   __syncthreads();
   // column j of the row: piece j / 8, element j % 8, summed over the per_pass threads that hold that piece
-  if (t < chunks * 8u) {
+  const bool holds = t < chunks * 8u;
+  float sum = 0.f;
+  if (holds) {
     const unsigned c = t >> 3, e = t & 7u;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     unsigned q = 0;
@@ -1991,8 +1999,25 @@ __global__ void __launch_bounds__(1024) attn_pv_whole_row_kernel(const half_t* _
       s3 += red[(q + 3) * chunks + c][e];
     }
     for (; q < per_pass; ++q) s0 += red[q * chunks + c][e];
-    out[(h * n + r) * d + first * 8u + t] = static_cast<half_t>((s0 + s1) + (s2 + s3));
+    sum = (s0 + s1) + (s2 + s3);
   }
+  if (nsplit > 1) {
+    const size_t tile = static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x;  // (row, head, columns)
+    float* tile_ws = ws + tile * nsplit * cols;
+    if (holds) __hip_atomic_store(tile_ws + static_cast<size_t>(blockIdx.z) * cols + t, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0));  // (device-scope stores: drained = visible to every XCD)
+    __syncthreads();
+    if (t == 0) {
+      const unsigned before = __hip_atomic_fetch_add(arrivals + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = before == nsplit - 1 ? 1u : 0u;
+      if (before == nsplit - 1) __hip_atomic_store(arrivals + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-armed for the next launch
+    }
+    __syncthreads();
+    if (is_last == 0 || !holds) return;
+    sum = 0.f;
+    for (unsigned z = 0; z < nsplit; ++z) sum += __hip_atomic_load(tile_ws + static_cast<size_t>(z) * cols + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (holds) out[(h * n + r) * d + first * 8u + t] = static_cast<half_t>(sum);
 }
 
 // Library-owned scratch memory, one set per (device, stream):
@@ -2676,7 +2701,16 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       // are too few to pull V in)
       const int64_t pieces = d / 8;
       const int halves = pieces % 2 == 0 && heads * n * 2 <= kNumCU ? 2 : 1;
-      if (n >= 2 && n <= 8 && heads * n <= kNumCU && pieces <= 128 && (m < (halves == 2 ? 6144 : 3072) || !mfma_ok)) {
+      // many keys (from ~3000) and room on the chip for several workgroups per (head, row): the workgroups share the keys,
+      // a run each, and meet in the split-K workspace (1 row against 4096 / 8192 keys in 8 runs 11.8 / 15.0 us, the row
+      // kernel 16.8 / 30.6; 2 rows in 4 runs 12.1 / 16.9 against 16.5 / 28.0; 4 rows in 2 runs 15.1 / 23.8 against 16.3 /
+      // 28.0 in halves / on the tiles; up to 2048 keys the hand-over costs more than it saves: 8.2 against 7.1)
+      int runs = 1;
+      while (heads * n * runs * 2 <= kNumCU && runs < 8) runs *= 2;
+      if (m >= 3072 && runs >= 2 && pieces <= 128) {
+        rows = true;
+        cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, static_cast<int32_t>(d)}, runs, 0};
+      } else if (n >= 2 && n <= 8 && heads * n <= kNumCU && pieces <= 128 && (m < (halves == 2 ? 6144 : 3072) || !mfma_ok)) {
         rows = true;
         cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, static_cast<int32_t>(d / halves)}, 1, 0};
       } else if (n >= 2 && n <= 8 && m >= 3072 && heads * n <= kNumCU && mfma_ok) {
@@ -2734,11 +2768,18 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     const int64_t cols = cfg.tile[2] > 0 ? cfg.tile[2] : d;
     if (cfg.tile[0] != 1 || cfg.tile[1] != 8) return fail("attn_pv: the whole-row kernel takes one row per workgroup and 8-column pieces");
     if (cfg.block != 256 && cfg.block != 512 && cfg.block != 1024) return fail("attn_pv: the whole-row kernel uses 256, 512 or 1024 threads, got %d", cfg.block);
+    if (cols > cfg.block) return fail("attn_pv: the whole-row kernel stores a column per thread: %lld columns per workgroup need more than %d threads", (long long)cols, cfg.block);
     if (cols % 8 != 0 || d % cols != 0 || cols / 8 > 128) return fail("attn_pv: the whole-row kernel takes columns per workgroup that divide d, in pieces of 8, at most 1024 (d=%lld, %lld)", (long long)d, (long long)cols);
-    if (cfg.split_k > 1) return fail("attn_pv: the row kernels do not split K");
+    const int nsplit = cfg.split_k < 1 ? 1 : cfg.split_k;
+    if (nsplit > 64) return fail("attn_pv: the whole-row kernel splits the keys over at most 64 workgroups, got %d", nsplit);
     if (n > 65535 || heads * (d / cols) > 0x7fffffff) return fail("attn_pv: too many workgroups for the row kernel");
-    hipLaunchKernelGGL(attn_pv_whole_row_kernel, dim3(static_cast<unsigned>(heads * (d / cols)), static_cast<unsigned>(n)), dim3(cfg.block), 0, s, a, w, c, n, m, d,
-                       static_cast<unsigned>(cols));
+    const size_t tiles = static_cast<size_t>(heads * (d / cols) * n);
+    float* partials = nullptr;
+    unsigned* arrivals = nullptr;
+    std::unique_lock<std::recursive_mutex> ws_lock;  // held until the launch is enqueued
+    if (nsplit > 1 && split_scratch(s, tiles * nsplit * cols * sizeof(float), tiles, nsplit, &partials, &arrivals, &ws_lock) != 0) return -1;
+    hipLaunchKernelGGL(attn_pv_whole_row_kernel, dim3(static_cast<unsigned>(heads * (d / cols)), static_cast<unsigned>(n), static_cast<unsigned>(nsplit)),
+                       dim3(cfg.block), 0, s, a, w, c, n, m, d, static_cast<unsigned>(cols), static_cast<unsigned>(nsplit), partials, arrivals);
     return check_launch("attn_pv");
   }
   if (cfg.variant == DTAS_GEMM_SKINNY) {

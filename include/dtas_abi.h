@@ -309,7 +309,8 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
  * the workgroups of a (head, tile) split m and meet in the split-K workspace), or a DTAS_GEMM_SKINNY row
  * {block 256, tile {1|2|4|8, 8, 0}} for the kernel that serves a handful of rows (decoding), or {block 1024, tile {1, 8, 0}}
  * for one workgroup per (head, row) that reads the head's V in one contiguous sweep (d <= 1024) -- tile[2] = c > 0
- * (a multiple of 8 that divides d; block 256, 512 or 1024): d / c workgroups per (head, row), c columns each.  With m % 8 != 0
+ * (a multiple of 8 that divides d, at most `block`; block 256, 512 or 1024): d / c workgroups per (head, row), c columns
+ * each; split_k = s > 1 (at most 64): s workgroups share the keys, a run each, and meet in the split-K workspace.  With m % 8 != 0
  * or a P off a 16-byte boundary the MFMA kernels read the rows of P where they lie (16-byte pieces at 2-byte
  * alignment; the last m % 8 keys are added in the epilogue, in fp32, before the one rounding);
  * d % 8 != 0 or a V off 16 bytes fall back to the element-access kernel; m == 0 writes zeros. */

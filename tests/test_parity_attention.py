@@ -189,22 +189,25 @@ def test_pv_whole_row_kernel(oracle, heads, n, m, d):
     pi = rng.integers(0, 3, size=(heads, n, m)).astype(np.float16)
     vi = rng.integers(-3, 4, size=(heads, m, d)).astype(np.float16)
     want_i = np.einsum("hnm,hmd->hnd", pi.astype(np.float64), vi.astype(np.float64))
-    shares = [(1024, 0), (1024, d)] + [(block, d // parts) for block, parts in ((1024, 2), (512, 2), (256, d // 8)) if (d // 8) % parts == 0]
-    for block, cols in shares:
-        c = cfg(variant=_lib.GEMM_SKINNY, block=block, vec=8, tile=[1, 8, cols])
+    shares = [(1024, 0, 1), (1024, d, 1), (1024, d, 2), (1024, 0, 8), (512, d, 64)]
+    shares += [(block, d // parts, split) for block, parts, split in ((1024, 2, 1), (512, 2, 4), (256, d // 8, 1)) if (d // 8) % parts == 0]
+    for block, cols, split in shares:  # (split: the workgroups of a (head, row) share the keys and meet in the workspace)
+        if (cols or d) > block:
+            continue  # (a thread per column of the workgroup's share)
+        c = cfg(variant=_lib.GEMM_SKINNY, block=block, vec=8, tile=[1, 8, cols], split_k=split)
         out = Guarded((heads, n, d), torch.float16)
         ops.attn_pv(dev(p), dev(v), out.t, c)
         _check_pv(out.check(), p, v, oracle)
         ops.attn_pv(dev(pi), dev(vi), out.t, c)
         assert np.array_equal(out.check().astype(np.float64), want_i)
     out = Guarded((heads, n, d), torch.float16)
-    for bad in (dict(block=1024, tile=[2, 8, 0]), dict(block=1024, tile=[1, 8, 12]), dict(block=128, tile=[1, 8, d]), dict(block=1024, tile=[1, 8, 2 * d])):
+    for bad in (dict(block=1024, tile=[2, 8, 0]), dict(block=1024, tile=[1, 8, 12]), dict(block=128, tile=[1, 8, d]), dict(block=1024, tile=[1, 8, 2 * d]), dict(block=256, tile=[1, 8, d], split_k=128)):
         with pytest.raises(_lib.DtasError):
             ops.attn_pv(dev(p), dev(v), out.t, cfg(variant=_lib.GEMM_SKINNY, vec=8, **bad))
 
 
-@pytest.mark.parametrize("n", [2, 3, 4, 5, 8, 12])
-@pytest.mark.parametrize("m", [77, 512, 1024, 4096, 4097])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 12])
+@pytest.mark.parametrize("m", [77, 512, 1024, 3072, 4096, 4097])
 def test_pv_few_rows_builtin_choice(oracle, n, m):
     # 2 .. 12 query rows: two- or four-row workgroups of the row kernel, one workgroup per row sweeping the head's V
     # (3 .. 8 rows, up to ~3000 keys), or 64-row MFMA tiles with the keys split (any key count: P is read where it lies)
