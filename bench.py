@@ -209,13 +209,18 @@ def _workload(name: str, n: int, extra=None):
                 2 * (n * K + N * K + n * N), 2 * n * N * K)
     if name == "attn_scores_f16_f32":
         # fused_NT_matmul1_divide_maximum_minimum_cast2: 32 heads of 80, n = m; the fp32 scores dominate the bytes
+        # (extra = (rows, m): a handful of query rows against m keys, the decode step's form; what it moves is K)
         heads, d = 32, 80
-        mask = torch.full((n, n), 65504.0, dtype=torch.float16, device="cuda").tril_().add_(
-            torch.full((n, n), -65504.0, dtype=torch.float16, device="cuda").triu_(1))
-        make = lambda s: (normal((heads, n, d), s), normal((heads, n, d), s + 50), mask, empty((heads, n, n), torch.float32))
-        return (make, lambda b: call(L.dtas_attn_scores_f16_f32, P(b[0]), P(b[1]), P(b[2]), P(b[3]), heads, n, n, d,
+        rows, m = (extra if extra else (n, n))
+        if extra:
+            mask = torch.zeros((rows, m), dtype=torch.float16, device="cuda")
+        else:
+            mask = torch.full((n, n), 65504.0, dtype=torch.float16, device="cuda").tril_().add_(
+                torch.full((n, n), -65504.0, dtype=torch.float16, device="cuda").triu_(1))
+        make = lambda s: (normal((heads, rows, d), s), normal((heads, m, d), s + 50), mask, empty((heads, rows, m), torch.float32))
+        return (make, lambda b: call(L.dtas_attn_scores_f16_f32, P(b[0]), P(b[1]), P(b[2]), P(b[3]), heads, rows, m, d,
                                      0.11179039301310044, None, stream),
-                2 * 2 * heads * n * d + 2 * n * n + 4 * heads * n * n, 2 * heads * n * n * d)
+                2 * heads * (rows + m) * d + 2 * rows * m + 4 * heads * rows * m, 2 * heads * rows * m * d)
     if name == "attn_pv_f16":
         # matmul8 (n = m) / matmul10 (extra = (1, m): one query row): 32 heads of 80; the probabilities dominate the bytes
         heads, d = 32, 80
@@ -426,6 +431,9 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("attn_scores_f16_f32", n, None, steps, warmup))
         rows.append(measure("attn_pv_f16", n, None, steps, warmup))
     rows.append(measure("attn_pv_f16", 1, (1, 2048), steps, warmup))      # matmul10: decoding against 2048 keys
+    rows.append(measure("attn_pv_f16", 1, (1, 8192), steps, warmup))      # ... against 8192 (the keys shared by workgroups)
+    rows.append(measure("attn_scores_f16_f32", 1, (1, 2048), steps, warmup))  # the decode step's scores
+    rows.append(measure("attn_scores_f16_f32", 1, (1, 8192), steps, warmup))
     # a sequence length off every vector width: rows that start at any element
     for op in ("softmax_f16", "attn_scores_f16_f32", "attn_pv_f16"):
         rows.append(measure(op, 1025, None, steps, warmup))
