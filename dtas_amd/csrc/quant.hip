@@ -189,6 +189,14 @@ __device__ __forceinline__ half_t finish_q8(float acc, const half_t* bias, int64
   if (kind == DTAS_EPI_BIAS_GELU) t = gelu_erf_f16_steps(t);
   return t;
 }
+// the same with the bias element already in a register (requested before W is streamed: read at the end it costs the
+// launch a round trip to memory of its own)
+__device__ __forceinline__ half_t finish_q8_with(float acc, bool has_bias, half_t bias_j, int kind) {
+  half_t t = static_cast<half_t>(acc);
+  if (has_bias) t = static_cast<half_t>(static_cast<float>(t) + static_cast<float>(bias_j));
+  if (kind == DTAS_EPI_BIAS_GELU) t = gelu_erf_f16_steps(t);
+  return t;
+}
 
 // Workgroup = R rows of Wq; lane t takes the 16-byte chunks t, t + block, ... (16 weights, 32 bytes
 // of x) of every row, so a wavefront reads 1 KiB of a row at a time, non-temporal.
@@ -211,6 +219,8 @@ __global__ void __launch_bounds__(512) gemv_q8_kernel(const half_t* __restrict__
   float acc[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  // thread r < R stores row row0 + r: its bias element, requested now and kept as loaded
+  const half_t e_bias = bias && threadIdx.x < R && row0 + threadIdx.x < N ? bias[row0 + threadIdx.x] : static_cast<half_t>(0.f);
 
 #pragma unroll 2
   for (int64_t i = threadIdx.x; i < nchunk; i += blockDim.x) {
@@ -237,6 +247,7 @@ __global__ void __launch_bounds__(512) gemv_q8_kernel(const half_t* __restrict__
     }
   }
 
+  asm volatile("" ::"v"(e_bias));  // (it exists by now: its load stays where it was written)
   const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -247,7 +258,7 @@ __global__ void __launch_bounds__(512) gemv_q8_kernel(const half_t* __restrict__
   if (threadIdx.x < R && row0 + threadIdx.x < N) {
     float sum = 0.f;
     for (int w = 0; w < nwaves; ++w) sum += part[w][threadIdx.x];
-    y[row0 + threadIdx.x] = finish_q8(sum, bias, row0 + threadIdx.x, kind);
+    y[row0 + threadIdx.x] = finish_q8_with(sum, bias != nullptr, e_bias, kind);
   }
 }
 
