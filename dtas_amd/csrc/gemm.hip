@@ -1721,6 +1721,17 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(const half_t* __restrict
   float v[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) v[i] = 0.f;
+  // the lane that will store value idx = r * MV + m requests its bias and residual elements now and keeps them as loaded
+  // (read after the reduction they cost the launch a round trip to memory of their own)
+  constexpr int kShift = NV == 64 ? 0 : NV == 32 ? 1 : NV == 16 ? 2 : NV == 8 ? 3 : NV == 4 ? 4 : 5;
+  const unsigned idx = l >> kShift;  // = r * MV + m
+  const int64_t out_row = row0 + idx / MV, out_m = idx % MV;
+  const bool stores = (l & ((1u << kShift) - 1u)) == 0 && out_row < N && out_m < M;
+  const bool add2 = ep.kind == DTAS_EPI_BIAS_ADD2 || ep.kind == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  const half_t hz = static_cast<half_t>(0.f);
+  const half_t e_bias = stores && ep.bias ? ep.bias[out_row] : hz;
+  const half_t e_r1 = stores && add2 ? ep.res1[out_m * N + out_row] : hz;
+  const half_t e_r2 = stores && add2 ? ep.res2[out_m * N + out_row] : hz;
   auto dot8 = [](u32x4 a, u32x4 b, float acc) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1757,6 +1768,7 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(const half_t* __restrict
       for (int r = 0; r < R; ++r) v[r * MV + m] = dot8(xr, wr[r], v[r * MV + m]);
     }
   }
+  asm volatile("" ::"v"(e_bias), "v"(e_r1), "v"(e_r2));  // (they exist by now: their loads stay where they were written)
   // reduce-scatter over the 64 lanes
   int n = NV;
 #pragma unroll
@@ -1775,11 +1787,10 @@ __global__ void __launch_bounds__(256) gemm_rows_kernel(const half_t* __restrict
       v[0] += __shfl_xor(v[0], d, 64);
     }
   }
-  constexpr int kShift = NV == 64 ? 0 : NV == 32 ? 1 : NV == 16 ? 2 : NV == 8 ? 3 : NV == 4 ? 4 : 5;
-  if ((l & ((1u << kShift) - 1u)) == 0) {
-    const unsigned idx = l >> kShift;  // = r * MV + m
-    const int64_t row = row0 + idx / MV, m = idx % MV;
-    if (row < N && m < M) finish(v[0], ep, C, m, row, N);
+  if (stores) {
+    const half_t r = epilogue_value(round_h(v[0]), ep, static_cast<float>(e_bias), static_cast<float>(e_r1), static_cast<float>(e_r2));
+    if (ep.out_f32) static_cast<float*>(C)[out_m * N + out_row] = static_cast<float>(r);
+    else static_cast<half_t*>(C)[out_m * N + out_row] = r;
   }
 }
 
