@@ -52,8 +52,10 @@
 //              the LDS and the MFMA.  For a W with many rows (4096 < N <= 16384, K <= 4096) the looping
 //              form: a workgroup keeps its columns over the whole of K, walked through a ring of LDS stages.
 // ROWS kernel (M <= 4; the built-in choice for M = 2): W streamed in whole rows on the vector ALU.
-// Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles) and
-//              attn_pv_rows_kernel (P.V for a handful of query rows).
+// Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles), attn_scores_rows_kernel (a handful
+//              of query rows: a workgroup sweeps a run of the head's keys), attn_pv_rows_kernel (P.V for one or two query
+//              rows) and attn_pv_whole_row_kernel (P.V for a few query rows: a workgroup sweeps the head's V, the keys
+//              shared between workgroups when they are many).
 #include "dtas_device.h"
 #include "dtas_host.h"
 
