@@ -520,6 +520,8 @@ def main() -> int:
                          "gemv_f16 | gemv_f32 | gemv_q8_f16 | gemv_q8_f32 | take_q8_f16 | take_f16 | rotary_f16 | split3_f16 | swap_axes_f16 | attn_mask_f16 | softmax_temperature_f32 | gemm_f16 | gemm_q8_f16 | gemm_add2_f16 | gemm_gelu_f16 (the last five take --nk; attn_scores n = m)")
     ap.add_argument("--n", type=int, default=4096, help="dynamic extent of the workload (rows n, or GEMM M)")
     ap.add_argument("--nk", default="4096x4096", help="N x K of the gemv/gemm workloads")
+    ap.add_argument("--keys", type=int, default=0,
+                    help="attn_scores_f16_f32 / attn_pv_f16: n query rows against this many keys (the decode step's form with --n 1); 0: n = m")
     ap.add_argument("--operands", default="normal", choices=["normal", "zeros", "ones", "ints"],
                     help="gemm_f16 only: normal = the benchmark's A ~ N(0,1), W ~ N(0,0.02); zeros / ones / ints (-2..2) "
                          "run the same launches on operands that draw less power")
@@ -551,6 +553,8 @@ def main() -> int:
         return 2
 
     extra = tuple(int(v) for v in args.nk.split("x")) if args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32", "take_q8_f16", "take_f16", "gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") else None
+    if args.workload in ("attn_scores_f16_f32", "attn_pv_f16") and args.keys > 0:
+        extra = (args.n, args.keys)
     head = measure(args.workload, args.n, extra, args.steps, args.warmup, streaming=not args.cache_resident)
     is_gemm = args.workload in ("gemm_f16", "gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") and head["bound"] == "mfma"
     info = None
@@ -569,7 +573,7 @@ def main() -> int:
     elif args.workload == "softmax_f32_f16":
         workload_key = f"{args.workload} [12800, n={args.n}]"
     elif args.workload in ("attn_scores_f16_f32", "attn_pv_f16"):
-        workload_key = f"{args.workload} [32 heads of 80, n=m={args.n}]"
+        workload_key = f"{args.workload} [32 heads of 80, n=m={args.n}]" if args.keys <= 0 else f"{args.workload} [32 heads of 80, n={args.n}, m={args.keys}]"
     elif extra is None:
         workload_key = f"{args.workload} [n={args.n}, 4096]"
     elif args.workload in ("gemv_f16", "gemv_f32", "gemv_q8_f16", "gemv_q8_f32"):
