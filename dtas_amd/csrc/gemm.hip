@@ -983,10 +983,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     __syncthreads();
     const bool last = *is_last != 0;
     if (!last) return;
+    // The sum is p0 + p1 + ... in split order whoever arrived last.  The last arriver's own partial is still in its
+    // registers: as split 0 it is the first term, and of two splits the sum is the same in either order (a + b = b + a
+    // exactly) -- then only the others' partials are read back; otherwise all of them, from zero.
+    const bool keep_own = z == 0 || my_split == 2;
+    if (!keep_own) {
 #pragma unroll
-    for (int q = 0; q < kPer; ++q) {
-      pair_set(q, 0, 0.f);
-      pair_set(q, 1, 0.f);
+      for (int q = 0; q < kPer; ++q) {
+        pair_set(q, 0, 0.f);
+        pair_set(q, 1, 0.f);
+      }
     }
     // The partials are added in split order, but requested kGroup tiles at a time (up to 64 loads per lane):
     // one tile per round trip made the combine cost ~1.2 us per split, which capped useful splits at 4.
@@ -1010,9 +1016,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           pair_set(q, 1, pair_get(q, 1) + pr[1]);
         }
     };
-    unsigned k = 0;
-    for (; k + kGroup <= my_split; k += kGroup) add_partials(k, std::integral_constant<int, kGroup>{});
-    for (; k < my_split; ++k) add_partials(k, std::integral_constant<int, 1>{});
+    unsigned k = keep_own && z == 0 ? 1u : 0u;
+    const unsigned k_end = keep_own && z != 0 ? 1u : my_split;  // (two splits, the second one last: p0 alone)
+    for (; k + kGroup <= k_end; k += kGroup) add_partials(k, std::integral_constant<int, kGroup>{});
+    for (; k < k_end; ++k) add_partials(k, std::integral_constant<int, 1>{});
   }
 
   // The sums go through the LDS so that the stores are whole rows of the wavefront tile: staged as 8-byte slots of
