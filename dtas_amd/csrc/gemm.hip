@@ -2572,7 +2572,7 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
       keys_per_wg = ceil_div(want < 2 * per_pass ? 2 * per_pass : want, per_pass) * per_pass;
     }
     const int64_t gx = ceil_div(m, keys_per_wg), gz = ceil_div(n, R);
-    if (gx > 0x7fffffff || gz > 65535) return fail("attn_scores: too many workgroups for the row kernel");
+    if (gx > 0x7fffffff || gz > 65535 || keys_per_wg > 0x7fffffff) return fail("attn_scores: too many workgroups for the row kernel");
     const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(heads), static_cast<unsigned>(gz));
     const half_t* q_ = static_cast<const half_t*>(Q);
     const half_t* k_ = static_cast<const half_t*>(Kmat);
