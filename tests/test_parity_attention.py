@@ -372,3 +372,46 @@ def test_attention_full_size_properties(oracle):
     want = oracle.c.attn_pv(np.ascontiguousarray(pn[:, rows]), vn, threads=8).astype(np.float64)
     got = o[:, rows].cpu().numpy().astype(np.float64)
     assert (np.abs(got - want) <= 1e-4 + 2.0 ** -9 * np.abs(want)).all()
+
+
+@pytest.mark.parametrize("n", [1, 2, 4, 8])
+def test_decode_attention_against_the_prefill_kernels_and_properties(oracle, n):
+    """A handful of query rows against 8192 keys, 32 heads of 80 (the decode step and short continuations): the row
+    kernels return what the same rows return as part of a long prompt (same arithmetic per score; P.V within the fp32
+    summation order), a one-hot P returns a row of V exactly, and sampled heads match the oracle."""
+    heads, m, d = 32, 8192, 80
+    g = torch.Generator(device="cuda").manual_seed(11 + n)
+    q = torch.randn(heads, n, d, device="cuda", generator=g).half()
+    k = torch.randn(heads, m, d, device="cuda", generator=g).half()
+    v = torch.randn(heads, m, d, device="cuda", generator=g).half()
+    mask = torch.full((n, m), 65504.0, dtype=torch.float16, device="cuda")
+    mask[:, m - 5:] = -65504.0
+    sc = torch.empty(heads, n, m, dtype=torch.float32, device="cuda")
+    ops.attn_scores(q, k, mask, sc, SCALE)
+    # the same rows as the last rows of a 128-row block go through the MFMA tiles
+    qq = torch.zeros(heads, 128, d, dtype=torch.float16, device="cuda")
+    qq[:, 128 - n:] = q
+    mm = torch.full((128, m), 65504.0, dtype=torch.float16, device="cuda")
+    mm[128 - n:] = mask
+    big = torch.empty(heads, 128, m, dtype=torch.float32, device="cuda")
+    ops.attn_scores(qq, k, mm, big, SCALE)
+    torch.cuda.synchronize()
+    same = (big[:, 128 - n:] == sc).float().mean().item()
+    assert same > 0.999 and bool(((big[:, 128 - n:] - sc).abs() <= 2.0 ** -9 * sc.abs() + 1e-3).all())
+    assert bool((sc[:, :, m - 5:] == -65504.0).all()) and bool((sc.half().float() == sc).all())
+    want = oracle.c.attn_scores(q[:2].cpu().numpy(), k[:2].cpu().numpy(), mask.cpu().numpy(), SCALE, threads=8)
+    got = sc[:2].cpu().numpy()
+    assert (np.abs(got - want) <= 1e-3 + 2.0 ** -9 * np.abs(want)).all() and (got == want).mean() > 0.98
+    # P.V: one-hot rows pick rows of V; softmaxed rows against the oracle
+    pick = torch.randint(0, m, (heads, n), device="cuda", generator=g)
+    p = torch.zeros(heads, n, m, dtype=torch.float16, device="cuda")
+    p.scatter_(2, pick.unsqueeze(-1), 1.0)
+    o = torch.empty(heads, n, d, dtype=torch.float16, device="cuda")
+    ops.attn_pv(p, v, o)
+    assert bool((o == torch.gather(v, 1, pick.unsqueeze(-1).expand(-1, -1, d))).all())
+    p = torch.softmax(sc, -1).half()
+    ops.attn_pv(p, v, o)
+    torch.cuda.synchronize()
+    want = oracle.c.attn_pv(p[:2].cpu().numpy(), v[:2].cpu().numpy(), threads=8).astype(np.float64)
+    got = o[:2].cpu().numpy().astype(np.float64)
+    assert (np.abs(got - want) <= 1e-4 + 2.0 ** -9 * np.abs(want)).all()
