@@ -52,7 +52,8 @@
 //              the LDS and the MFMA.  For a W with many rows (4096 < N <= 16384, K <= 4096) the looping
 //              form: a workgroup keeps its columns over the whole of K, walked through a ring of LDS stages.
 // ROWS kernel (M <= 4; the built-in choice for M = 2): W streamed in whole rows on the vector ALU.
-// Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles), attn_scores_rows_kernel (a handful
+// Also here: attn_scores_kernel (Q.K^T for head dimensions up to 128, walking tiles; attn_scores_pipe_kernel: its two-deep
+//              pipeline for head dimensions 80 and 96), attn_scores_rows_kernel (a handful
 //              of query rows: a workgroup sweeps a run of the head's keys), attn_pv_rows_kernel (P.V for one or two query
 //              rows) and attn_pv_whole_row_kernel (P.V for a few query rows: a workgroup sweeps the head's V, the keys
 //              shared between workgroups when they are many).
@@ -141,6 +142,20 @@ __device__ __forceinline__ half_t epilogue_value_k(half_t mm, bool has_bias, flo
   } else if (KIND == DTAS_EPI_BIAS_GELU) {
     t = gelu_erf_f16_steps(t);
   }
+  return t;
+}
+
+// The scores' three steps on four values as packed fp16 instructions: fp32 holds the product of two fp16 numbers exactly,
+// so the fp16 product rounded once is what the step computed through fp32 gives, and maximum and minimum are exact (the
+// same NaN rule as fmaxf / fminf: the other operand) -- the same bits for a quarter of the instructions, in an epilogue
+// that is bound by them (a 128x64 tile is 32 scores per lane).
+__device__ __forceinline__ f16x4 scores_steps_vec(f16x4 mm, float scale, f16x4 mask) {
+#pragma clang fp contract(off)
+  const half_t sc = static_cast<half_t>(scale), low = static_cast<half_t>(-65504.f);
+  const f16x4 s4 = {sc, sc, sc, sc}, low4 = {low, low, low, low};
+  f16x4 t = mm * s4;                      // T_divide (a multiply by fp16(1/sqrt(d)))
+  t = __builtin_elementwise_max(t, low4);  // T_maximum
+  t = __builtin_elementwise_min(t, mask);  // T_minimum with the mask
   return t;
 }
 
@@ -1306,9 +1321,7 @@ __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restri
       f16x4 hv = *reinterpret_cast<const f16x4*>(region + mr * kRowB + ((slot ^ (mr & (kSlots - 1))) * 8));
       const int64_t row = m0 + wm * WTM + mr;
       if (row >= n) continue;
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        hv[e] = epilogue_value_k<kEpiScores>(hv[e], false, scale, 0.f, static_cast<float>(mk[p][e]), 0.f);
+      hv = scores_steps_vec(hv, scale, mk[p]);
       float* dst = out + (static_cast<int64_t>(batch) * n + row) * m + col;
       if (vec_ok) {
         const f32x4v wide = {static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]), static_cast<float>(hv[3])};
@@ -1324,6 +1337,200 @@ __global__ void __launch_bounds__(256) attn_scores_kernel(const half_t* __restri
     }
     __syncthreads();  // the staging regions are free: the next tile's operands may land
   }
+}
+
+// The walking scores kernel for head dimensions 64 + 8 TC (TC = 2: the model's 80; 4: 96), rows of whole sectors, as a
+// two-deep pipeline.  In attn_scores_kernel a workgroup's tile is a chain -- request the operands, wait for them,
+// multiply, stage, store, and wait for the stores to drain before the next operands may land -- hidden only by the
+// other two workgroups of the CU.  Here the tail of the head dimension (k = 64 ..) is kept in rows of its own 16 TC bytes
+// instead of a second 128-byte k tile, so a tile's operands take 24 KiB + 192 x 16 TC bytes and two sets fit twice per
+// CU: the next tile's operands and mask are requested as soon as the MFMAs of the current one are done, and land while
+// it is staged and its epilogue computed; the results wait in registers and are stored after the next tile's operands
+// have been waited for, so that no wait for loads ever waits for stores issued just before (loads and stores share one
+// counter, in order).  Tile numbering, mask, staging and epilogue as in attn_scores_kernel<128, 64>.
+template <int TC>
+__global__ void __launch_bounds__(256) attn_scores_pipe_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kmat,
+                                                               const half_t* __restrict__ mask, float* __restrict__ out,
+                                                               int64_t n, int64_t m, int64_t d, float scale, unsigned tiles_m,
+                                                               unsigned tiles_n, unsigned heads, unsigned pinned) {
+  constexpr int BM = 128, BN = 64, NW = 4, WN = 2, WTM = BM / 2, WTN = BN / 2, MT = WTM / 32, NT = WTN / 32;
+  constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
+  constexpr int kTB = 16 * TC;                                // bytes of a row's tail
+  constexpr int kABytes = BM * kRowBytes, kMain = (BM + BN) * kRowBytes;
+  constexpr int kTailA = kMain, kTailW = kMain + BM * kTB, kSet = kMain + (BM + BN) * kTB;
+  constexpr int kRowsPerTailLoad = 64 / TC;                   // rows a 1 KiB load of tails covers
+  static_assert(TC == 2 || TC == 4, "tails of 16 or 32 elements");
+  static_assert(BM % (kRowsPerTailLoad * NW) == 0 || BM / kRowsPerTailLoad <= NW, "tail loads per wavefront");
+  static_assert(BM * BN * 2 <= kSet, "epilogue staging must fit an operand set");
+  __shared__ __attribute__((aligned(1024))) char lds[2 * kSet];
+
+  const unsigned t = threadIdx.x, l = t & 63u;
+  const unsigned wv = __builtin_amdgcn_readfirstlane(t >> 6), wm = wv / WN, wn = wv % WN;
+  const unsigned row_bytes = static_cast<unsigned>(d) * 2u;
+  const unsigned r_in = 2u * (l >> 4) + (((l >> 3) & 1u) ^ (wv & 1u));
+  const unsigned c_in = (l & 7u) ^ r_in;
+  const unsigned g_off = (8u * wv + r_in) * row_bytes + c_in * 16u;
+  const unsigned g_step = 8u * NW * row_bytes;
+  const unsigned t_row = l / TC, t_off = t_row * row_bytes + 128u + (l % TC) * 16u;  // this lane's piece of a tail load
+  unsigned lds_rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) lds_rd[ks] = lds_chunk_offset(l & 31u, 2u * ks + (l >> 5));
+  const unsigned a_base = wm * WTM * 128u, b_base = kABytes + wn * WTN * 128u;
+
+  constexpr int kSlots = WTN / 4, kRowB = WTN * 2, kRowsPerPass = 64 / kSlots, kPasses = WTM / kRowsPerPass;
+  const unsigned slot = l % kSlots, rsub = l / kSlots;
+
+  const unsigned per_batch = tiles_m * tiles_n, total = per_batch * heads;
+  const unsigned span_base = per_batch / kNumXCD, span_rem = per_batch % kNumXCD;
+  const unsigned walk_end = pinned ? kNumXCD * heads * (span_base + (span_rem ? 1u : 0u)) : total;
+  // tile index -> (head, tile row, tile column); false: nothing at this index (a shorter span has ended)
+  auto locate = [&](unsigned tix, unsigned& batch, unsigned& tm, unsigned& tn) -> bool {
+    unsigned pid;
+    if (pinned) {
+      const unsigned xcd = tix % kNumXCD, local = tix / kNumXCD;
+      const unsigned span = span_base + (xcd < span_rem ? 1u : 0u), first = xcd * span_base + (xcd < span_rem ? xcd : span_rem);
+      if (local >= span * heads) return false;
+      batch = __builtin_amdgcn_readfirstlane(local / span);
+      pid = __builtin_amdgcn_readfirstlane(first + local % span);
+    } else {
+      const unsigned gid = xcd_contiguous_id(tix, total);
+      batch = __builtin_amdgcn_readfirstlane(gid / per_batch);
+      pid = __builtin_amdgcn_readfirstlane(gid % per_batch);
+    }
+    tm = __builtin_amdgcn_readfirstlane(pid / tiles_n);
+    tn = __builtin_amdgcn_readfirstlane(pid % tiles_n);
+    return true;
+  };
+  // every operand piece of a tile into set `base`, asynchronously (rows past the extents read as zeros), and this lane's
+  // part of the mask tile into `mk`
+  auto request = [&](unsigned batch, unsigned tm, unsigned tn, char* base, f16x4 (&mk)[kPasses]) {
+    const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
+    const int64_t rows_a = n - m0 < BM ? n - m0 : BM, rows_w = m - n0 < BN ? m - n0 : BN;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(Q + (static_cast<int64_t>(batch) * n + m0) * d, static_cast<unsigned>(rows_a) * row_bytes);
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(Kmat + (static_cast<int64_t>(batch) * m + n0) * d, static_cast<unsigned>(rows_w) * row_bytes);
+#pragma unroll
+    for (int i = 0; i < LA; ++i) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + wv * 1024 + i * NW * 1024), 16, g_off, i * g_step, 0, 0);
+#pragma unroll
+    for (int i = 0; i < LB; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + wv * 1024 + i * NW * 1024), 16, g_off, i * g_step, 0, 0);
+    // tails: load j covers rows j * kRowsPerTailLoad ..; wavefront w takes loads w, w + 4, ... of A and of W
+#pragma unroll
+    for (int j = 0; j < BM / kRowsPerTailLoad; ++j)
+      if (static_cast<unsigned>(j % NW) == wv)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + kTailA + j * 1024), 16, t_off, j * kRowsPerTailLoad * row_bytes, 0, 0);
+#pragma unroll
+    for (int j = 0; j < BN / kRowsPerTailLoad; ++j)
+      if (static_cast<unsigned>(j % NW) == wv)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kTailW + j * 1024), 16, t_off, j * kRowsPerTailLoad * row_bytes, 0, 0);
+    const int64_t col = n0 + wn * WTN + slot * 4;
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const int64_t row = m0 + wm * WTM + p * kRowsPerPass + rsub;
+      const f16x4 zero = {};
+      mk[p] = row < n && col + 3 < m ? *reinterpret_cast<const f16x4_a2*>(mask + row * m + col) : zero;  // (m % 16 == 0: whole vectors)
+    }
+  };
+  // the results of a tile, held until the next tile's operands have been waited for
+  f32x4v held[kPasses];
+  int64_t held_at[kPasses];  // element offset of each vector; -1: nothing to store
+  auto store_held = [&]() {
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p)
+      if (held_at[p] >= 0) __builtin_nontemporal_store(held[p], reinterpret_cast<f32x4v*>(out + held_at[p]));
+  };
+#pragma unroll
+  for (int p = 0; p < kPasses; ++p) held_at[p] = -1;
+
+  f16x4 mk_cur[kPasses], mk_nxt[kPasses];
+  unsigned batch = 0, tm = 0, tn = 0;
+  unsigned tix = blockIdx.x;
+  bool have = false;
+  for (; tix < walk_end && !have; tix += have ? 0u : gridDim.x) have = locate(tix, batch, tm, tn);
+  int cur = 0;
+  if (have) request(batch, tm, tn, lds, mk_cur);
+  while (have) {
+    // the next tile of this workgroup, if any
+    unsigned nbatch = 0, ntm = 0, ntn = 0;
+    bool more = false;
+    unsigned nix = tix + gridDim.x;
+    for (; nix < walk_end && !more; nix += more ? 0u : gridDim.x) more = locate(nix, nbatch, ntm, ntn);
+    char* set = lds + cur * kSet;
+    __builtin_amdgcn_s_waitcnt(0x0070);  // this tile's operands have landed (the stores before them left long ago)
+    __builtin_amdgcn_s_barrier();
+    store_held();                         // the previous tile's results: they drain while this tile is computed
+    f32x16 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      f16x8 fa[MT], fb[NT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const f16x8*>(set + a_base + i * 4096 + lds_rd[ks]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const f16x8*>(set + b_base + j * 4096 + lds_rd[ks]);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int ks = 0; ks < TC / 2; ++ks) {  // the tail: lane l supplies row l & 31, piece 2 ks + (l >> 5) of it
+      f16x8 fa[MT], fb[NT];
+      const unsigned at = (l & 31u) * kTB + (2u * ks + (l >> 5)) * 16u;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa[i] = *reinterpret_cast<const f16x8*>(set + kTailA + (wm * WTM + i * 32) * kTB + at);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb[j] = *reinterpret_cast<const f16x8*>(set + kTailW + (wn * WTN + j * 32) * kTB + at);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+    // every wavefront is done with this set (its fragments are in registers: the MFMAs above consumed them): it becomes
+    // the staging area; the other set is free as well.  (A bare barrier: a wait for the stores just issued is what this
+    // kernel is built to avoid.)
+    DTAS_SCHED_FENCE();
+    __builtin_amdgcn_s_barrier();
+    DTAS_SCHED_FENCE();
+    if (more) request(nbatch, ntm, ntn, lds + (cur ^ 1) * kSet, mk_nxt);
+    // ---- epilogue, as in attn_scores_kernel: staged in a wavefront-private region of this set
+    char* region = set + wv * (WTM * kRowB);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const unsigned mr = i * 32 + (l & 31u);
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f16x4 hv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) hv[e] = static_cast<half_t>(acc[i][j][g * 4 + e]);
+          const unsigned sl = j * 8 + g * 2 + (l >> 5);
+          *reinterpret_cast<f16x4*>(region + mr * kRowB + ((sl ^ (mr & (kSlots - 1))) * 8)) = hv;
+        }
+    }
+    const int64_t m0 = static_cast<int64_t>(tm) * BM, col = static_cast<int64_t>(tn) * BN + wn * WTN + slot * 4;
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) {
+      const unsigned mr = p * kRowsPerPass + rsub;
+      f16x4 hv = *reinterpret_cast<const f16x4*>(region + mr * kRowB + ((slot ^ (mr & (kSlots - 1))) * 8));
+      const int64_t row = m0 + wm * WTM + mr;
+      hv = scores_steps_vec(hv, scale, mk_cur[p]);
+      held[p] = f32x4v{static_cast<float>(hv[0]), static_cast<float>(hv[1]), static_cast<float>(hv[2]), static_cast<float>(hv[3])};
+      held_at[p] = row < n && col + 3 < m ? (static_cast<int64_t>(batch) * n + row) * m + col : -1;
+    }
+#pragma unroll
+    for (int p = 0; p < kPasses; ++p) mk_cur[p] = mk_nxt[p];
+    have = more;
+    batch = nbatch; tm = ntm; tn = ntn;
+    tix = nix;
+    cur ^= 1;
+  }
+  store_held();
 }
 
 // M <= 16 * MT.  Workgroup = 16 columns of C; wavefront w takes k steps w, w + nwaves, ...
@@ -2612,6 +2819,24 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
     // tile, started in tile order, keeps them closer than workgroups that walk (n = m = 4097: 0.79 against 1.05 ms,
     // 3001: 0.43 / 0.53; whole sectors: walking is ahead, 122 against 135 us at 2048)
     const bool whole_sectors = m % 16 == 0 && aligned(out, 64);
+    // head dimensions 80 and 96 on rows of whole sectors: the two-deep pipeline (two workgroups per CU), 2-8 % ahead
+    // of three workgroups per CU that each wait out their own loads and stores (n = m = 512 / 1536 / 2048: 10.7 / 66.5 /
+    // 110.5 against 11.6 / 70.0 / 113.3 us)
+    if (whole_sectors && (d == 80 || d == 96)) {
+      const int64_t grid_p = total < 2 * kNumCU ? total : 2 * kNumCU;
+      const unsigned pin = n * m >= (int64_t{1} << 21) ? 1u : 0u;
+      const half_t* q_ = static_cast<const half_t*>(Q);
+      const half_t* k_ = static_cast<const half_t*>(Kmat);
+      const half_t* m_ = static_cast<const half_t*>(mask);
+      const float sc = static_cast<float>(static_cast<half_t>(scale));
+      if (d == 80)
+        hipLaunchKernelGGL(attn_scores_pipe_kernel<2>, dim3(static_cast<unsigned>(grid_p)), dim3(256), 0, static_cast<hipStream_t>(stream), q_, k_, m_,
+                           static_cast<float*>(out), n, m, d, sc, tm, tn, static_cast<unsigned>(heads), pin);
+      else
+        hipLaunchKernelGGL(attn_scores_pipe_kernel<4>, dim3(static_cast<unsigned>(grid_p)), dim3(256), 0, static_cast<hipStream_t>(stream), q_, k_, m_,
+                           static_cast<float*>(out), n, m, d, sc, tm, tn, static_cast<unsigned>(heads), pin);
+      return check_launch("attn_scores");
+    }
     const int64_t grid = !whole_sectors || total < 3 * kNumCU ? total : 3 * kNumCU;
     hipLaunchKernelGGL((attn_scores_kernel<128, 64>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const half_t*>(Q), static_cast<const half_t*>(Kmat), static_cast<const half_t*>(mask),

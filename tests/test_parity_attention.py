@@ -39,11 +39,13 @@ def test_scores_builtin_config(oracle, n, m):
 
 
 @pytest.mark.parametrize("heads,n,m,d", [(3, 70, 131, 8), (2, 129, 65, 64), (5, 300, 260, 128), (2, 100, 90, 136), (1, 1, 3, 72),
-                                         (40, 520, 512, 80), (3, 1300, 1700, 80), (2, 2049, 1030, 80)])
+                                         (40, 520, 512, 80), (3, 1300, 1700, 80), (2, 2049, 1030, 80), (40, 520, 512, 96), (9, 700, 2048, 80),
+                                         (12, 1300, 1712, 96)])
 def test_scores_builtin_other_head_dims(oracle, heads, n, m, d):
     # d <= 128 is served by the kernel that walks tiles (one or two k tiles), beyond that by the general one;
     # 40 heads x 5 x 8 tiles = 1600 tiles: more than one tile per workgroup; from 2 M scores per head on an XCD keeps a
-    # span of tiles and walks the heads: 11 x 27 and 17 x 17 tiles do not divide by the 8 XCDs (spans of unequal length)
+    # span of tiles and walks the heads: 11 x 27 and 17 x 17 tiles do not divide by the 8 XCDs (spans of unequal length);
+    # d = 80 and 96 with rows of whole 64-byte sectors (m % 16 == 0) take the two-deep pipeline (tails of 16 / 32 elements)
     q, k, mask = _inputs(heads, n, m, d, n + m + d)
     out = Guarded((heads, n, m), torch.float32)
     ops.attn_scores(dev(q), dev(k), dev(mask), out.t, SCALE)
