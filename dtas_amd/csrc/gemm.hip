@@ -159,6 +159,19 @@ __device__ __forceinline__ f16x4 scores_steps_vec(f16x4 mm, float scale, f16x4 m
   return t;
 }
 
+// "+ bias" and the two residual additions on a vector of fp16 values, each step one packed fp16 addition: T_add = mm +
+// bias, T_add_1 = res1 + T_add, T_add_2 = T_add_1 + res2 (before_dl.py:163-206), every one rounded to fp16.
+template <typename V, bool ADD2>
+__device__ __forceinline__ V add_steps_vec(V t, bool has_bias, V bias, V r1, V r2) {
+#pragma clang fp contract(off)
+  if (has_bias) t = t + bias;
+  if (ADD2) {
+    t = r1 + t;
+    t = t + r2;
+  }
+  return t;
+}
+
 __device__ __forceinline__ half_t epilogue_value(half_t mm, const GemmEpilogue& ep, float bias_j, float r1, float r2) {
   const bool hb = ep.bias != nullptr;
   switch (ep.kind) {
@@ -1137,7 +1150,11 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
         const int64_t at = row * N + col;
         if constexpr (KIND == DTAS_EPI_BIAS_GELU) {
           hv = gelu_erf_f16_steps_vec<cvec_t, kVecC>(hv, has_bias, bvh);
-        } else if (KIND != DTAS_EPI_BIAS || has_bias) {  // "+ bias" etc. act on the sum already rounded to fp16
+        } else if constexpr (KIND == DTAS_EPI_BIAS || kAdd2) {
+          // "+ bias", "+ residual" act on the sum already rounded to fp16, each step rounded to fp16: as packed fp16
+          // additions (an fp16 sum rounded once is what the step computed through fp32 and rounded gives: the same bits)
+          hv = add_steps_vec<cvec_t, kAdd2>(hv, has_bias, bvh, r1v[u], r2v[u]);
+        } else {
 #pragma unroll
           for (int e = 0; e < kVecC; ++e)
             hv[e] = epilogue_value_k<KIND>(hv[e], has_bias, ep.scale, bv[e], static_cast<float>(r1v[u][e]),
