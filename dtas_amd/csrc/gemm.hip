@@ -1154,6 +1154,14 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           // "+ bias", "+ residual" act on the sum already rounded to fp16, each step rounded to fp16: as packed fp16
           // additions (an fp16 sum rounded once is what the step computed through fp32 and rounded gives: the same bits)
           hv = add_steps_vec<cvec_t, kAdd2>(hv, has_bias, bvh, r1v[u], r2v[u]);
+        } else if constexpr (KIND == kEpiScores) {
+#pragma unroll
+          for (int h4 = 0; h4 < kVecC / 4; ++h4) {
+            const f16x4 part = scores_steps_vec(f16x4{hv[4 * h4], hv[4 * h4 + 1], hv[4 * h4 + 2], hv[4 * h4 + 3]}, ep.scale,
+                                                f16x4{r1v[u][4 * h4], r1v[u][4 * h4 + 1], r1v[u][4 * h4 + 2], r1v[u][4 * h4 + 3]});
+#pragma unroll
+            for (int e = 0; e < 4; ++e) hv[4 * h4 + e] = part[e];
+          }
         } else {
 #pragma unroll
           for (int e = 0; e < kVecC; ++e)
