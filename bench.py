@@ -26,6 +26,7 @@ For the gemm_f16 workload two more switches: `--operands zeros|ones|ints` runs t
 bits hardly toggle (how far the card's power limit sets the rate on the benchmark's random operands), and
 `--beside-library` times torch.matmul -- the vendor's GEMM library -- on the same operand pool and reports it as
 `library_gemm`, a yardstick that is never part of `value`.
+For the two attention workloads `--keys m` sets the key count apart from `--n` (the decode step: `--n 1 --keys 2048`).
 One GPU only: `--gpus N` with N > 1 exits with a message.
 """
 from __future__ import annotations
