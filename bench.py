@@ -16,12 +16,16 @@ The same JSON line also carries
                  duration measured with HIP events on the launch stream inside the timed region;
   cpu_baseline : the CPU oracle (a port of the PrimFunc loop nest, oracle/cpu_ref.c) on a bounded
                  sample of the same workload, on this machine's host cores;
-  roofline.families : the other families of the metric in short -- the large-n fraction of the HBM roof for
-                 add / copy / casts / RMSNorm / layer norm / softmax / each GEMV shape, TFLOP/s and the fraction
-                 of the MFMA roof for the GEMM at M = 2048 / 4096 / 8192 per (N, K);
-  cpu_baseline.families : the oracle on bounded samples of a GEMV and a GEMM point;
-  sweep        : every op family over the dynamic extent n (GB/s or TFLOP/s and roofline fraction),
-                 all of them HBM-streaming (rotating buffer sets, the GEMM's W included).
+  roofline.fam_* : the other families of the metric as flat scalar keys (nested values do not survive every
+                 consumer of the line) -- `fam_<op>_<shape>_frac` = fraction of the op's roof (HBM for add / copy /
+                 casts / RMSNorm / layer norm / softmax / GEMV and for GEMM while its bytes bound it, MFMA otherwise)
+                 and `fam_<op>_<shape>_us` = the launch; every GEMM point of the M sweep at the three (N, K), and the
+                 reference's own GEMM shapes (N, K) = (2560, 10240), (10240, 2560), (7680, 10240) at n = 256 / 1024 / 4096;
+  cpu_baseline.* : beside the headline sample, the oracle on all host cores and on bounded samples of a GEMV and a
+                 GEMM point, flat as well (`all_cores_value`, `gemv_f16_4096x4096_gbs_1core`, ...);
+  the sweep    : every op family over the dynamic extent n (GB/s or TFLOP/s and roofline fraction), all of them
+                 HBM-streaming (rotating buffer sets, the GEMM's W included), printed as one `sweep {...}` text line per
+                 row *before* the JSON line, which is the last line of stdout (`--out` writes the rows to a file).
 For the gemm_f16 workload two more switches: `--operands zeros|ones|ints` runs the same launches on operands whose
 bits hardly toggle (how far the card's power limit sets the rate on the benchmark's random operands), and
 `--beside-library` times torch.matmul -- the vendor's GEMM library -- on the same operand pool and reports it as
@@ -385,7 +389,7 @@ def cpu_baseline(name: str, n: int, budget_s: float = 12.0) -> dict:
     many, repsn = run(cores, budget_s * 0.4)
     return {"value": round(one, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{name} n={n} H={H}, {reps1} full passes of the oracle (oracle/cpu_ref.c), 1 thread",
-            "all_cores": {"value": round(many, 3), "cores": cores, "passes": repsn}}
+            "all_cores_value": round(many, 3), "all_cores": cores, "all_cores_passes": repsn}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -393,6 +397,8 @@ SWEEP_N = [1, 16, 128, 1024, 4096]
 SWEEP_M = [1, 16, 64, 256, 1024, 2048, 4096, 8192]
 GEMV_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
 GEMM_NK = [(4096, 4096), (11008, 4096), (4096, 11008)]
+# the reference's own GEMM sweeps (experiment/testIR/GEMM/m_n2560_k10240, m_n10240_k2560, m_n7680_k10240: data/*.json)
+GEMM_NK_REFERENCE = [(2560, 10240), (10240, 2560), (7680, 10240)]
 
 
 def sweep(steps: int, warmup: int) -> list:
@@ -400,6 +406,7 @@ def sweep(steps: int, warmup: int) -> list:
     for op in ("add_f16", "copy_f16", "cast_f32_f16", "cast_f16_f32", "rms_norm_f16", "layer_norm_f32_f16", "softmax_f16"):
         for n in SWEEP_N:
             rows.append(measure(op, n, None, steps, warmup))
+    rows.append(measure("softmax_f16", 8192, None, steps, warmup))   # the far end of the dynamic range: [262144, 8192]
     for n in (1024, 2048, 4096):   # the reference's published softmax form: fp32 in, 12800 rows x n
         rows.append(measure("softmax_f32_f16", n, None, steps, warmup))
     for nk in GEMV_SHAPES:
@@ -420,6 +427,9 @@ def sweep(steps: int, warmup: int) -> list:
         rows.append(measure("layer_norm_f32", n, None, steps, warmup))
     for nk in GEMM_NK:
         for m in SWEEP_M:
+            rows.append(measure("gemm_f16", m, nk, steps, warmup))
+    for nk in GEMM_NK_REFERENCE:
+        for m in (256, 1024, 4096):
             rows.append(measure("gemm_f16", m, nk, steps, warmup))
     # the model's own fused shapes (dolly-v2-3b: hidden 2560, 32 heads of 80)
     for m in (1, 16, 256, 2048):   # m = 1: the decode forms (fused_NT_matmul8_add5_add7_add7, ..9_add6_gelu1) on the GEMV kernel
@@ -442,28 +452,31 @@ def sweep(steps: int, warmup: int) -> list:
 
 
 def families(rows: list) -> dict:
-    """The metric's families in short, from the sweep rows: fraction of the HBM roof at the largest n of the
-    memory-bound ops, TFLOP/s and fraction of the MFMA roof of the GEMM at M >= 2048."""
+    """The metric's families as flat scalar keys, from the sweep rows: `fam_<op>_<shape>_frac` is the fraction of the
+    op's roof (HBM at the largest n of the memory-bound ops and for every GEMM point whose bytes bound it, MFMA for
+    the other GEMM points); GEMM points also carry `_us`, and `_tflops` where the MFMA roof applies."""
     out = {}
     for op in ("add_f16", "copy_f16", "cast_f32_f16", "cast_f16_f32", "rms_norm_f16", "layer_norm_f32_f16", "softmax_f16"):
-        big = [r for r in rows if r["op"] == op and r["n"] == 4096 and "NK" not in r]
-        if big:
-            out[f"{op} n=4096"] = {"GB/s": round(big[0]["gbs"], 1), "frac": round(big[0]["frac"], 3)}
+        for r in rows:
+            if r["op"] == op and "NK" not in r and r["n"] in (4096, 8192):
+                out[f"fam_{op}_n{r['n']}_frac"] = round(r["frac"], 3)
     for r in rows:
         if r["op"] == "softmax_f32_f16":
-            out[f"softmax_f32_f16 12800x{r['n']}"] = {"GB/s": round(r["gbs"], 1), "frac": round(r["frac"], 3), "us": r["us"]}
+            out[f"fam_softmax_f32_f16_12800x{r['n']}_frac"] = round(r["frac"], 3)
         if r["op"] == "gemv_f16":
-            out[f"gemv_f16 {r['NK'][0]}x{r['NK'][1]}"] = {"GB/s": round(r["gbs"], 1), "frac": round(r["frac"], 3)}
-        if r["op"] == "gemm_f16" and r["n"] >= 2048:
-            out[f"gemm_f16 M={r['n']} {r['NK'][0]}x{r['NK'][1]}"] = {"TFLOP/s": round(r["tflops"], 1), "frac": round(r["frac"], 3)}
-        if r["op"] == "gemm_f16" and r["n"] in (16, 64, 256):
-            out[f"gemm_f16 M={r['n']} {r['NK'][0]}x{r['NK'][1]}"] = {"us": r["us"], "W TB/s": round(2e-12 * r["NK"][0] * r["NK"][1] / (r["us"] * 1e-6), 2),
-                                                                    "bound": r["bound"], "frac": round(r["frac"], 3)}
+            out[f"fam_gemv_f16_{r['NK'][0]}x{r['NK'][1]}_frac"] = round(r["frac"], 3)
+    for r in rows:
+        if r["op"] == "gemm_f16":
+            key = f"fam_gemm_f16_M{r['n']}_{r['NK'][0]}x{r['NK'][1]}"
+            out[key + "_us"] = round(r["us"], 2)
+            if r["bound"] == "mfma":
+                out[key + "_tflops"] = round(r["tflops"], 1)
+            out[key + ("_frac" if r["bound"] == "mfma" else "_frac_hbm")] = round(r["frac"], 3)
     return out
 
 
 def cpu_families(budget_s: float = 6.0) -> dict:
-    """The oracle on bounded samples of a GEMV and a GEMM point (one thread and all host cores)."""
+    """The oracle on bounded samples of a GEMV and a GEMM point (one thread and all host cores), as flat keys."""
     import numpy as np
 
     import oracle
@@ -493,11 +506,10 @@ def cpu_families(budget_s: float = 6.0) -> dict:
     flops = 2.0 * M * N * K
     f1, q1 = rate(lambda: oracle.c.gemm(a, w, threads=1), flops, budget_s * 0.4)
     fn_, qn = rate(lambda: oracle.c.gemm(a, w, threads=cores), flops, budget_s * 0.3)
-    return {"gemv_f16 4096x4096": {"value": round(g1 / 1e9, 3), "unit": "GB/s", "cores": 1, "passes": r1,
-                                   "all_cores": {"value": round(gn / 1e9, 3), "cores": cores, "passes": rn}},
-            "gemm_f16 N=K=4096": {"value": round(f1 / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "passes": q1,
-                                  "sample": f"{M} rows of A against the whole W (the oracle is row-parallel: the rate does not depend on M)",
-                                  "all_cores": {"value": round(fn_ / 1e12, 5), "cores": cores, "passes": qn}}}
+    return {"gemv_f16_4096x4096_gbs_1core": round(g1 / 1e9, 3), "gemv_f16_4096x4096_gbs_all_cores": round(gn / 1e9, 3),
+            "gemv_f16_4096x4096_passes": r1 + rn,
+            "gemm_f16_4096x4096_tflops_1core": round(f1 / 1e12, 5), "gemm_f16_4096x4096_tflops_all_cores": round(fn_ / 1e12, 5),
+            "gemm_f16_sample": f"{M} rows of A against the whole W, {q1 + qn} passes (the oracle is row-parallel: the rate does not depend on M)"}
 
 
 def recorded_traffic(workload_key: str):
@@ -620,15 +632,18 @@ def main() -> int:
         line["cpu_baseline"] = None
     if not args.no_sweep:
         rows = sweep(max(3, args.steps // 40), 1)
-        line["roofline"]["families"] = families(rows)
+        line["roofline"].update(families(rows))
         if line["cpu_baseline"] is not None:
-            line["cpu_baseline"]["families"] = cpu_families()
-        line["sweep"] = [{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
-                          if k in ("op", "n", "NK", "us", "gbs", "tflops", "bound", "frac")} for r in rows]
+            line["cpu_baseline"].update(cpu_families())
+        # the sweep rows go out as text lines ahead of the JSON line, which stays short enough to be read whole
+        for r in rows:
+            print("sweep " + json.dumps({k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()
+                                         if k in ("op", "n", "NK", "us", "gbs", "tflops", "bound", "frac")}))
+        line["config"]["sweep_rows"] = len(rows)
         if args.out:
             with open(args.out, "w") as f:
                 json.dump(rows, f, indent=1)
-    print(json.dumps(line))
+    print(json.dumps(line), flush=True)
     return 0
 
 

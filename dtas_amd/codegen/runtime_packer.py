@@ -259,6 +259,32 @@ class FunctionTable:
         expr = f"({a}/{div} * {s1} + {b}/{div})"
         return f"  int64_t index = {expr} > {last} ? {last} : {expr};\n"
 
+    def select_function_text(self, name: str) -> List[str]:
+        """C text of ``<name>_select(extents...)``: what select() does, for C callers of the generated
+        header -- the index statement behind a guard that returns NULL (the library sizes the launch
+        itself) for any extent above its upper bound, so both dispatchers run the same thing there."""
+        args = [a for a in self.dynamic_args[:2]]
+        if not args or not self.index_table or not self.call_table:
+            body = f"  return {'&' + name + '_call_table[0]' if self.call_table else '0'};"
+            return [f"static inline const dtas_config* {name}_select(void) {{", body, "}"]
+        params = ", ".join(f"int64_t {a}" for a in args)
+        guard = " || ".join(f"{a} > {self.upper_bound[a]}" for a in args if a in self.upper_bound)
+        lines = [f"static inline const dtas_config* {name}_select({params}) {{"]
+        if guard:
+            lines.append(f"  if ({guard}) return 0;  /* above the tuned range: cfg = NULL, the library's own choice */")
+        if len(args) == 2:   # each extent's bucket is clamped on its own before the two are combined
+            div = self.range_div_factor
+            sizes = [-(-self.upper_bound[a] // div) for a in args]
+            a, b = args
+            lines.append(f"  int64_t ia = {a}/{div} > {sizes[0] - 1} ? {sizes[0] - 1} : {a}/{div}, ib = {b}/{div} > {sizes[1] - 1} ? {sizes[1] - 1} : {b}/{div};")
+            last = len(self.index_table) - 1
+            lines.append(f"  int64_t index = ia * {sizes[1]} + ib > {last} ? {last} : ia * {sizes[1]} + ib;")
+        else:
+            lines.append(self.index_stmt().rstrip("\n"))
+        lines.append(f"  return &{name}_call_table[{name}_index_table[index]];")
+        lines.append("}")
+        return lines
+
     def select(self, values: Dict[str, int]) -> Optional[KernelEntryInfo]:
         """The row for these extents, or None where the library sizes the launch itself: a
         function without tuned rows, and any extent above its upper bound.  The reference runs the
@@ -362,8 +388,9 @@ class RuntimePacker:
 
     def header_text(self) -> str:
         out = ["/* Generated dispatcher tables (same information as dispatch_table.json) for C callers:",
-               " * index with the index statement, then pass &<func>_call_table[<func>_index_table[index]]",
-               " * as the `cfg` argument of the entry point in dtas_abi.h. */", '#include "dtas_abi.h"', ""]
+               " * <func>_select(extents) returns the row for these extents -- index with the index statement, then",
+               " * &<func>_call_table[<func>_index_table[index]] -- or NULL above the tuned range; pass it as the `cfg`",
+               " * argument of the entry point in dtas_abi.h. */", '#include "dtas_abi.h"', ""]
         for name, t in self.tables.items():
             rows = []
             for e in t.call_table:
@@ -376,6 +403,7 @@ class RuntimePacker:
             idx = ",".join(str(i) for i in t.index_table) or "0"
             out.append(f"static const int64_t {name}_index_table[] = {{{idx}}};")
             out.append(f"/* {t.index_stmt().strip()} */")
+            out += t.select_function_text(name)
             out.append("")
         return "\n".join(out)
 

@@ -1,0 +1,94 @@
+// The dynamic-n GEMMs on 8-bit weights (q8f16_1: four bytes to a word, an fp16 scale per 32 elements of a row):
+// fused_fused_decode2_fused_NT_matmul6_add4 and its fused-epilogue relatives
+// (experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py:371-502), C = epilogue(A . dequant(Wq)^T).
+// Few rows: the W-streaming kernel on the bytes (gemm_stream.hip).  Otherwise the tile kernel with the dequantiser in
+// its W path (template flag WQ, instantiated here), or the dequantiser into a library-owned fp16 buffer followed by
+// the fp16 GEMM.
+#include "gemm_tile_kernel.h"
+
+extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias, const void* res1,
+                                      const void* res2, void* C, int64_t M, int64_t N, int64_t K, int32_t epilogue,
+                                      const dtas_config* user, void* stream) {
+  using namespace dtas;
+  clear_error();
+  if (M < 0 || N < 0 || K < 0) return fail("gemm_q8: negative extent M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  if (K % 32 != 0) return fail("gemm_q8: K must be a multiple of the scale group, 32 (K=%lld)", (long long)K);
+  if (epilogue < DTAS_EPI_BIAS || epilogue > DTAS_EPI_BIAS_GELU) return fail("gemm_q8: unknown epilogue %d", epilogue);
+  if (M == 0 || N == 0) return 0;
+  if ((K != 0 && (M > INT64_MAX / 8 / K || N > INT64_MAX / 8 / K)) || M > INT64_MAX / 8 / N) return fail("gemm_q8: extents overflow");
+  const bool add2 = epilogue == DTAS_EPI_BIAS_ADD2 || epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32;
+  if (!A || !Wq || !scale || !C) {
+    if (K > 0 || !C) return fail("gemm_q8: NULL buffer");
+  }
+  if (add2 && (!res1 || !res2)) return fail("gemm_q8: epilogue %d needs both residuals", epilogue);
+  if (!add2 && (res1 || res2)) return fail("gemm_q8: epilogue %d takes no residuals", epilogue);
+  const int out_bytes = epilogue == DTAS_EPI_BIAS_ADD2_CAST_F32 ? 4 : 2;
+  if (overlaps(C, M * N * out_bytes, A, M * K * 2) || overlaps(C, M * N * out_bytes, Wq, N * K) ||
+      overlaps(C, M * N * out_bytes, scale, N * (K / 32) * 2) ||
+      (add2 && (overlaps(C, M * N * out_bytes, res1, M * N * 2) || overlaps(C, M * N * out_bytes, res2, M * N * 2))))
+    return fail("gemm_q8: output overlaps an input");
+  // one row with a plain or GELU epilogue is the dequantising GEMV
+  if (!user && M == 1 && (epilogue == DTAS_EPI_BIAS || epilogue == DTAS_EPI_BIAS_GELU))
+    return dtas_gemv_q8_f16(A, Wq, scale, bias, C, N, K, epilogue, nullptr, stream);
+  GemmEpilogue ep = {static_cast<const half_t*>(bias), static_cast<const half_t*>(res1), static_cast<const half_t*>(res2),
+                     epilogue, out_bytes == 4 ? 1 : 0, 0.f, 0, 0, 0, 0, 1, 0, static_cast<const half_t*>(scale)};
+  // Few rows of A: the launch is one read of the bytes of W.  The W-streaming kernel widens them on their way
+  // from the LDS into the MFMA (cfg: DTAS_GEMM_STREAM with tile 16x64x512, 16x64x1024 or 32x64x512).
+  {
+    const bool stream_ok = K > 0 && K % 256 == 0 && aligned(A, 16) && aligned(Wq, 16) && aligned(scale, 16) && K < (int64_t{1} << 24);
+    const half_t* a = static_cast<const half_t*>(A);
+    const half_t* w = static_cast<const half_t*>(Wq);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (user && user->variant == DTAS_GEMM_STREAM) {
+      const int bm = user->tile[0], bn = user->tile[1], bk = user->tile[2];
+      if (!((bm == 16 && bn == 64 && (bk == 512 || bk == 1024)) || ((bm == 32 || bm == 64) && bn == 64 && bk == 512)))
+        return fail("gemm_q8: the W-streaming kernel takes tiles 16x64x512, 16x64x1024, 32x64x512 and 64x64x512 for 8-bit weights, got %dx%dx%d", bm, bn, bk);
+      if (user->block != 256) return fail("gemm_q8: the 64-column streaming tile uses 256 threads, got %d", user->block);
+      if (M > bm) return fail("gemm_q8: a streaming tile of %d rows cannot hold M=%lld", bm, (long long)M);
+      if (!stream_ok) return fail("gemm_q8: the W-streaming kernel needs K %% 256 == 0 and 16-byte aligned A, W and scales");
+      return launch_gemm_stream_q8(bm, bk, s, a, w, ep, C, M, N, K);
+    }
+    if (!user && stream_ok && M <= 32) {
+      // measured at the model's shapes (M = 16: 10.1 against 25.6 us at 7680x2560, 14.9 against 92 at 2560x10240;
+      // M = 32: 14.0 against 26.3 and 20.5 against 33.8).  512-element slices (three workgroups per CU) unless K is
+      // long: from 16 slices on the hand-over of the partial sums costs more than the second workgroup hides
+      if (M > 16) return launch_gemm_stream_q8(32, 512, s, a, w, ep, C, M, N, K);
+      return launch_gemm_stream_q8(16, K >= 8192 ? 1024 : 512, s, a, w, ep, C, M, N, K);
+    }
+    // up to 64 rows (one workgroup per CU) only where the column tiles number at most a quarter of the CUs' slots:
+    // 14.0 against 26.3 us at 64 x 2560 x 2560 and 25.1 against 39.5 at 4096 x 4096, but 38 against 27 at N = 10240
+    if (!user && stream_ok && M <= 64 && N <= 4096 && K <= 4096) return launch_gemm_stream_q8(64, 512, s, a, w, ep, C, M, N, K);
+  }
+  // Two routes.  Dequantising in the W path of the GEMM (no intermediate) runs on a plain burst pipeline without
+  // split K: measured at the model's shapes it wins for M <= 64 with K <= 4096 (18 against 24 us at 7680x2560)
+  // and loses beyond (M = 2048: 109 against 84 us; K = 10240: 2x or more).  Otherwise: the dequantiser into a
+  // library-owned fp16 buffer, then the fp16 GEMM with everything its table offers.  A cfg selects the first route.
+  if (!user && !(M <= 64 && K <= 4096)) {
+    void* wbuf = nullptr;
+    std::lock_guard<std::recursive_mutex> ws_lock(g_ws_mutex);  // until both launches are enqueued
+    if (operand_workspace(static_cast<hipStream_t>(stream), static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
+    if (dtas_decode_q8_f16(Wq, scale, wbuf, N, K, nullptr, stream) != 0) return -1;
+    return dtas_gemm_f16_fused(A, wbuf, bias, res1, res2, C, M, N, K, epilogue, nullptr, stream);
+  }
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, 64, kBK}, 1, 0};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const half_t* a = static_cast<const half_t*>(A);
+  const half_t* w = static_cast<const half_t*>(Wq);  // (bytes; the kernels take the pointer as they take fp16 W)
+  const bool vec_ok = aligned(A, 16) && aligned(Wq, 16) && aligned(scale, 2) && N * K < (int64_t{1} << 32) && K > 0;
+  if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;
+  if (cfg.vec == 1) {
+    int64_t grid = ceil_div(M * N, 256);
+    grid = grid > 65536 ? 65536 : grid;
+    return launch_gemm_scalar("gemm_q8", static_cast<unsigned>(grid), 1, s, a, w, ep, C, M, N, K, false);
+  }
+  if (cfg.vec != 8) return fail("gemm_q8: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+  if (cfg.variant != DTAS_GEMM_MFMA) return fail("gemm_q8: only the MFMA kernels serve 8-bit weights");
+  if (cfg.split_k > 1) return fail("gemm_q8: K is not split for 8-bit weights");
+  int64_t la[7];
+  if (describe_gemm(M, N, K, cfg, la) != 0) return -1;
+  const int bm = cfg.tile[0], bn = cfg.tile[1];
+  if (bm == 256 && bn == 128 && cfg.unroll == 3) return launch_mfma<256, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, 1);
+  if (bm == 128 && bn == 128 && cfg.unroll == 3) return launch_mfma<128, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, 1);
+  if (bm == 64 && bn == 64 && cfg.unroll == 2) return launch_mfma<64, 64, 2, 2, 2, false, true>(s, a, w, ep, C, M, N, K, 1);
+  return fail("gemm_q8: 8-bit weights come with tiles 256x128 and 128x128 (three stages) and 64x64 (two), got %dx%d with %d", bm, bn, cfg.unroll);
+}

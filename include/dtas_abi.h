@@ -249,7 +249,20 @@ int dtas_gemv_f16_fused(const void* x, const void* W, const void* bias, const vo
 
 /* ---- GEMM: fused_NT_matmul4_add1 (before_dl.py:320-341) -------------------
  * C[M,N] = A[M,K] . W[N,K]^T (+ bias[N] when bias != NULL); M is the dynamic extent;
- * fp16 in/out, fp32 accumulate on MFMA. */
+ * fp16 in/out, fp32 accumulate on MFMA.
+ * Memory orderings a launch with K split over workgroups relies on (the partial tiles and arrival counters in the
+ * workspace are the only data of the library that one workgroup writes and another reads within a launch):
+ *  (1) a partial tile is written with device-scope (agent) relaxed atomic stores, which write through the XCD's L2;
+ *      the writing wavefront then waits until none of its stores is outstanding, and a write-through store is
+ *      acknowledged only once it is visible to every XCD;
+ *  (2) a workgroup barrier follows, and only then one thread adds 1 to the tile's counter with a device-scope
+ *      relaxed atomic read-modify-write, which is performed at the memory side, once, for all XCDs;
+ *  (3) the workgroup that reads nsplit - 1 there therefore knows that steps (1)-(2) of every other part are complete;
+ *      it reads the other parts' tiles with device-scope relaxed atomic loads, which do not hit in its own L2, adds
+ *      them in part order (the sum does not depend on who arrives last), and sets the counter back to 0.
+ *  No release/acquire fence is used (a device-scope fence writes back and invalidates a whole L2); the order rests on
+ *  (1)'s wait and on (2) following the barrier.  Launches that share a workspace must not overlap: the library keeps
+ *  one workspace per (device, stream). */
 int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N,
                   int64_t K, const dtas_config* cfg, void* stream);
 
@@ -264,7 +277,9 @@ int dtas_gemm_f16(const void* A, const void* W, const void* bias, void* C, int64
  * holds returns -1 and says how much (pass a cfg with split_k = 1, or a smaller split).  All calls on one GPU share
  * the array, whatever their streams: calls that overlap in time on one GPU race -- order them (one stream, or
  * events).  dtas_init() resolves the array's address on the current device; otherwise the first call on a
- * device does. */
+ * device does, which asks the runtime for a symbol address: a call under stream capture therefore requires that
+ * dtas_init() (or an uncaptured call) has run on that device before.  The counters are never cleared by a call:
+ * the array is zero when the library's code is loaded and every launch leaves its counters at zero. */
 #define DTAS_STATIC_SCRATCH_PARTIAL_BYTES (32u << 20)
 #define DTAS_STATIC_SCRATCH_COUNTERS 4096u
 int dtas_gemm_f16_static(const void* A, const void* W, const void* bias, void* C, int64_t M, int64_t N,

@@ -113,6 +113,14 @@ def test_argument_errors_return_minus_one_with_a_message():
     assert "unknown op" in _lib.last_error()
 
 
+def test_attn_scores_with_an_empty_head_dimension_fails_before_any_division():
+    # d = 0 passes the d % 8 check; the row kernel's launch shape divides by d / 8, so it must be refused first
+    fake_q, fake_k, fake_m, fake_o = 0x10000, 0x20000000, 0x30000000, 0x40000000   # never dereferenced
+    cfg = _lib.DtasConfig.from_dict({"variant": _lib.GEMM_SKINNY, "block": 1024, "vec": 8, "unroll": 1, "tile": [1, 8, 0], "split_k": 1})
+    assert _call("dtas_attn_scores_f16_f32", fake_q, fake_k, fake_m, fake_o, 1, 1, 8, 0, 0.1, ctypes.byref(cfg), None) == -1
+    assert "head dimensions from 8" in _lib.last_error()
+
+
 def test_empty_extent_is_a_successful_no_op():
     assert _call("dtas_add_f16", None, None, None, 0, 4096, None, None) == 0
     assert _lib.last_error() == ""            # a success clears the previous message

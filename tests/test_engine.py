@@ -101,6 +101,43 @@ def test_past_the_upper_bound_the_library_sizes_the_launch(tmp_path):
                 assert info.launch_args[0] >= 1 and info.launch_args[3] >= 64
 
 
+def test_generated_header_and_python_dispatcher_agree_also_past_the_upper_bound(tmp_path):
+    """The C text written beside the tables (<func>_select) and FunctionTable.select() choose the same row for the
+    same extents, and both hand extents above the upper bound to the library (NULL / None)."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("needs gcc")
+    rt = Engine(3, work_dir=str(tmp_path)).tune_module(_module(), MI355X(), 256)
+    probes = {1: [1, 255, 256, 257, 1024, 4095, 4096, 4097, 40000],
+              2: [(1, 1), (300, 511), (4096, 512), (4096, 1), (4097, 5), (17, 513), (9000, 9000)]}
+    cases, body = [], []
+    for name, table in rt.tables.items():
+        args = table.dynamic_args[:2]
+        if not args or not table.index_table:
+            continue
+        for probe in probes[len(args)]:
+            vals = (probe,) if len(args) == 1 else probe
+            cases.append((name, table, dict(zip(args, vals))))
+            call = f"{name}_select({', '.join(str(v) for v in vals)})"
+            body.append(f'  printf("%ld\\n", {call} ? (long)({call} - {name}_call_table) : -1L);')
+    assert len(cases) > 30
+    src = tmp_path / "sel.c"
+    src.write_text('#include <stdio.h>\n#include "dispatch_tables.h"\nint main(void) {\n' + "\n".join(body) + "\n  return 0;\n}\n")
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    exe = tmp_path / "sel"
+    subprocess.check_call([gcc, "-std=c99", "-Wall", "-Wno-unused-function", "-Wno-unused-const-variable", "-Werror", "-I", include, "-I", str(tmp_path), str(src), "-o", str(exe)])
+    got = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
+    for (name, table, values), row in zip(cases, got):
+        entry = table.select(values)
+        want = -1 if entry is None else table.call_table.index(entry)
+        assert row == want, (name, values, row, want)
+        beyond = any(values[a] > table.upper_bound[a] for a in values)
+        assert (want == -1) == beyond, (name, values)
+
+
 def test_merge_two_dynamic_extents(tmp_path):
     from dtas_amd.codegen.compile_result import CompileResult
     from dtas_amd.common.config import ReductionConfig

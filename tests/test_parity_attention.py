@@ -99,6 +99,23 @@ def test_scores_errors():
     assert _lib.lib().dtas_attn_scores_f16_f32(None, None, None, None, 0, 0, 0, 80, SCALE, None, None) == 0   # empty: no-op
 
 
+def test_scores_with_an_empty_head_dimension():
+    # d = 0: every product is an empty sum, so out = min(max(0, -65504), mask); one query row reaches the built-in
+    # choice that takes the row kernel for d >= 8 (its launch shape divides by d / 8)
+    for n, m in ((1, 40), (3, 4096), (70, 33)):
+        rng = np.random.default_rng(n)
+        mask = np.where(rng.random((n, m)) < 0.5, 65504.0, -65504.0).astype(np.float16)
+        dummy = torch.zeros(8, dtype=torch.float16, device="cuda")
+        out = torch.full((2, n, m), 7.0, dtype=torch.float32, device="cuda")
+        mask_d = dev(mask)
+        rc = _lib.lib().dtas_attn_scores_f16_f32(dummy.data_ptr(), dummy.data_ptr(), mask_d.data_ptr(), out.data_ptr(), 2, n, m, 0,
+                                                 SCALE, None, None)
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        want = np.minimum(np.float32(0), mask.astype(np.float32))
+        assert np.array_equal(out.cpu().numpy(), np.broadcast_to(want, (2, n, m)))
+
+
 def test_scores_through_the_primfunc_descriptor(oracle):
     from dtas_amd import primfuncs as pf
     from dtas_amd.codegen.runtime_packer import bind_extents, call_primfunc

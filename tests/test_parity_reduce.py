@@ -113,11 +113,14 @@ def test_softmax_f16_benchmark_config(oracle, n):
     assert np.abs(got.astype(np.float64).sum(-1) - 1).max() < n * 2.0 ** -11 + 1e-3
 
 
-@pytest.mark.parametrize("n", [2048, 4096])
+@pytest.mark.parametrize("n", [2048, 4096, 8192])
 def test_softmax_f16_large_rows_sampled(oracle, n):
-    # [32n, n] is up to 1 GiB: run all of it, compare sampled rows with the oracle, row sums for all
+    # [32n, n] is 1 GiB at n = 4096 and 4 GiB at 8192, the far end of the dynamic range: run all of it, compare
+    # sampled rows with the oracle, row sums for all
     g = torch.Generator(device="cuda").manual_seed(4)
-    x = (torch.randn(32 * n, n, device="cuda", generator=g) * 2).half()
+    x = torch.empty(32 * n, n, dtype=torch.float16, device="cuda")
+    for r0 in range(0, 32 * n, 32768):     # in slabs: the fp32 draw of the whole tensor would be 8 GiB at n = 8192
+        x[r0:r0 + 32768] = (torch.randn(min(32768, 32 * n - r0), n, device="cuda", generator=g) * 2).half()
     out = torch.empty_like(x)
     ops.softmax(x, out)
     torch.cuda.synchronize()
@@ -125,7 +128,7 @@ def test_softmax_f16_large_rows_sampled(oracle, n):
     xs = x[torch.from_numpy(rows).cuda()].cpu().numpy()
     got = out[torch.from_numpy(rows).cuda()].cpu().numpy()
     _check(got, oracle.c.softmax(xs), oracle.np64.softmax(xs))
-    sums = out.float().sum(-1)
+    sums = torch.cat([out[r0:r0 + 32768].float().sum(-1) for r0 in range(0, 32 * n, 32768)])
     assert float((sums - 1).abs().max()) < n * 2.0 ** -11 + 1e-3
     assert bool((out.argmax(-1) == x.argmax(-1)).float().mean() > 0.999)  # ties in fp16 aside
 

@@ -77,3 +77,52 @@ def test_static_scratch_gemm_refuses_what_the_array_cannot_hold():
     wide_w = torch.zeros(8192, 1024, dtype=torch.float16, device="cuda")
     rc = L.dtas_gemm_f16_static(big_a.data_ptr(), wide_w.data_ptr(), None, out2.data_ptr(), M, 8192, 1024, ctypes.byref(c64), None)
     assert rc == -1 and "counters" in _lib.last_error()
+
+
+def test_static_scratch_gemm_on_the_w_streaming_kernel():
+    L = _lib.lib()
+    # 16 rows against 4096 x 4096: the built-in row is the W-streaming kernel, whose K slices meet in the scratch as well
+    small = _problem(16, 4096, 4096, 5)
+    assert _lib.select_bucket(_lib.OP_GEMM_F16, 16, 4096, 4096).config.variant == _lib.GEMM_STREAM
+    assert_bits_equal(_run(L.dtas_gemm_f16_static, *small, None), _run(L.dtas_gemm_f16, *small, None))
+
+
+def test_static_scratch_gemm_allocates_no_device_memory():
+    L = _lib.lib()
+    assert L.dtas_init() == 0, _lib.last_error()
+    a, w, bias = _problem(96, 4096, 4096, 6)
+    out = torch.empty(96, 4096, dtype=torch.float16, device="cuda")
+    fresh = torch.cuda.Stream()          # a stream that owns no workspace yet
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    rc = L.dtas_gemm_f16_static(a.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), 96, 4096, 4096, None, fresh.cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "the static entry point changed the device's free memory"
+    # the same launch through the allocating entry point on that stream takes its 32 MiB workspace: the check above can see one
+    rc = L.dtas_gemm_f16(a.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), 96, 4096, 4096, None, fresh.cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert free0 - torch.cuda.mem_get_info()[0] >= 32 << 20
+
+
+def test_static_scratch_gemm_under_stream_capture_replays_the_same_bits():
+    L = _lib.lib()
+    assert L.dtas_init() == 0, _lib.last_error()   # resolves the scratch address: required before a captured call
+    a, w, bias = _problem(96, 4096, 4096, 7)
+    eager = _run(L.dtas_gemm_f16_static, a, w, bias, None)
+    out = torch.zeros(96, 4096, dtype=torch.float16, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        rc = L.dtas_gemm_f16_static(a.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), 96, 4096, 4096, None,
+                                    torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    other = _problem(40, 1000, 2048, 8)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(out.cpu().numpy(), eager)
+        # eager work on the same scratch between the replays
+        _run(L.dtas_gemm_f16_static, *other, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=3, tile=[128, 128, 64], split_k=3))
