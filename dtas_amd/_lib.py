@@ -22,7 +22,7 @@ ABI_VERSION = 1
 ELT_VECTOR, ELT_SCALAR = 0, 1
 RED_WAVE_ROW, RED_BLOCK_ROW, RED_STREAM_ROW = 0, 1, 2
 GEMV_SPLITK, GEMV_RF16 = 0, 1
-GEMM_MFMA, GEMM_SKINNY, GEMM_ROWS, GEMM_STREAM = 0, 1, 2, 3
+GEMM_MFMA, GEMM_SKINNY, GEMM_ROWS, GEMM_STREAM, GEMM_MFMA_ACC16 = 0, 1, 2, 3, 4
 # enum dtas_epilogue
 EPI_BIAS, EPI_BIAS_ADD2, EPI_BIAS_ADD2_CAST_F32, EPI_BIAS_GELU = 0, 1, 2, 3
 

@@ -8,7 +8,18 @@ from . import _lib
 
 PACKED_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libdtas_packed.so")
 FUNCTIONS = ("add", "copy", "cast", "fused_layer_norm_cast1", "fused_softmax_cast", "fused_NT_matmul4_add1",
-             "fused_NT_matmul10_add5")
+             "fused_NT_matmul10_add5", "fused_NT_matmul_add", "fused_NT_matmul6_add4",
+             # the fused-epilogue GEMMs (prefill and decode names)
+             "fused_NT_matmul2_add1_add3_add3", "fused_NT_matmul2_add1_add3_add3_cast", "fused_NT_matmul3_add2_gelu",
+             "fused_NT_matmul8_add5_add7_add7", "fused_NT_matmul8_add5_add7_add7_cast5", "fused_NT_matmul9_add6_gelu1",
+             # attention: scores and P.V, under the names of both model files
+             "fused_NT_matmul1_divide_maximum_minimum_cast2", "fused_NT_matmul7_divide1_maximum1_minimum1_cast7",
+             "fused_NT_matmul1_divide1_maximum_minimum_cast2", "fused_NT_matmul7_divide2_maximum1_minimum1_cast7",
+             "matmul8", "matmul10", "matmul9", "matmul1",
+             # 8-bit weights
+             "fused_fused_decode2_fused_NT_matmul_add", "fused_fused_decode2_fused_NT_matmul6_add4",
+             "fused_fused_decode4_fused_NT_matmul3_add2_gelu", "fused_fused_decode4_fused_NT_matmul9_add6_gelu1",
+             "fused_fused_decode5_fused_NT_matmul4_add1", "fused_fused_decode5_fused_NT_matmul10_add5")
 TCODE_OPAQUE_HANDLE, TCODE_NULLPTR, TCODE_DLTENSOR_HANDLE, TCODE_NDARRAY_HANDLE = 3, 4, 7, 13
 KDLCUDA, KDLROCM = 2, 10
 
@@ -31,7 +42,7 @@ class TVMValue(ctypes.Union):
     _fields_ = [("v_int64", ctypes.c_int64), ("v_float64", ctypes.c_double), ("v_handle", ctypes.c_void_p)]
 
 
-DTYPES = {"float16": (2, 16), "float32": (2, 32), "int8": (0, 8), "int32": (0, 32), "float64": (2, 64)}
+DTYPES = {"float16": (2, 16), "float32": (2, 32), "int8": (0, 8), "int32": (0, 32), "uint32": (1, 32), "float64": (2, 64)}
 _handle = None
 
 

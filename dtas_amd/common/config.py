@@ -242,6 +242,9 @@ class MFMAConfig(Config):
         self.block_threads = 256
         self.stages = 0          # LDS stages of the load pipeline (0 = as many as the tile allows)
         self.split_k = 1         # workgroups that share a tile and split its K extent
+        # the reference's scheduled arithmetic: an fp16 accumulator rounded once per k step of 16 (its wmma 16x16x16
+        # fragments with a float16 accumulator, experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py:19,37)
+        self.acc_f16 = False
         self.in_vec_len_a = 8
         self.in_vec_len_b = 8
         self.swizzle = True
@@ -265,7 +268,7 @@ class MFMAConfig(Config):
                 "mfma_shape": (self.mfma_m, self.mfma_n, self.mfma_k), "i": self.i, "j": self.j,
                 "micro_shape": (self.micro_shape_x, self.micro_shape_y, self.micro_shape_k),
                 "skinny": self.skinny, "stream": self.stream, "block_threads": self.block_threads, "stages": self.stages,
-                "split_k": self.split_k, "in_vec_len_a": self.in_vec_len_a, "in_vec_len_b": self.in_vec_len_b}
+                "split_k": self.split_k, "acc_f16": self.acc_f16, "in_vec_len_a": self.in_vec_len_a, "in_vec_len_b": self.in_vec_len_b}
 
     def from_dict(self, dic: Dict) -> "MFMAConfig":
         self.__init__()
@@ -277,10 +280,15 @@ class MFMAConfig(Config):
         self.block_threads = dic.get("block_threads", 256)
         self.stages = dic.get("stages", 0)
         self.split_k = dic.get("split_k", 1)
+        self.acc_f16 = dic.get("acc_f16", False)
         return self
 
     def to_abi(self):
         c = _lib.DtasConfig()
+        if self.acc_f16:   # one kernel shape: 64x64 per workgroup, a k step of 16 per instruction
+            c.variant, c.block, c.vec, c.unroll, c.split_k = _lib.GEMM_MFMA_ACC16, 256, 8, 1, 1
+            c.tile[0], c.tile[1], c.tile[2] = 64, 64, 16
+            return c
         c.variant = _lib.GEMM_SKINNY if self.skinny else _lib.GEMM_STREAM if self.stream else _lib.GEMM_MFMA
         c.block, c.vec = self.block_threads, 8
         c.unroll = 4 if self.skinny else 1 if self.stream else self.stages

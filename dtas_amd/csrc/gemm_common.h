@@ -71,6 +71,9 @@ int launch_gemm_stream(const dtas_config& cfg, hipStream_t s, const half_t* A, c
 // 8-bit W (bytes [N][K], scales in ep.wscale): rows of A in {16, 32, 64}, K slices of 512 or 1024 (16 rows only)
 int launch_gemm_stream_q8(int rows_a, int k_slice, hipStream_t s, const half_t* A, const half_t* Wq, const GemmEpilogue& ep, void* C,
                           int64_t M, int64_t N, int64_t K);
+// DTAS_GEMM_MFMA_ACC16: the accumulator rounded to fp16 after every k step of 16 (cfg.vec 8: 16-byte operand loads, else elements)
+int launch_gemm_acc16(const dtas_config& cfg, hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C,
+                      int64_t M, int64_t N, int64_t K);
 // one thread per element of C: any K and alignment; grid.y = batch; w_kmajor: W is [K][N]; ep.wscale set: 8-bit W
 int launch_gemm_scalar(const char* what, unsigned grid_x, unsigned batch, hipStream_t s, const half_t* A, const half_t* W,
                        const GemmEpilogue& ep, void* C, int64_t M, int64_t N, int64_t K, bool w_kmajor);

@@ -8,7 +8,8 @@
 //              (4096 < N <= 16384, K <= 4096) the looping form: a workgroup keeps its columns over the whole of K,
 //              walked through a ring of LDS stages.
 // ROWS kernel (M <= 4; the built-in choice for M = 2): W streamed in whole rows on the vector ALU.
-// The element-access kernel (any K and alignment; k-major or 8-bit W as well) is here too.
+// The element-access kernel (any K and alignment; k-major or 8-bit W as well) is here too, and the kernel that keeps
+// the reference's fp16 accumulator (DTAS_GEMM_MFMA_ACC16).
 // Replaces, for these shapes, the kernels DTAS's WMMA rule generates (python/dtas/schedule/tir_wmma.py:20-222), which
 // pad M up to a whole tile.
 #include "gemm_common.h"
@@ -525,6 +526,57 @@ __global__ void __launch_bounds__(256) gemm_scalar_kernel(const half_t* __restri
   }
 }
 
+// The reference's scheduled GEMM arithmetic (DTAS_GEMM_MFMA_ACC16): its WMMA rule keeps the accumulator fragment in fp16
+// and updates it with one 16x16x16 tensor-core instruction per k step (python/dtas/schedule/tir_wmma.py:20-222; the
+// generated kernel experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py:19,37).  Here a k step of 16 is
+// one v_mfma_f32_32x32x16_f16 whose sums are rounded to fp16 (and widened again) before the next step reads them, so
+// every step's 16 products meet the accumulator at fp32 precision and the result is rounded once per step.
+// Workgroup = 64 x 64 of C, a wavefront 32 x 32; lane l supplies row (l & 31), elements 8 * (l >> 5) .. + 8 of the
+// step for both operands, straight from global memory (W rows are the first MFMA operand: accumulator register 4 g + e
+// of lane l is C row l & 31, column 8 g + 4 (l >> 5) + e).  Nothing is pipelined: a step waits for its rounding.
+template <bool VEC>
+__global__ void __launch_bounds__(256) gemm_acc16_kernel(const half_t* __restrict__ A, const half_t* __restrict__ W, GemmEpilogue ep,
+                                                         void* __restrict__ C, int64_t M, int64_t N, int64_t K, unsigned tiles_n) {
+  const unsigned t = threadIdx.x, l = t & 63u, wv = t >> 6;
+  const int64_t m0 = static_cast<int64_t>(blockIdx.x / tiles_n) * 64 + (wv >> 1) * 32;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x % tiles_n) * 64 + (wv & 1u) * 32;
+  if (m0 >= M || n0 >= N) return;  // (no barrier below: a wavefront without work just leaves)
+  const int64_t arow = m0 + (l & 31u) < M ? m0 + (l & 31u) : M - 1;  // clamped rows are computed and never stored
+  const int64_t wrow = n0 + (l & 31u) < N ? n0 + (l & 31u) : N - 1;
+  const half_t* ap = A + arow * K + 8 * (l >> 5);
+  const half_t* wp = W + wrow * K + 8 * (l >> 5);
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  for (int64_t k0 = 0; k0 < K; k0 += 16) {
+    const int64_t k = k0 + 8 * (l >> 5);
+    f16x8 fa, fw;
+    if (VEC) {  // K % 8 == 0: a lane's 8 elements are all inside the row or all past its end
+      const f16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+      fa = k < K ? *reinterpret_cast<const f16x8*>(ap + k0) : zero;
+      fw = k < K ? *reinterpret_cast<const f16x8*>(wp + k0) : zero;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        fa[e] = k + e < K ? ap[k0 + e] : static_cast<half_t>(0.f);
+        fw[e] = k + e < K ? wp[k0 + e] : static_cast<half_t>(0.f);
+      }
+    }
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw, fa, acc, 0, 0, 0);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = static_cast<float>(static_cast<half_t>(acc[v]));
+  }
+  const int64_t row = m0 + (l & 31u);
+  if (row >= M) return;
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int64_t col = n0 + 8 * g + 4 * (l >> 5) + e;
+      if (col < N) finish(acc[4 * g + e], ep, C, row, col, N);
+    }
+}
+
 // The W-streaming kernel: 16 * WAVES columns and SEG * 512 elements of K per workgroup, K slices met in the workspace.
 template <int MT, int SEG, int WAVES, bool Q8 = false>
 int launch_stream(hipStream_t s, const half_t* A, const half_t* W, const GemmEpilogue& ep, void* C, int64_t M, int64_t N, int64_t K) {
@@ -599,6 +651,16 @@ int launch_gemm_stream_q8(int rows_a, int k_slice, hipStream_t s, const half_t* 
   if (rows_a == 16 && k_slice == 512) return launch_stream<1, 1, 4, true>(s, a, wq, ep, C, M, N, K);
   if (rows_a == 16 && k_slice == 1024) return launch_stream<1, 2, 4, true>(s, a, wq, ep, C, M, N, K);
   return fail("gemm_q8: no W-streaming kernel for %d rows and K slices of %d", rows_a, k_slice);
+}
+
+int launch_gemm_acc16(const dtas_config& cfg, hipStream_t s, const half_t* a, const half_t* w, const GemmEpilogue& ep, void* C,
+                      int64_t M, int64_t N, int64_t K) {
+  const int64_t tm = ceil_div(M, 64), tn = ceil_div(N, 64);
+  if (tm * tn > 0x7fffffff || tn > 0x7fffffff) return fail("gemm: too many workgroups");
+  const dim3 grid(static_cast<unsigned>(tm * tn)), block(256);
+  if (cfg.vec == 8) hipLaunchKernelGGL(gemm_acc16_kernel<true>, grid, block, 0, s, a, w, ep, C, M, N, K, static_cast<unsigned>(tn));
+  else hipLaunchKernelGGL(gemm_acc16_kernel<false>, grid, block, 0, s, a, w, ep, C, M, N, K, static_cast<unsigned>(tn));
+  return check_launch("gemm");
 }
 
 int launch_gemm_scalar(const char* what, unsigned grid_x, unsigned batch, hipStream_t s, const half_t* a, const half_t* w,

@@ -84,6 +84,19 @@ void tail_split_256(int64_t M, int64_t N, int64_t K, int* nsplit, unsigned* unsp
 int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64_t la[7]) {
   for (int i = 0; i < 7; ++i) la[i] = 0;
   la[1] = la[2] = 1;
+  if (cfg.variant == DTAS_GEMM_MFMA_ACC16) {  // the reference's fp16 accumulator, rounded once per k step of 16
+    if (cfg.tile[0] != 64 || cfg.tile[1] != 64 || cfg.tile[2] != 16) return fail("gemm: the fp16-accumulator kernel takes tile 64x64x16, got %dx%dx%d", cfg.tile[0], cfg.tile[1], cfg.tile[2]);
+    if (cfg.block != 256) return fail("gemm: the fp16-accumulator kernel uses 256 threads, got %d", cfg.block);
+    if (cfg.vec != 8 && cfg.vec != 1) return fail("gemm: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
+    if (cfg.split_k > 1) return fail("gemm: the fp16 accumulator is rounded step by step along K: K cannot be split (split_k = %d)", cfg.split_k);
+    const int64_t tm = ceil_div(M, 64), tn = ceil_div(N, 64);
+    if (tm * tn > 0x7fffffff) return fail("gemm: too many tiles");
+    la[0] = tm * tn;
+    la[3] = 256;
+    la[5] = tm;
+    la[6] = tn;
+    return 0;
+  }
   if (cfg.vec == 1) {  // element-access fallback
     int64_t grid = ceil_div(M * N, 256);
     la[0] = grid > 65536 ? 65536 : (grid < 1 ? 1 : grid);
@@ -282,6 +295,7 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   const half_t* w = static_cast<const half_t*>(W);
   const GemmEpilogue& b = ep;
   void* c = C;
+  if (cfg.variant == DTAS_GEMM_MFMA_ACC16) return launch_gemm_acc16(cfg, s, a, w, b, c, M, N, K);
   if (cfg.vec == 1) return launch_gemm_scalar("gemm", static_cast<unsigned>(la[0]), 1, s, a, w, b, c, M, N, K, false);
   if (cfg.variant == DTAS_GEMM_ROWS) return launch_gemm_rows(cfg, la, s, a, w, b, c, M, N, K);
   if (cfg.variant == DTAS_GEMM_SKINNY) return launch_gemm_skinny(cfg, la, s, a, w, b, c, M, N, K);

@@ -102,13 +102,20 @@ enum dtas_variant {
   DTAS_GEMM_SKINNY = 1,   /* small M: weight-streaming MFMA 16x16x32, split over N and K */
   DTAS_GEMM_ROWS = 2,     /* M <= 4: W streamed once in whole rows (tile[1] per wavefront) against tile[0] >= M
                              rows of A on the vector ALU; tile = {2|4, 1|2|4, 8}, block 64 / 128 / 256 */
-  DTAS_GEMM_STREAM = 3    /* M <= tile[0] in {16, 32, 64}: W streamed once, 1 KiB of a row per access, through the LDS to
+  DTAS_GEMM_STREAM = 3,   /* M <= tile[0] in {16, 32, 64}: W streamed once, 1 KiB of a row per access, through the LDS to
                              MFMA 16x16x32; a workgroup of tile[1] / 16 wavefronts owns tile[1] in {64, 128} columns and
                              tile[2] in {512, 1024} elements of K, the K slices are added up in the workspace;
                              (tile[0] + tile[1]) * tile[2] * 2 bytes of LDS, block = 4 * tile[1].
                              tile[2] = 256 is the looping form for a W with many rows: tile = {16, 16 | 64, 256}, a
                              workgroup owns its columns over the whole of K and walks it in segments of 256 through a
                              ring of four LDS stages; no workspace */
+  DTAS_GEMM_MFMA_ACC16 = 4 /* the reference's scheduled arithmetic: an fp16 accumulator updated once per k step of 16 by one
+                             matrix-core instruction, as its wmma 16x16x16 kernels with a float16 "wmma.accumulator" do
+                             (experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py:19,37): the 16 products
+                             of a step are added to the accumulator at fp32 precision and the sum is rounded to fp16 before
+                             the next step.  tile = {64, 64, 16}, block 256, vec 8 or 1, split_k 1 (the rounding order
+                             admits no K split); any M; never the built-in choice.  A mode for comparing against the
+                             reference's own numbers, not for speed: every step waits for its rounding */
 };
 
 /* One row of a call table: the launch-relevant part of the reference's *Config classes

@@ -82,6 +82,51 @@ int32_t fused_softmax_cast(void* args, int32_t* arg_type_ids, int32_t num_args, 
  * (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py:320-341); fused_NT_matmul10_add5: the same with n = 1 (:96-113) */
 int32_t fused_NT_matmul4_add1(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
 int32_t fused_NT_matmul10_add5(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+/* the same PrimFunc under the names the model graphs use for the 7680 x 2560 projection: dynamic n (:552-572) and n = 1 (:343-360) */
+int32_t fused_NT_matmul_add(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul6_add4(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+
+/* ---- the fused-epilogue GEMMs of the model graph (experiment/ModelIR/dolly-v2-3b-q0f16/before_dl.py); every step an fp16
+ * tensor, as dtas_gemm_f16_fused spells them.  n is read from the shapes: the prefill form (dynamic n) and the decode form
+ * (n = 1; the 8-bit model's graph swaps the two names) of a PrimFunc are one function.
+ * fused_NT_matmul2_add1_add3_add3(lv (1, n, K), W (N, K), bias (N), res1 (1, n, N), res2 (1, n, N), out (1, n, N)) (:163-200),
+ * .._cast: the same with a float32 output (:202-246); decode names fused_NT_matmul8_add5_add7_add7 (:408-439), .._cast5 (:442-480).
+ * fused_NT_matmul3_add2_gelu(lv (1, n, K), W (N, K), bias (N), out (1, n, N)) (:248-318); decode name fused_NT_matmul9_add6_gelu1 (:483-549). */
+int32_t fused_NT_matmul2_add1_add3_add3(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul2_add1_add3_add3_cast(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul3_add2_gelu(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul8_add5_add7_add7(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul8_add5_add7_add7_cast5(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul9_add6_gelu1(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+
+/* ---- the two batched attention matmuls.
+ * fused_NT_matmul1_divide_maximum_minimum_cast2(q (1, H, n, d), k (1, H, m, d), mask (1, 1, n, m), out (1, H, n, m) float32)
+ * (:116-160; n and m dynamic; the product is multiplied by the fp16 constant 1 / sqrt(d), 0.1118 for d = 80, clamped at -65504 and
+ * cut by the mask); decode name fused_NT_matmul7_divide1_maximum1_minimum1_cast7 (:363-406); in the 8-bit model's file
+ * (dolly-v2-3b-q8f16_1/before_dl.py:83-126, :203-248) the same two are fused_NT_matmul1_divide1_maximum_minimum_cast2 and
+ * fused_NT_matmul7_divide2_maximum1_minimum1_cast7.
+ * matmul8(A (1, H, n, m), B (1, H, m, d), out (1, H, n, d)) (:915-929) and matmul10, its n = 1 form (:899-912); matmul9 / matmul1 in
+ * the 8-bit model's file (:1000-1015, :984-998). */
+int32_t fused_NT_matmul1_divide_maximum_minimum_cast2(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul7_divide1_maximum1_minimum1_cast7(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul1_divide1_maximum_minimum_cast2(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_NT_matmul7_divide2_maximum1_minimum1_cast7(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t matmul8(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t matmul10(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t matmul9(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t matmul1(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+
+/* ---- GEMMs on 8-bit weights (experiment/ModelIR/dolly-v2-3b-q8f16_1/before_dl.py): W = (fp16(byte) - 127) * scale, four bytes to
+ * a uint32 word, an fp16 scale per 32 elements of a row; parameter order (Wq (N, K/4) uint32, scale (N, K/32), lv (1, n, K), bias (N),
+ * out (1, n, N)).  fused_fused_decode2_fused_NT_matmul_add (:401-426, n = 1) / .._matmul6_add4 (:371-399, dynamic n);
+ * fused_fused_decode4_fused_NT_matmul3_add2_gelu (:428-502, n = 1) / .._matmul9_add6_gelu1 (:504-581, dynamic n);
+ * fused_fused_decode5_fused_NT_matmul4_add1 (:613-638, n = 1) / .._matmul10_add5 (:583-611, dynamic n). */
+int32_t fused_fused_decode2_fused_NT_matmul_add(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_fused_decode2_fused_NT_matmul6_add4(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_fused_decode4_fused_NT_matmul3_add2_gelu(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_fused_decode4_fused_NT_matmul9_add6_gelu1(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_fused_decode5_fused_NT_matmul4_add1(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
+int32_t fused_fused_decode5_fused_NT_matmul10_add5(void* args, int32_t* arg_type_ids, int32_t num_args, void* out_ret_value, int32_t* out_ret_tcode, void* resource_handle);
 
 /* TVM enqueues on the calling thread's current stream; this sets that stream (a hipStream_t, NULL = the default
  * stream) for the calls the calling host thread makes through the functions above. */

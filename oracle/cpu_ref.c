@@ -276,10 +276,27 @@ void oracle_softmax_f16_f16(const f16* x, f16* out, int64_t rows, int64_t cols, 
  *              fp32-accumulate contract of the benchmark configs.
  * acc_f16 = 1: the PrimFunc text literally: the running sum is an fp16 buffer,
  *              acc = f16(acc + f16(a*w)) for k ascending.
+ * acc_f16 = 2: the reference's scheduled GEMM: an fp16 accumulator fragment updated once per k step of 16 by
+ *              one tensor-core instruction (wmma 16x16x16 with "wmma.accumulator" in float16,
+ *              experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py:19,37): the 16 exact products
+ *              of a step are added to the accumulator at fp32 precision (k ascending here; the order inside
+ *              the instruction is not part of any interface) and the result is rounded to fp16 once per step.
  * Pinned by: fp64 numpy A @ W.T (rtol 1e-2), exact cases (K = 1, identity /
  * permutation W, one-hot rows), brute force on tiny ragged shapes,
  * torch.matmul on CPU.
  * ======================================================================== */
+/* One element's product with an fp16 accumulator rounded once per k step of 16 (acc_f16 = 2). */
+static f16 dot_f16_k16(const f16* a, const f16* w, int64_t K) {
+  f16 acc = 0;
+  for (int64_t k0 = 0; k0 < K; k0 += 16) {
+    float s = h2f(acc);
+    const int64_t k1 = k0 + 16 < K ? k0 + 16 : K;
+    for (int64_t k = k0; k < k1; ++k) s = s + h2f(a[k]) * h2f(w[k]);
+    acc = f2h(s);
+  }
+  return acc;
+}
+
 void oracle_gemm_f16(const f16* A, const f16* W, const f16* bias, f16* C, int64_t M, int64_t N,
                      int64_t K, int acc_f16, int nthreads) {
   OMP_FOR(nthreads)
@@ -288,7 +305,9 @@ void oracle_gemm_f16(const f16* A, const f16* W, const f16* bias, f16* C, int64_
     const f16* a = A + i * K;
     const f16* w = W + j * K;
     f16 r;
-    if (acc_f16) {
+    if (acc_f16 == 2) {
+      r = dot_f16_k16(a, w, K);
+    } else if (acc_f16) {
       f16 acc = 0;
       for (int64_t k = 0; k < K; ++k) acc = f2h(h2f(acc) + h2f(f2h(h2f(a[k]) * h2f(w[k]))));
       r = acc;
@@ -363,7 +382,8 @@ void oracle_gemm_f16_f32out(const f16* A, const f16* W, float* C, int64_t M, int
  *   kind 1: C = (res1 + (mm + bias)) + res2              fp16 out
  *   kind 2: the same, T.Cast("float32")                  fp32 out
  *   kind 3: t = mm + bias; C = t * (0.5 + f16(f16(erf(f32(f16(t * f16(0.70710678...))))) * 0.5))
- * mm is the fp32-accumulated product rounded once (acc_f16 = 1: the literal fp16 running sum).
+ * mm is the fp32-accumulated product rounded once (acc_f16 = 1: the literal fp16 running sum; 2: an fp16
+ * accumulator rounded once per k step of 16, see oracle_gemm_f16).
  * erf is libm's erff; the device uses its own erff, both well inside the fp16 rounding that
  * follows except at rounding boundaries, which the parity tests allow for (1 fp16 ulp).
  * Pinned by: numpy float16 arithmetic step by step, scipy.special.erf in float64 (tolerance),
@@ -378,7 +398,9 @@ void oracle_gemm_f16_fused(const f16* A, const f16* W, const f16* bias, const f1
     const f16* a = A + i * K;
     const f16* w = W + j * K;
     f16 t;
-    if (acc_f16) {
+    if (acc_f16 == 2) {
+      t = dot_f16_k16(a, w, K);
+    } else if (acc_f16) {
       f16 acc = 0;
       for (int64_t k = 0; k < K; ++k) acc = f2h(h2f(acc) + h2f(f2h(h2f(a[k]) * h2f(w[k]))));
       t = acc;

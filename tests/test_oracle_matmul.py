@@ -83,6 +83,50 @@ def test_fp16_accumulate_follows_the_primfunc_text(oracle):
     assert not np.array_equal(oracle.c.gemm(a, w, acc_f16=True), oracle.c.gemm(a, w))
 
 
+def test_fp16_accumulator_rounded_once_per_k_step_of_16(oracle):
+    """acc_f16 = 2 restates the reference's scheduled GEMM: an fp16 accumulator fragment updated once per k step of
+    16 (experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py:19,37).  Pinned without repeating
+    the formula: by results that only this grouping gives."""
+    # (1) up to 16 terms there is one step: the fp32 sum rounded once, i.e. the fp32-accumulate mode bit for bit
+    for K in (1, 7, 16):
+        a, w = _inputs(3, 5, K, seed=20 + K)
+        assert np.array_equal(oracle.c.gemm(a, w, acc_f16=2).view(np.uint16), oracle.c.gemm(a, w).view(np.uint16))
+    # (2) where the accumulator stalls tells the step length: every product is 1/16, so a step of g terms adds g/16,
+    # and an fp16 sum stops growing where half its spacing reaches the increment (ties go to the even neighbour):
+    # one term at a time at 128, steps of 8 at 1024, of 16 at 2048, of 32 at 4096; fp32 accumulation reaches K/16
+    K = 16 * 8192
+    a = np.ones((1, K), np.float16)
+    w = np.full((1, K), 1 / 16, np.float16)
+    assert float(oracle.c.gemm(a, w, acc_f16=2)[0, 0]) == 2048.0
+    assert float(oracle.c.gemm(a, w, acc_f16=1)[0, 0]) == 128.0
+    assert float(oracle.c.gemm(a, w)[0, 0]) == 8192.0
+    # (3) inside a step the sum is not rounded: 2048 + sixteen 1s in one step is 2064 (one at a time each would be lost),
+    # and the steps are aligned at multiples of 16 from k = 0: eight 1s at the end of a step and eight at the start of
+    # the next are two ties, both lost
+    def run(entries, K=48):
+        wv = np.zeros((1, K), np.float16)
+        for k, v in entries:
+            wv[0, k] = v
+        return float(oracle.c.gemm(np.ones((1, K), np.float16), wv, acc_f16=2)[0, 0])
+    assert run([(0, 2048)] + [(k, 1) for k in range(16, 32)]) == 2064.0
+    assert run([(0, 2048)] + [(k, 1) for k in range(24, 32)]) == 2056.0      # eight in one step: 2056 is representable
+    assert run([(0, 2048)] + [(k, 1) for k in range(31, 33)]) == 2048.0      # one in each of two steps: each a tie, lost
+    assert run([(0, 2048)] + [(k, 1) for k in range(30, 32)]) == 2050.0      # the same two inside one step survive
+    # (4) the fused form takes its product from the same sum, and a K that is not a multiple of 16 ends with a short step
+    a, w = _inputs(4, 6, 200, seed=31)
+    bias = np.linspace(-1, 1, 6).astype(np.float16)
+    plain = oracle.c.gemm(a, w, bias, acc_f16=2)
+    assert np.array_equal(oracle.c.gemm_fused(a, w, bias, None, None, 0, acc_f16=2).view(np.uint16), plain.view(np.uint16))
+    f64 = a.astype(np.float64) @ w.astype(np.float64).T + bias.astype(np.float64)
+    assert np.abs(plain.astype(np.float64) - f64).max() < 0.05 * max(1.0, np.abs(f64).max())
+    head = oracle.c.gemm(a[:, :192].copy(), w[:, :192].copy(), acc_f16=2).astype(np.float32)
+    tail = (a[:, 192:].astype(np.float32)[:, None, :] * w[:, 192:].astype(np.float32)[None, :, :])
+    want = head.copy()
+    for k in range(8):
+        want = want + tail[:, :, k]
+    assert np.array_equal(oracle.c.gemm(a, w, acc_f16=2), want.astype(np.float16))
+
+
 def test_gemv_rf_follows_the_order_of_the_reference_schedule(oracle):
     """oracle.c.gemv_rf restates experiment/testIR/GEMV/m1n2560k10240/IR/5wt.py:11-92.  Each case below has a result
     that one stage's order fixes: 2048 + 1 is a tie in fp16 (spacing 2) and rounds back to 2048, so ones added one at

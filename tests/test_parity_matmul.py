@@ -367,6 +367,91 @@ def test_gemm_k_not_multiple_of_8_and_errors(oracle):
     _check(out.check(), oracle.c.gemm(a, w), oracle.np64.gemm(a, w))
 
 
+# ---- the reference's scheduled GEMM arithmetic: an fp16 accumulator rounded once per k step of 16
+# (experiment/testIR/GEMM/m_n2560_k10240/wmma/16x16x16/i2j4_x7y2_in8.py:19,37) -------------------------------------
+ACC16 = dict(variant=_lib.GEMM_MFMA_ACC16, block=256, vec=8, unroll=1, tile=[64, 64, 16], split_k=1)
+
+
+def _check_acc16(got, want, f64):
+    """Against oracle.c.gemm(acc_f16=2): the same roundings step by step; inside a step the matrix core adds its 16
+    exact products in an order of its own, so a sum that lands on a rounding boundary may fall to the other side --
+    one fp16 ulp there, which later steps carry along."""
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    assert np.isfinite(g).all()
+    scale = max(1.0, float(np.abs(f64).max()))
+    assert (np.abs(g - w) <= 4 * 2.0 ** -10 * np.maximum(np.abs(w), 0.25 * scale)).all(), float(np.abs(g - w).max())
+    assert (got == want).mean() > 0.9, float((got == want).mean())
+    # an fp16 running sum loses what fp32 accumulation keeps: the bound against float64 grows with sqrt(K / 16) roundings
+    assert np.abs(g - f64).max() <= 0.02 * scale + 1e-2
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (5, 7, 8), (33, 65, 72), (70, 130, 136), (300, 260, 200), (64, 2560, 2560), (256, 512, 10240)])
+def test_gemm_fp16_accumulator_per_k_step_of_16(oracle, M, N, K):
+    a, w = _inputs(M, N, K, 40 + M)
+    bias = np.random.default_rng(M).uniform(-1, 1, N).astype(np.float16)
+    out = Guarded((M, N), torch.float16)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, cfg(**ACC16))
+    _check_acc16(out.check(), oracle.c.gemm(a, w, bias, acc_f16=2, threads=8), oracle.np64.gemm(a, w, bias))
+
+
+def test_gemm_fp16_accumulator_exact_cases_element_accesses_epilogues_and_errors(oracle):
+    def run(a, w, **kw):
+        out = Guarded((a.shape[0], w.shape[0]), torch.float16)
+        ops.gemm(dev(a), dev(w), None, out.t, cfg(**{**ACC16, **kw}))
+        return out.check()
+    # where the accumulator stalls tells the step: products of 1/16, a step adds 1.0 and an fp16 sum stops at 2048
+    # (fp32 accumulation reaches 8192, one product at a time 128)
+    K = 16 * 8192
+    a = np.ones((3, K), np.float16)
+    w = np.full((2, K), 1 / 16, np.float16)
+    assert (run(a, w) == 2048.0).all()
+    fp32 = Guarded((3, 2), torch.float16)
+    ops.gemm(dev(a), dev(w), None, fp32.t, cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, tile=[64, 64, 64]))
+    assert (fp32.check() == 8192.0).all()
+    # inside a step nothing is rounded (2048 + 2 ones = 2050), across steps each tie is lost; steps start at k = 0, 16, ...
+    def one(entries, K=48):
+        wv = np.zeros((1, K), np.float16)
+        for k, v in entries:
+            wv[0, k] = v
+        return float(run(np.ones((1, K), np.float16), wv)[0, 0])
+    assert one([(0, 2048), (30, 1), (31, 1)]) == 2050.0
+    assert one([(0, 2048), (31, 1), (32, 1)]) == 2048.0
+    assert one([(0, 2048)] + [(k, 1) for k in range(16, 32)]) == 2064.0
+    # small integers: every sum is exact, so the result is the oracle's bit for bit (a transposed operand or a
+    # misplaced accumulator register fails here), on a shape that leaves tiles and the last step ragged
+    rng = np.random.default_rng(3)
+    ai = rng.integers(-3, 4, (70, 136)).astype(np.float16)
+    wi = rng.integers(-3, 4, (90, 136)).astype(np.float16)
+    assert_bits_equal(run(ai, wi), oracle.c.gemm(ai, wi, acc_f16=2))
+    # K % 8 != 0 (and odd pointers): element accesses, same arithmetic
+    a7, w7 = _inputs(9, 20, 77, 9)
+    _check_acc16(run(a7, w7), oracle.c.gemm(a7, w7, acc_f16=2), oracle.np64.gemm(a7, w7))
+    assert_bits_equal(run(ai[:, :77].copy(), wi[:, :77].copy()), oracle.c.gemm(ai[:, :77].copy(), wi[:, :77].copy(), acc_f16=2))
+    # the fused epilogues act on the fp16 sum as everywhere else
+    a2, w2 = _inputs(37, 96, 264, 11)
+    bias = rng.uniform(-1, 1, 96).astype(np.float16)
+    r1, r2 = rng.standard_normal((37, 96)).astype(np.float16), rng.standard_normal((37, 96)).astype(np.float16)
+    for kind in (1, 2, 3):
+        out = Guarded((37, 96), torch.float32 if kind == 2 else torch.float16)
+        ops.gemm(dev(a2), dev(w2), dev(bias), out.t, cfg(**ACC16), epilogue=kind, res1=dev(r1) if kind < 3 else None,
+                 res2=dev(r2) if kind < 3 else None)
+        want = oracle.c.gemm_fused(a2, w2, bias, r1 if kind < 3 else None, r2 if kind < 3 else None, kind, acc_f16=2)
+        g, wv = out.check().astype(np.float64), want.astype(np.float64)
+        assert (np.abs(g - wv) <= 4 * 2.0 ** -10 * np.maximum(np.abs(wv), 1.0)).all()
+    # what the mode cannot be combined with
+    o = torch.empty(9, 20, dtype=torch.float16, device="cuda")
+    for bad, msg in ((dict(split_k=2), "cannot be split"), (dict(tile=[128, 128, 16]), "64x64x16"), (dict(block=512), "256 threads")):
+        with pytest.raises(_lib.DtasError, match=msg):
+            ops.gemm(dev(a7[:, :72].copy()), dev(w7[:, :72].copy()), None, o, cfg(**{**ACC16, **bad}))
+    # the Python config object reaches the same kernel
+    from dtas_amd.common.config import MFMAConfig
+    c = MFMAConfig()
+    c.acc_f16 = True
+    abi = c.to_abi()
+    assert (abi.variant, abi.block, list(abi.tile)) == (_lib.GEMM_MFMA_ACC16, 256, [64, 64, 16])
+    assert MFMAConfig().from_dict(c.to_dict()).acc_f16
+
+
 SPLIT_TILES = [(256, 256), (128, 128), (128, 64), (64, 64)]
 
 

@@ -93,6 +93,8 @@ def test_static_scratch_gemm_allocates_no_device_memory():
     a, w, bias = _problem(96, 4096, 4096, 6)
     out = torch.empty(96, 4096, dtype=torch.float16, device="cuda")
     fresh = torch.cuda.Stream()          # a stream that owns no workspace yet
+    with torch.cuda.stream(fresh):       # (the runtime sets a stream's queue up at its first launch, which takes device memory: not ours)
+        out.zero_()
     torch.cuda.synchronize()
     free0 = torch.cuda.mem_get_info()[0]
     rc = L.dtas_gemm_f16_static(a.data_ptr(), w.data_ptr(), bias.data_ptr(), out.data_ptr(), 96, 4096, 4096, None, fresh.cuda_stream)
