@@ -9,7 +9,9 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdtas_gfx950.so")
+# DTAS_LIBRARY: another build of the same library (same ABI), e.g. one made with other compile-time constants to be
+# measured beside the product's; unset, the library built in-tree next to this file
+LIB_PATH = os.environ.get("DTAS_LIBRARY") or os.path.join(_HERE, "libdtas_gfx950.so")
 
 ABI_VERSION = 1
 

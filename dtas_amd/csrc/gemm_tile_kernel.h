@@ -4,6 +4,12 @@
 #pragma once
 #include "gemm_common.h"
 
+// Tile rows per group of the tile order (groups of this many tile rows are walked column-wise, and each XCD takes a
+// contiguous span of that order: with 32 workgroups resident per XCD a group of 8 makes an XCD's patch 8 x 4 tiles).
+#ifndef DTAS_GEMM_TILE_GROUP
+#define DTAS_GEMM_TILE_GROUP 8
+#endif
+
 namespace dtas {
 namespace {
 
@@ -82,7 +88,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   // nsplit > 1: nsplit consecutive workgroups (same XCD) share a tile and split its k tiles
   const unsigned my_split = __builtin_amdgcn_readfirstlane(whole ? 1u : nsplit);
   const unsigned pid = __builtin_amdgcn_readfirstlane(whole ? wgid : wgid / nsplit), z = __builtin_amdgcn_readfirstlane(whole ? 0u : wgid % nsplit);
-  constexpr unsigned kGroup = 8;
+  constexpr unsigned kGroup = DTAS_GEMM_TILE_GROUP;
   const unsigned width = kGroup * tiles_n;
   const unsigned first_m = (pid / width) * kGroup;
   const unsigned gsize = tiles_m - first_m < kGroup ? tiles_m - first_m : kGroup;
