@@ -784,12 +784,13 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
     }
     if (!rows) {
       // what this op moves is P (2*n*m bytes per head).  Measured over n = m = 128 .. 4096 with 32 heads of 80:
-      // 64-row tiles while 128-row tiles would leave most CUs idle; 128-row tiles with three stages up to
-      // one per CU; 256-row tiles with three stages beyond (n = m = 1280: 37 us against 44 for 128x128
-      // with three stages and 61 with two; 2048: 74 / 79 / 98).  Head dimensions up to 64 keep the
+      // 64-row tiles (three stages) while 128-row tiles would leave half of the CUs idle (n = m = 512: 8.9 us against
+      // 11.0 for 128x128); 128-row tiles with three stages up to one per CU; 256-row tiles with three stages beyond
+      // (n = m = 1280: 30.5 us against 37.9 for 128x128 with three stages and 47.0 with two; 2048: 73 / 75 / 82, every
+      // tile within 5 %: there the launch is bound by how P streams in, 128 bytes of a row per request).  Head dimensions up to 64 keep the
       // 64-column tiles: two workgroups of two stages per CU
       const int64_t t128 = heads * ceil_div(n, 128);
-      if (t128 <= kNumCU / 4) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, bn, kBK}, 1, 0};
+      if (t128 <= kNumCU / 2) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, bn == 128 ? 3 : 2, {64, bn, kBK}, 1, 0};
       else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
       else if (bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
       else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
@@ -861,20 +862,22 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   }
   if (cfg.variant != DTAS_GEMM_MFMA) return fail("attn_pv: unknown variant %d", cfg.variant);
   const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
-  if (cfg.unroll > 3) return fail("attn_pv: the transposing kernels hold two or three LDS stages, got %d", cfg.unroll);
   if (m * d >= (int64_t{1} << 31)) return fail("attn_pv: a head's V exceeds the 4 GiB a buffer descriptor spans");
   int64_t la[7];
-  if (describe_gemm(n, d, m, cfg, la) != 0) return -1;
+  if (describe_gemm(n, d, m, cfg, la) != 0) return -1;   // (also: no more LDS stages than the tile allows)
   const int bm = cfg.tile[0], bn = cfg.tile[1];
-  const bool three = cfg.unroll == 3;
+  const int ns = cfg.unroll >= 2 ? cfg.unroll : 2;
   ep.lda = m;
   ep.k_tail = static_cast<unsigned>(m - m_main);
-  if (bm == 256 && bn == 128 && three) return launch_mfma<256, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m_main, sk, b);
-  if (bm == 128 && bn == 128 && three) return launch_mfma<128, 128, 2, 2, 3, true>(s, a, w, ep, out, n, d, m_main, sk, b);
-  if (three) return fail("attn_pv: three stages come with the 256x128 and 128x128 tiles, got %dx%d", bm, bn);
-  if (bm == 128 && bn == 128) return launch_mfma<128, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
-  if (bm == 64 && bn == 128) return launch_mfma<64, 128, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
-  if (bm == 128 && bn == 64) return launch_mfma<128, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
-  if (bm == 64 && bn == 64) return launch_mfma<64, 64, 2, 2, 2, true>(s, a, w, ep, out, n, d, m_main, sk, b);
+#define DTAS_PV_CASE(BM_, BN_, NS_) \
+  if (bm == BM_ && bn == BN_ && ns == NS_) return launch_mfma<BM_, BN_, 2, 2, NS_, true>(s, a, w, ep, out, n, d, m_main, sk, b)
+  // (four stages measured level with or behind three on every tile, n = m = 256 .. 4096: not instantiated)
+  DTAS_PV_CASE(256, 128, 3);
+  DTAS_PV_CASE(128, 128, 2); DTAS_PV_CASE(128, 128, 3);
+  DTAS_PV_CASE(64, 128, 2); DTAS_PV_CASE(64, 128, 3);
+  DTAS_PV_CASE(128, 64, 2);
+  DTAS_PV_CASE(64, 64, 2);
+#undef DTAS_PV_CASE
+  if (ns != 2) return fail("attn_pv: three LDS stages come with the 256x128, 128x128 and 64x128 tiles, two with every tile but 256x128; got %dx%d with %d", bm, bn, ns);
   return fail("attn_pv: no transposing MFMA kernel for tile %dx%d", bm, bn);
 }

@@ -59,18 +59,39 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
     // 14.0 against 26.3 us at 64 x 2560 x 2560 and 25.1 against 39.5 at 4096 x 4096, but 38 against 27 at N = 10240
     if (!user && stream_ok && M <= 64 && N <= 4096 && K <= 4096) return launch_gemm_stream_q8(64, 512, s, a, w, ep, C, M, N, K);
   }
-  // Two routes.  Dequantising in the W path of the GEMM (no intermediate) runs on a plain burst pipeline without
-  // split K: measured at the model's shapes it wins for M <= 64 with K <= 4096 (18 against 24 us at 7680x2560)
-  // and loses beyond (M = 2048: 109 against 84 us; K = 10240: 2x or more).  Otherwise: the dequantiser into a
-  // library-owned fp16 buffer, then the fp16 GEMM with everything its table offers.  A cfg selects the first route.
-  if (!user && !(M <= 64 && K <= 4096)) {
+  // Two routes.  (1) Dequantising in the W path of the tile kernel: no intermediate, W read once per row of tiles as
+  // bytes; a plain burst pipeline on 4 wavefronts, with K split over workgroups while the tiles leave CUs idle.
+  // (2) The dequantiser into a library-owned fp16 buffer, then the fp16 GEMM with everything its table offers: 3 more
+  // bytes per weight through memory (9-14 us at the model's shapes), worth it once the GEMM itself is long.
+  // Measured at the model's shapes with rotating weights, us, route 1 (tile, K parts) / route 2 / the fp16 GEMM on
+  // fp16 weights: 7680x2560, M = 64 / 128 / 256 / 512 / 1024: 16.4 (64x64, 4) / 28.0 / 14.3, 21.9 (64x64, 3) / 29.6 /
+  // 17.7, 26.8 (128x128, 2) / 33.6 / 25.3, 38.6 (128x128, 1) / 41.4 / 33.4, 58.8 / 52.6 / 43.3; 10240x2560, M = 64 / 128 /
+  // 256 / 512: 19.5 / 29.9 / 18.7, 24.2 (128x128, 3) / 34.7 / 26.0, 35.1 / 40.5 / 33.3, 56.4 / 48.8 / 39.6; 2560x10240,
+  // M = 64 / 256 / 512 / 1024: 25.7 (64x64, 8) / 34.0 / 22.6, 37.4 (128x128, 6) / 44.1 / 38.5, 52.9 / 57.3 / 50.0, 87.9 /
+  // 76.0 / 66.8.  So route 1 up to 512 rows while 128x128 tiles fit the chip in one round; 64x64 tiles (two stages, ~2
+  // workgroups per CU wanted) up to 128 rows unless they already number more than the CUs, 128x128 (three stages, one
+  // per CU) beyond; K parts to fill the chip, each at least 4 k tiles.  A cfg selects route 1 with its own tile and split.
+  const int64_t t128 = ceil_div(M, 128) * ceil_div(N, 128), t64 = ceil_div(M, 64) * ceil_div(N, 64), ktiles = ceil_div(K, kBK);
+  const bool fused_route = M <= 512 && t128 <= kNumCU;
+  if (!user && !fused_route) {
     void* wbuf = nullptr;
     std::lock_guard<std::recursive_mutex> ws_lock(g_ws_mutex);  // until both launches are enqueued
     if (operand_workspace(static_cast<hipStream_t>(stream), static_cast<size_t>(N) * K * 2, &wbuf) != 0) return -1;
     if (dtas_decode_q8_f16(Wq, scale, wbuf, N, K, nullptr, stream) != 0) return -1;
     return dtas_gemm_f16_fused(A, wbuf, bias, res1, res2, C, M, N, K, epilogue, nullptr, stream);
   }
-  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, 64, kBK}, 1, 0};
+  dtas_config cfg;
+  if (user) {
+    cfg = *user;
+  } else {
+    const bool small = M <= 128 && t64 <= kNumCU;
+    int64_t parts = small ? (2 * kNumCU - 32 + t64 / 2) / t64 : kNumCU / t128;  // (rounded to ~480 workgroups of 64x64; one round of 128x128)
+    if (parts > 8) parts = 8;
+    if (parts > ktiles / 4) parts = ktiles / 4;
+    if (parts < 1) parts = 1;
+    cfg = small ? dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, 64, kBK}, static_cast<int32_t>(parts), 0}
+                : dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, static_cast<int32_t>(parts), 0};
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const half_t* a = static_cast<const half_t*>(A);
   const half_t* w = static_cast<const half_t*>(Wq);  // (bytes; the kernels take the pointer as they take fp16 W)
@@ -83,12 +104,12 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
   }
   if (cfg.vec != 8) return fail("gemm_q8: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
   if (cfg.variant != DTAS_GEMM_MFMA) return fail("gemm_q8: only the MFMA kernels serve 8-bit weights");
-  if (cfg.split_k > 1) return fail("gemm_q8: K is not split for 8-bit weights");
+  const int sk = cfg.split_k < 1 ? 1 : cfg.split_k;
   int64_t la[7];
   if (describe_gemm(M, N, K, cfg, la) != 0) return -1;
   const int bm = cfg.tile[0], bn = cfg.tile[1];
-  if (bm == 256 && bn == 128 && cfg.unroll == 3) return launch_mfma<256, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, 1);
-  if (bm == 128 && bn == 128 && cfg.unroll == 3) return launch_mfma<128, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, 1);
-  if (bm == 64 && bn == 64 && cfg.unroll == 2) return launch_mfma<64, 64, 2, 2, 2, false, true>(s, a, w, ep, C, M, N, K, 1);
+  if (bm == 256 && bn == 128 && cfg.unroll == 3) return launch_mfma<256, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, sk);
+  if (bm == 128 && bn == 128 && cfg.unroll == 3) return launch_mfma<128, 128, 2, 2, 3, false, true>(s, a, w, ep, C, M, N, K, sk);
+  if (bm == 64 && bn == 64 && cfg.unroll == 2) return launch_mfma<64, 64, 2, 2, 2, false, true>(s, a, w, ep, C, M, N, K, sk);
   return fail("gemm_q8: 8-bit weights come with tiles 256x128 and 128x128 (three stages) and 64x64 (two), got %dx%d with %d", bm, bn, cfg.unroll);
 }

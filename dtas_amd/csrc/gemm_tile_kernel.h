@@ -13,10 +13,11 @@
 namespace dtas {
 namespace {
 
-// WT: W is given k-major ([K][N], N contiguous -- the V operand of attention's P.V); its tiles are
-// then transposed on the way into the LDS (two stages, 4 wavefronts only).
+// WT: W is given k-major ([K][N], N contiguous -- the V operand of attention's P.V); its tiles sit in the LDS as they lie
+// in memory (the same direct-to-LDS loads and pipelines as a row-major W) and the MFMA fragments are read with the
+// transposing LDS read ds_read_b64_tr_b16 (4 wavefronts only).
 // WQ: W is 8-bit with an fp16 scale per 32 elements of a row (Wq bytes [N][K], ep.wscale [N][K/32]); its
-// tiles are dequantised on their way into the LDS by the same register path.
+// tiles pass through registers and are dequantised on their way into the LDS.
 // M16: 8 wavefronts (256x256, 256x128, 128x256) on v_mfma_f32_16x16x32_f16 with one barrier per k tile (see the main loop).
 template <int BM, int BN, int WM, int WN, int NS, bool WT = false, bool WQ = false, bool M16 = false>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* __restrict__ A,
@@ -34,9 +35,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   static_assert(NW % 2 == 0 && LA >= 1 && LB >= 1 && MT >= 1 && NT >= 1, "tile / wavefront split");
   static_assert(NS >= 2 && NS <= 4 && (NW != 8 || NS == 2), "stage count");
   static_assert((NS - 1) * (LA + LB) <= 63, "outstanding loads must fit the vmcnt field");
-  constexpr bool WREG = WT || WQ;  // W tiles pass through registers (transposed or dequantised), not the direct-to-LDS path
+  constexpr bool WREG = WQ;  // W tiles pass through registers (dequantised), not the direct-to-LDS path
   static_assert(!WREG || (NS <= 3 && NW == 4), "the register W path is written for two or three stages and 4 wavefronts");
   static_assert(!(WT && WQ), "k-major 8-bit weights are not served");
+  static_assert(!WT || (NW == 4 && BN >= 64), "the k-major W path is written for the 4-wavefront 32x32x16 loops");
   static_assert(M16 == (NW == 8) && (!M16 || !WREG), "8 wavefronts run the 16x16x32 loop, and only they");
   // 256x256 and every 8-wavefront tile: a ring of 5 operand units, each the larger operand's rows of a k tile
   constexpr bool kRing = BM + BN == 512 || M16;
@@ -103,11 +105,45 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const int64_t lda = WT && ep.lda ? ep.lda : K;  // (with a row-major W both operands' rows are K long)
   const unsigned row_bytes = static_cast<unsigned>(lda) * 2u;
   const __amdgpu_buffer_rsrc_t ra = make_rsrc(A + m0 * lda, static_cast<unsigned>(rows_a) * row_bytes);
-  const __amdgpu_buffer_rsrc_t rw = make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
+  // row-major W: the tile's rows; k-major W ([K][N], the V of P.V): the whole matrix, so that k rows past K read as zeros
+  const __amdgpu_buffer_rsrc_t rw = WT ? make_rsrc(W, static_cast<unsigned>(K * N * 2))
+                                       : make_rsrc(W + n0 * K, static_cast<unsigned>(rows_w) * row_bytes);
   const unsigned r_in = 2u * (l >> 4) + (((l >> 3) & 1u) ^ (wv & 1u));  // row inside the 8-row block
   const unsigned c_in = (l & 7u) ^ r_in;                                // chunk of that row
   const unsigned g_off = (8u * wv + r_in) * row_bytes + c_in * 16u;
   const unsigned g_step = 8u * NW * row_bytes;
+
+  // ---- k-major W (WT).  A W tile is 64 k x BN columns of W[K][N] and sits in the LDS as it lies in memory: k row after
+  // k row of BN * 2 bytes, brought in by the same direct-to-LDS block loads (slot p of a 1 KiB block <- lane p; columns past N
+  // and k rows past K are out of range and arrive as zeros).  The MFMA wants a lane to hold 8 consecutive k of one column:
+  // ds_read_b64_tr_b16 delivers that -- in each group of 16 lanes, lane r names 8 bytes (4 columns of one k row) and lane i
+  // receives element i & 3 of the rows that lanes i >> 2, 4 + (i >> 2), 8 + (i >> 2), 12 + (i >> 2) named; with lane r naming
+  // k row r >> 2, columns 4 (r & 3) .. + 3, lane i receives 4 consecutive k of column i.  16-byte chunk c of k row k is kept at
+  // chunk position c ^ wt_swz(k), which spreads the 32 lanes the LDS serves together (4 k rows x two 16-column groups) over all
+  // 64 banks (a k row is a whole number of bank rows, or half of one when BN = 64).
+  constexpr int kWtRowB = BN * 2, kWtRpb = 1024 / kWtRowB;  // bytes per k row in the LDS; k rows per 1 KiB block
+  static_assert(!WT || (kWtRpb >= 1 && 1024 % kWtRowB == 0 && (NW * kWtRpb) % 4 == 0), "k rows per block");
+  auto wt_swz = [](unsigned k) -> unsigned { return BN >= 128 ? 4u * (k & 3u) : 4u * ((k >> 1) & 1u); };
+  const unsigned wt_k = wv * kWtRpb + (l * 16u) / kWtRowB;                 // k row (inside a stage) of this lane's slot in block 0
+  const unsigned wt_c = (((l * 16u) % kWtRowB) / 16u) ^ wt_swz(wt_k);      // the chunk that belongs at this lane's slot
+  const bool wt_col_ok = n0 + 8 * static_cast<int64_t>(wt_c) < N;         // (N % 8 == 0: a chunk is all-in or all-out)
+  const unsigned wt_off = static_cast<unsigned>((static_cast<int64_t>(wt_k) * N + n0 + 8 * wt_c) * 2);
+  // one block load further: NW * kWtRpb k rows on.  The block's offset is added to the lane's (vector) offset, which the
+  // descriptor's range check covers: k rows past K must read as zeros (the k tail is added in the epilogue, and what lies
+  // behind a head's V is another head's), and an out-of-range lane (0x80000000 + ...) stays out of range
+  const unsigned wt_step = static_cast<unsigned>(NW * kWtRpb * N * 2);
+  // fragment reads: lane l = 16 g + r; group g serves columns 16 (g & 1) .. + 15 of a 32-column block and k 8 (g >> 1) .. + 7
+  // of a k16 step, in two reads of 4 k each
+  unsigned wt_rd[NT];
+  {
+    const unsigned g = l >> 4, r = l & 15u;
+    const unsigned krow = 8u * (g >> 1) + (r >> 2);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const unsigned c = (wn * WTN + j * 32 + 16u * (g & 1u)) / 8u + ((r >> 1) & 1u);
+      wt_rd[j] = krow * kWtRowB + ((c ^ wt_swz(krow)) * 16u) + (r & 1u) * 8u;
+    }
+  }
 
   // ---- LDS -> MFMA operands: lane l supplies row (l & 31), chunk 2*ks + (l >> 5)
   unsigned lds_rd[4];
@@ -136,6 +172,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const int kt0 = static_cast<int>(z) * kt_per;
   const int ktiles = ktiles_all - kt0 < kt_per ? (ktiles_all - kt0 > 0 ? ktiles_all - kt0 : 0) : kt_per;
 
+  // k-major W: this lane's byte offset in W for k tile kt of this workgroup (k rows past K lie past the descriptor's range)
+  auto wt_lane_off = [&](int kt) -> unsigned {
+    return wt_col_ok ? wt_off + static_cast<unsigned>(static_cast<int64_t>(kt0 + kt) * kBK * N * 2) : kOob;
+  };
   // tile kt -> LDS stage kt % NS, asynchronously (completion is counted by vmcnt)
   auto fetch = [&](int kt) {
     // a chunk past K is pointed out of range; K % 8 == 0, so chunks are all-in or all-out
@@ -146,116 +186,100 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
     for (int i = 0; i < LA; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, 0);
-    if constexpr (!WREG) {
+    if constexpr (WT) {
+      const unsigned woff = wt_lane_off(kt);
+#pragma unroll
+      for (int i = 0; i < LB; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, woff + i * wt_step, 0, 0, 0);
+    } else if constexpr (!WREG) {
 #pragma unroll
       for (int i = 0; i < LB; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
     }
   };
 
-  // ---- k-major W.  A tile is 64 k x BN columns of W[K][N]; an item is 8 columns of two
-  // consecutive k rows: a lane loads the two 16-byte pieces into registers (wt_load, issued just
-  // before the tile's A blocks) and later (wt_commit, once the tile is next in line) stores eight
-  // 4-byte words {W[k][c], W[k+1][c]} to where the row-major path would have put them.  Item -> lane
-  // is chosen so that a wavefront's 64 stores hit 64 distinct banks: 32 k pairs x 2 adjacent column
-  // chunks.  The pieces come through buffer loads (out of range -> zeros), so every lane issues the
-  // same number of loads per tile whatever its columns: the waits below count them.  Columns past N
-  // are never written: the W parts of all stages are zeroed once, up front.
-  // 8-bit W: an item is 16 weights of a row (16 bytes -> two 16-byte chunks of fp16) and their scale; lane
-  // t takes piece t % 4 of row t / 4 (+ 64 rows per further item), so a wavefront reads 64 contiguous bytes
-  // of each of 16 rows.  Every row of the tile is written every time (rows past N as zeros): nothing to clear.
+  // ---- 8-bit W through registers: an item is 16 weights of a row (16 bytes -> two 16-byte chunks of fp16) and their
+  // scale: a lane loads them into registers (wt_load, issued just before the tile's A blocks) and later (wt_commit, once
+  // the tile is next in line) stores the dequantised chunks to where the row-major path would have put them; lane t takes
+  // piece t % 4 of row t / 4 (+ 64 rows per further item), so a wavefront reads 64 contiguous bytes of each of 16 rows.
+  // The pieces come through buffer loads (out of range -> zeros), so every lane issues the same number of loads per tile
+  // whatever its rows: the waits below count them.  Every row of the tile is written every time (rows past N as zeros).
   constexpr int kWtItems = WREG ? 4 * BN / (64 * NW) : 1;
   constexpr int kWtSlots = WREG ? NS - 1 : 1;  // register sets: one per tile in flight
-  constexpr int kWtLoads = 2 * kWtItems;  // per lane and tile: k-major two pieces per item, 8-bit a piece and its scale
-  u32x4 wt_reg[kWtSlots][kWtItems][WQ ? 1 : 2];
+  constexpr int kWtLoads = 2 * kWtItems;  // per lane and tile: a piece and its scale per item
+  u32x4 wt_reg[kWtSlots][kWtItems][1];
   unsigned short wq_scale[kWtSlots][kWtItems];
-  const __amdgpu_buffer_rsrc_t rv = make_rsrc(W, WT ? static_cast<unsigned>(K * N * 2) : WQ ? static_cast<unsigned>(K * N) : 0u);
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(W, WQ ? static_cast<unsigned>(K * N) : 0u);
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(ep.wscale, WQ ? static_cast<unsigned>((K / 32) * N * 2) : 0u);
-  auto wt_item = [&](int i, unsigned& cc, unsigned& kp) {
-    const unsigned item = t + i * 64 * NW;
-    cc = ((item >> 6) << 1) | (item & 1u);
-    kp = (item >> 1) & 31u;
-  };
   auto wt_load = [&](int kt, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
-    if constexpr (WQ) {
 #pragma unroll
-      for (int i = 0; i < kWtItems; ++i) {
-        const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
-        const int64_t row = n0 + r, k = static_cast<int64_t>(kt0 + kt) * kBK + c4 * 16;
-        const bool in = row < N && k < K;  // K % 32 == 0: a piece and its scale group are all-in or all-out
-        wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, in ? static_cast<unsigned>(row * K + k) : kOob, 0, 0);
-        wq_scale[SLOT][i] = __builtin_amdgcn_raw_buffer_load_b16(rs, in ? static_cast<unsigned>((row * (K >> 5) + (k >> 5)) * 2) : kOob, 0, 0);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < kWtItems; ++i) {
-        unsigned cc, kp;
-        wt_item(i, cc, kp);
-        const int64_t col = n0 + cc * 8, k = static_cast<int64_t>(kt0 + kt) * kBK + 2 * kp;
-        const unsigned at = static_cast<unsigned>((k * N + col) * 2), row = static_cast<unsigned>(N) * 2u;
-        wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k < K) ? at : kOob, 0, 0);
-        wt_reg[SLOT][i][1] = __builtin_amdgcn_raw_buffer_load_b128(rv, (col < N && k + 1 < K) ? at + row : kOob, 0, 0);
-      }
+    for (int i = 0; i < kWtItems; ++i) {
+      const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
+      const int64_t row = n0 + r, k = static_cast<int64_t>(kt0 + kt) * kBK + c4 * 16;
+      const bool in = row < N && k < K;  // K % 32 == 0: a piece and its scale group are all-in or all-out
+      wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, in ? static_cast<unsigned>(row * K + k) : kOob, 0, 0);
+      wq_scale[SLOT][i] = __builtin_amdgcn_raw_buffer_load_b16(rs, in ? static_cast<unsigned>((row * (K >> 5) + (k >> 5)) * 2) : kOob, 0, 0);
     }
   };
   auto wt_commit = [&](int kt, auto slot_tag) {
     constexpr int SLOT = decltype(slot_tag)::value;
     char* base = lds + (kt % NS) * kStage + kABytes;
-    if constexpr (WQ) {
 #pragma unroll
-      for (int i = 0; i < kWtItems; ++i) {
-        const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
-        const half_t sc = __builtin_bit_cast(half_t, wq_scale[SLOT][i]);
-        const f16x2 s2 = {sc, sc};
-        u32x4 out[2];
+    for (int i = 0; i < kWtItems; ++i) {
+      const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
+      const half_t sc = __builtin_bit_cast(half_t, wq_scale[SLOT][i]);
+      const f16x2 s2 = {sc, sc};
+      u32x4 out[2];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          f16x2 lo, hi;
-          const unsigned word = wt_reg[SLOT][i][0][w];
-          dequant_q8_word(word, s2, lo, hi);
-          out[w >> 1][(w & 1) * 2] = __builtin_bit_cast(unsigned, lo);
-          out[w >> 1][(w & 1) * 2 + 1] = __builtin_bit_cast(unsigned, hi);
-        }
-        *reinterpret_cast<u32x4*>(base + lds_chunk_offset(r, 2 * c4)) = out[0];
-        *reinterpret_cast<u32x4*>(base + lds_chunk_offset(r, 2 * c4 + 1)) = out[1];
+      for (int w = 0; w < 4; ++w) {
+        f16x2 lo, hi;
+        const unsigned word = wt_reg[SLOT][i][0][w];
+        dequant_q8_word(word, s2, lo, hi);
+        out[w >> 1][(w & 1) * 2] = __builtin_bit_cast(unsigned, lo);
+        out[w >> 1][(w & 1) * 2 + 1] = __builtin_bit_cast(unsigned, hi);
       }
-    } else {
-#pragma unroll
-      for (int i = 0; i < kWtItems; ++i) {
-        unsigned cc, kp;
-        wt_item(i, cc, kp);
-        if (n0 + cc * 8 >= N) continue;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const unsigned a = wt_reg[SLOT][i][0][j], b = wt_reg[SLOT][i][1][j];
-          const unsigned r = cc * 8 + 2 * j;
-          *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r, kp >> 2) + (kp & 3u) * 4u) = (a & 0xffffu) | (b << 16);
-          *reinterpret_cast<unsigned*>(base + lds_chunk_offset(r + 1, kp >> 2) + (kp & 3u) * 4u) = (a >> 16) | (b & 0xffff0000u);
-        }
-      }
+      *reinterpret_cast<u32x4*>(base + lds_chunk_offset(r, 2 * c4)) = out[0];
+      *reinterpret_cast<u32x4*>(base + lds_chunk_offset(r, 2 * c4 + 1)) = out[1];
     }
   };
-  if constexpr (WT) {
-    const u32x4 zero = {0u, 0u, 0u, 0u};
-    for (int s = 0; s < NS; ++s)
-      for (unsigned at = t * 16u; at < static_cast<unsigned>(BN * kRowBytes); at += 64 * NW * 16)
-        *reinterpret_cast<u32x4*>(lds + s * kStage + kABytes + at) = zero;
-    __syncthreads();
-  }
 
   f16x8 fa[2][MT], fb[2][NT];
   auto read_a = [&](int set, int i, const char* stage, int ks) {
     fa[set][i] = *reinterpret_cast<const f16x8*>(stage + a_base + i * 4096 + lds_rd[ks]);
   };
+  // (k-major W) The transposing reads are issued as inline assembly: through the compiler's builtin every one of them
+  // is preceded by a wait for all outstanding direct-to-LDS loads (the compiler takes the read to alias them), which
+  // serialises the pipeline.  The compiler then knows nothing of these reads' completion either: wait_frag_b() is the
+  // wait, placed where the fragments are first used.
+  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_ptr_t)lds));
   auto read_b = [&](int set, int j, const char* stage, int ks) {
-    fb[set][j] = *reinterpret_cast<const f16x8*>(stage + b_base + j * 4096 + lds_rd[ks]);
+    if constexpr (WT) {
+      // k 16 ks + 8 (g >> 1) .. + 7 of this lane's column: two transposing reads of 4 k each
+      const unsigned at = lds_base + static_cast<unsigned>(stage - lds) + kABytes + ks * 16 * kWtRowB + wt_rd[j];
+      f16x4 lo, hi;
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(at));
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi) : "v"(at + 4 * kWtRowB));
+      fb[set][j] = f16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    } else {
+      fb[set][j] = *reinterpret_cast<const f16x8*>(stage + b_base + j * 4096 + lds_rd[ks]);
+    }
+  };
+  // (k-major W) every LDS read issued so far has returned; the W fragments of `set` pass through an empty statement that
+  // follows the wait, so nothing that uses them can be moved ahead of it
+  auto wait_frag_b = [&](int set) {
+    if constexpr (WT) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < NT; ++j) asm volatile("" : "+v"(fb[set][j]));
+    }
   };
   // The MT*NT MFMAs of register set `set`, with the MT+NT fragment reads of the next step (from
   // `stage`, step `ks`, into the other set) spread evenly between them.  W rows are the first MFMA
   // operand, so a lane ends up with 4 consecutive columns of one C row per accumulator quad.
   auto step = [&](int set, const char* stage, int ks, bool reads) {
     constexpr int kReads = MT + NT, kMfma = MT * NT;
+    wait_frag_b(set);
 #pragma unroll
     for (int q = 0; q < kMfma; ++q) {
       if (reads) {
@@ -542,16 +566,21 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
     };
     // block load l (0 .. kL-1: A blocks, then W blocks) of a tile into `stage`
-    auto fetch_one = [&](int l_, unsigned voff, char* stage) {
+    // (k-major W: the W blocks take the lane's offset in W, `woff`)
+    auto fetch_one = [&](int l_, unsigned voff, char* stage, unsigned woff = 0u) {
       if (l_ < LA)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(stage + wv * 1024 + l_ * NW * 1024), 16, voff, l_ * g_step, 0, 0);
+      else if constexpr (WT)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(stage + kABytes + wv * 1024 + (l_ - LA) * NW * 1024), 16,
+                                                 woff + (l_ - LA) * wt_step, 0, 0, 0);
       else
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(stage + kABytes + wv * 1024 + (l_ - LA) * NW * 1024), 16, voff,
                                                  (l_ - LA) * g_step, 0, 0);
     };
     // MFMAs of `set`, the next step's fragment reads, and part `part` of a tile's loads (if `dma`)
-    auto step_dma = [&](int set, const char* stage, int ks, bool reads, bool dma, int part, unsigned voff, char* dst) {
+    auto step_dma = [&](int set, const char* stage, int ks, bool reads, bool dma, int part, unsigned voff, char* dst, unsigned woff) {
       constexpr int kReads = MT + NT, kMfma = MT * NT;
+      wait_frag_b(set);
 #pragma unroll
       for (int q = 0; q < kMfma; ++q) {
         if (reads) {
@@ -568,7 +597,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
           const int lo = part * kL / 4, hi = (part + 1) * kL / 4;
 #pragma unroll
           for (int l_ = 0; l_ < kL; ++l_)
-            if (l_ >= lo && l_ < hi && (l_ - lo) * kMfma / (hi - lo) == q) fetch_one(l_, voff, dst);
+            if (l_ >= lo && l_ < hi && (l_ - lo) * kMfma / (hi - lo) == q) fetch_one(l_, voff, dst, woff);
         }
         DTAS_SCHED_FENCE();
       }
@@ -576,16 +605,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // every stage is free: tile 0, tiles 1 .. NS-2 whole and part 0 of tile NS-1 are requested together, and only
     // tile 0 is waited for (loads complete in order: whole tiles requested after it may stay outstanding)
     if (ktiles > 0) {
-      const unsigned v0 = lane_off(0);
+      const unsigned v0 = lane_off(0), w0 = WT ? wt_lane_off(0) : 0u;
 #pragma unroll
-      for (int l_ = 0; l_ < kL; ++l_) fetch_one(l_, v0, lds);
+      for (int l_ = 0; l_ < kL; ++l_) fetch_one(l_, v0, lds, w0);
     }
 #pragma unroll
     for (int p = 1; p < NS; ++p) {
       if (p < ktiles) {
-        const unsigned vp = lane_off(p);
+        const unsigned vp = lane_off(p), wp = WT ? wt_lane_off(p) : 0u;
 #pragma unroll
-        for (int l_ = 0; l_ < (p < NS - 1 ? kL : kL / 4); ++l_) fetch_one(l_, vp, lds + p * kStage);
+        for (int l_ = 0; l_ < (p < NS - 1 ? kL : kL / 4); ++l_) fetch_one(l_, vp, lds + p * kStage, wp);
       }
     }
     wait_whole_tiles<kL, NS - 2>(ktiles - 1);
@@ -606,9 +635,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       char* late = lds + wrap(cur_s + NS - 1) * kStage;  // stage of tile kt-1 = of tile kt+NS-1
       const bool have_late = steady || kt + NS - 1 < ktiles, have_new = steady || kt + NS < ktiles;
       const unsigned v_late = lane_off(kt + NS - 1), v_new = lane_off(kt + NS);
-      step_dma(0, cur, 1, true, have_late, 1, v_late, late);
-      step_dma(1, cur, 2, true, have_late, 2, v_late, late);
-      step_dma(0, cur, 3, true, have_late, 3, v_late, late);
+      const unsigned w_late = WT ? wt_lane_off(kt + NS - 1) : 0u, w_new = WT ? wt_lane_off(kt + NS) : 0u;
+      step_dma(0, cur, 1, true, have_late, 1, v_late, late, w_late);
+      step_dma(1, cur, 2, true, have_late, 2, v_late, late, w_late);
+      step_dma(0, cur, 3, true, have_late, 3, v_late, late, w_late);
       // tile kt+1 must have landed; later tiles (at most NS-2 of them) may stay in flight.  Loads
       // complete in order, so it is enough to allow that many tiles' worth of loads outstanding.
       if (steady) {
@@ -618,7 +648,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       }
       __builtin_amdgcn_s_barrier();  // ... and every wavefront has finished reading tile kt
       DTAS_SCHED_FENCE();
-      step_dma(1, nxt, 0, steady || kt + 1 < ktiles, have_new, 0, v_new, cur);
+      step_dma(1, nxt, 0, steady || kt + 1 < ktiles, have_new, 0, v_new, cur, w_new);
       cur_s = wrap(cur_s + 1);
     };
     static_assert((NS - 2) * kL <= 63, "outstanding loads must fit the vmcnt field");

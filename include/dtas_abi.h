@@ -325,9 +325,10 @@ int dtas_attn_scores_f16_f32(const void* Q, const void* K, const void* mask, voi
 /* ---- attention output: matmul8 (before_dl.py:915-929; n dynamic) and matmul10 (:899-912; n = 1) ----
  * out[h,i,:] = sum_k P[h,i,k] * V[h,k,:]
  * P[heads,n,m] (the softmaxed scores), V[heads,m,d], out[heads,n,d], all fp16; n and m are the dynamic
- * extents.  V is k-major (its rows run along d), so its tiles are transposed on the way into the LDS.
+ * extents.  V is k-major (its rows run along d): its tiles lie in the LDS as in memory and the matrix-core operands
+ * are read from there transposed.
  * fp32 accumulation, one rounding to fp16.  cfg, when given: a DTAS_GEMM_MFMA row for the per-head
- * (n, d, m) problem with tile {64|128, 64|128, 64} and two stages, or {128|256, 128, 64} and three (split_k > 1:
+ * (n, d, m) problem with tile {64|128, 64|128, 64} and two stages, or {64|128|256, 128, 64} and three (split_k > 1:
  * the workgroups of a (head, tile) split m and meet in the split-K workspace), or a DTAS_GEMM_SKINNY row
  * {block 256, tile {1|2|4|8, 8, 0}} for the kernel that serves a handful of rows (decoding), or {block 1024, tile {1, 8, 0}}
  * for one workgroup per (head, row) that reads the head's V in one contiguous sweep (d <= 1024) -- tile[2] = c > 0
@@ -374,10 +375,13 @@ int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, 
  * with tile {256,128,64} or {128,128,64} and unroll 3, or {64,64,64} and unroll 2; or a DTAS_GEMM_STREAM row
  * (block 256, tile {16,64,512}, {16,64,1024}, {32,64,512} or {64,64,512}; M <= tile[0]; K % 256 == 0; 16-byte
  * aligned A, Wq and scale): the W-streaming kernel on the bytes of W, widened between the LDS and the MFMA; its K
- * slices meet in the split-K workspace.  One row with a bias or GELU epilogue goes to dtas_gemv_q8_f16.  With
- * cfg == NULL: M <= 32 (M <= 64 with N, K <= 4096) takes the W-streaming kernel where it applies; otherwise
- * M > 64 or K > 4096 take the two-pass route: dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on
- * demand, at most 1 GiB; same sharing rule as the split-K workspace), then dtas_gemm_f16_fused. */
+ * slices meet in the split-K workspace.  A DTAS_GEMM_MFMA row may carry split_k in [1, 16]: that many workgroups share
+ * a tile and meet in the split-K workspace as in dtas_gemm_f16.  One row with a bias or GELU epilogue goes to
+ * dtas_gemv_q8_f16.  With cfg == NULL: M <= 32 (M <= 64 with N, K <= 4096) takes the W-streaming kernel where it
+ * applies; up to 512 rows, while 128x128 tiles fit the chip in one round, the tile kernel dequantises in its W path
+ * (64x64 tiles up to 128 rows, 128x128 beyond; K split over workgroups to fill the chip); beyond that the two-pass route:
+ * dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on demand, at most
+ * 1 GiB; same sharing rule as the split-K workspace), then dtas_gemm_f16_fused. */
 int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias,
                            const void* res1, const void* res2, void* C, int64_t M, int64_t N, int64_t K,
                            int32_t epilogue, const dtas_config* cfg, void* stream);

@@ -218,7 +218,11 @@ def _check_gemm_q8(got, a, wq, scale, bias, r1, r2, kind, oracle):
 Q8_GEMM_CONFIGS = [None,
                    dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64]),
                    dict(variant=0, block=256, vec=8, unroll=3, tile=[128, 128, 64]),
-                   dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64])]
+                   dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64]),
+                   # K split over workgroups: the parts meet in the split-K workspace as the fp16 GEMM's do
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64], split_k=2),
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[128, 128, 64], split_k=3),
+                   dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=8)]
 
 
 @pytest.mark.parametrize("which", range(len(Q8_GEMM_CONFIGS)))
@@ -239,7 +243,7 @@ def test_gemm_q8_every_tile_on_ragged_shapes(oracle, which, M, N, K, kind):
     _check_gemm_q8(out.check(), a, wq, scale, bias, r1, r2, kind, oracle)
 
 
-@pytest.mark.parametrize("M", [1, 16, 32, 64, 256, 2048])
+@pytest.mark.parametrize("M", [1, 16, 32, 64, 128, 256, 512, 2048])
 @pytest.mark.parametrize("N,K,kind", [(7680, 2560, 0), (10240, 2560, 3), (2560, 10240, 0), (2560, 2560, 1)])
 def test_gemm_q8_at_the_models_shapes(oracle, M, N, K, kind):
     rng = np.random.default_rng(M + N + kind)
@@ -337,8 +341,18 @@ def test_gemm_q8_exact_cases_fallback_and_errors(oracle):
     c = torch.empty(9, 96, dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.DtasError, match="8-bit weights come with tiles"):
         ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=0, block=256, vec=8, unroll=2, tile=[128, 128, 64]))
-    with pytest.raises(_lib.DtasError, match="not split"):
-        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=2))
+    with pytest.raises(_lib.DtasError, match=r"split_k must be in \[1, 16\]"):
+        ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, cfg(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=17))
+    # K split over workgroups gives the same bits whoever arrives last, launch after launch
+    big = rng.standard_normal((70, 1056)).astype(np.float16)
+    wq2, scale2 = _weights(130, 1056, 5)
+    first = None
+    for _ in range(5):
+        out = Guarded((70, 130), torch.float16)
+        ops.gemm_q8(dev(big), _words(wq2), dev(scale2), None, out.t, cfg(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=4))
+        got = out.check()
+        first = got if first is None else first
+        assert np.array_equal(got.view(np.uint16), first.view(np.uint16))
     with pytest.raises(_lib.DtasError, match="needs both residuals"):
         ops.gemm_q8(dev(a), _words(wq), dev(scale), None, c, None, _lib.EPI_BIAS_ADD2)
     assert _lib.lib().dtas_gemm_q8_f16_fused(None, None, None, None, None, None, None, 0, 96, 128, 0, None, None) == 0
