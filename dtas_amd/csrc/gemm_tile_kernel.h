@@ -9,6 +9,10 @@
 #ifndef DTAS_GEMM_TILE_GROUP
 #define DTAS_GEMM_TILE_GROUP 8
 #endif
+// Cache policy bits of the direct-to-LDS operand loads (the builtin's last argument: 1 = sc0, 2 = nt, 16 = sc1).
+#ifndef DTAS_GEMM_LOAD_AUX
+#define DTAS_GEMM_LOAD_AUX 0
+#endif
 
 namespace dtas {
 namespace {
@@ -185,16 +189,16 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // (the block's row offset rides in the scalar offset operand: no vector add per load)
 #pragma unroll
     for (int i = 0; i < LA; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + i * NW * 1024), 16, off, i * g_step, 0, DTAS_GEMM_LOAD_AUX);
     if constexpr (WT) {
       const unsigned woff = wt_lane_off(kt);
 #pragma unroll
       for (int i = 0; i < LB; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, woff + i * wt_step, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, woff + i * wt_step, 0, 0, DTAS_GEMM_LOAD_AUX);
     } else if constexpr (!WREG) {
 #pragma unroll
       for (int i = 0; i < LB; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + kABytes + i * NW * 1024), 16, off, i * g_step, 0, DTAS_GEMM_LOAD_AUX);
     }
   };
 
@@ -390,10 +394,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
       char* base = lds + slot * kUnit + (wv & 3u) * 1024;
       if (hi) {
 #pragma unroll
-        for (int q = 0; q < kLoadsW; ++q) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
+        for (int q = 0; q < kLoadsW; ++q) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, DTAS_GEMM_LOAD_AUX);
       } else {
 #pragma unroll
-        for (int q = 0; q < kLoadsA; ++q) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, 0);
+        for (int q = 0; q < kLoadsA; ++q) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(base + q * 4096), 16, voff, q * g16_step, 0, DTAS_GEMM_LOAD_AUX);
       }
     };
     // fragment of 16 rows x 32 k: lane l supplies row (l & 15) and the 8 k of lane group l >> 4.  Which chunk of the
@@ -485,8 +489,8 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // block load b of a unit (the descriptor is named here, not passed down through the lambdas)
     auto fetch_one = [&](bool is_w, unsigned voff, int slot, int b) {
       lds_ptr_t dst = (lds_ptr_t)(lds + slot * kUnit + wv * 1024 + b * NW * 1024);
-      if (is_w) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, dst, 16, voff, b * g_step, 0, 0);
-      else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff, b * g_step, 0, 0);
+      if (is_w) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, dst, 16, voff, b * g_step, 0, DTAS_GEMM_LOAD_AUX);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, voff, b * g_step, 0, DTAS_GEMM_LOAD_AUX);
     };
     // MFMAs of register set `set`; reads of step `ks_next` of (pa, pw) into the other set; half `dpart`
     // of a unit's loads.  DMA: 0 = none, 1 = always, 2 = if `cond`.
@@ -569,13 +573,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // (k-major W: the W blocks take the lane's offset in W, `woff`)
     auto fetch_one = [&](int l_, unsigned voff, char* stage, unsigned woff = 0u) {
       if (l_ < LA)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(stage + wv * 1024 + l_ * NW * 1024), 16, voff, l_ * g_step, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(stage + wv * 1024 + l_ * NW * 1024), 16, voff, l_ * g_step, 0, DTAS_GEMM_LOAD_AUX);
       else if constexpr (WT)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(stage + kABytes + wv * 1024 + (l_ - LA) * NW * 1024), 16,
-                                                 woff + (l_ - LA) * wt_step, 0, 0, 0);
+                                                 woff + (l_ - LA) * wt_step, 0, 0, DTAS_GEMM_LOAD_AUX);
       else
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(stage + kABytes + wv * 1024 + (l_ - LA) * NW * 1024), 16, voff,
-                                                 (l_ - LA) * g_step, 0, 0);
+                                                 (l_ - LA) * g_step, 0, DTAS_GEMM_LOAD_AUX);
     };
     // MFMAs of `set`, the next step's fragment reads, and part `part` of a tile's loads (if `dma`)
     auto step_dma = [&](int set, const char* stage, int ks, bool reads, bool dma, int part, unsigned voff, char* dst, unsigned woff) {
