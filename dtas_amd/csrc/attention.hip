@@ -869,6 +869,12 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
   const int ns = cfg.unroll >= 2 ? cfg.unroll : 2;
   ep.lda = m;
   ep.k_tail = static_cast<unsigned>(m - m_main);
+  // Rows of P a multiple of 4 KiB apart (m = 2048, 4096, ...; a few elements more still count): the same k tile of every
+  // row lies in the same few memory channels, and workgroups that walk k in lockstep queue up there.  Each then starts
+  // at a k tile of its own.  Measured, lockstep / staggered us, 32 heads of 80: n x m = 1024 x 2048 38.0 / 34.2, 2048 x
+  // 2048 73.3 / 57.5, 4096 x 2048 137 / 110, 2048 x 4096 131 / 103, 1024 x 8192 135 / 103, 2048 x 6144 174 / 151, 2048 x
+  // 2049 77.6 / 70.3; other row pitches lose 1-7 % (1024 x 1024 18.9 / 19.6, 2048 x 1024 32.8 / 35.4, 2048 x 1984 53.2 / 54.8).
+  ep.k_stagger = (m * 2) % 4096 < 32 ? 1u : 0u;
 #define DTAS_PV_CASE(BM_, BN_, NS_) \
   if (bm == BM_ && bn == BN_ && ns == NS_) return launch_mfma<BM_, BN_, 2, 2, NS_, true>(s, a, w, ep, out, n, d, m_main, sk, b)
   // (four stages measured level with or behind three on every tile, n = m = 256 .. 4096: not instantiated)

@@ -30,6 +30,7 @@ struct GemmEpilogue {
   unsigned tiles_unsplit; // one problem only: tiles [0, tiles_unsplit) are computed whole, only the rest is split over nsplit workgroups
   unsigned k_tail;        // k-major W only (P.V): A's rows and W hold k_tail (< 8) more k than K, which the MFMA loop leaves out and
                           // the epilogue adds (A's rows are then fetched at whatever alignment lda gives them)
+  unsigned k_stagger;     // k-major W only (P.V): workgroup i starts at its k tile i mod (its k tiles) and wraps around
 };
 
 // Attention scores, fused_NT_matmul1_divide_maximum_minimum_cast2 (before_dl.py:116-160):

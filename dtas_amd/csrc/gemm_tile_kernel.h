@@ -175,16 +175,27 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
   const int kt_per = (ktiles_all + static_cast<int>(my_split) - 1) / static_cast<int>(my_split);
   const int kt0 = static_cast<int>(z) * kt_per;
   const int ktiles = ktiles_all - kt0 < kt_per ? (ktiles_all - kt0 > 0 ? ktiles_all - kt0 : 0) : kt_per;
+  // k-major W (P.V): a workgroup starts at a k tile of its own and wraps around.  The rows of P lie a power of two apart
+  // when the key count is one, so the same k tile of every row maps to the same few memory channels, and workgroups
+  // that all start at k tile 0 walk the channels in lockstep (the bare load pattern of 32 x 2048 x 2048 with 256-row
+  // tiles: 4.3 TB/s in lockstep, 5.8 staggered, 6.0 with rows 4224 bytes apart).  Which k tile comes when is a function
+  // of the tile alone, so a launch still adds in the same order every time.
+  const int kt_rot = WT && ep.k_stagger && ktiles > 1 ? static_cast<int>(__builtin_amdgcn_readfirstlane((batch_u * total + pid) % static_cast<unsigned>(ktiles))) : 0;
+  auto kt_abs = [&](int kt) -> int {  // k tile of the matrix that is this workgroup's kt-th
+    if constexpr (!WT) return kt0 + kt;
+    const int v = kt + kt_rot;
+    return kt0 + (v >= ktiles ? v - ktiles : v);
+  };
 
   // k-major W: this lane's byte offset in W for k tile kt of this workgroup (k rows past K lie past the descriptor's range)
   auto wt_lane_off = [&](int kt) -> unsigned {
-    return wt_col_ok ? wt_off + static_cast<unsigned>(static_cast<int64_t>(kt0 + kt) * kBK * N * 2) : kOob;
+    return wt_col_ok ? wt_off + static_cast<unsigned>(static_cast<int64_t>(kt_abs(kt)) * kBK * N * 2) : kOob;
   };
   // tile kt -> LDS stage kt % NS, asynchronously (completion is counted by vmcnt)
   auto fetch = [&](int kt) {
     // a chunk past K is pointed out of range; K % 8 == 0, so chunks are all-in or all-out
-    const unsigned off = (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K)
-                             ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+    const unsigned off = (static_cast<int64_t>(kt_abs(kt)) * kBK + c_in * 8 < K)
+                             ? g_off + static_cast<unsigned>(kt_abs(kt)) * kRowBytes : kOob;
     char* base = lds + (kt % NS) * kStage + wv * 1024;
     // (the block's row offset rides in the scalar offset operand: no vector add per load)
 #pragma unroll
@@ -220,7 +231,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
 #pragma unroll
     for (int i = 0; i < kWtItems; ++i) {
       const unsigned item = t + i * 64 * NW, r = item >> 2, c4 = item & 3u;
-      const int64_t row = n0 + r, k = static_cast<int64_t>(kt0 + kt) * kBK + c4 * 16;
+      const int64_t row = n0 + r, k = static_cast<int64_t>(kt_abs(kt)) * kBK + c4 * 16;
       const bool in = row < N && k < K;  // K % 32 == 0: a piece and its scale group are all-in or all-out
       wt_reg[SLOT][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rv, in ? static_cast<unsigned>(row * K + k) : kOob, 0, 0);
       wq_scale[SLOT][i] = __builtin_amdgcn_raw_buffer_load_b16(rs, in ? static_cast<unsigned>((row * (K >> 5) + (k >> 5)) * 2) : kOob, 0, 0);
@@ -388,7 +399,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     const unsigned g16 = (8u * (wv & 3u) + r16) * row_bytes + c16 * 16u;
     const unsigned g16_step = 32u * row_bytes;
     auto lane_off16 = [&](int kt) -> unsigned {
-      return (static_cast<int64_t>(kt0 + kt) * kBK + c16 * 8 < K && kt < ktiles) ? g16 + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+      return (static_cast<int64_t>(kt_abs(kt)) * kBK + c16 * 8 < K && kt < ktiles) ? g16 + static_cast<unsigned>(kt_abs(kt)) * kRowBytes : kOob;
     };
     auto fetch16 = [&](int slot, unsigned voff) {
       char* base = lds + slot * kUnit + (wv & 3u) * 1024;
@@ -484,7 +495,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     const unsigned a_frag = wm * WTM * 128u, b_frag = wn * WTN * 128u;
     // per-lane byte offset of this lane's chunk in k tile kt of either operand (out of range past K)
     auto lane_off = [&](int kt) -> unsigned {
-      return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+      return (static_cast<int64_t>(kt_abs(kt)) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt_abs(kt)) * kRowBytes : kOob;
     };
     // block load b of a unit (the descriptor is named here, not passed down through the lambdas)
     auto fetch_one = [&](bool is_w, unsigned voff, int slot, int b) {
@@ -567,7 +578,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     // loop carries no conditions.
     constexpr int kL = LA + LB;
     auto lane_off = [&](int kt) -> unsigned {
-      return (static_cast<int64_t>(kt0 + kt) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt0 + kt) * kRowBytes : kOob;
+      return (static_cast<int64_t>(kt_abs(kt)) * kBK + c_in * 8 < K) ? g_off + static_cast<unsigned>(kt_abs(kt)) * kRowBytes : kOob;
     };
     // block load l (0 .. kL-1: A blocks, then W blocks) of a tile into `stage`
     // (k-major W: the W blocks take the lane's offset in W, `woff`)

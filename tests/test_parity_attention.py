@@ -187,6 +187,24 @@ def test_pv_split_over_workgroups(oracle, tile, stages, split, heads, n, m, d):
         first = got
 
 
+@pytest.mark.parametrize("tile,stages", [((64, 128), 3), ((128, 128), 2), ((128, 128), 3), ((256, 128), 3), ((64, 64), 2)])
+@pytest.mark.parametrize("heads,n,m,d", [(5, 300, 2048, 80), (3, 130, 2049, 80), (2, 70, 4096, 128), (3, 260, 2056, 80), (7, 64, 2048, 64)])
+def test_pv_with_rows_of_p_a_multiple_of_4_kib_apart(oracle, tile, stages, heads, n, m, d):
+    """Key counts whose rows of P lie (nearly) a multiple of 4 KiB apart: every workgroup starts its walk over the keys
+    at a k tile of its own and wraps around (the last, partial k tile and the m % 8 tail then come mid-walk).  The
+    order is a function of the tile, so two runs give the same bits."""
+    p, v = _pv_inputs(heads, n, m, d, n + m + d)
+    row = cfg(variant=_lib.GEMM_MFMA, block=256, vec=8, unroll=stages, tile=[tile[0], tile[1], 64])
+    first = None
+    for _ in range(2):
+        out = Guarded((heads, n, d), torch.float16)
+        ops.attn_pv(dev(p), dev(v), out.t, row)
+        got = out.check()
+        _check_pv(got, p, v, oracle)
+        assert first is None or np.array_equal(first, got)
+        first = got
+
+
 @pytest.mark.parametrize("rows", [1, 2, 4, 8])
 @pytest.mark.parametrize("heads,n,m,d", [(32, 1, 515, 80), (32, 1, 4096, 80), (3, 3, 64, 8), (2, 11, 1000, 128), (1, 8, 1, 16),
                                          (2, 5, 300, 264)])
