@@ -792,8 +792,16 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       const int64_t t128 = heads * ceil_div(n, 128);
       if (t128 <= kNumCU / 2) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, bn == 128 ? 3 : 2, {64, bn, kBK}, 1, 0};
       else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
-      else if (bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
-      else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
+      else if (bn == 128) {
+        cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
+        // Rows of P off the 16-byte grid cost the loads of a workgroup more, and a last round of 256-row tiles that leaves
+        // CUs idle then shows: 64-row tiles (two workgroups per CU) instead -- n = m = 1025: 29.9 against 35.0 us (160
+        // workgroups of 256 rows), 2049: 84.9 / 94.9, 3001: 159 / 170; with rows on the grid the big tiles stay ahead
+        // whatever the fill (1088: 25.0 against 29.0), and so they do off the grid from three quarters of the CUs on
+        // (1281: 43.9 / 45.9, 1537: 50.0 / 54.0)
+        const int64_t last_round = (heads * ceil_div(n, 256)) % kNumCU;
+        if (!p_vec && last_round != 0 && last_round * 10 < kNumCU * 7) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {64, 128, kBK}, 1, 0};
+      } else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
       // 128-row tiles (one workgroup per CU) gain only while all parts run at once: 512 rows against 4096 keys
       // take 47 us in two parts, 58 whole, 80 in eight.  Partial tiles of 256 rows cost more to combine than a
       // split saves.
