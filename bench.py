@@ -472,6 +472,22 @@ def families(rows: list) -> dict:
             if r["bound"] == "mfma":
                 out[key + "_tflops"] = round(r["tflops"], 1)
             out[key + ("_frac" if r["bound"] == "mfma" else "_frac_hbm")] = round(r["frac"], 3)
+    # the graph's other PrimFuncs (attention matmuls, fused epilogues, 8-bit weights, index-only ops), at their larger points
+    for r in rows:
+        op, n = r["op"], r["n"]
+        frac = "_frac" if r["bound"] == "mfma" else "_frac_hbm"
+        if op in ("attn_scores_f16_f32", "attn_pv_f16") and n >= 1024:
+            out[f"fam_{op}_n{n}_us"] = round(r["us"], 2)
+            out[f"fam_{op}_n{n}_frac_hbm"] = round(r["frac"], 3)
+        elif op in ("gemm_q8_f16", "gemm_add2_f16", "gemm_gelu_f16") and n >= 16:
+            key = f"fam_{op}_M{n}_{r['NK'][0]}x{r['NK'][1]}"
+            out[key + "_us"] = round(r["us"], 2)
+            out[key + frac] = round(r["frac"], 3)
+        elif op in ("gemv_q8_f16", "gemv_q8_f32", "gemv_f32"):
+            out[f"fam_{op}_{r['NK'][0]}x{r['NK'][1]}_frac_hbm"] = round(r["frac"], 3)
+        elif op in ("layer_norm_f32", "take_q8_f16", "take_f16", "rotary_f16", "split3_f16", "swap_axes_f16", "attn_mask_f16",
+                    "softmax_temperature_f32") and n >= 4096:
+            out[f"fam_{op}_n{n}_frac_hbm"] = round(r["frac"], 3)
     return out
 
 
