@@ -156,6 +156,7 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   // no candidate is faster than it streams W: TB/s measured at M = 64 against a 50280 x 2560 W
   const double w_mb = 2.0 * static_cast<double>(n) * static_cast<double>(k) * 1e-6;
   auto floored = [&](double us, double tbs) { return us > w_mb / tbs ? us : w_mb / tbs; };
+  auto relief = [](double fill) { return fill <= 0.5 ? 0.63 : 0.63 + 0.74 * (fill - 0.5); };
   {
     // 256x256 on 8 wavefronts (16x16x32 MFMA): a round of the chip costs ~8 us plus 1.50 us per k tile with every CU
     // busy; with half of the CUs or fewer busy the card clocks higher and a k tile takes 0.63 of that, linearly in
@@ -163,7 +164,6 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     // (tail_split_256), which costs ~15 / 18 / 21 us to combine the partial tiles.
     const int64_t tiles = static_cast<int64_t>(tiles_of(256, 256));
     const int64_t full = tiles / kNumCU, rem = tiles % kNumCU;
-    auto relief = [](double fill) { return fill <= 0.5 ? 0.63 : 0.63 + 0.74 * (fill - 0.5); };
     double us = static_cast<double>(full) * (8.0 + 1.50 * kt);
     if (rem > 0) {
       int split = 1;
@@ -175,6 +175,17 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
         us += 8.0 + 1.50 * kt * relief(static_cast<double>(rem) / kNumCU);
     }
     consider(floored(us, 3.5), 256, 256, 512, 2, 0);
+  }
+  {
+    // 192x256 on 8 wavefronts (96x64 each, the same loop): 1.18 us per k tile with every CU busy -- as many flops per us
+    // as 256x256 -- and the same relief in a partly filled round; there for the tile counts it fills the chip better
+    // with (M = 4096 against N = 2560: 220 tiles where 256x256 makes 160, 196 against 219 us at K = 10240; 3072 x 4096:
+    // 256 tiles against 192; 2048 x 10240: 440 against 320)
+    const int64_t tiles = static_cast<int64_t>(tiles_of(192, 256));
+    const int64_t full = tiles / kNumCU, rem = tiles % kNumCU;
+    double us = static_cast<double>(full) * (8.0 + 1.18 * kt);
+    if (rem > 0) us += 8.0 + 1.18 * kt * relief(static_cast<double>(rem) / kNumCU);
+    consider(floored(us, 3.5), 192, 256, 512, 2, 1);
   }
   // 256x128 on 8 wavefronts (64x64 each, the 16x16x32 ring loop): 1.00 us per k tile against 1.045 us on 4 wavefronts
   consider(floored(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.0 * kt, 3.5), 256, 128, 512, 2, 1);

@@ -767,9 +767,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const half_t* _
     constexpr int kTilePairs = BM * BN / 2;  // 8-byte units per partial tile
     const unsigned tile_g = batch_u * total + pid - unsplit;  // this tile among all problems' tiles
     unsigned long long* tile_ws = reinterpret_cast<unsigned long long*>(ws) + static_cast<size_t>(tile_g) * nsplit * kTilePairs;
-    unsigned long long* mine = tile_ws + static_cast<size_t>(z) * kTilePairs + wv * (MT * NT * 8 * 64);
     // pair q of a lane's accumulators (in whatever order the main loop keeps them)
-    constexpr int kPer = MT * NT * 8;  // 8-byte units per lane and partial tile
+    constexpr int kPer = M16 ? MT16 * NT16 * 2 : MT * NT * 8;  // 8-byte units per lane and partial tile
+    static_assert(kPer * 64 * NW == kTilePairs, "the wavefronts' partial tiles tile the workgroup's");
+    unsigned long long* mine = tile_ws + static_cast<size_t>(z) * kTilePairs + wv * (kPer * 64);
     auto pair_get = [&](int q, int e) -> float {
       if constexpr (M16) return acc16[q / (NT16 * 2)][(q / 2) % NT16][2 * (q % 2) + e];
       else return acc[q / (NT * 8)][(q / 8) % NT][2 * (q % 8) + e];

@@ -106,23 +106,27 @@ int describe_gemm(int64_t M, int64_t N, int64_t K, const dtas_config& cfg, int64
   if (cfg.vec != 8) return fail("gemm: vector width must be 8 (128 bit) or 1, got %d", cfg.vec);
   if (cfg.variant == DTAS_GEMM_MFMA) {
     const int bm = cfg.tile[0], bn = cfg.tile[1];
+    // tiles of 192 rows (8 wavefronts only): between the others in size, for tile counts that fill the chip better
+    const bool with_192 = bm == 192 && (bn == 256 || bn == 128);  // (192 columns: the epilogue's lane map wants wavefront tiles of 64 columns)
     const bool known = (bm == 256 && bn == 256) || (bm == 256 && bn == 128) || (bm == 128 && bn == 256) ||
                        (bm == 128 && bn == 128) || (bm == 64 && bn == 128) || (bm == 128 && bn == 64) ||
-                       (bm == 64 && bn == 64);
+                       (bm == 64 && bn == 64) || with_192;
     if (!known || cfg.tile[2] != kBK) return fail("gemm: no MFMA kernel for tile %dx%dx%d", bm, bn, cfg.tile[2]);
     // 256x256 comes as 8 wavefronts (two per SIMD, 128x64 each) or 4 (one per SIMD, 128x128 each); 256x128 and
     // 128x256 as 4 wavefronts on whole-tile stages or 8 (64x64 each) on the 16x16x32 ring loop (128x128 on that
     // loop, 64x32 per wavefront, measured slower than on 4 wavefronts at every M: not instantiated)
     const bool four_waves = bm == 256 && bn == 256 && cfg.block == 256;
-    const bool eight_waves = bm + bn == 384 && cfg.block == 512;
+    const bool eight_waves = (bm + bn == 384 || with_192) && cfg.block == 512;
+    if (with_192 && !eight_waves) return fail("gemm: the %dx%d MFMA kernel uses 512 threads, got %d", bm, bn, cfg.block);
     if (cfg.block != mfma_threads(bm, bn) && !four_waves && !eight_waves)
       return fail("gemm: the %dx%d MFMA kernel uses %d threads, got %d", bm, bn, mfma_threads(bm, bn), cfg.block);
     if (K * 2 * (bm > bn ? bm : bn) >= (int64_t{1} << 31)) return fail("gemm: K=%lld too large for 32-bit tile offsets", (long long)K);
     const int64_t tm = ceil_div(M, bm), tn = ceil_div(N, bn);
     if (tm * tn > 0x7fffffff) return fail("gemm: too many tiles");
     // cfg.unroll = LDS stages (the depth of the load pipeline); 0 or 1 = as many as fit
-    if (cfg.unroll < 0 || cfg.unroll > mfma_max_stages(bm, bn))
-      return fail("gemm: the %dx%d tile holds at most %d LDS stages, got %d", bm, bn, mfma_max_stages(bm, bn), cfg.unroll);
+    const int max_stages = with_192 ? 2 : mfma_max_stages(bm, bn);
+    if (cfg.unroll < 0 || cfg.unroll > max_stages)
+      return fail("gemm: the %dx%d tile holds at most %d LDS stages, got %d", bm, bn, max_stages, cfg.unroll);
     int nsplit = cfg.split_k < 1 ? 1 : cfg.split_k;
     if (nsplit > 16) return fail("gemm: split_k must be in [1, 16], got %d", cfg.split_k);
     // split_k = 0 on the 8-wavefront 256x256 tile: only the tiles of a last, partly filled round are split
@@ -220,6 +224,8 @@ int launch_tile_f16(const dtas_config& cfg, hipStream_t s, const half_t* a, cons
   if (cfg.block == 512) {  // 8 wavefronts on the 16x16x32 ring loop
     if (bm == 256 && bn == 128) return launch_mfma<256, 128, 4, 2, 2, false, false, true>(s, a, w, b, c, M, N, K, sk, batch);
     if (bm == 128 && bn == 256) return launch_mfma<128, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, sk, batch);
+    if (bm == 192 && bn == 256) return launch_mfma<192, 256, 2, 4, 2, false, false, true>(s, a, w, b, c, M, N, K, sk, batch);
+    if (bm == 192 && bn == 128) return launch_mfma<192, 128, 4, 2, 2, false, false, true>(s, a, w, b, c, M, N, K, sk, batch);
   }
   if (bm == 256 && bn == 128) return ns == 2 ? launch_mfma<256, 128, 2, 2, 2>(s, a, w, b, c, M, N, K, sk, batch)
                                              : launch_mfma<256, 128, 2, 2, 3>(s, a, w, b, c, M, N, K, sk, batch);

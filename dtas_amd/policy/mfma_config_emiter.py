@@ -16,7 +16,7 @@ from ..common.config import MFMAConfig, Range
 from .base_config_emiter import BaseConfigEmiter
 
 # (micro_x, micro_y) per wavefront of the 2x2-wavefront kernels (the 256x256 tile runs 2x4 wavefronts)
-_TILES = [(4, 4), (4, 2), (2, 4), (2, 2), (1, 2), (2, 1), (1, 1)]
+_TILES = [(4, 4), (3, 4), (4, 2), (2, 4), (2, 2), (1, 2), (2, 1), (1, 1)]
 _LDS = 160 * 1024
 
 
@@ -29,7 +29,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
 
     @staticmethod
     def max_stages(tile_m: int, tile_n: int) -> int:
-        return 2 if tile_m + tile_n >= 512 else 3 if tile_m + tile_n >= 384 else 4
+        return 2 if tile_m + tile_n >= 512 or tile_m == 192 else 3 if tile_m + tile_n >= 384 else 4
 
     def preferred(self, m_hi: int, N: int, K: int = 4096):
         """(tile_m, tile_n, stages, split_k) under the cost model fitted to sweeps on an MI355X (the same
@@ -68,7 +68,11 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 us256 += 8.0 + 1.50 * cdiv(ktiles, split) * relief(rem * split / cus) + 12.0 + 3.0 * (split - 1)
             else:
                 us256 += 8.0 + 1.50 * ktiles * relief(rem / cus)
+        # 192x256 on 8 wavefronts (96x64 each): 1.18 us per k tile with every CU busy, the same relief
+        full192, rem192 = divmod(tiles(192, 256), cus)
+        us192 = full192 * (8.0 + 1.18 * ktiles) + ((8.0 + 1.18 * ktiles * relief(rem192 / cus)) if rem192 else 0.0)
         cands = [(floored(us256, 3.5), (256, 256, 2, 0)),
+                 (floored(us192, 3.5), (192, 256, 2, 1)),
                  (floored(rounds(tiles(256, 128), cus) * 1.0 * ktiles, 3.5), (256, 128, 2, 1)),
                  (floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1))]
         for split in (1, 2, 3, 4):
@@ -198,6 +202,9 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 if (mx, my) == (4, 4):
                     # the 256x256 kernel runs 2x4 wavefronts of 128x64 (two per SIMD)
                     c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 2, 4, 4, 2, 512
+                if (mx, my) == (3, 4):
+                    # 192x256: 2x4 wavefronts of 96x64 on the same ring loop
+                    c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 2, 4, 3, 2, 512
                 if (mx, my) == (4, 2) and stages == 2:
                     # 256x128 with two "stages": 4x2 wavefronts of 64x64 on the ring loop of the 256x256 kernel
                     c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 4, 2, 2, 2, 512

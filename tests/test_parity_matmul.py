@@ -281,18 +281,28 @@ def test_gemm_streaming_tile_is_reproducible_exact_and_refuses_what_it_cannot_ho
             _lib.describe_launch(_lib.OP_GEMM_F16, 8, 64, 64, cfg(variant=_lib.GEMM_STREAM, block=block, vec=8, unroll=1, tile=tile))
 
 
-@pytest.mark.parametrize("bm,bn", [(256, 128), (128, 256)])
+@pytest.mark.parametrize("bm,bn", [(256, 128), (128, 256), (192, 256), (192, 128)])
 @pytest.mark.parametrize("split", [1, 2, 3])
-@pytest.mark.parametrize("M,N,K", [(5, 7, 8), (300, 260, 200), (257, 513, 1096), (512, 512, 64), (256, 256, 4096), (700, 300, 4104)])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 8), (300, 260, 200), (257, 513, 1096), (512, 512, 64), (256, 256, 4096), (700, 300, 4104),
+                                   (193, 257, 72), (960, 520, 264)])
 def test_gemm_rectangular_tiles_with_eight_wavefronts(oracle, bm, bn, split, M, N, K):
-    # block = 512 on 256x128 / 128x256: 64x64 per wavefront on the ring loop of the 256x256 kernel
+    # block = 512 on 256x128 / 128x256 / 192x256 / 192x128: 64x64, 96x64 or 48x64 per wavefront on the ring loop of the
+    # 256x256 kernel (the ring's units are the larger side's rows of a k tile)
     a, w = _inputs(M, N, K, M + N + K)
     bias = np.random.default_rng(1).uniform(-1, 1, N).astype(np.float16)
     out = Guarded((M, N), torch.float16)
     c = cfg(variant=_lib.GEMM_MFMA, block=512, vec=8, unroll=2, tile=[bm, bn, 64], split_k=split)
     ops.gemm(dev(a), dev(w), dev(bias), out.t, c)
     _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
-    assert list(_lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c).launch_args)[3:5] == [512, 5 * 256 * 128]
+    assert list(_lib.describe_launch(_lib.OP_GEMM_F16, M, N, K, c).launch_args)[3:5] == [512, 5 * max(bm, bn) * 128]
+
+
+def test_gemm_tiles_of_192_rows_come_with_eight_wavefronts_and_two_stages():
+    for bad, msg in ((dict(block=256), "512 threads"), (dict(unroll=3), "at most 2 LDS stages"), (dict(tile=[256, 192, 64]), "no MFMA kernel")):
+        c = dict(variant=_lib.GEMM_MFMA, block=512, vec=8, unroll=2, tile=[192, 256, 64])
+        c.update(bad)
+        with pytest.raises(_lib.DtasError, match=msg):
+            _lib.describe_launch(_lib.OP_GEMM_F16, 512, 512, 512, cfg(**c))
 
 
 @pytest.mark.parametrize("mv,r", [(2, 1), (2, 2), (2, 4), (4, 1), (4, 2), (4, 4)])
@@ -612,7 +622,22 @@ FUSED_CONFIGS = [None,
                  dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64]),
                  dict(variant=0, block=256, vec=8, unroll=4, tile=[64, 64, 64], split_k=3),
                  dict(variant=1, block=512, vec=8, unroll=4, tile=[80, 16, 32]),
-                 dict(variant=0, block=512, vec=8, unroll=2, tile=[256, 128, 64], split_k=2)]
+                 dict(variant=0, block=512, vec=8, unroll=2, tile=[256, 128, 64], split_k=2),
+                 dict(variant=0, block=512, vec=8, unroll=2, tile=[192, 256, 64]),
+                 dict(variant=0, block=512, vec=8, unroll=2, tile=[192, 128, 64], split_k=2)]
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3])
+@pytest.mark.parametrize("tile,split", [((192, 256), 1), ((192, 256), 2), ((192, 128), 1), ((192, 128), 3)])
+def test_gemm_fused_epilogues_on_tiles_of_192_rows(oracle, kind, tile, split):
+    M, N, K = 400, 520, 264      # three tile rows, the last one ragged
+    a, w, bias, r1, r2 = _fused_inputs(M, N, K, M + N + K + kind)
+    res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+    out = Guarded((M, N), torch.float32 if kind == 2 else torch.float16)
+    c = cfg(variant=0, block=512, vec=8, unroll=2, tile=[tile[0], tile[1], 64], split_k=split)
+    ops.gemm(dev(a), dev(w), dev(bias), out.t, c, epilogue=kind, res1=res[0], res2=res[1])
+    want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+    _check_fused(out.check(), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
 
 
 @pytest.mark.parametrize("kind", [1, 2, 3])
