@@ -189,6 +189,13 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   }
   // 256x128 on 8 wavefronts (64x64 each, the 16x16x32 ring loop): 1.00 us per k tile against 1.045 us on 4 wavefronts
   consider(floored(gemm_rounds(tiles_of(256, 128), kNumCU) * 1.0 * kt, 3.5), 256, 128, 512, 2, 1);
+  // 192x128 on 8 wavefronts (48x64 each), where its tiles fill three quarters of the chip or more in one round: ~6 us plus
+  // 0.66 us per k tile (2048 x 2560 x 2560: 220 tiles, 29.8 us against 32.6 for the 160 tiles of 256x128; 1536 x 4096 x 4096:
+  // 48.2 against 49.7).  With fewer tiles the split tiles are ahead of what this model says of them (1024 x 2560 x 4096:
+  // 37.0 against 31.3), a second round costs it more than its share (1536 x 11008 x 4096: 164 against 145), and past 64 k
+  // tiles each one takes it 0.8 us (1536 x 4096 x 11008: 144 against 138 for 256x256)
+  if (tiles_of(192, 128) <= kNumCU && tiles_of(192, 128) * 4 >= 3 * kNumCU && kt <= 64)
+    consider(floored(6.0 + gemm_rounds(tiles_of(192, 128), kNumCU) * 0.66 * kt, 3.5), 192, 128, 512, 2, 1);
   consider(floored(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 3.1), 128, 128, 256, 2, 1);
   for (int split = 1; split <= 4; ++split) {
     if (split > 1 && ktiles / split < 8) continue;

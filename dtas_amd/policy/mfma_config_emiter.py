@@ -16,7 +16,7 @@ from ..common.config import MFMAConfig, Range
 from .base_config_emiter import BaseConfigEmiter
 
 # (micro_x, micro_y) per wavefront of the 2x2-wavefront kernels (the 256x256 tile runs 2x4 wavefronts)
-_TILES = [(4, 4), (3, 4), (4, 2), (2, 4), (2, 2), (1, 2), (2, 1), (1, 1)]
+_TILES = [(4, 4), (3, 4), (4, 2), (3, 2), (2, 4), (2, 2), (1, 2), (2, 1), (1, 1)]
 _LDS = 160 * 1024
 
 
@@ -73,8 +73,12 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         us192 = full192 * (8.0 + 1.18 * ktiles) + ((8.0 + 1.18 * ktiles * relief(rem192 / cus)) if rem192 else 0.0)
         cands = [(floored(us256, 3.5), (256, 256, 2, 0)),
                  (floored(us192, 3.5), (192, 256, 2, 1)),
-                 (floored(rounds(tiles(256, 128), cus) * 1.0 * ktiles, 3.5), (256, 128, 2, 1)),
-                 (floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1))]
+                 (floored(rounds(tiles(256, 128), cus) * 1.0 * ktiles, 3.5), (256, 128, 2, 1))]
+        # 192x128 on 8 wavefronts (48x64 each), one round that fills three quarters of the chip or more: ~6 us plus
+        # 0.66 us per k tile up to 64 of them
+        if 3 * cus <= 4 * tiles(192, 128) <= 4 * cus and ktiles <= 64:
+            cands.append((floored(6.0 + rounds(tiles(192, 128), cus) * 0.66 * ktiles, 3.5), (192, 128, 2, 1)))
+        cands.append((floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1)))
         for split in (1, 2, 3, 4):
             if split > 1 and ktiles // split < 8:
                 continue
@@ -205,6 +209,10 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 if (mx, my) == (3, 4):
                     # 192x256: 2x4 wavefronts of 96x64 on the same ring loop
                     c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 2, 4, 3, 2, 512
+                if (mx, my) == (3, 2):
+                    # 192x128: 4x2 wavefronts of 48x64 (16x16x32 blocks) on the ring loop; the vocabulary's 32-wide micro
+                    # blocks do not express 48 rows, so the 2x2 shape stands for the tile's extents
+                    c.block_threads = 512
                 if (mx, my) == (4, 2) and stages == 2:
                     # 256x128 with two "stages": 4x2 wavefronts of 64x64 on the ring loop of the 256x256 kernel
                     c.i, c.j, c.micro_shape_x, c.micro_shape_y, c.block_threads = 4, 2, 2, 2, 512

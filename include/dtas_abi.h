@@ -98,7 +98,8 @@ enum dtas_variant {
   DTAS_GEMM_MFMA = 0,     /* LDS-tiled MFMA, tile = tile[0] x tile[1] x 64 with tile[0], tile[1] in {64, 128, 256}
                              (64x256 and 256x64 excepted); block 256 (4 wavefronts), or 512 (8 wavefronts, 16x16x32
                              MFMA, a ring of five operand units instead of `unroll` stages) for 256x256, 256x128
-                             and 128x256; 256x256 takes either */
+                             and 128x256; 256x256 takes either.  192x256 and 192x128 exist with block 512 and
+                             unroll 2 only */
   DTAS_GEMM_SKINNY = 1,   /* small M: weight-streaming MFMA 16x16x32, split over N and K */
   DTAS_GEMM_ROWS = 2,     /* M <= 4: W streamed once in whole rows (tile[1] per wavefront) against tile[0] >= M
                              rows of A on the vector ALU; tile = {2|4, 1|2|4, 8}, block 64 / 128 / 256 */

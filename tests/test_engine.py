@@ -247,7 +247,7 @@ def test_builtin_tables_name_a_launchable_kernel_for_every_bucket_and_shape():
                 assert list(again.launch_args) == list(info.launch_args), (M, N, K)
                 assert info.bucket_lo <= max(M, 1) and (M <= info.bucket_hi or info.index == 511), (M, N, K, info.bucket_lo, info.bucket_hi)
                 if c.variant == _lib.GEMM_MFMA:
-                    assert (c.tile[0], c.tile[1]) in {(256, 256), (192, 256), (256, 128), (128, 128), (128, 64), (64, 64)} and c.tile[2] == 64
+                    assert (c.tile[0], c.tile[1]) in {(256, 256), (192, 256), (256, 128), (192, 128), (128, 128), (128, 64), (64, 64)} and c.tile[2] == 64
                     # (split_k = 0, the 8-wavefront 256x256 tile only: the library splits just the tiles of a partly filled last round)
                     assert (c.split_k == 0 and tuple(c.tile[:2]) == (256, 256) and c.block == 512) or \
                         (1 <= c.split_k <= 4 and (c.split_k == 1 or -(-K // 64) // c.split_k >= 8)), (M, N, K, c.split_k)
