@@ -264,7 +264,7 @@ __global__ void __launch_bounds__(kBlock) take_f16_kernel(const u32x4* __restric
        t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     int64_t row = ids[t / per_row];
     row = row < 0 ? 0 : row >= V ? V - 1 : row;
-    out[t] = A[row * per_row + t % per_row];
+    store_stream(A[row * per_row + t % per_row], out + t);
   }
 }
 __global__ void __launch_bounds__(kBlock) take_f16_scalar_kernel(const half_t* __restrict__ A, const int* __restrict__ ids,
@@ -359,8 +359,72 @@ __global__ void __launch_bounds__(kBlock) rotary20_kernel(const half_t* __restri
       }
       raw = __builtin_bit_cast(u32x4, r);
     }
-    *reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row) * d + 8 * v) = raw;
+    store_stream(raw, reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row) * d + 8 * v));
     if (pieces - t <= step) break;   // (t + step might wrap in 32 bits)
+  }
+}
+
+// The same for rows of 3 .. 64 pieces (the model's have 10) without the partner loads: a wavefront takes whole rows,
+// floor(64 / pieces per row) of them, one piece per lane (60 of the model's 64 lanes work), and the three lanes of a
+// row that hold the rotated pieces get their partners' words from one another through ds_bpermute -- piece 0 wants
+// elements 10..17 (words 1..3 of the next lane, word 0 of the one after), piece 1 elements 18, 19 (word 1 of the next
+// lane) and 0..5 (words 0..2 of the lane before), piece 2 elements 6..9 (word 3 two lanes back, word 0 one back).
+// The tables' 8 elements come as one 16-byte load (piece 2: elements 12..19, of which it uses the upper four), asked
+// for together with the piece.  At n = 4096 (32 heads, d = 80): 9.2 us against 11.5 for the kernel above, which was
+// 12.2 before its stores became streaming ones; two or more chunks of rows per pass of a wavefront are slower.
+__global__ void __launch_bounds__(kBlock) rotary20_rows_kernel(const half_t* __restrict__ A, const half_t* __restrict__ cs,
+                                                               const half_t* __restrict__ sn, half_t* __restrict__ out,
+                                                               uint32_t rows, uint32_t heads, uint32_t per_row, int64_t pos0) {
+#pragma clang fp contract(off)
+  typedef u32x4 __attribute__((aligned(8))) u32x4_a8;
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t rows_per_chunk = 64u / per_row;
+  const uint32_t rr = lane / per_row, v = lane - rr * per_row;
+  const bool lane_used = rr < rows_per_chunk;
+  const uint32_t chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
+  const uint32_t waves = gridDim.x * (kBlock / 64);
+  // the lanes the partner words come from, as byte addresses for ds_bpermute
+  const int from0 = static_cast<int>(((v == 0 ? lane + 2 : lane - 1) & 63u) << 2);
+  const int from_next = static_cast<int>(((lane + 1) & 63u) << 2), from_prev = static_cast<int>(((lane - 1) & 63u) << 2);
+  const int from2 = v == 0 ? from_next : from_prev;
+  const int from3 = v == 0 ? from_next : static_cast<int>(((lane - 2) & 63u) << 2);
+  const uint32_t table_at = v < 2 ? 8 * v : 12;
+  for (uint32_t c = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); c < chunks; c += waves) {   // (uniform over the wavefront)
+    const uint32_t row = c * rows_per_chunk + rr;
+    const bool on = lane_used && row < rows;
+    const int64_t at = (static_cast<int64_t>(row) * per_row + v) * 8;
+    u32x4 raw = {0, 0, 0, 0}, cw = {0, 0, 0, 0}, sw = {0, 0, 0, 0};
+    if (on) raw = load_stream(reinterpret_cast<const u32x4*>(A + at));
+    if (on && v < 3) {
+      const int64_t toff = (pos0 + row / heads) * 20 + table_at;
+      cw = *reinterpret_cast<const u32x4_a8*>(cs + toff);
+      sw = *reinterpret_cast<const u32x4_a8*>(sn + toff);
+    }
+    const uint32_t w0 = __builtin_amdgcn_ds_bpermute(from0, static_cast<int>(raw[0]));
+    const uint32_t w1n = __builtin_amdgcn_ds_bpermute(from_next, static_cast<int>(raw[1]));
+    const uint32_t w1p = __builtin_amdgcn_ds_bpermute(from_prev, static_cast<int>(raw[1]));
+    const uint32_t w2 = __builtin_amdgcn_ds_bpermute(from2, static_cast<int>(raw[2]));
+    const uint32_t w3 = __builtin_amdgcn_ds_bpermute(from3, static_cast<int>(raw[3]));
+    if (on && v < 3) {
+      const f16x8 x = __builtin_bit_cast(f16x8, raw);
+      // the partners of the piece's 8 elements, and how many of the leading ones are negated
+      const u32x4 pw = v == 0 ? u32x4{w1n, w2, w3, w0} : v == 1 ? u32x4{w1n, w0, w1p, w2} : u32x4{w3, w0, 0u, 0u};
+      const f16x8 far = __builtin_bit_cast(f16x8, pw);
+      const int negated = v == 0 ? 8 : v == 1 ? 2 : 0;
+      const f16x8 c8 = __builtin_bit_cast(f16x8, cw), s8 = __builtin_bit_cast(f16x8, sw);
+      f16x8 r = x;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (e >= 4 && v == 2) continue;   // elements 20..23 are not rotated
+        const half_t partner = e < negated ? static_cast<half_t>(static_cast<float>(far[e]) * -1.f) : far[e];
+        const half_t cj = v == 2 ? c8[(e + 4) & 7] : c8[e], sj = v == 2 ? s8[(e + 4) & 7] : s8[e];
+        const half_t t1 = static_cast<half_t>(static_cast<float>(cj) * static_cast<float>(x[e]));
+        const half_t t2 = static_cast<half_t>(static_cast<float>(sj) * static_cast<float>(partner));
+        r[e] = static_cast<half_t>(static_cast<float>(t1) + static_cast<float>(t2));
+      }
+      raw = __builtin_bit_cast(u32x4, r);
+    }
+    if (on) store_stream(raw, reinterpret_cast<u32x4*>(out + at));
   }
 }
 
@@ -407,8 +471,43 @@ __global__ void __launch_bounds__(kBlock) swap_axes_kernel(const u32x4* __restri
   for (I t = static_cast<I>(blockIdx.x) * kBlock + threadIdx.x; t < total; t += step) {
     const I r = t / per_row, p = t - r * per_row;   // output row r = ib * a + ia
     const I ib = r / a, ia = r - ib * a;
-    out[t] = A[(static_cast<int64_t>(ia) * b + ib) * per_row + p];
+    store_stream(A[(static_cast<int64_t>(ia) * b + ib) * per_row + p], out + t);
     if (total - t <= step) break;   // (t + step might wrap in 32 bits)
+  }
+}
+
+// The same for rows of up to 1 KiB (the model's are 160 bytes): a workgroup moves the tile of kSwapA consecutive ia by
+// kSwapB consecutive ib in the order of the output, so that what it writes (kSwapB runs of kSwapA rows) and what it
+// reads (kSwapA runs of kSwapB rows) are both runs of whole 128-byte lines; addresses are a base per workgroup plus
+// 32-bit offsets, and a thread loads up to four pieces before it stores them.  At a = 4096, b = 32, d = 80: 8.8 us
+// against 9.6 for the kernel above (10.7 before its stores became streaming ones); at a = 1024 4.0 either way.
+constexpr int kSwapA = 4, kSwapB = 8;
+__global__ void __launch_bounds__(kBlock) swap_axes_tile_kernel(const u32x4* __restrict__ A, u32x4* __restrict__ out, int64_t a,
+                                                                int64_t b, uint32_t per_row, uint32_t b_groups) {
+  const uint32_t ig = blockIdx.x / b_groups, bg = blockIdx.x - ig * b_groups;
+  const int64_t i0 = static_cast<int64_t>(ig) * kSwapA, b0 = static_cast<int64_t>(bg) * kSwapB;
+  const uint32_t ni = a - i0 < kSwapA ? static_cast<uint32_t>(a - i0) : kSwapA;
+  const uint32_t nb = b - b0 < kSwapB ? static_cast<uint32_t>(b - b0) : kSwapB;
+  const uint32_t run = ni * per_row, tile = nb * run;   // pieces of one output run, of the tile
+  const u32x4* src = A + (i0 * b + b0) * per_row;
+  u32x4* dst = out + (b0 * a + i0) * per_row;
+  const uint32_t in_row = static_cast<uint32_t>(b) * per_row, out_plane = static_cast<uint32_t>(a) * per_row;   // (the host checks that they fit)
+  for (uint32_t u0 = threadIdx.x; u0 < tile; u0 += 4 * kBlock) {
+    u32x4 v[4];
+    uint32_t to[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t u = u0 + k * kBlock;
+      if (u < tile) {
+        const uint32_t jb = u / run, rem = u - jb * run;
+        const uint32_t ii = rem / per_row, p = rem - ii * per_row;
+        v[k] = src[ii * in_row + jb * per_row + p];
+        to[k] = jb * out_plane + rem;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (u0 + k * kBlock < tile) store_stream(v[k], dst + to[k]);
   }
 }
 
@@ -424,8 +523,43 @@ __global__ void __launch_bounds__(kBlock) split3_kernel(const T* __restrict__ A,
     const I r = t / (3 * per_sec), c = t - r * (3 * per_sec);
     const I sec = c / per_sec, j = c - sec * per_sec;
     T* o = sec == 0 ? o0 : sec == 1 ? o1 : o2;
-    o[static_cast<int64_t>(r) * per_sec + j] = A[t];
+    store_stream(A[t], o + static_cast<int64_t>(r) * per_sec + j);
     if (total - t <= step) break;   // (t + step might wrap in 32 bits)
+  }
+}
+
+// The same for sections of up to 1 KiB (the model's are 160 bytes), 16-byte pieces: a workgroup takes kSplitRows rows
+// of A and walks them section by section, so that its stores are three runs of kSplitRows x d elements, whole
+// 128-byte lines; the lines of A are read by the three walks within the one workgroup.  Addresses are a base per
+// workgroup plus 32-bit offsets, and a thread loads up to four pieces before it stores them.  At 131072 rows, d = 80:
+// 21.8 us against 23.1 for the kernel above (24.4 before its stores became streaming ones), at 32768 rows 7.1 / 7.7.
+constexpr int kSplitRows = 8;
+__global__ void __launch_bounds__(kBlock) split3_tile_kernel(const u32x4* __restrict__ A, u32x4* __restrict__ o0, u32x4* __restrict__ o1,
+                                                             u32x4* __restrict__ o2, int64_t rows, uint32_t per_sec) {
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * kSplitRows;
+  const uint32_t nr = rows - r0 < kSplitRows ? static_cast<uint32_t>(rows - r0) : kSplitRows;
+  const uint32_t run = nr * per_sec, tile = 3 * run;
+  const u32x4* src = A + r0 * 3 * per_sec;
+  for (uint32_t u0 = threadIdx.x; u0 < tile; u0 += 4 * kBlock) {
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t u = u0 + k * kBlock;
+      if (u < tile) {
+        const uint32_t sec = u / run, rem = u - sec * run;
+        const uint32_t rr = rem / per_sec, j = rem - rr * per_sec;
+        v[k] = src[(rr * 3 + sec) * per_sec + j];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t u = u0 + k * kBlock;
+      if (u < tile) {
+        const uint32_t sec = u / run, rem = u - sec * run;
+        u32x4* o = sec == 0 ? o0 : sec == 1 ? o1 : o2;
+        store_stream(v[k], o + r0 * per_sec + rem);
+      }
+    }
   }
 }
 
@@ -549,10 +683,12 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
   const int64_t bytes = n * heads * d * 2;
   if (overlaps(out, bytes, A, bytes) || overlaps(out, bytes, cos_t, max_pos * rot * 2) || overlaps(out, bytes, sin_t, max_pos * rot * 2))
     return fail("rotary: output overlaps an input");
-  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, kBlock, 8, 1, {0, 0, 0}, 1, 0};
+  // cfg.unroll picks the kernel: 0 (built in) whole rows per wavefront where the shape has that form, 1 a piece per
+  // thread with its partners loaded, 2 the kernel for any rotated width
+  dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, kBlock, 8, 0, {0, 0, 0}, 1, 0};
   if (cfg.block != kBlock || cfg.vec != 8) return fail("rotary: the kernel uses %d threads and 8 elements per thread", kBlock);
   const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
-  if (rot == 20 && d >= 32 && cfg.unroll <= 1 && aligned(cos_t, 8) && aligned(sin_t, 8)) {  // the model's shape (cfg.unroll = 2 forces the general kernel)
+  if (rot == 20 && d >= 32 && cfg.unroll <= 1 && aligned(cos_t, 8) && aligned(sin_t, 8)) {  // the model's shape
     const int64_t pieces20 = n * heads * (d / 8);
     int64_t grid = ceil_div(pieces20, kBlock);
     grid = grid > cap ? cap : grid;
@@ -560,6 +696,14 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
     const half_t* a = static_cast<const half_t*>(A);
     const half_t* c = static_cast<const half_t*>(cos_t);
     const half_t* sn = static_cast<const half_t*>(sin_t);
+    if (d <= 512 && cfg.unroll == 0 && n * heads < (int64_t{1} << 31)) {   // rows of up to 64 pieces: whole rows per wavefront
+      const int64_t rows = n * heads, per_wave = 64 / (d / 8);
+      int64_t g = ceil_div(ceil_div(rows, per_wave), kBlock / 64);
+      g = g > cap ? cap : g;
+      hipLaunchKernelGGL(rotary20_rows_kernel, dim3(static_cast<unsigned>(g)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
+                         static_cast<uint32_t>(rows), static_cast<uint32_t>(heads), static_cast<uint32_t>(d / 8), m - n);
+      return check_launch("rotary");
+    }
     if (pieces20 < (int64_t{1} << 31) && heads < (int64_t{1} << 31) && d < (int64_t{1} << 31))
       hipLaunchKernelGGL(rotary20_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
                          static_cast<uint32_t>(pieces20), static_cast<uint32_t>(heads), static_cast<uint32_t>(d), m - n);
@@ -610,6 +754,13 @@ int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d
   grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total = a * b * (d / 8);
+  // rows of up to 1 KiB: by tiles of kSwapA x kSwapB rows (a launch holds fewer than 2^32 threads; the kernel's offsets 32 bits)
+  const int64_t groups = ceil_div(a, kSwapA) * ceil_div(b, kSwapB);
+  if (d <= 512 && a > 1 && b > 1 && groups < (int64_t{1} << 23) && a * (d / 8) < (int64_t{1} << 28) && b * (d / 8) < (int64_t{1} << 28)) {
+    hipLaunchKernelGGL(swap_axes_tile_kernel, dim3(static_cast<unsigned>(groups)), dim3(kBlock), 0, st, static_cast<const u32x4*>(A),
+                       static_cast<u32x4*>(out), a, b, static_cast<uint32_t>(d / 8), static_cast<uint32_t>(ceil_div(b, kSwapB)));
+    return check_launch("swap_axes");
+  }
   if (total < (int64_t{1} << 31))
     hipLaunchKernelGGL(swap_axes_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<const u32x4*>(A),
                        static_cast<u32x4*>(out), static_cast<uint32_t>(a), static_cast<uint32_t>(b), static_cast<uint32_t>(d / 8),
@@ -646,6 +797,11 @@ int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t r
   if (vec) {
     const u32x4* a = static_cast<const u32x4*>(A);
     u32x4 *p0 = static_cast<u32x4*>(out0), *p1 = static_cast<u32x4*>(out1), *p2 = static_cast<u32x4*>(out2);
+    if (d <= 512 && ceil_div(rows, kSplitRows) < (int64_t{1} << 23)) {   // sections of up to 1 KiB: by tiles of rows (a launch holds fewer than 2^32 threads)
+      hipLaunchKernelGGL(split3_tile_kernel, dim3(static_cast<unsigned>(ceil_div(rows, kSplitRows))), blk, 0, st, a, p0, p1, p2, rows,
+                         static_cast<uint32_t>(per_sec));
+      return check_launch("split3");
+    }
     if (narrow) hipLaunchKernelGGL((split3_kernel<u32x4, uint32_t>), g, blk, 0, st, a, p0, p1, p2, static_cast<uint32_t>(per_sec), static_cast<uint32_t>(total));
     else hipLaunchKernelGGL((split3_kernel<u32x4, int64_t>), g, blk, 0, st, a, p0, p1, p2, per_sec, total);
   } else {

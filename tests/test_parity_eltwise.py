@@ -276,7 +276,10 @@ def test_take_clips_ids_scalar_path_descriptor_and_errors(oracle):
 
 
 @pytest.mark.parametrize("n,m,heads,d,rot", [(1, 1, 32, 80, 20), (1, 2048, 32, 80, 20), (300, 300, 32, 80, 20), (257, 4096, 32, 80, 20),
-                                             (7, 9, 3, 64, 64), (5, 5, 2, 16, 0), (33, 40, 4, 128, 32)])
+                                             (7, 9, 3, 64, 64), (5, 5, 2, 16, 0), (33, 40, 4, 128, 32),
+                                             # rot = 20 with rows of 3, 4, 7, 64 and 65 pieces; one row; rows that end a chunk early
+                                             (19, 4096, 5, 24, 20), (130, 130, 3, 32, 20), (41, 50, 7, 56, 20), (9, 9, 2, 512, 20),
+                                             (3, 3, 2, 520, 20), (1, 7, 1, 80, 20), (4096, 4096, 32, 80, 20)])
 def test_rotary_is_bit_exact(oracle, n, m, heads, d, rot):
     rng = np.random.default_rng(n + m + d)
     a = rng.standard_normal((1, n, heads, d)).astype(np.float16)
@@ -286,9 +289,10 @@ def test_rotary_is_bit_exact(oracle, n, m, heads, d, rot):
     ops.rotary(dev(a), dev(cos), dev(sin), out.t, m)
     want = oracle.c.rotary(a, cos, sin, m, threads=8)
     assert_bits_equal(out.check(), want)
-    out = Guarded(a.shape, torch.float16)      # the kernel for any rotated width, also where the model's has its own
-    ops.rotary(dev(a), dev(cos), dev(sin), out.t, m, cfg(variant=_lib.ELT_VECTOR, block=256, vec=8, unroll=2))
-    assert_bits_equal(out.check(), want)
+    for unroll in (1, 2):                      # a piece per thread; the kernel for any rotated width, also where the model's has its own
+        out = Guarded(a.shape, torch.float16)
+        ops.rotary(dev(a), dev(cos), dev(sin), out.t, m, cfg(variant=_lib.ELT_VECTOR, block=256, vec=8, unroll=unroll))
+        assert_bits_equal(out.check(), want)
 
 
 def test_rotary_errors():
@@ -326,7 +330,8 @@ def test_attn_mask_beyond_32_bit_indices():
     del out
 
 
-@pytest.mark.parametrize("a,b,d", [(1, 32, 80), (300, 32, 80), (32, 300, 80), (4096, 32, 80), (5, 3, 8)])
+@pytest.mark.parametrize("a,b,d", [(1, 32, 80), (300, 32, 80), (32, 300, 80), (4096, 32, 80), (5, 3, 8), (9, 17, 8), (13, 8, 512),
+                                   (4, 5, 520), (8, 8, 80), (2, 2, 24)])
 def test_swap_axes_is_exact(oracle, a, b, d):
     rng = np.random.default_rng(a + b)
     x = rng.integers(0, 2 ** 16, (1, a, b, d), dtype=np.uint16).view(np.float16)
@@ -346,7 +351,8 @@ def test_mask_and_swap_errors():
         _lib.check(L.dtas_swap_axes_f16(x.data_ptr(), x.data_ptr(), 2, 3, 8, None), "swap")
 
 
-@pytest.mark.parametrize("lead,d", [((1, 1, 32), 80), ((1, 300, 32), 80), ((1, 4096, 32), 80), ((7,), 3), ((33, 5), 12)])
+@pytest.mark.parametrize("lead,d", [((1, 1, 32), 80), ((1, 300, 32), 80), ((1, 4096, 32), 80), ((7,), 3), ((33, 5), 12),
+                                    ((37,), 512), ((3, 11), 520), ((65,), 8), ((32,), 16)])
 def test_split3_is_exact(oracle, lead, d):
     rng = np.random.default_rng(d + len(lead))
     x = rng.integers(0, 2 ** 16, lead + (3 * d,), dtype=np.uint16).view(np.float16)

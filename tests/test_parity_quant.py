@@ -360,14 +360,19 @@ def test_gemm_q8_exact_cases_fallback_and_errors(oracle):
 
 # ---- the embedding gather and the fp32-scale vocabulary projection (before_dl.py:346-369, :640-657) ----------
 
-@pytest.mark.parametrize("V,K,n", [(50280, 2560, 1), (50280, 2560, 300), (50280, 2560, 4096), (7, 32, 19), (100, 96, 1)])
+@pytest.mark.parametrize("V,K,n", [(50280, 2560, 1), (50280, 2560, 300), (50280, 2560, 4096), (7, 32, 19), (100, 96, 1),
+                                   (100, 96, 45), (20, 4128, 5), (9, 2048, 3), (11, 2016, 70)])
 def test_take_is_bit_exact(oracle, V, K, n):
     wq, scale = _weights(V, K, V + n)
     ids = np.random.default_rng(n).integers(0, V, n).astype(np.int32)
     ids[0], ids[-1] = V - 1, 0
     out = Guarded((n, K), torch.float16)
     ops.take_q8(_words(wq), dev(scale), dev(ids), out.t)
-    assert np.array_equal(out.check().view(np.uint16), oracle.c.take_q8(wq, scale, ids, threads=8).view(np.uint16))
+    want = oracle.c.take_q8(wq, scale, ids, threads=8).view(np.uint16)
+    assert np.array_equal(out.check().view(np.uint16), want)
+    out = Guarded((n, K), torch.float16)          # a grid cap: the grid-stride kernel
+    ops.take_q8(_words(wq), dev(scale), dev(ids), out.t, cfg(variant=_lib.ELT_VECTOR, block=256, vec=8, grid_cap=3))
+    assert np.array_equal(out.check().view(np.uint16), want)
 
 
 def test_take_clips_ids_scalar_path_and_errors(oracle):
