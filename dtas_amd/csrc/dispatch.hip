@@ -130,7 +130,7 @@ dtas_config gemv_policy(int64_t N, int64_t K) {
 //  * few tiles: K split over up to 4 workgroups per tile, each partial tile costing the last
 //    workgroup ~4 us (128x128), ~2.5 us (128x64), ~1 us (64x64; 2.5 us with more than one per CU)
 //    to add up; 256x128 splits while its workgroups fit one round and each keeps 32 k tiles or
-//    more (~6 us per partial tile);
+//    more (~4.5 us per partial tile: 512 x 5120 x 13824 in 3 parts 86.8 us against 98.2 for 256x256, 640 x 4096 x 8192 in 2 parts 63.8 against 67.3);
 //  * a floor: W (2NK bytes) streams at 3.1 .. 4.3 TB/s depending on the tile (few rows against a very wide W);
 //  * M <= 32: the W-streaming SKINNY kernel, whose time grows with N*K (about 3.5 TB/s of W).
 struct GemmChoice {
@@ -206,7 +206,7 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     consider(floored((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.5) * split : 0.0), 4.3), 64, 64, 256, 4, split);
     const double t256128 = tiles_of(256, 128) * split;
     if (split > 1 && steps >= 32 && t256128 <= kNumCU)
-      consider(floored(gemm_rounds(t256128, kNumCU) * 1.0 * steps + 6.0 * split, 3.5), 256, 128, 512, 2, split);
+      consider(floored(gemm_rounds(t256128, kNumCU) * 1.0 * steps + 4.5 * split, 3.5), 256, 128, 512, 2, split);
     const double t12864 = tiles_of(128, 64) * split;
     if (t12864 <= kNumCU)
       consider(floored(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 3.4), 128, 64, 256, 4, split);

@@ -42,7 +42,8 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         to 4 workgroups per tile at ~4 us (128x128) / ~1 us (64x64; 2.5 us with more than one per CU) per partial
         tile; 128x64 (4 stages, at most one workgroup per CU) 0.47 us per k tile whatever the fill and ~2.5 us
         per partial tile; 256x128 splits too while its workgroups fit one round and each keeps 32 k tiles or
-        more (~6 us per partial tile).  No candidate is faster than W (2NK bytes) streams through it: 3.1 .. 4.3 TB/s
+        more (~4.5 us per partial tile: 512 x 5120 x 13824 in 3 parts 86.8 us against 98.2 for 256x256, 640 x 4096 x 8192 in 2 parts
+        63.8 against 67.3).  No candidate is faster than W (2NK bytes) streams through it: 3.1 .. 4.3 TB/s
         by tile, measured with 64 rows against a 50280 x 2560 W."""
         cdiv = lambda a, b: -(-a // b)
         cus = self.arch.num_sm
@@ -92,7 +93,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                           (64, 64, 4, split)))
             t256128 = tiles(256, 128) * split
             if split > 1 and steps >= 32 and t256128 <= cus:
-                cands.append((floored(rounds(t256128, cus) * 1.0 * steps + 6.0 * split, 3.5), (256, 128, 2, split)))
+                cands.append((floored(rounds(t256128, cus) * 1.0 * steps + 4.5 * split, 3.5), (256, 128, 2, split)))
             t12864 = tiles(128, 64) * split
             if t12864 <= cus:
                 cands.append((floored(0.47 * steps + (2.5 * split if split > 1 else 0.0), 3.4), (128, 64, 4, split)))
