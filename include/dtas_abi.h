@@ -28,7 +28,9 @@
  *    ordered by it, launches on different streams use different workspaces and may overlap; the
  *    library holds its lock from looking a workspace up to enqueueing the launch, so host threads may
  *    share a stream.  At most 16 streams per device hold one (the one used longest ago is released
- *    first, which waits for the device).  A cfg with split_k = 1 uses none; dtas_gemm_f16_static
+ *    first, which waits for the device).  A recorded HIP graph holds the workspace's address: the
+ *    first split launch on a stream, and any launch that makes its workspace grow, belong before the
+ *    recording.  A cfg with split_k = 1 uses none; dtas_gemm_f16_static
  *    never allocates.  dtas_gemm_q8_f16_fused keeps a second buffer of that kind
  *    (an fp16 copy of the weights it was given) under the same rules;
  *  - `cfg` selects the kernel variant and launch shape explicitly (what one row of the

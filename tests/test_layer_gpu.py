@@ -157,3 +157,68 @@ def test_sampling_head(oracle):
     got = probs.cpu().numpy()
     assert np.abs(got - want).max() < 1e-2 and np.abs(got / want - 1).max() < 2e-2
     assert int(got.argmax()) == int(want.argmax()) and abs(float(got.astype(np.float64).sum()) - 1) < 1e-4
+
+
+def _decode_step(Ws, caches, bufs, x, cos, sin, m):
+    """The decode graph's layers (n = 1) as plain launches on the current stream: no checks, no synchronisation, every
+    buffer allocated beforehand -- what a caller records into a HIP graph."""
+    n, cur = 1, x
+    for W, (kh, vh), b in zip(Ws, caches, bufs):
+        ops.attn_mask(b["mask"])
+        ops.cast(cur, b["x32"])
+        ops.layer_norm(b["x32"], W["ln1_g"], W["ln1_b"], b["h1"])
+        ops.gemv(b["h1"], W["qkv_w"], W["qkv_b"], b["qkv"])
+        ops.split3(b["qkv"].view(n, HEADS, 3 * D), b["q"], b["k"], b["v"])
+        ops.rotary(b["q"], cos, sin, b["qr"], m)
+        ops.rotary(b["k"], cos, sin, b["kr"], m)
+        kh[:, m - 1, :].copy_(b["kr"][0])                         # the cache append: the runtime's part
+        vh[:, m - 1, :].copy_(b["v"][0])
+        ops.swap_axes(b["qr"], b["qh"])
+        ops.attn_scores(b["qh"], kh, b["mask"], b["scores"])
+        ops.softmax(b["scores"], b["probs"])
+        ops.attn_pv(b["probs"], vh, b["ctx"])
+        ops.swap_axes(b["ctx"], b["merged"])
+        ops.layer_norm(b["x32"], W["ln2_g"], W["ln2_b"], b["h2"])
+        ops.gemv(b["h2"], W["up_w"], W["up_b"], b["up"], epilogue=_lib.EPI_BIAS_GELU)
+        ops.gemv(b["up"], W["down_w"], W["down_b"], b["down"])
+        ops.gemv(b["merged"].view(n, H), W["o_w"], W["o_b"], b["y"], epilogue=_lib.EPI_BIAS_ADD2, res1=b["down"], res2=cur)
+        cur = b["y"]
+    return cur
+
+
+@pytest.mark.parametrize("past", [63, 4000])      # (4000 keys: P.V shares the keys between workgroups through the workspace)
+def test_decode_layers_recorded_into_a_graph_replay_the_same_bits(past):
+    """Two layers of the decode step recorded into a HIP graph (the launch-bound loop of serving: 20 launches of a few
+    microseconds per layer) and replayed three times, with eager launches on the same stream's workspace between the
+    replays; every replay gives the bits of the eager run.  The stream is warmed up first: a workspace is allocated at
+    a stream's first split launch, and nothing may allocate while a graph is recorded."""
+    W = _weights()
+    layers, m = 2, past + 1
+    Wd = {k: dev(v) for k, v in W.items()}
+    rng = np.random.default_rng(past)
+    x = dev(rng.standard_normal((1, H)).astype(np.float16))
+    cache = lambda: dev((rng.standard_normal((HEADS, m, D)) * 0.5).astype(np.float16))
+    caches = [(cache(), cache()) for _ in range(layers)]
+    E = lambda *s, dt=torch.float16: torch.empty(*s, dtype=dt, device="cuda")
+    bufs = [dict(mask=E(1, 1, 1, m), x32=E(1, H, dt=torch.float32), h1=E(1, H), qkv=E(1, 3 * H), q=E(1, HEADS, D), k=E(1, HEADS, D),
+                 v=E(1, HEADS, D), qr=E(1, HEADS, D), kr=E(1, HEADS, D), qh=E(HEADS, 1, D), scores=E(HEADS, 1, m, dt=torch.float32),
+                 probs=E(HEADS, 1, m), ctx=E(HEADS, 1, D), merged=E(1, HEADS, D), h2=E(1, H), up=E(1, FF), down=E(1, H), y=E(1, H))
+            for _ in range(layers)]
+    step = lambda: _decode_step([Wd] * layers, caches, bufs, x, Wd["cos"], Wd["sin"], m)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        eager = step().clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        y = step()
+    a, w, c = torch.randn(40, 2048, device="cuda").half(), torch.randn(1000, 2048, device="cuda").half(), E(40, 1000)
+    for _ in range(3):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(y.cpu().numpy(), eager.cpu().numpy())
+        with torch.cuda.stream(side):       # eager work between the replays: a split GEMM and another sequence length's P.V
+            ops.gemm(a, w, None, c)
+            ops.attn_pv(torch.rand(HEADS, 1, 3500, device="cuda").half(), torch.randn(HEADS, 3500, D, device="cuda").half(), E(HEADS, 1, D))
+        torch.cuda.synchronize()
