@@ -215,6 +215,11 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   // 12.8 us at 4096 x 4096, 7.2 against 10.2 at 2560 x 2560; with more workgroups than CUs a workgroup's loads,
   // MFMAs and the hand-over of its partial sums are no longer hidden behind another's, and the tiles win again
   if (M_hi <= 16 && ceil_div(n, 64) * ceil_div(k, 1024) <= kNumCU) return make(DTAS_GEMM_STREAM, 256, 8, 1, 16, 64, 1024);
+  // 17 .. 32 rows: the same with 32 rows of A and 512 of K per workgroup, where that gives a quarter of a round or more
+  // and at most one (8.4 against 9.8 us at 2560 x 2560, 9.5 / 10.7 at 2048 x 4096, 11.4 / 13.9 at 1024 x 8192, 8.9 / 10.2 at
+  // 3072 x 2560; behind at 1024 x 1024, whose 32 workgroups leave the chip idle)
+  if (M_hi > 16 && M_hi <= 32 && ceil_div(n, 64) * ceil_div(k, 512) <= kNumCU && ceil_div(n, 64) * ceil_div(k, 512) >= kNumCU / 4)
+    return make(DTAS_GEMM_STREAM, 256, 8, 1, 32, 64, 512);
   // M <= 16 against more rows of W: the looping form (the whole of K per workgroup, nothing handed over) while its
   // workgroups run in one round -- 16 columns each (one wavefront, two workgroups per CU) for 4096 < N <= 8192, 64
   // columns (one per CU) for 8192 <= N <= 16384 -- and K is short enough for a round to be worth its start:

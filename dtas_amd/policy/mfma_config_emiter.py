@@ -125,10 +125,14 @@ class MFMAConfigEmiter(BaseConfigEmiter):
         return split, tiles - rem
 
     def prefers_stream(self, m_hi: int, N: int, K: int) -> bool:
-        """M <= 16 and at most one workgroup per CU of the W-streaming kernel (64 columns x 1024 of K each):
+        """M <= 32 and at most one workgroup per CU of the W-streaming kernel (M <= 16: 64 columns x 1024 of K each):
         measured 10.9 against 12.8 us at 4096 x 4096, 7.2 against 10.2 at 2560 x 2560; beyond one round of
         workgroups the tiles win again (libdtas: gemm_policy)."""
-        return m_hi <= 16 and -(-N // 64) * -(-K // 1024) <= self.arch.num_sm
+        if m_hi <= 16:
+            return -(-N // 64) * -(-K // 1024) <= self.arch.num_sm
+        # 17 .. 32 rows: 32 rows of A and 512 of K per workgroup, between a quarter of a round and one round of them
+        # (8.4 against 9.8 us at 2560 x 2560, 11.4 / 13.9 at 1024 x 8192)
+        return m_hi <= 32 and self.arch.num_sm // 4 <= -(-N // 64) * -(-K // 512) <= self.arch.num_sm
 
     def prefers_stream_loop(self, m_hi: int, N: int, K: int) -> int:
         """Columns per workgroup (16 or 64) of the looping W-streaming kernel where it leads, else 0: M <= 16, K <= 4096

@@ -256,8 +256,9 @@ def test_builtin_tables_name_a_launchable_kernel_for_every_bucket_and_shape():
                     assert M <= 16 and K <= 4096 and (list(c.tile[:2]), c.block) in (([16, 16], 64), ([16, 64], 256))
                     assert (256 < info.launch_args[0] <= 512) if c.tile[1] == 16 else (128 <= info.launch_args[0] <= 256)
                 elif c.variant == _lib.GEMM_STREAM:
-                    # at most one workgroup per CU, 64 columns x 1024 of K each
-                    assert M <= 16 and list(c.tile) == [16, 64, 1024] and c.block == 256 and info.launch_args[0] <= 256
+                    # at most one workgroup per CU: 64 columns x 1024 of K each up to 16 rows, x 512 of K for 17 .. 32
+                    assert c.block == 256 and info.launch_args[0] <= 256
+                    assert (M <= 16 and list(c.tile) == [16, 64, 1024]) or (16 < M <= 32 and list(c.tile) == [32, 64, 512] and info.launch_args[0] >= 64)
                 else:
                     assert c.variant == _lib.GEMM_SKINNY and M <= 32 and c.tile[0] >= min(M, 32)
             info = _lib.select_bucket(_lib.OP_GEMV_F16, 1, N, K)
