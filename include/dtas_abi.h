@@ -378,7 +378,7 @@ int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, 
 /* dtas_gemm_q8_f16_fused: C[M,N] = epilogue(A[M,K] . W^T) with W dequantised on its way into the LDS, never
  * written: the dynamic-n forms fused_fused_decode2_fused_NT_matmul6_add4 (:371-399), ..decode4.._matmul9_add6_gelu1
  * (:504-581), ..decode5.._matmul4_add1; epilogues as dtas_gemm_f16_fused.  cfg, when given: a DTAS_GEMM_MFMA row
- * with tile {256,128,64} or {128,128,64} and unroll 3, or {64,64,64} and unroll 2; or a DTAS_GEMM_STREAM row
+ * with tile {256,128,64}, {128,128,64}, {128,64,64} or {64,128,64} and unroll 3, or {64,64,64} and unroll 2 or 3; or a DTAS_GEMM_STREAM row
  * (block 256, tile {16,64,512}, {16,64,1024}, {32,64,512} or {64,64,512}; M <= tile[0]; K % 256 == 0; 16-byte
  * aligned A, Wq and scale): the W-streaming kernel on the bytes of W, widened between the LDS and the MFMA; its K
  * slices meet in the split-K workspace.  A DTAS_GEMM_MFMA row may carry split_k in [1, 16]: that many workgroups share
