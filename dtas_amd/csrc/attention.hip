@@ -790,7 +790,33 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       // tile within 5 %: there the launch is bound by how P streams in, 128 bytes of a row per request).  Head dimensions up to 64 keep the
       // 64-column tiles: two workgroups of two stages per CU
       const int64_t t128 = heads * ceil_div(n, 128);
-      if (t128 <= kNumCU / 2) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, bn == 128 ? 3 : 2, {64, bn, kBK}, 1, 0};
+      bool fitted = false;
+      if (bn == 128 && t128 <= kNumCU) {
+        // Up to one 128-row tile per CU (n <= 1024 with 32 heads): 64x128 and 128x128 with three stages or 64x64 with two, the
+        // keys in 1 / 2 / 4 / 8 parts, by us = start + (k tiles per part) x (cost of one at that many workgroups) + hand-over,
+        // fitted to a sweep of n = 16 .. 768 against 512 .. 8192 keys (32 heads of 80, P and V from memory).  Measured, new /
+        // old choice: 256 rows against 1024 / 4096 / 8192 keys 12.1 / 26.7 / 42.9 us (16.7 / 42.4 / 61.5), 384 against 1024 /
+        // 2048 / 4096 13.2 / 21.4 / 31.2 (24.6 / 33.3 / 43.7), 128 against 4096 18.9 (24.6), 128 x 128 4.7 (6.3)
+        const double hand64[4] = {0.0, 1.6, 4.0, 7.0}, hand[4] = {0.0, 2.5, 4.3, 6.5}, hand128[4] = {0.0, 4.0, 8.0, 16.0};
+        const int64_t t64 = heads * ceil_div(n, 64);
+        double best = 1e30;
+        for (int i = 0; i < 4; ++i) {
+          const int parts = 1 << i;
+          if (i > 0 && ktiles < 2 * parts) break;
+          const double steps = static_cast<double>(ceil_div(ktiles, parts));
+          const double w64 = static_cast<double>(t64 * parts), w128 = static_cast<double>(t128 * parts);
+          // 64x64, two stages: short sweeps on a chip that is not full
+          const double us_a = w64 <= 128 && steps <= 8 ? 4.2 + (0.3 + 0.3 * w64 / 192.0) * steps + hand64[i] : 1e30;
+          // 64x128, three stages (two workgroups per CU)
+          const double us_b = w64 <= 2 * kNumCU ? 5.2 + 0.55 * (w64 <= kNumCU ? 1.0 : 1.15 * w64 / kNumCU) * steps + hand[i] : 1e30;
+          // 128x128, three stages (one per CU)
+          const double us_c = w128 <= kNumCU ? 7.1 + (0.45 + 0.3 * (w128 / kNumCU) * (w128 / kNumCU)) * steps + hand128[i] : 1e30;
+          if (us_a < best) best = us_a, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, 64, kBK}, parts, 0};
+          if (us_b < best) best = us_b, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {64, 128, kBK}, parts, 0};
+          if (us_c < best) best = us_c, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, parts, 0};
+        }
+        fitted = true;
+      } else if (t128 <= kNumCU / 2) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, bn == 128 ? 3 : 2, {64, bn, kBK}, 1, 0};
       else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
       else if (bn == 128) {
         cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
@@ -808,7 +834,7 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       const int64_t wgs = heads * ceil_div(n, cfg.tile[0]);
       const int64_t wg_limit = cfg.tile[0] <= 64 ? 4 * kNumCU : kNumCU;
       double us;
-      if (wgs < kNumCU && cfg.tile[0] <= 128) cfg.split_k = key_split(wgs, wg_limit, ktiles, &us);
+      if (!fitted && wgs < kNumCU && cfg.tile[0] <= 128) cfg.split_k = key_split(wgs, wg_limit, ktiles, &us);
     }
   }
   if (cfg.vec == 8 && cfg.variant == DTAS_GEMM_SKINNY && !v_vec) cfg.vec = 1;
