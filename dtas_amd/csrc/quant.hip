@@ -334,9 +334,10 @@ extern "C" int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale
   if (!y || (K > 0 && (!x || !Wq || !scale))) return fail("gemv_q8: NULL buffer");
   if (overlaps(y, N * 2, Wq, N * K) || overlaps(y, N * 2, x, K * 2) || overlaps(y, N * 2, scale, N * (K / 32) * 2))
     return fail("gemv_q8: output overlaps an input");
-  // measured over the model's and the benchmark's shapes: 256 threads; 2 rows per workgroup, 4 once that
-  // still leaves every CU a dozen workgroups
-  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 8 : 2, 0, 0}, 1, 0};   // (50280 x 2560: 45 / 30 / 25 / 24 us with 1 / 2 / 4 / 8 rows per workgroup)
+  // measured over N = 2560 .. 50280 against K = 2560 .. 11008 (12 launch shapes each): 4 rows per workgroup from 4096 rows
+  // on, 2 below; 8 wavefronts for K >= 8192 with those 4 rows, 4 wavefronts otherwise (7680 x 10240: 15.4 us against 17.7 for 2 rows on 4 wavefronts,
+  // 11008 x 5120: 11.8 / 13.9, 4096 x 5120: 6.4 / 7.4; level at K = 4096)
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, K >= 8192 && N >= 4096 ? 512 : 256, 8, 2, {N >= 4096 ? 4 : 2, 0, 0}, 1, 0};
   if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
   int64_t la[7];
   if (describe_gemv(N, K, cfg, la) != 0) return -1;
@@ -400,7 +401,7 @@ extern "C" int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale
   if (!y || (K > 0 && (!x || !Wq || !scale))) return fail("gemv_q8_f32: NULL buffer");
   if (overlaps(y, N * 4, Wq, N * K) || overlaps(y, N * 4, x, K * 4) || overlaps(y, N * 4, scale, N * (K / 32) * 4))
     return fail("gemv_q8_f32: output overlaps an input");
-  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 4 : 2, 0, 0}, 1, 0};
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 8 : 2, 0, 0}, 1, 0};   // (50280 x 2560: 45 / 30 / 25 / 24 us with 1 / 2 / 4 / 8 rows per workgroup)
   if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
   int64_t la[7];
   if (describe_gemv(N, K, cfg, la) != 0) return -1;

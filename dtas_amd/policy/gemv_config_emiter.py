@@ -23,8 +23,9 @@ class GEMVConfigEmiter(BaseConfigEmiter):
                 c.TILE_S, c.TR = rows, threads
                 out.append(c)
         # measured on MI355X: one row per 4-wavefront workgroup is best or within noise for K = 4096;
-        # rows of K >= 8192 do better with 8 wavefronts on two rows
-        best = (2, 512) if K >= 8192 else (1, 256)
+        # rows of K >= 8192 do better with 8 wavefronts on two rows, and rows that leave the last pass of 4 wavefronts
+        # partly empty (K = 2560) with two rows on those 4
+        best = (2, 512) if K >= 8192 else (2, 256) if K % 2048 != 0 else (1, 256)
 
         def score(c: GEMVConfig):
             return ((c.TILE_S, c.TR) != best, c.TILE_S, c.TR != 256)
