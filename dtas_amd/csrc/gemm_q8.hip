@@ -86,8 +86,9 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
   } else {
     // three tiles of three stages -- 64x64 (three workgroups per CU), 128x64 (two), 128x128 (one) -- with K in 1 .. 8 parts of
     // 4 k tiles or more: us = start + (k tiles per part) x (cost of one, growing with the workgroups on the chip) + a
-    // hand-over per part, fitted to a sweep of the model's shapes at M = 96 .. 512 (7680 x 2560, M = 256: 128x64 in 2 parts
-    // 22.3 us, 26.0 before; 2560 x 2560, M = 256: 64x64 in 3 parts 14.1, 22.5 before; 10240 x 2560, M = 192: 64x64 25.2, 34.5)
+    // hand-over per part, fitted to a sweep of the model's shapes at M = 96 .. 512 with the weights streamed from memory
+    // (2560 x 2560, M = 256: 64x64 in 3 parts 15.4 us, 22 before; 10240 x 2560, M = 192: 64x64 28.3, 34 before; within 10 % of
+    // the best of 36 configurations on the sweep's 24 shapes, 3 % on average)
     const int64_t t12864 = ceil_div(M, 128) * ceil_div(N, 64);
     // (rows 5, 6, 10, ... KiB of fp16 apart: a loaded chip takes a k tile of the 128x64 tile 20-25 % longer -- 2560 x 10240,
     // M = 512 in 3 parts: 58.6 us where the fit without it says 47.6, 128x128 53.6)
@@ -98,10 +99,10 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
       if (parts > 1 && ktiles / parts < 4) break;
       const double steps = static_cast<double>(ceil_div(ktiles, parts));
       const double w64 = static_cast<double>(t64 * parts), w12864 = static_cast<double>(t12864 * parts), w128 = static_cast<double>(t128 * parts);
-      const double us64 = w64 <= 512 ? 4.4 + (0.30 + 0.22 * w64 / 480.0) * steps + 1.2 * (parts - 1) : 1e30;
-      const double b12864 = 0.18 + 0.52 * (odd_pitch ? 1.35 : 1.0) * w12864 / 480.0;
-      const double us12864 = w12864 <= 512 ? 6.8 + (b12864 < 0.44 ? 0.44 : b12864) * steps + 1.5 * (parts - 1) : 1e30;
-      const double us128 = w128 <= kNumCU ? 10.8 + (0.40 + 0.225 * w128 / 240.0) * steps + 2.8 * (parts - 1) : 1e30;
+      const double us64 = w64 <= 512 ? 4.4 + (0.30 + 0.26 * w64 / 480.0) * steps + 1.33 * (parts - 1) : 1e30;
+      const double b12864 = 0.18 + 0.69 * (odd_pitch ? 1.35 : 1.0) * w12864 / 480.0;
+      const double us12864 = w12864 <= 512 ? 8.4 + (b12864 < 0.44 ? 0.44 : b12864) * steps + 1.5 * (parts - 1) : 1e30;
+      const double us128 = w128 <= kNumCU ? 9.2 + (0.373 + 0.45 * w128 / 480.0) * steps + 1.87 * (parts - 1) : 1e30;
       if (us64 < best) best = us64, cfg.tile[0] = 64, cfg.tile[1] = 64, cfg.split_k = parts;
       if (us12864 < best) best = us12864, cfg.tile[0] = 128, cfg.tile[1] = 64, cfg.split_k = parts;
       if (us128 < best) best = us128, cfg.tile[0] = 128, cfg.tile[1] = 128, cfg.split_k = parts;
