@@ -385,7 +385,7 @@ int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, 
  * a tile and meet in the split-K workspace as in dtas_gemm_f16.  One row with a bias or GELU epilogue goes to
  * dtas_gemv_q8_f16.  With cfg == NULL: M <= 32 (M <= 64 with N, K <= 4096) takes the W-streaming kernel where it
  * applies; up to 512 rows, while 128x128 tiles fit the chip in one round, the tile kernel dequantises in its W path
- * (64x64 tiles up to 128 rows, 128x128 beyond; K split over workgroups to fill the chip); beyond that the two-pass route:
+ * (64x64, 128x64 or 128x128 tiles of three stages with K in 1 .. 8 parts, by a fitted cost model); beyond that the two-pass route:
  * dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on demand, at most
  * 1 GiB; same sharing rule as the split-K workspace), then dtas_gemm_f16_fused. */
 int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void* scale, const void* bias,
