@@ -17,6 +17,11 @@ namespace dtas {
 namespace {
 
 constexpr int kBlock = 256;
+// Workgroups per launch of the index-only kernels: a thread per 16-byte piece for as long as a launch may hold them
+// (fewer than 2^32 threads) and a grid-stride loop beyond.  A grid capped at a few dozen workgroups per CU that loops
+// writes slower: the [16384, 16384] mask, 537 MB, takes 107 us with 64 workgroups per CU looping 8 times and 77 us (7.0 TB/s)
+// with a workgroup per 4 KiB; 134 MB 23.7 / 22.0.
+constexpr int64_t kMaxGrid = int64_t{1} << 23;
 
 // ---- raw fixed-size accesses ------------------------------------------------------
 template <int BYTES>
@@ -441,16 +446,23 @@ __global__ void __launch_bounds__(kBlock) attn_mask_kernel(half_t* __restrict__ 
   for (I t = (static_cast<I>(blockIdx.x) * kBlock + threadIdx.x) * 8; t < total; t += step) {
     I i = t / m, jj = t - i * m;
     f16x8 v;
+    if (m - jj >= 8) {   // the 8 elements lie in one row: element e is above the diagonal when e > i + shift - jj
+      const int64_t last_kept = static_cast<int64_t>(i) + static_cast<int64_t>(shift) - static_cast<int64_t>(jj);
+      const int keep = last_kept < 0 ? 0 : last_kept >= 7 ? 8 : static_cast<int>(last_kept) + 1;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      v[e] = static_cast<half_t>(jj > i + shift ? -65504.f : 65504.f);
-      if (++jj == m) {
-        jj = 0;
-        ++i;
+      for (int e = 0; e < 8; ++e) v[e] = static_cast<half_t>(e < keep ? 65504.f : -65504.f);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[e] = static_cast<half_t>(jj > i + shift ? -65504.f : 65504.f);
+        if (++jj == m) {
+          jj = 0;
+          ++i;
+        }
       }
     }
     if (total - t >= 8) {
-      __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(out + t));
+      store_stream(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4*>(out + t));
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
@@ -655,7 +667,7 @@ int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t 
   if (cfg.vec == 8 && !(H % 8 == 0 && aligned(A, 16) && aligned(out, 16))) cfg.vec = 1;
   const int64_t items = cfg.vec == 8 ? n * (H / 8) : n * H;
   int64_t grid = ceil_div(items, kBlock);
-  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : kMaxGrid;
   grid = grid > cap ? cap : grid;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (cfg.vec == 8)
@@ -687,7 +699,7 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
   // thread with its partners loaded, 2 the kernel for any rotated width
   dtas_config cfg = user ? *user : dtas_config{DTAS_ELT_VECTOR, kBlock, 8, 0, {0, 0, 0}, 1, 0};
   if (cfg.block != kBlock || cfg.vec != 8) return fail("rotary: the kernel uses %d threads and 8 elements per thread", kBlock);
-  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : kMaxGrid;
   if (rot == 20 && d >= 32 && cfg.unroll <= 1 && aligned(cos_t, 8) && aligned(sin_t, 8)) {  // the model's shape
     const int64_t pieces20 = n * heads * (d / 8);
     int64_t grid = ceil_div(pieces20, kBlock);
@@ -730,7 +742,7 @@ int dtas_attn_mask_f16(void* out, int64_t n, int64_t m, void* stream) {
   if (!out) return fail("attn_mask: NULL buffer");
   if (!aligned(out, 16)) return fail("attn_mask: the output must be 16-byte aligned");
   int64_t grid = ceil_div(ceil_div(n * m, 8), kBlock);
-  grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+  grid = grid > kMaxGrid ? kMaxGrid : grid;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n * m + 8 < (int64_t{1} << 31))   // + 8: the last thread's t stays below 2^31 as well
     hipLaunchKernelGGL(attn_mask_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, static_cast<half_t*>(out),
@@ -751,7 +763,7 @@ int dtas_swap_axes_f16(const void* A, void* out, int64_t a, int64_t b, int64_t d
   if (!aligned(A, 16) || !aligned(out, 16)) return fail("swap_axes: buffers must be 16-byte aligned");
   if (overlaps(out, a * b * d * 2, A, a * b * d * 2)) return fail("swap_axes: output overlaps the input");
   int64_t grid = ceil_div(a * b * (d / 8), kBlock);
-  grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+  grid = grid > kMaxGrid ? kMaxGrid : grid;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total = a * b * (d / 8);
   // rows of up to 1 KiB: by tiles of kSwapA x kSwapB rows (a launch holds fewer than 2^32 threads; the kernel's offsets 32 bits)
@@ -789,7 +801,7 @@ int dtas_split3_f16(const void* A, void* out0, void* out1, void* out2, int64_t r
   const bool vec = d % 8 == 0 && aligned(A, 16) && aligned(out0, 16) && aligned(out1, 16) && aligned(out2, 16);
   const int64_t per_sec = vec ? d / 8 : d;
   int64_t grid = ceil_div(rows * 3 * per_sec, kBlock);
-  grid = grid > int64_t{kNumCU} * 64 ? int64_t{kNumCU} * 64 : grid;
+  grid = grid > kMaxGrid ? kMaxGrid : grid;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total = rows * 3 * per_sec;
   const bool narrow = total < (int64_t{1} << 31);   // 32-bit indices while they fit

@@ -380,7 +380,7 @@ extern "C" int dtas_take_q8_f16(const void* Wq, const void* scale, const void* i
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t items = cfg.vec == 8 ? n * K / 8 : n * K;
   int64_t grid = ceil_div(items, 256);
-  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{kNumCU} * 64;
+  const int64_t cap = cfg.grid_cap > 0 ? cfg.grid_cap : int64_t{1} << 23;   // (a thread per item while a launch may hold them: a capped grid that loops is slower)
   grid = grid > cap ? cap : grid;
   if (cfg.vec == 8)
     hipLaunchKernelGGL(take_q8_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, static_cast<const u32x2*>(Wq),
