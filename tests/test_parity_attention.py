@@ -151,7 +151,10 @@ def _check_pv(got, p, v, oracle):
 
 
 @pytest.mark.parametrize("n,m", [(1, 1), (1, 77), (1, 2048), (3, 300), (8, 129), (9, 64), (9, 77), (64, 64), (130, 200),
-                                 (257, 520), (1024, 1024)])
+                                 (257, 520), (1024, 1024),
+                                 # the fitted choice of tile and key split up to one 128-row tile per CU: 64x64 whole and in parts,
+                                 # 64x128 in 2 / 4 / 8 parts, 128x128 in 2 parts
+                                 (128, 128), (64, 1024), (256, 1024), (256, 4096), (128, 4100), (16, 8192), (384, 4096), (192, 2049)])
 def test_pv_builtin_config(oracle, n, m):
     p, v = _pv_inputs(32, n, m, 80, 3 * n + m)
     out = Guarded((1, 32, n, 80), torch.float16)
