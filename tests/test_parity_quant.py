@@ -222,7 +222,12 @@ Q8_GEMM_CONFIGS = [None,
                    # K split over workgroups: the parts meet in the split-K workspace as the fp16 GEMM's do
                    dict(variant=0, block=256, vec=8, unroll=3, tile=[256, 128, 64], split_k=2),
                    dict(variant=0, block=256, vec=8, unroll=3, tile=[128, 128, 64], split_k=3),
-                   dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=8)]
+                   dict(variant=0, block=256, vec=8, unroll=2, tile=[64, 64, 64], split_k=8),
+                   # the three-stage tiles of the fitted built-in choice
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[64, 64, 64]),
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[128, 64, 64], split_k=2),
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[64, 128, 64]),
+                   dict(variant=0, block=256, vec=8, unroll=3, tile=[64, 64, 64], split_k=6)]
 
 
 @pytest.mark.parametrize("which", range(len(Q8_GEMM_CONFIGS)))
@@ -243,7 +248,7 @@ def test_gemm_q8_every_tile_on_ragged_shapes(oracle, which, M, N, K, kind):
     _check_gemm_q8(out.check(), a, wq, scale, bias, r1, r2, kind, oracle)
 
 
-@pytest.mark.parametrize("M", [1, 16, 32, 64, 128, 256, 512, 2048])
+@pytest.mark.parametrize("M", [1, 16, 32, 64, 96, 128, 192, 256, 384, 512, 2048])
 @pytest.mark.parametrize("N,K,kind", [(7680, 2560, 0), (10240, 2560, 3), (2560, 10240, 0), (2560, 2560, 1)])
 def test_gemm_q8_at_the_models_shapes(oracle, M, N, K, kind):
     rng = np.random.default_rng(M + N + kind)
