@@ -77,7 +77,8 @@ class ReductionConfigEmiter(BaseConfigEmiter):
         """Candidates for libdtas_gfx950.so's row kernels, the library's own built-in choice first:
         a workgroup per row with about two 128-bit vectors per thread (sized in multiples of 64 threads
         so that no lane idles), several rows per trip once there are >= 8 rows per CU; for dynamic rows
-        (softmax: 32 rows per unit of row length) a wavefront per row below 512 vectors."""
+        (softmax: 32 rows per unit of row length) a wavefront per row up to 512 vectors, four
+        wavefronts per row up to 2048."""
         vec = 16 // in_bytes
         nvec = -(-re_range.end // vec)
         rows = row_range.end
@@ -102,7 +103,9 @@ class ReductionConfigEmiter(BaseConfigEmiter):
         pref = round64(-(-nvec // 2))                       # ~2 vectors per thread
         narrow = round64(-(-nvec // 5))                     # ~5 vectors per thread
         two_params = self.func_info.in_dtype == "float32" and not self.func_info.dyn_red   # layer norm: gamma and beta
-        multi = (2 if two_params else 4) if many_rows else 1
+        multi = (2 if two_params else 4) if many_rows and not self.func_info.dyn_red else 1   # softmax: one row per trip
+        if self.func_info.dyn_red and 512 <= nvec <= 2048:
+            pref = 256                                      # softmax rows of 2 .. 8 vectors per thread of 4 wavefronts
         block_sizes = [pref, narrow] + [t for t in (64, 128, 256, 320, 512, 1024) if t not in (pref, narrow)]
         if two_params and many_rows and rows <= 16 * self.arch.num_sm:
             block_sizes = [narrow, pref] + block_sizes[2:]
@@ -113,7 +116,7 @@ class ReductionConfigEmiter(BaseConfigEmiter):
                     block_rows.append(cand("shared.dyn", tx, rpt))
         wave_order = (64, 128, 256, 512) if nvec <= 64 else (256, 128, 512, 64)
         wave_rows = [cand("local", tx, rpt) for rpt in (1, 2) for tx in wave_order]
-        wave_first = self.func_info.dyn_red and nvec < 64 * 8 and rows > 2 * self.arch.num_sm
+        wave_first = self.func_info.dyn_red and (nvec < 64 * 8 or (nvec == 64 * 8 and rows <= 32 * self.arch.num_sm)) and rows > 2 * self.arch.num_sm
         ordered = (wave_rows + block_rows) if wave_first else (block_rows[:2] + wave_rows[:2] + block_rows[2:] + wave_rows[2:])
         out = [c for c in ordered if c is not None]
         stream = cand("cache", 1024 if re_range.end >= 4096 else 256)

@@ -235,6 +235,22 @@ def test_reduction_emitters_lead_with_the_librarys_builtin_choice():
                 assert got[k] == want[k], (func.name, n_hi, got, want)
 
 
+def test_softmax_emitter_leads_with_the_librarys_builtin_choice():
+    # rows of dynamic length m, 32 * n of them: a wavefront per row up to 512 vectors, then four wavefronts per row
+    # up to 2048, then wider workgroups
+    for func, op in ((pf.fused_softmax_cast3(32), _lib.OP_SOFTMAX_F32_F16), (pf.softmax_scores(32), _lib.OP_SOFTMAX_F16)):
+        for n_hi in (16, 128, 1024):
+            for m_hi in (64, 256, 1024, 2048, 4096, 8192, 16384, 32768):
+                names = [v.name for v in func.dynamic_args]
+                if names == ["n"]:
+                    n_hi = m_hi                     # square scores: one extent is both the row factor and the row length
+                want = _lib.select_bucket(op, m_hi, 32 * n_hi, m_hi).config.to_dict()
+                ranges = tuple(Range(nm, (n_hi if nm == "n" else m_hi) - 15, n_hi if nm == "n" else m_hi) for nm in names)
+                got = _first_candidate(func, ranges)
+                for k in ("variant", "block", "vec", "unroll"):
+                    assert got[k] == want[k], (func.name, n_hi, m_hi, got, want)
+
+
 def test_builtin_tables_name_a_launchable_kernel_for_every_bucket_and_shape():
     # whatever the extents, the row the built-in table returns must be one its own launch description accepts
     # (no GPU needed: both are host code), with a tile the kernels exist for and a split that keeps 8 k tiles

@@ -133,7 +133,19 @@ def test_softmax_f16_large_rows_sampled(oracle, n):
     assert bool((out.argmax(-1) == x.argmax(-1)).float().mean() > 0.999)  # ties in fp16 aside
 
 
-@pytest.mark.parametrize("rows,cols", [(12800, 400), (1000, 1000), (32 * 5, 4096), (7, 8192), (3, 3000), (5, 20000)])
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (600, 4096), (700, 12288), (520, 5002), (530, 16384), (96, 40000)])
+def test_softmax_f16_rows_not_tied_to_the_row_length(oracle, rows, cols):
+    # chunked attention: every branch of the built-in choice (a wavefront per row at exactly 8 vectors per lane
+    # and few rows, four wavefronts per row up to 2048 vectors, wider workgroups and the streaming form beyond)
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2).astype(np.float16)
+    out = Guarded(x.shape, torch.float16)
+    ops.softmax(dev(x), out.t)
+    _check(out.check(), oracle.c.softmax(x, threads=8), oracle.np64.softmax(x))
+
+
+@pytest.mark.parametrize("rows,cols", [(12800, 400), (1000, 1000), (32 * 5, 4096), (7, 8192), (3, 3000), (5, 20000),
+                                       (4096, 2048), (600, 2048), (600, 6144), (520, 5001), (300, 8192), (130, 16384)])
 def test_softmax_f32_reference_signature(oracle, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = (rng.standard_normal((1, rows, cols)) * 2).astype(np.float32)
