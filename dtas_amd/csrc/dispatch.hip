@@ -83,20 +83,70 @@ dtas_config block_row(int vec, int64_t nvec, int rows_per_trip) {
   return make(DTAS_RED_BLOCK_ROW, static_cast<int>(block), vec, rows_per_trip);
 }
 
-// Norms: n rows of static length H, a workgroup per row.  From ~8 rows per CU on, a workgroup
-// takes several rows per trip: their loads are in flight together and the per-column parameters
-// are fetched once for all of them (4 rows for RMSNorm's one parameter vector, 2 for
-// LayerNorm's two fp32 ones, which cost registers).
+// the vectors-per-thread counts the register kernels are instantiated for
+int64_t row_iters(int64_t nvec, int64_t block) {
+  const int64_t v = (nvec + block - 1) / block;
+  for (int64_t i : {1, 2, 3, 4, 5, 6, 8, 10, 12, 16})
+    if (i >= v) return i;
+  return 17;
+}
+
+int64_t round64(int64_t v) { return v < 64 ? 64 : v > 1024 ? 1024 : (v + 63) / 64 * 64; }
+
+// A workgroup of `block` threads per `rpt` rows where the kernels have that form (2 rows up to 8 vectors per
+// thread, 4 up to 4, more than 8 vectors per thread in all only up to 512 threads); else block_row's choice.
+dtas_config row_cfg(int vec, int64_t nvec, int64_t block, int rpt) {
+  const int64_t it = row_iters(nvec, block);
+  const bool ok = it <= 16 && (rpt == 1 || (rpt == 2 && it <= 8) || (rpt == 4 && it <= 4)) && (it * rpt <= 8 || block <= 512);
+  return ok ? make(DTAS_RED_BLOCK_ROW, static_cast<int>(block), vec, rpt) : block_row(vec, nvec, rpt);
+}
+
+// Norms: n rows of static length H, a workgroup per row or per few rows.  Rows of 320 .. 1024 vectors (RMSNorm:
+// H = 2560 .. 8192) and 512 .. 2048 (LayerNorm, the same H) follow sweeps of every block size x rows per trip
+// at H = 2560, 4096, 5120, 8192 and n = 256 .. 16384, which show three regimes:
+//  * up to 4 rows per CU: one row per workgroup and ~2 vectors per thread (latency: the most threads per row);
+//  * 4 .. 16-24 rows per CU: the configs that keep every row resident in one round win, and among them those
+//    that take several rows per trip (the per-column parameters are fetched once per trip: LayerNorm's two
+//    fp32 vectors are otherwise twice the traffic of the row itself) in workgroups of 128 .. 256 threads
+//    (LayerNorm H = 5120, n = 1536: 9.6 us against 13.2 with one row of 640 threads, whose 1536 workgroups
+//    need two rounds; RMSNorm H = 8192, n = 4096: 22.5 against 26.6);
+//  * beyond: RMSNorm one row per trip at ~3 vectors per thread (H = 8192, n = 16384: 85.4 against 94.0 with
+//    4 rows per trip), LayerNorm two rows at ~2.
+// Mean / worst ratio to the best swept config over that grid: 1.02 / 1.15 (1.08 / 1.37 with the single rule
+// "~2 vectors per thread, 4 or 2 rows per trip from 8 rows per CU").  Other row lengths keep that single rule.
 dtas_config norm_policy(int op, int64_t n_hi, int64_t H) {
-  const int vec = op == DTAS_OP_RMS_NORM_F16 ? 8 : 4;
+  const bool rms = op == DTAS_OP_RMS_NORM_F16;
+  const int vec = rms ? 8 : 4;
   const int64_t nvec = (H + vec - 1) / vec;
-  if (op == DTAS_OP_RMS_NORM_F16) return block_row(vec, nvec, n_hi >= 8 * kNumCU ? 4 : 1);
+  const int64_t pref = round64((nvec + 1) / 2), narrow = round64((nvec + 4) / 5);
+  const int64_t n4 = 4 * kNumCU, n8 = 8 * kNumCU, n12 = 12 * kNumCU, n16 = 16 * kNumCU, n24 = 24 * kNumCU;
+  if (rms && nvec >= 256 && nvec <= 1024) {
+    if (n_hi <= n4) return block_row(vec, nvec, 1);
+    if (n_hi < n8 || (n_hi == n8 && nvec < 1024)) return row_cfg(vec, nvec, pref < 256 ? pref : 256, 2);
+    if (n_hi <= n24 && nvec < 512) return row_cfg(vec, nvec, pref, n_hi <= n12 ? 2 : 4);
+    if (n_hi <= n16) return row_cfg(vec, nvec, nvec >= 512 ? 256 : pref, 4);
+    return row_cfg(vec, nvec, round64((nvec + 2) / 3), 1);
+  }
+  if (!rms && nvec >= 512 && nvec <= 2048) {
+    if (n_hi < n4) return block_row(vec, nvec, 1);
+    if (n_hi < n8) {
+      if (nvec <= 640) return row_cfg(vec, nvec, pref, n_hi <= n4 ? 1 : 2);
+      return row_cfg(vec, nvec, nvec <= 1024 ? 320 : 256, 2);
+    }
+    if (n_hi <= n16) {
+      if (nvec <= 640) return row_cfg(vec, nvec, narrow, 2);
+      if (nvec <= 1024) return n_hi <= n12 ? row_cfg(vec, nvec, 128, 2) : row_cfg(vec, nvec, 256, 4);
+      if (n_hi <= n8) return nvec < 2048 ? row_cfg(vec, nvec, 256, 2) : row_cfg(vec, nvec, 512, 4);
+      return row_cfg(vec, nvec, 768, 2);
+    }
+    return block_row(vec, nvec, 2);
+  }
+  if (rms) return block_row(vec, nvec, n_hi >= n8 ? 4 : 1);
   // LayerNorm, 8 to 16 rows per CU: narrow workgroups (about five vectors per thread) are all
   // co-resident and measured ~15 % faster than wide ones, which need a second, partial round.
-  const int64_t narrow = ((nvec + 4) / 5 + 63) / 64 * 64;
-  if (n_hi >= 8 * kNumCU && n_hi <= 16 * kNumCU && narrow <= 1024 && (nvec + narrow - 1) / narrow <= 5)
-    return make(DTAS_RED_BLOCK_ROW, static_cast<int>(narrow), vec, 2);
-  return block_row(vec, nvec, n_hi >= 8 * kNumCU ? 2 : 1);
+  if (n_hi >= n8 && n_hi <= n16 && (nvec + narrow - 1) / narrow <= 5 && narrow <= 512)
+    return row_cfg(vec, nvec, narrow, 2);
+  return block_row(vec, nvec, n_hi >= n8 ? 2 : 1);
 }
 
 // Softmax: 32*n rows of dynamic length n (the reduction axis is the dynamic one).  One wavefront

@@ -73,6 +73,46 @@ class ReductionConfigEmiter(BaseConfigEmiter):
             return sorted(configs, key=lambda c: (c.max_active_blocks_per_sm, c.len_tx, c.vector_size), reverse=True)[:topk]
         return configs
 
+    @staticmethod
+    def _norm_choice(rms: bool, n_hi: int, nvec: int, num_cu: int) -> Optional[Tuple[int, int]]:
+        """(threads, rows per trip) of the library's built-in choice for a norm over rows of ``nvec`` 128-bit
+        vectors, where it was fitted to sweeps (dispatch.hip:norm_policy, the same rule): up to 4 rows per CU one
+        row per workgroup at ~2 vectors per thread; up to 16 .. 24 rows per CU the forms that keep every row
+        resident in one round and fetch the per-column parameters once for several rows; beyond, RMSNorm one row
+        at ~3 vectors per thread and LayerNorm two rows at ~2.  None outside the fitted row lengths."""
+        def round64(v: int) -> int:
+            return min(1024, max(64, -(-v // 64) * 64))
+
+        pref, narrow = round64(-(-nvec // 2)), round64(-(-nvec // 5))
+        n4, n8, n12, n16, n24 = (k * num_cu for k in (4, 8, 12, 16, 24))
+        if rms and 256 <= nvec <= 1024:
+            if n_hi <= n4:
+                return pref, 1
+            if n_hi < n8 or (n_hi == n8 and nvec < 1024):
+                return min(pref, 256), 2
+            if n_hi <= n24 and nvec < 512:
+                return pref, 2 if n_hi <= n12 else 4
+            if n_hi <= n16:
+                return (256 if nvec >= 512 else pref), 4
+            return round64(-(-nvec // 3)), 1
+        if not rms and 512 <= nvec <= 2048:
+            if n_hi < n4:
+                return pref, 1
+            if n_hi < n8:
+                if nvec <= 640:
+                    return pref, 1 if n_hi <= n4 else 2
+                return (320 if nvec <= 1024 else 256), 2
+            if n_hi <= n16:
+                if nvec <= 640:
+                    return narrow, 2
+                if nvec <= 1024:
+                    return (128, 2) if n_hi <= n12 else (256, 4)
+                if n_hi <= n8:
+                    return (256, 2) if nvec < 2048 else (512, 4)
+                return 768, 2
+            return pref, 2
+        return None
+
     def _gfx950_candidates(self, re_range: Range, row_range: Range, in_bytes: int, topk: int) -> List[ReductionConfig]:
         """Candidates for libdtas_gfx950.so's row kernels, the library's own built-in choice first:
         a workgroup per row with about two 128-bit vectors per thread (sized in multiples of 64 threads
@@ -107,7 +147,7 @@ class ReductionConfigEmiter(BaseConfigEmiter):
         if self.func_info.dyn_red and 512 <= nvec <= 2048:
             pref = 256                                      # softmax rows of 2 .. 8 vectors per thread of 4 wavefronts
         block_sizes = [pref, narrow] + [t for t in (64, 128, 256, 320, 512, 1024) if t not in (pref, narrow)]
-        if two_params and many_rows and rows <= 16 * self.arch.num_sm:
+        if two_params and many_rows and rows <= 16 * self.arch.num_sm and -(-nvec // narrow) <= 5 and narrow <= 512:
             block_sizes = [narrow, pref] + block_sizes[2:]
         block_rows = []
         for tx in block_sizes:
@@ -118,6 +158,10 @@ class ReductionConfigEmiter(BaseConfigEmiter):
         wave_rows = [cand("local", tx, rpt) for rpt in (1, 2) for tx in wave_order]
         wave_first = self.func_info.dyn_red and (nvec < 64 * 8 or (nvec == 64 * 8 and rows <= 32 * self.arch.num_sm)) and rows > 2 * self.arch.num_sm
         ordered = (wave_rows + block_rows) if wave_first else (block_rows[:2] + wave_rows[:2] + block_rows[2:] + wave_rows[2:])
+        fitted = None if self.func_info.dyn_red else self._norm_choice(not two_params, rows, nvec, self.arch.num_sm)
+        if fitted is not None and cand("shared.dyn", *fitted) is not None:
+            ordered = [cand("shared.dyn", *fitted)] + [c for c in ordered if c is not None and
+                                                         (c.temp_storage, c.len_tx, c.rows_per_trip) != ("shared.dyn",) + fitted]
         out = [c for c in ordered if c is not None]
         stream = cand("cache", 1024 if re_range.end >= 4096 else 256)
         stream.vector_size = 1

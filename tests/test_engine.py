@@ -226,13 +226,28 @@ def test_gemm_emitter_leads_with_the_librarys_builtin_choice(N, K):
 
 
 def test_reduction_emitters_lead_with_the_librarys_builtin_choice():
-    cases = [(pf.rms_norm(4096), _lib.OP_RMS_NORM_F16, 4096), (pf.fused_layer_norm_cast1(2560), _lib.OP_LAYER_NORM_F32_F16, 2560)]
+    cases = [(mk(H), op, H) for H in (1024, 2560, 4096, 5120, 6144, 8192, 16384)
+             for mk, op in ((pf.rms_norm, _lib.OP_RMS_NORM_F16), (pf.fused_layer_norm_cast1, _lib.OP_LAYER_NORM_F32_F16))]
     for func, op, H in cases:
-        for n_hi in (16, 256, 1024, 2048, 4096, 8192):
+        for n_hi in (16, 256, 1024, 1040, 1536, 2032, 2048, 2064, 3072, 3088, 4096, 4112, 6144, 6160, 8192):
             want = _lib.select_bucket(op, n_hi, H, 0).config.to_dict()
             got = _first_candidate(func, (Range("n", n_hi - 15, n_hi),))
             for k in ("variant", "block", "vec", "unroll"):
                 assert got[k] == want[k], (func.name, n_hi, got, want)
+
+
+def test_builtin_reduction_rows_are_launchable_for_every_extent():
+    # the table row for any row count x row length must be a form the register kernels exist in (select_bucket
+    # describes its launch and fails otherwise): LayerNorm over rows of 16384 once named 832 threads x 2 rows
+    lengths = (1, 8, 64, 100, 777, 1024, 2048, 2560, 3072, 4096, 4100, 5120, 6144, 8192, 10240, 12288, 16384, 20000, 32768, 65536)
+    for n_hi in (1, 16, 512, 1024, 1040, 2047, 2048, 3000, 4096, 4097, 6144, 8192, 10 ** 5):
+        for H in lengths:
+            for op in (_lib.OP_RMS_NORM_F16, _lib.OP_LAYER_NORM_F32_F16):
+                info = _lib.select_bucket(op, n_hi, H, 0)
+                assert info.launch_args[0] >= 1 and 64 <= info.launch_args[3] <= 1024, (op, n_hi, H)
+            for op in (_lib.OP_SOFTMAX_F32_F16, _lib.OP_SOFTMAX_F16):
+                info = _lib.select_bucket(op, H, 32 * n_hi, H)
+                assert info.launch_args[0] >= 1 and 64 <= info.launch_args[3] <= 1024, (op, n_hi, H)
 
 
 def test_softmax_emitter_leads_with_the_librarys_builtin_choice():

@@ -42,6 +42,43 @@ def test_rms_norm_other_row_lengths(oracle, H):
     _check(out.check(), oracle.c.rms_norm(x, w), oracle.np64.rms_norm(x, w))
 
 
+# one n per branch of the built-in choice (rows per CU: up to 4, 4 .. 8, 8, 8 .. 12, 12 .. 16, 16 .. 24, beyond)
+REGIME_N = [1000, 1500, 2048, 3000, 4090, 6001, 8200]
+
+
+@pytest.mark.parametrize("n", REGIME_N)
+@pytest.mark.parametrize("H", [2560, 5120, 6144, 8192, 16384])
+def test_rms_norm_builtin_over_row_lengths_and_counts(oracle, n, H):
+    rng = np.random.default_rng(n + H)
+    x = rng.standard_normal((n, H), dtype=np.float32).astype(np.float16)
+    w = rng.uniform(0.5, 1.5, H).astype(np.float16)
+    out = Guarded(x.shape, torch.float16)
+    ops.rms_norm(dev(x), dev(w), out.t)
+    got = out.check()
+    rows = np.unique(np.concatenate([[0, 1, 2, 3, n - 4, n - 3, n - 2, n - 1], rng.integers(0, n, 120)]))
+    _check(got[rows], oracle.c.rms_norm(x[rows], w), oracle.np64.rms_norm(x[rows], w))
+    # every row, against the closed form of its own output: sum (out / w)^2 = H * sum x^2 / (sum x^2 + H eps)
+    ss = (x.astype(np.float64) ** 2).sum(-1)
+    assert np.abs(((got.astype(np.float64) / w.astype(np.float64)) ** 2).sum(-1) / (H * ss / (ss + H * 1e-5)) - 1).max() < 5e-3
+
+
+@pytest.mark.parametrize("n", REGIME_N)
+@pytest.mark.parametrize("H", [4096, 5120, 6144, 8192, 16384])
+def test_layer_norm_builtin_over_row_lengths_and_counts(oracle, n, H):
+    rng = np.random.default_rng(n + H + 1)
+    x = (rng.standard_normal((n, H), dtype=np.float32) * 2 + 0.5)
+    g = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    b = rng.uniform(-1, 1, H).astype(np.float32)
+    out = Guarded(x.shape, torch.float16)
+    ops.layer_norm(dev(x), dev(g), dev(b), out.t)
+    got = out.check()
+    rows = np.unique(np.concatenate([[0, 1, 2, 3, n - 4, n - 3, n - 2, n - 1], rng.integers(0, n, 120)]))
+    _check(got[rows], oracle.c.layer_norm(x[rows], g, b), oracle.np64.layer_norm(x[rows], g, b))
+    # every row: the normalised values ((out - beta) / gamma) have mean 0 and variance 1
+    z = (got.astype(np.float64) - b) / g
+    assert np.abs(z.mean(-1)).max() < 5e-3 and np.abs(z.var(-1) - 1).max() < 1e-2
+
+
 RED_VARIANTS = [(_lib.RED_WAVE_ROW, b) for b in (64, 128, 256, 512)] + \
                [(_lib.RED_BLOCK_ROW, b) for b in (64, 256, 512, 1024)] + [(_lib.RED_STREAM_ROW, b) for b in (64, 256, 1024)]
 
