@@ -73,4 +73,12 @@ class ElementwiseConfigEmiter(BaseConfigEmiter):
             short = c.grid_size < target // 2
             return (c.vector_size != preferred, short and c.unroll_depth > 1, -c.unroll_depth if not short else c.unroll_depth)
 
-        return sorted(configs, key=score)[:topk]
+        ranked = sorted(configs, key=score)
+        # eight accesses per thread only while all workgroups are resident at once (8 per CU, 6 for the two-input
+        # ops); beyond one round many short workgroups are ahead (dispatch.hip:elementwise_policy, the same rule)
+        two_inputs = len(self.func_info.func.params) > 2
+        first = ranked[0]
+        if first.unroll_depth == 8 and num_elements // first.vector_size // (256 * 8) > (6 if two_inputs else 8) * self.arch.num_sm:
+            want = 2 if (self.func_info.in_dtype, self.func_info.out_dtype) == ("float32", "float16") else 1
+            ranked.sort(key=lambda c: (c.vector_size != first.vector_size, c.unroll_depth != want))
+        return ranked[:topk]

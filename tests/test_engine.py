@@ -236,6 +236,24 @@ def test_reduction_emitters_lead_with_the_librarys_builtin_choice():
                 assert got[k] == want[k], (func.name, n_hi, got, want)
 
 
+def test_elementwise_emitter_leads_with_the_librarys_builtin_choice():
+    # the deepest unroll that leaves every CU a few workgroups -- and one access per thread (two for the cast to
+    # fp16) once eight per thread no longer fit the chip in one round
+    cases = [(pf.add("float16", H), _lib.OP_ADD_F16, H) for H in (2560, 4096)] + \
+            [(pf.cast("float32", "float16", H), _lib.OP_CAST_F32_F16, H) for H in (2560, 4096)] + \
+            [(pf.cast("float16", "float32", 4096), _lib.OP_CAST_F16_F32, 4096), (pf.copy("float16", 4096), _lib.OP_COPY_F16, 4096),
+             (pf.add("float32", 4096), _lib.OP_ADD_F32, 4096), (pf.add("int8", 4096), _lib.OP_ADD_I8, 4096)]
+    seen = set()
+    for func, op, H in cases:
+        for n_hi in (16, 128, 512, 1024, 2048, 4096, 4112, 5120, 6144, 6160, 7168, 8192):
+            want = _lib.select_bucket(op, n_hi, H, 0).config.to_dict()
+            got = _first_candidate(func, (Range("n", n_hi - 15, n_hi),))
+            for k in ("variant", "block", "vec", "unroll"):
+                assert got[k] == want[k], (func.name, H, n_hi, got, want)
+            seen.add((op, want["unroll"]))
+    assert {(_lib.OP_ADD_F16, 8), (_lib.OP_ADD_F16, 1), (_lib.OP_CAST_F32_F16, 2), (_lib.OP_COPY_F16, 8)} <= seen
+
+
 def test_builtin_reduction_rows_are_launchable_for_every_extent():
     # the table row for any row count x row length must be a form the register kernels exist in (select_bucket
     # describes its launch and fails otherwise): LayerNorm over rows of 16384 once named 832 threads x 2 rows
