@@ -157,9 +157,10 @@ dtas_config norm_policy(int op, int64_t n_hi, int64_t H) {
 // Softmax: 32*n rows of dynamic length n (the reduction axis is the dynamic one).  One wavefront
 // per row (reductions on the DPP path only) up to 8 vectors per lane; short rows launch one
 // row per workgroup so that the many small workgroups spread evenly.  Longer rows, or few
-// rows, take a workgroup per row: 4 wavefronts up to 8 vectors per lane (several such workgroups
-// share a CU and overlap one row's reduction with another's loads: 4096 rows of 8192 fp32 33.2 us
-// against 38.9 with 1024 threads, 16384 rows 124 against 138), wider ones beyond.
+// rows, take a workgroup per row: up to 2048 vectors 4 wavefronts while there are at most 32 rows per CU
+// (several such workgroups share a CU and overlap one row's reduction with another's loads: 4096 rows of
+// 8192 fp32 33.2 us against 38.9 with 1024 threads) and 4 .. 8 wavefronts at ~3 vectors per thread for
+// more rows; wider workgroups for longer rows.
 dtas_config softmax_policy(int op, int64_t cols_hi, int64_t rows) {
   const int vec = op == DTAS_OP_SOFTMAX_F16 ? 8 : 4;
   const int64_t nvec = (cols_hi + vec - 1) / vec;
@@ -167,7 +168,12 @@ dtas_config softmax_policy(int op, int64_t cols_hi, int64_t rows) {
   // against 13.8 -- beyond, four wavefronts per row are as fast or 2 % faster)
   if ((nvec < 64 * 8 || (nvec == 64 * 8 && rows > 0 && rows <= 32 * kNumCU)) && (rows <= 0 || rows > 2 * kNumCU))
     return make(DTAS_RED_WAVE_ROW, nvec <= 64 ? 64 : 256, vec, 1);
-  if (nvec >= 64 * 8 && nvec <= 256 * 8) return make(DTAS_RED_BLOCK_ROW, 256, vec, 1);
+  if (nvec >= 64 * 8 && nvec <= 256 * 8) {
+    // (beyond 32 rows per CU ~3 vectors per thread in 256 .. 512 threads: 262144 rows of 8192 fp16 1387 us against 1491)
+    int64_t block = 256;
+    if (rows <= 0 || rows > 32 * kNumCU) block = round64((nvec + 2) / 3) < 256 ? 256 : round64((nvec + 2) / 3) > 512 ? 512 : round64((nvec + 2) / 3);
+    return make(DTAS_RED_BLOCK_ROW, static_cast<int>(block), vec, 1);
+  }
   return block_row(vec, nvec, 1);
 }
 

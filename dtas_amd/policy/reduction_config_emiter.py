@@ -145,7 +145,9 @@ class ReductionConfigEmiter(BaseConfigEmiter):
         two_params = self.func_info.in_dtype == "float32" and not self.func_info.dyn_red   # layer norm: gamma and beta
         multi = (2 if two_params else 4) if many_rows and not self.func_info.dyn_red else 1   # softmax: one row per trip
         if self.func_info.dyn_red and 512 <= nvec <= 2048:
-            pref = 256                                      # softmax rows of 2 .. 8 vectors per thread of 4 wavefronts
+            # softmax rows of 512 .. 2048 vectors: 4 wavefronts up to 32 rows per CU, ~3 vectors per thread in 256 .. 512
+            # threads beyond
+            pref = 256 if rows <= 32 * self.arch.num_sm else min(512, max(256, round64(-(-nvec // 3))))
         block_sizes = [pref, narrow] + [t for t in (64, 128, 256, 320, 512, 1024) if t not in (pref, narrow)]
         if two_params and many_rows and rows <= 16 * self.arch.num_sm and -(-nvec // narrow) <= 5 and narrow <= 512:
             block_sizes = [narrow, pref] + block_sizes[2:]
