@@ -337,7 +337,11 @@ extern "C" int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale
   // measured over N = 2560 .. 50280 against K = 2560 .. 11008 (12 launch shapes each): 4 rows per workgroup from 4096 rows
   // on, 2 below; 8 wavefronts for K >= 8192 with those 4 rows, 4 wavefronts otherwise (7680 x 10240: 15.4 us against 17.7 for 2 rows on 4 wavefronts,
   // 11008 x 5120: 11.8 / 13.9, 4096 x 5120: 6.4 / 7.4; level at K = 4096)
-  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, K >= 8192 && N >= 4096 ? 512 : 256, 8, 2, {N >= 4096 ? 4 : 2, 0, 0}, 1, 0};
+  // short rows (K <= 2048) from 12288 rows on: 2 wavefronts, and 8 rows per workgroup when K <= 1024 and N >= 16384 (28672 x 1024:
+  // 8.1 us against 10.0; 13824 x 1024: 5.4 / 6.3 with 4 rows; 28672 x 2048: 11.8 / 13.0)
+  const int q8_block = K >= 8192 && N >= 4096 ? 512 : K <= 2048 && N >= 12288 ? 128 : 256;
+  const int q8_rows = N >= 4096 ? (K <= 1024 && N >= 16384 ? 8 : 4) : 2;
+  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, q8_block, 8, 2, {q8_rows, 0, 0}, 1, 0};
   if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
   int64_t la[7];
   if (describe_gemv(N, K, cfg, la) != 0) return -1;

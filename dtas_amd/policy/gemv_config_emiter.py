@@ -25,7 +25,13 @@ class GEMVConfigEmiter(BaseConfigEmiter):
         # measured on MI355X: one row per 4-wavefront workgroup is best or within noise for K = 4096;
         # rows of K >= 8192 do better with 8 wavefronts on two rows, and rows that leave the last pass of 4 wavefronts
         # partly empty (K = 2560) with two rows on those 4
-        best = (2, 512) if K >= 8192 else (2, 256) if K % 2048 != 0 else (1, 256)
+        # (short rows: up to 1024 elements one pass of 2 wavefronts, up to 2048 one pass of 4, several rows per workgroup)
+        best = (2, 512) if K >= 8192 else (4 if N >= 12288 else 2, 128) if K <= 1024 else (2, 256) if K <= 2048 or K % 2048 != 0 else (1, 256)
+
+        if not any((c.TILE_S, c.TR) == best for c in out):
+            c = GEMVConfig()
+            c.TILE_S, c.TR = best
+            out.append(c)
 
         def score(c: GEMVConfig):
             return ((c.TILE_S, c.TR) != best, c.TILE_S, c.TR != 256)

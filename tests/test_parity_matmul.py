@@ -27,7 +27,9 @@ def _inputs(M, N, K, seed):
     return rng.standard_normal((M, K)).astype(np.float16), (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
 
 
-GEMV_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)]
+GEMV_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096),
+               # short rows (2 wavefronts on 2 or 4 rows, 4 on 2) and the other branches of the built-in choice
+               (5120, 1024), (13824, 1024), (8192, 2048), (3000, 520), (7680, 2560), (2560, 10240), (300, 72)]
 
 
 @pytest.mark.parametrize("N,K", GEMV_SHAPES)

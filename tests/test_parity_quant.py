@@ -69,7 +69,8 @@ def _check_gemv(got, x, wq, scale, bias, kind, oracle):
     assert (got == want).mean() > 0.9
 
 
-@pytest.mark.parametrize("N,K", [(7680, 2560), (2560, 10240), (10240, 2560), (50280, 2560), (33, 64), (5, 32)])
+@pytest.mark.parametrize("N,K", [(7680, 2560), (2560, 10240), (10240, 2560), (50280, 2560), (33, 64), (5, 32),
+                                 (13824, 1024), (16400, 512), (12300, 2048), (5120, 1024), (4096, 8192)])
 @pytest.mark.parametrize("kind", [_lib.EPI_BIAS, _lib.EPI_BIAS_GELU])
 def test_gemv_builtin_config(oracle, N, K, kind):
     rng = np.random.default_rng(N + K + kind)
