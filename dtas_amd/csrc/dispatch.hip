@@ -270,7 +270,8 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     consider(floored(6.0 + gemm_rounds(tiles_of(192, 128), kNumCU) * 0.66 * kt, 3.5), 192, 128, 512, 2, 1);
   consider(floored(gemm_rounds(tiles_of(128, 128), 2 * kNumCU) * 1.14 * kt, 3.1), 128, 128, 256, 2, 1);
   for (int split = 1; split <= 4; ++split) {
-    if (split > 1 && ktiles / split < 8) continue;
+    // (K <= 1024: a launch is mostly its start, and a hand-over costs what the shorter loop saves: 512 x 1024 x 1024 7.8 us whole, 8.6 in two parts)
+    if (split > 1 && (ktiles / split < 8 || ktiles <= 16)) continue;
     const double steps = static_cast<double>(ceil_div(ktiles, split));
     const double t128 = tiles_of(128, 128) * split, t64 = tiles_of(64, 64) * split;
     if (split == 1 || t128 <= kNumCU)

@@ -81,7 +81,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             cands.append((floored(6.0 + rounds(tiles(192, 128), cus) * 0.66 * ktiles, 3.5), (192, 128, 2, 1)))
         cands.append((floored(rounds(tiles(128, 128), 2 * cus) * 1.14 * ktiles, 3.1), (128, 128, 2, 1)))
         for split in (1, 2, 3, 4):
-            if split > 1 and ktiles // split < 8:
+            if split > 1 and (ktiles // split < 8 or ktiles <= 16):    # (K <= 1024: a hand-over costs what the shorter loop saves)
                 continue
             steps = cdiv(ktiles, split)
             t128, t64 = tiles(128, 128) * split, tiles(64, 64) * split

@@ -211,7 +211,7 @@ def _first_candidate(func, ranges):
     return get_config_emiter_template(info.kind)(info, MI355X()).emit_config(ranges, 20)[0].to_abi().to_dict()
 
 
-@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (2560, 10240)])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (2560, 10240), (4096, 1024), (1024, 1024), (8192, 8192)])
 def test_gemm_emitter_leads_with_the_librarys_builtin_choice(N, K):
     # the closed-form policy exists twice (C tables for cfg == NULL, Python emitter for the tuner's
     # first candidate): they must not drift apart
