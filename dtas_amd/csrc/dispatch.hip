@@ -291,7 +291,8 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   // 17 .. 32 rows: the same with 32 rows of A and 512 of K per workgroup, where that gives a quarter of a round or more
   // and at most one (8.4 against 9.8 us at 2560 x 2560, 9.5 / 10.7 at 2048 x 4096, 11.4 / 13.9 at 1024 x 8192, 8.9 / 10.2 at
   // 3072 x 2560; behind at 1024 x 1024, whose 32 workgroups leave the chip idle)
-  if (M_hi > 16 && M_hi <= 32 && ceil_div(n, 64) * ceil_div(k, 512) <= kNumCU && ceil_div(n, 64) * ceil_div(k, 512) >= kNumCU / 4)
+  // (from K = 2048 on: at 4096 x 1024 the 64x64 tiles take 7.4 us, this form 8.2)
+  if (M_hi > 16 && M_hi <= 32 && k >= 2048 && ceil_div(n, 64) * ceil_div(k, 512) <= kNumCU && ceil_div(n, 64) * ceil_div(k, 512) >= kNumCU / 4)
     return make(DTAS_GEMM_STREAM, 256, 8, 1, 32, 64, 512);
   // M <= 16 against more rows of W: the looping form (the whole of K per workgroup, nothing handed over) while its
   // workgroups run in one round -- 16 columns each (one wavefront, two workgroups per CU) for 4096 < N <= 8192, 64

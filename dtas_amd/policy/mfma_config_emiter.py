@@ -132,7 +132,8 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             return -(-N // 64) * -(-K // 1024) <= self.arch.num_sm
         # 17 .. 32 rows: 32 rows of A and 512 of K per workgroup, between a quarter of a round and one round of them
         # (8.4 against 9.8 us at 2560 x 2560, 11.4 / 13.9 at 1024 x 8192)
-        return m_hi <= 32 and self.arch.num_sm // 4 <= -(-N // 64) * -(-K // 512) <= self.arch.num_sm
+        # (from K = 2048 on: at 4096 x 1024 the 64x64 tiles take 7.4 us, this form 8.2)
+        return m_hi <= 32 and K >= 2048 and self.arch.num_sm // 4 <= -(-N // 64) * -(-K // 512) <= self.arch.num_sm
 
     def prefers_stream_loop(self, m_hi: int, N: int, K: int) -> int:
         """Columns per workgroup (16 or 64) of the looping W-streaming kernel where it leads, else 0: M <= 16, K <= 4096
