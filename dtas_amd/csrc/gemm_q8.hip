@@ -55,9 +55,10 @@ extern "C" int dtas_gemm_q8_f16_fused(const void* A, const void* Wq, const void*
       if (M > 16) return launch_gemm_stream_q8(32, 512, s, a, w, ep, C, M, N, K);
       return launch_gemm_stream_q8(16, K >= 8192 ? 1024 : 512, s, a, w, ep, C, M, N, K);
     }
-    // up to 64 rows (one workgroup per CU) only where the column tiles number at most a quarter of the CUs' slots:
-    // 14.0 against 26.3 us at 64 x 2560 x 2560 and 25.1 against 39.5 at 4096 x 4096, but 38 against 27 at N = 10240
-    if (!user && stream_ok && M <= 64 && N <= 4096 && K <= 4096) return launch_gemm_stream_q8(64, 512, s, a, w, ep, C, M, N, K);
+    // up to 64 rows only while its workgroups (64 columns x 512 of K each) run in one round: 48 rows against 2560 x 2560 /
+    // 2048 x 4096 / 4096 x 2048 11.3 / 12.1 / 10.6 us where the tiles take 11.8 / 12.8 / 11.5, but 16.4 / 16.5 / 21.2 against
+    // 13.0 / 12.5 / 15.5 at 3072 x 3072 / 4096 x 2560 / 4096 x 4096
+    if (!user && stream_ok && M <= 64 && ceil_div(N, 64) * ceil_div(K, 512) <= kNumCU) return launch_gemm_stream_q8(64, 512, s, a, w, ep, C, M, N, K);
   }
   // Two routes.  (1) Dequantising in the W path of the tile kernel: no intermediate, W read once per row of tiles as
   // bytes; a plain burst pipeline on 4 wavefronts, with K split over workgroups while the tiles leave CUs idle.

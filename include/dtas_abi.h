@@ -383,7 +383,7 @@ int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale, void* y, 
  * aligned A, Wq and scale): the W-streaming kernel on the bytes of W, widened between the LDS and the MFMA; its K
  * slices meet in the split-K workspace.  A DTAS_GEMM_MFMA row may carry split_k in [1, 16]: that many workgroups share
  * a tile and meet in the split-K workspace as in dtas_gemm_f16.  One row with a bias or GELU epilogue goes to
- * dtas_gemv_q8_f16.  With cfg == NULL: M <= 32 (M <= 64 with N, K <= 4096) takes the W-streaming kernel where it
+ * dtas_gemv_q8_f16.  With cfg == NULL: M <= 32 (M <= 64 while N / 64 x K / 512 workgroups fit one round of the chip) takes the W-streaming kernel where it
  * applies; up to 512 rows, while 128x128 tiles fit the chip in one round, the tile kernel dequantises in its W path
  * (64x64, 128x64 or 128x128 tiles of three stages with K in 1 .. 8 parts, by a fitted cost model); beyond that the two-pass route:
  * dtas_decode_q8_f16 into a per-device fp16 buffer of its own (allocated on first use, grown on demand, at most

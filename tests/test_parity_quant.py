@@ -266,6 +266,21 @@ def test_gemm_q8_at_the_models_shapes(oracle, M, N, K, kind):
                    None if r1 is None else np.ascontiguousarray(r1[rows]), None if r2 is None else np.ascontiguousarray(r2[rows]), kind, oracle)
 
 
+@pytest.mark.parametrize("M", [33, 48, 64])
+@pytest.mark.parametrize("N,K", [(2048, 4096), (4096, 2048), (3072, 3072), (4096, 2560), (4096, 4096)])
+def test_gemm_q8_33_to_64_rows_either_side_of_one_round_of_the_streaming_form(oracle, M, N, K):
+    # 64 columns x 512 of K per workgroup: the first two shapes are one round of the chip (the W-streaming kernel),
+    # the others more (the tiles with K in parts)
+    rng = np.random.default_rng(M + N + K)
+    wq, scale = _weights(N, K, N + K + 1)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    out = Guarded((1, M, N), torch.float16)
+    ops.gemm_q8(dev(a).view(1, M, K), _words(wq), dev(scale), dev(bias), out.t)
+    rows = np.unique(np.concatenate([np.arange(8), [M // 2, M - 1]]))
+    _check_gemm_q8(out.check().reshape(M, N)[rows], np.ascontiguousarray(a[rows]), wq, scale, bias, None, None, 0, oracle)
+
+
 Q8_STREAM_TILES = [(16, 64, 512), (16, 64, 1024), (32, 64, 512), (64, 64, 512)]
 
 
