@@ -83,15 +83,23 @@ struct AddOp {
   typedef T In;
   typedef T Out;
   static constexpr int kInputs = 2;
+  static constexpr bool kBytewise = false;
   static __device__ __forceinline__ T apply(T a, T b) { return a + b; }
+  static __device__ __forceinline__ uint32_t apply_word(uint32_t a, uint32_t) { return a; }  // (unused)
 };
 template <>
 struct AddOp<int8_t> {
   typedef int8_t In;
   typedef int8_t Out;
   static constexpr int kInputs = 2;
+  static constexpr bool kBytewise = true;
   static __device__ __forceinline__ int8_t apply(int8_t a, int8_t b) {
     return static_cast<int8_t>(static_cast<uint8_t>(static_cast<uint8_t>(a) + static_cast<uint8_t>(b)));
+  }
+  // four bytes at once, each modulo 256: the low 7 bits of every byte add without reaching the next byte, and the top
+  // bit of a byte's sum is the xor of the two top bits and the carry into it
+  static __device__ __forceinline__ uint32_t apply_word(uint32_t a, uint32_t b) {
+    return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
   }
 };
 // Copy moves bit patterns through integer registers, so NaN payloads survive.
@@ -100,7 +108,9 @@ struct CopyOp {
   typedef Bits In;
   typedef Bits Out;
   static constexpr int kInputs = 1;
+  static constexpr bool kBytewise = sizeof(Bits) == 1;
   static __device__ __forceinline__ Bits apply(Bits a, Bits) { return a; }
+  static __device__ __forceinline__ uint32_t apply_word(uint32_t a, uint32_t) { return a; }
 };
 // Cast: fp16 -> fp32 is exact; fp32 -> fp16 rounds to nearest even and overflows to +-inf
 // (v_cvt_f16_f32), fp16 subnormal results are kept.
@@ -109,7 +119,9 @@ struct CastOp {
   typedef TI In;
   typedef TO Out;
   static constexpr int kInputs = 1;
+  static constexpr bool kBytewise = false;
   static __device__ __forceinline__ TO apply(TI a, TI) { return static_cast<TO>(a); }
+  static __device__ __forceinline__ uint32_t apply_word(uint32_t a, uint32_t) { return a; }  // (unused)
 };
 
 // ---- kernels ------------------------------------------------------------------------
@@ -138,14 +150,25 @@ __global__ void __launch_bounds__(kBlock) elt_vector_kernel(const void* __restri
     for (int u = 0; u < U; ++u) {
       const int64_t i = first + u * kBlock;
       if (full || i < nvec) {
-        Elems<TI, VEC> ea, eb;
-        Elems<TO, VEC> eo;
-        __builtin_memcpy(&ea, &ra[u], sizeof(ea));
-        if (Op::kInputs == 2) __builtin_memcpy(&eb, &rb[u], sizeof(eb)); else eb = ea;
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) eo.v[e] = Op::apply(ea.v[e], eb.v[e]);
         RO ro;
-        __builtin_memcpy(&ro, &eo, sizeof(ro));
+        if constexpr (Op::kBytewise && VEC % 4 == 0) {
+          // whole 32-bit words at once (byte by byte the compiler unpacks and repacks every element, and the launch is
+          // bound by that arithmetic: the int8 add over [8192, 4096] took 39.5 us at 8 vectors per thread, 18.0 at one)
+          uint32_t wa[VEC / 4], wb[VEC / 4], wo[VEC / 4];
+          __builtin_memcpy(wa, &ra[u], sizeof(wa));
+          if (Op::kInputs == 2) __builtin_memcpy(wb, &rb[u], sizeof(wb));
+#pragma unroll
+          for (int e = 0; e < VEC / 4; ++e) wo[e] = Op::apply_word(wa[e], Op::kInputs == 2 ? wb[e] : wa[e]);
+          __builtin_memcpy(&ro, wo, sizeof(ro));
+        } else {
+          Elems<TI, VEC> ea, eb;
+          Elems<TO, VEC> eo;
+          __builtin_memcpy(&ea, &ra[u], sizeof(ea));
+          if (Op::kInputs == 2) __builtin_memcpy(&eb, &rb[u], sizeof(eb)); else eb = ea;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) eo.v[e] = Op::apply(ea.v[e], eb.v[e]);
+          __builtin_memcpy(&ro, &eo, sizeof(ro));
+        }
         ro.store(out, i);
       }
     }
