@@ -825,8 +825,15 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
         // workgroups of 256 rows), 2049: 84.9 / 94.9, 3001: 159 / 170; with rows on the grid the big tiles stay ahead
         // whatever the fill (1088: 25.0 against 29.0), and so they do off the grid from three quarters of the CUs on
         // (1281: 43.9 / 45.9, 1537: 50.0 / 54.0)
-        const int64_t last_round = (heads * ceil_div(n, 256)) % kNumCU;
+        const int64_t w256 = heads * ceil_div(n, 256), last_round = w256 % kNumCU;
         if (!p_vec && last_round != 0 && last_round * 10 < kNumCU * 7) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {64, 128, kBK}, 1, 0};
+        // Rows on the grid, and the 256-row tiles make one round of the chip and a thin second one: the smaller tiles'
+        // rounds end closer together -- 64-row tiles up to 1.3 rounds (40 heads, n = m = 1600: 56.8 us against 63.7;
+        // 32 heads, 2560: 97.4 / 109.7; not against more than 4096 keys: 64 heads, 1280 x 8192: 328 / 314), 128-row tiles
+        // up to 1.5 (32 heads, 3072: 126 / 135; 64 heads, 1536: 73.9 / 78.2; 64 heads, 1280 x 8192: 291 / 314).  Measured
+        // with 16 .. 64 heads of 80 and 128 at n = 1100 .. 4096; from 1.5 rounds on the 256-row tiles are ahead again
+        else if (p_vec && w256 > kNumCU && w256 * 10 <= kNumCU * 13 && ktiles <= 64) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {64, 128, kBK}, 1, 0};
+        else if (p_vec && w256 > kNumCU && w256 * 2 <= kNumCU * 3) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
       } else cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {128, bn, kBK}, 1, 0};
       // 128-row tiles (one workgroup per CU) gain only while all parts run at once: 512 rows against 4096 keys
       // take 47 us in two parts, 58 whole, 80 in eight.  Partial tiles of 256 rows cost more to combine than a

@@ -154,7 +154,9 @@ def _check_pv(got, p, v, oracle):
                                  (257, 520), (1024, 1024),
                                  # the fitted choice of tile and key split up to one 128-row tile per CU: 64x64 whole and in parts,
                                  # 64x128 in 2 / 4 / 8 parts, 128x128 in 2 parts
-                                 (128, 128), (64, 1024), (256, 1024), (256, 4096), (128, 4100), (16, 8192), (384, 4096), (192, 2049)])
+                                 (128, 128), (64, 1024), (256, 1024), (256, 4096), (128, 4100), (16, 8192), (384, 4096), (192, 2049),
+                                 # 256-row tiles would make one round and a thin second one: 64-row tiles (1.125 rounds), 128-row (1.5)
+                                 (2304, 512), (3072, 256)])
 def test_pv_builtin_config(oracle, n, m):
     p, v = _pv_inputs(32, n, m, 80, 3 * n + m)
     out = Guarded((1, 32, n, 80), torch.float16)
