@@ -797,7 +797,9 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
         // fitted to a sweep of n = 16 .. 768 against 512 .. 8192 keys (32 heads of 80, P and V from memory).  Measured, new /
         // old choice: 256 rows against 1024 / 4096 / 8192 keys 12.1 / 26.7 / 42.9 us (16.7 / 42.4 / 61.5), 384 against 1024 /
         // 2048 / 4096 13.2 / 21.4 / 31.2 (24.6 / 33.3 / 43.7), 128 against 4096 18.9 (24.6), 128 x 128 4.7 (6.3)
-        const double hand64[4] = {0.0, 1.6, 4.0, 7.0}, hand[4] = {0.0, 2.5, 4.3, 6.5}, hand128[4] = {0.0, 4.0, 8.0, 16.0};
+        // (the constants refitted over 16 / 32 / 40 / 64 heads of 128 as well: mean ratio to the best of 28 configurations 1.004 /
+        // 1.006 / 1.013 / 1.035 -- 1.010 / 1.009 / 1.051 / 1.042 with the first fit -- and 1.001 still on the 32 heads of 80)
+        const double hand64[4] = {0.0, 1.6, 4.0, 4.9}, hand[4] = {0.0, 2.1, 3.9, 7.8}, hand128[4] = {0.0, 3.4, 8.0, 16.0};
         const int64_t t64 = heads * ceil_div(n, 64);
         double best = 1e30;
         for (int i = 0; i < 4; ++i) {
@@ -808,9 +810,9 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
           // 64x64, two stages: short sweeps on a chip that is not full
           const double us_a = w64 <= 128 && steps <= 8 ? 4.2 + (0.3 + 0.3 * w64 / 192.0) * steps + hand64[i] : 1e30;
           // 64x128, three stages (two workgroups per CU)
-          const double us_b = w64 <= 2 * kNumCU ? 5.2 + 0.55 * (w64 <= kNumCU ? 1.0 : 1.15 * w64 / kNumCU) * steps + hand[i] : 1e30;
+          const double us_b = w64 <= 2 * kNumCU ? 5.7 + 0.51 * (w64 <= kNumCU ? 1.0 : 1.25 * w64 / kNumCU) * steps + hand[i] : 1e30;
           // 128x128, three stages (one per CU)
-          const double us_c = w128 <= kNumCU ? 7.1 + (0.45 + 0.3 * (w128 / kNumCU) * (w128 / kNumCU)) * steps + hand128[i] : 1e30;
+          const double us_c = w128 <= kNumCU ? 7.4 + (0.45 + 0.335 * (w128 / kNumCU) * (w128 / kNumCU)) * steps + hand128[i] : 1e30;
           if (us_a < best) best = us_a, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 2, {64, 64, kBK}, parts, 0};
           if (us_b < best) best = us_b, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {64, 128, kBK}, parts, 0};
           if (us_c < best) best = us_c, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, parts, 0};
