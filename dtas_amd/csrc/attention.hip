@@ -601,6 +601,12 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
       // whole passes; enough workgroups to fill the chip twice, at least two passes each
       const int64_t want = ceil_div(m * heads * ceil_div(n, R), 2 * kNumCU);
       keys_per_wg = ceil_div(want < 2 * per_pass ? 2 * per_pass : want, per_pass) * per_pass;
+      // (whole passes can leave a few workgroups more than two per CU, and those few a round of their own -- 40 heads of
+      // 128 against 4096 keys: 13 x 40 = 520 workgroups, 16.2 us; 11 x 40: 13.3 -- so the keys are dealt to no more
+      // workgroups than fit at once)
+      const int64_t per_key_run = heads * ceil_div(n, R);
+      if (per_key_run <= 2 * kNumCU && ceil_div(m, keys_per_wg) * per_key_run > 2 * kNumCU)
+        keys_per_wg = ceil_div(ceil_div(m, (2 * kNumCU) / per_key_run), per_pass) * per_pass;
     }
     const int64_t gx = ceil_div(m, keys_per_wg), gz = ceil_div(n, R);
     if (gx > 0x7fffffff || gz > 65535 || keys_per_wg > 0x7fffffff) return fail("attn_scores: too many workgroups for the row kernel");
@@ -632,7 +638,9 @@ extern "C" int dtas_attn_scores_f16_f32(const void* Q, const void* Kmat, const v
   // one or two rows always, three or four against many keys (with K from memory, 32 heads of 80, us: 1 row against 2048 /
   // 4096 / 8192 keys 4.7 / 7.0 / 11.6 where the 64x64 tiles take 6.0 / 10.5 / 18.8; 2 rows 5.6 / 8.3 / 14.5 against 6.1 /
   // 10.6 / 18.8; 4 rows 6.7 / 9.3 / 16.4 against 6.1 / 10.6 / 19.2; 8 rows lose: 11.1 against 6.2 at 2048)
-  if (!user && d >= 8 && d / 8 <= 128 && (n <= 2 || (n <= 4 && m >= 3072))) return launch_rows(n <= 1 ? 1 : n <= 2 ? 2 : 4, 0);
+  // (head dimensions above 96: one row only -- 32 heads of 128, 4 rows against 4096 keys: 16.2 us where the 64x64 tiles take 11.3,
+  // 2 rows against 2048: 7.3 / 6.6; one row 9.9 / 11.2)
+  if (!user && d >= 8 && d / 8 <= 128 && (d <= 96 ? (n <= 2 || (n <= 4 && m >= 3072)) : n <= 1)) return launch_rows(n <= 1 ? 1 : n <= 2 ? 2 : 4, 0);
   const unsigned tm = static_cast<unsigned>(ceil_div(n, 128)), tn = static_cast<unsigned>(ceil_div(m, 64));
   const int64_t total = static_cast<int64_t>(tm) * tn * heads;
   const bool small = n <= 64 || total < kNumCU;
