@@ -754,10 +754,13 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       // keys are many: ~4.5 + 0.7 n m / 1000 us and ~6 + 0.4 n m / 1000 us, measured at n = 2 .. 12 against 512 ..
       // 4096 keys) unless the 64-row MFMA tiles with their keys split come out ahead (from ~8 rows against 4096
       // keys, ~12 against 512: 15 us against 25 at n = 8, m = 4096)
-      const double nm = 1e-3 * static_cast<double>(n) * static_cast<double>(m);
-      const double r2 = 4.5 + 0.7 * nm, r4 = n >= 4 ? 6.0 + 0.4 * nm : 1e30;
+      // (n m as it weighs with 32 heads of 80, where these were measured: the row kernels' time goes with the heads and the
+      // head dimension -- 8 rows against 2048 keys, 40 heads of 128: 37.5 us on the row kernel, 12.6 on the tiles)
+      const double nm = 1e-3 * static_cast<double>(n) * static_cast<double>(m) * (static_cast<double>(heads * d) / (32.0 * 80.0));
+      // (one row, the one-row form of the row kernel: 1.6 + 2.9 nm -- 7.3 / 10.9 / 14.9 / 20.0 us against 2048 keys with 32 heads of 80 / 32 / 40 / 64 heads of 128)
+      const double r2 = n == 1 ? 1.6 + 2.9 * nm : 4.5 + 0.7 * nm, r4 = n >= 4 ? 6.0 + 0.4 * nm : 1e30;
       double mfma_us = 1e30;
-      const bool mfma_ok = n >= 2 && (p_vec || (aligned(P, 2) && m >= 8));  // (any key count: P is read where it lies)
+      const bool mfma_ok = p_vec || (aligned(P, 2) && m >= 8);  // (any key count: P is read where it lies)
       if (mfma_ok) {
         key_split(heads, 4 * kNumCU, ktiles, &mfma_us);
         mfma_us = mfma_us + 1.5 < 5.5 ? 5.5 : mfma_us + 1.5;  // (no launch of the tiles takes less: 2 rows against 77 keys 7.5 us, the row kernel 4.6)
@@ -777,13 +780,17 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
       // 28.0 in halves / on the tiles; up to 2048 keys the hand-over costs more than it saves: 8.2 against 7.1)
       int runs = 1;
       while (heads * n * runs * 2 <= kNumCU && runs < 8) runs *= 2;
-      if (m >= 3072 && runs >= 2 && pieces <= 128) {
+      // (a workgroup's sweep of V, keys x head dimension, is what the whole-row forms pay for: the limits below are the 3072 /
+      // 6144 / 4096 keys of 80 they were measured at -- 8 rows against 8192 keys, 16 heads of 128, in 2 runs: 33.2 us, the tiles 18.8)
+      const int64_t md = m * d, kMd = 80;
+      const double whole_row_runs_us = 7.0 + 5e-5 * static_cast<double>(ceil_div(m, runs) * d) + 0.5 * runs;  // (4 rows of 128 against 4096 keys in 2 runs: 20.7 us, the tiles 16.0; 4 rows of 80 against 8192: 23.4 / 19.2)
+      if (m >= 3072 && runs >= 2 && pieces <= 128 && (!mfma_ok || whole_row_runs_us <= mfma_us)) {
         rows = true;
         cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, static_cast<int32_t>(d)}, runs, 0};
-      } else if (n >= 2 && n <= 8 && heads * n <= kNumCU && pieces <= 128 && (m < (halves == 2 ? 6144 : 3072) || !mfma_ok)) {
+      } else if (n >= 2 && n <= 8 && heads * n <= kNumCU && pieces <= 128 && (md < (halves == 2 ? 6144 : 3072) * kMd || !mfma_ok)) {
         rows = true;
         cfg = dtas_config{DTAS_GEMM_SKINNY, 1024, 8, 1, {1, 8, static_cast<int32_t>(d / halves)}, 1, 0};
-      } else if (n >= 2 && n <= 8 && m >= 3072 && heads * n <= kNumCU && mfma_ok) {
+      } else if (n >= 2 && n <= 8 && md >= 3072 * kMd && heads * n <= kNumCU && mfma_ok) {
         rows = false;  // (4 rows against 4096 / 8192 keys with V from memory: the row kernel 33 / 61 us, one sweep per row 22 / 39, the tiles 19 / 28)
       } else {
         rows = mfma_us >= (r2 < r4 ? r2 : r4);

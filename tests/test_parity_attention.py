@@ -164,8 +164,20 @@ def test_pv_builtin_config(oracle, n, m):
     _check_pv(out.check().reshape(32, n, 80), p, v, oracle)
 
 
+@pytest.mark.parametrize("heads,n,m,d", [(40, 1, 2048, 128), (64, 1, 2048, 128), (40, 8, 2048, 128), (16, 8, 8192, 128), (40, 2, 8192, 128),
+                                         (32, 4, 4096, 128), (32, 2, 8192, 128), (64, 12, 1024, 128), (40, 1, 520, 128), (40, 1, 1001, 96)])
+def test_pv_few_rows_with_other_head_counts_and_dimensions(oracle, heads, n, m, d):
+    # the choice between the row kernels and the tiles goes with heads x head dimension: one row on the tiles with their
+    # keys in parts (40 and 64 heads of 128), the tiles instead of the row kernel or of the sweep in key runs, and the
+    # cases that stay on those
+    p, v = _pv_inputs(heads, n, m, d, heads + n + m)
+    out = Guarded((1, heads, n, d), torch.float16)
+    ops.attn_pv(dev(p).view(1, heads, n, m), dev(v).view(1, heads, m, d), out.t)
+    _check_pv(out.check().reshape(heads, n, d), p, v, oracle)
+
+
 @pytest.mark.parametrize("tile,stages", [((64, 64), 2), ((64, 128), 2), ((64, 128), 3), ((128, 64), 2), ((128, 128), 2), ((128, 128), 3), ((256, 128), 3)])
-@pytest.mark.parametrize("heads,n,m,d", [(3, 70, 136, 80), (2, 300, 264, 64), (1, 33, 8, 8), (2, 50, 72, 136), (1, 129, 1032, 128),
+@pytest.mark.parametrize("heads,n,m,d", [(2, 1, 264, 128), (3, 70, 136, 80), (2, 300, 264, 64), (1, 33, 8, 8), (2, 50, 72, 136), (1, 129, 1032, 128),
                                          (2, 260, 64, 80), (2, 20, 128, 80), (1, 515, 192, 80)])
 def test_pv_every_tile(oracle, tile, stages, heads, n, m, d):
     # m = 8 .. 1032: one k tile, two, three (every prologue / drain case of the two- and three-stage pipelines), many
