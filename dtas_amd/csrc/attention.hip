@@ -833,7 +833,23 @@ extern "C" int dtas_attn_pv_f16(const void* P, const void* V, void* out, int64_t
           if (us_c < best) best = us_c, cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, parts, 0};
         }
         fitted = true;
-      } else if (t128 <= kNumCU / 2) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, bn == 128 ? 3 : 2, {64, bn, kBK}, 1, 0};
+      } else if (t128 <= kNumCU / 2) {
+        cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, bn == 128 ? 3 : 2, {64, bn, kBK}, 1, 0};
+        if (bn == 64) {
+          // head dimensions up to 64: the 64x64 term of the fit above, the keys in parts while the workgroups number at most
+          // two per CU (32 heads of 64: 256 rows against 4096 keys 30.3 -> 24.4 us in 4 parts, 512 against 2048 28.2 -> 21.4 in 2)
+          const double hand64[4] = {0.0, 1.6, 4.0, 4.9};
+          const int64_t t64 = heads * ceil_div(n, 64);
+          double best = 1e30;
+          for (int i = 0; i < 4; ++i) {
+            const int parts = 1 << i;
+            if (i > 0 && (ktiles < 2 * parts || t64 * parts > 2 * kNumCU)) break;
+            const double us = 4.2 + (0.3 + 0.3 * static_cast<double>(t64 * parts) / 192.0) * static_cast<double>(ceil_div(ktiles, parts)) + hand64[i];
+            if (us < best) best = us, cfg.split_k = parts;
+          }
+          fitted = true;
+        }
+      }
       else if (t128 <= kNumCU && bn == 128) cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {128, 128, kBK}, 1, 0};
       else if (bn == 128) {
         cfg = dtas_config{DTAS_GEMM_MFMA, 256, 8, 3, {256, 128, kBK}, 1, 0};
