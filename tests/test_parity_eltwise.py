@@ -279,7 +279,12 @@ def test_take_clips_ids_scalar_path_descriptor_and_errors(oracle):
                                              (7, 9, 3, 64, 64), (5, 5, 2, 16, 0), (33, 40, 4, 128, 32),
                                              # rot = 20 with rows of 3, 4, 7, 64 and 65 pieces; one row; rows that end a chunk early
                                              (19, 4096, 5, 24, 20), (130, 130, 3, 32, 20), (41, 50, 7, 56, 20), (9, 9, 2, 512, 20),
-                                             (3, 3, 2, 520, 20), (1, 7, 1, 80, 20), (4096, 4096, 32, 80, 20)])
+                                             (3, 3, 2, 520, 20), (1, 7, 1, 80, 20), (4096, 4096, 32, 80, 20),
+                                             # rotated widths in whole 16-byte pieces (a multiple of 16): all of d, half, a quarter; 16 itself
+                                             (300, 4096, 32, 128, 128), (1, 77, 40, 128, 128), (513, 600, 64, 128, 64), (50, 50, 12, 64, 64),
+                                             (77, 100, 8, 64, 32), (9, 4000, 3, 48, 16), (2049, 2049, 32, 128, 128), (31, 31, 5, 96, 48),
+                                             # other widths stay with the kernel for any width
+                                             (40, 64, 32, 96, 24), (6, 6, 2, 40, 36)])
 def test_rotary_is_bit_exact(oracle, n, m, heads, d, rot):
     rng = np.random.default_rng(n + m + d)
     a = rng.standard_normal((1, n, heads, d)).astype(np.float16)
