@@ -789,6 +789,61 @@ __global__ void __launch_bounds__(1024) softmax_temp_split_kernel(const float* _
   }
 }
 
+// The same for rows of more than 65536 elements (vocabularies of 128256 or 151936): the row does not fit the registers
+// of one workgroup, so the two passes over the whole row read it from the cache again, four vectors in flight per
+// thread; a thread adds up the same elements in the same order as above.
+__global__ void __launch_bounds__(1024) softmax_temp_split_loop_kernel(const float* __restrict__ A, const float* __restrict__ temp,
+                                                                       float* __restrict__ out, int64_t cols, int parts) {
+  __shared__ float slots[64];
+  int phase = 0;
+  const float t = temp ? *temp : 1.f;
+  const int64_t row = blockIdx.x / parts;
+  const int part = blockIdx.x % parts;
+  const float* x = A + row * cols;
+  const float sign = t < 0.f ? -1.f : 1.f;
+  float hi = kNegMax;
+  for (int64_t k0 = static_cast<int64_t>(threadIdx.x) * 4; k0 < cols; k0 += 4 * 4096) {
+    f32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t k = k0 + u * 4096;
+      v[u] = *reinterpret_cast<const f32x4*>(x + (k < cols ? k : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (k0 + u * 4096 < cols) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hi = fmaxf(hi, sign * v[u][e]);
+      }
+  }
+  const float xm = sign * block_reduce<MaxOp>(hi, slots, phase);
+  const float mx = fmaxf(kNegMax, xm / t);
+  const float rt = kLog2e * __builtin_amdgcn_rcpf(t);
+  float s = 0.f;
+  for (int64_t k0 = static_cast<int64_t>(threadIdx.x) * 4; k0 < cols; k0 += 4 * 4096) {
+    f32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t k = k0 + u * 4096;
+      v[u] = *reinterpret_cast<const f32x4*>(x + (k < cols ? k : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (k0 + u * 4096 < cols) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s += __builtin_amdgcn_exp2f((v[u][e] - xm) * rt);
+      }
+  }
+  s = block_reduce<SumOp>(s, slots, phase);
+  const int64_t k = (static_cast<int64_t>(part) * 1024 + threadIdx.x) * 4;
+  if (k < cols) {
+    f32x4 w = *reinterpret_cast<const f32x4*>(x + k);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = expf(w[e] / t - mx) / s;
+    *reinterpret_cast<f32x4*>(out + row * cols + k) = w;
+  }
+}
+
 }  // namespace dtas
 
 extern "C" {
@@ -834,19 +889,22 @@ static int run_softmax_f32(const char* what, const void* logits, const void* tem
   if (!logits || (with_temperature && !temperature) || !out) return fail("%s: NULL buffer", what);
   if (!aligned(logits, 4) || (with_temperature && !aligned(temperature, 4)) || !aligned(out, 4)) return fail("%s: buffers must be 4-byte aligned", what);
   if (overlaps(out, rows * cols * 4, logits, rows * cols * 4)) return fail("%s: output overlaps the input", what);
-  const bool vec = cols % 4 == 0 && aligned(logits, 16) && aligned(out, 16) && cols <= 4096 * 16;
+  const bool vec_any = cols % 4 == 0 && aligned(logits, 16) && aligned(out, 16);
+  const bool vec = vec_any && cols <= 4096 * 16;
   const unsigned grid = static_cast<unsigned>(rows > int64_t{kNumCU} * 8 ? int64_t{kNumCU} * 8 : rows);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const float* x = static_cast<const float*>(logits);
   const float* t = static_cast<const float*>(temperature);
   float* o = static_cast<float*>(out);
   const int64_t parts = ceil_div(cols, 4096);
-  if (vec && parts > 1 && rows * parts <= 2 * kNumCU) {
+  if (vec_any && parts > 1 && rows * parts <= 2 * kNumCU) {
     const unsigned wgs = static_cast<unsigned>(rows * parts);
     if (parts <= 4)
       hipLaunchKernelGGL(softmax_temp_split_kernel<4>, dim3(wgs), dim3(1024), 0, st, x, t, o, cols, static_cast<int>(parts));
-    else
+    else if (parts <= 16)
       hipLaunchKernelGGL(softmax_temp_split_kernel<16>, dim3(wgs), dim3(1024), 0, st, x, t, o, cols, static_cast<int>(parts));
+    else   // (a row of 128256: 86 us with one workgroup walking it element by element)
+      hipLaunchKernelGGL(softmax_temp_split_loop_kernel, dim3(wgs), dim3(1024), 0, st, x, t, o, cols, static_cast<int>(parts));
   } else if (vec && cols <= 4096)
     hipLaunchKernelGGL(softmax_temp_kernel<1>, dim3(grid), dim3(1024), 0, st, x, t, o, rows, cols);
   else if (vec && cols <= 4096 * 4)

@@ -298,7 +298,7 @@ def test_reduction_errors():
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 50280), (1, 1), (3, 4096), (2, 4100), (5, 16384), (2, 50281), (1, 65540), (4, 100000),
-                                       (700, 64)])
+                                       (700, 64), (1, 128256), (2, 151936), (1, 65536), (3, 262144)])
 @pytest.mark.parametrize("t", [0.7, 1.0, -0.8])
 def test_softmax_temperature(oracle, rows, cols, t):
     rng = np.random.default_rng(rows * 7 + cols)
@@ -332,7 +332,7 @@ def test_softmax_temperature_unaligned_and_errors(oracle):
         ops.softmax_temperature(xd, torch.tensor(0.9, dtype=torch.float16, device="cuda"), out.t)
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 50280), (3, 4096), (2, 50281), (300, 1000)])
+@pytest.mark.parametrize("rows,cols", [(1, 50280), (3, 4096), (2, 50281), (300, 1000), (1, 128256), (2, 151936)])
 def test_softmax_f32(oracle, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
