@@ -858,14 +858,14 @@ int dtas_layer_norm_f32(const void* x, const void* gamma, const void* beta, void
   if (!aligned(x, 4) || !aligned(gamma, 4) || !aligned(beta, 4) || !aligned(out, 4)) return fail("layer_norm_f32: buffers must be 4-byte aligned");
   if (overlaps(out, n * H * 4, x, n * H * 4) || overlaps(out, n * H * 4, gamma, H * 4) || overlaps(out, n * H * 4, beta, H * 4))
     return fail("layer_norm_f32: output overlaps an input");
-  const bool vec = H % 4 == 0 && H <= 4096 && aligned(x, 16) && aligned(out, 16) && aligned(gamma, 16) && aligned(beta, 16);
+  const bool vec = H % 4 == 0 && H <= 8192 && aligned(x, 16) && aligned(out, 16) && aligned(gamma, 16) && aligned(beta, 16);
   const unsigned grid = static_cast<unsigned>(n > int64_t{kNumCU} * 32 ? int64_t{kNumCU} * 32 : n);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const float* xp = static_cast<const float*>(x);
   const float* gp = static_cast<const float*>(gamma);
   const float* bp = static_cast<const float*>(beta);
   float* op = static_cast<float*>(out);
-  if (vec && n >= 2 * kNumCU) {   // many rows: a wavefront each
+  if (vec && H <= 4096 && n >= 2 * kNumCU) {   // many rows: a wavefront each
     const unsigned wgrid = static_cast<unsigned>(ceil_div(n, 4) > int64_t{kNumCU} * 32 ? int64_t{kNumCU} * 32 : ceil_div(n, 4));
     if (H <= 1024) hipLaunchKernelGGL(layer_norm_f32_wave_kernel<4>, dim3(wgrid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
     else if (H <= 2560) hipLaunchKernelGGL(layer_norm_f32_wave_kernel<10>, dim3(wgrid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
@@ -875,7 +875,10 @@ int dtas_layer_norm_f32(const void* x, const void* gamma, const void* beta, void
   if (vec && H <= 1024) hipLaunchKernelGGL(layer_norm_f32_kernel<1>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
   else if (vec && H <= 2048) hipLaunchKernelGGL(layer_norm_f32_kernel<2>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
   else if (vec && H <= 3072) hipLaunchKernelGGL(layer_norm_f32_kernel<3>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
-  else if (vec) hipLaunchKernelGGL(layer_norm_f32_kernel<4>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  else if (vec && H <= 4096) hipLaunchKernelGGL(layer_norm_f32_kernel<4>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  // (rows of up to 8192: in registers as well -- [4096, 8192] took 83 us with two passes of element accesses)
+  else if (vec && H <= 6144) hipLaunchKernelGGL(layer_norm_f32_kernel<6>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
+  else if (vec) hipLaunchKernelGGL(layer_norm_f32_kernel<8>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
   else hipLaunchKernelGGL(layer_norm_f32_kernel<0>, dim3(grid), dim3(256), 0, st, xp, gp, bp, op, n, H, eps);
   return check_launch("layer_norm_f32");
 }

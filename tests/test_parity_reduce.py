@@ -352,7 +352,8 @@ def test_softmax_f32(oracle, rows, cols):
 
 
 @pytest.mark.parametrize("n,H", [(1, 2560), (37, 2560), (4096, 2560), (5, 1024), (3, 4096), (7, 4100), (6, 777), (2, 10000),
-                                 (600, 1024), (520, 4096), (513, 1028), (515, 8), (2049, 2564)])   # from 512 rows: a wavefront per row
+                                 (600, 1024), (520, 4096), (513, 1028), (515, 8), (2049, 2564),   # from 512 rows: a wavefront per row
+                                 (3, 5120), (700, 6144), (5, 8192), (600, 8192), (2, 8196)])       # rows of up to 8192 in registers
 def test_layer_norm_f32(oracle, n, H):
     rng = np.random.default_rng(n + H)
     x = (rng.standard_normal((n, H)) * 2 + 0.5).astype(np.float32)
