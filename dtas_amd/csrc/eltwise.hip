@@ -428,6 +428,47 @@ __global__ void __launch_bounds__(kBlock) rotary16_kernel(const half_t* __restri
   }
 }
 
+// Rotated widths that are a multiple of 4 but not of 16 (24 of 96): two neighbouring elements have neighbouring
+// partners and table entries, so a rotated piece takes four 4-byte loads of each instead of eight 2-byte ones (all
+// inside the rotated part of the row, at 4-byte alignment).
+template <typename I>
+__global__ void __launch_bounds__(kBlock) rotary4_kernel(const half_t* __restrict__ A, const half_t* __restrict__ cs,
+                                                         const half_t* __restrict__ sn, half_t* __restrict__ out,
+                                                         I pieces, I heads, I per_row, I rot, int64_t pos0) {
+#pragma clang fp contract(off)
+  const I step = static_cast<I>(gridDim.x) * kBlock, half_rot = rot >> 1;
+  for (I t = static_cast<I>(blockIdx.x) * kBlock + threadIdx.x; t < pieces; t += step) {
+    const I row = t / per_row, v = t - row * per_row, j0 = 8 * v;
+    const half_t* a = A + static_cast<int64_t>(row) * per_row * 8;
+    u32x4 raw = *reinterpret_cast<const u32x4*>(a + j0);
+    if (j0 < rot) {
+      const half_t* cr = cs + (pos0 + row / heads) * static_cast<int64_t>(rot);
+      const half_t* sr = sn + (pos0 + row / heads) * static_cast<int64_t>(rot);
+      f16x8 x = __builtin_bit_cast(f16x8, raw);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const I j = j0 + 2 * q;
+        if (j < rot) {   // (rot % 4 == 0: a pair is rotated or not as a whole, and lies on one side of rot / 2)
+          const bool low = j < half_rot;
+          const f16x2 p = __builtin_bit_cast(f16x2, *reinterpret_cast<const uint32_t*>(a + (low ? j + half_rot : j - half_rot)));
+          const f16x2 c = __builtin_bit_cast(f16x2, *reinterpret_cast<const uint32_t*>(cr + j));
+          const f16x2 sj = __builtin_bit_cast(f16x2, *reinterpret_cast<const uint32_t*>(sr + j));
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const half_t partner = low ? static_cast<half_t>(static_cast<float>(p[e]) * -1.f) : p[e];
+            const half_t t1 = static_cast<half_t>(static_cast<float>(c[e]) * static_cast<float>(x[2 * q + e]));
+            const half_t t2 = static_cast<half_t>(static_cast<float>(sj[e]) * static_cast<float>(partner));
+            x[2 * q + e] = static_cast<half_t>(static_cast<float>(t1) + static_cast<float>(t2));
+          }
+        }
+      }
+      raw = __builtin_bit_cast(u32x4, x);
+    }
+    store_stream(raw, reinterpret_cast<u32x4*>(out + static_cast<int64_t>(row) * per_row * 8 + j0));
+    if (pieces - t <= step) break;   // (t + step might wrap in 32 bits)
+  }
+}
+
 // The same for rows of 3 .. 64 pieces (the model's have 10) without the partner loads: a wavefront takes whole rows,
 // floor(64 / pieces per row) of them, one piece per lane (60 of the model's 64 lanes work), and the three lanes of a
 // row that hold the rotated pieces get their partners' words from one another through ds_bpermute -- piece 0 wants
@@ -798,6 +839,19 @@ int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* o
     else
       hipLaunchKernelGGL(rotary16_kernel<int64_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
                          pieces, heads, d / 8, rot / 8, m - n);
+    return check_launch("rotary");
+  }
+  if (rot > 0 && rot % 4 == 0 && cfg.unroll <= 1 && aligned(cos_t, 4) && aligned(sin_t, 4)) {  // partners and table entries in pairs
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half_t* a = static_cast<const half_t*>(A);
+    const half_t* c = static_cast<const half_t*>(cos_t);
+    const half_t* sn = static_cast<const half_t*>(sin_t);
+    if (pieces < (int64_t{1} << 31) && heads < (int64_t{1} << 31) && rot < (int64_t{1} << 31))
+      hipLaunchKernelGGL(rotary4_kernel<uint32_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
+                         static_cast<uint32_t>(pieces), static_cast<uint32_t>(heads), static_cast<uint32_t>(d / 8), static_cast<uint32_t>(rot), m - n);
+    else
+      hipLaunchKernelGGL(rotary4_kernel<int64_t>, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, st, a, c, sn, static_cast<half_t*>(out),
+                         pieces, heads, d / 8, rot, m - n);
     return check_launch("rotary");
   }
   hipLaunchKernelGGL(rotary_f16_kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, static_cast<hipStream_t>(stream),

@@ -284,7 +284,9 @@ def test_take_clips_ids_scalar_path_descriptor_and_errors(oracle):
                                              (300, 4096, 32, 128, 128), (1, 77, 40, 128, 128), (513, 600, 64, 128, 64), (50, 50, 12, 64, 64),
                                              (77, 100, 8, 64, 32), (9, 4000, 3, 48, 16), (2049, 2049, 32, 128, 128), (31, 31, 5, 96, 48),
                                              # other widths stay with the kernel for any width
-                                             (40, 64, 32, 96, 24), (6, 6, 2, 40, 36)])
+                                             # a multiple of 4 (partners and table entries in pairs); other even widths (the kernel for any width)
+                                             (40, 64, 32, 96, 24), (6, 6, 2, 40, 36), (300, 4096, 64, 96, 24), (5, 5, 2, 16, 4), (9, 20, 3, 40, 12),
+                                             (33, 33, 4, 32, 28), (4, 4, 2, 24, 18), (7, 8, 3, 16, 6), (3, 3, 1, 8, 2)])
 def test_rotary_is_bit_exact(oracle, n, m, heads, d, rot):
     rng = np.random.default_rng(n + m + d)
     a = rng.standard_normal((1, n, heads, d)).astype(np.float16)
