@@ -232,8 +232,9 @@ int dtas_take_f16(const void* A, const void* ids, void* out, int64_t n, int64_t 
  * length of the whole sequence, m >= n), each step an fp16 value:
  *   out[j] = cos[j] * A[j] + sin[j] * (j < rot/2 ? A[j + rot/2] * -1 : A[j - rot/2])   (j < rot);  A[j] else.
  * cfg, when given: {DTAS_ELT_VECTOR, block 256, vec 8, unroll 0 | 1 | 2}; unroll names the kernel (0: whole rows per
- * wavefront, for rot = 20 and d <= 512; 1: a 16-byte piece per thread, for rot = 20; 2: any rot) -- the results are
- * the same bits. */
+ * wavefront, for rot = 20 and d <= 512; 1: a 16-byte piece per thread with its partners and table entries in the widest
+ * loads the width allows -- rot = 20, rot % 16 == 0, rot % 4 == 0; 2: element by element, any even rot) -- the results
+ * are the same bits; 0 and 1 step down to the next form where theirs does not apply. */
 int dtas_rotary_f16(const void* A, const void* cos_t, const void* sin_t, void* out, int64_t n, int64_t m,
                     int64_t heads, int64_t d, int64_t rot, int64_t max_pos, const dtas_config* cfg, void* stream);
 
