@@ -339,8 +339,9 @@ extern "C" int dtas_gemv_q8_f16(const void* x, const void* Wq, const void* scale
   // 11008 x 5120: 11.8 / 13.9, 4096 x 5120: 6.4 / 7.4; level at K = 4096)
   // short rows (K <= 2048) from 12288 rows on: 2 wavefronts, and 8 rows per workgroup when K <= 1024 and N >= 16384 (28672 x 1024:
   // 8.1 us against 10.0; 13824 x 1024: 5.4 / 6.3 with 4 rows; 28672 x 2048: 11.8 / 13.0)
-  const int q8_block = K >= 8192 && N >= 4096 ? 512 : K <= 2048 && N >= 12288 ? 128 : 256;
-  const int q8_rows = N >= 4096 ? (K <= 1024 && N >= 16384 ? 8 : 4) : 2;
+  // (one wavefront on 4 rows up to K = 1024: 50280 x 768 11.0 -> 9.3 us, x 512 10.2 -> 8.8)
+  const int q8_block = K >= 8192 && N >= 4096 ? 512 : K <= 1024 && N >= 12288 ? 64 : K <= 2048 && N >= 12288 ? 128 : 256;
+  const int q8_rows = N >= 4096 ? 4 : 2;
   dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, q8_block, 8, 2, {q8_rows, 0, 0}, 1, 0};
   if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
   int64_t la[7];
@@ -405,7 +406,12 @@ extern "C" int dtas_gemv_q8_f32(const void* x, const void* Wq, const void* scale
   if (!y || (K > 0 && (!x || !Wq || !scale))) return fail("gemv_q8_f32: NULL buffer");
   if (overlaps(y, N * 4, Wq, N * K) || overlaps(y, N * 4, x, K * 4) || overlaps(y, N * 4, scale, N * (K / 32) * 4))
     return fail("gemv_q8_f32: output overlaps an input");
-  dtas_config cfg = user ? *user : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 8 : 2, 0, 0}, 1, 0};   // (50280 x 2560: 45 / 30 / 25 / 24 us with 1 / 2 / 4 / 8 rows per workgroup)
+  // (50280 x 2560: 45 / 30 / 25 / 24 us with 1 / 2 / 4 / 8 rows per workgroup; short rows leave most of 4 wavefronts idle:
+  // one wavefront on 4 rows up to K = 1024 -- 50257 x 768 16.0 -> 9.7 us, 128256 x 1024 35.3 -> 23.6 -- two up to 2048)
+  dtas_config cfg = user ? *user
+                    : K <= 1024 ? dtas_config{DTAS_GEMV_SPLITK, 64, 8, 2, {4, 0, 0}, 1, 0}
+                    : K <= 2048 ? dtas_config{DTAS_GEMV_SPLITK, 128, 8, 2, {4, 0, 0}, 1, 0}
+                                : dtas_config{DTAS_GEMV_SPLITK, 256, 8, 2, {N >= 16384 ? 8 : 2, 0, 0}, 1, 0};
   if (cfg.vec == 8 && !(aligned(x, 16) && aligned(Wq, 16))) cfg.vec = 1;
   int64_t la[7];
   if (describe_gemv(N, K, cfg, la) != 0) return -1;

@@ -16,7 +16,7 @@ class GEMVConfigEmiter(BaseConfigEmiter):
         N, K = self.func_info.func.params[1].shape
         out = []
         for rows in (1, 2, 4, 8):
-            for threads in (256, 128, 512):
+            for threads in (256, 128, 512, 64):
                 if threads * 8 > max(K, 512):
                     continue
                 c = GEMVConfig()
@@ -26,7 +26,7 @@ class GEMVConfigEmiter(BaseConfigEmiter):
         # rows of K >= 8192 do better with 8 wavefronts on two rows, and rows that leave the last pass of 4 wavefronts
         # partly empty (K = 2560) with two rows on those 4
         # (short rows: up to 1024 elements one pass of 2 wavefronts, up to 2048 one pass of 4, several rows per workgroup)
-        best = (2, 512) if K >= 8192 else (4 if N >= 12288 else 2, 128) if K <= 1024 else (2, 256) if K <= 2048 or K % 2048 != 0 else (1, 256)
+        best = (2, 512) if K >= 8192 else (4, 64) if K <= 512 and N >= 12288 else (4 if N >= 12288 else 2, 128) if K <= 1024 else (2, 256) if K <= 2048 or K % 2048 != 0 else (1, 256)
 
         if not any((c.TILE_S, c.TR) == best for c in out):
             c = GEMVConfig()

@@ -237,7 +237,7 @@ def test_reduction_emitters_lead_with_the_librarys_builtin_choice():
 
 
 @pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (2560, 2560), (28672, 1024), (5120, 1024),
-                                 (8192, 2048), (4096, 520), (32000, 4096), (2560, 10240)])
+                                 (8192, 2048), (4096, 520), (32000, 4096), (2560, 10240), (50280, 512), (4096, 512)])
 def test_gemv_emitter_leads_with_the_librarys_builtin_choice(N, K):
     want = _lib.select_bucket(_lib.OP_GEMV_F16, 1, N, K).config.to_dict()
     got = _first_candidate(pf.fused_NT_matmul_add_gemv(N, K, bias=True), ())

@@ -29,7 +29,7 @@ def _inputs(M, N, K, seed):
 
 GEMV_SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096),
                # short rows (2 wavefronts on 2 or 4 rows, 4 on 2) and the other branches of the built-in choice
-               (5120, 1024), (13824, 1024), (8192, 2048), (3000, 520), (7680, 2560), (2560, 10240), (300, 72)]
+               (5120, 1024), (13824, 1024), (8192, 2048), (3000, 520), (7680, 2560), (2560, 10240), (300, 72), (20000, 512), (12288, 264)]
 
 
 @pytest.mark.parametrize("N,K", GEMV_SHAPES)

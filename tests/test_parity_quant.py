@@ -70,7 +70,7 @@ def _check_gemv(got, x, wq, scale, bias, kind, oracle):
 
 
 @pytest.mark.parametrize("N,K", [(7680, 2560), (2560, 10240), (10240, 2560), (50280, 2560), (33, 64), (5, 32),
-                                 (13824, 1024), (16400, 512), (12300, 2048), (5120, 1024), (4096, 8192)])
+                                 (13824, 1024), (16400, 512), (12300, 2048), (5120, 1024), (4096, 8192), (20000, 768)])
 @pytest.mark.parametrize("kind", [_lib.EPI_BIAS, _lib.EPI_BIAS_GELU])
 def test_gemv_builtin_config(oracle, N, K, kind):
     rng = np.random.default_rng(N + K + kind)
@@ -435,7 +435,7 @@ def _check_gemv_f32(got, x, wq, scale, oracle):
     assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 2 * (K + 2) * 2.0 ** -24 * mag).all()
 
 
-@pytest.mark.parametrize("N,K", [(50280, 2560), (2560, 10240), (33, 64), (5, 32)])
+@pytest.mark.parametrize("N,K", [(50280, 2560), (2560, 10240), (33, 64), (5, 32), (50257, 768), (32000, 2048), (300, 1024), (32000, 4096)])
 def test_gemv_f32_scales_builtin_config(oracle, N, K):
     wq, scale = _weights_f32(N, K, N + K)
     x = np.random.default_rng(1).standard_normal(K).astype(np.float32)
