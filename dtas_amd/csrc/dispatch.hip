@@ -228,7 +228,9 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
   const double kt = static_cast<double>(ktiles);
   // no candidate is faster than it streams W: TB/s measured at M = 64 against a 50280 x 2560 W
   const double w_mb = 2.0 * static_cast<double>(n) * static_cast<double>(k) * 1e-6;
-  auto floored = [&](double us, double tbs) { return us > w_mb / tbs ? us : w_mb / tbs; };
+  // (candidates that all sit on the floor are told apart by their own estimates: 256 x 32000 x 4096, 125 tiles of 256x256
+  // 89.0 us, 250 of 256x128 74.4)
+  auto floored = [&](double us, double tbs) { return (us > w_mb / tbs ? us : w_mb / tbs) + 1e-3 * us; };
   auto relief = [](double fill) { return fill <= 0.5 ? 0.63 : 0.63 + 0.74 * (fill - 0.5); };
   {
     // 256x256 on 8 wavefronts (16x16x32 MFMA): a round of the chip costs ~8 us plus 1.50 us per k tile with every CU

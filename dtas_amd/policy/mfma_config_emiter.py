@@ -55,7 +55,8 @@ class MFMAConfigEmiter(BaseConfigEmiter):
 
         tiles = lambda bm, bn: cdiv(m_hi, bm) * cdiv(N, bn)
         w_mb = 2.0 * float(N) * float(K) * 1e-6
-        floored = lambda us, tbs: us if us > w_mb / tbs else w_mb / tbs     # W streams at 3.1 .. 4.3 TB/s, by tile
+        # W streams at 3.1 .. 4.3 TB/s, by tile; candidates that all sit on that floor are told apart by their own estimates
+        floored = lambda us, tbs: (us if us > w_mb / tbs else w_mb / tbs) + 1e-3 * us
         # 256x256 on 8 wavefronts: ~8 us per round of the chip plus 1.50 us per k tile with every CU busy, 0.63 of that
         # with half of the CUs or fewer busy (the card clocks higher), linear in between; split_k = 0: the tiles of
         # a partly filled last round are shared by 2..4 workgroups each (~15 / 18 / 21 us to combine)
