@@ -292,7 +292,10 @@ extern "C" int dtas_gemm_f16_fused(const void* A, const void* W, const void* bia
   dtas_config cfg = user ? *user : builtin_config(DTAS_OP_GEMM_F16, M, N, K).cfg;
   const bool vec_ok = K % 8 == 0 && aligned(A, 16) && aligned(W, 16);
   // two rows of A (the first bucket's table row is sized for 16): W streamed in whole rows, as the GEMV does
-  if (!user && M == 2 && vec_ok) cfg = dtas_config{DTAS_GEMM_ROWS, 64, 8, 1, {2, 2, 8}, 1, 0};
+  if (!user && M == 2 && vec_ok) cfg = dtas_config{DTAS_GEMM_ROWS, 64, 8, 1, {2, N <= 2560 ? 1 : 2, 8}, 1, 0};
+  // three or four rows against a W of few rows: a row of W per wavefront fills the chip where 64-column tiles do not
+  // (4 x 2560 x 2560: 5.3 us against 7.6, 2560 x 10240: 14.1 / 18.5; level at 4096 x 4096, behind at 7680 x 2560: 11.5 / 10.1)
+  if (!user && (M == 3 || M == 4) && vec_ok && (N <= 2560 || (N <= 4096 && K <= 4096))) cfg = dtas_config{DTAS_GEMM_ROWS, 64, 8, 1, {4, 1, 8}, 1, 0};
   if (cfg.vec == 8 && !vec_ok) cfg.vec = 1;  // K % 8 != 0 or odd pointers: element accesses
   int64_t la[7];
   if (describe_gemm(M, N, K, cfg, la) != 0) return -1;

@@ -320,6 +320,18 @@ def test_gemm_row_kernel_every_variant(oracle, mv, r, block, N, K):
         _check(out.check(), oracle.c.gemm(a, w, bias, threads=8), oracle.np64.gemm(a, w, bias))
 
 
+@pytest.mark.parametrize("M", [3, 4])
+def test_gemm_three_and_four_rows_against_few_rows_of_w_take_the_row_kernel(oracle, M):
+    # built-in: the row kernel up to 2560 rows of W (or 4096 x 4096), the tiles beyond; every epilogue
+    for kind, N, K in ((0, 2560, 2560), (1, 2560, 10240), (2, 4096, 4096), (3, 1000, 520), (0, 7680, 2560)):
+        a, w, bias, r1, r2 = _fused_inputs(M, N, K, 50 + kind + M)
+        res = (dev(r1), dev(r2)) if kind in (1, 2) else (None, None)
+        out = Guarded((1, M, N), torch.float32 if kind == 2 else torch.float16)
+        ops.gemm(dev(a), dev(w), dev(bias), out.t, None, epilogue=kind, res1=res[0], res2=res[1])
+        want = oracle.c.gemm_fused(a, w, bias, r1 if kind in (1, 2) else None, r2 if kind in (1, 2) else None, kind, threads=8)
+        _check_fused(out.check().reshape(M, N), want, oracle.np64.gemm_fused(a, w, bias, r1, r2, kind), kind, r1, r2)
+
+
 def test_gemm_two_rows_take_the_row_kernel_with_every_epilogue_and_errors(oracle):
     for kind, N, K in ((0, 4096, 4096), (1, 2560, 2560), (2, 2560, 2560), (3, 10240, 2560)):
         a, w, bias, r1, r2 = _fused_inputs(2, N, K, 40 + kind)
