@@ -285,7 +285,7 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
       consider(floored(gemm_rounds(t256128, kNumCU) * 1.0 * steps + 4.5 * split, 3.5), 256, 128, 512, 2, split);
     const double t12864 = tiles_of(128, 64) * split;
     if (t12864 <= kNumCU)
-      consider(floored(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 3.4), 128, 64, 256, 4, split);
+      consider(floored(0.47 * steps + (split > 1 ? 2.5 * split : 0.0), 3.8), 128, 64, 256, 4, split);   // (128 x 8192 x 8192 in two parts: 38.4 us, 3.5 TB/s of W)
   }
   // M <= 16 and at most one workgroup per CU of the W-streaming kernel (64 columns x 1024 of K each): 10.9 against
   // 12.8 us at 4096 x 4096, 7.2 against 10.2 at 2560 x 2560; with more workgroups than CUs a workgroup's loads,

@@ -97,7 +97,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
                 cands.append((floored(rounds(t256128, cus) * 1.0 * steps + 4.5 * split, 3.5), (256, 128, 2, split)))
             t12864 = tiles(128, 64) * split
             if t12864 <= cus:
-                cands.append((floored(0.47 * steps + (2.5 * split if split > 1 else 0.0), 3.4), (128, 64, 4, split)))
+                cands.append((floored(0.47 * steps + (2.5 * split if split > 1 else 0.0), 3.8), (128, 64, 4, split)))
         best = cands[0]
         for c in cands[1:]:          # first strict minimum, in the library's order of evaluation
             if c[0] < best[0]:
