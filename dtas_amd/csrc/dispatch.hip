@@ -278,7 +278,7 @@ dtas_config gemm_policy(int64_t M_hi, int64_t N, int64_t K) {
     const double steps = static_cast<double>(ceil_div(ktiles, split));
     const double t128 = tiles_of(128, 128) * split, t64 = tiles_of(64, 64) * split;
     if (split == 1 || t128 <= kNumCU)
-      consider(floored((t128 <= kNumCU ? 0.8 + 0.2 * t128 / kNumCU : gemm_rounds(t128, kNumCU)) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), 4.1), 128, 128, 256, 4, split);
+      consider(floored((t128 <= kNumCU ? 0.8 + 0.2 * t128 / kNumCU : gemm_rounds(t128, kNumCU)) * 0.665 * steps + (split > 1 ? 4.0 * split : 0.0), split > 1 ? 3.5 : 4.1), 128, 128, 256, 4, split);   // (in K parts W streams slower: 128 x 14336 x 4096 in two parts 39.1 us, 3.0 TB/s)
     consider(floored((t64 <= kNumCU ? 1.0 : 0.82 * static_cast<double>(ceil_div(static_cast<int64_t>(t64), kNumCU))) * 0.33 * steps + (split > 1 ? (t64 <= kNumCU ? 1.0 : 2.5) * split : 0.0), 4.3), 64, 64, 256, 4, split);
     const double t256128 = tiles_of(256, 128) * split;
     if (split > 1 && steps >= 32 && t256128 <= kNumCU)

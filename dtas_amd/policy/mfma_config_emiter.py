@@ -88,7 +88,7 @@ class MFMAConfigEmiter(BaseConfigEmiter):
             t128, t64 = tiles(128, 128) * split, tiles(64, 64) * split
             if split == 1 or t128 <= cus:
                 cands.append((floored((0.8 + 0.2 * t128 / cus if t128 <= cus else rounds(t128, cus)) * 0.665 * steps
-                                      + (4.0 * split if split > 1 else 0.0), 4.1), (128, 128, 4, split)))
+                                      + (4.0 * split if split > 1 else 0.0), 4.1 if split == 1 else 3.5), (128, 128, 4, split)))
             cands.append((floored((1.0 if t64 <= cus else 0.82 * -(-int(t64) // cus)) * 0.33 * steps
                                   + ((1.0 if t64 <= cus else 2.5) * split if split > 1 else 0.0), 4.3),
                           (64, 64, 4, split)))
